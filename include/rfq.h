@@ -1,0 +1,179 @@
+/*
+ * rfq.h -- C ABI of librfq: MI355X (gfx950) kernels for ROCmForge's
+ * quantized-weight path: block dequantisation fused into the decode GEMV and
+ * the prefill GEMM.
+ *
+ * The library is a drop-in for the device side of ROCmForge's operator
+ * surface.  Each entry point names the reference interface it replaces
+ * (paths relative to the ROCmForge tree).  Conventions:
+ *   - plain C types only; "d_" pointers are device pointers (what
+ *     HipBuffer::as_ptr() returns, src/backend/hip_backend/memory.rs:540-547),
+ *     "h_" pointers are host pointers;
+ *   - packed weights are the bytes exactly as ROCmForge stores them,
+ *     little-endian, blocks running along K, matrix rows contiguous
+ *     ([n_rows, n_cols] row-major, the layout documented at
+ *     src/kernels/matmul/quantized/q4_0.rs:139-148);
+ *   - every function returns an rfq_status (0 = success, like HIP_SUCCESS,
+ *     src/backend/hip_backend/ffi.rs:78); rfq_last_error() gives the text;
+ *   - device entry points only enqueue work on the caller's stream
+ *     (hipStream_t passed as void*, NULL = the default stream) and never
+ *     synchronise, unless the comment says otherwise;
+ *   - the caller owns every buffer; the library keeps no reference to them.
+ */
+#ifndef RFQ_H
+#define RFQ_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RFQ_VERSION 100 /* 0.1.0 */
+
+#if defined(_WIN32)
+#define RFQ_API
+#else
+#define RFQ_API __attribute__((visibility("default")))
+#endif
+
+/* Block formats; the values are GgufTensorType's ids
+ * (src/loader/tensor_type.rs:16-32). */
+typedef enum rfq_format {
+    RFQ_Q4_0 = 2,        /* 20 B / 32: f32 scale + 16 nibble bytes           */
+    RFQ_Q8_0 = 8,        /* 36 B / 32: f32 scale + 32 offset-binary bytes    */
+    RFQ_Q4_K = 12,       /* 256 B / 256: 8 f16 scales, 8 i8 mins, nibbles    */
+    RFQ_Q6_K = 14,       /* 256 B / 256: 16 f16 scales, 6-bit stream         */
+    RFQ_MXFP4 = 20,      /* 17 B / 32: i8 exponent + 16 nibble bytes         */
+    RFQ_MXFP6_E2M3 = 21, /* 25 B / 32: i8 exponent + 24 packed bytes         */
+    RFQ_MXFP6_E3M2 = 22  /* decoded exactly like E2M3 (src/loader/dequant.rs:693) */
+} rfq_format;
+
+typedef enum rfq_status {
+    RFQ_OK = 0,
+    RFQ_E_BADARG = -1,      /* null pointer, non-positive dimension, unknown enum   */
+    RFQ_E_SIZE = -2,        /* byte count does not match the shape                  */
+    RFQ_E_UNSUPPORTED = -3, /* valid request this build has no kernel for; the Rust
+                               wrapper maps it to HipError::KernelLoadFailed so the
+                               *_with_fallback paths still fall back
+                               (src/kernels/quant/q4_0.rs:236-251)                  */
+    RFQ_E_HIP = -4,         /* a HIP runtime call failed                            */
+    RFQ_E_NOMEM = -5        /* device or host allocation failed                     */
+} rfq_status;
+
+typedef enum rfq_dtype { RFQ_F32 = 0, RFQ_F16 = 1, RFQ_BF16 = 2 } rfq_dtype;
+
+/* Operand encodings of a prepared MXFP matrix (see rfq_mx_prepare). */
+typedef enum rfq_mx_kind { RFQ_MX_AUTO = 0, RFQ_MX_FP4 = 4, RFQ_MX_FP8 = 8 } rfq_mx_kind;
+
+/* ---- library ------------------------------------------------------------ */
+
+RFQ_API int rfq_version(void);
+/* Thread-local description of the last failure on this thread ("" if none). */
+RFQ_API const char *rfq_last_error(void);
+/* Elements per block / bytes per block the decoders stride by
+ * (GgufTensorType::block_size, src/loader/tensor_type.rs:77-88; strides at
+ * src/kernels/quant/q4_0.rs:269, q8_0.rs:33, q4_k.rs:206, q6_k.rs:206,
+ * src/loader/dequant.rs:47,91).  0 for an unknown format. */
+RFQ_API size_t rfq_block_elems(int fmt);
+RFQ_API size_t rfq_block_bytes(int fmt);
+/* ceil(n_elems / block_elems) * block_bytes. */
+RFQ_API size_t rfq_packed_bytes(int fmt, size_t n_elems);
+
+/* ---- dequantisation ------------------------------------------------------ */
+
+/* Packed bytes on the device -> f32 on the device, bit-exact with the CPU
+ * decoders, including their short-input behaviour: out is n_elems floats,
+ * every element the CPU loop would not reach is written as 0.0.
+ * Replaces the kernel launches inside dequantize_q4_0_kernel_cached
+ * (src/kernels/quant/q4_0.rs:107-153), dequantize_q4_k_gpu_kernel
+ * (q4_k.rs:99-148), dequantize_q6_k_gpu_kernel (q6_k.rs:102-149) and the
+ * unused mxfp/q8_0 dequant kernels (kernels/mxfp_dequant.hip, q8_0_dequant.hip). */
+RFQ_API int rfq_dequant(int fmt, const void *d_packed, size_t packed_bytes, float *d_out, size_t n_elems,
+                void *stream);
+
+/* Host bytes -> device f32: uploads through a temporary device buffer, runs
+ * rfq_dequant, synchronises the stream and frees the temporary -- the whole
+ * body of dequantize_q4_0_kernel_cached / dequantize_q4_k_gpu_kernel /
+ * dequantize_q6_k_gpu_kernel (same files as above). */
+RFQ_API int rfq_dequant_upload(int fmt, const uint8_t *h_packed, size_t packed_bytes, float *d_out,
+                       size_t n_elems, void *stream);
+
+/* Host bytes -> host f32 through the GPU (upload, kernel, download;
+ * synchronous).  Backs rocmforge::loader::dequant_q4_0 / dequant_q8_0 /
+ * dequant_q4_k / dequant_q6_k (src/loader/mod.rs:116-127), dequant_mxfp4 /
+ * dequant_mxfp6 (src/loader/dequant.rs:41,85) and the quantised arms of
+ * loader::dequantize (dequant.rs:673-700). */
+RFQ_API int rfq_dequant_host(int fmt, const uint8_t *h_packed, size_t packed_bytes, float *h_out,
+                     size_t n_elems);
+
+/* ---- decode GEMV (and small batches) -------------------------------------- */
+
+/* d_y[m, n] = d_x[m, k] . dequant(W)[n, k]^T, fp32 accumulation, 1 <= m <= 8,
+ * k a multiple of the block size, w_bytes == n * (k / block_elems) * block_bytes.
+ * Replaces matmul_q4_0_gpu (src/kernels/matmul/quantized/q4_0.rs:209-260) and
+ * its q4_k / q6_k twins (q4_k.rs:221-268, q6_k.rs:211-258), for every format. */
+RFQ_API int rfq_gemv(int fmt, const void *d_w, size_t w_bytes, const float *d_x, float *d_y, int m, int n,
+             int k, void *stream);
+
+/* The reference's raw-pointer launch signatures, argument order
+ * (activations, weights, output, m, n, k) as in matmul_q4_0_gpu
+ * (src/kernels/matmul/quantized/q4_0.rs:209-217) and the kernels' own
+ * parameter lists (kernels/q4_0_matmul.hip:153-160).  The byte size of the
+ * weights is implied by n and k. */
+RFQ_API int rfq_matmul_q4_0(const float *d_act, const uint8_t *d_w, float *d_out, int m, int n, int k, void *stream);
+RFQ_API int rfq_matmul_q8_0(const float *d_act, const uint8_t *d_w, float *d_out, int m, int n, int k, void *stream);
+RFQ_API int rfq_matmul_q4_k(const float *d_act, const uint8_t *d_w, float *d_out, int m, int n, int k, void *stream);
+RFQ_API int rfq_matmul_q6_k(const float *d_act, const uint8_t *d_w, float *d_out, int m, int n, int k, void *stream);
+
+/* Host-resident weights, device input and output, m = 1: allocate, upload,
+ * multiply, synchronise, free -- the observable behaviour of matmul_q4_0 /
+ * matmul_q4_k / matmul_q6_k / matmul_q8_0
+ * (src/kernels/matmul/quantized/q4_0.rs:153-203, q4_k.rs:173-215,
+ * q6_k.rs:163-205, q8_0.rs:69-106).  d_out receives n_rows floats. */
+RFQ_API int rfq_matmul_host_weights(int fmt, const uint8_t *h_w, size_t w_bytes, const float *d_input,
+                            size_t n_rows, size_t n_cols, float *d_out, void *stream);
+
+/* ---- prefill GEMM ----------------------------------------------------------- */
+
+/* d_out[m, n] = d_a[m, k] (fp16) . dequant(W)[n, k]^T on the fp16 matrix
+ * cores with fp32 accumulation; out_dtype is RFQ_F32 or RFQ_F16.  Formats:
+ * Q4_0, Q8_0, Q4_K, Q6_K.  k a multiple of 256 for the K-formats, of 32
+ * otherwise.  The reference has no fused prefill GEMM (its matmul_q* hard-wire
+ * m = 1, src/kernels/matmul/quantized/q4_0.rs:169; larger m goes through
+ * dequantise + hipBLAS SGEMM, src/tensor/matmul.rs:134-214); this is the same
+ * contraction. */
+RFQ_API int rfq_gemm_f16(int fmt, const void *d_w, size_t w_bytes, const void *d_a_f16, void *d_out,
+                 int out_dtype, int m, int n, int k, void *stream);
+
+/* MXFP matrices feed the gfx950 block-scaled matrix instruction, whose element
+ * and scale encodings differ from the bytes ROCmForge stores (signed exponent
+ * byte, its own E2M1/E2M3 value tables, a +-8 / +-7.5 clamp).  A matrix
+ * [rows, k] (k a multiple of 128) is therefore re-encoded once, value for
+ * value, into a caller-owned device buffer:
+ *   RFQ_MX_FP4: every block of the matrix is expressible as OCP E2M1 codes
+ *               with a (possibly shifted) E8M0 scale -- 4-bit operand, full rate;
+ *   RFQ_MX_FP8: E4M3 codes, which hold every value the reference decoders can
+ *               produce; always possible; half rate.  MXFP6 always takes this.
+ * rfq_mx_prepared_bytes: buffer size for the given kind (AUTO -> the FP8 size).
+ * rfq_mx_prepare: kind_req = AUTO picks FP4 when the whole matrix allows it
+ *   (this reads one flag back and therefore synchronises the stream); FP8
+ *   never synchronises; FP4 fails with RFQ_E_UNSUPPORTED (after a sync) when a
+ *   block is not expressible.  *kind_out receives the encoding written.
+ * This is the one-time weight upload step (src/loader/gguf/gpu_upload.rs:57-125
+ * does the analogous dequantise-at-load for the K formats). */
+RFQ_API size_t rfq_mx_prepared_bytes(int fmt, int kind, int rows, int k);
+RFQ_API int rfq_mx_prepare(int fmt, int kind_req, const void *d_raw, size_t raw_bytes, int rows, int k,
+                   void *d_prepared, size_t prepared_bytes, int *kind_out, void *stream);
+
+/* d_out[m, n] = A[m, k] . W[n, k]^T from two prepared operands, fp32
+ * accumulation in the matrix core, out_dtype RFQ_F32 or RFQ_BF16.
+ * m, n multiples of 32 are not required; k a multiple of 128 is. */
+RFQ_API int rfq_gemm_mx(const void *d_a_prep, int a_kind, const void *d_w_prep, int w_kind, void *d_out,
+                int out_dtype, int m, int n, int k, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RFQ_H */

@@ -1,0 +1,598 @@
+/*
+ * rf_oracle.c -- CPU restatement of ROCmForge's quantized dequant / matmul path.
+ *
+ * THIS IS TEST INFRASTRUCTURE, NOT PRODUCT CODE.  It exists only so that the
+ * HIP kernels can be checked against the arithmetic the reference performs on
+ * the CPU.  Only tests, the smoke check and the bench's cpu_baseline leg may
+ * link or call it; nothing in the shipped library does.
+ *
+ * Every function cites the reference file:line it follows (paths relative to
+ * the ROCmForge tree).  The reference is Rust; there is no Rust toolchain to
+ * build it here, so each function is pinned by the reference's own unit-test
+ * vectors and by independent closed-form / brute-force checks in tests/.
+ *
+ * Parity status per function:
+ *   pinned   : rf_dequant_q4_0, rf_dequant_q8_0, rf_dequant_q4_k,
+ *              rf_dequant_q6_k, rf_dequant_mxfp4, rf_dequant_mxfp6,
+ *              rf_decode_e2m1, rf_decode_e2m3, rf_encode_e2m1, rf_encode_e2m3,
+ *              rf_pack_6bit, rf_unpack_6bit, rf_pack_mxfp4, rf_pack_mxfp6,
+ *              rf_unpack_mxfp4, rf_unpack_mxfp6, rf_cpu_matmul_f32,
+ *              rf_f16_to_f32, rf_data_size
+ *   parity unpinned (no reference vector, reasoned from compiler-rt source):
+ *              rf_powi_f32 for exponent -128 only (returns 0.0), hence the
+ *              MXFP scale byte 0x80; rf_e8m0_from_f32 when log2 lands on an
+ *              exact .5 tie (affects generated inputs only, never compute).
+ *
+ * Build: gcc -O2 -ffp-contract=off -fno-fast-math -fopenmp -shared -fPIC
+ * (no FMA contraction: Rust never fuses a*b+c).
+ */
+#include <math.h>
+#include <stddef.h>
+#include <stdint.h>
+#include <string.h>
+
+#define RF_API __attribute__((visibility("default")))
+
+/* ------------------------------------------------------------------ */
+/* scalar helpers                                                      */
+/* ------------------------------------------------------------------ */
+
+/* IEEE binary16 -> binary32 widening, exact (subnormals, inf, nan kept).
+ * Stands for half::f16::from_bits(b).to_f32() (crate half 2.7.1) used at
+ * src/kernels/quant/q4_k.rs:236 and q6_k.rs:236. */
+RF_API float rf_f16_to_f32(uint16_t h)
+{
+    uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t exp = (h >> 10) & 0x1Fu;
+    uint32_t man = h & 0x3FFu;
+    uint32_t bits;
+    if (exp == 0) {
+        if (man == 0) {
+            bits = sign;
+        } else { /* subnormal: normalise */
+            int e = -1;
+            do { man <<= 1; e++; } while ((man & 0x400u) == 0);
+            bits = sign | ((uint32_t)(127 - 15 - e) << 23) | ((man & 0x3FFu) << 13);
+        }
+    } else if (exp == 31) {
+        bits = sign | 0x7F800000u | (man << 13);
+    } else {
+        bits = sign | ((exp + 112u) << 23) | (man << 13);
+    }
+    float f;
+    memcpy(&f, &bits, 4);
+    return f;
+}
+
+/* f32::powi lowers to llvm.powi.f32 -> compiler-rt __powisf2: repeated
+ * squaring on |b|, reciprocal at the end for negative b.  Used by
+ * E8M0::to_f32 (src/loader/mxfp.rs:23-25) and decode_e2m1/e2m3
+ * (mxfp.rs:243,292).  For b = -128 the squaring overflows to +inf and the
+ * reciprocal gives 0.0. */
+RF_API float rf_powi_f32(float a, int b)
+{
+    const int recip = b < 0;
+    float r = 1.0f;
+    for (;;) {
+        if (b & 1) r *= a;
+        b /= 2;
+        if (b == 0) break;
+        a *= a;
+    }
+    return recip ? 1.0f / r : r;
+}
+
+static float clampf(float v, float lo, float hi)
+{
+    /* f32::clamp: if v < lo -> lo; if v > hi -> hi; else v (NaN stays) */
+    if (v < lo) return lo;
+    if (v > hi) return hi;
+    return v;
+}
+
+/* src/loader/mxfp.rs:234-244 */
+RF_API float rf_decode_e2m1(uint8_t bits)
+{
+    if (bits == 0) return 0.0f;
+    float sign = (bits & 0x08) ? -1.0f : 1.0f;
+    int exp = (int)((bits >> 1) & 0x03) - 1;
+    float mant = (float)(bits & 0x01);
+    return sign * (1.0f + mant) * rf_powi_f32(2.0f, exp);
+}
+
+/* src/loader/mxfp.rs:283-293 */
+RF_API float rf_decode_e2m3(uint8_t bits)
+{
+    if (bits == 0) return 0.0f;
+    float sign = (bits & 0x20) ? -1.0f : 1.0f;
+    int exp = (int)((bits >> 3) & 0x03) - 1;
+    float mant = (float)(bits & 0x07) / 8.0f;
+    return sign * (1.0f + mant) * rf_powi_f32(2.0f, exp);
+}
+
+/* src/loader/mxfp.rs:200-231 */
+RF_API uint8_t rf_encode_e2m1(float value)
+{
+    if (value == 0.0f) return 0;
+    uint8_t sign = (value < 0.0f) ? 0x08 : 0x00;
+    float a = fabsf(value);
+    float clamped = fminf(fmaxf(a, 0.5f), 8.0f);
+    uint8_t best = 0;
+    float best_err = 3.40282347e+38f;
+    for (int e = 0; e < 4; e++) {
+        for (int m = 0; m < 2; m++) {
+            float decoded = (1.0f + (float)m) * rf_powi_f32(2.0f, e - 1);
+            float err = fabsf(clamped - decoded);
+            if (err < best_err) {
+                best_err = err;
+                best = (uint8_t)((e << 1) | m);
+            }
+        }
+    }
+    return sign | best;
+}
+
+/* src/loader/mxfp.rs:249-280 */
+RF_API uint8_t rf_encode_e2m3(float value)
+{
+    if (value == 0.0f) return 0;
+    uint8_t sign = (value < 0.0f) ? 0x20 : 0x00;
+    float a = fabsf(value);
+    float clamped = fminf(fmaxf(a, 0.5f), 7.5f);
+    uint8_t best = 0;
+    float best_err = 3.40282347e+38f;
+    for (int e = 0; e < 4; e++) {
+        for (int m = 0; m < 8; m++) {
+            float mant = (float)m / 8.0f;
+            float decoded = (1.0f + mant) * rf_powi_f32(2.0f, e - 1);
+            float err = fabsf(clamped - decoded);
+            if (err < best_err) {
+                best_err = err;
+                best = (uint8_t)((e << 3) | m);
+            }
+        }
+    }
+    return sign | best;
+}
+
+/* E8M0::from_f32, src/loader/mxfp.rs:29-43.  Returns the signed exponent. */
+RF_API int8_t rf_e8m0_from_f32(float value)
+{
+    if (value == 0.0f || isnan(value)) return 0;
+    if (isinf(value)) return 127;
+    float l = log2f(fabsf(value));
+    l = clampf(l, -127.0f, 127.0f);
+    return (int8_t)roundf(l); /* f32::round = half away from zero */
+}
+
+/* E8M0::to_f32, src/loader/mxfp.rs:23-25 */
+RF_API float rf_e8m0_to_f32(int8_t e) { return rf_powi_f32(2.0f, (int)e); }
+
+/* src/loader/mxfp.rs:297-320 (LSB-first bit stream) */
+RF_API void rf_pack_6bit(const uint8_t *values, size_t count, uint8_t *packed /* ceil(count*6/8), pre-zeroed by us */)
+{
+    size_t nbytes = (count * 6 + 7) / 8;
+    memset(packed, 0, nbytes);
+    for (size_t i = 0; i < count; i++) {
+        size_t bit_pos = i * 6;
+        size_t byte_idx = bit_pos / 8;
+        unsigned bit_offset = (unsigned)(bit_pos % 8);
+        uint8_t v = values[i] & 0x3F;
+        if (bit_offset <= 2) {
+            packed[byte_idx] |= (uint8_t)(v << bit_offset);
+        } else {
+            unsigned first = 8 - bit_offset;
+            packed[byte_idx] |= (uint8_t)(v << bit_offset);
+            packed[byte_idx + 1] |= (uint8_t)(v >> first);
+        }
+    }
+}
+
+/* src/loader/mxfp.rs:324-353 */
+RF_API void rf_unpack_6bit(const uint8_t *packed, size_t packed_len, size_t count, uint8_t *values)
+{
+    for (size_t i = 0; i < count; i++) {
+        size_t bit_pos = i * 6;
+        size_t byte_idx = bit_pos / 8;
+        unsigned bit_offset = (unsigned)(bit_pos % 8);
+        values[i] = 0;
+        if (byte_idx < packed_len) {
+            if (bit_offset <= 2) {
+                values[i] = (packed[byte_idx] >> bit_offset) & 0x3F;
+            } else {
+                unsigned first = 8 - bit_offset;
+                unsigned second = 6 - first;
+                uint8_t p1 = (packed[byte_idx] >> bit_offset) & (uint8_t)((1u << first) - 1);
+                uint8_t p2 = (byte_idx + 1 < packed_len)
+                                 ? (packed[byte_idx + 1] & (uint8_t)((1u << second) - 1))
+                                 : 0;
+                values[i] = p1 | (uint8_t)(p2 << first);
+            }
+        }
+    }
+}
+
+static float block_absmax(const float *v, size_t n)
+{
+    float m = 0.0f;
+    for (size_t i = 0; i < n; i++) {
+        float a = fabsf(v[i]);
+        /* f32::max ignores a NaN operand */
+        if (a > m || isnan(m)) m = a;
+    }
+    return m;
+}
+
+/* MxfpBlock::pack_mxfp4, src/loader/mxfp.rs:77-117.  values: up to 32 floats
+ * (n_values <= 32); out: 17 bytes = exponent byte + 16 nibble bytes, element
+ * 2j in the HIGH nibble of byte j. */
+RF_API void rf_pack_mxfp4(const float *values, size_t n_values, uint8_t *out17)
+{
+    float max_val = block_absmax(values, n_values);
+    int8_t e = (max_val == 0.0f) ? 0 : rf_e8m0_from_f32(max_val);
+    float scale = rf_e8m0_to_f32(e);
+    memset(out17, 0, 17);
+    out17[0] = (uint8_t)e;
+    size_t n = n_values < 32 ? n_values : 32;
+    for (size_t i = 0; i < n; i++) {
+        float normalized = (scale > 0.0f) ? values[i] / scale : values[i];
+        uint8_t enc = rf_encode_e2m1(normalized);
+        if ((i & 1) == 0) out17[1 + i / 2] |= (uint8_t)(enc << 4);
+        else out17[1 + i / 2] |= (uint8_t)(enc & 0x0F);
+    }
+}
+
+/* MxfpBlock::pack_mxfp6, src/loader/mxfp.rs:142-174. out: 25 bytes. */
+RF_API void rf_pack_mxfp6(const float *values, size_t n_values, uint8_t *out25)
+{
+    float max_val = block_absmax(values, n_values);
+    int8_t e = (max_val == 0.0f) ? 0 : rf_e8m0_from_f32(max_val);
+    float scale = rf_e8m0_to_f32(e);
+    uint8_t codes[32];
+    size_t n = n_values < 32 ? n_values : 32;
+    for (size_t i = 0; i < n; i++) {
+        float normalized = (scale > 0.0f) ? values[i] / scale : values[i];
+        codes[i] = rf_encode_e2m3(normalized);
+    }
+    memset(out25, 0, 25);
+    out25[0] = (uint8_t)e;
+    rf_pack_6bit(codes, n, out25 + 1);
+}
+
+/* MxfpBlock::unpack_mxfp4, src/loader/mxfp.rs:120-139 */
+RF_API void rf_unpack_mxfp4(const uint8_t *blk17, float *out32)
+{
+    float scale = rf_e8m0_to_f32((int8_t)blk17[0]);
+    for (int i = 0; i < 32; i++) {
+        uint8_t b = blk17[1 + i / 2];
+        uint8_t nib = (i % 2 == 0) ? ((b >> 4) & 0x0F) : (b & 0x0F);
+        out32[i] = clampf(scale * rf_decode_e2m1(nib), -8.0f, 8.0f);
+    }
+}
+
+/* MxfpBlock::unpack_mxfp6, src/loader/mxfp.rs:177-190 (LSB-first unpack; note
+ * this is NOT the extraction the loader's dequant_mxfp6 uses). */
+RF_API void rf_unpack_mxfp6(const uint8_t *blk25, float *out32)
+{
+    uint8_t codes[32];
+    rf_unpack_6bit(blk25 + 1, 24, 32, codes);
+    float scale = rf_e8m0_to_f32((int8_t)blk25[0]);
+    for (int i = 0; i < 32; i++)
+        out32[i] = clampf(scale * rf_decode_e2m3(codes[i]), -7.5f, 7.5f);
+}
+
+/* ------------------------------------------------------------------ */
+/* canonical dequantisers (what rocmforge::loader::dequant_* resolve to) */
+/* ------------------------------------------------------------------ */
+
+static float rd_f32le(const uint8_t *p)
+{
+    uint32_t u = (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16) | ((uint32_t)p[3] << 24);
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+/* dequantize_q4_0_cpu, src/kernels/quant/q4_0.rs:266-310 */
+RF_API void rf_dequant_q4_0(const uint8_t *data, size_t len, size_t n, float *out)
+{
+    size_t n_blocks = (n + 31) / 32;
+    for (size_t i = 0; i < n; i++) out[i] = 0.0f;
+    for (size_t b = 0; b < n_blocks; b++) {
+        size_t off = b * 20;
+        if (off + 4 > len) break;
+        float scale = rd_f32le(data + off);
+        size_t ds = off + 4, base = b * 32;
+        for (size_t i = 0; i < 16; i++) {
+            if (ds + i >= len) break;
+            uint8_t packed = data[ds + i];
+            int low = (int)(packed & 0x0F) - 8;
+            if (base + i * 2 < n) out[base + i * 2] = scale * (float)low;
+            int high = (int)((packed >> 4) & 0x0F) - 8;
+            if (base + i * 2 + 1 < n) out[base + i * 2 + 1] = scale * (float)high;
+        }
+    }
+}
+
+/* dequantize_q8_0, src/kernels/quant/q8_0.rs:23-71 (block order is
+ * irrelevant: every block writes a disjoint slice) */
+RF_API void rf_dequant_q8_0(const uint8_t *data, size_t len, size_t n, float *out)
+{
+    size_t blocks = (n + 31) / 32;
+    for (size_t i = 0; i < n; i++) out[i] = 0.0f;
+    for (size_t b = 0; b < blocks; b++) {
+        size_t start = b * 36;
+        if (start + 4 > len) continue;
+        float scale = rd_f32le(data + start);
+        size_t qs = start + 4;
+        size_t qe = qs + 32 < len ? qs + 32 : len;
+        for (size_t i = 0; qs + i < qe; i++) {
+            size_t idx = b * 32 + i;
+            if (idx < n) out[idx] = ((float)data[qs + i] - 128.0f) * scale;
+        }
+    }
+}
+
+/* dequantize_q4_k_cpu, src/kernels/quant/q4_k.rs:201-273 */
+RF_API void rf_dequant_q4_k(const uint8_t *data, size_t len, size_t n, float *out)
+{
+    size_t nsb = (n + 255) / 256;
+    for (size_t i = 0; i < n; i++) out[i] = 0.0f;
+    for (size_t s = 0; s < nsb; s++) {
+        size_t so = s * 256;
+        if (so + 256 > len) break;
+        size_t scales_start = so, mins_start = so + 16, quants_start = so + 32;
+        for (size_t sub = 0; sub < 8; sub++) {
+            size_t sub_start = s * 256 + sub * 32;
+            if (sub_start >= n) break;
+            size_t sc_off = scales_start + sub * 2;
+            float scale = 1.0f;
+            if (sc_off + 2 <= len)
+                scale = rf_f16_to_f32((uint16_t)(data[sc_off] | (data[sc_off + 1] << 8)));
+            size_t mn_off = mins_start + sub;
+            float mn = 0.0f;
+            if (mn_off < len) mn = (float)(int8_t)data[mn_off];
+            for (size_t i = 0; i < 32; i++) {
+                size_t idx = sub_start + i;
+                if (idx >= n) break;
+                size_t bit_pos = i * 4;
+                size_t byte_idx = bit_pos / 8;
+                unsigned bit_offset = (unsigned)(bit_pos % 8);
+                size_t qo = quants_start + sub * 28 + byte_idx;
+                if (qo + 1 < len) {
+                    uint16_t combined = (uint16_t)(((uint16_t)data[qo + 1] << 8) | data[qo]);
+                    uint8_t q = (uint8_t)((combined >> bit_offset) & 0x0F);
+                    out[idx] = mn + (float)q * scale;
+                }
+            }
+        }
+    }
+}
+
+/* dequantize_q6_k_cpu, src/kernels/quant/q6_k.rs:201-266 */
+RF_API void rf_dequant_q6_k(const uint8_t *data, size_t len, size_t n, float *out)
+{
+    size_t nb = (n + 255) / 256;
+    for (size_t i = 0; i < n; i++) out[i] = 0.0f;
+    for (size_t b = 0; b < nb; b++) {
+        size_t bs = b * 256;
+        if (bs + 256 > len) break;
+        size_t scales_start = bs, quants_start = bs + 32;
+        for (size_t i = 0; i < 256; i++) {
+            size_t idx = b * 256 + i;
+            if (idx >= n) break;
+            size_t sc_off = scales_start + (i / 16) * 2;
+            float scale = 1.0f;
+            if (sc_off + 2 <= len)
+                scale = rf_f16_to_f32((uint16_t)(data[sc_off] | (data[sc_off + 1] << 8)));
+            unsigned bit_offset = (unsigned)((i * 6) % 8);
+            size_t byte_idx = (i * 6) / 8;
+            if (quants_start + byte_idx + 1 < len) {
+                uint16_t combined = (uint16_t)(((uint16_t)data[quants_start + byte_idx + 1] << 8) |
+                                               data[quants_start + byte_idx]);
+                uint8_t q = (uint8_t)((combined >> bit_offset) & 0x3F);
+                float sv = (q >= 32) ? (float)(int8_t)((int8_t)q - 64) : (float)q;
+                out[idx] = sv * scale;
+            }
+        }
+    }
+}
+
+/* dequant_mxfp4, src/loader/dequant.rs:41-82 */
+RF_API void rf_dequant_mxfp4(const uint8_t *data, size_t len, size_t n, float *out)
+{
+    size_t blocks = (n + 31) / 32;
+    for (size_t i = 0; i < n; i++) out[i] = 0.0f;
+    for (size_t b = 0; b < blocks; b++) {
+        size_t bs = b * 17;
+        if (bs + 1 > len) break;
+        float scale = rf_powi_f32(2.0f, (int)(int8_t)data[bs]);
+        size_t ds = bs + 1;
+        size_t de = ds + 16 < len ? ds + 16 : len;
+        for (size_t bo = 0; ds + bo < de; bo++) {
+            uint8_t packed = data[ds + bo];
+            for (int j = 0; j < 2; j++) {
+                size_t idx = b * 32 + bo * 2 + (size_t)j;
+                if (idx < n) {
+                    uint8_t bits = (j == 0) ? ((packed >> 4) & 0x0F) : (packed & 0x0F);
+                    float val = scale * rf_decode_e2m1(bits);
+                    out[idx] = clampf(val, -8.0f, 8.0f);
+                }
+            }
+        }
+    }
+}
+
+/* dequant_mxfp6, src/loader/dequant.rs:85-132.  Used for both Mxfp6E2m3 and
+ * Mxfp6E3m2 (dequant.rs:693).  Note the ">> (10 - bit_offset)" extraction and
+ * that element 31 of a block is never written. */
+RF_API void rf_dequant_mxfp6(const uint8_t *data, size_t len, size_t n, float *out)
+{
+    size_t blocks = (n + 31) / 32;
+    for (size_t i = 0; i < n; i++) out[i] = 0.0f;
+    for (size_t b = 0; b < blocks; b++) {
+        size_t bs = b * 25;
+        if (bs + 1 > len) break;
+        float scale = rf_powi_f32(2.0f, (int)(int8_t)data[bs]);
+        size_t ds = bs + 1;
+        size_t de = ds + 24 < len ? ds + 24 : len;
+        const uint8_t *pd = data + ds;
+        size_t plen = de - ds;
+        for (size_t i = 0; i < 32; i++) {
+            size_t idx = b * 32 + i;
+            if (idx >= n) break;
+            unsigned bit_offset = (unsigned)((i * 6) % 8);
+            size_t byte_idx = (i * 6) / 8;
+            if (byte_idx + 1 < plen) {
+                uint16_t combined = (uint16_t)(((uint16_t)pd[byte_idx + 1] << 8) | pd[byte_idx]);
+                uint8_t bits = (uint8_t)((combined >> (10 - bit_offset)) & 0x3F);
+                float val = scale * rf_decode_e2m3(bits);
+                out[idx] = clampf(val, -7.5f, 7.5f);
+            }
+        }
+    }
+}
+
+/* GgufTensorType ids, src/loader/tensor_type.rs:16-32 */
+enum { RF_F32 = 0, RF_F16 = 1, RF_Q4_0 = 2, RF_Q8_0 = 8, RF_Q4_K = 12, RF_Q6_K = 14,
+       RF_MXFP4 = 20, RF_MXFP6_E2M3 = 21, RF_MXFP6_E3M2 = 22 };
+
+/* GgufTensor::data_size, src/loader/gguf_tensor.rs:41-75 (Q4_0 is sized
+ * 36 bytes per block there although the decoder strides 20). */
+RF_API size_t rf_data_size(int type, size_t n)
+{
+    switch (type) {
+    case RF_F32: return n * 4;
+    case RF_F16: return n * 2;
+    case RF_Q4_0: return ((n + 31) / 32) * 36;
+    case RF_Q8_0: return ((n + 31) / 32) * 36;
+    case 10: case 11: case RF_Q4_K: case 13: case RF_Q6_K: return ((n + 255) / 256) * 256;
+    case RF_MXFP4: return ((n + 31) / 32) * 17;
+    case RF_MXFP6_E2M3: case RF_MXFP6_E3M2: return ((n + 31) / 32) * 25;
+    default: return 0;
+    }
+}
+
+/* Bytes per block that the DECODERS stride by (q4_0.rs:269, q8_0.rs:33,
+ * q4_k.rs:206, q6_k.rs:206, dequant.rs:47,91). */
+RF_API size_t rf_block_bytes(int type)
+{
+    switch (type) {
+    case RF_Q4_0: return 20;
+    case RF_Q8_0: return 36;
+    case RF_Q4_K: case RF_Q6_K: return 256;
+    case RF_MXFP4: return 17;
+    case RF_MXFP6_E2M3: case RF_MXFP6_E3M2: return 25;
+    default: return 0;
+    }
+}
+
+/* loader::dequantize dispatcher, src/loader/dequant.rs:673-700 (the formats
+ * on this path).  Returns 0 on success, -1 for a type outside the path. */
+RF_API int rf_dequantize(int type, const uint8_t *data, size_t len, size_t n, float *out)
+{
+    switch (type) {
+    case RF_F32:
+        for (size_t i = 0; i < n && i * 4 + 4 <= len; i++) out[i] = rd_f32le(data + 4 * i);
+        return 0;
+    case RF_F16:
+        for (size_t i = 0; i < n && i * 2 + 2 <= len; i++)
+            out[i] = rf_f16_to_f32((uint16_t)(data[2 * i] | (data[2 * i + 1] << 8)));
+        return 0;
+    case RF_Q4_0: rf_dequant_q4_0(data, len, n, out); return 0;
+    case RF_Q8_0: rf_dequant_q8_0(data, len, n, out); return 0;
+    case RF_Q4_K: rf_dequant_q4_k(data, len, n, out); return 0;
+    case RF_Q6_K: rf_dequant_q6_k(data, len, n, out); return 0;
+    case RF_MXFP4: rf_dequant_mxfp4(data, len, n, out); return 0;
+    case RF_MXFP6_E2M3:
+    case RF_MXFP6_E3M2: rf_dequant_mxfp6(data, len, n, out); return 0;
+    default: return -1;
+    }
+}
+
+/* ------------------------------------------------------------------ */
+/* matmul                                                              */
+/* ------------------------------------------------------------------ */
+
+/* cpu_matmul_f32, src/tensor/matmul.rs:219-233: a[m,k] . b[k,n], each output
+ * a sequential fp32 sum over l ascending, product rounded before the add. */
+RF_API void rf_cpu_matmul_f32(const float *a, const float *b, size_t m, size_t n, size_t k, float *c)
+{
+    for (size_t i = 0; i < m; i++) {
+        for (size_t j = 0; j < n; j++) {
+            float sum = 0.0f;
+            for (size_t l = 0; l < k; l++) sum += a[i * k + l] * b[l * n + j];
+            c[i * n + j] = sum;
+        }
+    }
+}
+
+/* Same arithmetic with the weight matrix stored [n,k] (rows of K, the layout
+ * matmul_q4_0's doc comment states, src/kernels/matmul/quantized/q4_0.rs:139-148):
+ * c[i,j] = sum_{l ascending} a[i,l] * w[j,l].  Per-output summation order and
+ * rounding are identical to rf_cpu_matmul_f32 on w transposed; rows of the
+ * output are spread over OpenMP threads, which does not change any value. */
+RF_API void rf_matmul_nk_f32(const float *a, const float *w, size_t m, size_t n, size_t k, float *c)
+{
+#pragma omp parallel for schedule(static)
+    for (long j = 0; j < (long)n; j++) {
+        const float *wr = w + (size_t)j * k;
+        for (size_t i = 0; i < m; i++) {
+            const float *ar = a + i * k;
+            float sum = 0.0f;
+            for (size_t l = 0; l < k; l++) sum += ar[l] * wr[l];
+            c[i * n + (size_t)j] = sum;
+        }
+    }
+}
+
+/* Quantised matmul as the reference's CPU path composes it
+ * (matmul_q4_0_cpu_fallback, src/kernels/matmul/quantized/q4_0.rs:274-311;
+ * benches/matmul_bench.rs:360-365): dequantise every weight to f32, then the
+ * naive matmul.  Weights [n,k] row-major, blocks along k, row r starting at
+ * byte r * (k / block_elems) * block_bytes.  scratch_row: k floats per thread
+ * are allocated internally.  rows_sel (optional): only these output columns
+ * are computed (c is then [m, n_sel]); pass NULL for all. */
+RF_API int rf_qmatmul_nk(int type, const uint8_t *w, size_t w_len, const float *a, size_t m, size_t n,
+                         size_t k, const int64_t *rows_sel, size_t n_sel, float *c)
+{
+    size_t bb = rf_block_bytes(type);
+    size_t be = (type == RF_Q4_K || type == RF_Q6_K) ? 256 : 32;
+    if (bb == 0 || k % be != 0) return -1;
+    size_t row_bytes = (k / be) * bb;
+    if (w_len < row_bytes * n) return -2;
+    size_t nout = rows_sel ? n_sel : n;
+    int rc = 0;
+#pragma omp parallel
+    {
+        float *wr = (float *)__builtin_malloc(k * sizeof(float));
+#pragma omp for schedule(static)
+        for (long jj = 0; jj < (long)nout; jj++) {
+            size_t j = rows_sel ? (size_t)rows_sel[jj] : (size_t)jj;
+            if (!wr || j >= n) { rc = -3; continue; }
+            rf_dequantize(type, w + j * row_bytes, row_bytes, k, wr);
+            for (size_t i = 0; i < m; i++) {
+                const float *ar = a + i * k;
+                float sum = 0.0f;
+                for (size_t l = 0; l < k; l++) sum += ar[l] * wr[l];
+                c[i * nout + (size_t)jj] = sum;
+            }
+        }
+        __builtin_free(wr);
+    }
+    return rc;
+}
+
+/* Single-threaded twin of the above used for the timed CPU baseline: full
+ * dequantise of the weight tensor into wd[n*k] (as dequantize_q4_0 does in
+ * the reference), then rf_matmul_nk_f32 restricted to one thread by the
+ * caller (omp_set_num_threads).  Kept separate so the baseline times exactly
+ * the two reference stages. */
+RF_API int rf_qmatmul_nk_staged(int type, const uint8_t *w, size_t w_len, const float *a, size_t m,
+                                size_t n, size_t k, float *wd, float *c)
+{
+    int r = rf_dequantize(type, w, w_len, n * k, wd);
+    if (r) return r;
+    rf_matmul_nk_f32(a, wd, m, n, k, c);
+    return 0;
+}

@@ -1,0 +1,71 @@
+"""ctypes binding of librfq.so.  There is no fallback: if the library has not
+been built, importing a symbol raises."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "librfq.so")
+
+OK, E_BADARG, E_SIZE, E_UNSUPPORTED, E_HIP, E_NOMEM = 0, -1, -2, -3, -4, -5
+F32, F16, BF16 = 0, 1, 2
+MX_AUTO, MX_FP4, MX_FP8 = 0, 4, 8
+
+
+class RfqError(RuntimeError):
+    def __init__(self, status: int, message: str):
+        super().__init__(f"rfq status {status}: {message}")
+        self.status = status
+        self.message = message
+
+
+def lib_path() -> str:
+    return _SO
+
+
+_lib = None
+
+_vp, _sz, _i = C.c_void_p, C.c_size_t, C.c_int
+_SIGNATURES = {
+    "rfq_version": ([], _i),
+    "rfq_last_error": ([], C.c_char_p),
+    "rfq_block_elems": ([_i], _sz),
+    "rfq_block_bytes": ([_i], _sz),
+    "rfq_packed_bytes": ([_i, _sz], _sz),
+    "rfq_dequant": ([_i, _vp, _sz, _vp, _sz, _vp], _i),
+    "rfq_dequant_upload": ([_i, _vp, _sz, _vp, _sz, _vp], _i),
+    "rfq_dequant_host": ([_i, _vp, _sz, _vp, _sz], _i),
+    "rfq_gemv": ([_i, _vp, _sz, _vp, _vp, _i, _i, _i, _vp], _i),
+    "rfq_matmul_q4_0": ([_vp, _vp, _vp, _i, _i, _i, _vp], _i),
+    "rfq_matmul_q8_0": ([_vp, _vp, _vp, _i, _i, _i, _vp], _i),
+    "rfq_matmul_q4_k": ([_vp, _vp, _vp, _i, _i, _i, _vp], _i),
+    "rfq_matmul_q6_k": ([_vp, _vp, _vp, _i, _i, _i, _vp], _i),
+    "rfq_matmul_host_weights": ([_i, _vp, _sz, _vp, _sz, _sz, _vp, _vp], _i),
+    "rfq_gemm_f16": ([_i, _vp, _sz, _vp, _vp, _i, _i, _i, _i, _vp], _i),
+    "rfq_mx_prepared_bytes": ([_i, _i, _i, _i], _sz),
+    "rfq_mx_prepare": ([_i, _i, _vp, _sz, _i, _i, _vp, _sz, C.POINTER(C.c_int), _vp], _i),
+    "rfq_gemm_mx": ([_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _vp], _i),
+}
+
+
+def lib() -> C.CDLL:
+    """The loaded library; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_SO):
+            raise FileNotFoundError(
+                f"{_SO} is missing: build it with `make -C rocmforge_amd/csrc` "
+                "(or __graft_entry__.build()); there is no CPU fallback")
+        L = C.CDLL(_SO)
+        for name, (args, res) in _SIGNATURES.items():
+            fn = getattr(L, name)
+            fn.argtypes = args
+            fn.restype = res
+        _lib = L
+    return _lib
+
+
+def check(status: int) -> None:
+    if status != OK:
+        raise RfqError(status, lib().rfq_last_error().decode("utf-8", "replace"))

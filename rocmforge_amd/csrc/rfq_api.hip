@@ -1,0 +1,242 @@
+// C ABI entry points of librfq: argument validation on the host, then one
+// launcher per operation.  No kernel is launched before its operand sizes have
+// been checked against what the kernel and its grid assume.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <mutex>
+
+#include "rfq_common.hpp"
+
+namespace rfq {
+
+static thread_local char g_err[512] = "";
+
+int fail(int status, const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof g_err, fmt, ap);
+    va_end(ap);
+    return status;
+}
+
+int hip_fail(hipError_t e, const char *what)
+{
+    snprintf(g_err, sizeof g_err, "%s: %s", what, hipGetErrorString(e));
+    return e == hipErrorOutOfMemory ? RFQ_E_NOMEM : RFQ_E_HIP;
+}
+
+int device_cu_count()
+{
+    // One value per device id; devices are few, so a small fixed table.
+    static int cus[64];
+    static std::mutex mu;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    std::lock_guard<std::mutex> lock(mu);
+    if (cus[dev] == 0) {
+        int v = 0;
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) v = 256;
+        cus[dev] = v;
+    }
+    return cus[dev];
+}
+
+static bool known_format(int fmt) { return fmt_block_elems(fmt) != 0; }
+
+// Weight bytes of an [n, k] matrix, or 0 if k does not divide into blocks.
+static size_t matrix_bytes(int fmt, int n, int k)
+{
+    int be = fmt_block_elems(fmt);
+    if (be == 0 || k % be != 0) return 0;
+    return (size_t)n * (size_t)(k / be) * (size_t)fmt_block_bytes(fmt);
+}
+
+static int check_gemv(const char *who, int fmt, const void *w, size_t w_bytes, bool have_bytes, const void *x,
+                      const void *y, int m, int n, int k)
+{
+    if (!known_format(fmt)) return fail(RFQ_E_BADARG, "%s: unknown format %d", who, fmt);
+    if (!w || !x || !y) return fail(RFQ_E_BADARG, "%s: null pointer", who);
+    if (m <= 0 || n <= 0 || k <= 0)
+        return fail(RFQ_E_BADARG, "%s: dimensions must be positive (m=%d n=%d k=%d)", who, m, n, k);
+    size_t need = matrix_bytes(fmt, n, k);
+    if (need == 0)
+        return fail(RFQ_E_SIZE, "%s: k=%d is not a multiple of the %d-element block", who, k, fmt_block_elems(fmt));
+    if (have_bytes && w_bytes != need)
+        return fail(RFQ_E_SIZE, "%s: weight buffer has %zu bytes, [%d x %d] needs %zu", who, w_bytes, n, k, need);
+    return RFQ_OK;
+}
+
+} // namespace rfq
+
+using namespace rfq;
+
+extern "C" {
+
+int rfq_version(void) { return RFQ_VERSION; }
+
+const char *rfq_last_error(void) { return g_err; }
+
+size_t rfq_block_elems(int fmt) { return (size_t)fmt_block_elems(fmt); }
+size_t rfq_block_bytes(int fmt) { return (size_t)fmt_block_bytes(fmt); }
+
+size_t rfq_packed_bytes(int fmt, size_t n_elems)
+{
+    size_t be = (size_t)fmt_block_elems(fmt);
+    if (be == 0) return 0;
+    return ((n_elems + be - 1) / be) * (size_t)fmt_block_bytes(fmt);
+}
+
+int rfq_dequant(int fmt, const void *d_packed, size_t packed_bytes, float *d_out, size_t n_elems, void *stream)
+{
+    if (!known_format(fmt)) return fail(RFQ_E_BADARG, "rfq_dequant: unknown format %d", fmt);
+    if (n_elems == 0) return RFQ_OK;
+    if (!d_out) return fail(RFQ_E_BADARG, "rfq_dequant: null output");
+    if (!d_packed && packed_bytes) return fail(RFQ_E_BADARG, "rfq_dequant: null input with %zu bytes", packed_bytes);
+    return launch_dequant(fmt, (const uint8_t *)d_packed, packed_bytes, d_out, n_elems, (hipStream_t)stream);
+}
+
+int rfq_dequant_upload(int fmt, const uint8_t *h_packed, size_t packed_bytes, float *d_out, size_t n_elems,
+                       void *stream)
+{
+    if (!known_format(fmt)) return fail(RFQ_E_BADARG, "rfq_dequant_upload: unknown format %d", fmt);
+    if (n_elems == 0) return RFQ_OK;
+    if (!d_out) return fail(RFQ_E_BADARG, "rfq_dequant_upload: null output");
+    if (!h_packed && packed_bytes) return fail(RFQ_E_BADARG, "rfq_dequant_upload: null input");
+    hipStream_t s = (hipStream_t)stream;
+    // Only the bytes the decoder can reach are uploaded.
+    size_t need = rfq_packed_bytes(fmt, n_elems);
+    size_t bytes = packed_bytes < need ? packed_bytes : need;
+    void *d_in = nullptr;
+    if (bytes) {
+        RFQ_HIP(hipMalloc(&d_in, bytes));
+        hipError_t e = hipMemcpyAsync(d_in, h_packed, bytes, hipMemcpyHostToDevice, s);
+        if (e != hipSuccess) { (void)hipFree(d_in); return hip_fail(e, "hipMemcpyAsync(H2D)"); }
+    }
+    int rc = launch_dequant(fmt, (const uint8_t *)d_in, bytes, d_out, n_elems, s);
+    hipError_t e = hipStreamSynchronize(s);
+    if (d_in) (void)hipFree(d_in);
+    if (rc != RFQ_OK) return rc;
+    if (e != hipSuccess) return hip_fail(e, "hipStreamSynchronize");
+    return RFQ_OK;
+}
+
+int rfq_dequant_host(int fmt, const uint8_t *h_packed, size_t packed_bytes, float *h_out, size_t n_elems)
+{
+    if (!known_format(fmt)) return fail(RFQ_E_BADARG, "rfq_dequant_host: unknown format %d", fmt);
+    if (n_elems == 0) return RFQ_OK;
+    if (!h_out) return fail(RFQ_E_BADARG, "rfq_dequant_host: null output");
+    float *d_out = nullptr;
+    RFQ_HIP(hipMalloc((void **)&d_out, n_elems * sizeof(float)));
+    int rc = rfq_dequant_upload(fmt, h_packed, packed_bytes, d_out, n_elems, nullptr);
+    if (rc == RFQ_OK) {
+        hipError_t e = hipMemcpy(h_out, d_out, n_elems * sizeof(float), hipMemcpyDeviceToHost);
+        if (e != hipSuccess) rc = hip_fail(e, "hipMemcpy(D2H)");
+    }
+    (void)hipFree(d_out);
+    return rc;
+}
+
+int rfq_gemv(int fmt, const void *d_w, size_t w_bytes, const float *d_x, float *d_y, int m, int n, int k,
+             void *stream)
+{
+    int rc = check_gemv("rfq_gemv", fmt, d_w, w_bytes, true, d_x, d_y, m, n, k);
+    if (rc != RFQ_OK) return rc;
+    if (m > 8) return fail(RFQ_E_UNSUPPORTED, "rfq_gemv: m=%d > 8; use rfq_gemm_f16 for prefill", m);
+    return launch_gemv(fmt, (const uint8_t *)d_w, d_x, d_y, m, n, k, (hipStream_t)stream);
+}
+
+static int matmul_raw(const char *who, int fmt, const float *d_act, const uint8_t *d_w, float *d_out, int m, int n,
+                      int k, void *stream)
+{
+    int rc = check_gemv(who, fmt, d_w, 0, false, d_act, d_out, m, n, k);
+    if (rc != RFQ_OK) return rc;
+    if (m > 8) return fail(RFQ_E_UNSUPPORTED, "%s: m=%d > 8; use rfq_gemm_f16 for prefill", who, m);
+    return launch_gemv(fmt, d_w, d_act, d_out, m, n, k, (hipStream_t)stream);
+}
+
+int rfq_matmul_q4_0(const float *a, const uint8_t *w, float *o, int m, int n, int k, void *s)
+{
+    return matmul_raw("rfq_matmul_q4_0", RFQ_Q4_0, a, w, o, m, n, k, s);
+}
+int rfq_matmul_q8_0(const float *a, const uint8_t *w, float *o, int m, int n, int k, void *s)
+{
+    return matmul_raw("rfq_matmul_q8_0", RFQ_Q8_0, a, w, o, m, n, k, s);
+}
+int rfq_matmul_q4_k(const float *a, const uint8_t *w, float *o, int m, int n, int k, void *s)
+{
+    return matmul_raw("rfq_matmul_q4_k", RFQ_Q4_K, a, w, o, m, n, k, s);
+}
+int rfq_matmul_q6_k(const float *a, const uint8_t *w, float *o, int m, int n, int k, void *s)
+{
+    return matmul_raw("rfq_matmul_q6_k", RFQ_Q6_K, a, w, o, m, n, k, s);
+}
+
+int rfq_matmul_host_weights(int fmt, const uint8_t *h_w, size_t w_bytes, const float *d_input, size_t n_rows,
+                            size_t n_cols, float *d_out, void *stream)
+{
+    if (n_rows == 0 || n_cols == 0 || n_rows > 0x7fffffffu || n_cols > 0x7fffffffu)
+        return fail(RFQ_E_BADARG, "rfq_matmul_host_weights: bad shape %zu x %zu", n_rows, n_cols);
+    int rc = check_gemv("rfq_matmul_host_weights", fmt, h_w, w_bytes, true, d_input, d_out, 1, (int)n_rows, (int)n_cols);
+    if (rc != RFQ_OK) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    void *d_w = nullptr;
+    RFQ_HIP(hipMalloc(&d_w, w_bytes));
+    hipError_t e = hipMemcpyAsync(d_w, h_w, w_bytes, hipMemcpyHostToDevice, s);
+    if (e != hipSuccess) { (void)hipFree(d_w); return hip_fail(e, "hipMemcpyAsync(H2D)"); }
+    rc = launch_gemv(fmt, (const uint8_t *)d_w, d_input, d_out, 1, (int)n_rows, (int)n_cols, s);
+    e = hipStreamSynchronize(s);
+    (void)hipFree(d_w);
+    if (rc != RFQ_OK) return rc;
+    if (e != hipSuccess) return hip_fail(e, "hipStreamSynchronize");
+    return RFQ_OK;
+}
+
+int rfq_gemm_f16(int fmt, const void *d_w, size_t w_bytes, const void *d_a_f16, void *d_out, int out_dtype, int m,
+                 int n, int k, void *stream)
+{
+    int rc = check_gemv("rfq_gemm_f16", fmt, d_w, w_bytes, true, d_a_f16, d_out, m, n, k);
+    if (rc != RFQ_OK) return rc;
+    if (out_dtype != RFQ_F32 && out_dtype != RFQ_F16)
+        return fail(RFQ_E_BADARG, "rfq_gemm_f16: out_dtype %d is neither F32 nor F16", out_dtype);
+    return launch_gemm_f16(fmt, (const uint8_t *)d_w, d_a_f16, d_out, out_dtype, m, n, k, (hipStream_t)stream);
+}
+
+size_t rfq_mx_prepared_bytes(int fmt, int kind, int rows, int k)
+{
+    return mx_prepared_bytes(fmt, kind, rows, k);
+}
+
+int rfq_mx_prepare(int fmt, int kind_req, const void *d_raw, size_t raw_bytes, int rows, int k, void *d_prepared,
+                   size_t prepared_bytes, int *kind_out, void *stream)
+{
+    if (fmt != RFQ_MXFP4 && fmt != RFQ_MXFP6_E2M3 && fmt != RFQ_MXFP6_E3M2)
+        return fail(RFQ_E_BADARG, "rfq_mx_prepare: format %d is not an MXFP format", fmt);
+    if (!d_raw || !d_prepared) return fail(RFQ_E_BADARG, "rfq_mx_prepare: null pointer");
+    if (rows <= 0 || k <= 0) return fail(RFQ_E_BADARG, "rfq_mx_prepare: bad shape %d x %d", rows, k);
+    if (k % 128 != 0) return fail(RFQ_E_SIZE, "rfq_mx_prepare: k=%d is not a multiple of 128", k);
+    if (kind_req != RFQ_MX_AUTO && kind_req != RFQ_MX_FP4 && kind_req != RFQ_MX_FP8)
+        return fail(RFQ_E_BADARG, "rfq_mx_prepare: unknown kind %d", kind_req);
+    size_t need = matrix_bytes(fmt, rows, k);
+    if (raw_bytes != need)
+        return fail(RFQ_E_SIZE, "rfq_mx_prepare: raw buffer has %zu bytes, [%d x %d] needs %zu", raw_bytes, rows, k, need);
+    return launch_mx_prepare(fmt, kind_req, (const uint8_t *)d_raw, rows, k, d_prepared, prepared_bytes, kind_out,
+                             (hipStream_t)stream);
+}
+
+int rfq_gemm_mx(const void *d_a_prep, int a_kind, const void *d_w_prep, int w_kind, void *d_out, int out_dtype, int m,
+                int n, int k, void *stream)
+{
+    if (!d_a_prep || !d_w_prep || !d_out) return fail(RFQ_E_BADARG, "rfq_gemm_mx: null pointer");
+    if (m <= 0 || n <= 0 || k <= 0) return fail(RFQ_E_BADARG, "rfq_gemm_mx: bad shape m=%d n=%d k=%d", m, n, k);
+    if (k % 128 != 0) return fail(RFQ_E_SIZE, "rfq_gemm_mx: k=%d is not a multiple of 128", k);
+    if ((a_kind != RFQ_MX_FP4 && a_kind != RFQ_MX_FP8) || (w_kind != RFQ_MX_FP4 && w_kind != RFQ_MX_FP8))
+        return fail(RFQ_E_BADARG, "rfq_gemm_mx: operand kinds must be FP4 or FP8 (a=%d w=%d)", a_kind, w_kind);
+    if (out_dtype != RFQ_F32 && out_dtype != RFQ_BF16)
+        return fail(RFQ_E_BADARG, "rfq_gemm_mx: out_dtype %d is neither F32 nor BF16", out_dtype);
+    return launch_gemm_mx(d_a_prep, a_kind, d_w_prep, w_kind, d_out, out_dtype, m, n, k, (hipStream_t)stream);
+}
+
+} // extern "C"

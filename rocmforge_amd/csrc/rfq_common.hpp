@@ -1,0 +1,124 @@
+// Shared declarations for librfq (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "rfq.h"
+
+namespace rfq {
+
+// ---- format traits ---------------------------------------------------------
+template <int FMT> struct Fmt;
+template <> struct Fmt<RFQ_Q4_0> { static constexpr int BE = 32, BB = 20; };
+template <> struct Fmt<RFQ_Q8_0> { static constexpr int BE = 32, BB = 36; };
+template <> struct Fmt<RFQ_Q4_K> { static constexpr int BE = 256, BB = 256; };
+template <> struct Fmt<RFQ_Q6_K> { static constexpr int BE = 256, BB = 256; };
+template <> struct Fmt<RFQ_MXFP4> { static constexpr int BE = 32, BB = 17; };
+template <> struct Fmt<RFQ_MXFP6_E2M3> { static constexpr int BE = 32, BB = 25; };
+
+// MXFP6_E3M2 is decoded exactly like E2M3 by the reference
+// (src/loader/dequant.rs:693), so it shares every kernel.
+inline int canonical_format(int fmt) { return fmt == RFQ_MXFP6_E3M2 ? RFQ_MXFP6_E2M3 : fmt; }
+
+inline int fmt_block_elems(int fmt)
+{
+    switch (fmt) {
+    case RFQ_Q4_0: case RFQ_Q8_0: case RFQ_MXFP4: case RFQ_MXFP6_E2M3: case RFQ_MXFP6_E3M2: return 32;
+    case RFQ_Q4_K: case RFQ_Q6_K: return 256;
+    default: return 0;
+    }
+}
+inline int fmt_block_bytes(int fmt)
+{
+    switch (fmt) {
+    case RFQ_Q4_0: return 20;
+    case RFQ_Q8_0: return 36;
+    case RFQ_Q4_K: case RFQ_Q6_K: return 256;
+    case RFQ_MXFP4: return 17;
+    case RFQ_MXFP6_E2M3: case RFQ_MXFP6_E3M2: return 25;
+    default: return 0;
+    }
+}
+
+// ---- error plumbing (rfq_api.hip) ------------------------------------------
+int fail(int status, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+int hip_fail(hipError_t e, const char *what);
+#define RFQ_HIP(call)                                              \
+    do {                                                           \
+        hipError_t e_ = (call);                                    \
+        if (e_ != hipSuccess) return ::rfq::hip_fail(e_, #call);   \
+    } while (0)
+// Kernel launches report through hipGetLastError.
+#define RFQ_LAUNCH_CHECK(what)                                     \
+    do {                                                           \
+        hipError_t e_ = hipGetLastError();                         \
+        if (e_ != hipSuccess) return ::rfq::hip_fail(e_, what);    \
+    } while (0)
+
+int device_cu_count();
+
+// ---- launchers implemented per .hip file -----------------------------------
+int launch_dequant(int fmt, const uint8_t *d_in, size_t in_bytes, float *d_out, size_t n, hipStream_t s);
+int launch_gemv(int fmt, const uint8_t *d_w, const float *d_x, float *d_y, int m, int n, int k, hipStream_t s);
+int launch_gemm_f16(int fmt, const uint8_t *d_w, const void *d_a, void *d_out, int out_dtype, int m, int n,
+                    int k, hipStream_t s);
+size_t mx_prepared_bytes(int fmt, int kind, int rows, int k);
+int launch_mx_prepare(int fmt, int kind_req, const uint8_t *d_raw, int rows, int k, void *d_prep,
+                      size_t prep_bytes, int *kind_out, hipStream_t s);
+int launch_gemm_mx(const void *d_a, int a_kind, const void *d_w, int w_kind, void *d_out, int out_dtype, int m,
+                   int n, int k, hipStream_t s);
+
+#if defined(__HIPCC__)
+// ---- device-side decode helpers ---------------------------------------------
+
+// Loads that make no alignment promise (gfx950 global memory accepts any
+// byte address for dword..dwordx4 accesses).
+template <typename T> __device__ __forceinline__ T ld(const uint8_t *p)
+{
+    T v;
+    __builtin_memcpy(&v, p, sizeof(T));
+    return v;
+}
+
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t h)
+{
+    _Float16 v;
+    __builtin_memcpy(&v, &h, 2);
+    return (float)v; // exact widening, subnormals kept
+}
+
+// 2^e for the MXFP exponent byte read as i8, reproducing f32::powi(2.0, e):
+// exact for -127..127 (2^-127 is subnormal), 0.0 for -128 (the repeated
+// squaring overflows and the reciprocal of +inf is taken).
+__device__ __forceinline__ float mx_scale(int e)
+{
+    uint32_t bits = e >= -126 ? (uint32_t)(e + 127) << 23 : (e == -127 ? 0x00400000u : 0u);
+    return __uint_as_float(bits);
+}
+
+// MxfpBlock::decode_e2m1 (src/loader/mxfp.rs:234-244): 0 for code 0, otherwise
+// sign * (1 + mant) * 2^(exp-1)  ==  +-2^(((code&7)+1)/2 - 1).
+__device__ __forceinline__ float decode_e2m1(uint32_t q)
+{
+    uint32_t c = q & 7u;
+    uint32_t bits = ((q & 8u) << 28) | ((126u + ((c + 1u) >> 1)) << 23);
+    return q == 0u ? 0.0f : __uint_as_float(bits);
+}
+
+// MxfpBlock::decode_e2m3 (src/loader/mxfp.rs:283-293): 0 for code 0, otherwise
+// sign * (1 + mant/8) * 2^(exp-1); the fields map straight onto an f32.
+__device__ __forceinline__ float decode_e2m3(uint32_t q)
+{
+    uint32_t bits = ((q & 32u) << 26) | ((126u + ((q >> 3) & 3u)) << 23) | ((q & 7u) << 20);
+    return q == 0u ? 0.0f : __uint_as_float(bits);
+}
+
+// f32::clamp for finite bounds.
+__device__ __forceinline__ float clampf(float v, float lo, float hi) { return fminf(fmaxf(v, lo), hi); }
+
+// Signed 6-bit field (two's complement) starting at bit `off` of w.
+__device__ __forceinline__ int sbfe6(uint32_t w, uint32_t off) { return ((int)(w << (26u - off))) >> 26; }
+#endif
+
+} // namespace rfq

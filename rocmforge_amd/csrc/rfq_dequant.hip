@@ -1,0 +1,246 @@
+// Block dequantisation kernels, bit-exact with ROCmForge's CPU decoders.
+//
+// These kernels are bound by the f32 write stream (4 B out for 0.53-1.13 B in),
+// so the mapping is chosen for the stores: one thread decodes 4 consecutive
+// elements and issues one 16-byte store; a wavefront writes 1 KiB contiguous.
+// Whole blocks go through the fast kernel; anything ragged (element count not
+// a multiple of the block, or fewer bytes than the shape needs) goes through a
+// bounds-checked per-element kernel that follows the CPU loops' early exits.
+//
+// Compiled with -ffp-contract=off so no multiply-add is fused (the reference
+// never fuses).
+#include "rfq_common.hpp"
+
+namespace rfq {
+namespace {
+
+// ---- 4 consecutive elements e0..e0+3 (e0 % 4 == 0) of one whole block -------
+
+template <int FMT> __device__ __forceinline__ float4 decode_quad(const uint8_t *blk, int e0);
+
+// src/kernels/quant/q4_0.rs:289-306
+template <> __device__ __forceinline__ float4 decode_quad<RFQ_Q4_0>(const uint8_t *blk, int e0)
+{
+    float scale = ld<float>(blk);
+    uint32_t w = ld<uint16_t>(blk + 4 + (e0 >> 1));
+    float4 r;
+    r.x = scale * (float)((int)(w & 15u) - 8);
+    r.y = scale * (float)((int)((w >> 4) & 15u) - 8);
+    r.z = scale * (float)((int)((w >> 8) & 15u) - 8);
+    r.w = scale * (float)((int)((w >> 12) & 15u) - 8);
+    return r;
+}
+
+// src/kernels/quant/q8_0.rs:55-59
+template <> __device__ __forceinline__ float4 decode_quad<RFQ_Q8_0>(const uint8_t *blk, int e0)
+{
+    float scale = ld<float>(blk);
+    uint32_t w = ld<uint32_t>(blk + 4 + e0);
+    float4 r;
+    r.x = ((float)(w & 255u) - 128.0f) * scale;
+    r.y = ((float)((w >> 8) & 255u) - 128.0f) * scale;
+    r.z = ((float)((w >> 16) & 255u) - 128.0f) * scale;
+    r.w = ((float)(w >> 24) - 128.0f) * scale;
+    return r;
+}
+
+// src/kernels/quant/q4_k.rs:222-268
+template <> __device__ __forceinline__ float4 decode_quad<RFQ_Q4_K>(const uint8_t *blk, int e0)
+{
+    int sb = e0 >> 5, i = e0 & 31;
+    float scale = f16_bits_to_f32(ld<uint16_t>(blk + 2 * sb));
+    float mn = (float)(int8_t)blk[16 + sb];
+    uint32_t w = ld<uint16_t>(blk + 32 + 28 * sb + (i >> 1));
+    float4 r;
+    r.x = mn + (float)(w & 15u) * scale;
+    r.y = mn + (float)((w >> 4) & 15u) * scale;
+    r.z = mn + (float)((w >> 8) & 15u) * scale;
+    r.w = mn + (float)((w >> 12) & 15u) * scale;
+    return r;
+}
+
+// src/kernels/quant/q6_k.rs:221-261: element i sits at bit 6*i of the stream
+// at +32, so four elements starting at a multiple of 4 are exactly 3 bytes.
+template <> __device__ __forceinline__ float4 decode_quad<RFQ_Q6_K>(const uint8_t *blk, int e0)
+{
+    float scale = f16_bits_to_f32(ld<uint16_t>(blk + 2 * (e0 >> 4)));
+    const uint8_t *p = blk + 32 + 3 * (e0 >> 2);
+    uint32_t w = (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16);
+    float4 r;
+    r.x = (float)sbfe6(w, 0) * scale;
+    r.y = (float)sbfe6(w, 6) * scale;
+    r.z = (float)sbfe6(w, 12) * scale;
+    r.w = (float)sbfe6(w, 18) * scale;
+    return r;
+}
+
+// src/loader/dequant.rs:53-77: element 2j is the HIGH nibble of byte j.
+template <> __device__ __forceinline__ float4 decode_quad<RFQ_MXFP4>(const uint8_t *blk, int e0)
+{
+    float scale = mx_scale((int)(int8_t)blk[0]);
+    uint32_t w = ld<uint16_t>(blk + 1 + (e0 >> 1));
+    float4 r;
+    r.x = clampf(scale * decode_e2m1((w >> 4) & 15u), -8.0f, 8.0f);
+    r.y = clampf(scale * decode_e2m1(w & 15u), -8.0f, 8.0f);
+    r.z = clampf(scale * decode_e2m1((w >> 12) & 15u), -8.0f, 8.0f);
+    r.w = clampf(scale * decode_e2m1((w >> 8) & 15u), -8.0f, 8.0f);
+    return r;
+}
+
+// src/loader/dequant.rs:107-127.  With b = the 24 packed bytes and j = e0/4,
+// "(u16le[b + (6i)/8] >> (10 - (6i)%8)) & 63" reduces to
+//   i=4j  : b[3j+1] >> 2
+//   i=4j+1: (b[3j] >> 4) | ((b[3j+1] & 3) << 4)
+//   i=4j+2: (b[3j+1] >> 6) | ((b[3j+2] & 15) << 2)
+//   i=4j+3: b[3j+3] & 63, which needs byte 24 for j = 7: the reference skips
+//           that element, it stays 0.0.
+template <> __device__ __forceinline__ float4 decode_quad<RFQ_MXFP6_E2M3>(const uint8_t *blk, int e0)
+{
+    float scale = mx_scale((int)(int8_t)blk[0]);
+    int j = e0 >> 2;
+    const uint8_t *b = blk + 1 + 3 * j;
+    uint32_t b0 = b[0], b1 = b[1], b2 = b[2];
+    float4 r;
+    r.x = clampf(scale * decode_e2m3(b1 >> 2), -7.5f, 7.5f);
+    r.y = clampf(scale * decode_e2m3((b0 >> 4) | ((b1 & 3u) << 4)), -7.5f, 7.5f);
+    r.z = clampf(scale * decode_e2m3((b1 >> 6) | ((b2 & 15u) << 2)), -7.5f, 7.5f);
+    r.w = 0.0f;
+    if (j < 7) r.w = clampf(scale * decode_e2m3((uint32_t)b[3] & 63u), -7.5f, 7.5f);
+    return r;
+}
+
+template <int FMT, bool ALIGNED16>
+__global__ void __launch_bounds__(256)
+dequant_blocks_kernel(const uint8_t *__restrict__ in, float *__restrict__ out, size_t n_quads)
+{
+    constexpr int QPB = Fmt<FMT>::BE / 4;
+    size_t t = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= n_quads) return;
+    size_t b = t / QPB;
+    int e0 = (int)(t % QPB) * 4;
+    float4 v = decode_quad<FMT>(in + b * Fmt<FMT>::BB, e0);
+    float *o = out + t * 4;
+    if (ALIGNED16) {
+        *reinterpret_cast<float4 *>(o) = v;
+    } else {
+        o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+    }
+}
+
+// ---- one element with the CPU loops' bounds behaviour ------------------------
+
+template <int FMT> __device__ float decode_checked(const uint8_t *in, size_t len, size_t idx);
+
+template <> __device__ float decode_checked<RFQ_Q4_0>(const uint8_t *in, size_t len, size_t idx)
+{
+    size_t off = (idx / 32) * 20;
+    if (off + 4 > len) return 0.0f;             // q4_0.rs:273-275
+    size_t e = idx % 32, p = off + 4 + e / 2;
+    if (p >= len) return 0.0f;                  // q4_0.rs:290-292
+    uint32_t q = (e & 1) ? (in[p] >> 4) : (in[p] & 15u);
+    return ld<float>(in + off) * (float)((int)q - 8);
+}
+
+template <> __device__ float decode_checked<RFQ_Q8_0>(const uint8_t *in, size_t len, size_t idx)
+{
+    size_t off = (idx / 32) * 36;
+    if (off + 4 > len) return 0.0f;             // q8_0.rs:35-37
+    size_t p = off + 4 + idx % 32;
+    if (p >= len) return 0.0f;                  // q8_0.rs:50-51
+    return ((float)in[p] - 128.0f) * ld<float>(in + off);
+}
+
+template <> __device__ float decode_checked<RFQ_Q4_K>(const uint8_t *in, size_t len, size_t idx)
+{
+    size_t off = (idx / 256) * 256;
+    if (off + 256 > len) return 0.0f;           // q4_k.rs:208-210
+    float4 v = decode_quad<RFQ_Q4_K>(in + off, (int)(idx % 256) & ~3);
+    int l = (int)(idx & 3);
+    return l == 0 ? v.x : l == 1 ? v.y : l == 2 ? v.z : v.w;
+}
+
+template <> __device__ float decode_checked<RFQ_Q6_K>(const uint8_t *in, size_t len, size_t idx)
+{
+    size_t off = (idx / 256) * 256;
+    if (off + 256 > len) return 0.0f;           // q6_k.rs:208-210
+    float4 v = decode_quad<RFQ_Q6_K>(in + off, (int)(idx % 256) & ~3);
+    int l = (int)(idx & 3);
+    return l == 0 ? v.x : l == 1 ? v.y : l == 2 ? v.z : v.w;
+}
+
+template <> __device__ float decode_checked<RFQ_MXFP4>(const uint8_t *in, size_t len, size_t idx)
+{
+    size_t off = (idx / 32) * 17;
+    if (off + 1 > len) return 0.0f;             // dequant.rs:49-51
+    size_t e = idx % 32, p = off + 1 + e / 2;
+    if (p >= len) return 0.0f;                  // dequant.rs:59-61
+    uint32_t q = (e & 1) ? (in[p] & 15u) : (in[p] >> 4);
+    return clampf(mx_scale((int)(int8_t)in[off]) * decode_e2m1(q), -8.0f, 8.0f);
+}
+
+template <> __device__ float decode_checked<RFQ_MXFP6_E2M3>(const uint8_t *in, size_t len, size_t idx)
+{
+    size_t off = (idx / 32) * 25;
+    if (off + 1 > len) return 0.0f;             // dequant.rs:93-95
+    size_t avail = len - (off + 1);
+    size_t plen = avail < 24 ? avail : 24;      // dequant.rs:102-104
+    size_t i = idx % 32;
+    uint32_t bit_offset = (uint32_t)((i * 6) % 8);
+    size_t bi = (i * 6) / 8;
+    if (bi + 1 >= plen) return 0.0f;            // dequant.rs:117
+    const uint8_t *pd = in + off + 1;
+    uint32_t combined = ((uint32_t)pd[bi + 1] << 8) | pd[bi];
+    uint32_t q = (combined >> (10u - bit_offset)) & 63u;
+    return clampf(mx_scale((int)(int8_t)in[off]) * decode_e2m3(q), -7.5f, 7.5f);
+}
+
+template <int FMT>
+__global__ void __launch_bounds__(256)
+dequant_checked_kernel(const uint8_t *__restrict__ in, size_t len, float *__restrict__ out, size_t first, size_t n)
+{
+    size_t idx = first + (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx < n) out[idx] = decode_checked<FMT>(in, len, idx);
+}
+
+template <int FMT>
+int run(const uint8_t *d_in, size_t in_bytes, float *d_out, size_t n, hipStream_t s)
+{
+    constexpr size_t BE = Fmt<FMT>::BE, BB = Fmt<FMT>::BB;
+    size_t full = n / BE;
+    if (in_bytes / BB < full) full = in_bytes / BB;
+    size_t n_quads = full * (BE / 4);
+    if (n_quads) {
+        size_t grid = (n_quads + 255) / 256;
+        if (grid > 0x7fffffffu) return fail(RFQ_E_SIZE, "rfq_dequant: %zu elements exceed one launch", n);
+        if ((reinterpret_cast<uintptr_t>(d_out) & 15u) == 0)
+            hipLaunchKernelGGL((dequant_blocks_kernel<FMT, true>), dim3((unsigned)grid), dim3(256), 0, s, d_in, d_out, n_quads);
+        else
+            hipLaunchKernelGGL((dequant_blocks_kernel<FMT, false>), dim3((unsigned)grid), dim3(256), 0, s, d_in, d_out, n_quads);
+        RFQ_LAUNCH_CHECK("dequant_blocks_kernel");
+    }
+    size_t first = full * BE;
+    if (first < n) {
+        size_t grid = (n - first + 255) / 256;
+        if (grid > 0x7fffffffu) return fail(RFQ_E_SIZE, "rfq_dequant: ragged tail of %zu elements exceeds one launch", n - first);
+        hipLaunchKernelGGL((dequant_checked_kernel<FMT>), dim3((unsigned)grid), dim3(256), 0, s, d_in, in_bytes, d_out, first, n);
+        RFQ_LAUNCH_CHECK("dequant_checked_kernel");
+    }
+    return RFQ_OK;
+}
+
+} // namespace
+
+int launch_dequant(int fmt, const uint8_t *d_in, size_t in_bytes, float *d_out, size_t n, hipStream_t s)
+{
+    switch (canonical_format(fmt)) {
+    case RFQ_Q4_0: return run<RFQ_Q4_0>(d_in, in_bytes, d_out, n, s);
+    case RFQ_Q8_0: return run<RFQ_Q8_0>(d_in, in_bytes, d_out, n, s);
+    case RFQ_Q4_K: return run<RFQ_Q4_K>(d_in, in_bytes, d_out, n, s);
+    case RFQ_Q6_K: return run<RFQ_Q6_K>(d_in, in_bytes, d_out, n, s);
+    case RFQ_MXFP4: return run<RFQ_MXFP4>(d_in, in_bytes, d_out, n, s);
+    case RFQ_MXFP6_E2M3: return run<RFQ_MXFP6_E2M3>(d_in, in_bytes, d_out, n, s);
+    default: return fail(RFQ_E_BADARG, "rfq_dequant: unknown format %d", fmt);
+    }
+}
+
+} // namespace rfq

@@ -1,0 +1,95 @@
+"""Device-side operators over torch tensors (torch is only the allocator and
+the stream here; every computation is a librfq call).
+
+Mirrors the raw-pointer layer of ROCmForge's kernel wrappers:
+``matmul_q4_0_gpu`` and twins (src/kernels/matmul/quantized/q4_0.rs:209-260)
+and the dequant launches (src/kernels/quant/q4_0.rs:107-153).
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import torch
+
+from . import _lib
+from ._lib import check, lib
+from .quantize import BLOCK_BYTES, BLOCK_ELEMS
+
+
+def _stream() -> C.c_void_p:
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t: torch.Tensor) -> C.c_void_p:
+    return C.c_void_p(t.data_ptr())
+
+
+def _dev_u8(t: torch.Tensor) -> torch.Tensor:
+    if not (t.is_cuda and t.dtype == torch.uint8 and t.is_contiguous()):
+        raise ValueError("packed weights must be a contiguous uint8 device tensor")
+    return t
+
+
+def dequant(fmt: int, packed: torch.Tensor, n_elems: int, out: torch.Tensor | None = None) -> torch.Tensor:
+    """Packed device bytes -> f32 device tensor of n_elems."""
+    packed = _dev_u8(packed)
+    if out is None:
+        out = torch.empty(n_elems, dtype=torch.float32, device=packed.device)
+    check(lib().rfq_dequant(fmt, _ptr(packed), packed.numel(), _ptr(out), n_elems, _stream()))
+    return out
+
+
+def gemv(fmt: int, w: torch.Tensor, x: torch.Tensor, n: int, k: int, out: torch.Tensor | None = None) -> torch.Tensor:
+    """y[m, n] = x[m, k] . dequant(W)[n, k]^T (m <= 8), fp32."""
+    w = _dev_u8(w)
+    if x.dtype != torch.float32 or not x.is_contiguous():
+        raise ValueError("x must be contiguous float32")
+    m = 1 if x.dim() == 1 else x.shape[0]
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float32, device=x.device)
+    check(lib().rfq_gemv(fmt, _ptr(w), w.numel(), _ptr(x), _ptr(out), m, n, k, _stream()))
+    return out if x.dim() > 1 else out.view(n)
+
+
+def gemm_f16(fmt: int, w: torch.Tensor, a: torch.Tensor, n: int, k: int, out_dtype=torch.float16,
+             out: torch.Tensor | None = None) -> torch.Tensor:
+    """out[m, n] = a[m, k] (fp16) . dequant(W)[n, k]^T on the fp16 matrix cores."""
+    w = _dev_u8(w)
+    if a.dtype != torch.float16 or not a.is_contiguous() or a.dim() != 2:
+        raise ValueError("a must be a contiguous [m, k] float16 tensor")
+    m = a.shape[0]
+    code = {torch.float32: _lib.F32, torch.float16: _lib.F16}[out_dtype]
+    if out is None:
+        out = torch.empty((m, n), dtype=out_dtype, device=a.device)
+    check(lib().rfq_gemm_f16(fmt, _ptr(w), w.numel(), _ptr(a), _ptr(out), code, m, n, k, _stream()))
+    return out
+
+
+class MxOperand:
+    """A [rows, k] MXFP matrix re-encoded for the block-scaled matrix core."""
+
+    def __init__(self, fmt: int, raw: torch.Tensor, rows: int, k: int, kind: int = _lib.MX_AUTO):
+        raw = _dev_u8(raw)
+        nbytes = lib().rfq_mx_prepared_bytes(fmt, kind, rows, k)
+        if nbytes == 0:
+            raise ValueError(f"cannot size a prepared operand for fmt={fmt} rows={rows} k={k}")
+        self.buf = torch.empty(nbytes, dtype=torch.uint8, device=raw.device)
+        got = C.c_int(0)
+        check(lib().rfq_mx_prepare(fmt, kind, _ptr(raw), raw.numel(), rows, k, _ptr(self.buf), nbytes,
+                                   C.byref(got), _stream()))
+        self.kind, self.rows, self.k, self.fmt = got.value, rows, k, fmt
+
+
+def gemm_mx(a: MxOperand, w: MxOperand, out_dtype=torch.bfloat16, out: torch.Tensor | None = None) -> torch.Tensor:
+    """out[m, n] = A[m, k] . W[n, k]^T on the scaled f8f6f4 matrix core."""
+    if a.k != w.k:
+        raise ValueError("inner dimensions differ")
+    code = {torch.float32: _lib.F32, torch.bfloat16: _lib.BF16}[out_dtype]
+    if out is None:
+        out = torch.empty((a.rows, w.rows), dtype=out_dtype, device=a.buf.device)
+    check(lib().rfq_gemm_mx(_ptr(a.buf), a.kind, _ptr(w.buf), w.kind, _ptr(out), code, a.rows, w.rows, a.k, _stream()))
+    return out
+
+
+def row_bytes(fmt: int, k: int) -> int:
+    return (k // BLOCK_ELEMS[fmt]) * BLOCK_BYTES[fmt]

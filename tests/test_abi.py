@@ -1,0 +1,62 @@
+"""The C-ABI library loads without a GPU and exports every symbol that
+include/rfq.h declares; host-side argument validation works without a device."""
+import ctypes as C
+import os
+import re
+
+import rocmforge_amd
+from rocmforge_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "rfq.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"RFQ_API\s+[\w\s\*]+?\b(rfq_\w+)\s*\(", text)))
+
+
+def test_header_symbols_exported():
+    names = declared_symbols()
+    assert len(names) >= 18, names
+    L = C.CDLL(rocmforge_amd.lib_path())
+    for n in names:
+        assert hasattr(L, n), f"{n} declared in rfq.h but not exported"
+    assert set(names) == set(_lib._SIGNATURES), "binding and header disagree"
+
+
+def test_sizes_and_version():
+    L = rocmforge_amd.lib()
+    assert L.rfq_version() == 100
+    assert [L.rfq_block_bytes(f) for f in (2, 8, 12, 14, 20, 21, 22)] == [20, 36, 256, 256, 17, 25, 25]
+    assert [L.rfq_block_elems(f) for f in (2, 8, 12, 14, 20, 21, 22)] == [32, 32, 256, 256, 32, 32, 32]
+    assert L.rfq_block_bytes(3) == 0 and L.rfq_block_elems(99) == 0
+    assert L.rfq_packed_bytes(2, 4864 * 896) == 2723840           # Q4_0 4864 x 896
+    assert L.rfq_packed_bytes(8, 4096 * 4096) == 18874368
+    assert L.rfq_packed_bytes(12, 14336 * 4096) == 58720256
+    assert L.rfq_packed_bytes(20, 28672 * 8192) == 124780544
+    assert L.rfq_packed_bytes(21, 28672 * 8192) == 183500800
+    assert L.rfq_packed_bytes(12, 100) == 256 and L.rfq_packed_bytes(2, 33) == 40
+
+
+def test_validation_needs_no_device():
+    L = rocmforge_amd.lib()
+    one = C.c_void_p(16)  # never dereferenced: every call below fails validation first
+    assert L.rfq_dequant(99, one, 20, one, 32, None) == _lib.E_BADARG
+    assert b"unknown format" in L.rfq_last_error()
+    assert L.rfq_dequant(2, one, 20, None, 32, None) == _lib.E_BADARG
+    assert L.rfq_dequant(2, None, 0, None, 0, None) == _lib.OK            # nothing to do
+    assert L.rfq_gemv(2, None, 0, one, one, 1, 4, 32, None) == _lib.E_BADARG
+    assert L.rfq_gemv(2, one, 80, one, one, 0, 4, 32, None) == _lib.E_BADARG   # m = 0
+    assert L.rfq_gemv(2, one, 80, one, one, 1, 4, 33, None) == _lib.E_SIZE     # k % 32
+    assert L.rfq_gemv(12, one, 1024, one, one, 1, 4, 128, None) == _lib.E_SIZE  # k % 256
+    assert L.rfq_gemv(2, one, 81, one, one, 1, 4, 32, None) == _lib.E_SIZE     # byte count
+    assert b"needs 80" in L.rfq_last_error()
+    assert L.rfq_gemv(2, one, 80, one, one, 9, 4, 32, None) == _lib.E_UNSUPPORTED
+    assert L.rfq_matmul_q4_0(one, one, one, 1, 0, 32, None) == _lib.E_BADARG
+    assert L.rfq_matmul_host_weights(2, one, 80, one, 0, 32, one, None) == _lib.E_BADARG
+    assert L.rfq_gemm_f16(12, one, 256, one, one, 2, 1, 1, 256, None) == _lib.E_BADARG  # bf16 out
+    assert L.rfq_mx_prepare(12, 0, one, 17, 1, 128, one, 64, None, None) == _lib.E_BADARG
+    assert L.rfq_mx_prepare(20, 0, one, 68, 1, 100, one, 64, None, None) == _lib.E_SIZE
+    assert L.rfq_gemm_mx(one, 4, one, 4, one, 1, 32, 32, 128, None) == _lib.E_BADARG     # f16 out
+    assert L.rfq_gemm_mx(one, 5, one, 4, one, 0, 32, 32, 128, None) == _lib.E_BADARG
