@@ -1,0 +1,178 @@
+#!/usr/bin/env python3
+"""Headline bench: Q4_K decode GEMV, W [14336 x 4096], x fp32 [4096], batch 1.
+
+One step = one rfq_gemv call (one token's FFN projection).  The packed weights
+are resident in HBM before the timed region; the step loop rotates through
+enough distinct weight copies that the 256 MB last-level cache cannot hold
+them, so every step streams its 58.7 MB from HBM ("cold").  The metric is
+algorithmic bytes (packed W as stored + x + y) per second.
+
+Prints ONE JSON line.  Extra keys: `roofline` (HIP-event timing of the same
+launches against the 8 TB/s HBM peak), `cpu_baseline` (the CPU oracle timed on
+this host), `also` (the other configurations, one short run each).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+N, K = 14336, 4096
+CACHE_BYTES = 256 << 20
+
+
+def algorithmic_bytes(fmt, n, k, m, Q):
+    return Q.packed_bytes(fmt, n * k) + 4 * m * k + 4 * m * n
+
+
+def time_gemv(torch, fmt, n, k, m, copies, steps, warmup, Q, seed):
+    """Returns (wall seconds, device seconds) for `steps` rfq_gemv calls issued
+    back to back by the library's native loop on torch's current stream."""
+    import ctypes as C
+
+    import numpy as np
+
+    from rocmforge_amd import _lib
+    dev = torch.device("cuda:0")
+    w = Q.make_weights(fmt, n, k, seed=seed)
+    rng = np.random.Generator(np.random.PCG64(seed + 1))
+    x = rng.standard_normal((m, k), dtype=np.float32)
+    dws = [torch.from_numpy(w).to(dev) for _ in range(copies)]
+    ptrs = (C.c_void_p * copies)(*[t.data_ptr() for t in dws])
+    dx = torch.from_numpy(x).to(dev)
+    y = torch.empty((m, n), dtype=torch.float32, device=dev)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    ms = C.c_float(0)
+    L = _lib.lib()
+    # untimed warm-up (also loads the code object), then barrier
+    _lib.check(L.rfq_bench_gemv(fmt, ptrs, copies, w.size, C.c_void_p(dx.data_ptr()), C.c_void_p(y.data_ptr()),
+                                m, n, k, 0, max(warmup, 1), stream, C.byref(ms)))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    _lib.check(L.rfq_bench_gemv(fmt, ptrs, copies, w.size, C.c_void_p(dx.data_ptr()), C.c_void_p(y.data_ptr()),
+                                m, n, k, 0, steps, stream, C.byref(ms)))
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return wall, ms.value / 1e3, w, x, y.cpu().numpy()
+
+
+def cpu_baseline(fmt, w, x, n, k, budget_s=12.0):
+    """The CPU oracle (dequantise everything, then the sequential fp32 matmul)
+    on one host thread, repeated until ~budget_s of CPU work."""
+    import ctypes as C
+
+    import numpy as np
+
+    import oracle
+    L = oracle.lib()
+    gomp = C.CDLL("libgomp.so.1")
+    gomp.omp_set_num_threads(1)
+    wd = np.empty(n * k, np.float32)
+    c = np.empty(n, np.float32)
+    reps, spent = 0, 0.0
+    while spent < budget_s and reps < 64:
+        t = time.perf_counter()
+        rc = L.rf_qmatmul_nk_staged(fmt, w.ctypes.data_as(C.c_void_p), w.size, x.ctypes.data_as(C.c_void_p), 1, n, k,
+                                    wd.ctypes.data_as(C.c_void_p), c.ctypes.data_as(C.c_void_p))
+        assert rc == 0
+        spent += time.perf_counter() - t
+        reps += 1
+    gomp.omp_set_num_threads(os.cpu_count() or 1)
+    return spent / reps, reps, c
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=100)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--no-also", action="store_true", help="skip the secondary configurations")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build is single-GPU (one MI355X per box); run with --gpus 1. "
+                 "The path shards by output rows with no exchange during compute; see DESIGN.md.")
+
+    import numpy as np
+    import torch
+
+    from rocmforge_amd import quantize as Q
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    import rocmforge_amd
+    rocmforge_amd.lib()  # fail loudly if librfq.so is missing
+
+    fmt = Q.Q4_K
+    wbytes = Q.packed_bytes(fmt, N * K)
+    copies = -(-int(2.5 * CACHE_BYTES) // wbytes)          # 11 copies, 646 MB > 2.5x the last-level cache
+    abytes = algorithmic_bytes(fmt, N, K, 1, Q)
+    wall, dev_s, w, x, y = time_gemv(torch, fmt, N, K, 1, copies, args.steps, args.warmup, Q, 20260003)
+    ms_per_step = wall / args.steps * 1e3
+    value = abytes / (wall / args.steps) / 1e9
+    achieved = abytes / (dev_s / args.steps) / 1e9
+
+    # warm variant (one copy, cache-resident) for the record
+    wall_w, dev_w, *_ = time_gemv(torch, fmt, N, K, 1, 1, args.steps, args.warmup, Q, 20260003)
+
+    out = {
+        "metric": "Q4_K decode GEMV GB/s (% HBM peak); quant prefill GEMM TFLOP/s (% MFMA peak)",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "Q4_K decode GEMV W[14336x4096] (256-byte super-blocks), x fp32[4096], batch 1, "
+                               f"{copies} rotating weight copies (cold HBM)",
+                   "algorithmic_bytes_per_step": abytes, "weight_copies": copies},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "gemv_xreg_kernel<Q4_K,2,1>", "avg_launch_us": round(dev_s / args.steps * 1e6, 3),
+                     "warm_cache_gbs": round(abytes / (dev_w / args.steps) / 1e9, 1)},
+    }
+
+    if not args.no_also:
+        also = {}
+        for name, f, n, k, m, seed in (("Q6_K gemv 14336x4096", Q.Q6_K, N, K, 1, 20260013),
+                                       ("Q8_0 gemv 4096x4096 m1", Q.Q8_0, 4096, 4096, 1, 20260002),
+                                       ("Q8_0 gemv 4096x4096 m8", Q.Q8_0, 4096, 4096, 8, 20260002),
+                                       ("Q4_0 gemv 4864x896", Q.Q4_0, 4864, 896, 1, 20260001)):
+            c = -(-int(2.5 * CACHE_BYTES) // Q.packed_bytes(f, n * k))
+            c = min(c, 64)
+            _, d, *_ = time_gemv(torch, f, n, k, m, c, 500, 50, Q, seed)
+            b = algorithmic_bytes(f, n, k, m, Q)
+            also[name] = {"GB/s": round(b / (d / 500) / 1e9, 1), "us": round(d / 500 * 1e6, 2),
+                          "hbm_frac": round(b / (d / 500) / 1e9 / HBM_PEAK_GBS, 4)}
+        try:
+            import bench_gemm
+            also.update(bench_gemm.run(torch))
+        except ImportError:
+            pass
+        out["also"] = also
+
+    if not args.no_cpu:
+        t_cpu, reps, c = cpu_baseline(fmt, w, x[0], N, K)
+        ref = c.astype(np.float64)
+        rms = float(np.sqrt(np.mean(ref * ref)))
+        err = float(np.max(np.abs(y[0] - ref) / np.maximum(np.abs(ref), rms)))
+        out["cpu_baseline"] = {"value": round(abytes / t_cpu / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+                               "sample": f"the full 14336x4096 GEMV (dequantise all weights to f32, then the sequential "
+                                         f"fp32 matmul), {reps} repetitions on one host thread",
+                               "ms_per_step": round(t_cpu * 1e3, 2), "gpu_vs_cpu_max_rel_err": float(f"{err:.3e}")}
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,42 @@
+/*
+ * rfq_bench.h -- timing loops exported by librfq for the benchmark driver.
+ *
+ * Not part of the operator surface: these are the native counterpart of the
+ * hand-rolled "warm up, then time N iterations" loops in ROCmForge's
+ * benches/matmul_bench.rs:343-378 and benches/dequant_bench.rs:391-404.  Each
+ * enqueues `warmup` untimed and `steps` timed calls of the corresponding
+ * rfq_* entry point back to back on `stream`, brackets the timed ones with HIP
+ * events recorded on that same stream, synchronises, and returns the elapsed
+ * device time of the timed region in milliseconds.  Keeping the loop native
+ * keeps the host's launch rate above the ~10 us kernels being measured.
+ */
+#ifndef RFQ_BENCH_H
+#define RFQ_BENCH_H
+
+#include "rfq.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Step i multiplies by weight copy d_w_copies[i % copies] (all of w_bytes):
+ * with enough copies no step finds its weights in the last-level cache. */
+RFQ_API int rfq_bench_gemv(int fmt, const void *const *d_w_copies, int copies, size_t w_bytes, const float *d_x,
+                           float *d_y, int m, int n, int k, int warmup, int steps, void *stream,
+                           float *elapsed_ms);
+
+RFQ_API int rfq_bench_dequant(int fmt, const void *const *d_in_copies, int copies, size_t packed_bytes, float *d_out,
+                              size_t n_elems, int warmup, int steps, void *stream, float *elapsed_ms);
+
+RFQ_API int rfq_bench_gemm_f16(int fmt, const void *d_w, size_t w_bytes, const void *d_a_f16, void *d_out,
+                               int out_dtype, int m, int n, int k, int warmup, int steps, void *stream,
+                               float *elapsed_ms);
+
+RFQ_API int rfq_bench_gemm_mx(const void *d_a_prep, int a_kind, const void *d_w_prep, int w_kind, void *d_out,
+                              int out_dtype, int m, int n, int k, int warmup, int steps, void *stream,
+                              float *elapsed_ms);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RFQ_BENCH_H */

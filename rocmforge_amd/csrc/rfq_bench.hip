@@ -1,0 +1,77 @@
+// Native timing loops for the benchmark driver (see include/rfq_bench.h).
+#include "rfq_bench.h"
+
+#include "rfq_common.hpp"
+
+namespace {
+
+template <typename Step>
+int timed_loop(int warmup, int steps, void *stream, float *elapsed_ms, Step step)
+{
+    using namespace rfq;
+    if (steps <= 0 || warmup < 0 || !elapsed_ms) return fail(RFQ_E_BADARG, "rfq_bench: bad warmup/steps/elapsed_ms");
+    hipStream_t s = (hipStream_t)stream;
+    for (int i = 0; i < warmup; i++) {
+        int rc = step(i);
+        if (rc != RFQ_OK) return rc;
+    }
+    hipEvent_t e0, e1;
+    RFQ_HIP(hipEventCreate(&e0));
+    RFQ_HIP(hipEventCreate(&e1));
+    RFQ_HIP(hipStreamSynchronize(s));
+    RFQ_HIP(hipEventRecord(e0, s));
+    int rc = RFQ_OK;
+    for (int i = 0; i < steps && rc == RFQ_OK; i++) rc = step(warmup + i);
+    hipError_t er = hipEventRecord(e1, s);
+    hipError_t es = hipEventSynchronize(e1);
+    float ms = 0.f;
+    hipError_t et = hipEventElapsedTime(&ms, e0, e1);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    if (rc != RFQ_OK) return rc;
+    if (er != hipSuccess) return hip_fail(er, "hipEventRecord");
+    if (es != hipSuccess) return hip_fail(es, "hipEventSynchronize");
+    if (et != hipSuccess) return hip_fail(et, "hipEventElapsedTime");
+    *elapsed_ms = ms;
+    return RFQ_OK;
+}
+
+} // namespace
+
+extern "C" {
+
+int rfq_bench_gemv(int fmt, const void *const *d_w_copies, int copies, size_t w_bytes, const float *d_x, float *d_y,
+                   int m, int n, int k, int warmup, int steps, void *stream, float *elapsed_ms)
+{
+    if (!d_w_copies || copies <= 0) return rfq::fail(RFQ_E_BADARG, "rfq_bench_gemv: no weight copies");
+    return timed_loop(warmup, steps, stream, elapsed_ms, [&](int i) {
+        return rfq_gemv(fmt, d_w_copies[i % copies], w_bytes, d_x, d_y, m, n, k, stream);
+    });
+}
+
+int rfq_bench_dequant(int fmt, const void *const *d_in_copies, int copies, size_t packed_bytes, float *d_out,
+                      size_t n_elems, int warmup, int steps, void *stream, float *elapsed_ms)
+{
+    if (!d_in_copies || copies <= 0) return rfq::fail(RFQ_E_BADARG, "rfq_bench_dequant: no input copies");
+    return timed_loop(warmup, steps, stream, elapsed_ms, [&](int i) {
+        return rfq_dequant(fmt, d_in_copies[i % copies], packed_bytes, d_out, n_elems, stream);
+    });
+}
+
+int rfq_bench_gemm_f16(int fmt, const void *d_w, size_t w_bytes, const void *d_a_f16, void *d_out, int out_dtype,
+                       int m, int n, int k, int warmup, int steps, void *stream, float *elapsed_ms)
+{
+    return timed_loop(warmup, steps, stream, elapsed_ms, [&](int) {
+        return rfq_gemm_f16(fmt, d_w, w_bytes, d_a_f16, d_out, out_dtype, m, n, k, stream);
+    });
+}
+
+int rfq_bench_gemm_mx(const void *d_a_prep, int a_kind, const void *d_w_prep, int w_kind, void *d_out, int out_dtype,
+                      int m, int n, int k, int warmup, int steps, void *stream, float *elapsed_ms)
+{
+    return timed_loop(warmup, steps, stream, elapsed_ms, [&](int) {
+        return rfq_gemm_mx(d_a_prep, a_kind, d_w_prep, w_kind, d_out, out_dtype, m, n, k, stream);
+    });
+}
+
+} // extern "C"

@@ -1,0 +1,123 @@
+"""GPU parity: fused dequant + GEMV against the CPU oracle (dequantise, then
+the reference's sequential fp32 matmul)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from helpers import assert_close
+from rocmforge_amd import quantize as Q
+
+pytestmark = pytest.mark.gpu
+
+FORMATS = [Q.Q4_0, Q.Q8_0, Q.Q4_K, Q.Q6_K, Q.MXFP4, Q.MXFP6_E2M3]
+
+
+def gpu_gemv(fmt, w, x, n, k, cuda):
+    import torch
+    from rocmforge_amd import ops
+    dw = torch.from_numpy(np.ascontiguousarray(w)).to(cuda)
+    dx = torch.from_numpy(np.ascontiguousarray(x)).to(cuda)
+    y = ops.gemv(fmt, dw, dx, n, k)
+    torch.cuda.synchronize()
+    return y.cpu().numpy()
+
+
+def x_for(m, k, seed):
+    rng = np.random.Generator(np.random.PCG64(seed))
+    x = rng.standard_normal((m, k), dtype=np.float32)
+    return x[0] if m == 1 else x
+
+
+# k = 256..1024 takes the one-row-per-wavefront kernel, 2048 / 4096 / 8192 /
+# 14336 the register-resident one at 1, 2, 2x2 and 2x4 units per lane x
+# wavefronts per row, 32768 falls back again; n values exercise ragged teams.
+@pytest.mark.parametrize("fmt", FORMATS)
+@pytest.mark.parametrize("n,k", [(5, 256), (33, 1024), (64, 2048), (1001, 2048), (130, 4096), (257, 8192),
+                                 (19, 14336), (9, 32768), (2048, 1536)])
+def test_gemv_m1_shapes(fmt, n, k, oracle, cuda):
+    w = Q.make_weights(fmt, n, k, seed=3000 + fmt + n)
+    x = x_for(1, k, 4000 + k)
+    got = gpu_gemv(fmt, w, x, n, k, cuda)
+    want = oracle.qmatmul_nk(fmt, w, x, 1, n, k)[0]
+    assert_close(got, want, f"{Q.NAMES[fmt]} n={n} k={k}")
+
+
+@pytest.mark.parametrize("fmt", FORMATS)
+@pytest.mark.parametrize("m", [2, 3, 5, 8])
+def test_gemv_small_batches(fmt, m, oracle, cuda):
+    n, k = 301, 2048
+    w = Q.make_weights(fmt, n, k, seed=5000 + fmt)
+    x = x_for(m, k, 6000 + m)
+    got = gpu_gemv(fmt, w, x, n, k, cuda)
+    assert got.shape == (m, n)
+    assert_close(got, oracle.qmatmul_nk(fmt, w, x, m, n, k), f"{Q.NAMES[fmt]} m={m}")
+
+
+@pytest.mark.parametrize("fmt", [Q.MXFP4, Q.MXFP6_E2M3])
+def test_gemv_mx_random_codes_and_clamp(fmt, oracle, cuda):
+    # every code, exponents up to +6 so the +-8 / +-7.5 clamp is active
+    rng = np.random.default_rng(70 + fmt)
+    n, k = 96, 4096
+    w = Q.random_blocks(fmt, n * k // 32, rng, exp_range=(-9, 6))
+    x = x_for(1, k, 71)
+    assert_close(gpu_gemv(fmt, w, x, n, k, cuda), oracle.qmatmul_nk(fmt, w, x, 1, n, k)[0], Q.NAMES[fmt])
+
+
+# BASELINE configs: Q4_0 4864x896; Q8_0 4096x4096 at m = 1 and 8; Q4_K and Q6_K 14336x4096.
+@pytest.mark.parametrize("fmt,n,k,m,cfg", [(Q.Q4_0, 4864, 896, 1, 1), (Q.Q8_0, 4096, 4096, 1, 2),
+                                           (Q.Q8_0, 4096, 4096, 8, 2), (Q.Q4_K, 14336, 4096, 1, 3),
+                                           (Q.Q6_K, 14336, 4096, 1, 3)])
+def test_gemv_baseline_configs(fmt, n, k, m, cfg, oracle, cuda):
+    w = Q.make_weights(fmt, n, k, seed=20260000 + cfg)
+    x = x_for(m, k, 20260100 + cfg)
+    got = gpu_gemv(fmt, w, x, n, k, cuda)
+    want = oracle.qmatmul_nk(fmt, w, x, m, n, k)
+    e = assert_close(got.reshape(m, n), want, f"config {cfg} {Q.NAMES[fmt]} m={m}")
+    print(f"config {cfg} {Q.NAMES[fmt]} m={m}: max rel err {e:.2e}")
+
+
+def test_q4_k_onesided_real_data(oracle, cuda):
+    rng = np.random.default_rng(81)
+    n, k = 512, 4096
+    w = Q.quantize_q4_k_onesided(np.abs(rng.standard_normal((n, k)) * 0.02).astype(np.float32), rng)
+    x = x_for(1, k, 82)
+    assert_close(gpu_gemv(Q.Q4_K, w, x, n, k, cuda), oracle.qmatmul_nk(Q.Q4_K, w, x, 1, n, k)[0], "q4_k onesided")
+
+
+def test_linearity_at_full_size(cuda):
+    # size-independent property at the headline shape: W(a*x1 + x2) == a*W(x1) + W(x2)
+    n, k = 14336, 4096
+    w = Q.make_weights(Q.Q4_K, n, k, seed=91)
+    x1, x2 = x_for(1, k, 92), x_for(1, k, 93)
+    y1, y2 = gpu_gemv(Q.Q4_K, w, x1, n, k, cuda), gpu_gemv(Q.Q4_K, w, x2, n, k, cuda)
+    y = gpu_gemv(Q.Q4_K, w, (np.float32(0.5) * x1 + x2).astype(np.float32), n, k, cuda)
+    assert_close(y, 0.5 * y1.astype(np.float64) + y2, "linearity", tol=1e-4)
+
+
+def test_reference_signatures(oracle, cuda):
+    import torch
+    from rocmforge_amd import _lib
+    L = _lib.lib()
+    n, k = 256, 1024
+    x = x_for(1, k, 101)
+    dx = torch.from_numpy(x).to(cuda)
+    for fmt, fn in ((Q.Q4_0, L.rfq_matmul_q4_0), (Q.Q8_0, L.rfq_matmul_q8_0), (Q.Q4_K, L.rfq_matmul_q4_k),
+                    (Q.Q6_K, L.rfq_matmul_q6_k)):
+        w = Q.make_weights(fmt, n, k, seed=102 + fmt)
+        want = oracle.qmatmul_nk(fmt, w, x, 1, n, k)[0]
+        dw = torch.from_numpy(w).to(cuda)
+        out = torch.zeros(n, dtype=torch.float32, device=cuda)
+        # (activations, weights, output, m, n, k), as matmul_q4_0_gpu
+        _lib.check(fn(C.c_void_p(dx.data_ptr()), C.c_void_p(dw.data_ptr()), C.c_void_p(out.data_ptr()), 1, n, k, None))
+        torch.cuda.synchronize()
+        assert_close(out.cpu().numpy(), want, f"raw {Q.NAMES[fmt]}")
+        # host weights, device input/output, as matmul_q4_0(backend, &[u8], &HipBuffer, rows, cols, &HipBuffer)
+        out.zero_()
+        torch.cuda.synchronize()
+        _lib.check(L.rfq_matmul_host_weights(fmt, w.ctypes.data_as(C.c_void_p), w.size, C.c_void_p(dx.data_ptr()),
+                                             n, k, C.c_void_p(out.data_ptr()), None))
+        assert_close(out.cpu().numpy(), want, f"host weights {Q.NAMES[fmt]}")
+    # the all-0x88 Q4_0 weights of tests/q_dequant_tests.rs:396-489 give exactly zero
+    w = np.zeros((n * k // 32, 20), np.uint8); w[:, 0:4] = np.frombuffer(np.float32(1.0).tobytes(), np.uint8); w[:, 4:] = 0x88
+    assert np.all(np.abs(gpu_gemv(Q.Q4_0, w.ravel(), x, n, k, cuda)) < 1e-4)
