@@ -20,6 +20,19 @@
 // the four rows; an LDS hop only when a row is split over several wavefronts.
 #include "rfq_common.hpp"
 
+// Per-wavefront phase timestamps for tuning builds (-DRFQ_GEMV_TRACE); compiled
+// out of the library.
+#ifdef RFQ_GEMV_TRACE
+__device__ unsigned long long *rfq_trace_buf;
+#define RFQ_TS(slot)                                                                                   \
+    do {                                                                                               \
+        if ((threadIdx.x & 63) == 0 && rfq_trace_buf)                                                  \
+            rfq_trace_buf[((size_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * 8 + (slot)] = wall_clock64(); \
+    } while (0)
+#else
+#define RFQ_TS(slot) do { } while (0)
+#endif
+
 namespace rfq {
 namespace {
 
@@ -273,8 +286,16 @@ __device__ __forceinline__ float sum32(const float (&x)[32])
 // ---- m == 1, x resident in registers ----------------------------------------
 //
 // Block = 4 wavefronts = 4 / WPR teams.  Lane `tl` of a team (0 .. 64*WPR-1)
-// owns units tl + j * 64 * WPR, j < UPL, of EVERY row the team visits.
-template <int FMT, int UPL, int WPR>
+// owns units tl + j * 64 * WPR, j < UPL, of EVERY row the team visits.  A team
+// walks `rows_per_team` consecutive rows in groups of D: all loads of a group
+// are issued back to back (D rows x UPL units in flight per lane, no branch
+// between them so the hardware counters let row d be consumed while rows
+// d+1.. are still arriving), then the D rows are reduced.  Rows past the end
+// re-read the team's last valid row (same addresses, served by the cache) and
+// their result is dropped; lanes past the end of a row do the same with the
+// row's last unit.  HBM latency, not bandwidth, bounds a wavefront that has a
+// single row in flight, hence the depth.
+template <int FMT, int UPL, int WPR, int D>
 __global__ void __launch_bounds__(256)
 gemv_xreg_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ y, int n, int k,
                  int rows_per_team)
@@ -288,62 +309,354 @@ gemv_xreg_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
 
     float xs[UPL][32], xsum[UPL];
     bool live[UPL];
+    int unit[UPL];
 #pragma unroll
     for (int j = 0; j < UPL; j++) {
         int u = tl + j * TL;
         live[j] = u < ku;
-        if (live[j]) {
-            load_x32(x + (size_t)u * 32, xs[j]);
-        } else {
-#pragma unroll
-            for (int i = 0; i < 32; i++) xs[j][i] = 0.f;
-        }
-        xsum[j] = Unit<FMT>::NEEDS_XSUM ? sum32(xs[j]) : 0.f;
+        unit[j] = live[j] ? u : ku - 1;
+        load_x32(x + (size_t)unit[j] * 32, xs[j]);
     }
 
-    __shared__ float part[4];
+    __shared__ float part[D][4];
     const int row0 = (blockIdx.x * TEAMS + team) * rows_per_team;
+    int row_end = row0 + rows_per_team;
+    if (row_end > n) row_end = n;
+    const int row_last = row_end > row0 ? row_end - 1 : (n - 1);
 
-    Unit<FMT> cur[UPL], nxt[UPL];
-    if (row0 < n) {
+    Unit<FMT> buf[D][UPL];
+    auto load_group = [&](int g) {
 #pragma unroll
-        for (int j = 0; j < UPL; j++)
-            if (live[j]) cur[j].load(w + (size_t)row0 * rb, tl + j * TL);
-    }
-    for (int i = 0; i < rows_per_team; i++) {
-        const int r = row0 + i;
-        const bool have = r < n;
-        const bool have_next = (i + 1 < rows_per_team) && (r + 1 < n);
-        if (have_next) {
+        for (int d = 0; d < D; d++) {
+            int r = row0 + g + d;
+            if (r > row_last) r = row_last;
+            const uint8_t *row = w + (size_t)r * rb;
 #pragma unroll
-            for (int j = 0; j < UPL; j++)
-                if (live[j]) nxt[j].load(w + (size_t)(r + 1) * rb, tl + j * TL);
+            for (int j = 0; j < UPL; j++) buf[d][j].load(row, unit[j]);
         }
-        float acc = 0.f;
-        if (have) {
+    };
+    // x first, then the whole first group, and only then the first use of x:
+    // the weight loads are already in flight while the x sums are formed.
+    load_group(0);
 #pragma unroll
-            for (int j = 0; j < UPL; j++)
-                if (live[j]) acc += cur[j].dot(xs[j], xsum[j]);
+    for (int j = 0; j < UPL; j++) xsum[j] = Unit<FMT>::NEEDS_XSUM ? sum32(xs[j]) : 0.f;
+
+    for (int g = 0; g < rows_per_team; g += D) {
+        if (g > 0) load_group(g);
+        float res[D];
+#pragma unroll
+        for (int d = 0; d < D; d++) {
+            float acc = 0.f;
+#pragma unroll
+            for (int j = 0; j < UPL; j++) {
+                float t = buf[d][j].dot(xs[j], xsum[j]);
+                acc += live[j] ? t : 0.f;
+            }
+            res[d] = wave_sum(acc);
         }
-        acc = wave_sum(acc);
         if (WPR == 1) {
-            if (have && lane == 0) y[r] = acc;
+            if (lane == 0) {
+#pragma unroll
+                for (int d = 0; d < D; d++) {
+                    int r = row0 + g + d;
+                    if (g + d < rows_per_team && r < n) y[r] = res[d];
+                }
+            }
         } else {
-            // rows_per_team and the loop bounds are uniform over the block, so
-            // every wavefront reaches both barriers the same number of times.
-            if (lane == 0) part[wave] = acc;
+            // The group loop bounds are uniform over the block, so every
+            // wavefront reaches both barriers the same number of times.
+            if (lane == 0) {
+#pragma unroll
+                for (int d = 0; d < D; d++) part[d][wave] = res[d];
+            }
             __syncthreads();
-            if (have && wit == 0 && lane == 0) {
+            if (wit == 0 && lane < D) {
+                int r = row0 + g + lane;
                 float t = 0.f;
 #pragma unroll
-                for (int q = 0; q < WPR; q++) t += part[team * WPR + q];
-                y[r] = t;
+                for (int q = 0; q < WPR; q++) t += part[lane][team * WPR + q];
+                if (g + lane < rows_per_team && r < n) y[r] = t;
             }
             __syncthreads();
         }
-        if (have_next) {
+    }
+}
+
+// ---- m == 1, integer dot products ---------------------------------------------
+//
+// The float kernel above spends ~3 VALU instructions per weight (convert,
+// multiply-add, unpack) and is bound by them, not by HBM.  Here x is turned,
+// once per workgroup, into block-fixed-point: per unit of 32 values a power of
+// two s and 22-bit integers X_i = round(x_i / s), |X_i| < 2^22, split into
+// three byte limbs (X = top * 65536 + mid * 256 + low; top signed, mid and low
+// unsigned) and packed four elements to a dword in the order the weight bytes
+// unpack to.  The weights stay integers too, so a unit's 32 products are
+// 4-way byte dot products (v_dot4) with exact int32 sums:
+//     sum_i q_i x_i  =  s * (65536 * sum q.top + 256 * sum q.mid + sum q.low)
+// about 1.1 instructions per weight, and more accurate than an fp32
+// running sum (the only roundings: x to 22 bits relative to the unit's largest
+// value, and the final scaling).  A non-finite x value poisons its unit's s
+// with NaN, as it would poison the float sum.
+//
+// LDS holds, per unit, 24 limb dwords + s + sum(x) (stride 28 dwords).
+
+struct XPrep { uint32_t l[24]; float s, xsum; };
+
+__device__ __forceinline__ float dpp_xor1_f(float v)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true));
+}
+
+// Byte-transpose four 24-bit integers into (low, mid, top) limb dwords.
+__device__ __forceinline__ void limbs4(uint32_t x0, uint32_t x1, uint32_t x2, uint32_t x3, uint32_t *out3)
+{
+    uint32_t t01l = __builtin_amdgcn_perm(x1, x0, 0x05010400u); // b0x0 b0x1 b1x0 b1x1
+    uint32_t t23l = __builtin_amdgcn_perm(x3, x2, 0x05010400u);
+    uint32_t t01h = __builtin_amdgcn_perm(x1, x0, 0x0C0C0602u); // b2x0 b2x1 0 0
+    uint32_t t23h = __builtin_amdgcn_perm(x3, x2, 0x0C0C0602u);
+    out3[0] = __builtin_amdgcn_perm(t23l, t01l, 0x05040100u);
+    out3[1] = __builtin_amdgcn_perm(t23l, t01l, 0x07060302u);
+    out3[2] = __builtin_amdgcn_perm(t23h, t01h, 0x05040100u);
+}
+
+// One thread converts half a unit (16 consecutive x) and writes 12 limb
+// dwords; the two threads of a unit are neighbouring lanes.
+// NIBBLE: groups are elements 8d+{0,2,4,6} then 8d+{1,3,5,7} (low nibbles,
+// then high nibbles of four consecutive bytes); otherwise 4g+{0,1,2,3}.
+// TOPOFF: added to every integer before the split (2^22 makes the top limb
+// unsigned, 0..127, for formats whose weight bytes exceed 127).
+__device__ __forceinline__ void prep_load(const float *xp, float (&xv)[16])
+{
 #pragma unroll
-            for (int j = 0; j < UPL; j++) cur[j] = nxt[j];
+    for (int i = 0; i < 4; i++) {
+        float4 v = ld<float4>(reinterpret_cast<const uint8_t *>(xp + 4 * i));
+        xv[4 * i] = v.x; xv[4 * i + 1] = v.y; xv[4 * i + 2] = v.z; xv[4 * i + 3] = v.w;
+    }
+}
+
+template <bool NIBBLE, uint32_t TOPOFF>
+__device__ __forceinline__ void prep_convert(const float (&xv)[16], int half, uint32_t *lds_unit)
+{
+    float m = 0.f, sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; i++) { m = fmaxf(m, fabsf(xv[i])); sum += xv[i]; }
+    bool bad = false;
+#pragma unroll
+    for (int i = 0; i < 16; i++) bad |= !(fabsf(xv[i]) <= 3.40282347e+38f);
+    m = fmaxf(m, dpp_xor1_f(m));
+    sum += dpp_xor1_f(sum);
+    bad |= __builtin_amdgcn_update_dpp(0, (int)bad, 0xB1, 0xF, 0xF, true) != 0;
+    int e = (int)(__float_as_uint(m) >> 23);          // biased exponent of the largest |x|
+    int ie = 275 - e;                                 // 1/s = 2^(21 - (e - 127))
+    if (ie > 254) ie = 254;
+    float inv_s = __uint_as_float((uint32_t)ie << 23);
+    float sc = ie == 254 ? __uint_as_float(0x00400000u) : __uint_as_float((uint32_t)(254 - ie) << 23);
+    if (bad) sc = __uint_as_float(0x7FC00000u);
+    uint32_t X[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++)
+        X[i] = __float_as_uint(__builtin_fmaf(xv[i], inv_s, 12582912.0f)) - 0x4B400000u + TOPOFF;
+    uint32_t *o = lds_unit + half * 12;
+    if (NIBBLE) {
+#pragma unroll
+        for (int d = 0; d < 2; d++) {
+            limbs4(X[8 * d], X[8 * d + 2], X[8 * d + 4], X[8 * d + 6], o + (2 * d) * 3);
+            limbs4(X[8 * d + 1], X[8 * d + 3], X[8 * d + 5], X[8 * d + 7], o + (2 * d + 1) * 3);
+        }
+    } else {
+#pragma unroll
+        for (int g = 0; g < 4; g++) limbs4(X[4 * g], X[4 * g + 1], X[4 * g + 2], X[4 * g + 3], o + g * 3);
+    }
+    if (half == 0) {
+        lds_unit[24] = __float_as_uint(sc);
+        lds_unit[25] = __float_as_uint(sum);
+    }
+}
+
+// sum_i nibble_i * X_i for 16 weight bytes in low-nibble-first order.
+__device__ __forceinline__ float nib_idot(const U4 &q, const XPrep &xp)
+{
+    uint32_t alo = 0, amid = 0;
+    int atop = 0;
+#pragma unroll
+    for (int d = 0; d < 4; d++) {
+        uint32_t lo = q.v[d] & 0x0F0F0F0Fu, hi = (q.v[d] >> 4) & 0x0F0F0F0Fu;
+        const uint32_t *L = &xp.l[(2 * d) * 3], *H = &xp.l[(2 * d + 1) * 3];
+        alo = __builtin_amdgcn_udot4(lo, L[0], alo, false);
+        amid = __builtin_amdgcn_udot4(lo, L[1], amid, false);
+        atop = __builtin_amdgcn_sdot4((int)lo, (int)L[2], atop, false);
+        alo = __builtin_amdgcn_udot4(hi, H[0], alo, false);
+        amid = __builtin_amdgcn_udot4(hi, H[1], amid, false);
+        atop = __builtin_amdgcn_sdot4((int)hi, (int)H[2], atop, false);
+    }
+    return __builtin_fmaf((float)atop, 65536.0f, __builtin_fmaf((float)amid, 256.0f, (float)alo));
+}
+
+template <int FMT> struct IUnit;
+
+template <> struct IUnit<RFQ_Q4_K> : Unit<RFQ_Q4_K> {
+    static constexpr bool NIBBLE = true;
+    static constexpr uint32_t TOPOFF = 0;
+    __device__ __forceinline__ float idot(const XPrep &xp) const
+    {
+        return __builtin_fmaf(f16_bits_to_f32(sc) * xp.s, nib_idot(q, xp), (float)mn * xp.xsum);
+    }
+};
+
+template <> struct IUnit<RFQ_Q4_0> : Unit<RFQ_Q4_0> {
+    static constexpr bool NIBBLE = true;
+    static constexpr uint32_t TOPOFF = 0;
+    __device__ __forceinline__ float idot(const XPrep &xp) const
+    {
+        return scale * __builtin_fmaf(xp.s, nib_idot(q, xp), -8.0f * xp.xsum);
+    }
+};
+
+template <> struct IUnit<RFQ_Q8_0> : Unit<RFQ_Q8_0> {
+    static constexpr bool NIBBLE = false;
+    static constexpr uint32_t TOPOFF = 0x400000u; // weight bytes reach 255: keep every limb unsigned
+    __device__ __forceinline__ float idot(const XPrep &xp) const
+    {
+        uint32_t alo = 0, amid = 0, atop = 0, bsum = 0;
+#pragma unroll
+        for (int g = 0; g < 8; g++) {
+            const uint32_t *L = &xp.l[g * 3];
+            alo = __builtin_amdgcn_udot4(q.v[g], L[0], alo, false);
+            amid = __builtin_amdgcn_udot4(q.v[g], L[1], amid, false);
+            atop = __builtin_amdgcn_udot4(q.v[g], L[2], atop, false);
+            bsum = __builtin_amdgcn_udot4(q.v[g], 0x01010101u, bsum, false);
+        }
+        // top limbs carry +64: sum b*(top+64) - 64*sum b
+        float S = __builtin_fmaf((float)((int)atop - 64 * (int)bsum), 65536.0f,
+                                 __builtin_fmaf((float)amid, 256.0f, (float)alo));
+        return scale * __builtin_fmaf(xp.s, S, -128.0f * xp.xsum);
+    }
+};
+
+// Block = 4 wavefronts = 4 / WPR teams.  Lane `tl` of a team owns units
+// tl + j*64*WPR, j < UPL, of every row the team visits.  A team walks
+// `groups` groups of R consecutive rows; R is a compile-time constant so a
+// group is straight-line code: D rows are requested up front, then row i is
+// reduced and row i+D requested, so D rows (D * UPL unit loads per lane) stay in
+// flight while the matrix streams in and the hardware load counters release
+// each row exactly when it has arrived.  Deeper prefetch does not help: a CU
+// accepts only so many outstanding requests and later loads just block issue.
+// Rows past the end re-read the team's last valid row (a cache hit) and their
+// result is dropped; so do lanes past the end of a row with the last unit.
+template <int FMT, int UPL, int WPR, int R>
+__global__ void __launch_bounds__(256)
+gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ y, int n, int k,
+                 int groups)
+{
+    RFQ_TS(0);
+    using IU = IUnit<FMT>;
+    constexpr int TEAMS = 4 / WPR, TL = 64 * WPR;
+    constexpr int D = R < 3 ? R : 3;
+    extern __shared__ __attribute__((aligned(16))) uint32_t xlds[]; // [units][28]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int team = wave / WPR, wit = wave % WPR;
+    const int tl = wit * 64 + lane;
+    const int ku = k >> 5;
+    const size_t rb = row_bytes<FMT>(k);
+
+    bool live[UPL];
+    int unit[UPL];
+#pragma unroll
+    for (int j = 0; j < UPL; j++) {
+        int u = tl + j * TL;
+        live[j] = u < ku;
+        unit[j] = live[j] ? u : ku - 1;
+    }
+    const int rows_per_team = groups * R;
+    const int row0 = (blockIdx.x * TEAMS + team) * rows_per_team;
+    int row_end = row0 + rows_per_team;
+    if (row_end > n) row_end = n;
+    const int row_last = row_end > row0 ? row_end - 1 : (n - 1);
+
+    // x goes first so that it also returns first.
+    float xv[16];
+    const bool prep0 = (int)threadIdx.x < 2 * ku;
+    if (prep0) prep_load(x + (size_t)threadIdx.x * 16, xv);
+
+    IU buf[D][UPL];
+    auto load_row = [&](int slot, int i) {
+        int r = row0 + i;
+        if (r > row_last) r = row_last;
+        const uint8_t *row = w + (size_t)r * rb;
+#pragma unroll
+        for (int j = 0; j < UPL; j++) buf[slot][j].load(row, unit[j]);
+    };
+#pragma unroll
+    for (int d = 0; d < D; d++) load_row(d, d);
+    RFQ_TS(1);
+
+    // Cooperative conversion of x: 2*ku half-units over the 256 threads.
+    if (prep0) prep_convert<IU::NIBBLE, IU::TOPOFF>(xv, threadIdx.x & 1, xlds + (size_t)(threadIdx.x >> 1) * 28);
+    for (int h = threadIdx.x + 256; h < 2 * ku; h += 256) {
+        float xw[16];
+        prep_load(x + (size_t)h * 16, xw);
+        prep_convert<IU::NIBBLE, IU::TOPOFF>(xw, h & 1, xlds + (size_t)(h >> 1) * 28);
+    }
+    RFQ_TS(2);
+    __syncthreads();
+    XPrep xp[UPL];
+#pragma unroll
+    for (int j = 0; j < UPL; j++) {
+        const uint32_t *src = xlds + (size_t)unit[j] * 28;
+#pragma unroll
+        for (int i = 0; i < 24; i += 4) {
+            uint4 v = *reinterpret_cast<const uint4 *>(src + i);
+            xp[j].l[i] = v.x; xp[j].l[i + 1] = v.y; xp[j].l[i + 2] = v.z; xp[j].l[i + 3] = v.w;
+        }
+        xp[j].s = __uint_as_float(src[24]);
+        xp[j].xsum = __uint_as_float(src[25]);
+    }
+    RFQ_TS(3);
+
+    __shared__ float part[R][4];
+    for (int g = 0; g < groups; g++) {
+        const int base = g * R;
+        if (g > 0) {
+#pragma unroll
+            for (int d = 0; d < D; d++) load_row(d, base + d);
+        }
+        float res[R];
+#pragma unroll
+        for (int i = 0; i < R; i++) {
+            float acc = 0.f;
+#pragma unroll
+            for (int j = 0; j < UPL; j++) {
+                float t = buf[i % D][j].idot(xp[j]);
+                acc += live[j] ? t : 0.f;
+            }
+            if (i + D < R) load_row(i % D, base + i + D);
+            res[i] = wave_sum(acc);
+        }
+        RFQ_TS(4);
+        if (WPR == 1) {
+            if (lane == 0) {
+#pragma unroll
+                for (int i = 0; i < R; i++) {
+                    int r = row0 + base + i;
+                    if (r < row_end) y[r] = res[i];
+                }
+            }
+        } else {
+            // `groups` is uniform over the block, so every wavefront reaches
+            // both barriers the same number of times.
+            if (lane == 0) {
+#pragma unroll
+                for (int i = 0; i < R; i++) part[i][wave] = res[i];
+            }
+            __syncthreads();
+            if (wit == 0 && lane < R) {
+                int r = row0 + base + lane;
+                float t = 0.f;
+#pragma unroll
+                for (int q = 0; q < WPR; q++) t += part[lane][team * WPR + q];
+                if (r < row_end) y[r] = t;
+            }
+            __syncthreads();
         }
     }
 }
@@ -381,10 +694,15 @@ gemv_generic_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, 
     }
 }
 
+// Rows in flight per lane: as deep as the register file allows at two
+// wavefronts per SIMD (x: 32*UPL registers, each unit 5..9).
+template <int FMT> struct Depth { static constexpr int D = 8; };
+template <> struct Depth<RFQ_Q8_0> { static constexpr int D = 4; };
+
 template <int FMT, int UPL, int WPR>
 int run_xreg(const uint8_t *w, const float *x, float *y, int n, int k, hipStream_t s)
 {
-    constexpr int TEAMS = 4 / WPR;
+    constexpr int TEAMS = 4 / WPR, D = Depth<FMT>::D;
     // Two resident blocks per CU; then even out the rows so every team walks
     // the same number of them (no straggler tail on a ~10 us kernel).
     int cus = device_cu_count();
@@ -392,9 +710,60 @@ int run_xreg(const uint8_t *w, const float *x, float *y, int n, int k, hipStream
     int rows_per_team = (n + blocks * TEAMS - 1) / (blocks * TEAMS);
     if (rows_per_team < 1) rows_per_team = 1;
     blocks = (n + rows_per_team * TEAMS - 1) / (rows_per_team * TEAMS);
-    hipLaunchKernelGGL((gemv_xreg_kernel<FMT, UPL, WPR>), dim3(blocks), dim3(256), 0, s, w, x, y, n, k, rows_per_team);
+    hipLaunchKernelGGL((gemv_xreg_kernel<FMT, UPL, WPR, D>), dim3(blocks), dim3(256), 0, s, w, x, y, n, k,
+                       rows_per_team);
     RFQ_LAUNCH_CHECK("gemv_xreg_kernel");
     return RFQ_OK;
+}
+
+template <int FMT> struct HasIdot { static constexpr bool value = false; };
+template <> struct HasIdot<RFQ_Q4_K> { static constexpr bool value = true; };
+template <> struct HasIdot<RFQ_Q4_0> { static constexpr bool value = true; };
+template <> struct HasIdot<RFQ_Q8_0> { static constexpr bool value = true; };
+
+template <int FMT, int UPL, int WPR, int R>
+int launch_idot(const uint8_t *w, const float *x, float *y, int n, int k, int blocks, int groups, hipStream_t s)
+{
+    size_t lds = (size_t)(k / 32) * 28 * sizeof(uint32_t);
+    hipLaunchKernelGGL((gemv_idot_kernel<FMT, UPL, WPR, R>), dim3(blocks), dim3(256), lds, s, w, x, y, n, k, groups);
+    RFQ_LAUNCH_CHECK("gemv_idot_kernel");
+    return RFQ_OK;
+}
+
+template <int FMT, int UPL, int WPR>
+int run_idot(const uint8_t *w, const float *x, float *y, int n, int k, hipStream_t s)
+{
+    if constexpr (HasIdot<FMT>::value) {
+        constexpr int TEAMS = 4 / WPR;
+        // Aim at two resident blocks per CU, every team walking the same number
+        // of rows (a straggler is expensive on a ~10 us kernel).  Rows per team
+        // = groups * R with R from a small compiled set; take the pair that
+        // wastes the fewest row slots, the larger R on a tie.
+        const int slots = device_cu_count() * 2;
+        int want = (n + slots * TEAMS - 1) / (slots * TEAMS);
+        if (want < 1) want = 1;
+        static const int RS[4] = {2, 4, 7, 8};
+        int best_r = 8, best_groups = 1, best_blocks = 0;
+        long best_cost = -1;
+        for (int idx = 0; idx < 4; idx++) {
+            int r = RS[idx];
+            int groups = (want + r - 1) / r;
+            int blocks = (n + TEAMS * r * groups - 1) / (TEAMS * r * groups);
+            long waves_of_blocks = (blocks + slots - 1) / slots;
+            long cost = waves_of_blocks * r * groups;
+            if (best_cost < 0 || cost < best_cost || (cost == best_cost && r > best_r)) {
+                best_cost = cost; best_r = r; best_groups = groups; best_blocks = blocks;
+            }
+        }
+        switch (best_r) {
+        case 2: return launch_idot<FMT, UPL, WPR, 2>(w, x, y, n, k, best_blocks, best_groups, s);
+        case 4: return launch_idot<FMT, UPL, WPR, 4>(w, x, y, n, k, best_blocks, best_groups, s);
+        case 7: return launch_idot<FMT, UPL, WPR, 7>(w, x, y, n, k, best_blocks, best_groups, s);
+        default: return launch_idot<FMT, UPL, WPR, 8>(w, x, y, n, k, best_blocks, best_groups, s);
+        }
+    } else {
+        return run_xreg<FMT, UPL, WPR>(w, x, y, n, k, s);
+    }
 }
 
 template <int FMT, int M>
@@ -413,10 +782,10 @@ int run(const uint8_t *w, const float *x, float *y, int m, int n, int k, hipStre
 {
     const int ku = k / 32;
     if (m == 1 && ku > 32) {
-        if (ku <= 64) return run_xreg<FMT, 1, 1>(w, x, y, n, k, s);
-        if (ku <= 128) return run_xreg<FMT, 2, 1>(w, x, y, n, k, s);
-        if (ku <= 256) return run_xreg<FMT, 2, 2>(w, x, y, n, k, s);
-        if (ku <= 512) return run_xreg<FMT, 2, 4>(w, x, y, n, k, s);
+        if (ku <= 64) return run_idot<FMT, 1, 1>(w, x, y, n, k, s);
+        if (ku <= 128) return run_idot<FMT, 2, 1>(w, x, y, n, k, s);
+        if (ku <= 256) return run_idot<FMT, 2, 2>(w, x, y, n, k, s);
+        if (ku <= 512) return run_idot<FMT, 2, 4>(w, x, y, n, k, s);
     }
     switch (m) {
     case 1: return run_generic<FMT, 1>(w, x, y, n, k, s);
