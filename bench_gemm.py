@@ -1,0 +1,57 @@
+"""Prefill GEMM lines of the bench (imported by bench.py; also runnable alone).
+
+MXFP4 GEMM at M=2048, K=8192, N=28672 (bf16 out) and the MXFP6-weight variant,
+plus the Q4_K fp16 GEMM at M=512, K=4096, N=14336 when that kernel is built.
+FLOPs = 2*M*N*K; peaks: 10.1 PFLOP/s (FP4 scaled MFMA), 5.0 (FP8), 2.5 (fp16).
+"""
+from __future__ import annotations
+
+import ctypes as C
+import json
+import sys
+
+import numpy as np
+
+
+def _gauss(rows, k, seed, std):
+    rng = np.random.Generator(np.random.PCG64(seed))
+    return rng.standard_normal((rows, k), dtype=np.float32) * np.float32(std)
+
+
+def mx_gemm(torch, w_fmt, m=2048, n=28672, k=8192, steps=20, warmup=3):
+    from rocmforge_amd import _lib, ops, quantize as Q
+    dev = torch.device("cuda:0")
+    a_raw = Q.pack_mxfp4(_gauss(m, k, 20260005, 1.0))
+    slab_rows = 4096
+    pack = Q.pack_mxfp4 if w_fmt == Q.MXFP4 else Q.pack_mxfp6
+    w_raw = np.tile(pack(_gauss(slab_rows, k, 20260015 + w_fmt, 0.02)), n // slab_rows)
+    A = ops.MxOperand(Q.MXFP4, torch.from_numpy(a_raw).to(dev), m, k)
+    W = ops.MxOperand(w_fmt, torch.from_numpy(w_raw).to(dev), n, k)
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
+    ms = C.c_float(0)
+    L = _lib.lib()
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    args = (C.c_void_p(A.buf.data_ptr()), A.kind, C.c_void_p(W.buf.data_ptr()), W.kind, C.c_void_p(out.data_ptr()),
+            _lib.BF16, m, n, k)
+    _lib.check(L.rfq_bench_gemm_mx(*args, 0, warmup, stream, C.byref(ms)))
+    _lib.check(L.rfq_bench_gemm_mx(*args, 0, steps, stream, C.byref(ms)))
+    t = ms.value / 1e3 / steps
+    flops = 2.0 * m * n * k
+    peak = 10.1e15 if (A.kind == _lib.MX_FP4 and W.kind == _lib.MX_FP4) else 5.0e15
+    return {"TFLOP/s": round(flops / t / 1e12, 1), "us": round(t * 1e6, 1), "mfma_frac": round(flops / t / peak, 4),
+            "peak_TFLOP/s": peak / 1e12, "kinds": [A.kind, W.kind]}
+
+
+def run(torch):
+    from rocmforge_amd import quantize as Q
+    res = {}
+    res["MXFP4 gemm 2048x8192x28672 bf16"] = mx_gemm(torch, Q.MXFP4)
+    res["MXFP6-weight gemm 2048x8192x28672 bf16"] = mx_gemm(torch, Q.MXFP6_E2M3)
+    return res
+
+
+if __name__ == "__main__":
+    import os
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    import torch
+    print(json.dumps(run(torch)))

@@ -1,12 +1,486 @@
+// MXFP4 / MXFP6 prefill GEMM on the gfx950 block-scaled matrix instruction
+// (v_mfma_scale_f32_32x32x64_f8f6f4), plus the one-time operand re-encoding.
+//
+//   out[m, n] = sum_k A[m, k] * W[n, k]          fp32 accumulation in the matrix core
+//
+// Why a re-encoding: ROCmForge stores a signed exponent byte and decodes its
+// E2M1 / E2M3 codes with its own tables (code 1 -> 1.0, code 8 -> -0.5, ...,
+// clamp to +-8 / +-7.5), the instruction wants a biased E8M0 scale and OCP
+// element codes.  Every block is therefore decoded exactly as the reference
+// does and re-expressed, value for value, as
+//   FP4 kind: OCP E2M1 codes {0.5, 1, 2, 4} * 2^(E-127)   (only if the block's
+//             non-zero magnitudes span at most a factor 8 -- always the case
+//             for what the reference's own packer emits), or
+//   FP8 kind: OCP E4M3 codes * 2^(E-127)                   (always possible).
+// The operands keep the reference's values bit for bit, so the GEMM differs
+// from the CPU path only in summation order.
+//
+// Prepared layout ("fragment-major"): rows are grouped in tiles of 32, k in
+// steps of 64 (two MX blocks).  One (row-tile, k-step) page holds what the 64
+// lanes of a wavefront feed into one matrix instruction: lane l = (kb << 5) | r
+// owns row 32*rt + r and the scale of block 2*ks + kb.  FP4: the lane's 16
+// bytes are that block's 32 codes, 1 KiB pages.  FP8: 32 bytes per lane as two
+// 1 KiB half-pages, half-page b = elements 16*kb .. 16*kb+15 of block 2*ks + b
+// (the instruction's 8-bit operand order).  So every global -> LDS ->
+// register hop moves contiguous, 16-byte-per-lane, conflict-free data.
+// Scales follow the data: per (row-tile, group of 4 k-steps) one dword per
+// lane, byte b = scale of k-step 4*g + b (the instruction picks the byte).
+#include <mutex>
+
 #include "rfq_common.hpp"
+
 namespace rfq {
-size_t mx_prepared_bytes(int, int, int, int) { return 0; }
-int launch_mx_prepare(int, int, const uint8_t *, int, int, void *, size_t, int *, hipStream_t)
+namespace {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+struct MxLayout {
+    int rows, k, rt, ks, ks4;
+    size_t page_bytes, data_bytes, scale_bytes;
+    __host__ __device__ size_t total() const { return data_bytes + scale_bytes + 16; } // +16: status words
+};
+
+__host__ __device__ inline MxLayout mx_layout(int kind, int rows, int k)
 {
-    return fail(RFQ_E_UNSUPPORTED, "rfq_mx_prepare: not built yet");
+    MxLayout L;
+    L.rows = rows; L.k = k;
+    L.rt = (rows + 31) / 32;
+    L.ks = k / 64;
+    L.ks4 = (L.ks + 3) / 4;
+    L.page_bytes = kind == RFQ_MX_FP4 ? 1024 : 2048;
+    L.data_bytes = (size_t)L.rt * L.ks * L.page_bytes;
+    L.scale_bytes = (size_t)L.rt * L.ks4 * 256;
+    return L;
 }
-int launch_gemm_mx(const void *, int, const void *, int, void *, int, int, int, int, hipStream_t)
+
+// ---- decode one raw block into the reference's 32 values ----------------------
+
+template <int FMT> __device__ __forceinline__ void decode_block(const uint8_t *blk, float (&v)[32]);
+
+template <> __device__ __forceinline__ void decode_block<RFQ_MXFP4>(const uint8_t *blk, float (&v)[32])
 {
-    return fail(RFQ_E_UNSUPPORTED, "rfq_gemm_mx: not built yet");
+    float scale = mx_scale((int)(int8_t)blk[0]);
+#pragma unroll
+    for (int j = 0; j < 16; j++) {
+        uint32_t b = blk[1 + j];
+        v[2 * j] = clampf(scale * decode_e2m1(b >> 4), -8.0f, 8.0f);
+        v[2 * j + 1] = clampf(scale * decode_e2m1(b & 15u), -8.0f, 8.0f);
+    }
 }
+
+template <> __device__ __forceinline__ void decode_block<RFQ_MXFP6_E2M3>(const uint8_t *blk, float (&v)[32])
+{
+    float scale = mx_scale((int)(int8_t)blk[0]);
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const uint8_t *b = blk + 1 + 3 * j;
+        uint32_t b0 = b[0], b1 = b[1], b2 = b[2];
+        v[4 * j] = clampf(scale * decode_e2m3(b1 >> 2), -7.5f, 7.5f);
+        v[4 * j + 1] = clampf(scale * decode_e2m3((b0 >> 4) | ((b1 & 3u) << 4)), -7.5f, 7.5f);
+        v[4 * j + 2] = clampf(scale * decode_e2m3((b1 >> 6) | ((b2 & 15u) << 2)), -7.5f, 7.5f);
+        v[4 * j + 3] = j < 7 ? clampf(scale * decode_e2m3((uint32_t)b[3] & 63u), -7.5f, 7.5f) : 0.0f;
+    }
+}
+
+// Unbiased binary exponent of a finite non-zero float (subnormals included).
+__device__ __forceinline__ int exponent_of(float a)
+{
+    float t = fabsf(a) * 18446744073709551616.0f; // 2^64: exact, lifts subnormals into the normal range
+    return (int)((__float_as_uint(t) >> 23) & 255u) - 127 - 64;
+}
+
+// ---- re-encoding kernels --------------------------------------------------------
+//
+// One thread per (row, block).  Thread g: lane = g & 63, page = g >> 6.
+// status[0] is set to 1 if an FP4 re-encoding met a block it cannot express.
+
+template <int FMT, int KIND>
+__global__ void __launch_bounds__(256)
+mx_prepare_kernel(const uint8_t *__restrict__ raw, uint8_t *__restrict__ prep, MxLayout L)
+{
+    constexpr int BB = Fmt<FMT>::BB;
+    size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
+    size_t npages = (size_t)L.rt * L.ks;
+    if (g >= npages * 64) return;
+    int lane = (int)(g & 63);
+    size_t page = g >> 6;
+    int rt = (int)(page / L.ks), ks = (int)(page % L.ks);
+    int row = rt * 32 + (lane & 31), kb = ks * 2 + (lane >> 5);
+    uint32_t *status = reinterpret_cast<uint32_t *>(prep + L.data_bytes + L.scale_bytes);
+
+    float v[32];
+    if (row < L.rows) {
+        decode_block<FMT>(raw + ((size_t)row * (L.k / 32) + kb) * BB, v);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 32; i++) v[i] = 0.0f;
+    }
+    float vmax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 32; i++) vmax = fmaxf(vmax, fabsf(v[i]));
+
+    int E = 127; // biased E8M0 scale of the re-encoded block
+    uint32_t out[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) out[i] = 0;
+
+    if (KIND == RFQ_MX_FP4) {
+        // codes 1, 2, 4, 6 are 0.5, 1, 2, 4; put the largest magnitude on 4 (or
+        // lower if the scale exponent would leave the E8M0 range).
+        bool ok = true;
+        if (vmax > 0.0f) {
+            E = exponent_of(vmax) - 2 + 127;
+            if (E < 0) E = 0;
+#pragma unroll
+            for (int i = 0; i < 32; i++) {
+                uint32_t code = 0;
+                if (v[i] != 0.0f) {
+                    uint32_t bits = __float_as_uint(fabsf(v[i]) * 18446744073709551616.0f);
+                    int kx = (int)((bits >> 23) & 255u) - 127 - 64 - (E - 127); // log2(|v| / scale)
+                    bool pow2 = (bits & 0x7FFFFFu) == 0;
+                    if (!pow2 || kx < -1 || kx > 2) ok = false;
+                    code = kx == -1 ? 1u : kx == 0 ? 2u : kx == 1 ? 4u : 6u;
+                    if (v[i] < 0.0f) code |= 8u;
+                }
+                out[i >> 3] |= code << (4 * (i & 7)); // element 2j in the low nibble of byte j
+            }
+        }
+        if (!ok) status[0] = 1u;
+        uint4 *dst = reinterpret_cast<uint4 *>(prep + page * 1024 + (size_t)lane * 16);
+        *dst = make_uint4(out[0], out[1], out[2], out[3]);
+    } else {
+        // E4M3: sign, 4 exponent bits (bias 7), 3 mantissa bits.  Largest
+        // magnitude scaled into [4, 8): every other value of the block is at
+        // most 2^4 below it, inside the normal range.
+        if (vmax > 0.0f) {
+            E = exponent_of(vmax) - 2 + 127;
+            if (E < 0) E = 0;
+#pragma unroll
+            for (int i = 0; i < 32; i++) {
+                uint32_t code = 0;
+                if (v[i] != 0.0f) {
+                    uint32_t bits = __float_as_uint(fabsf(v[i]) * 18446744073709551616.0f);
+                    int p = (int)((bits >> 23) & 255u) - 127 - 64 - (E - 127); // exponent after scaling
+                    uint32_t m3 = (bits >> 20) & 7u;
+                    if (p >= -6) {
+                        code = ((uint32_t)(p + 7) << 3) | m3;
+                    } else if (p >= -9) {
+                        code = (8u | m3) >> (-6 - p); // subnormal: (1.mmm) shifted into the 3 fraction bits
+                    }
+                    if (v[i] < 0.0f) code |= 0x80u;
+                }
+                out[i >> 2] |= code << (8 * (i & 3));
+            }
+        }
+        // 8-bit operands: registers 0-3 of lane (r, h) carry elements 16h..16h+15
+        // of the k-step's FIRST block, registers 4-7 the same elements of its
+        // SECOND block (the scale of lane (r, h) still belongs to block h).
+        // This thread owns block kb = lane >> 5: its low 16 codes go to lane
+        // (r, 0), its high 16 to lane (r, 1), both in half-page kb.
+        uint8_t *dst = prep + page * 2048 + (size_t)(lane >> 5) * 1024 + (size_t)(lane & 31) * 16;
+        *reinterpret_cast<uint4 *>(dst) = make_uint4(out[0], out[1], out[2], out[3]);
+        *reinterpret_cast<uint4 *>(dst + 512) = make_uint4(out[4], out[5], out[6], out[7]);
+    }
+    prep[L.data_bytes + ((size_t)rt * L.ks4 + (ks >> 2)) * 256 + (size_t)lane * 4 + (ks & 3)] = (uint8_t)E;
+}
+
+// Scale bytes of k-steps past the end (k not a multiple of 256) and the status words.
+__global__ void mx_init_kernel(uint8_t *prep, MxLayout L)
+{
+    size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (g < L.scale_bytes) prep[L.data_bytes + g] = 127;
+    if (g < 4) reinterpret_cast<uint32_t *>(prep + L.data_bytes + L.scale_bytes)[g] = 0;
+}
+
+// ---- GEMM ---------------------------------------------------------------------
+//
+// Workgroup = 4 wavefronts, output tile 256 x 256, k advanced 128 per stage
+// (two matrix-instruction k-steps).  Wavefront (wm, wn) owns a 128 x 128
+// quadrant = 4 x 4 instruction tiles, 256 fp32 accumulators per lane.
+// Stage s+1 is fetched from global memory into registers while stage s is
+// multiplied out of LDS; LDS is double-buffered.
+
+template <int KIND> struct Pg { static constexpr int BYTES = KIND == RFQ_MX_FP4 ? 1024 : 2048; };
+template <int KIND> struct Cbsz { static constexpr int V = KIND == RFQ_MX_FP4 ? 4 : 0; };
+
+template <int KIND> __device__ __forceinline__ v8i read_frag(const uint8_t *page, int lane)
+{
+    v8i f;
+    uint4 lo = *reinterpret_cast<const uint4 *>(page + lane * 16);
+    f[0] = (int)lo.x; f[1] = (int)lo.y; f[2] = (int)lo.z; f[3] = (int)lo.w;
+    if (KIND == RFQ_MX_FP4) {
+        f[4] = 0; f[5] = 0; f[6] = 0; f[7] = 0;
+    } else {
+        uint4 hi = *reinterpret_cast<const uint4 *>(page + 1024 + lane * 16);
+        f[4] = (int)hi.x; f[5] = (int)hi.y; f[6] = (int)hi.z; f[7] = (int)hi.w;
+    }
+    return f;
+}
+
+__device__ __forceinline__ uint16_t f32_to_bf16(float f)
+{
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40u); // NaN stays NaN
+    return (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);                  // round to nearest even
+}
+
+constexpr int TM = 256, TN = 256;
+
+template <int AK, int BK_, bool OUT_BF16>
+__global__ void __launch_bounds__(256)
+gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, void *__restrict__ outp, int M, int N,
+               MxLayout LA, MxLayout LB)
+{
+    constexpr int PA = Pg<AK>::BYTES, PB = Pg<BK_>::BYTES;
+    constexpr int A_STAGE = 16 * PA, B_STAGE = 16 * PB;           // 8 row-tiles x 2 k-steps
+    constexpr int S_STAGE = 8 * 256;                              // 8 row-tiles x 64 lanes x dword
+    constexpr int STAGE = A_STAGE + B_STAGE + 2 * S_STAGE;
+    constexpr int A_CH = A_STAGE / 16 / 256, B_CH = B_STAGE / 16 / 256; // 16-byte chunks per thread
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave & 1, wn = wave >> 1;
+    // XCD-aware tile order: consecutive workgroup ids land on different XCDs
+    // (round robin over 8), so ids that share id / 8 run at the same time on
+    // different L2s.  Give each XCD a contiguous run of tiles that walks down
+    // the M tiles of one N tile first: the W tile stays in that XCD's L2.
+    const int tiles_m = (M + TM - 1) / TM, tiles_n = (N + TN - 1) / TN;
+    const int total = tiles_m * tiles_n;
+    int bid = blockIdx.x;
+    {
+        int xcd = bid & 7, slot = bid >> 3;
+        int per = (total + 7) / 8;
+        int t = xcd * per + slot;
+        if (slot >= per || t >= total) return; // uniform over the workgroup
+        bid = t;
+    }
+    const int tn = bid / tiles_m, tmi = bid % tiles_m;
+    const int rtA0 = tmi * 8, rtB0 = tn * 8;
+
+    const uint8_t *a_scale = ap + LA.data_bytes, *b_scale = bp + LB.data_bytes;
+
+    v16f acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+    uint4 ra[A_CH], rb[B_CH], rs;
+    const int nstages = LA.ks / 2;
+
+    // chunk c of a stage's A data: page (c >> 6) / (PA / 1024) ... computed per kind below
+    auto fetch = [&](int st) {
+        const int ks0 = st * 2;
+#pragma unroll
+        for (int i = 0; i < A_CH; i++) {
+            int c = tid + 256 * i;                         // 16-byte chunk inside the stage
+            int rtl = c / (2 * PA / 16);                   // row-tile 0..7 (its two k-step pages are contiguous)
+            int off = c % (2 * PA / 16);
+            int rt = rtA0 + rtl;
+            if (rt >= LA.rt) rt = LA.rt - 1;
+            ra[i] = *reinterpret_cast<const uint4 *>(ap + ((size_t)rt * LA.ks + ks0) * PA + (size_t)off * 16);
+        }
+#pragma unroll
+        for (int i = 0; i < B_CH; i++) {
+            int c = tid + 256 * i;
+            int rtl = c / (2 * PB / 16);
+            int off = c % (2 * PB / 16);
+            int rt = rtB0 + rtl;
+            if (rt >= LB.rt) rt = LB.rt - 1;
+            rb[i] = *reinterpret_cast<const uint4 *>(bp + ((size_t)rt * LB.ks + ks0) * PB + (size_t)off * 16);
+        }
+        {
+            // scales: threads 0..127 fetch A's 8 x 256 bytes, 128..255 B's
+            int c = tid & 127;
+            int rtl = c >> 4, off = c & 15;
+            bool isb = tid >= 128;
+            int rt = (isb ? rtB0 : rtA0) + rtl;
+            int rtmax = isb ? LB.rt : LA.rt;
+            if (rt >= rtmax) rt = rtmax - 1;
+            int ks4n = isb ? LB.ks4 : LA.ks4;
+            const uint8_t *sp = (isb ? b_scale : a_scale) + ((size_t)rt * ks4n + (ks0 >> 2)) * 256 + off * 16;
+            rs = *reinterpret_cast<const uint4 *>(sp);
+        }
+    };
+    auto stash = [&](int buf) {
+        uint8_t *base = lds + buf * STAGE;
+#pragma unroll
+        for (int i = 0; i < A_CH; i++) *reinterpret_cast<uint4 *>(base + (size_t)(tid + 256 * i) * 16) = ra[i];
+#pragma unroll
+        for (int i = 0; i < B_CH; i++)
+            *reinterpret_cast<uint4 *>(base + A_STAGE + (size_t)(tid + 256 * i) * 16) = rb[i];
+        *reinterpret_cast<uint4 *>(base + A_STAGE + B_STAGE + (size_t)tid * 16) = rs;
+    };
+
+    fetch(0);
+    stash(0);
+    __syncthreads();
+
+    for (int st = 0; st < nstages; st++) {
+        const int buf = st & 1;
+        if (st + 1 < nstages) fetch(st + 1);
+
+        const uint8_t *base = lds + buf * STAGE;
+        const uint8_t *sA = base + A_STAGE + B_STAGE, *sB = sA + S_STAGE;
+        // scale dwords of this stage's k-step group; the stage uses bytes
+        // 2*(st&1) and 2*(st&1)+1: shift them down so the byte selectors are
+        // compile-time constants.
+        const int sh = 16 * (st & 1);
+        int sa[4], sb[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            sa[i] = (int)(*reinterpret_cast<const uint32_t *>(sA + ((wm * 4 + i) * 64 + lane) * 4) >> sh);
+            sb[i] = (int)(*reinterpret_cast<const uint32_t *>(sB + ((wn * 4 + i) * 64 + lane) * 4) >> sh);
+        }
+#pragma unroll
+        for (int ksl = 0; ksl < 2; ksl++) {
+            v8i fa[4], fb[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                fa[i] = read_frag<AK>(base + ((wm * 4 + i) * 2 + ksl) * PA, lane);
+                fb[i] = read_frag<BK_>(base + A_STAGE + ((wn * 4 + i) * 2 + ksl) * PB, lane);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    if (ksl == 0)
+                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                            fa[i], fb[j], acc[i][j], Cbsz<AK>::V, Cbsz<BK_>::V, 0, sa[i], 0, sb[j]);
+                    else
+                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                            fa[i], fb[j], acc[i][j], Cbsz<AK>::V, Cbsz<BK_>::V, 1, sa[i], 1, sb[j]);
+                }
+        }
+        if (st + 1 < nstages) stash(buf ^ 1);
+        __syncthreads();
+    }
+
+    // Epilogue.  Accumulator register r of tile (i, j): row 8*(r/4) + 4*(lane/32) + r%4,
+    // column lane % 32.
+    const int m_base = tmi * TM + wm * 128, n_base = tn * TN + wn * 128;
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            int n = n_base + 32 * j + (lane & 31);
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                int m = m_base + 32 * i + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (m < M && n < N) {
+                    if (OUT_BF16)
+                        reinterpret_cast<uint16_t *>(outp)[(size_t)m * N + n] = f32_to_bf16(acc[i][j][r]);
+                    else
+                        reinterpret_cast<float *>(outp)[(size_t)m * N + n] = acc[i][j][r];
+                }
+            }
+        }
+}
+
+template <int AK, int BK_, bool OUT_BF16>
+int run_gemm(const uint8_t *a, const uint8_t *b, void *out, int m, int n, int k, hipStream_t s)
+{
+    MxLayout LA = mx_layout(AK, m, k), LB = mx_layout(BK_, n, k);
+    constexpr size_t STAGE = 16 * Pg<AK>::BYTES + 16 * Pg<BK_>::BYTES + 2 * 8 * 256;
+    constexpr size_t LDS = 2 * STAGE;
+    static std::once_flag once;
+    static hipError_t attr_err = hipSuccess;
+    std::call_once(once, [] {
+        attr_err = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_mx_kernel<AK, BK_, OUT_BF16>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS);
+    });
+    if (attr_err != hipSuccess) return hip_fail(attr_err, "hipFuncSetAttribute(gemm_mx_kernel)");
+    int tiles = ((m + TM - 1) / TM) * ((n + TN - 1) / TN);
+    int per = (tiles + 7) / 8;
+    hipLaunchKernelGGL((gemm_mx_kernel<AK, BK_, OUT_BF16>), dim3(per * 8), dim3(256), LDS, s, a, b, out, m, n, LA, LB);
+    RFQ_LAUNCH_CHECK("gemm_mx_kernel");
+    return RFQ_OK;
+}
+
+template <int FMT, int KIND>
+int run_prepare(const uint8_t *raw, uint8_t *prep, const MxLayout &L, hipStream_t s)
+{
+    size_t threads = (size_t)L.rt * L.ks * 64;
+    size_t init = L.scale_bytes > 4 ? L.scale_bytes : 4;
+    hipLaunchKernelGGL(mx_init_kernel, dim3((unsigned)((init + 255) / 256)), dim3(256), 0, s, prep, L);
+    RFQ_LAUNCH_CHECK("mx_init_kernel");
+    hipLaunchKernelGGL((mx_prepare_kernel<FMT, KIND>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, raw,
+                       prep, L);
+    RFQ_LAUNCH_CHECK("mx_prepare_kernel");
+    return RFQ_OK;
+}
+
+} // namespace
+
+size_t mx_prepared_bytes(int fmt, int kind, int rows, int k)
+{
+    if (fmt != RFQ_MXFP4 && fmt != RFQ_MXFP6_E2M3 && fmt != RFQ_MXFP6_E3M2) return 0;
+    if (rows <= 0 || k <= 0 || k % 128 != 0) return 0;
+    if (kind == RFQ_MX_AUTO) kind = RFQ_MX_FP8;
+    if (kind != RFQ_MX_FP4 && kind != RFQ_MX_FP8) return 0;
+    if (kind == RFQ_MX_FP4 && fmt != RFQ_MXFP4) return 0;
+    return mx_layout(kind, rows, k).total();
+}
+
+int launch_mx_prepare(int fmt, int kind_req, const uint8_t *d_raw, int rows, int k, void *d_prep, size_t prep_bytes,
+                      int *kind_out, hipStream_t s)
+{
+    const bool is4 = fmt == RFQ_MXFP4;
+    if (kind_req == RFQ_MX_FP4 && !is4)
+        return fail(RFQ_E_UNSUPPORTED, "rfq_mx_prepare: MXFP6 has no 4-bit re-encoding");
+    uint8_t *prep = static_cast<uint8_t *>(d_prep);
+    if ((reinterpret_cast<uintptr_t>(prep) & 15u) != 0)
+        return fail(RFQ_E_BADARG, "rfq_mx_prepare: prepared buffer must be 16-byte aligned");
+
+    if (is4 && kind_req != RFQ_MX_FP8) {
+        MxLayout L = mx_layout(RFQ_MX_FP4, rows, k);
+        size_t need = kind_req == RFQ_MX_AUTO ? mx_layout(RFQ_MX_FP8, rows, k).total() : L.total();
+        if (prep_bytes < need)
+            return fail(RFQ_E_SIZE, "rfq_mx_prepare: prepared buffer has %zu bytes, needs %zu", prep_bytes, need);
+        int rc = run_prepare<RFQ_MXFP4, RFQ_MX_FP4>(d_raw, prep, L, s);
+        if (rc != RFQ_OK) return rc;
+        uint32_t status = 0;
+        RFQ_HIP(hipMemcpyAsync(&status, prep + L.data_bytes + L.scale_bytes, 4, hipMemcpyDeviceToHost, s));
+        RFQ_HIP(hipStreamSynchronize(s));
+        if (status == 0) {
+            if (kind_out) *kind_out = RFQ_MX_FP4;
+            return RFQ_OK;
+        }
+        if (kind_req == RFQ_MX_FP4)
+            return fail(RFQ_E_UNSUPPORTED, "rfq_mx_prepare: a block's magnitudes span more than the 4-bit codes hold");
+        // AUTO: fall through to the 8-bit re-encoding
+    }
+    MxLayout L = mx_layout(RFQ_MX_FP8, rows, k);
+    if (prep_bytes < L.total())
+        return fail(RFQ_E_SIZE, "rfq_mx_prepare: prepared buffer has %zu bytes, needs %zu", prep_bytes, L.total());
+    int rc = is4 ? run_prepare<RFQ_MXFP4, RFQ_MX_FP8>(d_raw, prep, L, s)
+                 : run_prepare<RFQ_MXFP6_E2M3, RFQ_MX_FP8>(d_raw, prep, L, s);
+    if (rc != RFQ_OK) return rc;
+    if (kind_out) *kind_out = RFQ_MX_FP8;
+    return RFQ_OK;
+}
+
+int launch_gemm_mx(const void *d_a, int a_kind, const void *d_w, int w_kind, void *d_out, int out_dtype, int m,
+                   int n, int k, hipStream_t s)
+{
+    const uint8_t *a = static_cast<const uint8_t *>(d_a), *b = static_cast<const uint8_t *>(d_w);
+    if (((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15u) != 0)
+        return fail(RFQ_E_BADARG, "rfq_gemm_mx: prepared operands must be 16-byte aligned");
+    const bool bf = out_dtype == RFQ_BF16;
+    if (a_kind == RFQ_MX_FP4 && w_kind == RFQ_MX_FP4)
+        return bf ? run_gemm<RFQ_MX_FP4, RFQ_MX_FP4, true>(a, b, d_out, m, n, k, s)
+                  : run_gemm<RFQ_MX_FP4, RFQ_MX_FP4, false>(a, b, d_out, m, n, k, s);
+    if (a_kind == RFQ_MX_FP4 && w_kind == RFQ_MX_FP8)
+        return bf ? run_gemm<RFQ_MX_FP4, RFQ_MX_FP8, true>(a, b, d_out, m, n, k, s)
+                  : run_gemm<RFQ_MX_FP4, RFQ_MX_FP8, false>(a, b, d_out, m, n, k, s);
+    if (a_kind == RFQ_MX_FP8 && w_kind == RFQ_MX_FP4)
+        return bf ? run_gemm<RFQ_MX_FP8, RFQ_MX_FP4, true>(a, b, d_out, m, n, k, s)
+                  : run_gemm<RFQ_MX_FP8, RFQ_MX_FP4, false>(a, b, d_out, m, n, k, s);
+    return bf ? run_gemm<RFQ_MX_FP8, RFQ_MX_FP8, true>(a, b, d_out, m, n, k, s)
+              : run_gemm<RFQ_MX_FP8, RFQ_MX_FP8, false>(a, b, d_out, m, n, k, s);
+}
+
 } // namespace rfq
