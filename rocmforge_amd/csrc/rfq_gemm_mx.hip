@@ -195,11 +195,16 @@ __global__ void mx_init_kernel(uint8_t *prep, MxLayout L)
 
 // ---- GEMM ---------------------------------------------------------------------
 //
-// Workgroup = 4 wavefronts, output tile 256 x 256, k advanced 128 per stage
-// (two matrix-instruction k-steps).  Wavefront (wm, wn) owns a 128 x 128
-// quadrant = 4 x 4 instruction tiles, 256 fp32 accumulators per lane.
-// Stage s+1 is fetched from global memory into registers while stage s is
-// multiplied out of LDS; LDS is double-buffered.
+// Workgroup = 4 wavefronts in a WM x WN arrangement, each owning TI x TJ
+// instruction tiles (32 x 32) of the output: fp32 accumulators stay in
+// registers for the whole k loop (TI*TJ*16 per lane, one wavefront per SIMD).
+// k advances 128 per stage (two instruction k-steps).  A stage's operand pages
+// and scale dwords are copied global -> LDS by direct-to-LDS loads (no
+// registers in between) into a ring of NST stages, DIST = NST-1 stages ahead of
+// the multiply, so HBM / L2 latency is covered by DIST stages of matrix work.
+// One barrier per stage: after it, every wavefront has finished reading the
+// slot that the next prefetch overwrites, and every wavefront's share of the
+// current stage has landed.
 
 template <int KIND> struct Pg { static constexpr int BYTES = KIND == RFQ_MX_FP4 ? 1024 : 2048; };
 template <int KIND> struct Cbsz { static constexpr int V = KIND == RFQ_MX_FP4 ? 4 : 0; };
@@ -225,27 +230,76 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float f)
     return (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);                  // round to nearest even
 }
 
-constexpr int TM = 256, TN = 256;
+// s_waitcnt with only the vector-memory counter constrained (gfx9 encoding:
+// vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] at [15:14]).
+template <int N> __device__ __forceinline__ void wait_vmcnt()
+{
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
+}
 
-template <int AK, int BK_, bool OUT_BF16>
+// Direct global -> LDS copy, 64 lanes x 16 bytes: lane l's 16 bytes land at
+// lds_addr + 16*l (lds_addr is wave-uniform and travels in M0).  Written as
+// assembly on purpose: the compiler then keeps no book on these copies, so it
+// does not drain them (vmcnt(0)) in front of every LDS read or barrier; the
+// kernel waits for exactly the stage it needs with wait_vmcnt.  Loads the
+// compiler cannot see only make its own waits longer, never shorter: the
+// counter retires in order.
+__device__ __forceinline__ void lds_dma16(const uint8_t *gsrc, uint32_t lds_addr)
+{
+    // M0 is read when the instruction issues; it is put back right after.
+    uint32_t saved_m0;
+    asm volatile("s_mov_b32 %0, m0\n\t"
+                 "s_mov_b32 m0, %2\n\t"
+                 "global_load_lds_dwordx4 %1, off\n\t"
+                 "s_mov_b32 m0, %0"
+                 : "=&s"(saved_m0)
+                 : "v"(gsrc), "s"(lds_addr)
+                 : "memory");
+}
+
+// Workgroup barrier without the memory-model fence of __syncthreads (which
+// would drain every outstanding prefetch); the empty asm statements keep the
+// compiler from moving LDS accesses across it.
+__device__ __forceinline__ void barrier_no_drain()
+{
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
+template <int AK, int BK_, int WM, int WN, int TI, int TJ> struct GemmCfg {
+    static constexpr int RTA = WM * TI, RTB = WN * TJ;          // row tiles per workgroup
+    static constexpr int BM = RTA * 32, BN = RTB * 32;
+    static constexpr int PA = Pg<AK>::BYTES, PB = Pg<BK_>::BYTES;
+    static constexpr int A_STAGE = RTA * 2 * PA, B_STAGE = RTB * 2 * PB;
+    static constexpr int SA_RT = (RTA + 3) / 4 * 4, SB_RT = (RTB + 3) / 4 * 4;
+    static constexpr int S_STAGE = (SA_RT + SB_RT) * 256;
+    static constexpr int STAGE = A_STAGE + B_STAGE + S_STAGE;
+    static constexpr int A_WL = A_STAGE / 1024, B_WL = B_STAGE / 1024, S_WL = S_STAGE / 1024;
+    static constexpr int WL = A_WL + B_WL + S_WL;               // 1 KiB wave-loads per stage
+    static constexpr int WL_MIN = WL / 4, WL_MAX = (WL + 3) / 4; // per wavefront
+    static constexpr int LDS_MAX = 160 * 1024;
+    static constexpr int NST = LDS_MAX / STAGE >= 4 ? 4 : LDS_MAX / STAGE;
+    static constexpr int DIST = NST - 1;
+    static_assert(NST >= 2, "a stage must fit LDS twice");
+    static_assert((DIST - 1) * WL_MIN < 64, "prefetch depth exceeds the load counter");
+};
+
+template <int AK, int BK_, bool OUT_BF16, int WM, int WN, int TI, int TJ>
 __global__ void __launch_bounds__(256)
 gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, void *__restrict__ outp, int M, int N,
                MxLayout LA, MxLayout LB)
 {
-    constexpr int PA = Pg<AK>::BYTES, PB = Pg<BK_>::BYTES;
-    constexpr int A_STAGE = 16 * PA, B_STAGE = 16 * PB;           // 8 row-tiles x 2 k-steps
-    constexpr int S_STAGE = 8 * 256;                              // 8 row-tiles x 64 lanes x dword
-    constexpr int STAGE = A_STAGE + B_STAGE + 2 * S_STAGE;
-    constexpr int A_CH = A_STAGE / 16 / 256, B_CH = B_STAGE / 16 / 256; // 16-byte chunks per thread
+    using C = GemmCfg<AK, BK_, WM, WN, TI, TJ>;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave & 1, wn = wave >> 1;
+    const int wm = wave % WM, wn = wave / WM;
     // XCD-aware tile order: consecutive workgroup ids land on different XCDs
-    // (round robin over 8), so ids that share id / 8 run at the same time on
-    // different L2s.  Give each XCD a contiguous run of tiles that walks down
-    // the M tiles of one N tile first: the W tile stays in that XCD's L2.
-    const int tiles_m = (M + TM - 1) / TM, tiles_n = (N + TN - 1) / TN;
+    // (round robin over 8).  Each XCD gets a contiguous run of tiles that walks
+    // the M tiles of one N tile first, so a W tile is fetched into one L2 only.
+    const int tiles_m = (M + C::BM - 1) / C::BM, tiles_n = (N + C::BN - 1) / C::BN;
     const int total = tiles_m * tiles_n;
     int bid = blockIdx.x;
     {
@@ -256,97 +310,103 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
         bid = t;
     }
     const int tn = bid / tiles_m, tmi = bid % tiles_m;
-    const int rtA0 = tmi * 8, rtB0 = tn * 8;
-
+    const int rtA0 = tmi * C::RTA, rtB0 = tn * C::RTB;
     const uint8_t *a_scale = ap + LA.data_bytes, *b_scale = bp + LB.data_bytes;
 
-    v16f acc[4][4];
+    // Per-lane global source of each of this wavefront's wave-loads at stage 0;
+    // a stage advances data pages by 2 pages and scales by 128 bytes... every
+    // second stage (a scale dword covers 4 k-steps = 2 stages).
+    const uint8_t *src[C::WL_MAX];
+    int kind_of[C::WL_MAX]; // 0 = A data, 1 = B data, 2 = scales
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < C::WL_MAX; i++) {
+        int j = wave + 4 * i;
+        src[i] = ap;
+        kind_of[i] = 3;
+        if (j < C::A_WL) {
+            int off = j * 1024, rtl = off / (2 * C::PA), within = off % (2 * C::PA);
+            int rt = rtA0 + rtl;
+            if (rt >= LA.rt) rt = LA.rt - 1;
+            src[i] = ap + (size_t)rt * LA.ks * C::PA + within + lane * 16;
+            kind_of[i] = 0;
+        } else if (j < C::A_WL + C::B_WL) {
+            int off = (j - C::A_WL) * 1024, rtl = off / (2 * C::PB), within = off % (2 * C::PB);
+            int rt = rtB0 + rtl;
+            if (rt >= LB.rt) rt = LB.rt - 1;
+            src[i] = bp + (size_t)rt * LB.ks * C::PB + within + lane * 16;
+            kind_of[i] = 1;
+        } else if (j < C::WL) {
+            int q = j - C::A_WL - C::B_WL;           // 1 KiB = 4 row tiles x 256 bytes
+            int rtl = q * 4 + (lane >> 4);
+            bool isb = rtl >= C::SA_RT;
+            int r = isb ? rtl - C::SA_RT : rtl;
+            int rt = (isb ? rtB0 : rtA0) + r;
+            int rtmax = isb ? LB.rt : LA.rt;
+            if (rt >= rtmax) rt = rtmax - 1;
+            src[i] = (isb ? b_scale : a_scale) + (size_t)rt * (isb ? LB.ks4 : LA.ks4) * 256 + (lane & 15) * 16;
+            kind_of[i] = 2;
+        }
+    }
+    auto issue = [&](int st) {
+        // LDS byte address of the ring slot (the low 32 bits of a __shared__ pointer)
+        uint32_t slot = (uint32_t)(uintptr_t)(lds + (st % C::NST) * C::STAGE);
+        slot = __builtin_amdgcn_readfirstlane(slot);
 #pragma unroll
-        for (int j = 0; j < 4; j++)
+        for (int i = 0; i < C::WL_MAX; i++) {
+            int j = wave + 4 * i;
+            if (j < C::WL) {
+                size_t adv = kind_of[i] == 0 ? (size_t)st * 2 * C::PA
+                           : kind_of[i] == 1 ? (size_t)st * 2 * C::PB
+                                             : (size_t)(st >> 1) * 256;
+                lds_dma16(src[i] + adv, __builtin_amdgcn_readfirstlane(slot + j * 1024));
+            }
+        }
+    };
+
+    v16f acc[TI][TJ];
+#pragma unroll
+    for (int i = 0; i < TI; i++)
+#pragma unroll
+        for (int j = 0; j < TJ; j++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
-    uint4 ra[A_CH], rb[B_CH], rs;
     const int nstages = LA.ks / 2;
-
-    // chunk c of a stage's A data: page (c >> 6) / (PA / 1024) ... computed per kind below
-    auto fetch = [&](int st) {
-        const int ks0 = st * 2;
 #pragma unroll
-        for (int i = 0; i < A_CH; i++) {
-            int c = tid + 256 * i;                         // 16-byte chunk inside the stage
-            int rtl = c / (2 * PA / 16);                   // row-tile 0..7 (its two k-step pages are contiguous)
-            int off = c % (2 * PA / 16);
-            int rt = rtA0 + rtl;
-            if (rt >= LA.rt) rt = LA.rt - 1;
-            ra[i] = *reinterpret_cast<const uint4 *>(ap + ((size_t)rt * LA.ks + ks0) * PA + (size_t)off * 16);
-        }
-#pragma unroll
-        for (int i = 0; i < B_CH; i++) {
-            int c = tid + 256 * i;
-            int rtl = c / (2 * PB / 16);
-            int off = c % (2 * PB / 16);
-            int rt = rtB0 + rtl;
-            if (rt >= LB.rt) rt = LB.rt - 1;
-            rb[i] = *reinterpret_cast<const uint4 *>(bp + ((size_t)rt * LB.ks + ks0) * PB + (size_t)off * 16);
-        }
-        {
-            // scales: threads 0..127 fetch A's 8 x 256 bytes, 128..255 B's
-            int c = tid & 127;
-            int rtl = c >> 4, off = c & 15;
-            bool isb = tid >= 128;
-            int rt = (isb ? rtB0 : rtA0) + rtl;
-            int rtmax = isb ? LB.rt : LA.rt;
-            if (rt >= rtmax) rt = rtmax - 1;
-            int ks4n = isb ? LB.ks4 : LA.ks4;
-            const uint8_t *sp = (isb ? b_scale : a_scale) + ((size_t)rt * ks4n + (ks0 >> 2)) * 256 + off * 16;
-            rs = *reinterpret_cast<const uint4 *>(sp);
-        }
-    };
-    auto stash = [&](int buf) {
-        uint8_t *base = lds + buf * STAGE;
-#pragma unroll
-        for (int i = 0; i < A_CH; i++) *reinterpret_cast<uint4 *>(base + (size_t)(tid + 256 * i) * 16) = ra[i];
-#pragma unroll
-        for (int i = 0; i < B_CH; i++)
-            *reinterpret_cast<uint4 *>(base + A_STAGE + (size_t)(tid + 256 * i) * 16) = rb[i];
-        *reinterpret_cast<uint4 *>(base + A_STAGE + B_STAGE + (size_t)tid * 16) = rs;
-    };
-
-    fetch(0);
-    stash(0);
-    __syncthreads();
+    for (int d = 0; d < C::DIST; d++)
+        if (d < nstages) issue(d);
 
     for (int st = 0; st < nstages; st++) {
-        const int buf = st & 1;
-        if (st + 1 < nstages) fetch(st + 1);
+        // stage st has landed once at most the later DIST-1 stages are outstanding
+        if (st + C::DIST - 1 < nstages) wait_vmcnt<(C::DIST - 1) * C::WL_MIN>();
+        else wait_vmcnt<0>();
+        barrier_no_drain();
+        if (st + C::DIST < nstages) issue(st + C::DIST);
 
-        const uint8_t *base = lds + buf * STAGE;
-        const uint8_t *sA = base + A_STAGE + B_STAGE, *sB = sA + S_STAGE;
-        // scale dwords of this stage's k-step group; the stage uses bytes
-        // 2*(st&1) and 2*(st&1)+1: shift them down so the byte selectors are
-        // compile-time constants.
+        const uint8_t *base = lds + (st % C::NST) * C::STAGE;
+        const uint8_t *sA = base + C::A_STAGE + C::B_STAGE, *sB = sA + C::SA_RT * 256;
+        // The stage uses scale bytes 2*(st&1) and 2*(st&1)+1 of its dwords:
+        // shift them down so the instruction's byte selectors are constants.
         const int sh = 16 * (st & 1);
-        int sa[4], sb[4];
+        int sa[TI], sb[TJ];
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            sa[i] = (int)(*reinterpret_cast<const uint32_t *>(sA + ((wm * 4 + i) * 64 + lane) * 4) >> sh);
-            sb[i] = (int)(*reinterpret_cast<const uint32_t *>(sB + ((wn * 4 + i) * 64 + lane) * 4) >> sh);
-        }
+        for (int i = 0; i < TI; i++)
+            sa[i] = (int)(*reinterpret_cast<const uint32_t *>(sA + ((wm * TI + i) * 64 + lane) * 4) >> sh);
+#pragma unroll
+        for (int j = 0; j < TJ; j++)
+            sb[j] = (int)(*reinterpret_cast<const uint32_t *>(sB + ((wn * TJ + j) * 64 + lane) * 4) >> sh);
 #pragma unroll
         for (int ksl = 0; ksl < 2; ksl++) {
-            v8i fa[4], fb[4];
+            v8i fa[TI], fb[TJ];
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                fa[i] = read_frag<AK>(base + ((wm * 4 + i) * 2 + ksl) * PA, lane);
-                fb[i] = read_frag<BK_>(base + A_STAGE + ((wn * 4 + i) * 2 + ksl) * PB, lane);
-            }
+            for (int i = 0; i < TI; i++) fa[i] = read_frag<AK>(base + ((wm * TI + i) * 2 + ksl) * C::PA, lane);
 #pragma unroll
-            for (int i = 0; i < 4; i++)
+            for (int j = 0; j < TJ; j++)
+                fb[j] = read_frag<BK_>(base + C::A_STAGE + ((wn * TJ + j) * 2 + ksl) * C::PB, lane);
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
+            for (int i = 0; i < TI; i++)
+#pragma unroll
+                for (int j = 0; j < TJ; j++) {
                     if (ksl == 0)
                         acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
                             fa[i], fb[j], acc[i][j], Cbsz<AK>::V, Cbsz<BK_>::V, 0, sa[i], 0, sb[j]);
@@ -355,17 +415,15 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
                             fa[i], fb[j], acc[i][j], Cbsz<AK>::V, Cbsz<BK_>::V, 1, sa[i], 1, sb[j]);
                 }
         }
-        if (st + 1 < nstages) stash(buf ^ 1);
-        __syncthreads();
     }
 
     // Epilogue.  Accumulator register r of tile (i, j): row 8*(r/4) + 4*(lane/32) + r%4,
     // column lane % 32.
-    const int m_base = tmi * TM + wm * 128, n_base = tn * TN + wn * 128;
+    const int m_base = tmi * C::BM + wm * TI * 32, n_base = tn * C::BN + wn * TJ * 32;
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < TI; i++)
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
+        for (int j = 0; j < TJ; j++) {
             int n = n_base + 32 * j + (lane & 31);
 #pragma unroll
             for (int r = 0; r < 16; r++) {
@@ -380,24 +438,44 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
         }
 }
 
-template <int AK, int BK_, bool OUT_BF16>
-int run_gemm(const uint8_t *a, const uint8_t *b, void *out, int m, int n, int k, hipStream_t s)
+template <int AK, int BK_, bool OUT_BF16, int WM, int WN, int TI, int TJ>
+int launch_gemm_cfg(const uint8_t *a, const uint8_t *b, void *out, int m, int n, int k, hipStream_t s)
 {
+    using C = GemmCfg<AK, BK_, WM, WN, TI, TJ>;
     MxLayout LA = mx_layout(AK, m, k), LB = mx_layout(BK_, n, k);
-    constexpr size_t STAGE = 16 * Pg<AK>::BYTES + 16 * Pg<BK_>::BYTES + 2 * 8 * 256;
-    constexpr size_t LDS = 2 * STAGE;
+    constexpr size_t LDS = (size_t)C::NST * C::STAGE;
     static std::once_flag once;
     static hipError_t attr_err = hipSuccess;
     std::call_once(once, [] {
-        attr_err = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_mx_kernel<AK, BK_, OUT_BF16>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS);
+        attr_err = hipFuncSetAttribute(
+            reinterpret_cast<const void *>(&gemm_mx_kernel<AK, BK_, OUT_BF16, WM, WN, TI, TJ>),
+            hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS);
     });
     if (attr_err != hipSuccess) return hip_fail(attr_err, "hipFuncSetAttribute(gemm_mx_kernel)");
-    int tiles = ((m + TM - 1) / TM) * ((n + TN - 1) / TN);
+    int tiles = ((m + C::BM - 1) / C::BM) * ((n + C::BN - 1) / C::BN);
     int per = (tiles + 7) / 8;
-    hipLaunchKernelGGL((gemm_mx_kernel<AK, BK_, OUT_BF16>), dim3(per * 8), dim3(256), LDS, s, a, b, out, m, n, LA, LB);
+    hipLaunchKernelGGL((gemm_mx_kernel<AK, BK_, OUT_BF16, WM, WN, TI, TJ>), dim3(per * 8), dim3(256), LDS, s, a, b,
+                       out, m, n, LA, LB);
     RFQ_LAUNCH_CHECK("gemm_mx_kernel");
     return RFQ_OK;
+}
+
+// Two output tilings: 256 x 256 (2 x 2 wavefronts of 4 x 4 tiles) and 256 x 224
+// (4 x 1 wavefronts of 2 x 7 tiles).  The one that leaves the last round of
+// workgroups fuller wins (28672 = 128 * 224 fills 256 CUs exactly four times
+// at M = 2048; 256-wide tiles would run 3.5 rounds).
+template <int AK, int BK_, bool OUT_BF16>
+int run_gemm(const uint8_t *a, const uint8_t *b, void *out, int m, int n, int k, hipStream_t s)
+{
+    const int cus = device_cu_count();
+    auto rounds_cost = [&](int bm, int bn) {
+        long tiles = (long)((m + bm - 1) / bm) * ((n + bn - 1) / bn);
+        long rounds = (tiles + cus - 1) / cus;
+        return (double)rounds * bm * bn; // time ~ rounds x tile area
+    };
+    if (rounds_cost(256, 224) < rounds_cost(256, 256))
+        return launch_gemm_cfg<AK, BK_, OUT_BF16, 4, 1, 2, 7>(a, b, out, m, n, k, s);
+    return launch_gemm_cfg<AK, BK_, OUT_BF16, 2, 2, 4, 4>(a, b, out, m, n, k, s);
 }
 
 template <int FMT, int KIND>
