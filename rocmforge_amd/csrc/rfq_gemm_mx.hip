@@ -29,6 +29,23 @@
 
 #include "rfq_common.hpp"
 
+// Tuning builds can switch parts of the GEMM off (-DRFQ_MX_ABLATE=bits: 1 no
+// matrix instructions, 2 no global->LDS copies after the prologue, 4 no LDS
+// fragment reads inside the loop, 8 no output stores); the library is built without it.
+#ifndef RFQ_MX_ABLATE
+#define RFQ_MX_ABLATE 0
+#endif
+// -DRFQ_MX_TRACE: wavefront 0 of every workgroup sums the shader-clock cycles
+// it spends in each section of a stage and writes them to rfq_mx_trace.
+#ifdef RFQ_MX_TRACE
+__device__ unsigned long long *rfq_mx_trace;
+#define RFQ_MX_T(n) unsigned long long t##n = __builtin_readcyclecounter()
+#define RFQ_MX_ACC(slot, a, b) tacc[slot] += (b) - (a)
+#else
+#define RFQ_MX_T(n) do { } while (0)
+#define RFQ_MX_ACC(slot, a, b) do { } while (0)
+#endif
+
 namespace rfq {
 namespace {
 
@@ -200,11 +217,12 @@ __global__ void mx_init_kernel(uint8_t *prep, MxLayout L)
 // registers for the whole k loop (TI*TJ*16 per lane, one wavefront per SIMD).
 // k advances 128 per stage (two instruction k-steps).  A stage's operand pages
 // and scale dwords are copied global -> LDS by direct-to-LDS loads (no
-// registers in between) into a ring of NST stages, DIST = NST-1 stages ahead of
-// the multiply, so HBM / L2 latency is covered by DIST stages of matrix work.
-// One barrier per stage: after it, every wavefront has finished reading the
-// slot that the next prefetch overwrites, and every wavefront's share of the
-// current stage has landed.
+// registers in between) into a ring of NST slots; a slot is refilled NST
+// stages ahead as soon as every wavefront has read it for the last time, so
+// HBM / L2 latency is covered by more than NST-1 stages of matrix work.
+// One barrier per stage, in the middle of it: after it every wavefront is done
+// with the current slot and every wavefront's share of the next stage has
+// landed.
 
 template <int KIND> struct Pg { static constexpr int BYTES = KIND == RFQ_MX_FP4 ? 1024 : 2048; };
 template <int KIND> struct Cbsz { static constexpr int V = KIND == RFQ_MX_FP4 ? 4 : 0; };
@@ -280,10 +298,9 @@ template <int AK, int BK_, int WM, int WN, int TI, int TJ> struct GemmCfg {
     static constexpr int WL = A_WL + B_WL + S_WL;               // 1 KiB wave-loads per stage
     static constexpr int WL_MIN = WL / 4, WL_MAX = (WL + 3) / 4; // per wavefront
     static constexpr int LDS_MAX = 160 * 1024;
-    static constexpr int NST = LDS_MAX / STAGE >= 4 ? 4 : LDS_MAX / STAGE;
-    static constexpr int DIST = NST - 1;
+    static constexpr int NST = LDS_MAX / STAGE >= 4 ? 4 : LDS_MAX / STAGE; // ring slots
     static_assert(NST >= 2, "a stage must fit LDS twice");
-    static_assert((DIST - 1) * WL_MIN < 64, "prefetch depth exceeds the load counter");
+    static_assert((NST - 1) * WL_MIN < 64, "prefetch depth exceeds the load counter");
 };
 
 template <int AK, int BK_, bool OUT_BF16, int WM, int WN, int TI, int TJ>
@@ -294,7 +311,8 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
     using C = GemmCfg<AK, BK_, WM, WN, TI, TJ>;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6); // uniform, and the compiler may know it
     const int wm = wave % WM, wn = wave / WM;
     // XCD-aware tile order: consecutive workgroup ids land on different XCDs
     // (round robin over 8).  Each XCD gets a contiguous run of tiles that walks
@@ -347,20 +365,22 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
             kind_of[i] = 2;
         }
     }
+    // i-th copy of stage `st` by this wavefront into the ring slot at LDS address `slot`
+    auto issue_piece = [&](int st, uint32_t slot, int i) {
+        int j = wave + 4 * i;
+        if (j < C::WL) {
+            size_t adv = kind_of[i] == 0 ? (size_t)st * 2 * C::PA
+                       : kind_of[i] == 1 ? (size_t)st * 2 * C::PB
+                                         : (size_t)(st >> 1) * 256;
+            lds_dma16(src[i] + adv, __builtin_amdgcn_readfirstlane(slot + j * 1024));
+        }
+    };
     auto issue = [&](int st) {
         // LDS byte address of the ring slot (the low 32 bits of a __shared__ pointer)
         uint32_t slot = (uint32_t)(uintptr_t)(lds + (st % C::NST) * C::STAGE);
         slot = __builtin_amdgcn_readfirstlane(slot);
 #pragma unroll
-        for (int i = 0; i < C::WL_MAX; i++) {
-            int j = wave + 4 * i;
-            if (j < C::WL) {
-                size_t adv = kind_of[i] == 0 ? (size_t)st * 2 * C::PA
-                           : kind_of[i] == 1 ? (size_t)st * 2 * C::PB
-                                             : (size_t)(st >> 1) * 256;
-                lds_dma16(src[i] + adv, __builtin_amdgcn_readfirstlane(slot + j * 1024));
-            }
-        }
+        for (int i = 0; i < C::WL_MAX; i++) issue_piece(st, slot, i);
     };
 
     v16f acc[TI][TJ];
@@ -372,70 +392,198 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
     const int nstages = LA.ks / 2;
+    // Ring prologue: NST stages requested, stage 0 awaited.
 #pragma unroll
-    for (int d = 0; d < C::DIST; d++)
+    for (int d = 0; d < C::NST; d++)
         if (d < nstages) issue(d);
+    if (C::NST - 1 < nstages) wait_vmcnt<(C::NST - 1) * C::WL_MIN>();
+    else wait_vmcnt<0>();
+    barrier_no_drain();
 
-    for (int st = 0; st < nstages; st++) {
-        // stage st has landed once at most the later DIST-1 stages are outstanding
-        if (st + C::DIST - 1 < nstages) wait_vmcnt<(C::DIST - 1) * C::WL_MIN>();
-        else wait_vmcnt<0>();
-        barrier_no_drain();
-        if (st + C::DIST < nstages) issue(st + C::DIST);
-
-        const uint8_t *base = lds + (st % C::NST) * C::STAGE;
+    // One wavefront per SIMD owns the matrix core, so nothing but this
+    // instruction stream can hide latency: fragment registers are
+    // double-buffered by hand and every other piece of work of a stage (LDS
+    // reads of the next k-step, the refill copies, the barrier) is slotted
+    // between two matrix instructions (32 cycles each).  sched_barrier pins
+    // that order against the compiler's instruction scheduler.
+    constexpr int NMMA = TI * TJ, NFRAG = TI + TJ;
+    constexpr int PPS = (C::WL_MAX + NMMA - 1) / NMMA;      // refill copies per matrix-instruction slot
+    static_assert(NFRAG + 1 <= NMMA, "not enough matrix instructions to hide the fragment reads");
+    v8i fa0[TI], fb0[TJ], fa1[TI], fb1[TJ];
+    int sa[TI], sb[TJ], sa_n[TI], sb_n[TJ];
+    auto read_piece = [&](const uint8_t *base, int ksl, int q, v8i (&fa)[TI], v8i (&fb)[TJ]) {
+        if (q < TI) fa[q] = read_frag<AK>(base + ((wm * TI + q) * 2 + ksl) * C::PA, lane);
+        else fb[q - TI] = read_frag<BK_>(base + C::A_STAGE + ((wn * TJ + (q - TI)) * 2 + ksl) * C::PB, lane);
+    };
+    // The stage uses scale bytes 2*(st&1) and 2*(st&1)+1 of its dwords: shift
+    // them down so the instruction's byte selectors are constants.
+    auto scale_piece = [&](const uint8_t *base, int st, int q, int (&xa)[TI], int (&xb)[TJ]) {
         const uint8_t *sA = base + C::A_STAGE + C::B_STAGE, *sB = sA + C::SA_RT * 256;
-        // The stage uses scale bytes 2*(st&1) and 2*(st&1)+1 of its dwords:
-        // shift them down so the instruction's byte selectors are constants.
         const int sh = 16 * (st & 1);
-        int sa[TI], sb[TJ];
+        if (q < TI) xa[q] = (int)(*reinterpret_cast<const uint32_t *>(sA + ((wm * TI + q) * 64 + lane) * 4) >> sh);
+        else xb[q - TI] = (int)(*reinterpret_cast<const uint32_t *>(sB + ((wn * TJ + (q - TI)) * 64 + lane) * 4) >> sh);
+    };
 #pragma unroll
-        for (int i = 0; i < TI; i++)
-            sa[i] = (int)(*reinterpret_cast<const uint32_t *>(sA + ((wm * TI + i) * 64 + lane) * 4) >> sh);
-#pragma unroll
-        for (int j = 0; j < TJ; j++)
-            sb[j] = (int)(*reinterpret_cast<const uint32_t *>(sB + ((wn * TJ + j) * 64 + lane) * 4) >> sh);
-#pragma unroll
-        for (int ksl = 0; ksl < 2; ksl++) {
-            v8i fa[TI], fb[TJ];
-#pragma unroll
-            for (int i = 0; i < TI; i++) fa[i] = read_frag<AK>(base + ((wm * TI + i) * 2 + ksl) * C::PA, lane);
-#pragma unroll
-            for (int j = 0; j < TJ; j++)
-                fb[j] = read_frag<BK_>(base + C::A_STAGE + ((wn * TJ + j) * 2 + ksl) * C::PB, lane);
-#pragma unroll
-            for (int i = 0; i < TI; i++)
-#pragma unroll
-                for (int j = 0; j < TJ; j++) {
-                    if (ksl == 0)
-                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                            fa[i], fb[j], acc[i][j], Cbsz<AK>::V, Cbsz<BK_>::V, 0, sa[i], 0, sb[j]);
-                    else
-                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                            fa[i], fb[j], acc[i][j], Cbsz<AK>::V, Cbsz<BK_>::V, 1, sa[i], 1, sb[j]);
-                }
-        }
+    for (int q = 0; q < NFRAG; q++) {
+        read_piece(lds, 0, q, fa0, fb0);
+        scale_piece(lds, 0, q, sa, sb);
     }
 
-    // Epilogue.  Accumulator register r of tile (i, j): row 8*(r/4) + 4*(lane/32) + r%4,
-    // column lane % 32.
+#ifdef RFQ_MX_TRACE
+    unsigned long long tacc[6] = {0, 0, 0, 0, 0, 0};
+    unsigned long long t_begin = __builtin_readcyclecounter();
+#endif
+    for (int st = 0; st < nstages; st++) {
+        RFQ_MX_T(0);
+        const uint8_t *base = lds + (st % C::NST) * C::STAGE;
+        const uint8_t *nbase = lds + ((st + 1) % C::NST) * C::STAGE;
+        const bool more = st + 1 < nstages;
+        const bool refill = st + C::NST < nstages;
+        uint32_t slot = (uint32_t)(uintptr_t)(lds + (st % C::NST) * C::STAGE);
+        slot = __builtin_amdgcn_readfirstlane(slot);
+
+        // k-step 0 of the stage; its shadow: reads of k-step 1, then the hand-over.
+#pragma unroll
+        for (int q = 0; q < NMMA; q++) {
+            if (!(RFQ_MX_ABLATE & 1))
+                acc[q / TJ][q % TJ] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                    fa0[q / TJ], fb0[q % TJ], acc[q / TJ][q % TJ], Cbsz<AK>::V, Cbsz<BK_>::V, 0, sa[q / TJ], 0,
+                    sb[q % TJ]);
+            __builtin_amdgcn_sched_barrier(0);
+            if (q < NFRAG && !(RFQ_MX_ABLATE & 4)) read_piece(base, 1, q, fa1, fb1);
+            if (q == NMMA - 2) {
+                RFQ_MX_T(1);
+                RFQ_MX_ACC(0, t0, t1);
+                // Hand-over: this wavefront's last reads of the slot are
+                // complete (lgkmcnt), the next stage has landed (vmcnt),
+                // everyone agrees (barrier).  Afterwards the slot may be
+                // refilled NST stages ahead.
+                __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0) only
+                RFQ_MX_T(2);
+                RFQ_MX_ACC(1, t1, t2);
+                if (more) {
+                    if (st + C::NST - 1 < nstages) wait_vmcnt<(C::NST - 2) * C::WL_MIN>();
+                    else wait_vmcnt<0>();
+                }
+                RFQ_MX_T(3);
+                RFQ_MX_ACC(2, t2, t3);
+                barrier_no_drain();
+                RFQ_MX_T(4);
+                RFQ_MX_ACC(3, t3, t4);
+#ifdef RFQ_MX_TRACE
+                tacc[5] = t4; // start of the second half
+#endif
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // k-step 1; its shadow: refill copies, reads of the next stage's k-step 0 and scales.
+#pragma unroll
+        for (int q = 0; q < NMMA; q++) {
+            if (!(RFQ_MX_ABLATE & 1))
+                acc[q / TJ][q % TJ] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                    fa1[q / TJ], fb1[q % TJ], acc[q / TJ][q % TJ], Cbsz<AK>::V, Cbsz<BK_>::V, 1, sa[q / TJ], 1,
+                    sb[q % TJ]);
+            __builtin_amdgcn_sched_barrier(0);
+            if (refill && !(RFQ_MX_ABLATE & 2)) {
+#pragma unroll
+                for (int pp = 0; pp < PPS; pp++)
+                    if (q * PPS + pp < C::WL_MAX) issue_piece(st + C::NST, slot, q * PPS + pp);
+            }
+            if (q < NFRAG && more) {
+                if (!(RFQ_MX_ABLATE & 4)) read_piece(nbase, 0, q, fa0, fb0);
+                scale_piece(nbase, st + 1, q, sa_n, sb_n);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (RFQ_MX_ABLATE & 1) {
+#pragma unroll
+            for (int i = 0; i < TI; i++) acc[i][0][0] += (float)(fa0[i][0] ^ fa1[i][1]);
+#pragma unroll
+            for (int j = 0; j < TJ; j++) acc[0][j][1] += (float)(fb0[j][0] ^ fb1[j][1]);
+        }
+#pragma unroll
+        for (int i = 0; i < TI; i++) sa[i] = sa_n[i];
+#pragma unroll
+        for (int j = 0; j < TJ; j++) sb[j] = sb_n[j];
+#ifdef RFQ_MX_TRACE
+        {
+            unsigned long long t9 = __builtin_readcyclecounter();
+            tacc[4] += t9 - tacc[5];
+        }
+#endif
+    }
+#ifdef RFQ_MX_TRACE
+    unsigned long long t_loop_end = __builtin_readcyclecounter();
+#endif
+
+    // Epilogue.  Accumulator register r of tile (i, j) is row
+    // 8*(r/4) + 4*(lane/32) + r%4, column lane%32 of the tile: a lane owns
+    // single elements scattered over rows.  Interior wavefront blocks go through
+    // LDS (the ring is free now), one 32-row band at a time, and leave as whole
+    // rows in 16-byte stores; ragged blocks fall back to element stores.
+    constexpr int ES = OUT_BF16 ? 2 : 4;
+    constexpr int ROW_BYTES = TJ * 32 * ES;                 // one band row of this wavefront
+    constexpr int ROW_STRIDE = ROW_BYTES + 16;              // +4 dwords: the two half-waves (rows R, R+4) miss each other's banks
+    constexpr int CPR = ROW_BYTES / 16;                     // 16-byte chunks per row
+    static_assert(4 * 32 * ROW_STRIDE <= C::NST * C::STAGE, "epilogue staging exceeds the ring");
     const int m_base = tmi * C::BM + wm * TI * 32, n_base = tn * C::BN + wn * TJ * 32;
+    const bool interior = m_base + TI * 32 <= M && n_base + TJ * 32 <= N && ((size_t)N * ES) % 16 == 0 &&
+                          (reinterpret_cast<uintptr_t>(outp) & 15u) == 0 && !(RFQ_MX_ABLATE & 8);
+    barrier_no_drain(); // every wavefront is past its last fragment read
+    uint8_t *stage = lds + (size_t)wave * 32 * ROW_STRIDE;
+    if (interior) {
 #pragma unroll
-    for (int i = 0; i < TI; i++)
+        for (int i = 0; i < TI; i++) {
 #pragma unroll
-        for (int j = 0; j < TJ; j++) {
-            int n = n_base + 32 * j + (lane & 31);
+            for (int j = 0; j < TJ; j++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                int m = m_base + 32 * i + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                if (m < M && n < N) {
-                    if (OUT_BF16)
-                        reinterpret_cast<uint16_t *>(outp)[(size_t)m * N + n] = f32_to_bf16(acc[i][j][r]);
-                    else
-                        reinterpret_cast<float *>(outp)[(size_t)m * N + n] = acc[i][j][r];
+                for (int r = 0; r < 16; r++) {
+                    int row = 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                    uint8_t *dst = stage + row * ROW_STRIDE + (32 * j + (lane & 31)) * ES;
+                    if (OUT_BF16) *reinterpret_cast<uint16_t *>(dst) = f32_to_bf16(acc[i][j][r]);
+                    else *reinterpret_cast<float *>(dst) = acc[i][j][r];
+                }
+            // LDS operations of one wavefront execute in order: no barrier needed
+            // between its own writes and reads of its own staging area.
+#pragma unroll
+            for (int c0 = 0; c0 < 32 * CPR; c0 += 64) {
+                int c = c0 + lane;
+                if (c < 32 * CPR) {
+                    int row = c / CPR, col16 = c % CPR;
+                    uint4 v = *reinterpret_cast<const uint4 *>(stage + row * ROW_STRIDE + col16 * 16);
+                    uint8_t *o = reinterpret_cast<uint8_t *>(outp) +
+                                 ((size_t)(m_base + 32 * i + row) * N + n_base) * ES + col16 * 16;
+                    *reinterpret_cast<uint4 *>(o) = v;
                 }
             }
         }
+    } else {
+#pragma unroll
+        for (int i = 0; i < TI; i++)
+#pragma unroll
+            for (int j = 0; j < TJ; j++) {
+                int n = n_base + 32 * j + (lane & 31);
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    int m = m_base + 32 * i + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                    if ((RFQ_MX_ABLATE & 8) && (i | j | r)) continue;
+                    if (m < M && n < N) {
+                        if (OUT_BF16)
+                            reinterpret_cast<uint16_t *>(outp)[(size_t)m * N + n] = f32_to_bf16(acc[i][j][r]);
+                        else
+                            reinterpret_cast<float *>(outp)[(size_t)m * N + n] = acc[i][j][r];
+                    }
+                }
+            }
+    }
+#ifdef RFQ_MX_TRACE
+    if (tid == 0 && rfq_mx_trace) {
+        unsigned long long t_end = __builtin_readcyclecounter();
+        unsigned long long *o = rfq_mx_trace + (size_t)blockIdx.x * 8;
+        o[0] = tacc[0]; o[1] = tacc[1]; o[2] = tacc[2]; o[3] = tacc[3]; o[4] = tacc[4];
+        o[5] = t_loop_end - t_begin; o[6] = t_end - t_loop_end; o[7] = t_begin;
+    }
+#endif
 }
 
 template <int AK, int BK_, bool OUT_BF16, int WM, int WN, int TI, int TJ>
