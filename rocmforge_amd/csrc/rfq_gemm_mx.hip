@@ -29,27 +29,27 @@
 
 #include "rfq_common.hpp"
 
-// Tuning builds can switch parts of the GEMM off (-DRFQ_MX_ABLATE=bits: 1 no
-// matrix instructions, 2 no global->LDS copies after the prologue, 4 no LDS
-// fragment reads inside the loop, 8 no output stores); the library is built without it.
-#ifndef RFQ_MX_ABLATE
-#define RFQ_MX_ABLATE 0
-#endif
-// -DRFQ_MX_TRACE: wavefront 0 of every workgroup sums the shader-clock cycles
-// it spends in each section of a stage and writes them to rfq_mx_trace.
+// -DRFQ_MX_TRACE (tuning builds): every workgroup records wall-clock stamps
+// (100 MHz) at kernel entry, loop entry, loop exit and exit.
 #ifdef RFQ_MX_TRACE
 __device__ unsigned long long *rfq_mx_trace;
-#define RFQ_MX_T(n) unsigned long long t##n = __builtin_readcyclecounter()
-#define RFQ_MX_ACC(slot, a, b) tacc[slot] += (b) - (a)
+#define RFQ_MX_STAMP(slot)                                                                                     \
+    do {                                                                                                       \
+        if (threadIdx.x == 0 && rfq_mx_trace) rfq_mx_trace[(size_t)blockIdx.x * 4 + (slot)] = wall_clock64(); \
+    } while (0)
 #else
-#define RFQ_MX_T(n) do { } while (0)
-#define RFQ_MX_ACC(slot, a, b) do { } while (0)
+#define RFQ_MX_STAMP(slot) do { } while (0)
+#endif
+// Ring depth (W slots in LDS = A fragment sets in registers) of the 4-bit kernel.
+#ifndef RFQ_MX_RING
+#define RFQ_MX_RING 6
 #endif
 
 namespace rfq {
 namespace {
 
 typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
 struct MxLayout {
@@ -212,17 +212,9 @@ __global__ void mx_init_kernel(uint8_t *prep, MxLayout L)
 
 // ---- GEMM ---------------------------------------------------------------------
 //
-// Workgroup = 4 wavefronts in a WM x WN arrangement, each owning TI x TJ
-// instruction tiles (32 x 32) of the output: fp32 accumulators stay in
-// registers for the whole k loop (TI*TJ*16 per lane, one wavefront per SIMD).
-// k advances 128 per stage (two instruction k-steps).  A stage's operand pages
-// and scale dwords are copied global -> LDS by direct-to-LDS loads (no
-// registers in between) into a ring of NST slots; a slot is refilled NST
-// stages ahead as soon as every wavefront has read it for the last time, so
-// HBM / L2 latency is covered by more than NST-1 stages of matrix work.
-// One barrier per stage, in the middle of it: after it every wavefront is done
-// with the current slot and every wavefront's share of the next stage has
-// landed.
+// k advances 128 per stage (two instruction k-steps).  One barrier per stage,
+// in the middle of it: after it every wavefront is done with the current W
+// slot and every wavefront's share of the next stage has landed.
 
 template <int KIND> struct Pg { static constexpr int BYTES = KIND == RFQ_MX_FP4 ? 1024 : 2048; };
 template <int KIND> struct Cbsz { static constexpr int V = KIND == RFQ_MX_FP4 ? 4 : 0; };
@@ -286,34 +278,52 @@ __device__ __forceinline__ void barrier_no_drain()
     asm volatile("" ::: "memory");
 }
 
-template <int AK, int BK_, int WM, int WN, int TI, int TJ> struct GemmCfg {
-    static constexpr int RTA = WM * TI, RTB = WN * TJ;          // row tiles per workgroup
-    static constexpr int BM = RTA * 32, BN = RTB * 32;
-    static constexpr int PA = Pg<AK>::BYTES, PB = Pg<BK_>::BYTES;
-    static constexpr int A_STAGE = RTA * 2 * PA, B_STAGE = RTB * 2 * PB;
-    static constexpr int SA_RT = (RTA + 3) / 4 * 4, SB_RT = (RTB + 3) / 4 * 4;
-    static constexpr int S_STAGE = (SA_RT + SB_RT) * 256;
-    static constexpr int STAGE = A_STAGE + B_STAGE + S_STAGE;
-    static constexpr int A_WL = A_STAGE / 1024, B_WL = B_STAGE / 1024, S_WL = S_STAGE / 1024;
-    static constexpr int WL = A_WL + B_WL + S_WL;               // 1 KiB wave-loads per stage
-    static constexpr int WL_MIN = WL / 4, WL_MAX = (WL + 3) / 4; // per wavefront
-    static constexpr int LDS_MAX = 160 * 1024;
-    static constexpr int NST = LDS_MAX / STAGE >= 4 ? 4 : LDS_MAX / STAGE; // ring slots
-    static_assert(NST >= 2, "a stage must fit LDS twice");
-    static_assert((NST - 1) * WL_MIN < 64, "prefetch depth exceeds the load counter");
+// Workgroup = 4 wavefronts stacked along M, one per SIMD.  Wavefront w owns
+// rows [64w, 64w+64) of the 256-row tile and ALL its TJ*32 columns: TI = 2 by TJ
+// instruction tiles, 32*TJ fp32 accumulators per lane for the whole k loop.
+//   W pages (shared by the four wavefronts) travel global -> LDS by direct
+//     copies into a ring of RING stage slots, refilled RING stages ahead;
+//   A pages (private to a wavefront) travel global -> registers, RING-1 stages
+//     ahead, and never touch LDS.
+// Splitting the operands this way matters: with both in LDS the LDS port
+// (128 B/clk) saturates before the matrix cores do.
+template <int BK_, int TJ, int RING_> struct GemmCfg {
+    static constexpr int TI = 2, WM = 4, RING = RING_;
+    static constexpr int BM = WM * TI * 32, BN = TJ * 32;
+    static constexpr int PB = Pg<BK_>::BYTES;
+    static constexpr int B_STAGE = TJ * 2 * PB;
+    static constexpr int SB_RT = (TJ + 3) / 4 * 4;
+    static constexpr int S_STAGE = SB_RT * 256;
+    static constexpr int STAGE = B_STAGE + S_STAGE;
+    static constexpr int WL = STAGE / 1024;                       // 1 KiB wave-copies per stage
+    static constexpr int ND = (WL + 3) / 4;                       // per wavefront (padded with repeats)
 };
 
-template <int AK, int BK_, bool OUT_BF16, int WM, int WN, int TI, int TJ>
+template <int N> struct IC { static constexpr int value = N; };
+
+template <int AK, int BK_, bool OUT_BF16, int TJ, int RING>
 __global__ void __launch_bounds__(256)
 gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, void *__restrict__ outp, int M, int N,
                MxLayout LA, MxLayout LB)
 {
-    using C = GemmCfg<AK, BK_, WM, WN, TI, TJ>;
+    RFQ_MX_STAMP(0);
+    using C = GemmCfg<BK_, TJ, RING>;
+    constexpr int TI = C::TI, PA = Pg<AK>::BYTES;
+    constexpr int NMMA = TI * TJ;
+    constexpr int A_PER_FRAG = AK == RFQ_MX_FP4 ? 1 : 2;
+    constexpr int NA_OPS = TI * 2 * A_PER_FRAG + TI;          // vector loads per stage for A and its scales
+    constexpr int A_PPS = (NA_OPS + NMMA - 3) / (NMMA - 2);   // A loads per slot: all issued before the hand-over at slot NMMA-2
+    constexpr int D_PPS = (C::ND + NMMA - 1) / NMMA;          // W copies per slot
+    // Vector-memory operations a wavefront issues after the last one of stage
+    // s+1 and before the hand-over of stage s (see the schedule below).
+    constexpr int HANDOVER_VMCNT = (RING - 2) * (NA_OPS + C::ND);
+    constexpr int PROLOGUE_VMCNT = (RING - 1) * C::ND + (RING - 2) * NA_OPS;
+    static_assert(HANDOVER_VMCNT < 64 && PROLOGUE_VMCNT < 64, "prefetch depth exceeds the 6-bit load counter");
+    static_assert(TJ + 1 <= NMMA, "not enough matrix instructions to hide the fragment reads");
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6); // uniform, and the compiler may know it
-    const int wm = wave % WM, wn = wave / WM;
     // XCD-aware tile order: consecutive workgroup ids land on different XCDs
     // (round robin over 8).  Each XCD gets a contiguous run of tiles that walks
     // the M tiles of one N tile first, so a W tile is fetched into one L2 only.
@@ -328,59 +338,90 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
         bid = t;
     }
     const int tn = bid / tiles_m, tmi = bid % tiles_m;
-    const int rtA0 = tmi * C::RTA, rtB0 = tn * C::RTB;
-    const uint8_t *a_scale = ap + LA.data_bytes, *b_scale = bp + LB.data_bytes;
+    const int rtB0 = tn * TJ;
+    const uint8_t *b_scale = bp + LB.data_bytes;
+    const int nstages = LA.ks / 2;
+    const int last = nstages - 1;
 
-    // Per-lane global source of each of this wavefront's wave-loads at stage 0;
-    // a stage advances data pages by 2 pages and scales by 128 bytes... every
-    // second stage (a scale dword covers 4 k-steps = 2 stages).
-    const uint8_t *src[C::WL_MAX];
-    int kind_of[C::WL_MAX]; // 0 = A data, 1 = B data, 2 = scales
+    // ---- A: this lane's page pointers (k-step 0) and scale pointers --------
+    const uint8_t *a_ptr[TI], *as_ptr[TI];
 #pragma unroll
-    for (int i = 0; i < C::WL_MAX; i++) {
+    for (int i = 0; i < TI; i++) {
+        int rt = tmi * (C::WM * TI) + wave * TI + i;
+        if (rt >= LA.rt) rt = LA.rt - 1;
+        a_ptr[i] = ap + (size_t)rt * LA.ks * PA + lane * 16;
+        as_ptr[i] = ap + LA.data_bytes + (size_t)rt * LA.ks4 * 256 + lane * 4;
+    }
+    v8i areg[RING][TI][2];   // 8-bit A fragments
+    v4i areg4[RING][TI][2];  // 4-bit A fragments
+    int ascl[RING][TI];
+
+    // ---- W: per-lane global source of each of this wavefront's wave-copies ---
+    const uint8_t *src[C::ND];
+    bool is_scale[C::ND];
+    int dst_off[C::ND];
+#pragma unroll
+    for (int i = 0; i < C::ND; i++) {
         int j = wave + 4 * i;
-        src[i] = ap;
-        kind_of[i] = 3;
-        if (j < C::A_WL) {
-            int off = j * 1024, rtl = off / (2 * C::PA), within = off % (2 * C::PA);
-            int rt = rtA0 + rtl;
-            if (rt >= LA.rt) rt = LA.rt - 1;
-            src[i] = ap + (size_t)rt * LA.ks * C::PA + within + lane * 16;
-            kind_of[i] = 0;
-        } else if (j < C::A_WL + C::B_WL) {
-            int off = (j - C::A_WL) * 1024, rtl = off / (2 * C::PB), within = off % (2 * C::PB);
+        if (j >= C::WL) j = C::WL - 1;               // pad: repeat the last copy (same bytes, same place)
+        dst_off[i] = j * 1024;
+        if (j * 1024 < C::B_STAGE) {
+            int off = j * 1024, rtl = off / (2 * C::PB), within = off % (2 * C::PB);
             int rt = rtB0 + rtl;
             if (rt >= LB.rt) rt = LB.rt - 1;
             src[i] = bp + (size_t)rt * LB.ks * C::PB + within + lane * 16;
-            kind_of[i] = 1;
-        } else if (j < C::WL) {
-            int q = j - C::A_WL - C::B_WL;           // 1 KiB = 4 row tiles x 256 bytes
-            int rtl = q * 4 + (lane >> 4);
-            bool isb = rtl >= C::SA_RT;
-            int r = isb ? rtl - C::SA_RT : rtl;
-            int rt = (isb ? rtB0 : rtA0) + r;
-            int rtmax = isb ? LB.rt : LA.rt;
-            if (rt >= rtmax) rt = rtmax - 1;
-            src[i] = (isb ? b_scale : a_scale) + (size_t)rt * (isb ? LB.ks4 : LA.ks4) * 256 + (lane & 15) * 16;
-            kind_of[i] = 2;
+            is_scale[i] = false;
+        } else {
+            int q = j - C::B_STAGE / 1024;           // 1 KiB = 4 row tiles x 256 bytes
+            int rt = rtB0 + q * 4 + (lane >> 4);
+            if (rt >= LB.rt) rt = LB.rt - 1;
+            src[i] = b_scale + (size_t)rt * LB.ks4 * 256 + (lane & 15) * 16;
+            is_scale[i] = true;
         }
     }
+    // Prefetches past the last stage re-fetch the last stage (into slots and
+    // registers nobody reads again): every stage then issues the same number
+    // of operations and the wait counts below are constants.
+    auto clamp_stage = [&](int st) { return st < last ? st : last; };
     // i-th copy of stage `st` by this wavefront into the ring slot at LDS address `slot`
-    auto issue_piece = [&](int st, uint32_t slot, int i) {
-        int j = wave + 4 * i;
-        if (j < C::WL) {
-            size_t adv = kind_of[i] == 0 ? (size_t)st * 2 * C::PA
-                       : kind_of[i] == 1 ? (size_t)st * 2 * C::PB
-                                         : (size_t)(st >> 1) * 256;
-            lds_dma16(src[i] + adv, __builtin_amdgcn_readfirstlane(slot + j * 1024));
+    auto dma_piece = [&](int st, uint32_t slot, int i) {
+        size_t adv = is_scale[i] ? (size_t)(st >> 1) * 256 : (size_t)st * 2 * C::PB;
+        lds_dma16(src[i] + adv, __builtin_amdgcn_readfirstlane(slot + dst_off[i]));
+    };
+    auto slot_addr = [&](int ring_slot) {
+        return (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uintptr_t)(lds + ring_slot * C::STAGE));
+    };
+    // One vector load of A's stage `st` into ring set SET: pieces 0..NA_OPS-1.
+    // 4-bit A: the loads are written as assembly, like the W copies, so that
+    // the compiler keeps no count of them either -- its own count would ignore
+    // the W copies queued in between and drain them early.  Their results are
+    // first read after the hand-over wait of the previous stage, and every
+    // destination register stays live until then.  8-bit A (two loads per
+    // fragment) stays with compiler-tracked loads.
+    auto a_piece = [&](auto setc, int st, int piece) {
+        constexpr int SET = decltype(setc)::value;
+        if (piece < TI * 2 * A_PER_FRAG) {
+            int f = piece / A_PER_FRAG, half = piece % A_PER_FRAG, i = f >> 1, ksl = f & 1;
+            const uint8_t *pg = a_ptr[i] + (size_t)(st * 2 + ksl) * PA + half * 1024;
+            if (AK == RFQ_MX_FP4) {
+                asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(areg4[SET][i][ksl]) : "v"(pg) : "memory");
+            } else {
+                uint4 v = *reinterpret_cast<const uint4 *>(pg);
+                areg[SET][i][ksl][4 * half + 0] = (int)v.x; areg[SET][i][ksl][4 * half + 1] = (int)v.y;
+                areg[SET][i][ksl][4 * half + 2] = (int)v.z; areg[SET][i][ksl][4 * half + 3] = (int)v.w;
+            }
+        } else {
+            int i = piece - TI * 2 * A_PER_FRAG;
+            const uint8_t *sp = as_ptr[i] + (size_t)(st >> 1) * 256;
+            if (AK == RFQ_MX_FP4) asm volatile("global_load_dword %0, %1, off" : "=v"(ascl[SET][i]) : "v"(sp) : "memory");
+            else ascl[SET][i] = *reinterpret_cast<const int *>(sp);
         }
     };
-    auto issue = [&](int st) {
-        // LDS byte address of the ring slot (the low 32 bits of a __shared__ pointer)
-        uint32_t slot = (uint32_t)(uintptr_t)(lds + (st % C::NST) * C::STAGE);
-        slot = __builtin_amdgcn_readfirstlane(slot);
-#pragma unroll
-        for (int i = 0; i < C::WL_MAX; i++) issue_piece(st, slot, i);
+    auto a_frag = [&](auto setc, int i, int ksl) -> v8i {
+        constexpr int SET = decltype(setc)::value;
+        if (AK == RFQ_MX_FP4)
+            return __builtin_shufflevector(areg4[SET][i][ksl], areg4[SET][i][ksl], 0, 1, 2, 3, -1, -1, -1, -1);
+        return areg[SET][i][ksl];
     };
 
     v16f acc[TI][TJ];
@@ -390,131 +431,138 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
         for (int j = 0; j < TJ; j++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
-
-    const int nstages = LA.ks / 2;
-    // Ring prologue: NST stages requested, stage 0 awaited.
 #pragma unroll
-    for (int d = 0; d < C::NST; d++)
-        if (d < nstages) issue(d);
-    if (C::NST - 1 < nstages) wait_vmcnt<(C::NST - 1) * C::WL_MIN>();
-    else wait_vmcnt<0>();
+    for (int set = 0; set < RING; set++)
+#pragma unroll
+        for (int i = 0; i < TI; i++) {
+            ascl[set][i] = 0;
+#pragma unroll
+            for (int k2 = 0; k2 < 2; k2++) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) areg[set][i][k2][e] = 0;
+#pragma unroll
+                for (int e = 0; e < 4; e++) areg4[set][i][k2][e] = 0;
+            }
+        }
+
+    // ---- prologue: W(0), A(0), W(1), A(1), ..., A(RING-2), W(RING-1); then stage 0 awaited
+    auto prologue_stage = [&](auto setc) {
+        constexpr int SET = decltype(setc)::value;
+        const int st = clamp_stage(SET);
+        const uint32_t slot = slot_addr(SET);
+#pragma unroll
+        for (int i = 0; i < C::ND; i++) dma_piece(st, slot, i);
+        if (SET < RING - 1) {
+#pragma unroll
+            for (int pc = 0; pc < NA_OPS; pc++) a_piece(setc, st, pc);
+        }
+        asm volatile("" ::: "memory");
+    };
+    prologue_stage(IC<0>{});
+    prologue_stage(IC<1>{});
+    if (RING > 2) prologue_stage(IC<2 % RING>{});
+    if (RING > 3) prologue_stage(IC<3 % RING>{});
+    if (RING > 4) prologue_stage(IC<4 % RING>{});
+    if (RING > 5) prologue_stage(IC<5 % RING>{});
+    if (RING > 6) prologue_stage(IC<6 % RING>{});
+    if (RING > 7) prologue_stage(IC<7 % RING>{});
+    static_assert(RING >= 3 && RING <= 8, "ring depth");
+    wait_vmcnt<PROLOGUE_VMCNT>();
     barrier_no_drain();
 
-    // One wavefront per SIMD owns the matrix core, so nothing but this
-    // instruction stream can hide latency: fragment registers are
-    // double-buffered by hand and every other piece of work of a stage (LDS
-    // reads of the next k-step, the refill copies, the barrier) is slotted
-    // between two matrix instructions (32 cycles each).  sched_barrier pins
-    // that order against the compiler's instruction scheduler.
-    constexpr int NMMA = TI * TJ, NFRAG = TI + TJ;
-    constexpr int PPS = (C::WL_MAX + NMMA - 1) / NMMA;      // refill copies per matrix-instruction slot
-    static_assert(NFRAG + 1 <= NMMA, "not enough matrix instructions to hide the fragment reads");
-    v8i fa0[TI], fb0[TJ], fa1[TI], fb1[TJ];
-    int sa[TI], sb[TJ], sa_n[TI], sb_n[TJ];
-    auto read_piece = [&](const uint8_t *base, int ksl, int q, v8i (&fa)[TI], v8i (&fb)[TJ]) {
-        if (q < TI) fa[q] = read_frag<AK>(base + ((wm * TI + q) * 2 + ksl) * C::PA, lane);
-        else fb[q - TI] = read_frag<BK_>(base + C::A_STAGE + ((wn * TJ + (q - TI)) * 2 + ksl) * C::PB, lane);
+    // W fragments are double-buffered by hand (k-step 0 / k-step 1), W scales
+    // by stage parity.
+    v8i fb0[TJ], fb1[TJ];
+    int sb[2][TJ];
+    auto read_b = [&](const uint8_t *base, int ksl, int j, v8i (&fb)[TJ]) {
+        fb[j] = read_frag<BK_>(base + (j * 2 + ksl) * C::PB, lane);
     };
-    // The stage uses scale bytes 2*(st&1) and 2*(st&1)+1 of its dwords: shift
+    // A stage uses scale bytes 2*(st&1) and 2*(st&1)+1 of its dwords: shift
     // them down so the instruction's byte selectors are constants.
-    auto scale_piece = [&](const uint8_t *base, int st, int q, int (&xa)[TI], int (&xb)[TJ]) {
-        const uint8_t *sA = base + C::A_STAGE + C::B_STAGE, *sB = sA + C::SA_RT * 256;
-        const int sh = 16 * (st & 1);
-        if (q < TI) xa[q] = (int)(*reinterpret_cast<const uint32_t *>(sA + ((wm * TI + q) * 64 + lane) * 4) >> sh);
-        else xb[q - TI] = (int)(*reinterpret_cast<const uint32_t *>(sB + ((wn * TJ + (q - TI)) * 64 + lane) * 4) >> sh);
+    auto read_bscale = [&](const uint8_t *base, int st, int j, int (&xb)[TJ]) {
+        xb[j] = (int)(*reinterpret_cast<const uint32_t *>(base + C::B_STAGE + (j * 64 + lane) * 4) >> (16 * (st & 1)));
     };
 #pragma unroll
-    for (int q = 0; q < NFRAG; q++) {
-        read_piece(lds, 0, q, fa0, fb0);
-        scale_piece(lds, 0, q, sa, sb);
+    for (int j = 0; j < TJ; j++) {
+        read_b(lds, 0, j, fb0);
+        read_bscale(lds, 0, j, sb[0]);
     }
 
-#ifdef RFQ_MX_TRACE
-    unsigned long long tacc[6] = {0, 0, 0, 0, 0, 0};
-    unsigned long long t_begin = __builtin_readcyclecounter();
-#endif
-    for (int st = 0; st < nstages; st++) {
-        RFQ_MX_T(0);
-        const uint8_t *base = lds + (st % C::NST) * C::STAGE;
-        const uint8_t *nbase = lds + ((st + 1) % C::NST) * C::STAGE;
-        const bool more = st + 1 < nstages;
-        const bool refill = st + C::NST < nstages;
-        uint32_t slot = (uint32_t)(uintptr_t)(lds + (st % C::NST) * C::STAGE);
-        slot = __builtin_amdgcn_readfirstlane(slot);
+    // One stage with ring set SET = st % RING, PAR = st % 2.  It contains no
+    // branch; everything that is not a matrix instruction is slotted between
+    // two of them and sched_barrier pins that order.
+    auto stage = [&](auto setc, auto parc, int st) {
+        constexpr int SET = decltype(setc)::value, PAR = decltype(parc)::value;
+        using AHEAD = IC<(SET + RING - 1) % RING>;
+        const uint8_t *base = lds + SET * C::STAGE;
+        const uint8_t *nbase = lds + ((SET + 1) % RING) * C::STAGE;
+        const int st_a = clamp_stage(st + RING - 1), st_w = clamp_stage(st + RING);
+        int sa[TI];
+#pragma unroll
+        for (int i = 0; i < TI; i++) sa[i] = (int)((uint32_t)ascl[SET][i] >> (16 * (st & 1)));
 
-        // k-step 0 of the stage; its shadow: reads of k-step 1, then the hand-over.
+        // k-step 0; its shadow: W fragments of k-step 1, A loads RING-1 stages ahead, then the hand-over.
 #pragma unroll
         for (int q = 0; q < NMMA; q++) {
-            if (!(RFQ_MX_ABLATE & 1))
-                acc[q / TJ][q % TJ] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                    fa0[q / TJ], fb0[q % TJ], acc[q / TJ][q % TJ], Cbsz<AK>::V, Cbsz<BK_>::V, 0, sa[q / TJ], 0,
-                    sb[q % TJ]);
+            acc[q / TJ][q % TJ] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                a_frag(setc, q / TJ, 0), fb0[q % TJ], acc[q / TJ][q % TJ], Cbsz<AK>::V, Cbsz<BK_>::V, 0, sa[q / TJ], 0,
+                sb[PAR][q % TJ]);
             __builtin_amdgcn_sched_barrier(0);
-            if (q < NFRAG && !(RFQ_MX_ABLATE & 4)) read_piece(base, 1, q, fa1, fb1);
+            if (q < TJ) read_b(base, 1, q, fb1);
+#pragma unroll
+            for (int pp = 0; pp < A_PPS; pp++)
+                if (q * A_PPS + pp < NA_OPS) a_piece(AHEAD{}, st_a, q * A_PPS + pp);
             if (q == NMMA - 2) {
-                RFQ_MX_T(1);
-                RFQ_MX_ACC(0, t0, t1);
-                // Hand-over: this wavefront's last reads of the slot are
-                // complete (lgkmcnt), the next stage has landed (vmcnt),
-                // everyone agrees (barrier).  Afterwards the slot may be
-                // refilled NST stages ahead.
+                // Hand-over: this wavefront's last reads of the slot are complete
+                // (lgkmcnt), stage st+1 has landed in LDS and in registers
+                // (vmcnt: only what was issued after it may still be in
+                // flight), everyone agrees (barrier).
                 __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0) only
-                RFQ_MX_T(2);
-                RFQ_MX_ACC(1, t1, t2);
-                if (more) {
-                    if (st + C::NST - 1 < nstages) wait_vmcnt<(C::NST - 2) * C::WL_MIN>();
-                    else wait_vmcnt<0>();
-                }
-                RFQ_MX_T(3);
-                RFQ_MX_ACC(2, t2, t3);
+                wait_vmcnt<HANDOVER_VMCNT>();
                 barrier_no_drain();
-                RFQ_MX_T(4);
-                RFQ_MX_ACC(3, t3, t4);
-#ifdef RFQ_MX_TRACE
-                tacc[5] = t4; // start of the second half
-#endif
             }
             __builtin_amdgcn_sched_barrier(0);
         }
-        // k-step 1; its shadow: refill copies, reads of the next stage's k-step 0 and scales.
+        // k-step 1; its shadow: the slot's refill, W fragments and scales of the next stage.
+        const uint32_t slot = slot_addr(SET);
 #pragma unroll
         for (int q = 0; q < NMMA; q++) {
-            if (!(RFQ_MX_ABLATE & 1))
-                acc[q / TJ][q % TJ] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                    fa1[q / TJ], fb1[q % TJ], acc[q / TJ][q % TJ], Cbsz<AK>::V, Cbsz<BK_>::V, 1, sa[q / TJ], 1,
-                    sb[q % TJ]);
+            acc[q / TJ][q % TJ] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                a_frag(setc, q / TJ, 1), fb1[q % TJ], acc[q / TJ][q % TJ], Cbsz<AK>::V, Cbsz<BK_>::V, 1, sa[q / TJ], 1,
+                sb[PAR][q % TJ]);
             __builtin_amdgcn_sched_barrier(0);
-            if (refill && !(RFQ_MX_ABLATE & 2)) {
 #pragma unroll
-                for (int pp = 0; pp < PPS; pp++)
-                    if (q * PPS + pp < C::WL_MAX) issue_piece(st + C::NST, slot, q * PPS + pp);
-            }
-            if (q < NFRAG && more) {
-                if (!(RFQ_MX_ABLATE & 4)) read_piece(nbase, 0, q, fa0, fb0);
-                scale_piece(nbase, st + 1, q, sa_n, sb_n);
+            for (int pp = 0; pp < D_PPS; pp++)
+                if (q * D_PPS + pp < C::ND) dma_piece(st_w, slot, q * D_PPS + pp);
+            if (q < TJ) {
+                read_b(nbase, 0, q, fb0);
+                read_bscale(nbase, st + 1, q, sb[PAR ^ 1]);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
-        if (RFQ_MX_ABLATE & 1) {
-#pragma unroll
-            for (int i = 0; i < TI; i++) acc[i][0][0] += (float)(fa0[i][0] ^ fa1[i][1]);
-#pragma unroll
-            for (int j = 0; j < TJ; j++) acc[0][j][1] += (float)(fb0[j][0] ^ fb1[j][1]);
-        }
-#pragma unroll
-        for (int i = 0; i < TI; i++) sa[i] = sa_n[i];
-#pragma unroll
-        for (int j = 0; j < TJ; j++) sb[j] = sb_n[j];
-#ifdef RFQ_MX_TRACE
-        {
-            unsigned long long t9 = __builtin_readcyclecounter();
-            tacc[4] += t9 - tacc[5];
-        }
-#endif
+    };
+
+    RFQ_MX_STAMP(1);
+    // RING is even here or the parity is carried by a second copy of the body:
+    // unroll by lcm(RING, 2) so that ring set and stage parity are constants.
+    constexpr int UNROLL = (RING % 2 == 0) ? RING : 2 * RING;
+    for (int st = 0; st < nstages; st += UNROLL) {
+        stage(IC<0 % RING>{}, IC<0>{}, st);
+        if (st + 1 < nstages) stage(IC<1 % RING>{}, IC<1>{}, st + 1);
+        if (st + 2 < nstages) stage(IC<2 % RING>{}, IC<0>{}, st + 2);
+        if (UNROLL > 3 && st + 3 < nstages) stage(IC<3 % RING>{}, IC<1>{}, st + 3);
+        if (UNROLL > 4 && st + 4 < nstages) stage(IC<4 % RING>{}, IC<0>{}, st + 4);
+        if (UNROLL > 5 && st + 5 < nstages) stage(IC<5 % RING>{}, IC<1>{}, st + 5);
+        if (UNROLL > 6 && st + 6 < nstages) stage(IC<6 % RING>{}, IC<0>{}, st + 6);
+        if (UNROLL > 7 && st + 7 < nstages) stage(IC<7 % RING>{}, IC<1>{}, st + 7);
+        if (UNROLL > 8 && st + 8 < nstages) stage(IC<8 % RING>{}, IC<0>{}, st + 8);
+        if (UNROLL > 9 && st + 9 < nstages) stage(IC<9 % RING>{}, IC<1>{}, st + 9);
     }
-#ifdef RFQ_MX_TRACE
-    unsigned long long t_loop_end = __builtin_readcyclecounter();
-#endif
+    static_assert(UNROLL <= 10, "unroll");
+    // The trailing prefetches still write LDS slots and registers: drain them
+    // before either is reused.
+    wait_vmcnt<0>();
+    RFQ_MX_STAMP(2);
 
     // Epilogue.  Accumulator register r of tile (i, j) is row
     // 8*(r/4) + 4*(lane/32) + r%4, column lane%32 of the tile: a lane owns
@@ -525,12 +573,11 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
     constexpr int ROW_BYTES = TJ * 32 * ES;                 // one band row of this wavefront
     constexpr int ROW_STRIDE = ROW_BYTES + 16;              // +4 dwords: the two half-waves (rows R, R+4) miss each other's banks
     constexpr int CPR = ROW_BYTES / 16;                     // 16-byte chunks per row
-    static_assert(4 * 32 * ROW_STRIDE <= C::NST * C::STAGE, "epilogue staging exceeds the ring");
-    const int m_base = tmi * C::BM + wm * TI * 32, n_base = tn * C::BN + wn * TJ * 32;
+    const int m_base = tmi * C::BM + wave * TI * 32, n_base = tn * C::BN;
     const bool interior = m_base + TI * 32 <= M && n_base + TJ * 32 <= N && ((size_t)N * ES) % 16 == 0 &&
-                          (reinterpret_cast<uintptr_t>(outp) & 15u) == 0 && !(RFQ_MX_ABLATE & 8);
-    barrier_no_drain(); // every wavefront is past its last fragment read
-    uint8_t *stage = lds + (size_t)wave * 32 * ROW_STRIDE;
+                          (reinterpret_cast<uintptr_t>(outp) & 15u) == 0;
+    barrier_no_drain(); // every wavefront is past its last fragment read and its last copy
+    uint8_t *stagebuf = lds + (size_t)wave * 32 * ROW_STRIDE;
     if (interior) {
 #pragma unroll
         for (int i = 0; i < TI; i++) {
@@ -539,7 +586,7 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                     int row = 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                    uint8_t *dst = stage + row * ROW_STRIDE + (32 * j + (lane & 31)) * ES;
+                    uint8_t *dst = stagebuf + row * ROW_STRIDE + (32 * j + (lane & 31)) * ES;
                     if (OUT_BF16) *reinterpret_cast<uint16_t *>(dst) = f32_to_bf16(acc[i][j][r]);
                     else *reinterpret_cast<float *>(dst) = acc[i][j][r];
                 }
@@ -550,7 +597,7 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
                 int c = c0 + lane;
                 if (c < 32 * CPR) {
                     int row = c / CPR, col16 = c % CPR;
-                    uint4 v = *reinterpret_cast<const uint4 *>(stage + row * ROW_STRIDE + col16 * 16);
+                    uint4 v = *reinterpret_cast<const uint4 *>(stagebuf + row * ROW_STRIDE + col16 * 16);
                     uint8_t *o = reinterpret_cast<uint8_t *>(outp) +
                                  ((size_t)(m_base + 32 * i + row) * N + n_base) * ES + col16 * 16;
                     *reinterpret_cast<uint4 *>(o) = v;
@@ -566,7 +613,6 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                     int m = m_base + 32 * i + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                    if ((RFQ_MX_ABLATE & 8) && (i | j | r)) continue;
                     if (m < M && n < N) {
                         if (OUT_BF16)
                             reinterpret_cast<uint16_t *>(outp)[(size_t)m * N + n] = f32_to_bf16(acc[i][j][r]);
@@ -576,54 +622,44 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
                 }
             }
     }
-#ifdef RFQ_MX_TRACE
-    if (tid == 0 && rfq_mx_trace) {
-        unsigned long long t_end = __builtin_readcyclecounter();
-        unsigned long long *o = rfq_mx_trace + (size_t)blockIdx.x * 8;
-        o[0] = tacc[0]; o[1] = tacc[1]; o[2] = tacc[2]; o[3] = tacc[3]; o[4] = tacc[4];
-        o[5] = t_loop_end - t_begin; o[6] = t_end - t_loop_end; o[7] = t_begin;
-    }
-#endif
+    RFQ_MX_STAMP(3);
 }
 
-template <int AK, int BK_, bool OUT_BF16, int WM, int WN, int TI, int TJ>
+template <int AK, int BK_, bool OUT_BF16, int TJ, int RING>
 int launch_gemm_cfg(const uint8_t *a, const uint8_t *b, void *out, int m, int n, int k, hipStream_t s)
 {
-    using C = GemmCfg<AK, BK_, WM, WN, TI, TJ>;
+    using C = GemmCfg<BK_, TJ, RING>;
     MxLayout LA = mx_layout(AK, m, k), LB = mx_layout(BK_, n, k);
-    constexpr size_t LDS = (size_t)C::NST * C::STAGE;
+    constexpr size_t RINGB = (size_t)RING * C::STAGE;
+    constexpr size_t STAGING = (size_t)4 * 32 * (TJ * 32 * (OUT_BF16 ? 2 : 4) + 16);
+    constexpr size_t LDS = RINGB > STAGING ? RINGB : STAGING;
+    static_assert(LDS <= 160 * 1024, "LDS budget");
     static std::once_flag once;
     static hipError_t attr_err = hipSuccess;
     std::call_once(once, [] {
-        attr_err = hipFuncSetAttribute(
-            reinterpret_cast<const void *>(&gemm_mx_kernel<AK, BK_, OUT_BF16, WM, WN, TI, TJ>),
-            hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS);
+        attr_err = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_mx_kernel<AK, BK_, OUT_BF16, TJ, RING>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS);
     });
     if (attr_err != hipSuccess) return hip_fail(attr_err, "hipFuncSetAttribute(gemm_mx_kernel)");
     int tiles = ((m + C::BM - 1) / C::BM) * ((n + C::BN - 1) / C::BN);
     int per = (tiles + 7) / 8;
-    hipLaunchKernelGGL((gemm_mx_kernel<AK, BK_, OUT_BF16, WM, WN, TI, TJ>), dim3(per * 8), dim3(256), LDS, s, a, b,
-                       out, m, n, LA, LB);
+    hipLaunchKernelGGL((gemm_mx_kernel<AK, BK_, OUT_BF16, TJ, RING>), dim3(per * 8), dim3(256), LDS, s, a, b, out, m,
+                       n, LA, LB);
     RFQ_LAUNCH_CHECK("gemm_mx_kernel");
     return RFQ_OK;
 }
 
-// Two output tilings: 256 x 256 (2 x 2 wavefronts of 4 x 4 tiles) and 256 x 224
-// (4 x 1 wavefronts of 2 x 7 tiles).  The one that leaves the last round of
-// workgroups fuller wins (28672 = 128 * 224 fills 256 CUs exactly four times
-// at M = 2048; 256-wide tiles would run 3.5 rounds).
+// Output tiles are 256 rows by 224 columns for 4-bit operands (28672 = 128 * 224
+// fills 256 CUs exactly four times at M = 2048; 256-wide tiles would run 3.5
+// rounds and do not fit the register file next to the prefetch ring).
+// 8-bit operands need twice the registers per fragment: 128-column tiles.
 template <int AK, int BK_, bool OUT_BF16>
 int run_gemm(const uint8_t *a, const uint8_t *b, void *out, int m, int n, int k, hipStream_t s)
 {
-    const int cus = device_cu_count();
-    auto rounds_cost = [&](int bm, int bn) {
-        long tiles = (long)((m + bm - 1) / bm) * ((n + bn - 1) / bn);
-        long rounds = (tiles + cus - 1) / cus;
-        return (double)rounds * bm * bn; // time ~ rounds x tile area
-    };
-    if (rounds_cost(256, 224) < rounds_cost(256, 256))
-        return launch_gemm_cfg<AK, BK_, OUT_BF16, 4, 1, 2, 7>(a, b, out, m, n, k, s);
-    return launch_gemm_cfg<AK, BK_, OUT_BF16, 2, 2, 4, 4>(a, b, out, m, n, k, s);
+    if constexpr (AK == RFQ_MX_FP8 || BK_ == RFQ_MX_FP8)
+        return launch_gemm_cfg<AK, BK_, OUT_BF16, 4, 4>(a, b, out, m, n, k, s);
+    else
+        return launch_gemm_cfg<AK, BK_, OUT_BF16, 7, RFQ_MX_RING>(a, b, out, m, n, k, s);
 }
 
 template <int FMT, int KIND>
