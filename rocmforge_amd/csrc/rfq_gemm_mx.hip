@@ -40,6 +40,13 @@ __device__ unsigned long long *rfq_mx_trace;
 #else
 #define RFQ_MX_STAMP(slot) do { } while (0)
 #endif
+// -DRFQ_MX_SKIP=<mask> (tuning builds, results are wrong on purpose): leave out
+// 1 the A loads, 2 the W copies, 4 the LDS fragment reads, 8 the output stores,
+// to see what the loop time is made of.  No address depends on loaded data,
+// so the skipped parts change timing only.
+#ifndef RFQ_MX_SKIP
+#define RFQ_MX_SKIP 0
+#endif
 // Ring depth (W slots in LDS = A fragment sets in registers) of the 4-bit kernel.
 #ifndef RFQ_MX_RING
 #define RFQ_MX_RING 6
@@ -52,8 +59,13 @@ typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
+// k-steps (64 elements) of a prepared matrix are padded with zero pages to a
+// multiple of MX_KS_PAD, so that the GEMM's k loop is a whole number of trips
+// through its unrolled prefetch ring and needs no remainder code.
+constexpr int MX_KS_PAD = 12;
+
 struct MxLayout {
-    int rows, k, rt, ks, ks4;
+    int rows, k, rt, ks, ks4, ks_real; // ks: padded k-steps per row tile; ks_real: k / 64
     size_t page_bytes, data_bytes, scale_bytes;
     __host__ __device__ size_t total() const { return data_bytes + scale_bytes + 16; } // +16: status words
 };
@@ -63,8 +75,9 @@ __host__ __device__ inline MxLayout mx_layout(int kind, int rows, int k)
     MxLayout L;
     L.rows = rows; L.k = k;
     L.rt = (rows + 31) / 32;
-    L.ks = k / 64;
-    L.ks4 = (L.ks + 3) / 4;
+    L.ks_real = k / 64;
+    L.ks = (L.ks_real + MX_KS_PAD - 1) / MX_KS_PAD * MX_KS_PAD;
+    L.ks4 = L.ks / 4;
     L.page_bytes = kind == RFQ_MX_FP4 ? 1024 : 2048;
     L.data_bytes = (size_t)L.rt * L.ks * L.page_bytes;
     L.scale_bytes = (size_t)L.rt * L.ks4 * 256;
@@ -127,7 +140,7 @@ mx_prepare_kernel(const uint8_t *__restrict__ raw, uint8_t *__restrict__ prep, M
     uint32_t *status = reinterpret_cast<uint32_t *>(prep + L.data_bytes + L.scale_bytes);
 
     float v[32];
-    if (row < L.rows) {
+    if (row < L.rows && ks < L.ks_real) {
         decode_block<FMT>(raw + ((size_t)row * (L.k / 32) + kb) * BB, v);
     } else {
 #pragma unroll
@@ -202,7 +215,7 @@ mx_prepare_kernel(const uint8_t *__restrict__ raw, uint8_t *__restrict__ prep, M
     prep[L.data_bytes + ((size_t)rt * L.ks4 + (ks >> 2)) * 256 + (size_t)lane * 4 + (ks & 3)] = (uint8_t)E;
 }
 
-// Scale bytes of k-steps past the end (k not a multiple of 256) and the status words.
+// Scale bytes (before the re-encoding overwrites them) and the status words.
 __global__ void mx_init_kernel(uint8_t *prep, MxLayout L)
 {
     size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
@@ -219,19 +232,14 @@ __global__ void mx_init_kernel(uint8_t *prep, MxLayout L)
 template <int KIND> struct Pg { static constexpr int BYTES = KIND == RFQ_MX_FP4 ? 1024 : 2048; };
 template <int KIND> struct Cbsz { static constexpr int V = KIND == RFQ_MX_FP4 ? 4 : 0; };
 
-template <int KIND> __device__ __forceinline__ v8i read_frag(const uint8_t *page, int lane)
-{
-    v8i f;
-    uint4 lo = *reinterpret_cast<const uint4 *>(page + lane * 16);
-    f[0] = (int)lo.x; f[1] = (int)lo.y; f[2] = (int)lo.z; f[3] = (int)lo.w;
-    if (KIND == RFQ_MX_FP4) {
-        f[4] = 0; f[5] = 0; f[6] = 0; f[7] = 0;
-    } else {
-        uint4 hi = *reinterpret_cast<const uint4 *>(page + 1024 + lane * 16);
-        f[4] = (int)hi.x; f[5] = (int)hi.y; f[6] = (int)hi.z; f[7] = (int)hi.w;
-    }
-    return f;
-}
+// An operand fragment as it is kept in registers: a 4-bit fragment is 4
+// dwords.  The instruction names 8 registers whatever the format and ignores
+// the upper 4 for 4-bit data; widen() leaves them undefined, so they cost no
+// registers.
+template <int KIND> struct Frag { using type = v8i; };
+template <> struct Frag<RFQ_MX_FP4> { using type = v4i; };
+__device__ __forceinline__ v8i widen(v8i f) { return f; }
+__device__ __forceinline__ v8i widen(v4i f) { return __builtin_shufflevector(f, f, 0, 1, 2, 3, -1, -1, -1, -1); }
 
 __device__ __forceinline__ uint16_t f32_to_bf16(float f)
 {
@@ -248,24 +256,22 @@ template <int N> __device__ __forceinline__ void wait_vmcnt()
     __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
 }
 
-// Direct global -> LDS copy, 64 lanes x 16 bytes: lane l's 16 bytes land at
-// lds_addr + 16*l (lds_addr is wave-uniform and travels in M0).  Written as
-// assembly on purpose: the compiler then keeps no book on these copies, so it
-// does not drain them (vmcnt(0)) in front of every LDS read or barrier; the
-// kernel waits for exactly the stage it needs with wait_vmcnt.  Loads the
-// compiler cannot see only make its own waits longer, never shorter: the
-// counter retires in order.
-__device__ __forceinline__ void lds_dma16(const uint8_t *gsrc, uint32_t lds_addr)
+// The W copies are direct global -> LDS loads, 64 lanes x 16 bytes: lane l's
+// 16 bytes land at M0 + 16*l.  They (and the 4-bit A loads) are written as
+// assembly on purpose: the compiler then keeps no book on them, so it does not
+// drain them (vmcnt(0)) in front of every LDS read or barrier; the kernel
+// waits for exactly the stage it needs with wait_vmcnt.  Loads the compiler
+// cannot see only make its own waits longer, never shorter: the counter
+// retires in order.
+
+// Tells the compiler that a pointer is the same in every lane (it then lives
+// in scalar registers).
+__device__ __forceinline__ const uint8_t *uniform_ptr(const uint8_t *p)
 {
-    // M0 is read when the instruction issues; it is put back right after.
-    uint32_t saved_m0;
-    asm volatile("s_mov_b32 %0, m0\n\t"
-                 "s_mov_b32 m0, %2\n\t"
-                 "global_load_lds_dwordx4 %1, off\n\t"
-                 "s_mov_b32 m0, %0"
-                 : "=&s"(saved_m0)
-                 : "v"(gsrc), "s"(lds_addr)
-                 : "memory");
+    uint64_t v = reinterpret_cast<uint64_t>(p);
+    uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+    uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
+    return reinterpret_cast<const uint8_t *>(((uint64_t)hi << 32) | lo);
 }
 
 // Workgroup barrier without the memory-model fence of __syncthreads (which
@@ -287,6 +293,12 @@ __device__ __forceinline__ void barrier_no_drain()
 //     ahead, and never touch LDS.
 // Splitting the operands this way matters: with both in LDS the LDS port
 // (128 B/clk) saturates before the matrix cores do.
+//
+// Workgroups are persistent: one per CU, each walking its list of output
+// tiles.  The operand stream does not stop at a tile boundary -- while a
+// wavefront converts and stores the finished tile, the first RING stages of
+// its next tile are already in flight or landed, and the stores drain behind
+// the next tile's matrix work.
 template <int BK_, int TJ, int RING_> struct GemmCfg {
     static constexpr int TI = 2, WM = 4, RING = RING_;
     static constexpr int BM = WM * TI * 32, BN = TJ * 32;
@@ -297,6 +309,14 @@ template <int BK_, int TJ, int RING_> struct GemmCfg {
     static constexpr int STAGE = B_STAGE + S_STAGE;
     static constexpr int WL = STAGE / 1024;                       // 1 KiB wave-copies per stage
     static constexpr int ND = (WL + 3) / 4;                       // per wavefront (padded with repeats)
+    static constexpr int RING_BYTES = RING * STAGE;
+    // the epilogue stages a 32-row band JG instruction tiles (32 columns each) at a time
+    template <bool OUT_BF16> static constexpr int staging_tiles() { return OUT_BF16 ? TJ : (TJ > 1 ? TJ / 2 : 1); }
+    template <bool OUT_BF16> static constexpr int staging_row_stride()
+    {
+        return staging_tiles<OUT_BF16>() * 32 * (OUT_BF16 ? 2 : 4) + 16;
+    }
+    template <bool OUT_BF16> static constexpr int lds_bytes() { return RING_BYTES + 4 * 32 * staging_row_stride<OUT_BF16>(); }
 };
 
 template <int N> struct IC { static constexpr int value = N; };
@@ -314,107 +334,155 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
     constexpr int NA_OPS = TI * 2 * A_PER_FRAG + TI;          // vector loads per stage for A and its scales
     constexpr int A_PPS = (NA_OPS + NMMA - 3) / (NMMA - 2);   // A loads per slot: all issued before the hand-over at slot NMMA-2
     constexpr int D_PPS = (C::ND + NMMA - 1) / NMMA;          // W copies per slot
-    // Vector-memory operations a wavefront issues after the last one of stage
-    // s+1 and before the hand-over of stage s (see the schedule below).
-    constexpr int HANDOVER_VMCNT = (RING - 2) * (NA_OPS + C::ND);
-    constexpr int PROLOGUE_VMCNT = (RING - 1) * C::ND + (RING - 2) * NA_OPS;
-    static_assert(HANDOVER_VMCNT < 64 && PROLOGUE_VMCNT < 64, "prefetch depth exceeds the 6-bit load counter");
+    // Loads a wavefront issues after the last one of stage s+1 and before the
+    // hand-over of stage s (see the schedule below).  Loads complete in order
+    // among themselves, so "at most this many operations outstanding" proves
+    // that stage s+1 has arrived; stores in flight (from a tile's epilogue)
+    // can only make the wait longer, never too short.
+    constexpr int NA_CNT = (RFQ_MX_SKIP & 1) ? 0 : NA_OPS, ND_CNT = (RFQ_MX_SKIP & 2) ? 0 : C::ND;
+    // (the counter has 6 bits; a smaller number only waits for more than necessary)
+    constexpr int HANDOVER_EXACT = (RING - 2) * (NA_CNT + ND_CNT);
+    constexpr int PROLOGUE_EXACT = (RING - 1) * ND_CNT + (RING - 2) * NA_CNT;
+    constexpr int HANDOVER_VMCNT = HANDOVER_EXACT < 63 ? HANDOVER_EXACT : 63;
+    constexpr int PROLOGUE_VMCNT = PROLOGUE_EXACT < 63 ? PROLOGUE_EXACT : 63;
     static_assert(TJ + 1 <= NMMA, "not enough matrix instructions to hide the fragment reads");
+    static_assert(RING >= 4 && RING <= 8 && RING % 2 == 0, "ring depth: even, so that stage parity is a constant");
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
-    const int tid = threadIdx.x, lane = tid & 63;
+    const int tid = threadIdx.x, lane = tid & 63, lane_id = lane;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6); // uniform, and the compiler may know it
-    // XCD-aware tile order: consecutive workgroup ids land on different XCDs
-    // (round robin over 8).  Each XCD gets a contiguous run of tiles that walks
-    // the M tiles of one N tile first, so a W tile is fetched into one L2 only.
+    // XCD-aware tile lists: consecutive workgroup ids land on different XCDs
+    // (round robin over 8).  XCD x owns the contiguous run of tiles
+    // [x*per, (x+1)*per), ordered M-tile fastest, and its workgroups take them
+    // G8 apart: at any time an XCD works on a few W tiles times all M tiles, so
+    // each W tile is fetched into one L2 only and A is shared by neighbours.
     const int tiles_m = (M + C::BM - 1) / C::BM, tiles_n = (N + C::BN - 1) / C::BN;
     const int total = tiles_m * tiles_n;
-    int bid = blockIdx.x;
-    {
-        int xcd = bid & 7, slot = bid >> 3;
-        int per = (total + 7) / 8;
-        int t = xcd * per + slot;
-        if (slot >= per || t >= total) return; // uniform over the workgroup
-        bid = t;
-    }
-    const int tn = bid / tiles_m, tmi = bid % tiles_m;
-    const int rtB0 = tn * TJ;
+    const int per = (total + 7) / 8;
+    const int xcd = blockIdx.x & 7, G8 = gridDim.x >> 3;
+    auto tile_valid = [&](int idx) { return idx < per && xcd * per + idx < total; };
+    if (!tile_valid(blockIdx.x >> 3)) return; // uniform over the workgroup
     const uint8_t *b_scale = bp + LB.data_bytes;
     const int nstages = LA.ks / 2;
-    const int last = nstages - 1;
+    // (a whole number of trips through the unrolled ring: the prepared layout pads k)
 
-    // ---- A: this lane's page pointers (k-step 0) and scale pointers --------
-    const uint8_t *a_ptr[TI], *as_ptr[TI];
-#pragma unroll
-    for (int i = 0; i < TI; i++) {
-        int rt = tmi * (C::WM * TI) + wave * TI + i;
-        if (rt >= LA.rt) rt = LA.rt - 1;
-        a_ptr[i] = ap + (size_t)rt * LA.ks * PA + lane * 16;
-        as_ptr[i] = ap + LA.data_bytes + (size_t)rt * LA.ks4 * 256 + lane * 4;
-    }
+    // ---- operand addresses.  A load names a wavefront-uniform base (scalar
+    // registers, fixed for a tile), a per-lane byte offset (one register per
+    // stream, advanced by one add per stage) and an immediate.  Prefetches run
+    // ahead of the arithmetic and cross into the next tile RING stages before
+    // a tile ends, so two sets of bases exist: `pf`, in use by the prefetch
+    // streams, and `nx`, the tile after that one.  The switch happens at a fixed
+    // place of the last trip through the ring, by scalar selects: there is no
+    // branch between stages.
+    const uint32_t lane16 = lane * 16;
     v8i areg[RING][TI][2];   // 8-bit A fragments
     v4i areg4[RING][TI][2];  // 4-bit A fragments
     int ascl[RING][TI];
 
-    // ---- W: per-lane global source of each of this wavefront's wave-copies ---
-    const uint8_t *src[C::ND];
-    bool is_scale[C::ND];
+    // This wavefront's wave-copies of a W stage: copy i moves KiB j = wave + 4i
+    // of the stage image (pages first, then 256 scale bytes per row tile).
+    // Only the last copy of a wavefront can be a scale copy.
+    static_assert(C::S_STAGE <= 4096, "a wavefront may own at most one scale copy");
+    static_assert((4 * (C::ND - 2) + 3) * 1024 < C::B_STAGE, "only the last copy may hold scales");
     int dst_off[C::ND];
 #pragma unroll
     for (int i = 0; i < C::ND; i++) {
         int j = wave + 4 * i;
-        if (j >= C::WL) j = C::WL - 1;               // pad: repeat the last copy (same bytes, same place)
+        j = j < C::WL ? j : C::WL - 1;                   // pad: repeat the last copy (same bytes, same place)
         dst_off[i] = j * 1024;
-        if (j * 1024 < C::B_STAGE) {
+    }
+    const bool last_is_scale = dst_off[C::ND - 1] >= C::B_STAGE;
+    const uint32_t lds0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uintptr_t)lds); // LDS address of the ring
+    // Bases of tile `idx`; wl receives the per-lane offset of this wavefront's
+    // last W copy: lane*16 for a page copy, or the scale copy's offset (4 row
+    // tiles x 16 lanes x 16 bytes).
+    auto tile_bases = [&](int idx, const uint8_t *(&ba)[TI], const uint8_t *(&bas)[TI], const uint8_t *(&bw)[C::ND],
+                          uint32_t &wl) __attribute__((always_inline)) {
+        // (the lane number goes through an opaque statement so that nothing
+        // derived from it is hoisted out of the tile loop and kept in registers)
+        int lane = lane_id;
+        asm volatile("" : "+v"(lane));
+        const int t = xcd * per + idx, tmi = t % tiles_m, rtB0 = (t / tiles_m) * TJ;
+#pragma unroll
+        for (int i = 0; i < TI; i++) {
+            int rt = tmi * (C::WM * TI) + wave * TI + i;
+            rt = rt < LA.rt ? rt : LA.rt - 1;
+            ba[i] = uniform_ptr(ap + (size_t)rt * LA.ks * PA);
+            bas[i] = uniform_ptr(ap + LA.data_bytes + (size_t)rt * LA.ks4 * 256);
+        }
+        wl = lane * 16;
+#pragma unroll
+        for (int i = 0; i < C::ND; i++) {
+            const int j = dst_off[i] / 1024;
             int off = j * 1024, rtl = off / (2 * C::PB), within = off % (2 * C::PB);
             int rt = rtB0 + rtl;
-            if (rt >= LB.rt) rt = LB.rt - 1;
-            src[i] = bp + (size_t)rt * LB.ks * C::PB + within + lane * 16;
-            is_scale[i] = false;
-        } else {
-            int q = j - C::B_STAGE / 1024;           // 1 KiB = 4 row tiles x 256 bytes
-            int rt = rtB0 + q * 4 + (lane >> 4);
-            if (rt >= LB.rt) rt = LB.rt - 1;
-            src[i] = b_scale + (size_t)rt * LB.ks4 * 256 + (lane & 15) * 16;
-            is_scale[i] = true;
+            rt = rt < LB.rt ? rt : LB.rt - 1;
+            const uint8_t *pages = bp + (size_t)rt * LB.ks * C::PB + within;
+            if (i == C::ND - 1) {
+                int q = j - C::B_STAGE / 1024;           // 1 KiB = 4 row tiles x 256 bytes
+                int rs = rtB0 + q * 4 + (lane >> 4);
+                rs = rs < LB.rt ? rs : LB.rt - 1;        // >= rtB0: the tile exists
+                const uint32_t wsc = (uint32_t)(rs - rtB0) * (uint32_t)LB.ks4 * 256u + (lane & 15) * 16;
+                wl = last_is_scale ? wsc : wl;
+                bw[i] = uniform_ptr(last_is_scale ? b_scale + (size_t)rtB0 * LB.ks4 * 256 : pages);
+            } else {
+                bw[i] = uniform_ptr(pages);
+            }
         }
-    }
-    // Prefetches past the last stage re-fetch the last stage (into slots and
-    // registers nobody reads again): every stage then issues the same number
-    // of operations and the wait counts below are constants.
-    auto clamp_stage = [&](int st) { return st < last ? st : last; };
-    // i-th copy of stage `st` by this wavefront into the ring slot at LDS address `slot`
-    auto dma_piece = [&](int st, uint32_t slot, int i) {
-        size_t adv = is_scale[i] ? (size_t)(st >> 1) * 256 : (size_t)st * 2 * C::PB;
-        lds_dma16(src[i] + adv, __builtin_amdgcn_readfirstlane(slot + dst_off[i]));
     };
-    auto slot_addr = [&](int ring_slot) {
-        return (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uintptr_t)(lds + ring_slot * C::STAGE));
+    const uint8_t *pf_a[TI], *pf_as[TI], *pf_w[C::ND], *nx_a[TI], *nx_as[TI], *nx_w[C::ND];
+    uint32_t wl_nx = 0;
+    // per-lane offsets of the next A pages, A scales, W pages and this
+    // wavefront's last W copy to prefetch
+    uint32_t voffA, voffAS, voffW, voffWL;
+    // what a stage adds to voffWL: pages move 2 pages on, scale dwords cover two stages
+    const uint32_t incWL_even = last_is_scale ? 0u : 2u * C::PB, incWL_odd = last_is_scale ? 256u : 2u * C::PB;
+
+    // i-th copy of a W stage by this wavefront into ring slot SLOT.  The LDS
+    // address goes into M0 right before the copy (nothing else in this kernel
+    // uses M0).
+    auto dma_piece = [&](auto slotc, int i) {
+        constexpr int SLOT = decltype(slotc)::value;
+        if (RFQ_MX_SKIP & 2) return;
+        const uint32_t voff = i == C::ND - 1 ? voffWL : voffW;
+        const uint8_t *base = pf_w[i];
+        const int doff = dst_off[i] + (int)lds0;
+        asm volatile("s_add_u32 m0, %2, %3\n\t"
+                     "global_load_lds_dwordx4 %0, %1"
+                     :
+                     : "v"(voff), "s"(base), "s"(doff), "n"(SLOT * C::STAGE)
+                     : "memory", "scc");
     };
-    // One vector load of A's stage `st` into ring set SET: pieces 0..NA_OPS-1.
+    // One vector load of an A stage into ring set SET: pieces 0..NA_OPS-1.
     // 4-bit A: the loads are written as assembly, like the W copies, so that
     // the compiler keeps no count of them either -- its own count would ignore
     // the W copies queued in between and drain them early.  Their results are
     // first read after the hand-over wait of the previous stage, and every
     // destination register stays live until then.  8-bit A (two loads per
     // fragment) stays with compiler-tracked loads.
-    auto a_piece = [&](auto setc, int st, int piece) {
+    auto a_piece = [&](auto setc, int piece) {
         constexpr int SET = decltype(setc)::value;
+        if (RFQ_MX_SKIP & 1) return;
         if (piece < TI * 2 * A_PER_FRAG) {
-            int f = piece / A_PER_FRAG, half = piece % A_PER_FRAG, i = f >> 1, ksl = f & 1;
-            const uint8_t *pg = a_ptr[i] + (size_t)(st * 2 + ksl) * PA + half * 1024;
+            const int f = piece / A_PER_FRAG, half = piece % A_PER_FRAG, i = f >> 1, ksl = f & 1;
             if (AK == RFQ_MX_FP4) {
-                asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(areg4[SET][i][ksl]) : "v"(pg) : "memory");
+                const uint8_t *base = pf_a[i];
+                const uint32_t voff = voffA;
+                if (ksl == 0)
+                    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(areg4[SET][i][0]) : "v"(voff), "s"(base) : "memory");
+                else
+                    asm volatile("global_load_dwordx4 %0, %1, %2 offset:1024" : "=v"(areg4[SET][i][1]) : "v"(voff), "s"(base) : "memory");
             } else {
-                uint4 v = *reinterpret_cast<const uint4 *>(pg);
+                uint4 v = *reinterpret_cast<const uint4 *>(pf_a[i] + voffA + ksl * PA + half * 1024);
                 areg[SET][i][ksl][4 * half + 0] = (int)v.x; areg[SET][i][ksl][4 * half + 1] = (int)v.y;
                 areg[SET][i][ksl][4 * half + 2] = (int)v.z; areg[SET][i][ksl][4 * half + 3] = (int)v.w;
             }
         } else {
-            int i = piece - TI * 2 * A_PER_FRAG;
-            const uint8_t *sp = as_ptr[i] + (size_t)(st >> 1) * 256;
-            if (AK == RFQ_MX_FP4) asm volatile("global_load_dword %0, %1, off" : "=v"(ascl[SET][i]) : "v"(sp) : "memory");
-            else ascl[SET][i] = *reinterpret_cast<const int *>(sp);
+            const int i = piece - TI * 2 * A_PER_FRAG;
+            const uint8_t *base = pf_as[i];
+            const uint32_t voff = voffAS;
+            if (AK == RFQ_MX_FP4) asm volatile("global_load_dword %0, %1, %2" : "=v"(ascl[SET][i]) : "v"(voff), "s"(base) : "memory");
+            else ascl[SET][i] = *reinterpret_cast<const int *>(base + voff);
         }
     };
     auto a_frag = [&](auto setc, int i, int ksl) -> v8i {
@@ -425,12 +493,15 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
     };
 
     v16f acc[TI][TJ];
+    auto zero_acc = [&]() {
 #pragma unroll
-    for (int i = 0; i < TI; i++)
+        for (int i = 0; i < TI; i++)
 #pragma unroll
-        for (int j = 0; j < TJ; j++)
+            for (int j = 0; j < TJ; j++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+                for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+    };
+    zero_acc();
 #pragma unroll
     for (int set = 0; set < RING; set++)
 #pragma unroll
@@ -446,77 +517,123 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
         }
 
     // ---- prologue: W(0), A(0), W(1), A(1), ..., A(RING-2), W(RING-1); then stage 0 awaited
+    const int idx0 = blockIdx.x >> 3;
+    {
+        uint32_t wl0;
+        tile_bases(idx0, pf_a, pf_as, pf_w, wl0);
+        voffA = lane16; voffAS = lane * 4; voffW = lane16; voffWL = wl0;
+    }
+    // offsets move on after every stage; scale dwords cover two stages
+    auto step_a = [&](int s) { voffA += 2 * PA; if (s & 1) voffAS += 256; };
+    auto step_w = [&](int s) { voffW += 2 * C::PB; voffWL += (s & 1) ? incWL_odd : incWL_even; };
     auto prologue_stage = [&](auto setc) {
         constexpr int SET = decltype(setc)::value;
-        const int st = clamp_stage(SET);
-        const uint32_t slot = slot_addr(SET);
 #pragma unroll
-        for (int i = 0; i < C::ND; i++) dma_piece(st, slot, i);
+        for (int i = 0; i < C::ND; i++) dma_piece(setc, i);
+        step_w(SET);
         if (SET < RING - 1) {
 #pragma unroll
-            for (int pc = 0; pc < NA_OPS; pc++) a_piece(setc, st, pc);
+            for (int pc = 0; pc < NA_OPS; pc++) a_piece(setc, pc);
+            step_a(SET);
         }
         asm volatile("" ::: "memory");
     };
     prologue_stage(IC<0>{});
     prologue_stage(IC<1>{});
-    if (RING > 2) prologue_stage(IC<2 % RING>{});
-    if (RING > 3) prologue_stage(IC<3 % RING>{});
+    prologue_stage(IC<2>{});
+    prologue_stage(IC<3>{});
     if (RING > 4) prologue_stage(IC<4 % RING>{});
     if (RING > 5) prologue_stage(IC<5 % RING>{});
     if (RING > 6) prologue_stage(IC<6 % RING>{});
     if (RING > 7) prologue_stage(IC<7 % RING>{});
-    static_assert(RING >= 3 && RING <= 8, "ring depth");
     wait_vmcnt<PROLOGUE_VMCNT>();
     barrier_no_drain();
 
     // W fragments are double-buffered by hand (k-step 0 / k-step 1), W scales
-    // by stage parity.
-    v8i fb0[TJ], fb1[TJ];
+    // by stage parity.  LDS reads take a 16-bit immediate offset: one base
+    // register per 64 KiB window of the ring.
+    using WFrag = typename Frag<BK_>::type;
+    WFrag fb0[TJ], fb1[TJ];
     int sb[2][TJ];
-    auto read_b = [&](const uint8_t *base, int ksl, int j, v8i (&fb)[TJ]) {
-        fb[j] = read_frag<BK_>(base + (j * 2 + ksl) * C::PB, lane);
+    typedef const __attribute__((address_space(3))) uint8_t *lds_u8_ptr;
+    typedef const __attribute__((address_space(3))) v4i *lds_v4i_ptr;
+    typedef const __attribute__((address_space(3))) int *lds_i32_ptr;
+    lds_u8_ptr wf0 = (lds_u8_ptr)lds + lane16, wf1 = wf0 + 65536, wf2 = wf0 + 2 * 65536; // fragment reads: lane*16 + immediate
+    lds_u8_ptr ws0 = (lds_u8_ptr)lds + lane * 4, ws1 = ws0 + 65536, ws2 = ws0 + 2 * 65536; // scale reads: lane*4 + immediate
+    // keep the windows apart: no re-folding into one base plus a large constant
+    asm volatile("" : "+v"(wf1), "+v"(wf2), "+v"(ws1), "+v"(ws2));
+    static_assert(C::RING_BYTES <= 3 * 65536, "LDS windows");
+    auto read_b = [&](int slot, int ksl, int j, WFrag (&fb)[TJ]) {
+        if (RFQ_MX_SKIP & 4) return;
+        const int off = slot * C::STAGE + (j * 2 + ksl) * C::PB;
+        lds_u8_ptr w = (off >> 16) == 0 ? wf0 : (off >> 16) == 1 ? wf1 : wf2;
+        v4i lo = *reinterpret_cast<lds_v4i_ptr>(w + (off & 65535));
+        fb[j][0] = lo[0]; fb[j][1] = lo[1]; fb[j][2] = lo[2]; fb[j][3] = lo[3];
+        if constexpr (BK_ != RFQ_MX_FP4) {
+            const int off2 = off + 1024;
+            lds_u8_ptr w2 = (off2 >> 16) == 0 ? wf0 : (off2 >> 16) == 1 ? wf1 : wf2;
+            v4i hi = *reinterpret_cast<lds_v4i_ptr>(w2 + (off2 & 65535));
+            fb[j][4] = hi[0]; fb[j][5] = hi[1]; fb[j][6] = hi[2]; fb[j][7] = hi[3];
+        }
     };
-    // A stage uses scale bytes 2*(st&1) and 2*(st&1)+1 of its dwords: shift
-    // them down so the instruction's byte selectors are constants.
-    auto read_bscale = [&](const uint8_t *base, int st, int j, int (&xb)[TJ]) {
-        xb[j] = (int)(*reinterpret_cast<const uint32_t *>(base + C::B_STAGE + (j * 64 + lane) * 4) >> (16 * (st & 1)));
+    // Scale dword of lane l for row tile j sits at (j*64 + l)*4 of the scale part.
+    auto read_bscale = [&](int slot, int j, int (&xb)[TJ]) {
+        if (RFQ_MX_SKIP & 4) return;
+        const int off = slot * C::STAGE + C::B_STAGE + j * 256;
+        lds_u8_ptr w = (off >> 16) == 0 ? ws0 : (off >> 16) == 1 ? ws1 : ws2;
+        xb[j] = *reinterpret_cast<lds_i32_ptr>(w + (off & 65535));
     };
 #pragma unroll
     for (int j = 0; j < TJ; j++) {
-        read_b(lds, 0, j, fb0);
-        read_bscale(lds, 0, j, sb[0]);
+        if (RFQ_MX_SKIP & 4) {
+#pragma unroll
+            for (int e = 0; e < (BK_ == RFQ_MX_FP4 ? 4 : 8); e++) fb0[j][e] = fb1[j][e] = 0x22222222 + lane + j;
+            sb[0][j] = sb[1][j] = 0x7f7f7f7f;
+        }
+        read_b(0, 0, j, fb0);
+        read_bscale(0, j, sb[0]);
     }
 
-    // One stage with ring set SET = st % RING, PAR = st % 2.  It contains no
-    // branch; everything that is not a matrix instruction is slotted between
-    // two of them and sched_barrier pins that order.
-    auto stage = [&](auto setc, auto parc, int st) {
-        constexpr int SET = decltype(setc)::value, PAR = decltype(parc)::value;
+    // One stage with ring set SET (a constant: the body is instantiated RING
+    // times); `st` is the stage's number within its tile, st % RING == SET, and
+    // because RING is even SET also gives the stage's parity: a scale dword
+    // holds the bytes of two stages, the instruction's byte selectors are
+    // 2*(st&1) + k-step.  The body contains no branch; everything that is not a
+    // matrix instruction is slotted between two of them and sched_barrier pins
+    // that order.
+    auto stage = [&](auto setc, int st) {
+        constexpr int SET = decltype(setc)::value, PAR = SET & 1;
         using AHEAD = IC<(SET + RING - 1) % RING>;
-        const uint8_t *base = lds + SET * C::STAGE;
-        const uint8_t *nbase = lds + ((SET + 1) % RING) * C::STAGE;
-        const int st_a = clamp_stage(st + RING - 1), st_w = clamp_stage(st + RING);
-        int sa[TI];
-#pragma unroll
-        for (int i = 0; i < TI; i++) sa[i] = (int)((uint32_t)ascl[SET][i] >> (16 * (st & 1)));
+        // SET 0 of the last trip: the prefetch streams move on to the next tile
+        const bool cross = SET == 0 && st == nstages - RING;
 
         // k-step 0; its shadow: W fragments of k-step 1, A loads RING-1 stages ahead, then the hand-over.
 #pragma unroll
         for (int q = 0; q < NMMA; q++) {
             acc[q / TJ][q % TJ] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                a_frag(setc, q / TJ, 0), fb0[q % TJ], acc[q / TJ][q % TJ], Cbsz<AK>::V, Cbsz<BK_>::V, 0, sa[q / TJ], 0,
-                sb[PAR][q % TJ]);
+                a_frag(setc, q / TJ, 0), widen(fb0[q % TJ]), acc[q / TJ][q % TJ], Cbsz<AK>::V, Cbsz<BK_>::V,
+                2 * PAR, ascl[SET][q / TJ], 2 * PAR, sb[PAR][q % TJ]);
             __builtin_amdgcn_sched_barrier(0);
-            if (q < TJ) read_b(base, 1, q, fb1);
+            if (q < TJ) read_b(SET, 1, q, fb1);
 #pragma unroll
             for (int pp = 0; pp < A_PPS; pp++)
-                if (q * A_PPS + pp < NA_OPS) a_piece(AHEAD{}, st_a, q * A_PPS + pp);
+                if (q * A_PPS + pp < NA_OPS) a_piece(AHEAD{}, q * A_PPS + pp);
             if (q == NMMA - 2) {
+                // the A stream moves one stage on (slot st + RING - 1 has been issued)
+                if (SET == 0) {
+                    voffA = cross ? lane16 : voffA + 2 * PA;
+                    voffAS = cross ? lane16 >> 2 : voffAS + (((SET + RING - 1) & 1) ? 256 : 0);
+#pragma unroll
+                    for (int i = 0; i < TI; i++) {
+                        pf_a[i] = cross ? nx_a[i] : pf_a[i];
+                        pf_as[i] = cross ? nx_as[i] : pf_as[i];
+                    }
+                } else {
+                    step_a(SET + RING - 1);
+                }
                 // Hand-over: this wavefront's last reads of the slot are complete
-                // (lgkmcnt), stage st+1 has landed in LDS and in registers
-                // (vmcnt: only what was issued after it may still be in
-                // flight), everyone agrees (barrier).
+                // (lgkmcnt), the next stage's data has landed in LDS and in
+                // registers (vmcnt), everyone agrees (barrier).
                 __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0) only
                 wait_vmcnt<HANDOVER_VMCNT>();
                 barrier_no_drain();
@@ -524,104 +641,129 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
             __builtin_amdgcn_sched_barrier(0);
         }
         // k-step 1; its shadow: the slot's refill, W fragments and scales of the next stage.
-        const uint32_t slot = slot_addr(SET);
+        if (SET == 0) {
+            voffW = cross ? lane16 : voffW;
+            voffWL = cross ? wl_nx : voffWL;
+#pragma unroll
+            for (int i = 0; i < C::ND; i++) pf_w[i] = cross ? nx_w[i] : pf_w[i];
+        }
 #pragma unroll
         for (int q = 0; q < NMMA; q++) {
             acc[q / TJ][q % TJ] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                a_frag(setc, q / TJ, 1), fb1[q % TJ], acc[q / TJ][q % TJ], Cbsz<AK>::V, Cbsz<BK_>::V, 1, sa[q / TJ], 1,
-                sb[PAR][q % TJ]);
+                a_frag(setc, q / TJ, 1), widen(fb1[q % TJ]), acc[q / TJ][q % TJ], Cbsz<AK>::V, Cbsz<BK_>::V,
+                2 * PAR + 1, ascl[SET][q / TJ], 2 * PAR + 1, sb[PAR][q % TJ]);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int pp = 0; pp < D_PPS; pp++)
-                if (q * D_PPS + pp < C::ND) dma_piece(st_w, slot, q * D_PPS + pp);
+                if (q * D_PPS + pp < C::ND) dma_piece(setc, q * D_PPS + pp);
             if (q < TJ) {
-                read_b(nbase, 0, q, fb0);
-                read_bscale(nbase, st + 1, q, sb[PAR ^ 1]);
+                read_b((SET + 1) % RING, 0, q, fb0);
+                read_bscale((SET + 1) % RING, q, sb[PAR ^ 1]);
             }
+            if (q == NMMA - 1) step_w(SET);              // slot st + RING has been issued; RING is even
             __builtin_amdgcn_sched_barrier(0);
         }
     };
 
-    RFQ_MX_STAMP(1);
-    // RING is even here or the parity is carried by a second copy of the body:
-    // unroll by lcm(RING, 2) so that ring set and stage parity are constants.
-    constexpr int UNROLL = (RING % 2 == 0) ? RING : 2 * RING;
-    for (int st = 0; st < nstages; st += UNROLL) {
-        stage(IC<0 % RING>{}, IC<0>{}, st);
-        if (st + 1 < nstages) stage(IC<1 % RING>{}, IC<1>{}, st + 1);
-        if (st + 2 < nstages) stage(IC<2 % RING>{}, IC<0>{}, st + 2);
-        if (UNROLL > 3 && st + 3 < nstages) stage(IC<3 % RING>{}, IC<1>{}, st + 3);
-        if (UNROLL > 4 && st + 4 < nstages) stage(IC<4 % RING>{}, IC<0>{}, st + 4);
-        if (UNROLL > 5 && st + 5 < nstages) stage(IC<5 % RING>{}, IC<1>{}, st + 5);
-        if (UNROLL > 6 && st + 6 < nstages) stage(IC<6 % RING>{}, IC<0>{}, st + 6);
-        if (UNROLL > 7 && st + 7 < nstages) stage(IC<7 % RING>{}, IC<1>{}, st + 7);
-        if (UNROLL > 8 && st + 8 < nstages) stage(IC<8 % RING>{}, IC<0>{}, st + 8);
-        if (UNROLL > 9 && st + 9 < nstages) stage(IC<9 % RING>{}, IC<1>{}, st + 9);
-    }
-    static_assert(UNROLL <= 10, "unroll");
-    // The trailing prefetches still write LDS slots and registers: drain them
-    // before either is reused.
-    wait_vmcnt<0>();
-    RFQ_MX_STAMP(2);
-
-    // Epilogue.  Accumulator register r of tile (i, j) is row
+    // Epilogue of one tile.  Accumulator register r of tile (i, j) is row
     // 8*(r/4) + 4*(lane/32) + r%4, column lane%32 of the tile: a lane owns
-    // single elements scattered over rows.  Interior wavefront blocks go through
-    // LDS (the ring is free now), one 32-row band at a time, and leave as whole
-    // rows in 16-byte stores; ragged blocks fall back to element stores.
+    // single elements scattered over rows.  A 32-row band goes through this
+    // wavefront's LDS staging area (behind the ring), JG instruction tiles at a
+    // time, and leaves as whole rows: 16-byte stores for blocks inside the
+    // matrix with aligned rows, a bounds-checked element loop otherwise.  LDS
+    // operations of one wavefront execute in order, so no barrier is needed
+    // around its private staging area.
     constexpr int ES = OUT_BF16 ? 2 : 4;
-    constexpr int ROW_BYTES = TJ * 32 * ES;                 // one band row of this wavefront
-    constexpr int ROW_STRIDE = ROW_BYTES + 16;              // +4 dwords: the two half-waves (rows R, R+4) miss each other's banks
-    constexpr int CPR = ROW_BYTES / 16;                     // 16-byte chunks per row
-    const int m_base = tmi * C::BM + wave * TI * 32, n_base = tn * C::BN;
-    const bool interior = m_base + TI * 32 <= M && n_base + TJ * 32 <= N && ((size_t)N * ES) % 16 == 0 &&
-                          (reinterpret_cast<uintptr_t>(outp) & 15u) == 0;
-    barrier_no_drain(); // every wavefront is past its last fragment read and its last copy
-    uint8_t *stagebuf = lds + (size_t)wave * 32 * ROW_STRIDE;
-    if (interior) {
+    constexpr int JG = C::template staging_tiles<OUT_BF16>();
+    constexpr int ROW_STRIDE = C::template staging_row_stride<OUT_BF16>(); // +4 dwords: the two half-waves (rows R, R+4) miss each other's banks
+    auto epilogue = [&](int tile_idx) {
+        // The lane number goes through an opaque statement: everything derived
+        // from it is then computed here, where registers are free, instead of
+        // being hoisted out of the tile loop and kept alive across the k loop.
+        int lane = lane_id;
+        asm volatile("" : "+v"(lane));
+        uint8_t *stagebuf = lds + C::RING_BYTES + (size_t)wave * 32 * ROW_STRIDE;
+        const int t = xcd * per + tile_idx, tn = t / tiles_m, tmi = t % tiles_m;
+        const int m_base = tmi * C::BM + wave * TI * 32, n_base = tn * C::BN;
+        const bool interior = m_base + TI * 32 <= M && n_base + TJ * 32 <= N && ((size_t)N * ES) % 16 == 0 &&
+                              (reinterpret_cast<uintptr_t>(outp) & 15u) == 0;
+        if (RFQ_MX_SKIP & 8) {
+            // keep the accumulators alive without storing them (the test is never true for finite sums of products)
+            float keep = 0.0f;
 #pragma unroll
-        for (int i = 0; i < TI; i++) {
+            for (int i = 0; i < TI; i++)
 #pragma unroll
-            for (int j = 0; j < TJ; j++)
+                for (int j = 0; j < TJ; j++)
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    int row = 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                    uint8_t *dst = stagebuf + row * ROW_STRIDE + (32 * j + (lane & 31)) * ES;
-                    if (OUT_BF16) *reinterpret_cast<uint16_t *>(dst) = f32_to_bf16(acc[i][j][r]);
-                    else *reinterpret_cast<float *>(dst) = acc[i][j][r];
-                }
-            // LDS operations of one wavefront execute in order: no barrier needed
-            // between its own writes and reads of its own staging area.
-#pragma unroll
-            for (int c0 = 0; c0 < 32 * CPR; c0 += 64) {
-                int c = c0 + lane;
-                if (c < 32 * CPR) {
-                    int row = c / CPR, col16 = c % CPR;
-                    uint4 v = *reinterpret_cast<const uint4 *>(stagebuf + row * ROW_STRIDE + col16 * 16);
-                    uint8_t *o = reinterpret_cast<uint8_t *>(outp) +
-                                 ((size_t)(m_base + 32 * i + row) * N + n_base) * ES + col16 * 16;
-                    *reinterpret_cast<uint4 *>(o) = v;
-                }
-            }
+                    for (int r = 0; r < 16; r++) keep += acc[i][j][r];
+            if (keep == 1.2345e-30f) reinterpret_cast<float *>(outp)[lane] = keep;
+            return;
         }
-    } else {
 #pragma unroll
         for (int i = 0; i < TI; i++)
 #pragma unroll
-            for (int j = 0; j < TJ; j++) {
-                int n = n_base + 32 * j + (lane & 31);
+            for (int j0 = 0; j0 < TJ; j0 += JG) {
+                const int jn = TJ - j0 < JG ? TJ - j0 : JG;
+                const int cpr = jn * 32 * ES / 16;      // 16-byte chunks per staged row
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    int m = m_base + 32 * i + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                    if (m < M && n < N) {
-                        if (OUT_BF16)
-                            reinterpret_cast<uint16_t *>(outp)[(size_t)m * N + n] = f32_to_bf16(acc[i][j][r]);
-                        else
-                            reinterpret_cast<float *>(outp)[(size_t)m * N + n] = acc[i][j][r];
+                for (int j = j0; j < j0 + jn; j++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        int row = 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                        uint8_t *dst = stagebuf + row * ROW_STRIDE + (32 * (j - j0) + (lane & 31)) * ES;
+                        if (OUT_BF16) *reinterpret_cast<uint16_t *>(dst) = f32_to_bf16(acc[i][j][r]);
+                        else *reinterpret_cast<float *>(dst) = acc[i][j][r];
+                    }
+                const int m0 = m_base + 32 * i, n0 = n_base + 32 * j0;
+                if (interior) {
+#pragma unroll
+                    for (int c0 = 0; c0 < 32 * cpr; c0 += 64) {
+                        int c = c0 + lane;
+                        if (c < 32 * cpr) {
+                            int row = c / cpr, col16 = c % cpr;
+                            uint4 v = *reinterpret_cast<const uint4 *>(stagebuf + row * ROW_STRIDE + col16 * 16);
+                            uint8_t *o = reinterpret_cast<uint8_t *>(outp) + ((size_t)(m0 + row) * N + n0) * ES + col16 * 16;
+                            *reinterpret_cast<uint4 *>(o) = v;
+                        }
+                    }
+                } else {
+                    const int ncols = jn * 32;
+#pragma nounroll
+                    for (int e = lane; e < 32 * ncols; e += 64) {
+                        int row = e / ncols, col = e % ncols;
+                        if (m0 + row < M && n0 + col < N) {
+                            const uint8_t *sp = stagebuf + row * ROW_STRIDE + col * ES;
+                            size_t o = (size_t)(m0 + row) * N + n0 + col;
+                            if (OUT_BF16) reinterpret_cast<uint16_t *>(outp)[o] = *reinterpret_cast<const uint16_t *>(sp);
+                            else reinterpret_cast<float *>(outp)[o] = *reinterpret_cast<const float *>(sp);
+                        }
                     }
                 }
             }
+    };
+
+    RFQ_MX_STAMP(1);
+    for (int idx = idx0; tile_valid(idx); idx += G8) {
+        // past the last tile the streams fetch the start of the last tile again
+        // (into registers / LDS nobody reads): every stage issues the same
+        // number of loads and the wait counts are constants
+        tile_bases(tile_valid(idx + G8) ? idx + G8 : idx, nx_a, nx_as, nx_w, wl_nx);
+        for (int st = 0; st < nstages; st += RING) {
+            stage(IC<0>{}, st);
+            stage(IC<1>{}, st + 1);
+            stage(IC<2>{}, st + 2);
+            stage(IC<3>{}, st + 3);
+            if (RING > 4) stage(IC<4 % RING>{}, st + 4);
+            if (RING > 5) stage(IC<5 % RING>{}, st + 5);
+            if (RING > 6) stage(IC<6 % RING>{}, st + 6);
+            if (RING > 7) stage(IC<7 % RING>{}, st + 7);
+        }
+        epilogue(idx);
+        zero_acc();
     }
+    // The trailing prefetches still write LDS slots and registers: drain them
+    // before the wavefront ends.
+    wait_vmcnt<0>();
     RFQ_MX_STAMP(3);
 }
 
@@ -630,10 +772,9 @@ int launch_gemm_cfg(const uint8_t *a, const uint8_t *b, void *out, int m, int n,
 {
     using C = GemmCfg<BK_, TJ, RING>;
     MxLayout LA = mx_layout(AK, m, k), LB = mx_layout(BK_, n, k);
-    constexpr size_t RINGB = (size_t)RING * C::STAGE;
-    constexpr size_t STAGING = (size_t)4 * 32 * (TJ * 32 * (OUT_BF16 ? 2 : 4) + 16);
-    constexpr size_t LDS = RINGB > STAGING ? RINGB : STAGING;
+    constexpr size_t LDS = C::template lds_bytes<OUT_BF16>();
     static_assert(LDS <= 160 * 1024, "LDS budget");
+    static_assert((MX_KS_PAD / 2) % RING == 0, "the k padding of the prepared layout must cover the ring");
     static std::once_flag once;
     static hipError_t attr_err = hipSuccess;
     std::call_once(once, [] {
@@ -641,9 +782,12 @@ int launch_gemm_cfg(const uint8_t *a, const uint8_t *b, void *out, int m, int n,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS);
     });
     if (attr_err != hipSuccess) return hip_fail(attr_err, "hipFuncSetAttribute(gemm_mx_kernel)");
-    int tiles = ((m + C::BM - 1) / C::BM) * ((n + C::BN - 1) / C::BN);
-    int per = (tiles + 7) / 8;
-    hipLaunchKernelGGL((gemm_mx_kernel<AK, BK_, OUT_BF16, TJ, RING>), dim3(per * 8), dim3(256), LDS, s, a, b, out, m,
+    const int tiles = ((m + C::BM - 1) / C::BM) * ((n + C::BN - 1) / C::BN);
+    const int per = (tiles + 7) / 8;                       // tiles per XCD
+    int g8 = device_cu_count() / 8;                        // workgroups per XCD: one per CU
+    if (g8 < 1) g8 = 1;
+    if (g8 > per) g8 = per;
+    hipLaunchKernelGGL((gemm_mx_kernel<AK, BK_, OUT_BF16, TJ, RING>), dim3(g8 * 8), dim3(256), LDS, s, a, b, out, m,
                        n, LA, LB);
     RFQ_LAUNCH_CHECK("gemm_mx_kernel");
     return RFQ_OK;
@@ -657,7 +801,7 @@ template <int AK, int BK_, bool OUT_BF16>
 int run_gemm(const uint8_t *a, const uint8_t *b, void *out, int m, int n, int k, hipStream_t s)
 {
     if constexpr (AK == RFQ_MX_FP8 || BK_ == RFQ_MX_FP8)
-        return launch_gemm_cfg<AK, BK_, OUT_BF16, 4, 4>(a, b, out, m, n, k, s);
+        return launch_gemm_cfg<AK, BK_, OUT_BF16, 4, RFQ_MX_RING>(a, b, out, m, n, k, s);
     else
         return launch_gemm_cfg<AK, BK_, OUT_BF16, 7, RFQ_MX_RING>(a, b, out, m, n, k, s);
 }
