@@ -58,6 +58,8 @@ namespace {
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 
 // k-steps (64 elements) of a prepared matrix are padded with zero pages to a
 // multiple of MX_KS_PAD, so that the GEMM's k loop is a whole number of trips
@@ -240,13 +242,6 @@ template <int KIND> struct Frag { using type = v8i; };
 template <> struct Frag<RFQ_MX_FP4> { using type = v4i; };
 __device__ __forceinline__ v8i widen(v8i f) { return f; }
 __device__ __forceinline__ v8i widen(v4i f) { return __builtin_shufflevector(f, f, 0, 1, 2, 3, -1, -1, -1, -1); }
-
-__device__ __forceinline__ uint16_t f32_to_bf16(float f)
-{
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40u); // NaN stays NaN
-    return (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);                  // round to nearest even
-}
 
 // s_waitcnt with only the vector-memory counter constrained (gfx9 encoding:
 // vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] at [15:14]).
@@ -682,7 +677,6 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
         // being hoisted out of the tile loop and kept alive across the k loop.
         int lane = lane_id;
         asm volatile("" : "+v"(lane));
-        uint8_t *stagebuf = lds + C::RING_BYTES + (size_t)wave * 32 * ROW_STRIDE;
         const int t = xcd * per + tile_idx, tn = t / tiles_m, tmi = t % tiles_m;
         const int m_base = tmi * C::BM + wave * TI * 32, n_base = tn * C::BN;
         const bool interior = m_base + TI * 32 <= M && n_base + TJ * 32 <= N && ((size_t)N * ES) % 16 == 0 &&
@@ -699,6 +693,10 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
             if (keep == 1.2345e-30f) reinterpret_cast<float *>(outp)[lane] = keep;
             return;
         }
+        typedef __attribute__((address_space(3))) uint8_t *lds_w8_ptr;
+        lds_w8_ptr stage3 = (lds_w8_ptr)lds + C::RING_BYTES + wave * 32 * ROW_STRIDE;
+        // this lane's accumulator elements: rows 4*(lane/32) + {0..3, 8..11, 16..19, 24..27}, column lane%32 of a tile
+        lds_w8_ptr wr = stage3 + 4 * (lane >> 5) * ROW_STRIDE + (lane & 31) * ES;
 #pragma unroll
         for (int i = 0; i < TI; i++)
 #pragma unroll
@@ -708,25 +706,39 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
 #pragma unroll
                 for (int j = j0; j < j0 + jn; j++)
 #pragma unroll
-                    for (int r = 0; r < 16; r++) {
-                        int row = 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                        uint8_t *dst = stagebuf + row * ROW_STRIDE + (32 * (j - j0) + (lane & 31)) * ES;
-                        if (OUT_BF16) *reinterpret_cast<uint16_t *>(dst) = f32_to_bf16(acc[i][j][r]);
-                        else *reinterpret_cast<float *>(dst) = acc[i][j][r];
+                    for (int r = 0; r < 16; r += 2) {
+                        const int off = (8 * (r >> 2) + (r & 3)) * ROW_STRIDE + 32 * (j - j0) * ES; // r even: r + 1 is the next row
+                        if (OUT_BF16) {
+                            // one conversion instruction per pair (round to nearest even), one 16-bit write per half
+                            f32x2_t v = {acc[i][j][r], acc[i][j][r + 1]};
+                            bf16x2_t b = __builtin_convertvector(v, bf16x2_t);
+                            uint32_t u;
+                            __builtin_memcpy(&u, &b, 4);
+                            *reinterpret_cast<__attribute__((address_space(3))) uint16_t *>(wr + off) = (uint16_t)u;
+                            *reinterpret_cast<__attribute__((address_space(3))) uint16_t *>(wr + off + ROW_STRIDE) = (uint16_t)(u >> 16);
+                        } else {
+                            *reinterpret_cast<__attribute__((address_space(3))) float *>(wr + off) = acc[i][j][r];
+                            *reinterpret_cast<__attribute__((address_space(3))) float *>(wr + off + ROW_STRIDE) = acc[i][j][r + 1];
+                        }
                     }
                 const int m0 = m_base + 32 * i, n0 = n_base + 32 * j0;
                 if (interior) {
+                    // whole rows leave in 16-byte stores: a pass moves `rpi` rows, lane l the chunk l % cpr of row l / cpr
+                    const int rpi = 64 / cpr;
+                    static_assert(32 * ES * 16 / 16 <= 64 * 16, "a staged row is at most 64 chunks");
+                    const int row_l = lane / cpr, col16 = lane - row_l * cpr;
+                    lds_w8_ptr rd = stage3 + row_l * ROW_STRIDE + col16 * 16;
+                    uint8_t *o = reinterpret_cast<uint8_t *>(outp) + ((size_t)(m0 + row_l) * N + n0) * ES + col16 * 16;
+                    const size_t pass_bytes = (size_t)rpi * N * ES;
+                    if (lane < rpi * cpr) {
 #pragma unroll
-                    for (int c0 = 0; c0 < 32 * cpr; c0 += 64) {
-                        int c = c0 + lane;
-                        if (c < 32 * cpr) {
-                            int row = c / cpr, col16 = c % cpr;
-                            uint4 v = *reinterpret_cast<const uint4 *>(stagebuf + row * ROW_STRIDE + col16 * 16);
-                            uint8_t *o = reinterpret_cast<uint8_t *>(outp) + ((size_t)(m0 + row) * N + n0) * ES + col16 * 16;
-                            *reinterpret_cast<uint4 *>(o) = v;
+                        for (int it = 0; it < 32 / rpi; it++) {
+                            v4i v = *reinterpret_cast<const __attribute__((address_space(3))) v4i *>(rd + it * rpi * ROW_STRIDE);
+                            *reinterpret_cast<v4i *>(o + it * pass_bytes) = v;
                         }
                     }
                 } else {
+                    const uint8_t *stagebuf = lds + C::RING_BYTES + (size_t)wave * 32 * ROW_STRIDE;
                     const int ncols = jn * 32;
 #pragma nounroll
                     for (int e = lane; e < 32 * ncols; e += 64) {
