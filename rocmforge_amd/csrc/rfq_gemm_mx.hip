@@ -47,9 +47,10 @@ __device__ unsigned long long *rfq_mx_trace;
 #ifndef RFQ_MX_SKIP
 #define RFQ_MX_SKIP 0
 #endif
-// Ring depth (W slots in LDS = A fragment sets in registers) of the 4-bit kernel.
+// Ring depth (W slots in LDS = A fragment sets in registers) with 4-bit A
+// fragments; 8-bit A fragments take twice the registers and half the depth.
 #ifndef RFQ_MX_RING
-#define RFQ_MX_RING 6
+#define RFQ_MX_RING 8
 #endif
 
 namespace rfq {
@@ -64,7 +65,7 @@ typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 // k-steps (64 elements) of a prepared matrix are padded with zero pages to a
 // multiple of MX_KS_PAD, so that the GEMM's k loop is a whole number of trips
 // through its unrolled prefetch ring and needs no remainder code.
-constexpr int MX_KS_PAD = 12;
+constexpr int MX_KS_PAD = 16;
 
 struct MxLayout {
     int rows, k, rt, ks, ks4, ks_real; // ks: padded k-steps per row tile; ks_real: k / 64
@@ -305,13 +306,19 @@ template <int BK_, int TJ, int RING_> struct GemmCfg {
     static constexpr int WL = STAGE / 1024;                       // 1 KiB wave-copies per stage
     static constexpr int ND = (WL + 3) / 4;                       // per wavefront (padded with repeats)
     static constexpr int RING_BYTES = RING * STAGE;
-    // the epilogue stages a 32-row band JG instruction tiles (32 columns each) at a time
-    template <bool OUT_BF16> static constexpr int staging_tiles() { return OUT_BF16 ? TJ : (TJ > 1 ? TJ / 2 : 1); }
-    template <bool OUT_BF16> static constexpr int staging_row_stride()
+    // The epilogue stages RB full-width rows of a wavefront's 32-row band at a
+    // time: as many as fit behind the ring in 160 KiB of LDS.
+    template <bool OUT_BF16> static constexpr int staging_row_stride() { return TJ * 32 * (OUT_BF16 ? 2 : 4) + 16; }
+    template <bool OUT_BF16> static constexpr int staging_rows()
     {
-        return staging_tiles<OUT_BF16>() * 32 * (OUT_BF16 ? 2 : 4) + 16;
+        int rb = 32;
+        while (rb > 8 && RING_BYTES + 4 * rb * staging_row_stride<OUT_BF16>() > 160 * 1024) rb /= 2;
+        return rb;
     }
-    template <bool OUT_BF16> static constexpr int lds_bytes() { return RING_BYTES + 4 * 32 * staging_row_stride<OUT_BF16>(); }
+    template <bool OUT_BF16> static constexpr int lds_bytes()
+    {
+        return RING_BYTES + 4 * staging_rows<OUT_BF16>() * staging_row_stride<OUT_BF16>();
+    }
 };
 
 template <int N> struct IC { static constexpr int value = N; };
@@ -662,14 +669,14 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
 
     // Epilogue of one tile.  Accumulator register r of tile (i, j) is row
     // 8*(r/4) + 4*(lane/32) + r%4, column lane%32 of the tile: a lane owns
-    // single elements scattered over rows.  A 32-row band goes through this
-    // wavefront's LDS staging area (behind the ring), JG instruction tiles at a
-    // time, and leaves as whole rows: 16-byte stores for blocks inside the
-    // matrix with aligned rows, a bounds-checked element loop otherwise.  LDS
-    // operations of one wavefront execute in order, so no barrier is needed
-    // around its private staging area.
+    // single elements scattered over rows.  RB rows of a 32-row band at a time
+    // go through this wavefront's LDS staging area (behind the ring) and leave
+    // as whole rows: 16-byte stores for blocks inside the matrix with aligned
+    // rows, a bounds-checked element loop otherwise.  LDS operations of one
+    // wavefront execute in order, so no barrier is needed around its private
+    // staging area.
     constexpr int ES = OUT_BF16 ? 2 : 4;
-    constexpr int JG = C::template staging_tiles<OUT_BF16>();
+    constexpr int RB = C::template staging_rows<OUT_BF16>();
     constexpr int ROW_STRIDE = C::template staging_row_stride<OUT_BF16>(); // +4 dwords: the two half-waves (rows R, R+4) miss each other's banks
     auto epilogue = [&](int tile_idx) {
         // The lane number goes through an opaque statement: everything derived
@@ -694,20 +701,28 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
             return;
         }
         typedef __attribute__((address_space(3))) uint8_t *lds_w8_ptr;
-        lds_w8_ptr stage3 = (lds_w8_ptr)lds + C::RING_BYTES + wave * 32 * ROW_STRIDE;
+        lds_w8_ptr stage3 = (lds_w8_ptr)lds + C::RING_BYTES + wave * RB * ROW_STRIDE;
         // this lane's accumulator elements: rows 4*(lane/32) + {0..3, 8..11, 16..19, 24..27}, column lane%32 of a tile
         lds_w8_ptr wr = stage3 + 4 * (lane >> 5) * ROW_STRIDE + (lane & 31) * ES;
+        // whole rows leave in 16-byte stores: a pass moves `rpi` rows, lane l
+        // the chunk l % cpr of row l / cpr (rpi: the largest power of two with
+        // rpi * cpr <= 64)
+        constexpr int cpr = TJ * 32 * ES / 16;           // 16-byte chunks per row
+        constexpr int rpi = cpr <= 2 ? 32 : cpr <= 4 ? 16 : cpr <= 8 ? 8 : cpr <= 16 ? 4 : cpr <= 32 ? 2 : 1;
+        static_assert(cpr <= 64 && rpi <= RB, "row store mapping");
+        const int row_l = lane / cpr, col16 = lane - row_l * cpr;
+        lds_w8_ptr rd = stage3 + row_l * ROW_STRIDE + col16 * 16;
+        const size_t pass_bytes = (size_t)rpi * N * ES;
 #pragma unroll
         for (int i = 0; i < TI; i++)
 #pragma unroll
-            for (int j0 = 0; j0 < TJ; j0 += JG) {
-                const int jn = TJ - j0 < JG ? TJ - j0 : JG;
-                const int cpr = jn * 32 * ES / 16;      // 16-byte chunks per staged row
+            for (int h = 0; h < 32 / RB; h++) {
+                // registers r in [h*RB/2, (h+1)*RB/2) are rows [h*RB, (h+1)*RB) of the band
 #pragma unroll
-                for (int j = j0; j < j0 + jn; j++)
+                for (int j = 0; j < TJ; j++)
 #pragma unroll
-                    for (int r = 0; r < 16; r += 2) {
-                        const int off = (8 * (r >> 2) + (r & 3)) * ROW_STRIDE + 32 * (j - j0) * ES; // r even: r + 1 is the next row
+                    for (int r = h * RB / 2; r < (h + 1) * RB / 2; r += 2) {
+                        const int off = (8 * (r >> 2) + (r & 3) - h * RB) * ROW_STRIDE + 32 * j * ES; // r even: r + 1 is the next row
                         if (OUT_BF16) {
                             // one conversion instruction per pair (round to nearest even), one 16-bit write per half
                             f32x2_t v = {acc[i][j][r], acc[i][j][r + 1]};
@@ -721,31 +736,25 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
                             *reinterpret_cast<__attribute__((address_space(3))) float *>(wr + off + ROW_STRIDE) = acc[i][j][r + 1];
                         }
                     }
-                const int m0 = m_base + 32 * i, n0 = n_base + 32 * j0;
+                const int m0 = m_base + 32 * i + h * RB;
                 if (interior) {
-                    // whole rows leave in 16-byte stores: a pass moves `rpi` rows, lane l the chunk l % cpr of row l / cpr
-                    const int rpi = 64 / cpr;
-                    static_assert(32 * ES * 16 / 16 <= 64 * 16, "a staged row is at most 64 chunks");
-                    const int row_l = lane / cpr, col16 = lane - row_l * cpr;
-                    lds_w8_ptr rd = stage3 + row_l * ROW_STRIDE + col16 * 16;
-                    uint8_t *o = reinterpret_cast<uint8_t *>(outp) + ((size_t)(m0 + row_l) * N + n0) * ES + col16 * 16;
-                    const size_t pass_bytes = (size_t)rpi * N * ES;
+                    uint8_t *o = reinterpret_cast<uint8_t *>(outp) + ((size_t)(m0 + row_l) * N + n_base) * ES + col16 * 16;
                     if (lane < rpi * cpr) {
 #pragma unroll
-                        for (int it = 0; it < 32 / rpi; it++) {
+                        for (int it = 0; it < RB / rpi; it++) {
                             v4i v = *reinterpret_cast<const __attribute__((address_space(3))) v4i *>(rd + it * rpi * ROW_STRIDE);
                             *reinterpret_cast<v4i *>(o + it * pass_bytes) = v;
                         }
                     }
                 } else {
-                    const uint8_t *stagebuf = lds + C::RING_BYTES + (size_t)wave * 32 * ROW_STRIDE;
-                    const int ncols = jn * 32;
+                    const uint8_t *stagebuf = lds + C::RING_BYTES + (size_t)wave * RB * ROW_STRIDE;
+                    const int ncols = TJ * 32;
 #pragma nounroll
-                    for (int e = lane; e < 32 * ncols; e += 64) {
+                    for (int e = lane; e < RB * ncols; e += 64) {
                         int row = e / ncols, col = e % ncols;
-                        if (m0 + row < M && n0 + col < N) {
+                        if (m0 + row < M && n_base + col < N) {
                             const uint8_t *sp = stagebuf + row * ROW_STRIDE + col * ES;
-                            size_t o = (size_t)(m0 + row) * N + n0 + col;
+                            size_t o = (size_t)(m0 + row) * N + n_base + col;
                             if (OUT_BF16) reinterpret_cast<uint16_t *>(outp)[o] = *reinterpret_cast<const uint16_t *>(sp);
                             else reinterpret_cast<float *>(outp)[o] = *reinterpret_cast<const float *>(sp);
                         }
@@ -813,7 +822,7 @@ template <int AK, int BK_, bool OUT_BF16>
 int run_gemm(const uint8_t *a, const uint8_t *b, void *out, int m, int n, int k, hipStream_t s)
 {
     if constexpr (AK == RFQ_MX_FP8 || BK_ == RFQ_MX_FP8)
-        return launch_gemm_cfg<AK, BK_, OUT_BF16, 4, RFQ_MX_RING>(a, b, out, m, n, k, s);
+        return launch_gemm_cfg<AK, BK_, OUT_BF16, 4, (AK == RFQ_MX_FP4 ? RFQ_MX_RING : RFQ_MX_RING / 2)>(a, b, out, m, n, k, s);
     else
         return launch_gemm_cfg<AK, BK_, OUT_BF16, 7, RFQ_MX_RING>(a, b, out, m, n, k, s);
 }
