@@ -743,7 +743,7 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
 #pragma unroll
                         for (int it = 0; it < RB / rpi; it++) {
                             v4i v = *reinterpret_cast<const __attribute__((address_space(3))) v4i *>(rd + it * rpi * ROW_STRIDE);
-                            *reinterpret_cast<v4i *>(o + it * pass_bytes) = v;
+                            __builtin_nontemporal_store(v, reinterpret_cast<v4i *>(o + it * pass_bytes)); // written once, never read here
                         }
                     }
                 } else {
