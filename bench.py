@@ -26,6 +26,10 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 N, K = 14336, 4096
 CACHE_BYTES = 256 << 20
+# HBM bytes one launch of the headline kernel moves, from FETCH_SIZE / WRITE_SIZE
+# profiler counters scaled by a copy kernel of known size
+# (profiles/gemv_q4k_14336x4096_hbm_counters.txt): 57,631.7 KiB read + 64.0 KiB written.
+MEASURED_TRAFFIC_BYTES = 59080397
 
 
 def algorithmic_bytes(fmt, n, k, m, Q):
@@ -95,6 +99,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-also", action="store_true", help="skip the secondary configurations")
+    ap.add_argument("--no-warm", action="store_true", help="skip the cache-resident variant (profiling runs)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain elementwise copy of 256 MiB five times (for scaling HBM byte counters "
+                         "of a profiler against a kernel of known traffic)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build is single-GPU (one MI355X per box); run with --gpus 1. "
@@ -119,7 +127,9 @@ def main():
     achieved = abytes / (dev_s / args.steps) / 1e9
 
     # warm variant (one copy, cache-resident) for the record
-    wall_w, dev_w, *_ = time_gemv(torch, fmt, N, K, 1, 1, args.steps, args.warmup, Q, 20260003)
+    dev_w = None
+    if not args.no_warm:
+        _, dev_w, *_ = time_gemv(torch, fmt, N, K, 1, 1, args.steps, args.warmup, Q, 20260003)
 
     out = {
         "metric": "Q4_K decode GEMV GB/s (% HBM peak); quant prefill GEMM TFLOP/s (% MFMA peak)",
@@ -138,10 +148,18 @@ def main():
                                f"{copies} rotating weight copies (cold HBM)",
                    "algorithmic_bytes_per_step": abytes, "weight_copies": copies},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
                      "kernel": "gemv_idot_kernel<Q4_K,2,1,7>", "avg_launch_us": round(dev_s / args.steps * 1e6, 3),
-                     "warm_cache_gbs": round(abytes / (dev_w / args.steps) / 1e9, 1)},
+                     "warm_cache_gbs": round(abytes / (dev_w / args.steps) / 1e9, 1) if dev_w else None},
     }
+
+    if args.calibrate_copy:
+        src = torch.ones(64 << 20, dtype=torch.float32, device="cuda:0")
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            torch.add(src, 0.0, out=dst)                   # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        out["config"]["calibration_copy"] = "5 x torch.add(src, 0, out=dst), 2^26 floats each way"
 
     if not args.no_also:
         also = {}
