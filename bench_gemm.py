@@ -42,9 +42,31 @@ def mx_gemm(torch, w_fmt, m=2048, n=28672, k=8192, steps=20, warmup=3):
             "peak_TFLOP/s": peak / 1e12, "kinds": [A.kind, W.kind]}
 
 
+def kq_gemm(torch, fmt, m=512, n=14336, k=4096, steps=50, warmup=5):
+    """Q4_K / Q6_K prefill GEMM on the fp16 matrix cores, fp16 in and out."""
+    from rocmforge_amd import _lib, quantize as Q
+    dev = torch.device("cuda:0")
+    w = torch.from_numpy(Q.make_weights(fmt, n, k, seed=20260004)).to(dev)
+    a = torch.from_numpy(_gauss(m, k, 20260014, 1.0).astype(np.float16)).to(dev)
+    out = torch.empty((m, n), dtype=torch.float16, device=dev)
+    ms = C.c_float(0)
+    L = _lib.lib()
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    args = (fmt, C.c_void_p(w.data_ptr()), w.numel(), C.c_void_p(a.data_ptr()), C.c_void_p(out.data_ptr()), _lib.F16,
+            m, n, k)
+    _lib.check(L.rfq_bench_gemm_f16(*args, 0, warmup, stream, C.byref(ms)))
+    _lib.check(L.rfq_bench_gemm_f16(*args, 0, steps, stream, C.byref(ms)))
+    t = ms.value / 1e3 / steps
+    flops = 2.0 * m * n * k
+    return {"TFLOP/s": round(flops / t / 1e12, 1), "us": round(t * 1e6, 1), "mfma_frac": round(flops / t / 2.5e15, 4),
+            "peak_TFLOP/s": 2500.0}
+
+
 def run(torch):
     from rocmforge_amd import quantize as Q
     res = {}
+    res["Q4_K gemm 512x4096x14336 fp16"] = kq_gemm(torch, Q.Q4_K)
+    res["Q6_K gemm 512x4096x14336 fp16"] = kq_gemm(torch, Q.Q6_K)
     res["MXFP4 gemm 2048x8192x28672 bf16"] = mx_gemm(torch, Q.MXFP4)
     res["MXFP6-weight gemm 2048x8192x28672 bf16"] = mx_gemm(torch, Q.MXFP6_E2M3)
     return res
@@ -55,12 +77,14 @@ if __name__ == "__main__":
     import os
     sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
     ap = argparse.ArgumentParser()
-    ap.add_argument("--only", choices=["mxfp4", "mxfp6"], help="one configuration (for profiling runs)")
+    ap.add_argument("--only", choices=["mxfp4", "mxfp6", "q4_k"], help="one configuration (for profiling runs)")
     ap.add_argument("--steps", type=int, default=20)
     a = ap.parse_args()
     import torch
     from rocmforge_amd import quantize as Q
-    if a.only:
+    if a.only == "q4_k":
+        print(json.dumps(kq_gemm(torch, Q.Q4_K, steps=a.steps, warmup=2)))
+    elif a.only:
         print(json.dumps(mx_gemm(torch, Q.MXFP4 if a.only == "mxfp4" else Q.MXFP6_E2M3, steps=a.steps, warmup=2)))
     else:
         print(json.dumps(run(torch)))

@@ -1,0 +1,97 @@
+"""GPU parity: prefill GEMM for Q4_0 / Q8_0 / Q4_K / Q6_K on the fp16 matrix
+cores against the CPU oracle (dequantise as the reference does, then its
+sequential fp32 matmul over the fp16 activations widened to f32)."""
+import numpy as np
+import pytest
+
+from helpers import assert_close
+from rocmforge_amd import quantize as Q
+
+pytestmark = pytest.mark.gpu
+
+FORMATS = [Q.Q4_0, Q.Q8_0, Q.Q4_K, Q.Q6_K]
+
+
+def acts(m, k, seed):
+    rng = np.random.Generator(np.random.PCG64(seed))
+    return rng.standard_normal((m, k), dtype=np.float32).astype(np.float16)
+
+
+def weights(fmt, n, k, seed):
+    if fmt == Q.Q4_K and seed % 2:
+        # a real min/max-free quantisation of N(0, 0.02) data (one-sided sub-blocks) next to the synthetic blocks
+        rng = np.random.Generator(np.random.PCG64(seed))
+        return Q.quantize_q4_k_onesided(rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02))
+    return Q.make_weights(fmt, n, k, seed=seed)
+
+
+def run(fmt, w, a, n, k, cuda, out_dtype):
+    import torch
+    from rocmforge_amd import ops
+    out = ops.gemm_f16(fmt, torch.from_numpy(w).to(cuda), torch.from_numpy(a).to(cuda), n, k, out_dtype=out_dtype)
+    torch.cuda.synchronize()
+    return out
+
+
+@pytest.mark.parametrize("fmt", FORMATS)
+@pytest.mark.parametrize("m,n,k", [(1, 32, 256), (33, 70, 256), (300, 200, 512), (256, 128, 1024), (512, 259, 768)])
+def test_small_shapes_fp32_out(fmt, m, n, k, oracle, cuda):
+    import torch
+    w, a = weights(fmt, n, k, 100 + fmt + m), acts(m, k, 200 + n)
+    out = run(fmt, w, a, n, k, cuda, torch.float32).cpu().numpy()
+    want = oracle.qmatmul_nk(fmt, w, a.astype(np.float32), m, n, k)
+    assert_close(out, want, f"{Q.NAMES[fmt]} {m}x{n}x{k}")                # max rel err <= 1e-3
+
+
+@pytest.mark.parametrize("fmt", [Q.Q4_0, Q.Q8_0])
+def test_k_not_a_multiple_of_the_stage(fmt, oracle, cuda):
+    import torch
+    m, n, k = 40, 96, 96 + 64 * 3                                        # k % 64 == 32
+    w, a = weights(fmt, n, k, 7), acts(m, k, 8)
+    out = run(fmt, w, a, n, k, cuda, torch.float32).cpu().numpy()
+    assert_close(out, oracle.qmatmul_nk(fmt, w, a.astype(np.float32), m, n, k), "k tail")
+
+
+@pytest.mark.parametrize("fmt", FORMATS)
+def test_fp16_output_is_the_rounded_fp32_output(fmt, cuda):
+    import torch
+    m, n, k = 130, 264, 512
+    w, a = weights(fmt, n, k, 31), acts(m, k, 32)
+    f32 = run(fmt, w, a, n, k, cuda, torch.float32)
+    f16 = run(fmt, w, a, n, k, cuda, torch.float16)
+    assert torch.equal(f16, f32.to(torch.float16))                        # same accumulation, RNE cast
+
+
+@pytest.mark.parametrize("fmt", [Q.Q4_K, Q.Q6_K])
+def test_full_size_sampled(fmt, oracle, cuda):
+    """M=512, K=4096, N=14336, fp16 in and out: sampled output columns against
+    the oracle, and a checksum over every output:
+    sum_n out[m, n] = A[m, :] . sum_n W[n, :]."""
+    import torch
+    m, n, k = 512, 14336, 4096
+    w, a = Q.make_weights(fmt, n, k, seed=20260004), acts(m, k, 20260014)
+    f32 = run(fmt, w, a, n, k, cuda, torch.float32)
+    f16 = run(fmt, w, a, n, k, cuda, torch.float16)
+    assert torch.equal(f16, f32.to(torch.float16))
+    cols = np.array([0, 1, 31, 32, 127, 128, 4095, 7000, 14335])
+    want = oracle.qmatmul_nk(fmt, w, a.astype(np.float32), m, n, k, rows=cols)
+    got = f32[:, torch.from_numpy(cols).to(cuda)].cpu().numpy()
+    assert_close(got, want, "sampled fp32")
+    got16 = f16[:, torch.from_numpy(cols).to(cuda)].float().cpu().numpy()
+    assert_close(got16, want, "sampled fp16", tol=1e-3 + 2.0 ** -11)      # one fp16 rounding on top
+    wsum = oracle.dequantize(fmt, w, n * k).reshape(n, k).astype(np.float64).sum(axis=0)
+    check = f32.double().sum(dim=1).cpu().numpy()
+    # each output carries the fp16 rounding of its weights (about 1e-4 rms, random sign): the sums of
+    # 14336 of them agree to the same order; one wrong element would move a sum by about 1e-2
+    assert_close(check, a.astype(np.float64) @ wsum, "row checksums", tol=1e-3)
+
+
+def test_rejects_bad_arguments(cuda):
+    import torch
+    from rocmforge_amd import _lib, ops
+    w = torch.zeros(Q.packed_bytes(Q.Q4_K, 64 * 256), dtype=torch.uint8, device=cuda)
+    a = torch.zeros((4, 256), dtype=torch.float16, device=cuda)
+    with pytest.raises(_lib.RfqError):
+        ops.gemm_f16(Q.MXFP4, w, a, 64, 256)                              # MXFP goes through rfq_gemm_mx
+    with pytest.raises(_lib.RfqError):
+        ops.gemm_f16(Q.Q4_K, w[:-1], a, 64, 256)                          # byte count does not match the shape
