@@ -27,11 +27,30 @@
 
 #include "rfq_common.hpp"
 
+// -DRFQ_KQ_SKIP=<mask> (tuning builds, results are wrong on purpose): leave out
+// 1 the A loads, 2 the W loads, 4 the LDS fragment reads, 8 the LDS writes,
+// 16 the weight decoding, to see what a stage's time is made of.
+#ifndef RFQ_KQ_SKIP
+#define RFQ_KQ_SKIP 0
+#endif
+
 namespace rfq {
 namespace {
 
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
+template <int N> struct IC { static constexpr int value = N; };
+
+// Workgroup barrier for LDS hand-over that leaves global loads in flight
+// (__syncthreads would wait for the prefetches issued just before it): this
+// wavefront's LDS writes are complete (lgkmcnt), then everyone meets.
+__device__ __forceinline__ void lds_barrier()
+{
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0); vmcnt and expcnt unconstrained
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
 
 constexpr int BM = 256, BN = 128, BK = 64;
 constexpr int LDR = BK * 2 + 16;                 // bytes per LDS row: 64 fp16 + 16 pad (rows 36 dwords apart)
@@ -46,9 +65,12 @@ template <> struct Raw32<RFQ_Q4_0> {
     uint32_t d[ND];
     __device__ __forceinline__ void load(const uint8_t *row, int g)
     {
+        // few wide loads: every lane touches a different cache line, so the
+        // address path pays per instruction, not per byte
         const uint8_t *p = row + (size_t)g * 20;
-#pragma unroll
-        for (int i = 0; i < ND; i++) d[i] = ld<uint32_t>(p + 4 * i);
+        d[0] = ld<uint32_t>(p);
+        uint4 q = ld<uint4>(p + 4);
+        d[1] = q.x; d[2] = q.y; d[3] = q.z; d[4] = q.w;
     }
     __device__ __forceinline__ void zero()
     {
@@ -71,8 +93,10 @@ template <> struct Raw32<RFQ_Q8_0> {
     __device__ __forceinline__ void load(const uint8_t *row, int g)
     {
         const uint8_t *p = row + (size_t)g * 36;
-#pragma unroll
-        for (int i = 0; i < ND; i++) d[i] = ld<uint32_t>(p + 4 * i);
+        d[0] = ld<uint32_t>(p);
+        uint4 q0 = ld<uint4>(p + 4), q1 = ld<uint4>(p + 20);
+        d[1] = q0.x; d[2] = q0.y; d[3] = q0.z; d[4] = q0.w;
+        d[5] = q1.x; d[6] = q1.y; d[7] = q1.z; d[8] = q1.w;
     }
     __device__ __forceinline__ void zero()
     {
@@ -97,9 +121,11 @@ template <> struct Raw32<RFQ_Q4_K> {
     {
         const uint8_t *blk = row + (size_t)(g >> 3) * 256;
         const int sb = g & 7;
-        d[0] = (uint32_t)ld<uint16_t>(blk + 2 * sb) | ((uint32_t)blk[16 + sb] << 16);
-#pragma unroll
-        for (int i = 0; i < 4; i++) d[1 + i] = ld<uint32_t>(blk + 32 + 28 * sb + 4 * i);
+        // the aligned dwords that hold scale sb and min sb, then the 16 nibble bytes
+        uint32_t sc = ld<uint32_t>(blk + 2 * (sb & ~1)), mn = ld<uint32_t>(blk + 16 + (sb & ~3));
+        d[0] = ((sc >> (16 * (sb & 1))) & 0xFFFFu) | (((mn >> (8 * (sb & 3))) & 0xFFu) << 16);
+        uint4 q = ld<uint4>(blk + 32 + 28 * sb);
+        d[1] = q.x; d[2] = q.y; d[3] = q.z; d[4] = q.w;
     }
     __device__ __forceinline__ void zero()
     {
@@ -126,8 +152,9 @@ template <> struct Raw32<RFQ_Q6_K> {
         const uint8_t *blk = row + (size_t)(g >> 3) * 256;
         const int s = g & 7;
         d[0] = ld<uint32_t>(blk + 4 * s);
-#pragma unroll
-        for (int i = 0; i < 6; i++) d[1 + i] = ld<uint32_t>(blk + 32 + 24 * s + 4 * i);
+        uint4 q = ld<uint4>(blk + 32 + 24 * s);
+        uint2 q2 = ld<uint2>(blk + 32 + 24 * s + 16);
+        d[1] = q.x; d[2] = q.y; d[3] = q.z; d[4] = q.w; d[5] = q2.x; d[6] = q2.y;
     }
     __device__ __forceinline__ void zero()
     {
@@ -188,31 +215,61 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const _Float16 *__restrict__ a, co
     const uint8_t *w_row = w + (size_t)(w_row_ok ? n0 + wr : 0) * row_bytes;
     const int a_chunk = tid & 7, a_row0 = tid >> 3;               // rows a_row0 + 32*i
 
-    Raw32<FMT> raw;
-    uint4 ra[8];
-    auto fetch = [&](int st) {
+    // Global loads run three stages ahead of the arithmetic, through a ring of
+    // three register sets (indices are compile-time: the loop is unrolled by 3).
+    Raw32<FMT> raws[3];
+    uint4 ras[3][8];
+    // The loads are unconditional (clamped addresses): branches around them
+    // would make the compiler wait for every outstanding load at each join.
+    // Rows past M or N only feed outputs that are never stored; k past K is
+    // cancelled by zero weights (selected after the load), whatever finite
+    // activations the clamped address returns.
+    auto fetch = [&](auto slotc, int st) {
+        constexpr int S = decltype(slotc)::value;
         const int g = st * 2 + wg;
-        if (w_row_ok && g < groups) raw.load(w_row, g);
-        else raw.zero();
+        if (!(RFQ_KQ_SKIP & 2)) raws[S].load(w_row, g < groups ? g : groups - 1);
+        Raw32<FMT> z;
+        z.zero();
+#pragma unroll
+        for (int i = 0; i < Raw32<FMT>::ND; i++) raws[S].d[i] = g < groups ? raws[S].d[i] : z.d[i];
+        const int k = st * BK + a_chunk * 8, kc = k < K ? k : K - 8;
 #pragma unroll
         for (int i = 0; i < 8; i++) {
-            const int m = m0 + a_row0 + 32 * i, k = st * BK + a_chunk * 8;
-            if (m < M && k < K) ra[i] = *reinterpret_cast<const uint4 *>(a + (size_t)m * K + k);
-            else ra[i] = make_uint4(0, 0, 0, 0);
+            const int m = m0 + a_row0 + 32 * i, mc = m < M ? m : M - 1;
+            if (!(RFQ_KQ_SKIP & 1)) ras[S][i] = *reinterpret_cast<const uint4 *>(a + (size_t)mc * K + kc);
         }
     };
-    auto stash = [&](int buf) {
+    // decode + round to fp16 (registers only: free to overlap the matrix instructions)
+    auto convert = [&](auto slotc, v8h (&hw)[4]) {
+        constexpr int S = decltype(slotc)::value;
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                if (RFQ_KQ_SKIP & 16) hw[c][e] = (_Float16)(float)(raws[S].d[0] & 1023u);
+                else hw[c][e] = (_Float16)raws[S].value(8 * c + e); // round to nearest even
+            }
+    };
+    auto stash = [&](auto slotc, const v8h (&hw)[4], int buf) {
+        constexpr int S = decltype(slotc)::value;
         uint8_t *abase = lds + buf * STAGE_BYTES, *wbase = abase + A_BYTES;
+        if (RFQ_KQ_SKIP & 8) {
+            // keep the values alive without the writes (the test is never true for finite data)
+            float keep = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; i++) keep += __uint_as_float(ras[S][i].x ^ ras[S][i].y ^ ras[S][i].z ^ ras[S][i].w);
+#pragma unroll
+            for (int c = 0; c < 4; c++)
+#pragma unroll
+                for (int e = 0; e < 8; e++) keep += (float)hw[c][e];
+            if (keep == 1.2345e-30f) *reinterpret_cast<float *>(abase) = keep;
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < 8; i++)
-            *reinterpret_cast<uint4 *>(abase + (a_row0 + 32 * i) * LDR + a_chunk * 16) = ra[i];
+            *reinterpret_cast<uint4 *>(abase + (a_row0 + 32 * i) * LDR + a_chunk * 16) = ras[S][i];
 #pragma unroll
-        for (int c = 0; c < 4; c++) {
-            v8h h;
-#pragma unroll
-            for (int e = 0; e < 8; e++) h[e] = (_Float16)raw.value(8 * c + e); // round to nearest even
-            *reinterpret_cast<v8h *>(wbase + wr * LDR + wg * 64 + c * 16) = h;
-        }
+        for (int c = 0; c < 4; c++) *reinterpret_cast<v8h *>(wbase + wr * LDR + wg * 64 + c * 16) = hw[c];
     };
 
     v16f acc[2][4];
@@ -224,34 +281,68 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const _Float16 *__restrict__ a, co
             for (int r = 0; r < 16; r++) acc[j][i][r] = 0.0f;
 
     const int fr = lane & 31, fh = lane >> 5;                     // fragment row, k half
+    // Fragments of k-step ks+1 are read while the matrix instructions of k-step
+    // ks run (two register sets), so LDS latency is paid once per stage.
     auto compute = [&](int buf) {
         const uint8_t *abase = lds + buf * STAGE_BYTES, *wbase = abase + A_BYTES;
-#pragma unroll
-        for (int ks = 0; ks < BK / 16; ks++) {
-            v8h fw[2], fa[4];
+        v8h fw[2][2], fa[2][4];
+        auto load_frags = [&](int ks, int set) {
+            if (RFQ_KQ_SKIP & 4) return;
 #pragma unroll
             for (int j = 0; j < 2; j++)
-                fw[j] = *reinterpret_cast<const v8h *>(wbase + (wave_n * 64 + j * 32 + fr) * LDR + ks * 32 + fh * 16);
+                fw[set][j] = *reinterpret_cast<const v8h *>(wbase + (wave_n * 64 + j * 32 + fr) * LDR + ks * 32 + fh * 16);
 #pragma unroll
             for (int i = 0; i < 4; i++)
-                fa[i] = *reinterpret_cast<const v8h *>(abase + (wave_m * 128 + i * 32 + fr) * LDR + ks * 32 + fh * 16);
+                fa[set][i] = *reinterpret_cast<const v8h *>(abase + (wave_m * 128 + i * 32 + fr) * LDR + ks * 32 + fh * 16);
+        };
+        if (RFQ_KQ_SKIP & 4) {
+#pragma unroll
+            for (int set = 0; set < 2; set++) {
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+#pragma unroll
+                    for (int e = 0; e < 8; e++) fw[set][j][e] = (_Float16)(float)(lane + j + e);
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+#pragma unroll
+                    for (int e = 0; e < 8; e++) fa[set][i][e] = (_Float16)(float)(lane + i - e);
+            }
+        }
+        load_frags(0, 0);
+#pragma unroll
+        for (int ks = 0; ks < BK / 16; ks++) {
+            if (ks + 1 < BK / 16) load_frags(ks + 1, (ks + 1) & 1);
 #pragma unroll
             for (int j = 0; j < 2; j++)
 #pragma unroll
                 for (int i = 0; i < 4; i++)
-                    acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[j], fa[i], acc[j][i], 0, 0, 0);
+                    acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[ks & 1][j], fa[ks & 1][i], acc[j][i], 0, 0, 0);
         }
     };
 
-    fetch(0);
-    stash(0);
-    __syncthreads();
-    for (int st = 0; st < nstages; st++) {
-        const bool more = st + 1 < nstages;
-        if (more) fetch(st + 1);
+    // iteration st: stage st is in LDS; stage st+1 sits in register set NEXT
+    // (loaded two iterations ago); set FREE (stage st, already in LDS) takes stage st+3
+    auto iter = [&](auto nextc, auto freec, int st) {
+        v8h hw[4];
+        convert(nextc, hw);                    // (after the last stage this moves a stage nobody reads)
         compute(st & 1);
-        if (more) stash((st + 1) & 1);
-        __syncthreads();
+        stash(nextc, hw, (st + 1) & 1);
+        fetch(freec, st + 3);
+        lds_barrier();
+    };
+    {
+        v8h hw[4];
+        fetch(IC<0>{}, 0);
+        fetch(IC<1>{}, 1);
+        fetch(IC<2>{}, 2);
+        convert(IC<0>{}, hw);
+        stash(IC<0>{}, hw, 0);
+        lds_barrier();
+    }
+    for (int st = 0; st < nstages; st += 3) {
+        iter(IC<1>{}, IC<0>{}, st);
+        if (st + 1 < nstages) iter(IC<2>{}, IC<1>{}, st + 1);
+        if (st + 2 < nstages) iter(IC<0>{}, IC<2>{}, st + 2);
     }
 
     if (FMT == RFQ_Q4_K) {
@@ -261,6 +352,7 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const _Float16 *__restrict__ a, co
         // super-blocks; thread (wr, wg) expands the 16 mins of two of them.
         const int K2 = K / 16, nstages2 = (K2 + BK - 1) / BK;
         uint32_t mins[4];
+        uint4 (&ra)[8] = ras[0];
         auto fetch2 = [&](int st) {
 #pragma unroll
             for (int h = 0; h < 2; h++) {
@@ -298,13 +390,13 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const _Float16 *__restrict__ a, co
         };
         fetch2(0);
         stash2(0);
-        __syncthreads();
+        lds_barrier();
         for (int st = 0; st < nstages2; st++) {
             const bool more = st + 1 < nstages2;
             if (more) fetch2(st + 1);
             compute(st & 1);
             if (more) stash2((st + 1) & 1);
-            __syncthreads();
+            lds_barrier();
         }
     }
 
