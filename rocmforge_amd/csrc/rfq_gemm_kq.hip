@@ -18,11 +18,13 @@
 // pass over A into a stream-ordered temporary of M * K / 16 fp16 values.
 //
 // Workgroup tile 256 (m) x 128 (n), k advances 64 per stage, two LDS stages.
-// Thread t decodes the 32 weights (row t/2, k-group t%2) of a stage: exactly
-// one Q4_0/Q8_0 block or one Q4_K/Q6_K sub-block pair.  Four wavefronts in a
-// 2 (n) x 2 (m) arrangement, each 64 n x 128 m = 2 x 4 instruction tiles.  The
-// weight fragment is the instruction's first operand, so a lane ends up with
-// 4 consecutive n of one output row: 8- or 16-byte stores without a transpose.
+// 512 threads; thread t decodes 16 weights of a stage (row t/4, 32-element
+// group (t/2)%2, half t%2): half a Q4_0/Q8_0 block or half a Q4_K/Q6_K
+// sub-block.  Eight wavefronts in a 2 (n) x 4 (m) arrangement, two per SIMD
+// (one runs matrix instructions while the other decodes and moves data), each
+// 64 n x 64 m = 2 x 2 instruction tiles.  The weight fragment is the
+// instruction's first operand, so a lane ends up with 4 consecutive n of one
+// output row: 8- or 16-byte stores without a transpose.
 #include <mutex>
 
 #include "rfq_common.hpp"
@@ -39,6 +41,7 @@ namespace {
 
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
+typedef uint32_t v4u __attribute__((ext_vector_type(4))); // 16 bytes in flight (a builtin vector: plain loads and stores)
 template <int N> struct IC { static constexpr int value = N; };
 
 // Workgroup barrier for LDS hand-over that leaves global loads in flight
@@ -56,28 +59,23 @@ constexpr int BM = 256, BN = 128, BK = 64;
 constexpr int LDR = BK * 2 + 16;                 // bytes per LDS row: 64 fp16 + 16 pad (rows 36 dwords apart)
 constexpr int A_BYTES = BM * LDR, W_BYTES = BN * LDR, STAGE_BYTES = A_BYTES + W_BYTES;
 
-// ---- raw bytes of 32 consecutive weights of a row, and their f32 values -------
-template <int FMT> struct Raw32;
+// ---- raw bytes of 16 consecutive weights of a row (half `hf` of the 32-element
+// group g), and their f32 values.  Few wide loads: every lane touches a
+// different cache line, so the address path pays per instruction, not per byte.
+template <int FMT> struct Raw16;
 
 // src/kernels/quant/q4_0.rs:289-306: 20-byte block = f32 scale + 16 nibble bytes
-template <> struct Raw32<RFQ_Q4_0> {
-    static constexpr int ND = 5;
+template <> struct Raw16<RFQ_Q4_0> {
+    static constexpr int ND = 3;
     uint32_t d[ND];
-    __device__ __forceinline__ void load(const uint8_t *row, int g)
+    __device__ __forceinline__ void load(const uint8_t *row, int g, int hf)
     {
-        // few wide loads: every lane touches a different cache line, so the
-        // address path pays per instruction, not per byte
         const uint8_t *p = row + (size_t)g * 20;
         d[0] = ld<uint32_t>(p);
-        uint4 q = ld<uint4>(p + 4);
-        d[1] = q.x; d[2] = q.y; d[3] = q.z; d[4] = q.w;
+        uint2 q = ld<uint2>(p + 4 + 8 * hf);
+        d[1] = q.x; d[2] = q.y;
     }
-    __device__ __forceinline__ void zero()
-    {
-#pragma unroll
-        for (int i = 0; i < ND; i++) d[i] = 0;
-        d[1] = d[2] = d[3] = d[4] = 0x88888888u; // nibble 8 is 0.0
-    }
+    __device__ __forceinline__ void zero() { d[0] = 0; d[1] = d[2] = 0x88888888u; } // nibble 8 is 0.0
     __device__ __forceinline__ float value(int e) const
     {
         float scale = __uint_as_float(d[0]);
@@ -87,23 +85,17 @@ template <> struct Raw32<RFQ_Q4_0> {
 };
 
 // src/kernels/quant/q8_0.rs:55-59: 36-byte block = f32 scale + 32 offset-binary bytes
-template <> struct Raw32<RFQ_Q8_0> {
-    static constexpr int ND = 9;
+template <> struct Raw16<RFQ_Q8_0> {
+    static constexpr int ND = 5;
     uint32_t d[ND];
-    __device__ __forceinline__ void load(const uint8_t *row, int g)
+    __device__ __forceinline__ void load(const uint8_t *row, int g, int hf)
     {
         const uint8_t *p = row + (size_t)g * 36;
         d[0] = ld<uint32_t>(p);
-        uint4 q0 = ld<uint4>(p + 4), q1 = ld<uint4>(p + 20);
-        d[1] = q0.x; d[2] = q0.y; d[3] = q0.z; d[4] = q0.w;
-        d[5] = q1.x; d[6] = q1.y; d[7] = q1.z; d[8] = q1.w;
+        uint4 q = ld<uint4>(p + 4 + 16 * hf);
+        d[1] = q.x; d[2] = q.y; d[3] = q.z; d[4] = q.w;
     }
-    __device__ __forceinline__ void zero()
-    {
-        d[0] = 0;
-#pragma unroll
-        for (int i = 1; i < ND; i++) d[i] = 0x80808080u;
-    }
+    __device__ __forceinline__ void zero() { d[0] = 0; d[1] = d[2] = d[3] = d[4] = 0x80808080u; }
     __device__ __forceinline__ float value(int e) const
     {
         float scale = __uint_as_float(d[0]);
@@ -114,24 +106,18 @@ template <> struct Raw32<RFQ_Q8_0> {
 
 // src/kernels/quant/q4_k.rs:222-268: sub-block sb of a 256-byte super-block:
 // f16 scale at 2*sb, i8 min at 16+sb, 16 nibble bytes at 32+28*sb
-template <> struct Raw32<RFQ_Q4_K> {
-    static constexpr int ND = 5;
+template <> struct Raw16<RFQ_Q4_K> {
+    static constexpr int ND = 3;
     uint32_t d[ND];
-    __device__ __forceinline__ void load(const uint8_t *row, int g)
+    __device__ __forceinline__ void load(const uint8_t *row, int g, int hf)
     {
         const uint8_t *blk = row + (size_t)(g >> 3) * 256;
         const int sb = g & 7;
-        // the aligned dwords that hold scale sb and min sb, then the 16 nibble bytes
-        uint32_t sc = ld<uint32_t>(blk + 2 * (sb & ~1)), mn = ld<uint32_t>(blk + 16 + (sb & ~3));
-        d[0] = ((sc >> (16 * (sb & 1))) & 0xFFFFu) | (((mn >> (8 * (sb & 3))) & 0xFFu) << 16);
-        uint4 q = ld<uint4>(blk + 32 + 28 * sb);
-        d[1] = q.x; d[2] = q.y; d[3] = q.z; d[4] = q.w;
+        d[0] = ld<uint32_t>(blk + 2 * (sb & ~1)) >> (16 * (sb & 1)); // the aligned dword that holds scale sb
+        uint2 q = ld<uint2>(blk + 32 + 28 * sb + 8 * hf);
+        d[1] = q.x; d[2] = q.y;
     }
-    __device__ __forceinline__ void zero()
-    {
-#pragma unroll
-        for (int i = 0; i < ND; i++) d[i] = 0;
-    }
+    __device__ __forceinline__ void zero() { d[0] = d[1] = d[2] = 0; }
     // q * scale only (exact in f32): the min is contracted separately
     __device__ __forceinline__ float value(int e) const
     {
@@ -142,32 +128,27 @@ template <> struct Raw32<RFQ_Q4_K> {
 };
 
 // src/kernels/quant/q6_k.rs:221-261: element i of a 256-byte block: f16 scale
-// 2*(i/16), signed 6-bit field at bit 6*i of the stream at +32.  32 elements =
-// 2 scales (one dword) + 24 stream bytes.
-template <> struct Raw32<RFQ_Q6_K> {
-    static constexpr int ND = 7;
+// 2*(i/16), signed 6-bit field at bit 6*i of the stream at +32.  16 elements =
+// one scale + 12 stream bytes.
+template <> struct Raw16<RFQ_Q6_K> {
+    static constexpr int ND = 4;
     uint32_t d[ND];
-    __device__ __forceinline__ void load(const uint8_t *row, int g)
+    __device__ __forceinline__ void load(const uint8_t *row, int g, int hf)
     {
         const uint8_t *blk = row + (size_t)(g >> 3) * 256;
         const int s = g & 7;
-        d[0] = ld<uint32_t>(blk + 4 * s);
-        uint4 q = ld<uint4>(blk + 32 + 24 * s);
-        uint2 q2 = ld<uint2>(blk + 32 + 24 * s + 16);
-        d[1] = q.x; d[2] = q.y; d[3] = q.z; d[4] = q.w; d[5] = q2.x; d[6] = q2.y;
+        d[0] = ld<uint32_t>(blk + 4 * s) >> (16 * hf);
+        const uint8_t *p = blk + 32 + 24 * s + 12 * hf;
+        uint2 q = ld<uint2>(p);
+        d[1] = q.x; d[2] = q.y; d[3] = ld<uint32_t>(p + 8);
     }
-    __device__ __forceinline__ void zero()
-    {
-#pragma unroll
-        for (int i = 0; i < ND; i++) d[i] = 0;
-    }
+    __device__ __forceinline__ void zero() { d[0] = d[1] = d[2] = d[3] = 0; }
     __device__ __forceinline__ float value(int e) const
     {
-        float scale = f16_bits_to_f32((uint16_t)(e < 16 ? d[0] & 0xFFFFu : d[0] >> 16));
+        float scale = f16_bits_to_f32((uint16_t)(d[0] & 0xFFFFu));
         const int bit = 6 * e, w = bit >> 5, o = bit & 31;
-        uint64_t two = (uint64_t)d[1 + w] | ((uint64_t)d[1 + (w < 5 ? w + 1 : w)] << 32);
-        uint32_t f = (uint32_t)(two >> o);
-        return (float)sbfe6(f, 0) * scale;
+        uint64_t two = (uint64_t)d[1 + w] | ((uint64_t)d[1 + (w < 2 ? w + 1 : w)] << 32);
+        return (float)sbfe6((uint32_t)(two >> o), 0) * scale;
     }
 };
 
@@ -195,13 +176,13 @@ group_sums_kernel(const _Float16 *__restrict__ a, _Float16 *__restrict__ s2, int
 }
 
 template <int FMT, bool OUT_F16>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(512)
 gemm_kq_kernel(const uint8_t *__restrict__ w, const _Float16 *__restrict__ a, const _Float16 *__restrict__ s2,
                void *__restrict__ outp, int M, int N, int K)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wave_n = wave & 1, wave_m = wave >> 1;
+    const int wave_n = wave & 1, wave_m = wave >> 1;               // 2 x 4 wavefronts
     const int tiles_m = (M + BM - 1) / BM;
     const int tm = blockIdx.x % tiles_m, tn = blockIdx.x / tiles_m; // the m tiles of one W tile are neighbours
     const int m0 = tm * BM, n0 = tn * BN;
@@ -209,91 +190,105 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const _Float16 *__restrict__ a, co
     const size_t row_bytes = (size_t)(K / Fmt<FMT>::BE) * Fmt<FMT>::BB;
     const int nstages = (K + BK - 1) / BK;
 
-    // this thread's share of a stage: weights (row wr, group wg); 8 A chunks of 16 bytes
-    const int wr = tid >> 1, wg = tid & 1;
+    // this thread's share of a stage: 16 weights (row wr, group wg, half wh); 4 A chunks of 16 bytes
+    const int wr = tid >> 2, wg = (tid >> 1) & 1, wh = tid & 1;
     const bool w_row_ok = n0 + wr < N;
     const uint8_t *w_row = w + (size_t)(w_row_ok ? n0 + wr : 0) * row_bytes;
-    const int a_chunk = tid & 7, a_row0 = tid >> 3;               // rows a_row0 + 32*i
+    const int a_chunk = tid & 7, a_row0 = tid >> 3;               // rows a_row0 + 64*i
 
     // Global loads run three stages ahead of the arithmetic, through a ring of
     // three register sets (indices are compile-time: the loop is unrolled by 3).
-    Raw32<FMT> raws[3];
-    uint4 ras[3][8];
+    // (separate objects, not one array: nothing can then index the ring at run time)
+    Raw16<FMT> raw0, raw1, raw2;
+    v4u ra0[4], ra1[4], ra2[4];
+    auto raw_of = [&](auto slotc) -> Raw16<FMT> & {
+        constexpr int S = decltype(slotc)::value;
+        if constexpr (S == 0) return raw0;
+        else if constexpr (S == 1) return raw1;
+        else return raw2;
+    };
+    auto ra_of = [&](auto slotc) -> v4u (&)[4] {
+        constexpr int S = decltype(slotc)::value;
+        if constexpr (S == 0) return ra0;
+        else if constexpr (S == 1) return ra1;
+        else return ra2;
+    };
     // The loads are unconditional (clamped addresses): branches around them
     // would make the compiler wait for every outstanding load at each join.
     // Rows past M or N only feed outputs that are never stored; k past K is
     // cancelled by zero weights (selected after the load), whatever finite
     // activations the clamped address returns.
-    auto fetch = [&](auto slotc, int st) {
-        constexpr int S = decltype(slotc)::value;
+    auto fetch = [&](auto slotc, int st) __attribute__((always_inline)) {
+        Raw16<FMT> &raw = raw_of(slotc);
+        v4u (&ra)[4] = ra_of(slotc);
         const int g = st * 2 + wg;
-        if (!(RFQ_KQ_SKIP & 2)) raws[S].load(w_row, g < groups ? g : groups - 1);
-        Raw32<FMT> z;
+        if (!(RFQ_KQ_SKIP & 2)) raw.load(w_row, g < groups ? g : groups - 1, wh);
+        Raw16<FMT> z;
         z.zero();
 #pragma unroll
-        for (int i = 0; i < Raw32<FMT>::ND; i++) raws[S].d[i] = g < groups ? raws[S].d[i] : z.d[i];
+        for (int i = 0; i < Raw16<FMT>::ND; i++) raw.d[i] = g < groups ? raw.d[i] : z.d[i];
         const int k = st * BK + a_chunk * 8, kc = k < K ? k : K - 8;
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const int m = m0 + a_row0 + 32 * i, mc = m < M ? m : M - 1;
-            if (!(RFQ_KQ_SKIP & 1)) ras[S][i] = *reinterpret_cast<const uint4 *>(a + (size_t)mc * K + kc);
+        for (int i = 0; i < 4; i++) {
+            const int m = m0 + a_row0 + 64 * i, mc = m < M ? m : M - 1;
+            if (!(RFQ_KQ_SKIP & 1)) ra[i] = *reinterpret_cast<const v4u *>(a + (size_t)mc * K + kc);
         }
     };
     // decode + round to fp16 (registers only: free to overlap the matrix instructions)
-    auto convert = [&](auto slotc, v8h (&hw)[4]) {
-        constexpr int S = decltype(slotc)::value;
+    auto convert = [&](auto slotc, v8h (&hw)[2]) __attribute__((always_inline)) {
+        Raw16<FMT> &raw = raw_of(slotc);
 #pragma unroll
-        for (int c = 0; c < 4; c++)
+        for (int c = 0; c < 2; c++)
 #pragma unroll
             for (int e = 0; e < 8; e++) {
-                if (RFQ_KQ_SKIP & 16) hw[c][e] = (_Float16)(float)(raws[S].d[0] & 1023u);
-                else hw[c][e] = (_Float16)raws[S].value(8 * c + e); // round to nearest even
+                if (RFQ_KQ_SKIP & 16) hw[c][e] = (_Float16)(float)(raw.d[0] & 1023u);
+                else hw[c][e] = (_Float16)raw.value(8 * c + e); // round to nearest even
             }
     };
-    auto stash = [&](auto slotc, const v8h (&hw)[4], int buf) {
-        constexpr int S = decltype(slotc)::value;
+    auto stash = [&](auto slotc, const v8h (&hw)[2], int buf) __attribute__((always_inline)) {
+        v4u (&ra)[4] = ra_of(slotc);
         uint8_t *abase = lds + buf * STAGE_BYTES, *wbase = abase + A_BYTES;
         if (RFQ_KQ_SKIP & 8) {
             // keep the values alive without the writes (the test is never true for finite data)
             float keep = 0.0f;
 #pragma unroll
-            for (int i = 0; i < 8; i++) keep += __uint_as_float(ras[S][i].x ^ ras[S][i].y ^ ras[S][i].z ^ ras[S][i].w);
+            for (int i = 0; i < 4; i++) keep += __uint_as_float(ra[i][0] ^ ra[i][1] ^ ra[i][2] ^ ra[i][3]);
 #pragma unroll
-            for (int c = 0; c < 4; c++)
+            for (int c = 0; c < 2; c++)
 #pragma unroll
                 for (int e = 0; e < 8; e++) keep += (float)hw[c][e];
             if (keep == 1.2345e-30f) *reinterpret_cast<float *>(abase) = keep;
             return;
         }
 #pragma unroll
-        for (int i = 0; i < 8; i++)
-            *reinterpret_cast<uint4 *>(abase + (a_row0 + 32 * i) * LDR + a_chunk * 16) = ras[S][i];
+        for (int i = 0; i < 4; i++)
+            *reinterpret_cast<v4u *>(abase + (a_row0 + 64 * i) * LDR + a_chunk * 16) = ra[i];
 #pragma unroll
-        for (int c = 0; c < 4; c++) *reinterpret_cast<v8h *>(wbase + wr * LDR + wg * 64 + c * 16) = hw[c];
+        for (int c = 0; c < 2; c++) *reinterpret_cast<v8h *>(wbase + wr * LDR + wg * 64 + wh * 32 + c * 16) = hw[c];
     };
 
-    v16f acc[2][4];
+    v16f acc[2][2];
 #pragma unroll
     for (int j = 0; j < 2; j++)
 #pragma unroll
-        for (int i = 0; i < 4; i++)
+        for (int i = 0; i < 2; i++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[j][i][r] = 0.0f;
 
     const int fr = lane & 31, fh = lane >> 5;                     // fragment row, k half
     // Fragments of k-step ks+1 are read while the matrix instructions of k-step
     // ks run (two register sets), so LDS latency is paid once per stage.
-    auto compute = [&](int buf) {
+    auto compute = [&](int buf) __attribute__((always_inline)) {
         const uint8_t *abase = lds + buf * STAGE_BYTES, *wbase = abase + A_BYTES;
-        v8h fw[2][2], fa[2][4];
-        auto load_frags = [&](int ks, int set) {
+        v8h fw[2][2], fa[2][2];
+        auto load_frags = [&](int ks, int set) __attribute__((always_inline)) {
             if (RFQ_KQ_SKIP & 4) return;
 #pragma unroll
             for (int j = 0; j < 2; j++)
                 fw[set][j] = *reinterpret_cast<const v8h *>(wbase + (wave_n * 64 + j * 32 + fr) * LDR + ks * 32 + fh * 16);
 #pragma unroll
-            for (int i = 0; i < 4; i++)
-                fa[set][i] = *reinterpret_cast<const v8h *>(abase + (wave_m * 128 + i * 32 + fr) * LDR + ks * 32 + fh * 16);
+            for (int i = 0; i < 2; i++)
+                fa[set][i] = *reinterpret_cast<const v8h *>(abase + (wave_m * 64 + i * 32 + fr) * LDR + ks * 32 + fh * 16);
         };
         if (RFQ_KQ_SKIP & 4) {
 #pragma unroll
@@ -303,7 +298,7 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const _Float16 *__restrict__ a, co
 #pragma unroll
                     for (int e = 0; e < 8; e++) fw[set][j][e] = (_Float16)(float)(lane + j + e);
 #pragma unroll
-                for (int i = 0; i < 4; i++)
+                for (int i = 0; i < 2; i++)
 #pragma unroll
                     for (int e = 0; e < 8; e++) fa[set][i][e] = (_Float16)(float)(lane + i - e);
             }
@@ -315,15 +310,15 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const _Float16 *__restrict__ a, co
 #pragma unroll
             for (int j = 0; j < 2; j++)
 #pragma unroll
-                for (int i = 0; i < 4; i++)
+                for (int i = 0; i < 2; i++)
                     acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[ks & 1][j], fa[ks & 1][i], acc[j][i], 0, 0, 0);
         }
     };
 
     // iteration st: stage st is in LDS; stage st+1 sits in register set NEXT
     // (loaded two iterations ago); set FREE (stage st, already in LDS) takes stage st+3
-    auto iter = [&](auto nextc, auto freec, int st) {
-        v8h hw[4];
+    auto iter = [&](auto nextc, auto freec, int st) __attribute__((always_inline)) {
+        v8h hw[2];
         convert(nextc, hw);                    // (after the last stage this moves a stage nobody reads)
         compute(st & 1);
         stash(nextc, hw, (st + 1) & 1);
@@ -331,7 +326,7 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const _Float16 *__restrict__ a, co
         lds_barrier();
     };
     {
-        v8h hw[4];
+        v8h hw[2];
         fetch(IC<0>{}, 0);
         fetch(IC<1>{}, 1);
         fetch(IC<2>{}, 2);
@@ -339,45 +334,45 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const _Float16 *__restrict__ a, co
         stash(IC<0>{}, hw, 0);
         lds_barrier();
     }
+    // Whole trips through the ring only (no branch between the three bodies:
+    // the compiler would merge their tails and index the ring at run time);
+    // stages past the end multiply zero weights.
     for (int st = 0; st < nstages; st += 3) {
         iter(IC<1>{}, IC<0>{}, st);
-        if (st + 1 < nstages) iter(IC<2>{}, IC<1>{}, st + 1);
-        if (st + 2 < nstages) iter(IC<0>{}, IC<2>{}, st + 2);
+        iter(IC<2>{}, IC<1>{}, st + 1);
+        iter(IC<0>{}, IC<2>{}, st + 2);
     }
 
-    if (FMT == RFQ_Q4_K) {
+    if constexpr (FMT == RFQ_Q4_K) {
         // The min term: "k" runs over (sub-block, hi/lo) pairs, K2 = K / 16 of
         // them; weight (n, 2*sb + t) = min[n, sb], activation (m, 2*sb + t) =
         // hi or lo of S[m, sb].  A stage of 64 covers 32 sub-blocks = 4
-        // super-blocks; thread (wr, wg) expands the 16 mins of two of them.
+        // super-blocks; thread (wr, wg, wh) expands the 8 mins of one of them.
         const int K2 = K / 16, nstages2 = (K2 + BK - 1) / BK;
-        uint32_t mins[4];
-        uint4 (&ra)[8] = ras[0];
+        uint32_t mins[2];
+        v4u (&ra)[4] = ra0;
         auto fetch2 = [&](int st) {
-#pragma unroll
-            for (int h = 0; h < 2; h++) {
-                const int sblk = st * 4 + wg * 2 + h;             // super-block of this row
-                if (w_row_ok && sblk < K / 256) {
-                    mins[2 * h] = ld<uint32_t>(w_row + (size_t)sblk * 256 + 16);
-                    mins[2 * h + 1] = ld<uint32_t>(w_row + (size_t)sblk * 256 + 20);
-                } else {
-                    mins[2 * h] = mins[2 * h + 1] = 0;
-                }
+            const int sblk = st * 4 + wg * 2 + wh;                // super-block of this row
+            if (w_row_ok && sblk < K / 256) {
+                mins[0] = ld<uint32_t>(w_row + (size_t)sblk * 256 + 16);
+                mins[1] = ld<uint32_t>(w_row + (size_t)sblk * 256 + 20);
+            } else {
+                mins[0] = mins[1] = 0;
             }
 #pragma unroll
-            for (int i = 0; i < 8; i++) {
-                const int m = m0 + a_row0 + 32 * i, k2 = st * BK + a_chunk * 8;
-                if (m < M && k2 < K2) ra[i] = *reinterpret_cast<const uint4 *>(s2 + (size_t)m * K2 + k2);
-                else ra[i] = make_uint4(0, 0, 0, 0);
+            for (int i = 0; i < 4; i++) {
+                const int m = m0 + a_row0 + 64 * i, k2 = st * BK + a_chunk * 8;
+                if (m < M && k2 < K2) ra[i] = *reinterpret_cast<const v4u *>(s2 + (size_t)m * K2 + k2);
+                else ra[i] = v4u{0, 0, 0, 0};
             }
         };
         auto stash2 = [&](int buf) {
             uint8_t *abase = lds + buf * STAGE_BYTES, *wbase = abase + A_BYTES;
 #pragma unroll
-            for (int i = 0; i < 8; i++)
-                *reinterpret_cast<uint4 *>(abase + (a_row0 + 32 * i) * LDR + a_chunk * 16) = ra[i];
+            for (int i = 0; i < 4; i++)
+                *reinterpret_cast<v4u *>(abase + (a_row0 + 64 * i) * LDR + a_chunk * 16) = ra[i];
 #pragma unroll
-            for (int c = 0; c < 4; c++) {                          // 4 mins -> 8 fp16 (each twice)
+            for (int c = 0; c < 2; c++) {                          // 4 mins -> 8 fp16 (each twice)
                 v8h h;
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
@@ -385,7 +380,7 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const _Float16 *__restrict__ a, co
                     h[2 * e] = v;
                     h[2 * e + 1] = v;
                 }
-                *reinterpret_cast<v8h *>(wbase + wr * LDR + wg * 64 + c * 16) = h;
+                *reinterpret_cast<v8h *>(wbase + wr * LDR + wg * 64 + wh * 32 + c * 16) = h;
             }
         };
         fetch2(0);
@@ -406,8 +401,8 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const _Float16 *__restrict__ a, co
 #pragma unroll
     for (int j = 0; j < 2; j++)
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int m = m0 + wave_m * 128 + i * 32 + fr;
+        for (int i = 0; i < 2; i++) {
+            const int m = m0 + wave_m * 64 + i * 32 + fr;
             if (m >= M) continue;
 #pragma unroll
             for (int g = 0; g < 4; g++) {
@@ -456,7 +451,7 @@ int launch_cfg(const uint8_t *w, const void *a, void *out, int m, int n, int k, 
         hipLaunchKernelGGL(group_sums_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s,
                            reinterpret_cast<const _Float16 *>(a), s2, m, k);
     }
-    hipLaunchKernelGGL((gemm_kq_kernel<FMT, OUT_F16>), dim3(tiles), dim3(256), LDS, s, w,
+    hipLaunchKernelGGL((gemm_kq_kernel<FMT, OUT_F16>), dim3(tiles), dim3(512), LDS, s, w,
                        reinterpret_cast<const _Float16 *>(a), s2, out, m, n, k);
     hipError_t launch_err = hipGetLastError();
     if (s2) {
