@@ -196,22 +196,24 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const _Float16 *__restrict__ a, co
     const uint8_t *w_row = w + (size_t)(w_row_ok ? n0 + wr : 0) * row_bytes;
     const int a_chunk = tid & 7, a_row0 = tid >> 3;               // rows a_row0 + 64*i
 
-    // Global loads run three stages ahead of the arithmetic, through a ring of
-    // three register sets (indices are compile-time: the loop is unrolled by 3).
+    // Global loads run four stages ahead of the arithmetic, through a ring of
+    // four register sets (indices are compile-time: the loop is unrolled by 4).
     // (separate objects, not one array: nothing can then index the ring at run time)
-    Raw16<FMT> raw0, raw1, raw2;
-    v4u ra0[4], ra1[4], ra2[4];
+    Raw16<FMT> raw0, raw1, raw2, raw3;
+    v4u ra0[4], ra1[4], ra2[4], ra3[4];
     auto raw_of = [&](auto slotc) -> Raw16<FMT> & {
         constexpr int S = decltype(slotc)::value;
         if constexpr (S == 0) return raw0;
         else if constexpr (S == 1) return raw1;
-        else return raw2;
+        else if constexpr (S == 2) return raw2;
+        else return raw3;
     };
     auto ra_of = [&](auto slotc) -> v4u (&)[4] {
         constexpr int S = decltype(slotc)::value;
         if constexpr (S == 0) return ra0;
         else if constexpr (S == 1) return ra1;
-        else return ra2;
+        else if constexpr (S == 2) return ra2;
+        else return ra3;
     };
     // The loads are unconditional (clamped addresses): branches around them
     // would make the compiler wait for every outstanding load at each join.
@@ -316,13 +318,13 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const _Float16 *__restrict__ a, co
     };
 
     // iteration st: stage st is in LDS; stage st+1 sits in register set NEXT
-    // (loaded two iterations ago); set FREE (stage st, already in LDS) takes stage st+3
+    // (loaded three iterations ago); set FREE (stage st, already in LDS) takes stage st+4
     auto iter = [&](auto nextc, auto freec, int st) __attribute__((always_inline)) {
         v8h hw[2];
         convert(nextc, hw);                    // (after the last stage this moves a stage nobody reads)
         compute(st & 1);
         stash(nextc, hw, (st + 1) & 1);
-        fetch(freec, st + 3);
+        fetch(freec, st + 4);
         lds_barrier();
     };
     {
@@ -330,6 +332,7 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const _Float16 *__restrict__ a, co
         fetch(IC<0>{}, 0);
         fetch(IC<1>{}, 1);
         fetch(IC<2>{}, 2);
+        fetch(IC<3>{}, 3);
         convert(IC<0>{}, hw);
         stash(IC<0>{}, hw, 0);
         lds_barrier();
@@ -337,10 +340,11 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const _Float16 *__restrict__ a, co
     // Whole trips through the ring only (no branch between the three bodies:
     // the compiler would merge their tails and index the ring at run time);
     // stages past the end multiply zero weights.
-    for (int st = 0; st < nstages; st += 3) {
+    for (int st = 0; st < nstages; st += 4) {
         iter(IC<1>{}, IC<0>{}, st);
         iter(IC<2>{}, IC<1>{}, st + 1);
-        iter(IC<0>{}, IC<2>{}, st + 2);
+        iter(IC<3>{}, IC<2>{}, st + 2);
+        iter(IC<0>{}, IC<3>{}, st + 3);
     }
 
     if constexpr (FMT == RFQ_Q4_K) {
