@@ -1,0 +1,446 @@
+/*
+ * rocmforge_rfq.hpp -- C++17 host-side mirror of the ROCmForge operator surface
+ * for the quantized-weight path, on top of the C ABI in rfq.h.
+ *
+ * ROCmForge's host code is Rust; this header restates, name for name, the
+ * types and functions its benches and tests use on this path, so that C++
+ * callers (and the host tests in tests/host/) read like the reference's own:
+ *
+ *   GgufTensorType        src/loader/tensor_type.rs:16-112
+ *   TensorShape           src/loader/mmap_loader.rs:117-174
+ *   GgufTensor            src/loader/gguf_tensor.rs:8-75
+ *   loader::dequant_*     src/loader/mod.rs:116-127, src/loader/dequant.rs:41-132
+ *   loader::dequantize    src/loader/dequant.rs:673-700
+ *   HipBuffer             src/backend/hip_backend/memory.rs:19-31, 540-580
+ *   HipBackend            src/backend/hip_backend/backend.rs:104-200
+ *   matmul_q4_0 / q8_0 / q4_k / q6_k
+ *                         src/kernels/matmul/quantized/q4_0.rs:153, q8_0.rs:69, q4_k.rs:173, q6_k.rs:163
+ *   matmul_q4_0_gpu       src/kernels/matmul/quantized/q4_0.rs:209-260
+ *   dequantize_q4_0_kernel_cached, dequantize_q4_k_gpu_kernel, dequantize_q6_k_gpu_kernel
+ *                         src/kernels/quant/q4_0.rs:107, q4_k.rs:99, q6_k.rs:102
+ *   QuantFormat, QuantizedMatmulOp
+ *                         src/ggml/hip_backend/ops/batch_quantized.rs:20-90
+ *   validate_matmul_q4_0 / q8_0 (the checks of execute_matmul_q4_0 / q8_0)
+ *                         src/ggml/hip_backend/op_dispatch.rs:951-1083
+ *
+ * Rust's Result<T, E> becomes Result<T> below (ok / value / error text); no
+ * exceptions cross the C ABI.  Everything computes on the GPU through librfq:
+ * there is no CPU fallback here.
+ */
+#ifndef ROCMFORGE_RFQ_HPP
+#define ROCMFORGE_RFQ_HPP
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstdint>
+#include <cstring>
+#include <limits>
+#include <memory>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "rfq.h"
+
+namespace rocmforge {
+
+// ---- Result -----------------------------------------------------------------
+template <typename T> struct Result {
+    bool ok = false;
+    T value{};
+    std::string error;
+    static Result Ok(T v) { Result r; r.ok = true; r.value = std::move(v); return r; }
+    static Result Err(std::string e) { Result r; r.error = std::move(e); return r; }
+    explicit operator bool() const { return ok; }
+};
+struct Unit {};
+using Status = Result<Unit>;
+inline Status ok_status() { return Status::Ok(Unit{}); }
+
+namespace detail {
+inline Status from_rfq(int rc, const char *what)
+{
+    if (rc == RFQ_OK) return ok_status();
+    return Status::Err(std::string(what) + ": " + rfq_last_error());
+}
+inline size_t checked_mul(size_t a, size_t b)
+{
+    if (a != 0 && b > std::numeric_limits<size_t>::max() / a) return std::numeric_limits<size_t>::max();
+    return a * b;
+}
+inline size_t div_ceil(size_t a, size_t b) { return (a + b - 1) / b; }
+} // namespace detail
+
+// ---- GgufTensorType (src/loader/tensor_type.rs:16-112) -------------------------
+enum class GgufTensorType : uint32_t {
+    F32 = 0, F16 = 1, Q4_0 = 2, Q8_0 = 8, Q2_K = 10, Q3_K = 11, Q4_K = 12, Q5_K = 13, Q6_K = 14,
+    Mxfp4 = 20, Mxfp6E2m3 = 21, Mxfp6E3m2 = 22
+};
+
+inline Result<GgufTensorType> tensor_type_from_u32(uint32_t v)
+{
+    switch (v) {
+    case 0: case 1: case 2: case 8: case 10: case 11: case 12: case 13: case 14: case 20: case 21: case 22:
+        return Result<GgufTensorType>::Ok(static_cast<GgufTensorType>(v));
+    default: // ids 3, 6, 7 (Q4_1, Q5_0, Q5_1) and everything unknown are rejected
+        return Result<GgufTensorType>::Err("Unknown tensor type: " + std::to_string(v));
+    }
+}
+inline const char *to_string(GgufTensorType t)
+{
+    switch (t) {
+    case GgufTensorType::F32: return "FP32";
+    case GgufTensorType::F16: return "FP16";
+    case GgufTensorType::Q4_0: return "Q4_0";
+    case GgufTensorType::Q8_0: return "Q8_0";
+    case GgufTensorType::Q2_K: return "Q2_K";
+    case GgufTensorType::Q3_K: return "Q3_K";
+    case GgufTensorType::Q4_K: return "Q4_K";
+    case GgufTensorType::Q5_K: return "Q5_K";
+    case GgufTensorType::Q6_K: return "Q6_K";
+    case GgufTensorType::Mxfp4: return "MXFP4";
+    case GgufTensorType::Mxfp6E2m3: return "MXFP6_E2M3";
+    case GgufTensorType::Mxfp6E3m2: return "MXFP6_E3M2";
+    }
+    return "?";
+}
+// elements per block (1 for the plain float types)
+inline size_t block_size(GgufTensorType t)
+{
+    switch (t) {
+    case GgufTensorType::F32: case GgufTensorType::F16: return 1;
+    case GgufTensorType::Q4_0: case GgufTensorType::Q8_0: case GgufTensorType::Mxfp4:
+    case GgufTensorType::Mxfp6E2m3: case GgufTensorType::Mxfp6E3m2: return 32;
+    default: return 256;
+    }
+}
+inline bool is_quantized(GgufTensorType t) { return t != GgufTensorType::F32 && t != GgufTensorType::F16; }
+// bytes for the float types, the block size (in elements) for block formats -- as the reference defines it
+inline size_t element_size(GgufTensorType t)
+{
+    if (t == GgufTensorType::F32) return 4;
+    if (t == GgufTensorType::F16) return 2;
+    return block_size(t);
+}
+
+// ---- TensorShape (src/loader/mmap_loader.rs:117-174) ---------------------------
+class TensorShape {
+public:
+    static TensorShape from_dims(const std::vector<size_t> &dims)
+    {
+        TensorShape s;
+        s.dims_ = dims;
+        s.strides_.assign(dims.size(), 1);
+        for (size_t i = dims.size(); i-- > 0;)
+            if (i + 1 < dims.size()) s.strides_[i] = detail::checked_mul(s.strides_[i + 1], dims[i + 1]);
+        return s;
+    }
+    const std::vector<size_t> &dims() const { return dims_; }
+    const std::vector<size_t> &strides() const { return strides_; }
+    size_t total_elements() const
+    {
+        size_t n = 1;
+        for (size_t d : dims_) n = detail::checked_mul(n, d);
+        return n;
+    }
+
+private:
+    std::vector<size_t> dims_, strides_;
+};
+
+// ---- GgufTensor (src/loader/gguf_tensor.rs:8-75) ---------------------------------
+struct GgufTensor {
+    std::string name;
+    TensorShape shape;
+    GgufTensorType tensor_type = GgufTensorType::F32;
+    std::string quant_type;
+    uint64_t offset = 0;
+    std::vector<uint8_t> data;
+
+    GgufTensor() = default;
+    GgufTensor(std::string n, TensorShape s, GgufTensorType t, uint64_t off)
+        : name(std::move(n)), shape(std::move(s)), tensor_type(t), quant_type(to_string(t)), offset(off)
+    {
+    }
+    size_t total_elements() const { return shape.total_elements(); }
+    // Bytes the loader expects.  Q4_0 is counted as 4 + 32 per block here although the
+    // decoder strides by 20 (src/loader/gguf_tensor.rs:45-49): kept as the reference has it.
+    size_t data_size() const
+    {
+        const size_t n = total_elements();
+        switch (tensor_type) {
+        case GgufTensorType::F32: return detail::checked_mul(n, 4);
+        case GgufTensorType::F16: return detail::checked_mul(n, 2);
+        case GgufTensorType::Q4_0: case GgufTensorType::Q8_0: return detail::checked_mul(detail::div_ceil(n, 32), 36);
+        case GgufTensorType::Mxfp4: return detail::checked_mul(detail::div_ceil(n, 32), 17);
+        case GgufTensorType::Mxfp6E2m3: case GgufTensorType::Mxfp6E3m2:
+            return detail::checked_mul(detail::div_ceil(n, 32), 25);
+        default: return detail::checked_mul(detail::div_ceil(n, 256), 256);
+        }
+    }
+};
+
+// ---- loader ---------------------------------------------------------------------
+namespace loader {
+
+namespace detail_ {
+inline std::vector<float> through_gpu(int fmt, const uint8_t *data, size_t len, size_t n_elements)
+{
+    // the reference returns n_elements values, zero where the input was too short
+    std::vector<float> out(n_elements, 0.0f);
+    if (n_elements == 0) return out;
+    static const uint8_t none = 0;
+    int rc = rfq_dequant_host(fmt, len ? data : &none, len, out.data(), n_elements);
+    if (rc != RFQ_OK) out.assign(n_elements, std::numeric_limits<float>::quiet_NaN()); // loud, not silent
+    return out;
+}
+} // namespace detail_
+
+inline std::vector<float> dequant_q4_0(const std::vector<uint8_t> &data, size_t n_elements)
+{
+    return detail_::through_gpu(RFQ_Q4_0, data.data(), data.size(), n_elements);
+}
+inline std::vector<float> dequant_q8_0(const std::vector<uint8_t> &data, size_t n_elements)
+{
+    return detail_::through_gpu(RFQ_Q8_0, data.data(), data.size(), n_elements);
+}
+inline std::vector<float> dequant_q4_k(const std::vector<uint8_t> &data, size_t n_elements)
+{
+    return detail_::through_gpu(RFQ_Q4_K, data.data(), data.size(), n_elements);
+}
+inline std::vector<float> dequant_q6_k(const std::vector<uint8_t> &data, size_t n_elements)
+{
+    return detail_::through_gpu(RFQ_Q6_K, data.data(), data.size(), n_elements);
+}
+inline Result<std::vector<float>> dequant_mxfp4(const GgufTensor &t)
+{
+    return Result<std::vector<float>>::Ok(detail_::through_gpu(RFQ_MXFP4, t.data.data(), t.data.size(), t.total_elements()));
+}
+inline Result<std::vector<float>> dequant_mxfp6(const GgufTensor &t)
+{
+    return Result<std::vector<float>>::Ok(
+        detail_::through_gpu(RFQ_MXFP6_E2M3, t.data.data(), t.data.size(), t.total_elements()));
+}
+
+// src/loader/dequant.rs:673-700.  F32 / F16 are plain host conversions
+// (chunks_exact: a trailing partial element is dropped).
+inline Result<std::vector<float>> dequantize(const GgufTensor &t)
+{
+    using R = Result<std::vector<float>>;
+    switch (t.tensor_type) {
+    case GgufTensorType::F32: {
+        std::vector<float> out(t.data.size() / 4);
+        std::memcpy(out.data(), t.data.data(), out.size() * 4);
+        return R::Ok(std::move(out));
+    }
+    case GgufTensorType::F16: {
+        std::vector<float> out(t.data.size() / 2);
+        for (size_t i = 0; i < out.size(); i++) {
+            uint16_t h;
+            std::memcpy(&h, t.data.data() + 2 * i, 2);
+            uint32_t sign = (uint32_t)(h & 0x8000u) << 16, e = (h >> 10) & 31u, m = h & 1023u, bits;
+            if (e == 0) {
+                if (m == 0) bits = sign;
+                else { // subnormal: normalise
+                    int sh = 0;
+                    while (!(m & 1024u)) { m <<= 1; sh++; }
+                    bits = sign | ((uint32_t)(113 - sh) << 23) | ((m & 1023u) << 13);
+                }
+            } else if (e == 31) bits = sign | 0x7F800000u | (m << 13);
+            else bits = sign | ((e + 112u) << 23) | (m << 13);
+            std::memcpy(&out[i], &bits, 4);
+        }
+        return R::Ok(std::move(out));
+    }
+    case GgufTensorType::Q4_0: return R::Ok(dequant_q4_0(t.data, t.total_elements()));
+    case GgufTensorType::Q8_0: return R::Ok(dequant_q8_0(t.data, t.total_elements()));
+    case GgufTensorType::Q4_K: return R::Ok(dequant_q4_k(t.data, t.total_elements()));
+    case GgufTensorType::Q6_K: return R::Ok(dequant_q6_k(t.data, t.total_elements()));
+    case GgufTensorType::Mxfp4: return dequant_mxfp4(t);
+    case GgufTensorType::Mxfp6E2m3: case GgufTensorType::Mxfp6E3m2: return dequant_mxfp6(t);
+    default: return R::Err(std::string("dequantize: ") + to_string(t.tensor_type) + " is outside this library's path");
+    }
+}
+
+} // namespace loader
+
+// ---- HipBuffer / HipBackend -------------------------------------------------------
+class HipBuffer {
+public:
+    static Result<HipBuffer> create(size_t size)
+    {
+        void *p = nullptr;
+        hipError_t e = hipMalloc(&p, size ? size : 1);
+        if (e != hipSuccess) return Result<HipBuffer>::Err(std::string("hipMalloc failed: ") + hipGetErrorString(e));
+        HipBuffer b;
+        b.inner_ = std::shared_ptr<void>(p, [](void *q) { (void)hipFree(q); }); // freed on the last drop
+        b.size_ = size;
+        return Result<HipBuffer>::Ok(std::move(b));
+    }
+    size_t size() const { return size_; }
+    void *as_ptr() const { return inner_.get(); }
+    template <typename T> Status copy_from_host(const std::vector<T> &src)
+    {
+        if (src.size() * sizeof(T) > size_) return Status::Err("copy_from_host: source larger than the buffer");
+        hipError_t e = hipMemcpy(as_ptr(), src.data(), src.size() * sizeof(T), hipMemcpyHostToDevice);
+        return e == hipSuccess ? ok_status() : Status::Err(std::string("hipMemcpy H2D failed: ") + hipGetErrorString(e));
+    }
+    template <typename T> Status copy_to_host(std::vector<T> &dst) const
+    {
+        if (dst.size() * sizeof(T) > size_) return Status::Err("copy_to_host: destination larger than the buffer");
+        hipError_t e = hipMemcpy(dst.data(), as_ptr(), dst.size() * sizeof(T), hipMemcpyDeviceToHost);
+        return e == hipSuccess ? ok_status() : Status::Err(std::string("hipMemcpy D2H failed: ") + hipGetErrorString(e));
+    }
+
+private:
+    std::shared_ptr<void> inner_;
+    size_t size_ = 0;
+};
+
+// One stream, as the reference's process-wide backend has (the default stream here).
+class HipBackend {
+public:
+    static Result<HipBackend> create()
+    {
+        int n = 0;
+        if (hipGetDeviceCount(&n) != hipSuccess || n == 0) return Result<HipBackend>::Err("no HIP device");
+        return Result<HipBackend>::Ok(HipBackend{});
+    }
+    void *stream() const { return nullptr; }
+    Status synchronize() const
+    {
+        hipError_t e = hipStreamSynchronize(nullptr);
+        return e == hipSuccess ? ok_status() : Status::Err(std::string("synchronize failed: ") + hipGetErrorString(e));
+    }
+};
+
+// ---- dequantisation to device buffers (src/kernels/quant/q4_0.rs:107 and twins) ------
+inline Status dequantize_q4_0_kernel_cached(const HipBackend &b, const std::vector<uint8_t> &q, const HipBuffer &out,
+                                            size_t num_elements)
+{
+    if (out.size() < num_elements * sizeof(float)) return Status::Err("output buffer too small");
+    return detail::from_rfq(rfq_dequant_upload(RFQ_Q4_0, q.data(), q.size(), (float *)out.as_ptr(), num_elements, b.stream()),
+                            "dequantize_q4_0_kernel_cached");
+}
+inline Status dequantize_q4_k_gpu_kernel(const HipBackend &b, const std::vector<uint8_t> &q, const HipBuffer &out,
+                                         size_t num_elements)
+{
+    if (out.size() < num_elements * sizeof(float)) return Status::Err("output buffer too small");
+    return detail::from_rfq(rfq_dequant_upload(RFQ_Q4_K, q.data(), q.size(), (float *)out.as_ptr(), num_elements, b.stream()),
+                            "dequantize_q4_k_gpu_kernel");
+}
+inline Status dequantize_q6_k_gpu_kernel(const HipBackend &b, const std::vector<uint8_t> &q, const HipBuffer &out,
+                                         size_t num_elements)
+{
+    if (out.size() < num_elements * sizeof(float)) return Status::Err("output buffer too small");
+    return detail::from_rfq(rfq_dequant_upload(RFQ_Q6_K, q.data(), q.size(), (float *)out.as_ptr(), num_elements, b.stream()),
+                            "dequantize_q6_k_gpu_kernel");
+}
+
+// ---- quantized matmul (src/kernels/matmul/quantized/*.rs) ---------------------------
+// Host weights, device input [1 x n_cols] and output [1 x n_rows]; synchronous like the reference.
+inline Status matmul_host(int fmt, const char *who, const HipBackend &b, const std::vector<uint8_t> &w,
+                          const HipBuffer &input, size_t n_rows, size_t n_cols, const HipBuffer &output)
+{
+    if (input.size() < n_cols * sizeof(float)) return Status::Err(std::string(who) + ": input buffer too small");
+    if (output.size() < n_rows * sizeof(float)) return Status::Err(std::string(who) + ": output buffer too small");
+    return detail::from_rfq(rfq_matmul_host_weights(fmt, w.data(), w.size(), (const float *)input.as_ptr(), n_rows, n_cols,
+                                                    (float *)output.as_ptr(), b.stream()),
+                            who);
+}
+inline Status matmul_q4_0(const HipBackend &b, const std::vector<uint8_t> &w, const HipBuffer &in, size_t n_rows,
+                          size_t n_cols, const HipBuffer &out)
+{
+    return matmul_host(RFQ_Q4_0, "matmul_q4_0", b, w, in, n_rows, n_cols, out);
+}
+inline Status matmul_q8_0(const HipBackend &b, const std::vector<uint8_t> &w, const HipBuffer &in, size_t n_rows,
+                          size_t n_cols, const HipBuffer &out)
+{
+    return matmul_host(RFQ_Q8_0, "matmul_q8_0", b, w, in, n_rows, n_cols, out);
+}
+inline Status matmul_q4_k(const HipBackend &b, const std::vector<uint8_t> &w, const HipBuffer &in, size_t n_rows,
+                          size_t n_cols, const HipBuffer &out)
+{
+    return matmul_host(RFQ_Q4_K, "matmul_q4_k", b, w, in, n_rows, n_cols, out);
+}
+inline Status matmul_q6_k(const HipBackend &b, const std::vector<uint8_t> &w, const HipBuffer &in, size_t n_rows,
+                          size_t n_cols, const HipBuffer &out)
+{
+    return matmul_host(RFQ_Q6_K, "matmul_q6_k", b, w, in, n_rows, n_cols, out);
+}
+// raw device pointers, argument order (activations, weights, output, m, n, k)
+inline Status matmul_q4_0_gpu(const HipBackend &b, const float *act, const uint8_t *w, float *out, size_t m, size_t n,
+                              size_t k)
+{
+    return detail::from_rfq(rfq_matmul_q4_0(act, w, out, (int)m, (int)n, (int)k, b.stream()), "matmul_q4_0_gpu");
+}
+
+// ---- batch description types (src/ggml/hip_backend/ops/batch_quantized.rs:20-90) --------
+enum class QuantFormat { Q4_0, Q4_K, Q6_K, Q8_0 };
+inline float bytes_per_element(QuantFormat f)
+{
+    switch (f) {
+    case QuantFormat::Q4_0: return 20.0f / 32.0f;
+    case QuantFormat::Q8_0: return 36.0f / 32.0f;
+    default: return 1.0f;
+    }
+}
+inline const char *name(QuantFormat f)
+{
+    switch (f) {
+    case QuantFormat::Q4_0: return "Q4_0";
+    case QuantFormat::Q4_K: return "Q4_K";
+    case QuantFormat::Q6_K: return "Q6_K";
+    default: return "Q8_0";
+    }
+}
+inline int rfq_format_of(QuantFormat f)
+{
+    switch (f) {
+    case QuantFormat::Q4_0: return RFQ_Q4_0;
+    case QuantFormat::Q4_K: return RFQ_Q4_K;
+    case QuantFormat::Q6_K: return RFQ_Q6_K;
+    default: return RFQ_Q8_0;
+    }
+}
+struct QuantizedMatmulOp {
+    std::vector<uint8_t> weights; // [n_rows x n_cols], row-major blocks
+    size_t m = 1, n = 0, k = 0;
+    QuantFormat format = QuantFormat::Q4_0;
+    QuantizedMatmulOp(std::vector<uint8_t> w, size_t n_rows, size_t n_cols, QuantFormat f)
+        : weights(std::move(w)), m(1), n(n_rows), k(n_cols), format(f)
+    {
+    }
+    Status execute(const HipBackend &b, const HipBuffer &input, const HipBuffer &output) const
+    {
+        return matmul_host(rfq_format_of(format), name(format), b, weights, input, n, k, output);
+    }
+};
+
+// The shape checks of execute_matmul_q4_0 / q8_0 (src/ggml/hip_backend/op_dispatch.rs:951-1083):
+// 2-D operands, weight bytes = ceil(rows*cols/32) * block bytes, input k = weight columns.
+inline Status validate_matmul(const char *op, size_t block_bytes, const std::vector<size_t> &weights_shape,
+                              size_t weights_bytes, const std::vector<size_t> &input_shape)
+{
+    if (weights_shape.size() != 2 || input_shape.size() != 2) return Status::Err(std::string(op) + " expects 2D tensors");
+    const size_t n_rows = weights_shape[0], n_cols = weights_shape[1];
+    const size_t expected = ((n_rows * n_cols + 31) / 32) * block_bytes;
+    if (weights_bytes != expected)
+        return Status::Err(std::string(op) + " weights size mismatch: expected " + std::to_string(expected) +
+                           " bytes, got " + std::to_string(weights_bytes));
+    if (input_shape[1] != n_cols)
+        return Status::Err(std::string(op) + " dimension mismatch: k=" + std::to_string(input_shape[1]) +
+                           " weights_k=" + std::to_string(n_cols));
+    return ok_status();
+}
+inline Status validate_matmul_q4_0(const std::vector<size_t> &ws, size_t wbytes, const std::vector<size_t> &is)
+{
+    return validate_matmul("MatMulQ4_0", 20, ws, wbytes, is);
+}
+inline Status validate_matmul_q8_0(const std::vector<size_t> &ws, size_t wbytes, const std::vector<size_t> &is)
+{
+    return validate_matmul("MatMulQ8_0", 36, ws, wbytes, is);
+}
+
+} // namespace rocmforge
+#endif /* ROCMFORGE_RFQ_HPP */

@@ -1,0 +1,47 @@
+"""Writes tests/golden/vectors.npz: small packed inputs for every format and
+what the CPU oracle makes of them (dequantised values, GEMV and GEMM results).
+
+The inputs come from the seeded generators in rocmforge_amd.quantize plus raw
+random bytes (every code and exponent occurs); the expected outputs are the
+oracle's.  The oracle itself is pinned by the reference's own known-answer
+vectors and by brute force (tests/test_oracle_kat.py); these fixtures freeze
+its results so that the GPU parity tests can run where the oracle is not
+built, and so that a change in either side shows up as a diff.
+
+Run from the repository root:  python tests/golden/make_golden.py
+"""
+import os
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, ROOT)
+
+import oracle  # noqa: E402
+from rocmforge_amd import quantize as Q  # noqa: E402
+
+FORMATS = [Q.Q4_0, Q.Q8_0, Q.Q4_K, Q.Q6_K, Q.MXFP4, Q.MXFP6_E2M3]
+
+
+def main():
+    out = {}
+    rng = np.random.Generator(np.random.PCG64(20260100))
+    n, k, m = 16, 256, 2
+    for fmt in FORMATS:
+        name = Q.NAMES[fmt]
+        # (a) generator output, (b) raw random bytes with finite scales
+        w = Q.make_weights(fmt, n, k, seed=20260100 + fmt)
+        r = Q.random_blocks(fmt, n * k // Q.BLOCK_ELEMS[fmt], rng, exp_range=(-6, 4))
+        x = rng.standard_normal((m, k), dtype=np.float32)
+        for tag, blob in (("gen", w), ("raw", r)):
+            out[f"{name}.{tag}.bytes"] = blob
+            out[f"{name}.{tag}.dequant"] = oracle.dequantize(fmt, blob, n * k)
+            out[f"{name}.{tag}.gemv"] = oracle.qmatmul_nk(fmt, blob, x, m, n, k)
+        out[f"{name}.x"] = x
+    np.savez_compressed(os.path.join(os.path.dirname(os.path.abspath(__file__)), "vectors.npz"), **out)
+    print("wrote", len(out), "arrays")
+
+
+if __name__ == "__main__":
+    main()

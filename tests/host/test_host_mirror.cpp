@@ -1,0 +1,299 @@
+// Host tests of the C++ mirror (include/rocmforge_rfq.hpp): the reference's own
+// unit-test vectors for this path, run through the mirrored entry points -- so
+// every value comes from the GPU kernels.  Vectors and names follow
+//   src/kernels/quant/q4_0.rs:317-438, q8_0.rs:78-183, q4_k.rs:280-368, q6_k.rs:273-399,
+//   src/loader/mxfp_tests.rs:97-187 and 424-464, src/loader/dequant.rs:440-470,
+//   src/kernels/matmul/quantized/q4_0.rs:318-338, src/ggml/hip_backend/op_dispatch.rs:951-1014.
+// Prints one line per test; exit status 0 only if all passed.
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <functional>
+#include <string>
+#include <vector>
+
+#include "rocmforge_rfq.hpp"
+
+using namespace rocmforge;
+using bytes = std::vector<uint8_t>;
+
+static int failures = 0;
+#define EXPECT(cond)                                                                 \
+    do {                                                                             \
+        if (!(cond)) { std::printf("    FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond); failures++; } \
+    } while (0)
+
+static void put_f32(bytes &d, size_t off, float v) { std::memcpy(d.data() + off, &v, 4); }
+static void put_f16(bytes &d, size_t off, uint16_t bits) { std::memcpy(d.data() + off, &bits, 2); }
+static bool all_eq(const std::vector<float> &v, size_t a, size_t b, float want)
+{
+    for (size_t i = a; i < b; i++) if (v[i] != want) return false;
+    return true;
+}
+
+// ---- Q4_0 ---------------------------------------------------------------------
+static void test_dequantize_q4_0_zeros()
+{
+    bytes d(20, 0x88);
+    put_f32(d, 0, 1.0f);
+    auto r = loader::dequant_q4_0(d, 32);
+    EXPECT(r.size() == 32 && all_eq(r, 0, 32, 0.0f));
+}
+static void test_dequantize_q4_0_positive()
+{
+    bytes d(20, 0);
+    put_f32(d, 0, 2.0f);
+    for (int i = 0; i < 16; i++) d[4 + i] = (uint8_t)(((i + 1) << 4) | i);
+    auto r = loader::dequant_q4_0(d, 32);
+    EXPECT(r[0] == -16.0f && r[1] == -14.0f && r[30] == 14.0f && r[31] == -16.0f);
+}
+static void test_dequantize_q4_0_partial_and_multiple_blocks()
+{
+    bytes d(20, 0x88);
+    put_f32(d, 0, 1.0f);
+    auto r = loader::dequant_q4_0(d, 10);
+    EXPECT(r.size() == 10 && all_eq(r, 0, 10, 0.0f));
+    bytes d2(40, 0x88);
+    put_f32(d2, 0, 1.0f);
+    put_f32(d2, 20, 2.0f);
+    for (int i = 24; i < 40; i++) d2[i] = 0xCC;
+    r = loader::dequant_q4_0(d2, 64);
+    EXPECT(all_eq(r, 0, 32, 0.0f) && all_eq(r, 32, 64, 8.0f));
+    // short input: the blocks that are missing stay 0.0
+    r = loader::dequant_q4_0(d2, 96);
+    EXPECT(r.size() == 96 && all_eq(r, 64, 96, 0.0f));
+}
+
+// ---- Q8_0 ---------------------------------------------------------------------
+static void test_dequantize_q8_0_vectors()
+{
+    bytes d(36, 128);
+    put_f32(d, 0, 1.0f);
+    EXPECT(all_eq(loader::dequant_q8_0(d, 32), 0, 32, 0.0f));
+    put_f32(d, 0, 2.0f);
+    for (int i = 0; i < 32; i++) d[4 + i] = (uint8_t)(120 + i);
+    auto r = loader::dequant_q8_0(d, 32);
+    EXPECT(r[0] == -16.0f && r[15] == 14.0f && r[31] == 46.0f);
+    bytes d2(72, 128);
+    put_f32(d2, 0, 1.0f);
+    put_f32(d2, 36, 0.5f);
+    for (int i = 40; i < 72; i++) d2[i] = 138;
+    r = loader::dequant_q8_0(d2, 64);
+    EXPECT(all_eq(r, 0, 32, 0.0f) && all_eq(r, 32, 64, 5.0f));
+}
+
+// ---- Q4_K ---------------------------------------------------------------------
+static void test_dequantize_q4_k_single_block()
+{
+    bytes d(256, 0);
+    for (int i = 0; i < 8; i++) put_f16(d, 2 * i, 0x3C00); // 1.0
+    for (int i = 0; i < 224; i++) d[32 + i] = (uint8_t)(((i % 16) << 4) | (i % 16));
+    auto r = loader::dequant_q4_k(d, 256);
+    bool ok = true;
+    for (int i = 0; i < 256; i++) {
+        int sb = i / 32, e = i % 32, qo = sb * 28 + (e * 4) / 8;
+        unsigned combined = ((unsigned)d[32 + qo + 1] << 8) | d[32 + qo];
+        if (r[i] != (float)((combined >> ((e * 4) % 8)) & 15u)) ok = false;
+    }
+    EXPECT(ok);
+}
+static void test_dequantize_q4_k_partial_block_and_mins()
+{
+    bytes d(256, 0x88);
+    for (int i = 0; i < 32; i++) d[i] = 0;
+    for (int i = 0; i < 8; i++) put_f16(d, 2 * i, 0x3C00);
+    auto r = loader::dequant_q4_k(d, 100);
+    EXPECT(r.size() == 100 && all_eq(r, 0, 100, 8.0f));
+    d[16 + 1] = (uint8_t)(int8_t)-3; // min of sub-block 1
+    r = loader::dequant_q4_k(d, 256);
+    EXPECT(all_eq(r, 0, 32, 8.0f) && all_eq(r, 32, 64, 5.0f));
+}
+
+// ---- Q6_K ---------------------------------------------------------------------
+static void test_dequantize_q6_k_vectors()
+{
+    bytes d(256, 0);
+    for (int i = 0; i < 16; i++) put_f16(d, 2 * i, 0x4000); // 2.0
+    EXPECT(all_eq(loader::dequant_q6_k(d, 100), 0, 100, 0.0f));
+    for (int i = 0; i < 16; i++) put_f16(d, 2 * i, 0x3C00);
+    for (int i = 32; i < 224; i++) d[i] = 0xFF;                // every 6-bit field = 63 = -1
+    EXPECT(all_eq(loader::dequant_q6_k(d, 256), 0, 256, -1.0f));
+    for (int i = 0; i < 192; i++) d[32 + i] = (uint8_t)((i % 64) * 4);
+    auto r = loader::dequant_q6_k(d, 256);
+    bool finite = true;
+    for (float v : r) if (!std::isfinite(v)) finite = false;
+    EXPECT(finite);
+}
+
+// ---- MXFP ---------------------------------------------------------------------
+static GgufTensor mx_tensor(GgufTensorType t, size_t n, bytes data)
+{
+    GgufTensor g("w", TensorShape::from_dims({n}), t, 0);
+    g.data = std::move(data);
+    return g;
+}
+static void test_mxfp4_block_of_twos_and_clamp()
+{
+    // exponent byte 1 (scale 2.0), every nibble 0b0001 (decodes to 1.0): 2.0 each
+    bytes d(17, 0x11);
+    d[0] = 1;
+    auto r = loader::dequant_mxfp4(mx_tensor(GgufTensorType::Mxfp4, 32, d));
+    EXPECT(r.ok && r.value.size() == 32 && all_eq(r.value, 0, 32, 2.0f));
+    // code 7 decodes to 8.0; scale 4.0: clamped to +8; code 15 to -8
+    bytes c(17, 0x7F);
+    c[0] = 2;
+    r = loader::dequant_mxfp4(mx_tensor(GgufTensorType::Mxfp4, 32, c));
+    EXPECT(r.ok && r.value[0] == 8.0f && r.value[1] == -8.0f); // element 2j = HIGH nibble
+    GgufTensor t = mx_tensor(GgufTensorType::Mxfp4, 64, d);
+    EXPECT(t.data_size() == 34);
+}
+static void test_mxfp6_block_size_clamp_and_last_element()
+{
+    bytes d(25, 0xFF);
+    d[0] = 3; // scale 8: every code 0b111111 = -7.5 * 8 -> clamped to -7.5
+    auto r = loader::dequant_mxfp6(mx_tensor(GgufTensorType::Mxfp6E2m3, 32, d));
+    EXPECT(r.ok && r.value.size() == 32 && all_eq(r.value, 0, 31, -7.5f));
+    EXPECT(r.value[31] == 0.0f); // the loader never reaches the last element of a block
+    auto r2 = loader::dequantize(mx_tensor(GgufTensorType::Mxfp6E3m2, 32, d)); // decoded like E2M3
+    EXPECT(r2.ok && r2.value == r.value);
+    EXPECT(mx_tensor(GgufTensorType::Mxfp6E2m3, 32, d).data_size() == 25);
+}
+
+// ---- types ----------------------------------------------------------------------
+static void test_tensor_types_and_sizes()
+{
+    EXPECT(tensor_type_from_u32(20).ok && tensor_type_from_u32(20).value == GgufTensorType::Mxfp4);
+    EXPECT(tensor_type_from_u32(21).value == GgufTensorType::Mxfp6E2m3 && tensor_type_from_u32(22).value == GgufTensorType::Mxfp6E3m2);
+    EXPECT(!tensor_type_from_u32(3).ok && !tensor_type_from_u32(6).ok && !tensor_type_from_u32(7).ok && !tensor_type_from_u32(99).ok);
+    EXPECT(element_size(GgufTensorType::Mxfp4) == 32 && element_size(GgufTensorType::Q4_K) == 256 && element_size(GgufTensorType::F16) == 2);
+    EXPECT(block_size(GgufTensorType::Q8_0) == 32 && block_size(GgufTensorType::Q6_K) == 256 && block_size(GgufTensorType::F32) == 1);
+    EXPECT(std::string(to_string(GgufTensorType::Q4_K)) == "Q4_K" && std::string(to_string(GgufTensorType::F32)) == "FP32");
+    TensorShape s = TensorShape::from_dims({4, 8, 16});
+    EXPECT(s.total_elements() == 512 && s.strides()[0] == 128 && s.strides()[1] == 16 && s.strides()[2] == 1);
+    GgufTensor q4("t", TensorShape::from_dims({2, 32}), GgufTensorType::Q4_0, 0);
+    EXPECT(q4.data_size() == 2 * 36);            // as the reference counts it (the decoder strides by 20)
+    GgufTensor qk("t", TensorShape::from_dims({300}), GgufTensorType::Q4_K, 0);
+    EXPECT(qk.data_size() == 512 && qk.quant_type == "Q4_K");
+}
+static void test_dequantize_dispatch_f32_f16()
+{
+    GgufTensor f("f", TensorShape::from_dims({2}), GgufTensorType::F32, 0);
+    f.data.resize(9);                             // one trailing byte is dropped
+    float a = 1.5f, b = -2.25f;
+    std::memcpy(f.data.data(), &a, 4);
+    std::memcpy(f.data.data() + 4, &b, 4);
+    auto r = loader::dequantize(f);
+    EXPECT(r.ok && r.value.size() == 2 && r.value[0] == 1.5f && r.value[1] == -2.25f);
+    GgufTensor h("h", TensorShape::from_dims({4}), GgufTensorType::F16, 0);
+    h.data.resize(8);
+    put_f16(h.data, 0, 0x3C00); put_f16(h.data, 2, 0x4000); put_f16(h.data, 4, 0xC000); put_f16(h.data, 6, 0x0001);
+    r = loader::dequantize(h);
+    EXPECT(r.ok && r.value[0] == 1.0f && r.value[1] == 2.0f && r.value[2] == -2.0f && r.value[3] == std::ldexp(1.0f, -24));
+    GgufTensor q2("q", TensorShape::from_dims({256}), GgufTensorType::Q2_K, 0);
+    EXPECT(!loader::dequantize(q2).ok);
+}
+
+// ---- device buffers and matmul ------------------------------------------------------
+static void test_dequantize_q4_0_kernel_cached_and_twins()
+{
+    auto be = HipBackend::create();
+    EXPECT(be.ok);
+    bytes d(40, 0x88);
+    put_f32(d, 0, 1.0f);
+    put_f32(d, 20, 2.0f);
+    for (int i = 24; i < 40; i++) d[i] = 0xCC;
+    auto out = HipBuffer::create(64 * sizeof(float));
+    EXPECT(out.ok);
+    EXPECT(dequantize_q4_0_kernel_cached(be.value, d, out.value, 64).ok);
+    std::vector<float> h(64);
+    EXPECT(out.value.copy_to_host(h).ok && all_eq(h, 0, 32, 0.0f) && all_eq(h, 32, 64, 8.0f));
+    auto small = HipBuffer::create(16);
+    EXPECT(!dequantize_q4_0_kernel_cached(be.value, d, small.value, 64).ok);   // output too small
+    bytes k(256, 0x88);
+    for (int i = 0; i < 32; i++) k[i] = 0;
+    for (int i = 0; i < 8; i++) put_f16(k, 2 * i, 0x3C00);
+    auto outk = HipBuffer::create(256 * sizeof(float));
+    EXPECT(dequantize_q4_k_gpu_kernel(be.value, k, outk.value, 256).ok);
+    std::vector<float> hk(256);
+    EXPECT(outk.value.copy_to_host(hk).ok && all_eq(hk, 0, 256, 8.0f));
+}
+static void test_matmul_q4_0_against_dequantized_weights()
+{
+    // weights [n_rows=8, n_cols=64], input [64]: out = deq(W) . x, as q4_0.rs:318-338 checks it
+    const size_t n_rows = 8, n_cols = 64;
+    bytes w(n_rows * (n_cols / 32) * 20);
+    for (size_t b = 0; b < w.size() / 20; b++) {
+        put_f32(w, b * 20, 0.25f * (float)(b % 5 + 1));
+        for (int i = 0; i < 16; i++) w[b * 20 + 4 + i] = (uint8_t)((b * 37 + i * 11) & 0xFF);
+    }
+    std::vector<float> x(n_cols);
+    for (size_t i = 0; i < n_cols; i++) x[i] = 0.125f * (float)((int)(i % 9) - 4);
+    auto be = HipBackend::create();
+    auto in = HipBuffer::create(n_cols * 4), out = HipBuffer::create(n_rows * 4);
+    EXPECT(in.value.copy_from_host(x).ok);
+    EXPECT(matmul_q4_0(be.value, w, in.value, n_rows, n_cols, out.value).ok);
+    std::vector<float> y(n_rows), deq = loader::dequant_q4_0(w, n_rows * n_cols);
+    EXPECT(out.value.copy_to_host(y).ok);
+    bool close = true;
+    for (size_t r = 0; r < n_rows; r++) {
+        float s = 0.0f;
+        for (size_t c = 0; c < n_cols; c++) s += x[c] * deq[r * n_cols + c];   // cpu_matmul_f32 order
+        if (std::fabs(y[r] - s) > 1e-3f * std::fmax(std::fabs(s), 1.0f)) close = false;
+    }
+    EXPECT(close);
+    // the batch description type runs the same operation
+    QuantizedMatmulOp op(w, n_rows, n_cols, QuantFormat::Q4_0);
+    auto out2 = HipBuffer::create(n_rows * 4);
+    EXPECT(op.m == 1 && op.execute(be.value, in.value, out2.value).ok);
+    std::vector<float> y2(n_rows);
+    EXPECT(out2.value.copy_to_host(y2).ok && y2 == y);
+    // raw device pointers
+    auto dw = HipBuffer::create(w.size());
+    EXPECT(dw.value.copy_from_host(w).ok);
+    EXPECT(matmul_q4_0_gpu(be.value, (const float *)in.value.as_ptr(), (const uint8_t *)dw.value.as_ptr(),
+                           (float *)out2.value.as_ptr(), 1, n_rows, n_cols).ok);
+    EXPECT(be.value.synchronize().ok && out2.value.copy_to_host(y2).ok && y2 == y);
+    // wrong byte count is an error, not a crash
+    bytes shorter(w.begin(), w.end() - 20);
+    EXPECT(!matmul_q4_0(be.value, shorter, in.value, n_rows, n_cols, out.value).ok);
+}
+static void test_matmul_validation_like_op_dispatch()
+{
+    EXPECT(validate_matmul_q4_0({8, 64}, 8 * 2 * 20, {1, 64}).ok);
+    EXPECT(!validate_matmul_q4_0({8, 64}, 8 * 2 * 20 - 1, {1, 64}).ok);          // weights size mismatch
+    EXPECT(!validate_matmul_q4_0({8, 64}, 8 * 2 * 20, {1, 32}).ok);              // k != weights_k
+    EXPECT(!validate_matmul_q4_0({8, 64, 1}, 8 * 2 * 20, {1, 64}).ok);           // expects 2D tensors
+    EXPECT(validate_matmul_q8_0({4, 32}, 4 * 36, {8, 32}).ok);
+    EXPECT(bytes_per_element(QuantFormat::Q8_0) == 36.0f / 32.0f && std::string(name(QuantFormat::Q6_K)) == "Q6_K");
+}
+
+int main()
+{
+    struct T { const char *name; std::function<void()> fn; };
+    const T tests[] = {
+        {"test_dequantize_q4_0_zeros", test_dequantize_q4_0_zeros},
+        {"test_dequantize_q4_0_positive", test_dequantize_q4_0_positive},
+        {"test_dequantize_q4_0_partial_and_multiple_blocks", test_dequantize_q4_0_partial_and_multiple_blocks},
+        {"test_dequantize_q8_0_vectors", test_dequantize_q8_0_vectors},
+        {"test_dequantize_q4_k_single_block", test_dequantize_q4_k_single_block},
+        {"test_dequantize_q4_k_partial_block_and_mins", test_dequantize_q4_k_partial_block_and_mins},
+        {"test_dequantize_q6_k_vectors", test_dequantize_q6_k_vectors},
+        {"test_mxfp4_block_of_twos_and_clamp", test_mxfp4_block_of_twos_and_clamp},
+        {"test_mxfp6_block_size_clamp_and_last_element", test_mxfp6_block_size_clamp_and_last_element},
+        {"test_tensor_types_and_sizes", test_tensor_types_and_sizes},
+        {"test_dequantize_dispatch_f32_f16", test_dequantize_dispatch_f32_f16},
+        {"test_dequantize_q4_0_kernel_cached_and_twins", test_dequantize_q4_0_kernel_cached_and_twins},
+        {"test_matmul_q4_0_against_dequantized_weights", test_matmul_q4_0_against_dequantized_weights},
+        {"test_matmul_validation_like_op_dispatch", test_matmul_validation_like_op_dispatch},
+    };
+    for (const T &t : tests) {
+        int before = failures;
+        std::printf("%s ...\n", t.name);
+        std::fflush(stdout);
+        t.fn();
+        std::printf("%s %s\n", t.name, failures == before ? "ok" : "FAILED");
+        std::fflush(stdout);
+    }
+    std::printf("%d test(s) failed\n", failures);
+    return failures ? 1 : 0;
+}
