@@ -18,6 +18,8 @@
 //                the units and read x through the L1/L2 caches.
 // Reduction: DPP butterflies inside each row of 16 lanes, v_readlane across
 // the four rows; an LDS hop only when a row is split over several wavefronts.
+#include <mutex>
+
 #include "rfq_common.hpp"
 
 // Per-wavefront phase timestamps for tuning builds (-DRFQ_GEMV_TRACE); compiled
@@ -661,6 +663,121 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
     }
 }
 
+// ---- 2 <= m <= 8: the same integer-dot scheme with M activation vectors ----------
+//
+// Every weight unit is loaded once and dotted against the M prepared vectors,
+// whose limbs stay in registers (26 per unit and vector: one unit per lane,
+// WPR = ceil(units / 64) wavefronts per row).  Vectors past m_valid repeat the
+// last one and are not stored.  LDS holds the M prepared vectors.
+template <int FMT, int WPR, int R, int M>
+__global__ void __launch_bounds__(256)
+gemv_idot_batch_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ y, int n, int k,
+                       int groups, int m_valid)
+{
+    using IU = IUnit<FMT>;
+    constexpr int TEAMS = 4 / WPR, TL = 64 * WPR;
+    constexpr int D = R < 3 ? R : 3;
+    static_assert(R * M <= 64, "one lane per (row, vector) in the cross-wavefront sum");
+    extern __shared__ __attribute__((aligned(16))) uint32_t xlds[]; // [M][units][28]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int team = wave / WPR, wit = wave % WPR;
+    const int tl = wit * 64 + lane;
+    const int ku = k >> 5;
+    const size_t rb = row_bytes<FMT>(k);
+    const bool live = tl < ku;
+    const int unit = live ? tl : ku - 1;
+    (void)TL;
+
+    const int rows_per_team = groups * R;
+    const int row0 = (blockIdx.x * TEAMS + team) * rows_per_team;
+    int row_end = row0 + rows_per_team;
+    if (row_end > n) row_end = n;
+    const int row_last = row_end > row0 ? row_end - 1 : (n - 1);
+
+    IU buf[D];
+    auto load_row = [&](int slot, int i) {
+        int r = row0 + i;
+        if (r > row_last) r = row_last;
+        buf[slot].load(w + (size_t)r * rb, unit);
+    };
+#pragma unroll
+    for (int d = 0; d < D; d++) load_row(d, d);
+
+    // Cooperative conversion of the M vectors: 2*ku half-units each.
+    for (int h = threadIdx.x; h < 2 * ku * M; h += 256) {
+        const int v = h / (2 * ku), hh = h - v * 2 * ku;
+        const int vs = v < m_valid ? v : m_valid - 1;
+        float xw[16];
+        prep_load(x + (size_t)vs * k + (size_t)hh * 16, xw);
+        prep_convert<IU::NIBBLE, IU::TOPOFF>(xw, hh & 1, xlds + ((size_t)v * ku + (hh >> 1)) * 28);
+    }
+    __syncthreads();
+    XPrep xp[M];
+#pragma unroll
+    for (int v = 0; v < M; v++) {
+        const uint32_t *src = xlds + ((size_t)v * ku + unit) * 28;
+#pragma unroll
+        for (int i = 0; i < 24; i += 4) {
+            uint4 q = *reinterpret_cast<const uint4 *>(src + i);
+            xp[v].l[i] = q.x; xp[v].l[i + 1] = q.y; xp[v].l[i + 2] = q.z; xp[v].l[i + 3] = q.w;
+        }
+        xp[v].s = __uint_as_float(src[24]);
+        xp[v].xsum = __uint_as_float(src[25]);
+    }
+
+    __shared__ float part[R * M][4];
+    for (int g = 0; g < groups; g++) {
+        const int base = g * R;
+        if (g > 0) {
+#pragma unroll
+            for (int d = 0; d < D; d++) load_row(d, base + d);
+        }
+        float res[R][M];
+#pragma unroll
+        for (int i = 0; i < R; i++) {
+            float acc[M];
+#pragma unroll
+            for (int v = 0; v < M; v++) {
+                float t = buf[i % D].idot(xp[v]);
+                acc[v] = live ? t : 0.f;
+            }
+            if (i + D < R) load_row(i % D, base + i + D);
+#pragma unroll
+            for (int v = 0; v < M; v++) res[i][v] = wave_sum(acc[v]);
+        }
+        if (WPR == 1) {
+            if (lane == 0) {
+#pragma unroll
+                for (int i = 0; i < R; i++) {
+                    int r = row0 + base + i;
+#pragma unroll
+                    for (int v = 0; v < M; v++)
+                        if (r < row_end && v < m_valid) y[(size_t)v * n + r] = res[i][v];
+                }
+            }
+        } else {
+            // `groups` is uniform over the block, so every wavefront reaches
+            // both barriers the same number of times.
+            if (lane == 0) {
+#pragma unroll
+                for (int i = 0; i < R; i++)
+#pragma unroll
+                    for (int v = 0; v < M; v++) part[i * M + v][wave] = res[i][v];
+            }
+            __syncthreads();
+            if (wit == 0 && lane < R * M) {
+                const int i = lane / M, v = lane % M;
+                const int r = row0 + base + i;
+                float t = 0.f;
+#pragma unroll
+                for (int q = 0; q < WPR; q++) t += part[lane][team * WPR + q];
+                if (r < row_end && v < m_valid) y[(size_t)v * n + r] = t;
+            }
+            __syncthreads();
+        }
+    }
+}
+
 // ---- any m <= 8, any k: one row per wavefront ---------------------------------
 template <int FMT, int M>
 __global__ void __launch_bounds__(256)
@@ -766,6 +883,64 @@ int run_idot(const uint8_t *w, const float *x, float *y, int n, int k, hipStream
     }
 }
 
+template <int FMT, int WPR, int R, int M>
+int launch_idot_batch(const uint8_t *w, const float *x, float *y, int m, int n, int k, int blocks, int groups,
+                      hipStream_t s)
+{
+    const size_t lds = (size_t)M * (k / 32) * 28 * sizeof(uint32_t);
+    static std::once_flag once;
+    static hipError_t attr_err = hipSuccess;
+    std::call_once(once, [] {
+        attr_err = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_idot_batch_kernel<FMT, WPR, R, M>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 4096);
+    });
+    if (attr_err != hipSuccess) return hip_fail(attr_err, "hipFuncSetAttribute(gemv_idot_batch_kernel)");
+    hipLaunchKernelGGL((gemv_idot_batch_kernel<FMT, WPR, R, M>), dim3(blocks), dim3(256), lds, s, w, x, y, n, k, groups,
+                       m);
+    RFQ_LAUNCH_CHECK("gemv_idot_batch_kernel");
+    return RFQ_OK;
+}
+
+template <int FMT, int WPR, int M>
+int run_idot_batch(const uint8_t *w, const float *x, float *y, int m, int n, int k, hipStream_t s)
+{
+    if constexpr (HasIdot<FMT>::value) {
+        constexpr int TEAMS = 4 / WPR;
+        // one or two resident blocks per CU (LDS holds the M prepared vectors),
+        // every team walking the same number of rows
+        const size_t lds = (size_t)M * (k / 32) * 28 * sizeof(uint32_t);
+        const int slots = device_cu_count() * (lds > 72 * 1024 ? 1 : 2);
+        int want = (n + slots * TEAMS - 1) / (slots * TEAMS);
+        if (want < 1) want = 1;
+        constexpr int RMAX = 64 / M < 8 ? 64 / M : 8;
+        int best_r = RMAX, best_groups = 1, best_blocks = 0;
+        long best_cost = -1;
+        for (int r : {4, RMAX}) {
+            int groups = (want + r - 1) / r;
+            int blocks = (n + TEAMS * r * groups - 1) / (TEAMS * r * groups);
+            long waves_of_blocks = (blocks + slots - 1) / slots;
+            long cost = waves_of_blocks * r * groups;
+            if (best_cost < 0 || cost < best_cost || (cost == best_cost && r > best_r)) {
+                best_cost = cost; best_r = r; best_groups = groups; best_blocks = blocks;
+            }
+        }
+        if (best_r == 4) return launch_idot_batch<FMT, WPR, 4, M>(w, x, y, m, n, k, best_blocks, best_groups, s);
+        return launch_idot_batch<FMT, WPR, RMAX, M>(w, x, y, m, n, k, best_blocks, best_groups, s);
+    } else {
+        (void)w; (void)x; (void)y; (void)m; (void)n; (void)k; (void)s;
+        return RFQ_E_UNSUPPORTED;
+    }
+}
+
+template <int FMT, int M>
+int run_idot_batch_k(const uint8_t *w, const float *x, float *y, int m, int n, int k, hipStream_t s)
+{
+    const int ku = k / 32;
+    if (ku <= 64) return run_idot_batch<FMT, 1, M>(w, x, y, m, n, k, s);
+    if (ku <= 128) return run_idot_batch<FMT, 2, M>(w, x, y, m, n, k, s);
+    return run_idot_batch<FMT, 4, M>(w, x, y, m, n, k, s);
+}
+
 template <int FMT, int M>
 int run_generic(const uint8_t *w, const float *x, float *y, int n, int k, hipStream_t s)
 {
@@ -786,6 +961,11 @@ int run(const uint8_t *w, const float *x, float *y, int m, int n, int k, hipStre
         if (ku <= 128) return run_idot<FMT, 2, 1>(w, x, y, n, k, s);
         if (ku <= 256) return run_idot<FMT, 2, 2>(w, x, y, n, k, s);
         if (ku <= 512) return run_idot<FMT, 2, 4>(w, x, y, n, k, s);
+    }
+    if (HasIdot<FMT>::value && m > 1 && ku > 32 && ku <= 256) {
+        if (m <= 2) return run_idot_batch_k<FMT, 2>(w, x, y, m, n, k, s);
+        if (m <= 4) return run_idot_batch_k<FMT, 4>(w, x, y, m, n, k, s);
+        return run_idot_batch_k<FMT, 8>(w, x, y, m, n, k, s);
     }
     switch (m) {
     case 1: return run_generic<FMT, 1>(w, x, y, n, k, s);
