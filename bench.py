@@ -67,6 +67,29 @@ def time_gemv(torch, fmt, n, k, m, copies, steps, warmup, Q, seed):
     return wall, ms.value / 1e3, w, x, y.cpu().numpy()
 
 
+def time_dequant(torch, fmt, n, k, steps, warmup, Q, seed):
+    """Device seconds per rfq_dequant call of an [n, k] matrix; bytes moved = packed in + 4 per element out."""
+    import ctypes as C
+
+    from rocmforge_amd import _lib
+    dev = torch.device("cuda:0")
+    import numpy as np
+    slab = min(n, 4096)                                  # quantise a slab once, repeat it down the rows
+    w = np.tile(Q.make_weights(fmt, slab, k, seed=seed), n // slab) if n % slab == 0 else Q.make_weights(fmt, n, k, seed=seed)
+    copies = 4
+    dws = [torch.from_numpy(w).to(dev) for _ in range(copies)]
+    ptrs = (C.c_void_p * copies)(*[t.data_ptr() for t in dws])
+    out = torch.empty(n * k, dtype=torch.float32, device=dev)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    ms = C.c_float(0)
+    L = _lib.lib()
+    _lib.check(L.rfq_bench_dequant(fmt, ptrs, copies, w.size, C.c_void_p(out.data_ptr()), n * k, 0, warmup, stream,
+                                   C.byref(ms)))
+    _lib.check(L.rfq_bench_dequant(fmt, ptrs, copies, w.size, C.c_void_p(out.data_ptr()), n * k, 0, steps, stream,
+                                   C.byref(ms)))
+    return ms.value / 1e3 / steps, w.size + 4 * n * k
+
+
 def cpu_baseline(fmt, w, x, n, k, budget_s=12.0):
     """The CPU oracle (dequantise everything, then the sequential fp32 matmul)
     on one host thread, repeated until ~budget_s of CPU work."""
@@ -173,6 +196,12 @@ def main():
             b = algorithmic_bytes(f, n, k, m, Q)
             also[name] = {"GB/s": round(b / (d / 500) / 1e9, 1), "us": round(d / 500 * 1e6, 2),
                           "hbm_frac": round(b / (d / 500) / 1e9 / HBM_PEAK_GBS, 4)}
+        for name, f, n, k, seed in (("Q4_0 dequant 4096x4096", Q.Q4_0, 4096, 4096, 20260021),
+                                    ("Q4_K dequant 14336x4096", Q.Q4_K, N, K, 20260023),
+                                    ("MXFP4 dequant 28672x8192", Q.MXFP4, 28672, 8192, 20260025)):
+            t, b = time_dequant(torch, f, n, k, 50, 5, Q, seed)
+            also[name] = {"GB/s": round(b / t / 1e9, 1), "us": round(t * 1e6, 2), "hbm_frac": round(b / t / 1e9 / HBM_PEAK_GBS, 4),
+                          "Gelem/s": round(n * k / t / 1e9, 1)}
         try:
             import bench_gemm
             also.update(bench_gemm.run(torch))
