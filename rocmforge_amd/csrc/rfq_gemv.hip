@@ -289,20 +289,21 @@ __device__ __forceinline__ float sum32(const float (&x)[32])
 //
 // Block = 4 wavefronts = 4 / WPR teams.  Lane `tl` of a team (0 .. 64*WPR-1)
 // owns units tl + j * 64 * WPR, j < UPL, of EVERY row the team visits.  A team
-// walks `rows_per_team` consecutive rows in groups of D: all loads of a group
-// are issued back to back (D rows x UPL units in flight per lane, no branch
-// between them so the hardware counters let row d be consumed while rows
-// d+1.. are still arriving), then the D rows are reduced.  Rows past the end
+// walks `groups * R` consecutive rows, R (a compile-time constant) at a time,
+// with a rolling prefetch: three rows are in flight per lane, and as soon as a
+// row has been consumed its slot takes the row three further on, so loads and
+// arithmetic overlap.  Rows past the end
 // re-read the team's last valid row (same addresses, served by the cache) and
 // their result is dropped; lanes past the end of a row do the same with the
 // row's last unit.  HBM latency, not bandwidth, bounds a wavefront that has a
 // single row in flight, hence the depth.
-template <int FMT, int UPL, int WPR, int D>
+template <int FMT, int UPL, int WPR, int R>
 __global__ void __launch_bounds__(256)
 gemv_xreg_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ y, int n, int k,
-                 int rows_per_team)
+                 int groups)
 {
     constexpr int TEAMS = 4 / WPR, TL = 64 * WPR;
+    constexpr int D = R < 3 ? R : 3;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int team = wave / WPR, wit = wave % WPR;
     const int tl = wit * 64 + lane;
@@ -320,64 +321,68 @@ gemv_xreg_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
         load_x32(x + (size_t)unit[j] * 32, xs[j]);
     }
 
-    __shared__ float part[D][4];
+    __shared__ float part[R][4];
+    const int rows_per_team = groups * R;
     const int row0 = (blockIdx.x * TEAMS + team) * rows_per_team;
     int row_end = row0 + rows_per_team;
     if (row_end > n) row_end = n;
     const int row_last = row_end > row0 ? row_end - 1 : (n - 1);
 
     Unit<FMT> buf[D][UPL];
-    auto load_group = [&](int g) {
+    auto load_row = [&](int slot, int i) {
+        int r = row0 + i;
+        if (r > row_last) r = row_last;
+        const uint8_t *row = w + (size_t)r * rb;
 #pragma unroll
-        for (int d = 0; d < D; d++) {
-            int r = row0 + g + d;
-            if (r > row_last) r = row_last;
-            const uint8_t *row = w + (size_t)r * rb;
-#pragma unroll
-            for (int j = 0; j < UPL; j++) buf[d][j].load(row, unit[j]);
-        }
+        for (int j = 0; j < UPL; j++) buf[slot][j].load(row, unit[j]);
     };
-    // x first, then the whole first group, and only then the first use of x:
-    // the weight loads are already in flight while the x sums are formed.
-    load_group(0);
+    // x first, then the first rows, and only then the first use of x: the
+    // weight loads are already in flight while the x sums are formed.
+#pragma unroll
+    for (int d = 0; d < D; d++) load_row(d, d);
 #pragma unroll
     for (int j = 0; j < UPL; j++) xsum[j] = Unit<FMT>::NEEDS_XSUM ? sum32(xs[j]) : 0.f;
 
-    for (int g = 0; g < rows_per_team; g += D) {
-        if (g > 0) load_group(g);
-        float res[D];
+    for (int g = 0; g < groups; g++) {
+        const int base = g * R;
+        if (g > 0) {
 #pragma unroll
-        for (int d = 0; d < D; d++) {
+            for (int d = 0; d < D; d++) load_row(d, base + d);
+        }
+        float res[R];
+#pragma unroll
+        for (int i = 0; i < R; i++) {
             float acc = 0.f;
 #pragma unroll
             for (int j = 0; j < UPL; j++) {
-                float t = buf[d][j].dot(xs[j], xsum[j]);
+                float t = buf[i % D][j].dot(xs[j], xsum[j]);
                 acc += live[j] ? t : 0.f;
             }
-            res[d] = wave_sum(acc);
+            if (i + D < R) load_row(i % D, base + i + D); // the slot just consumed takes the row D further on
+            res[i] = wave_sum(acc);
         }
         if (WPR == 1) {
             if (lane == 0) {
 #pragma unroll
-                for (int d = 0; d < D; d++) {
-                    int r = row0 + g + d;
-                    if (g + d < rows_per_team && r < n) y[r] = res[d];
+                for (int i = 0; i < R; i++) {
+                    int r = row0 + base + i;
+                    if (r < row_end) y[r] = res[i];
                 }
             }
         } else {
-            // The group loop bounds are uniform over the block, so every
-            // wavefront reaches both barriers the same number of times.
+            // `groups` is uniform over the block, so every wavefront reaches
+            // both barriers the same number of times.
             if (lane == 0) {
 #pragma unroll
-                for (int d = 0; d < D; d++) part[d][wave] = res[d];
+                for (int i = 0; i < R; i++) part[i][wave] = res[i];
             }
             __syncthreads();
-            if (wit == 0 && lane < D) {
-                int r = row0 + g + lane;
+            if (wit == 0 && lane < R) {
+                int r = row0 + base + lane;
                 float t = 0.f;
 #pragma unroll
                 for (int q = 0; q < WPR; q++) t += part[lane][team * WPR + q];
-                if (g + lane < rows_per_team && r < n) y[r] = t;
+                if (r < row_end) y[r] = t;
             }
             __syncthreads();
         }
@@ -811,26 +816,53 @@ gemv_generic_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, 
     }
 }
 
-// Rows in flight per lane: as deep as the register file allows at two
-// wavefronts per SIMD (x: 32*UPL registers, each unit 5..9).
-template <int FMT> struct Depth { static constexpr int D = 8; };
-template <> struct Depth<RFQ_Q8_0> { static constexpr int D = 4; };
+// `per_cu` resident blocks per CU, every team walking the same number of rows
+// (a straggler is expensive on a ~10 us kernel).  Rows per team = groups * R
+// with R from a small compiled set; the pair that wastes the fewest row slots
+// wins, the larger R on a tie.
+struct RowPlan { int r, groups, blocks; };
+inline RowPlan plan_rows(int n, int teams, int per_cu)
+{
+    const int slots = device_cu_count() * per_cu;
+    int want = (n + slots * teams - 1) / (slots * teams);
+    if (want < 1) want = 1;
+    static const int RS[6] = {2, 4, 5, 6, 7, 8};
+    RowPlan best{8, 1, 0};
+    long best_cost = -1;
+    for (int idx = 0; idx < 6; idx++) {
+        int r = RS[idx];
+        int groups = (want + r - 1) / r;
+        int blocks = (n + teams * r * groups - 1) / (teams * r * groups);
+        long waves_of_blocks = (blocks + slots - 1) / slots;
+        long cost = waves_of_blocks * r * groups;
+        if (best_cost < 0 || cost < best_cost || (cost == best_cost && r > best.r)) {
+            best_cost = cost;
+            best = RowPlan{r, groups, blocks};
+        }
+    }
+    return best;
+}
+
+template <int FMT, int UPL, int WPR, int R>
+int launch_xreg(const uint8_t *w, const float *x, float *y, int n, int k, const RowPlan &p, hipStream_t s)
+{
+    hipLaunchKernelGGL((gemv_xreg_kernel<FMT, UPL, WPR, R>), dim3(p.blocks), dim3(256), 0, s, w, x, y, n, k, p.groups);
+    RFQ_LAUNCH_CHECK("gemv_xreg_kernel");
+    return RFQ_OK;
+}
 
 template <int FMT, int UPL, int WPR>
 int run_xreg(const uint8_t *w, const float *x, float *y, int n, int k, hipStream_t s)
 {
-    constexpr int TEAMS = 4 / WPR, D = Depth<FMT>::D;
-    // Two resident blocks per CU; then even out the rows so every team walks
-    // the same number of them (no straggler tail on a ~10 us kernel).
-    int cus = device_cu_count();
-    int blocks = cus * 2;
-    int rows_per_team = (n + blocks * TEAMS - 1) / (blocks * TEAMS);
-    if (rows_per_team < 1) rows_per_team = 1;
-    blocks = (n + rows_per_team * TEAMS - 1) / (rows_per_team * TEAMS);
-    hipLaunchKernelGGL((gemv_xreg_kernel<FMT, UPL, WPR, D>), dim3(blocks), dim3(256), 0, s, w, x, y, n, k,
-                       rows_per_team);
-    RFQ_LAUNCH_CHECK("gemv_xreg_kernel");
-    return RFQ_OK;
+    const RowPlan p = plan_rows(n, 4 / WPR, 2); // (three blocks per CU fit for Q6_K but run slower)
+    switch (p.r) {
+    case 2: return launch_xreg<FMT, UPL, WPR, 2>(w, x, y, n, k, p, s);
+    case 4: return launch_xreg<FMT, UPL, WPR, 4>(w, x, y, n, k, p, s);
+    case 5: return launch_xreg<FMT, UPL, WPR, 5>(w, x, y, n, k, p, s);
+    case 6: return launch_xreg<FMT, UPL, WPR, 6>(w, x, y, n, k, p, s);
+    case 7: return launch_xreg<FMT, UPL, WPR, 7>(w, x, y, n, k, p, s);
+    default: return launch_xreg<FMT, UPL, WPR, 8>(w, x, y, n, k, p, s);
+    }
 }
 
 template <int FMT> struct HasIdot { static constexpr bool value = false; };
