@@ -36,6 +36,14 @@
 #define RFQ_KQ_SKIP 0
 #endif
 
+#ifdef RFQ_KQ_TRACE
+__device__ long long rfq_kq_trace_dev[8];
+extern "C" __attribute__((visibility("default"))) int rfq_kq_trace(long long *out)
+{
+    return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(rfq_kq_trace_dev), sizeof(long long) * 8);
+}
+#endif
+
 namespace rfq {
 namespace {
 
@@ -56,133 +64,197 @@ __device__ __forceinline__ void lds_barrier()
 }
 
 constexpr int BM = 256, BN = 128, BK = 64;
+constexpr int TI = 2, TJ = 4;                    // instruction tiles of a wavefront: 64 m x 128 n
 constexpr int LDR = BK * 2 + 16;                 // bytes per LDS row: 64 fp16 + 16 pad (rows 36 dwords apart)
-constexpr int A_BYTES = BM * LDR, W_BYTES = BN * LDR, STAGE_BYTES = A_BYTES + W_BYTES;
+constexpr int W_BYTES = BN * LDR;                // one stage of decoded weights
 
-// ---- raw bytes of 16 consecutive weights of a row (half `hf` of the 32-element
-// group g), and their f32 values.  Few wide loads: every lane touches a
-// different cache line, so the address path pays per instruction, not per byte.
-template <int FMT> struct Raw16;
+// ---- raw bytes of one 32-element group g of a row, and its f32 values --------
+template <int FMT> struct Raw32;
 
 // src/kernels/quant/q4_0.rs:289-306: 20-byte block = f32 scale + 16 nibble bytes
-template <> struct Raw16<RFQ_Q4_0> {
-    static constexpr int ND = 3;
+template <> struct Raw32<RFQ_Q4_0> {
+    static constexpr bool TRIP_HEADER = false;
+    static constexpr int ND = 5;
     uint32_t d[ND];
-    __device__ __forceinline__ void load(const uint8_t *row, int g, int hf)
+    __device__ __forceinline__ void load(const uint8_t *row, int g)
     {
         const uint8_t *p = row + (size_t)g * 20;
         d[0] = ld<uint32_t>(p);
-        uint2 q = ld<uint2>(p + 4 + 8 * hf);
-        d[1] = q.x; d[2] = q.y;
+        v4u q = ld<v4u>(p + 4);
+        d[1] = q[0]; d[2] = q[1]; d[3] = q[2]; d[4] = q[3];
     }
-    __device__ __forceinline__ void zero() { d[0] = 0; d[1] = d[2] = 0x88888888u; } // nibble 8 is 0.0
-    __device__ __forceinline__ float value(int e) const
+    __device__ __forceinline__ void zero() { d[0] = 0; d[1] = d[2] = d[3] = d[4] = 0x88888888u; } // nibble 8 is 0.0
+    __device__ __forceinline__ void settle(int, uint32_t) {}
+    // elements 2P and 2P+1 of the group (P = 0..15)
+    __device__ __forceinline__ void piece(int P, v8h (&h)[4]) const
     {
-        float scale = __uint_as_float(d[0]);
-        uint32_t q = (d[1 + (e >> 3)] >> (4 * (e & 7))) & 15u; // element 2i = low nibble of byte i
-        return scale * (float)((int)q - 8);
+        const float scale = __uint_as_float(d[0]);
+#pragma unroll
+        for (int e = 2 * P; e < 2 * P + 2; e++) {                  // element 2i = low nibble of byte i
+            uint32_t q = (d[1 + (e >> 3)] >> (4 * (e & 7))) & 15u;
+            h[e >> 3][e & 7] = (_Float16)(scale * (float)((int)q - 8));
+        }
     }
 };
 
 // src/kernels/quant/q8_0.rs:55-59: 36-byte block = f32 scale + 32 offset-binary bytes
-template <> struct Raw16<RFQ_Q8_0> {
-    static constexpr int ND = 5;
+template <> struct Raw32<RFQ_Q8_0> {
+    static constexpr bool TRIP_HEADER = false;
+    static constexpr int ND = 9;
     uint32_t d[ND];
-    __device__ __forceinline__ void load(const uint8_t *row, int g, int hf)
+    __device__ __forceinline__ void load(const uint8_t *row, int g)
     {
         const uint8_t *p = row + (size_t)g * 36;
         d[0] = ld<uint32_t>(p);
-        uint4 q = ld<uint4>(p + 4 + 16 * hf);
-        d[1] = q.x; d[2] = q.y; d[3] = q.z; d[4] = q.w;
+        v4u q0 = ld<v4u>(p + 4), q1 = ld<v4u>(p + 20);
+        d[1] = q0[0]; d[2] = q0[1]; d[3] = q0[2]; d[4] = q0[3];
+        d[5] = q1[0]; d[6] = q1[1]; d[7] = q1[2]; d[8] = q1[3];
     }
-    __device__ __forceinline__ void zero() { d[0] = 0; d[1] = d[2] = d[3] = d[4] = 0x80808080u; }
-    __device__ __forceinline__ float value(int e) const
+    __device__ __forceinline__ void zero()
     {
-        float scale = __uint_as_float(d[0]);
-        uint32_t b = (d[1 + (e >> 2)] >> (8 * (e & 3))) & 255u;
-        return ((float)b - 128.0f) * scale;
+        d[0] = 0;
+#pragma unroll
+        for (int i = 1; i < ND; i++) d[i] = 0x80808080u;
+    }
+    __device__ __forceinline__ void settle(int, uint32_t) {}
+    __device__ __forceinline__ void piece(int P, v8h (&h)[4]) const
+    {
+        const float scale = __uint_as_float(d[0]);
+#pragma unroll
+        for (int e = 2 * P; e < 2 * P + 2; e++) {
+            uint32_t b = (d[1 + (e >> 2)] >> (8 * (e & 3))) & 255u;
+            h[e >> 3][e & 7] = (_Float16)(((float)b - 128.0f) * scale);
+        }
     }
 };
 
 // src/kernels/quant/q4_k.rs:222-268: sub-block sb of a 256-byte super-block:
 // f16 scale at 2*sb, i8 min at 16+sb, 16 nibble bytes at 32+28*sb
-template <> struct Raw16<RFQ_Q4_K> {
-    static constexpr int ND = 3;
+template <> struct Raw32<RFQ_Q4_K> {
+    static constexpr bool TRIP_HEADER = true;                     // scales and mins are loaded once per super-block
+    static constexpr int ND = 5;
     uint32_t d[ND];
-    __device__ __forceinline__ void load(const uint8_t *row, int g, int hf)
+    __device__ __forceinline__ void load(const uint8_t *row, int g)
     {
         const uint8_t *blk = row + (size_t)(g >> 3) * 256;
         const int sb = g & 7;
-        d[0] = ld<uint32_t>(blk + 2 * (sb & ~1)) >> (16 * (sb & 1)); // the aligned dword that holds scale sb
-        uint2 q = ld<uint2>(blk + 32 + 28 * sb + 8 * hf);
-        d[1] = q.x; d[2] = q.y;
+        v4u q = ld<v4u>(blk + 32 + 28 * sb);                      // (the scale comes with the super-block's header)
+        d[1] = q[0]; d[2] = q[1]; d[3] = q[2]; d[4] = q[3];
     }
-    __device__ __forceinline__ void zero() { d[0] = d[1] = d[2] = 0; }
-    // q * scale only (exact in f32): the min is contracted separately
-    __device__ __forceinline__ float value(int e) const
+    __device__ __forceinline__ void zero() { d[0] = d[1] = d[2] = d[3] = d[4] = 0; }
+    // d[0] becomes the f16 scale in both halves; `pair` is the header dword
+    // that holds the scales of sub-blocks g & ~1 and g | 1.
+    __device__ __forceinline__ void settle(int g, uint32_t pair) { d[0] = ((pair >> (16 * (g & 1))) & 0xFFFFu) * 0x10001u; }
+    // q * scale only: the min is contracted separately.  The product of the
+    // integer q and the f16 scale is exact in f32, so rounding it to fp16 is
+    // what a single fp16 multiplication returns: two weights per instruction.
+    // Byte P of the nibble stream holds elements 2P (low) and 2P+1 (high);
+    // 0x6400 | q reads 1024 + q, 0x5400 | (q << 4) reads 64 + q.
+    __device__ __forceinline__ void piece(int P, v8h (&h)[4]) const
     {
-        float scale = f16_bits_to_f32((uint16_t)(d[0] & 0xFFFFu));
-        uint32_t q = (d[1 + (e >> 3)] >> (4 * (e & 7))) & 15u;
-        return (float)q * scale;
+        typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+        const int c = P >> 2, b = P & 3;
+        const v2h bias = {(_Float16)-1024.0f, (_Float16)-64.0f};
+        v2h s2, v;
+        __builtin_memcpy(&s2, &d[0], 4);
+        const uint32_t spread = __builtin_amdgcn_perm(0u, d[1 + c], 0x0C000C00u | (uint32_t)b | ((uint32_t)b << 16));
+        const uint32_t bits = (spread & 0x00F0000Fu) | 0x54006400u;
+        __builtin_memcpy(&v, &bits, 4);
+        v = (v + bias) * s2;
+        h[c][2 * b] = v[0];
+        h[c][2 * b + 1] = v[1];
     }
 };
 
 // src/kernels/quant/q6_k.rs:221-261: element i of a 256-byte block: f16 scale
-// 2*(i/16), signed 6-bit field at bit 6*i of the stream at +32.  16 elements =
-// one scale + 12 stream bytes.
-template <> struct Raw16<RFQ_Q6_K> {
-    static constexpr int ND = 4;
+// 2*(i/16), signed 6-bit field at bit 6*i of the stream at +32.  32 elements =
+// two scales + 24 stream bytes.
+template <> struct Raw32<RFQ_Q6_K> {
+    static constexpr bool TRIP_HEADER = false;
+    static constexpr int ND = 7;
     uint32_t d[ND];
-    __device__ __forceinline__ void load(const uint8_t *row, int g, int hf)
+    __device__ __forceinline__ void load(const uint8_t *row, int g)
     {
         const uint8_t *blk = row + (size_t)(g >> 3) * 256;
         const int s = g & 7;
-        d[0] = ld<uint32_t>(blk + 4 * s) >> (16 * hf);
-        const uint8_t *p = blk + 32 + 24 * s + 12 * hf;
-        uint2 q = ld<uint2>(p);
-        d[1] = q.x; d[2] = q.y; d[3] = ld<uint32_t>(p + 8);
+        d[0] = ld<uint32_t>(blk + 4 * s);
+        const uint8_t *p = blk + 32 + 24 * s;
+        v4u q = ld<v4u>(p);
+        uint2 r = ld<uint2>(p + 16);
+        d[1] = q[0]; d[2] = q[1]; d[3] = q[2]; d[4] = q[3]; d[5] = r.x; d[6] = r.y;
     }
-    __device__ __forceinline__ void zero() { d[0] = d[1] = d[2] = d[3] = 0; }
-    __device__ __forceinline__ float value(int e) const
+    __device__ __forceinline__ void zero()
     {
-        float scale = f16_bits_to_f32((uint16_t)(d[0] & 0xFFFFu));
-        const int bit = 6 * e, w = bit >> 5, o = bit & 31;
-        uint64_t two = (uint64_t)d[1 + w] | ((uint64_t)d[1 + (w < 2 ? w + 1 : w)] << 32);
-        return (float)sbfe6((uint32_t)(two >> o), 0) * scale;
+#pragma unroll
+        for (int i = 0; i < ND; i++) d[i] = 0;
+    }
+    __device__ __forceinline__ void settle(int, uint32_t) {}
+    __device__ __forceinline__ void piece(int P, v8h (&h)[4]) const
+    {
+#pragma unroll
+        for (int e = 2 * P; e < 2 * P + 2; e++) {
+            const float scale = f16_bits_to_f32((uint16_t)((d[0] >> (16 * (e >> 4))) & 0xFFFFu));
+            const int bit = 6 * e, w = bit >> 5, o = bit & 31;
+            uint64_t two = (uint64_t)d[1 + w] | ((uint64_t)d[1 + (w < 5 ? w + 1 : w)] << 32);
+            h[e >> 3][e & 7] = (_Float16)((float)sbfe6((uint32_t)(two >> o), 0) * scale);
+        }
     }
 };
 
-// S[m, sb] = sum of the 32 activations of sub-block sb (fp32, in k order),
-// stored as the fp16 pair (hi, lo) with hi + lo = S to 2^-22: [M][K/32][2].
+// Activations in the order the matrix instruction reads them.  Unit (mt, st)
+// = 32 rows x 64 k; inside it chunk c (0..3) of lane (fr, fh) holds
+// A[32*mt + fr][64*st + 32*fh + 8*c .. +8]: at[((mt*nst + st)*4 + c)*64 + lane]
+// in 16-byte units, so that a wavefront's load of one chunk is 1 KiB of
+// consecutive bytes.  Rows past M and k past K are zero.
+// With SUMS (K a multiple of 256) also S[m, g] = sum of the 32 activations of
+// group g (fp32, in k order) as the fp16 pair (hi, lo) with hi + lo = S to
+// 2^-22, again in operand order: the 16 bytes of lane (fr, fh) in unit
+// (mt, super-block) are the pairs of sub-blocks 4*fh .. 4*fh+3 of row 32*mt+fr.
+template <bool SUMS>
 __global__ void __launch_bounds__(256)
-group_sums_kernel(const _Float16 *__restrict__ a, _Float16 *__restrict__ s2, int M, int K)
+arrange_a_kernel(const _Float16 *__restrict__ a, v4u *__restrict__ at, _Float16 *__restrict__ s2, int M, int K,
+                 int tiles32, int nst)
 {
-    const int groups = K / 32;
-    const size_t t = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (t >= (size_t)M * groups) return;
-    const uint4 *p = reinterpret_cast<const uint4 *>(a + t * 32);
-    float sum = 0.0f;
+    const int unit = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (unit >= tiles32 * nst) return;
+    const int mt = unit / nst, st = unit % nst, fr = lane & 31, fh = lane >> 5;
+    const int m = mt * 32 + fr, k0 = st * 64 + fh * 32;
+    const bool ok = m < M && k0 < K;
+    v4u v[4];
 #pragma unroll
     for (int c = 0; c < 4; c++) {
-        uint4 v = p[c];
-        v8h h;
-        __builtin_memcpy(&h, &v, 16);
-#pragma unroll
-        for (int e = 0; e < 8; e++) sum += (float)h[e];
+        v[c] = v4u{0, 0, 0, 0};
+        if (ok) v[c] = *reinterpret_cast<const v4u *>(a + (size_t)m * K + k0 + 8 * c);
+        at[((size_t)unit * 4 + c) * 64 + lane] = v[c];
     }
-    _Float16 hi = (_Float16)sum, lo = (_Float16)(sum - (float)hi);
-    s2[2 * t] = hi;
-    s2[2 * t + 1] = lo;
+    if (SUMS && ok) {
+        float sum = 0.0f;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            v8h h;
+            __builtin_memcpy(&h, &v[c], 16);
+#pragma unroll
+            for (int e = 0; e < 8; e++) sum += (float)h[e];
+        }
+        const _Float16 hi = (_Float16)sum, lo = (_Float16)(sum - (float)hi);
+        const int g = k0 / 32, sb = g & 7;
+        const size_t t = ((((size_t)mt * (K / 256) + (g >> 3)) * 2 + (sb >> 2)) * 32 + fr) * 4 + (sb & 3);
+        s2[2 * t] = hi;
+        s2[2 * t + 1] = lo;
+    }
 }
 
 template <int FMT, bool OUT_F16>
-__global__ void __launch_bounds__(512)
-gemm_kq_kernel(const uint8_t *__restrict__ w, const _Float16 *__restrict__ a, const _Float16 *__restrict__ s2,
+__global__ void __launch_bounds__(256)
+gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const _Float16 *__restrict__ s2,
                void *__restrict__ outp, int M, int N, int K)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+#ifdef RFQ_KQ_TRACE
+    const long long tr_e = wall_clock64();
+#endif
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wave_n = wave & 1, wave_m = wave >> 1;               // 2 x 4 wavefronts
+    const int fr = lane & 31, fh = lane >> 5;                     // fragment row, k half
     const int tiles_m = (M + BM - 1) / BM;
     const int tm = blockIdx.x % tiles_m, tn = blockIdx.x / tiles_m; // the m tiles of one W tile are neighbours
     const int m0 = tm * BM, n0 = tn * BN;
@@ -190,227 +262,314 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const _Float16 *__restrict__ a, co
     const size_t row_bytes = (size_t)(K / Fmt<FMT>::BE) * Fmt<FMT>::BB;
     const int nstages = (K + BK - 1) / BK;
 
-    // this thread's share of a stage: 16 weights (row wr, group wg, half wh); 4 A chunks of 16 bytes
-    const int wr = tid >> 2, wg = (tid >> 1) & 1, wh = tid & 1;
-    const bool w_row_ok = n0 + wr < N;
-    const uint8_t *w_row = w + (size_t)(w_row_ok ? n0 + wr : 0) * row_bytes;
-    const int a_chunk = tid & 7, a_row0 = tid >> 3;               // rows a_row0 + 64*i
+    // Weights: thread t decodes group t%2 of row t/2 of each stage into LDS.
+    const int wr = tid >> 1, wh = tid & 1;
+    const uint8_t *w_row = w + (size_t)(n0 + wr < N ? n0 + wr : N - 1) * row_bytes;
+    // Activations never pass through LDS: they arrive arranged in the order
+    // the matrix instruction reads them (arrange_a_kernel), so each lane loads
+    // its 4 x 16 bytes of a stage straight into the operand registers, and a
+    // wavefront's load instruction covers 1 KiB of consecutive bytes.  k-step
+    // c of a stage is k = 32*fh + 8*c .. +8 (any assignment of k to the
+    // instruction's k slots works as long as both operands use it); the
+    // weight fragment is read from LDS at the same k.
+    const int tiles32 = (M + 31) / 32;
+    const v4u *a_tile[TI];
+#pragma unroll
+    for (int i = 0; i < TI; i++) {
+        const int mt = m0 / 32 + wave * 2 + i;
+        a_tile[i] = at + (size_t)(mt < tiles32 ? mt : tiles32 - 1) * nstages * 256 + lane;
+    }
 
-    // Global loads run four stages ahead of the arithmetic, through a ring of
-    // four register sets (indices are compile-time: the loop is unrolled by 4).
-    // (separate objects, not one array: nothing can then index the ring at run time)
-    Raw16<FMT> raw0, raw1, raw2, raw3;
-    v4u ra0[4], ra1[4], ra2[4], ra3[4];
-    auto raw_of = [&](auto slotc) -> Raw16<FMT> & {
+    // Global loads run three stages ahead of the arithmetic through a ring of
+    // four register sets (separate objects with compile-time indices: the
+    // loop is unrolled by four, so nothing can index the ring at run time).
+    // The loads are unconditional (clamped addresses): rows past M or N only
+    // feed outputs that are never stored, and k past K meets zero weights.
+    Raw32<FMT> raw0, raw1, raw2, raw3;
+    v4u ra0[TI][4], ra1[TI][4], ra2[TI][4], ra3[TI][4];
+    auto raw_of = [&](auto slotc) -> Raw32<FMT> & {
         constexpr int S = decltype(slotc)::value;
         if constexpr (S == 0) return raw0;
         else if constexpr (S == 1) return raw1;
         else if constexpr (S == 2) return raw2;
         else return raw3;
     };
-    auto ra_of = [&](auto slotc) -> v4u (&)[4] {
+    auto ra_of = [&](auto slotc) -> v4u (&)[TI][4] {
         constexpr int S = decltype(slotc)::value;
         if constexpr (S == 0) return ra0;
         else if constexpr (S == 1) return ra1;
         else if constexpr (S == 2) return ra2;
         else return ra3;
     };
-    // The loads are unconditional (clamped addresses): branches around them
-    // would make the compiler wait for every outstanding load at each join.
-    // Rows past M or N only feed outputs that are never stored; k past K is
-    // cancelled by zero weights (selected after the load), whatever finite
-    // activations the clamped address returns.
-    auto fetch = [&](auto slotc, int st) __attribute__((always_inline)) {
-        Raw16<FMT> &raw = raw_of(slotc);
-        v4u (&ra)[4] = ra_of(slotc);
-        const int g = st * 2 + wg;
-        if (!(RFQ_KQ_SKIP & 2)) raw.load(w_row, g < groups ? g : groups - 1, wh);
-        Raw16<FMT> z;
+    auto fetch_w = [&](auto slotc, int st) __attribute__((always_inline)) {
+        const int g = st * 2 + wh;
+        if (!(RFQ_KQ_SKIP & 2)) raw_of(slotc).load(w_row, g < groups ? g : groups - 1);
+    };
+    auto fetch_a = [&](auto slotc, int st, int i, int c) __attribute__((always_inline)) {
+        if (!(RFQ_KQ_SKIP & 1)) ra_of(slotc)[i][c] = a_tile[i][(size_t)(st < nstages ? st : nstages - 1) * 256 + c * 64];
+    };
+    auto fetch_a_all = [&](auto slotc, int st) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < TI; i++)
+#pragma unroll
+            for (int c = 0; c < 4; c++) fetch_a(slotc, st, i, c);
+    };
+    // groups past the end of the row become zero weights (here, not at the
+    // load: a select right behind the load would wait for it)
+    auto settle = [&](auto slotc, int st, uint32_t pair) __attribute__((always_inline)) {
+        Raw32<FMT> &raw = raw_of(slotc);
+        Raw32<FMT> z;
         z.zero();
+        raw.settle(wh, pair);                                     // (group 2*stage + wh has the parity of wh)
 #pragma unroll
-        for (int i = 0; i < Raw16<FMT>::ND; i++) raw.d[i] = g < groups ? raw.d[i] : z.d[i];
-        const int k = st * BK + a_chunk * 8, kc = k < K ? k : K - 8;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int m = m0 + a_row0 + 64 * i, mc = m < M ? m : M - 1;
-            if (!(RFQ_KQ_SKIP & 1)) ra[i] = *reinterpret_cast<const v4u *>(a + (size_t)mc * K + kc);
-        }
-    };
-    // decode + round to fp16 (registers only: free to overlap the matrix instructions)
-    auto convert = [&](auto slotc, v8h (&hw)[2]) __attribute__((always_inline)) {
-        Raw16<FMT> &raw = raw_of(slotc);
-#pragma unroll
-        for (int c = 0; c < 2; c++)
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                if (RFQ_KQ_SKIP & 16) hw[c][e] = (_Float16)(float)(raw.d[0] & 1023u);
-                else hw[c][e] = (_Float16)raw.value(8 * c + e); // round to nearest even
-            }
-    };
-    auto stash = [&](auto slotc, const v8h (&hw)[2], int buf) __attribute__((always_inline)) {
-        v4u (&ra)[4] = ra_of(slotc);
-        uint8_t *abase = lds + buf * STAGE_BYTES, *wbase = abase + A_BYTES;
-        if (RFQ_KQ_SKIP & 8) {
-            // keep the values alive without the writes (the test is never true for finite data)
-            float keep = 0.0f;
-#pragma unroll
-            for (int i = 0; i < 4; i++) keep += __uint_as_float(ra[i][0] ^ ra[i][1] ^ ra[i][2] ^ ra[i][3]);
-#pragma unroll
-            for (int c = 0; c < 2; c++)
-#pragma unroll
-                for (int e = 0; e < 8; e++) keep += (float)hw[c][e];
-            if (keep == 1.2345e-30f) *reinterpret_cast<float *>(abase) = keep;
-            return;
-        }
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-            *reinterpret_cast<v4u *>(abase + (a_row0 + 64 * i) * LDR + a_chunk * 16) = ra[i];
-#pragma unroll
-        for (int c = 0; c < 2; c++) *reinterpret_cast<v8h *>(wbase + wr * LDR + wg * 64 + wh * 32 + c * 16) = hw[c];
+        for (int i = 0; i < Raw32<FMT>::ND; i++) raw.d[i] = st * 2 + wh < groups ? raw.d[i] : z.d[i];
     };
 
-    v16f acc[2][2];
+    // Four LDS buffers of decoded weights (buffer = stage % 4, a compile-time
+    // number inside the loop body, so every LDS offset is an immediate; two
+    // base registers because an immediate reaches 64 KiB).
+    const uint8_t *rd_base[2] = {lds + fr * LDR + fh * 64, lds + 2 * W_BYTES + fr * LDR + fh * 64};
+    uint8_t *wr_base[2] = {lds + wr * LDR + wh * 64, lds + 2 * W_BYTES + wr * LDR + wh * 64};
+    auto read_frag = [&](int buf, int j, int c) __attribute__((always_inline)) -> v8h {
+        if (RFQ_KQ_SKIP & 4) {
+            v8h r;
 #pragma unroll
-    for (int j = 0; j < 2; j++)
+            for (int e = 0; e < 8; e++) r[e] = (_Float16)(float)(lane + e);
+            return r;
+        }
+        return *reinterpret_cast<const v8h *>(rd_base[buf >> 1] + (buf & 1) * W_BYTES + j * 32 * LDR + c * 16);
+    };
+    auto stash = [&](int buf, int c, const v8h (&hw)[4]) __attribute__((always_inline)) {
+        if (RFQ_KQ_SKIP & 8) {
+            if ((float)hw[c][0] + (float)hw[c][1] + (float)hw[c][2] + (float)hw[c][3] + (float)hw[c][4] + (float)hw[c][5] + (float)hw[c][6] + (float)hw[c][7] == 1.2345e-30f)
+                *reinterpret_cast<v8h *>(wr_base[0]) = hw[c];
+            return;
+        }
+        *reinterpret_cast<v8h *>(wr_base[buf >> 1] + (buf & 1) * W_BYTES + c * 16) = hw[c];
+    };
+
+    v16f acc[TJ][TI];
 #pragma unroll
-        for (int i = 0; i < 2; i++)
+    for (int j = 0; j < TJ; j++)
+#pragma unroll
+        for (int i = 0; i < TI; i++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[j][i][r] = 0.0f;
 
-    const int fr = lane & 31, fh = lane >> 5;                     // fragment row, k half
-    // Fragments of k-step ks+1 are read while the matrix instructions of k-step
-    // ks run (two register sets), so LDS latency is paid once per stage.
-    auto compute = [&](int buf) __attribute__((always_inline)) {
-        const uint8_t *abase = lds + buf * STAGE_BYTES, *wbase = abase + A_BYTES;
-        v8h fw[2][2], fa[2][2];
-        auto load_frags = [&](int ks, int set) __attribute__((always_inline)) {
-            if (RFQ_KQ_SKIP & 4) return;
+    // The Q4_K min term rides along as one extra k-step per super-block (four
+    // stages = one trip through the ring): its 16 k slots are the (hi, lo)
+    // halves of the group sums S of the super-block's 8 sub-blocks; the weight
+    // is the sub-block's min in both slots.  The thread that decodes a row's
+    // sub-blocks loads the super-block's header (8 scales, its 4 mins) with
+    // the raw bytes of the super-block's first stage (ring slot 0), keeps it
+    // in set B while decoding that super-block's first two stages and in set
+    // A for the last two (one trip later), and writes the expanded mins to a
+    // small LDS area that all wavefronts read as the weight fragment.  S
+    // comes arranged in operand order, one 16-byte load per lane and m tile,
+    // with the A registers of the trip's first stage.
+    // (Every load is consumed in the loop iteration that issued it or at a
+    // fixed compile-time distance, so the wait counts stay exact.)
+    v4u hs_ring = {0, 0, 0, 0}, hsA = {0, 0, 0, 0}, hsB = {0, 0, 0, 0};
+    uint32_t hm_ring = 0, hmA = 0, hmB = 0;
+    v4u sa_cur[TI], sa_ring[TI];
+    const v4u *s_tile[TI];
+    v8h fm[TJ];
+    constexpr int MNR = 48;                                       // bytes per row of the min area (32 used)
+    uint8_t *mn_wr = lds + 4 * W_BYTES + wr * MNR + wh * 16;
+    const uint8_t *mn_rd = lds + 4 * W_BYTES + fr * MNR + fh * 16;
+    if constexpr (FMT == RFQ_Q4_K) {
 #pragma unroll
-            for (int j = 0; j < 2; j++)
-                fw[set][j] = *reinterpret_cast<const v8h *>(wbase + (wave_n * 64 + j * 32 + fr) * LDR + ks * 32 + fh * 16);
-#pragma unroll
-            for (int i = 0; i < 2; i++)
-                fa[set][i] = *reinterpret_cast<const v8h *>(abase + (wave_m * 64 + i * 32 + fr) * LDR + ks * 32 + fh * 16);
-        };
-        if (RFQ_KQ_SKIP & 4) {
-#pragma unroll
-            for (int set = 0; set < 2; set++) {
-#pragma unroll
-                for (int j = 0; j < 2; j++)
-#pragma unroll
-                    for (int e = 0; e < 8; e++) fw[set][j][e] = (_Float16)(float)(lane + j + e);
-#pragma unroll
-                for (int i = 0; i < 2; i++)
-#pragma unroll
-                    for (int e = 0; e < 8; e++) fa[set][i][e] = (_Float16)(float)(lane + i - e);
-            }
+        for (int i = 0; i < TI; i++) {
+            const int mt = m0 / 32 + wave * 2 + i;
+            s_tile[i] = reinterpret_cast<const v4u *>(s2) + (size_t)(mt < tiles32 ? mt : tiles32 - 1) * (K / 256) * 64 + lane;
         }
-        load_frags(0, 0);
+    }
+    auto fetch_hdr = [&](int trip) __attribute__((always_inline)) {
+        if constexpr (FMT == RFQ_Q4_K) {
+            if (RFQ_KQ_SKIP & 2) return;
+            const uint8_t *blk = w_row + (size_t)(trip < K / 256 ? trip : K / 256 - 1) * 256;
+            hs_ring = ld<v4u>(blk);
+            hm_ring = ld<uint32_t>(blk + 16 + 4 * wh);
+        }
+    };
+    auto fetch_sums = [&](int trip) __attribute__((always_inline)) {
+        if constexpr (FMT == RFQ_Q4_K) {
+            if (RFQ_KQ_SKIP & 32) return;
+            const int t = trip < K / 256 ? trip : K / 256 - 1;
 #pragma unroll
-        for (int ks = 0; ks < BK / 16; ks++) {
-            if (ks + 1 < BK / 16) load_frags(ks + 1, (ks + 1) & 1);
+            for (int i = 0; i < TI; i++) sa_ring[i] = s_tile[i][(size_t)t * 64];
+        }
+    };
+    // 4 i8 mins -> 8 fp16 (each twice): 0x6400 | (min ^ 0x80) reads 1024 + 128 + min
+    auto stash_mins = [&]() __attribute__((always_inline)) {
+        typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+        const v2h bias = {(_Float16)-1152.0f, (_Float16)-1152.0f};
+        const uint32_t u = hmA ^ 0x80808080u;
+        v8h h;
 #pragma unroll
-            for (int j = 0; j < 2; j++)
+        for (int b = 0; b < 4; b++) {
+            const uint32_t bits = __builtin_amdgcn_perm(0x64646464u, u, 0x04000400u | (uint32_t)b | ((uint32_t)b << 16));
+            v2h v;
+            __builtin_memcpy(&v, &bits, 4);
+            v = v + bias;
+            h[2 * b] = v[0];
+            h[2 * b + 1] = v[1];
+        }
+        *reinterpret_cast<v8h *>(mn_wr) = h;
+    };
+    auto compute_min = [&]() __attribute__((always_inline)) {
+        if constexpr (FMT == RFQ_Q4_K) {
 #pragma unroll
-                for (int i = 0; i < 2; i++)
-                    acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[ks & 1][j], fa[ks & 1][i], acc[j][i], 0, 0, 0);
+            for (int i = 0; i < TI; i++) {
+                v8h fa;
+                __builtin_memcpy(&fa, &sa_cur[i], 16);
+#pragma unroll
+                for (int j = 0; j < TJ; j++)
+                    acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fm[j], fa, acc[j][i], 0, 0, 0);
+            }
         }
     };
 
-    // iteration st: stage st is in LDS; stage st+1 sits in register set NEXT
-    // (loaded three iterations ago); set FREE (stage st, already in LDS) takes stage st+4
-    auto iter = [&](auto nextc, auto freec, int st) __attribute__((always_inline)) {
-        v8h hw[2];
-        convert(nextc, hw);                    // (after the last stage this moves a stage nobody reads)
-        compute(st & 1);
-        stash(nextc, hw, (st + 1) & 1);
-        fetch(freec, st + 4);
+    // One wavefront per SIMD: nothing hides a stall, so the body of a stage is
+    // laid out by hand as 32 slots of one matrix instruction plus a share of
+    // the stage's other work, and pinned in that order.  Iteration st (S =
+    // st%4) multiplies stage st (LDS buffer S, A registers of ring slot S):
+    //   * weight fragments are read one k-step ahead, the last ones from the
+    //     next stage's buffer (written during the previous iteration);
+    //   * slots 0..15 decode stage st+2 (ring slot S+2), slots 16..19 write it
+    //     to buffer S+2, slot 20 refills the slot's raw registers (stage st+6);
+    //   * (Q4_K) slot 24 of a trip's first stage writes the min fragment, slots
+    //     28..31 of its last stage read it;
+    //   * the four matrix instructions that read an A chunk are followed by
+    //     the load that refills it (stage st+4).
+    // One barrier per stage: behind it stage st+2 is visible, and nobody still
+    // reads the buffer the next iteration overwrites (st+3 = st-1 mod 4).
+    v8h fw[2][TJ];
+    auto iter = [&](auto sc, int st) __attribute__((always_inline)) {
+        constexpr int S = decltype(sc)::value, S1 = (S + 1) & 3, S2 = (S + 2) & 3;
+        Raw32<FMT> &raw = raw_of(IC<S2>{});
+        v4u (&ra)[TI][4] = ra_of(sc);
+        v8h hw[4];
+        if constexpr (FMT == RFQ_Q4_K) {
+            if (S == 0) {                                          // this trip's sums arrived with stage st's A
+#pragma unroll
+                for (int i = 0; i < TI; i++) sa_cur[i] = sa_ring[i];
+                fetch_sums(st / 4 + 1);
+            }
+            if (S == 2) {                                          // stage st+2 opens the next super-block
+                // (real moves: merged with hs_ring's registers, the copy would
+                // turn into one at the end of the loop body that waits for the
+                // refill issued below)
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    uint32_t v;
+                    asm volatile("v_mov_b32 %0, %1" : "=v"(v) : "v"(hs_ring[q]));
+                    hsB[q] = v;
+                }
+                asm volatile("v_mov_b32 %0, %1" : "=v"(hmB) : "v"(hm_ring));
+            }
+        }
+        settle(IC<S2>{}, st + 2, S < 2 ? hsA[S2] : hsB[S2]);       // stage st+2 is number S2 of its super-block
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+#pragma unroll
+            for (int t = 0; t < 8; t++) {
+                const int i = t >> 2, j = t & 3, p = c * 8 + t;
+                v8h fa;
+                __builtin_memcpy(&fa, &ra[i][c], 16);
+                acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[c & 1][j], fa, acc[j][i], 0, 0, 0);
+                if (t < 4) fw[(c + 1) & 1][t] = c < 3 ? read_frag(S, t, c + 1) : read_frag(S1, t, 0);
+                if (p < 16) {
+                    if (RFQ_KQ_SKIP & 16) { hw[p >> 2][2 * (p & 3)] = (_Float16)(float)raw.d[1]; hw[p >> 2][2 * (p & 3) + 1] = (_Float16)(float)raw.d[0]; }
+                    else raw.piece(p, hw);
+                }
+                else if (p < 20) stash(S2, p - 16, hw);
+                else if (p == 20) {
+                    fetch_w(IC<S2>{}, st + 6);
+                    if (S == 2) fetch_hdr((st + 6) / 4);
+                }
+                if constexpr (FMT == RFQ_Q4_K) {
+                    // the min fragment of this trip: written in its first stage, read in its last
+                    if (S == 0 && p == 24) stash_mins();
+                    if (S == 3 && p >= 28) fm[p - 28] = *reinterpret_cast<const v8h *>(mn_rd + (p - 28) * 32 * MNR);
+                }
+                if (j == 3) fetch_a(sc, st + 4, i, c);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         lds_barrier();
     };
     {
-        v8h hw[2];
-        fetch(IC<0>{}, 0);
-        fetch(IC<1>{}, 1);
-        fetch(IC<2>{}, 2);
-        fetch(IC<3>{}, 3);
-        convert(IC<0>{}, hw);
-        stash(IC<0>{}, hw, 0);
+        v8h hw[4];
+        fetch_w(IC<0>{}, 0);
+        fetch_a_all(IC<0>{}, 0);
+        fetch_w(IC<1>{}, 1);
+        fetch_a_all(IC<1>{}, 1);
+        fetch_w(IC<2>{}, 2);
+        fetch_a_all(IC<2>{}, 2);
+        fetch_w(IC<3>{}, 3);
+        fetch_a_all(IC<3>{}, 3);
+        fetch_hdr(0);
+        fetch_sums(0);
+        hsA = hs_ring;
+        // (a real move: the loop must not inherit a pending load on hmA, or its
+        // first use in the loop body would wait for younger loads every trip)
+        asm volatile("v_mov_b32 %0, %1" : "=v"(hmA) : "v"(hm_ring));
+        settle(IC<0>{}, 0, hsA[0]);
+#pragma unroll
+        for (int p = 0; p < 16; p++) raw0.piece(p, hw);
+#pragma unroll
+        for (int c = 0; c < 4; c++) stash(0, c, hw);
+        fetch_w(IC<0>{}, 4);
+        fetch_hdr(1);
+        settle(IC<1>{}, 1, hsA[1]);
+#pragma unroll
+        for (int p = 0; p < 16; p++) raw1.piece(p, hw);
+#pragma unroll
+        for (int c = 0; c < 4; c++) stash(1, c, hw);
+        fetch_w(IC<1>{}, 5);
         lds_barrier();
+#pragma unroll
+        for (int j = 0; j < TJ; j++) fw[0][j] = read_frag(0, j, 0);
     }
-    // Whole trips through the ring only (no branch between the three bodies:
-    // the compiler would merge their tails and index the ring at run time);
+#ifdef RFQ_KQ_TRACE
+    const long long tr_c0 = clock64(), tr_w0 = wall_clock64();
+#endif
+    // Whole trips through the ring only (no branch between the four bodies);
     // stages past the end multiply zero weights.
     for (int st = 0; st < nstages; st += 4) {
-        iter(IC<1>{}, IC<0>{}, st);
-        iter(IC<2>{}, IC<1>{}, st + 1);
-        iter(IC<3>{}, IC<2>{}, st + 2);
-        iter(IC<0>{}, IC<3>{}, st + 3);
-    }
-
-    if constexpr (FMT == RFQ_Q4_K) {
-        // The min term: "k" runs over (sub-block, hi/lo) pairs, K2 = K / 16 of
-        // them; weight (n, 2*sb + t) = min[n, sb], activation (m, 2*sb + t) =
-        // hi or lo of S[m, sb].  A stage of 64 covers 32 sub-blocks = 4
-        // super-blocks; thread (wr, wg, wh) expands the 8 mins of one of them.
-        const int K2 = K / 16, nstages2 = (K2 + BK - 1) / BK;
-        uint32_t mins[2];
-        v4u (&ra)[4] = ra0;
-        auto fetch2 = [&](int st) {
-            const int sblk = st * 4 + wg * 2 + wh;                // super-block of this row
-            if (w_row_ok && sblk < K / 256) {
-                mins[0] = ld<uint32_t>(w_row + (size_t)sblk * 256 + 16);
-                mins[1] = ld<uint32_t>(w_row + (size_t)sblk * 256 + 20);
-            } else {
-                mins[0] = mins[1] = 0;
-            }
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int m = m0 + a_row0 + 64 * i, k2 = st * BK + a_chunk * 8;
-                if (m < M && k2 < K2) ra[i] = *reinterpret_cast<const v4u *>(s2 + (size_t)m * K2 + k2);
-                else ra[i] = v4u{0, 0, 0, 0};
-            }
-        };
-        auto stash2 = [&](int buf) {
-            uint8_t *abase = lds + buf * STAGE_BYTES, *wbase = abase + A_BYTES;
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-                *reinterpret_cast<v4u *>(abase + (a_row0 + 64 * i) * LDR + a_chunk * 16) = ra[i];
-#pragma unroll
-            for (int c = 0; c < 2; c++) {                          // 4 mins -> 8 fp16 (each twice)
-                v8h h;
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    _Float16 v = (_Float16)(float)(int8_t)(mins[c] >> (8 * e));
-                    h[2 * e] = v;
-                    h[2 * e + 1] = v;
-                }
-                *reinterpret_cast<v8h *>(wbase + wr * LDR + wg * 64 + wh * 32 + c * 16) = h;
-            }
-        };
-        fetch2(0);
-        stash2(0);
-        lds_barrier();
-        for (int st = 0; st < nstages2; st++) {
-            const bool more = st + 1 < nstages2;
-            if (more) fetch2(st + 1);
-            compute(st & 1);
-            if (more) stash2((st + 1) & 1);
-            lds_barrier();
+        iter(IC<0>{}, st);
+        iter(IC<1>{}, st + 1);
+        iter(IC<2>{}, st + 2);
+        iter(IC<3>{}, st + 3);
+        compute_min();
+        if constexpr (FMT == RFQ_Q4_K) {
+            hsA = hsB;
+            hmA = hmB;
         }
     }
+#ifdef RFQ_KQ_TRACE
+    if (tid == 0 && blockIdx.x == RFQ_KQ_TRACE) {
+        rfq_kq_trace_dev[0] = clock64() - tr_c0;
+        rfq_kq_trace_dev[1] = wall_clock64() - tr_w0;
+        rfq_kq_trace_dev[2] = nstages;
+        rfq_kq_trace_dev[3] = tr_w0 - tr_e;
+    }
+    const long long tr_w1 = wall_clock64();
+#endif
 
     // Register r of tile (j, i): n = 8*(r/4) + 4*(lane/32) + r%4 within the
     // tile (four consecutive n per r/4), m = lane%32.
     const bool vec_ok = (N % 4) == 0 && (reinterpret_cast<uintptr_t>(outp) & 15u) == 0;
 #pragma unroll
-    for (int j = 0; j < 2; j++)
+    for (int j = 0; j < TJ; j++)
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
-            const int m = m0 + wave_m * 64 + i * 32 + fr;
+        for (int i = 0; i < TI; i++) {
+            const int m = m0 + wave * 64 + i * 32 + fr;
             if (m >= M) continue;
 #pragma unroll
             for (int g = 0; g < 4; g++) {
-                const int n = n0 + wave_n * 64 + j * 32 + 8 * g + 4 * fh;
+                const int n = n0 + j * 32 + 8 * g + 4 * fh;
                 const size_t o = (size_t)m * N + n;
                 if (vec_ok && n + 3 < N) {
                     if (OUT_F16) {
@@ -432,12 +591,16 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const _Float16 *__restrict__ a, co
                 }
             }
         }
+#ifdef RFQ_KQ_TRACE
+    __builtin_amdgcn_s_waitcnt(0);
+    if (tid == 0 && blockIdx.x == RFQ_KQ_TRACE) rfq_kq_trace_dev[4] = wall_clock64() - tr_w1;
+#endif
 }
 
 template <int FMT, bool OUT_F16>
 int launch_cfg(const uint8_t *w, const void *a, void *out, int m, int n, int k, hipStream_t s)
 {
-    constexpr int LDS = 2 * STAGE_BYTES;
+    constexpr int LDS = 4 * W_BYTES + BN * 48;                  // four weight stages + the Q4_K min fragment
     static_assert(LDS <= 160 * 1024, "LDS budget");
     static std::once_flag once;
     static hipError_t attr_err = hipSuccess;
@@ -447,19 +610,21 @@ int launch_cfg(const uint8_t *w, const void *a, void *out, int m, int n, int k, 
     });
     if (attr_err != hipSuccess) return hip_fail(attr_err, "hipFuncSetAttribute(gemm_kq_kernel)");
     const int tiles = ((m + BM - 1) / BM) * ((n + BN - 1) / BN);
-    _Float16 *s2 = nullptr;
-    if (FMT == RFQ_Q4_K) {
-        // stream-ordered temporary: allocation and release are queued like the kernels
-        RFQ_HIP(hipMallocAsync(reinterpret_cast<void **>(&s2), (size_t)m * (k / 16) * sizeof(_Float16), s));
-        const size_t threads = (size_t)m * (k / 32);
-        hipLaunchKernelGGL(group_sums_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s,
-                           reinterpret_cast<const _Float16 *>(a), s2, m, k);
-    }
-    hipLaunchKernelGGL((gemm_kq_kernel<FMT, OUT_F16>), dim3(tiles), dim3(512), LDS, s, w,
-                       reinterpret_cast<const _Float16 *>(a), s2, out, m, n, k);
+    // stream-ordered temporary (allocation and release are queued like the
+    // kernels): the arranged activations, then the Q4_K group sums
+    const int tiles32 = (m + 31) / 32, nst = (k + BK - 1) / BK;
+    const size_t at_bytes = (size_t)tiles32 * nst * 4096;
+    const size_t s2_bytes = FMT == RFQ_Q4_K ? (size_t)tiles32 * (k / 256) * 1024 : 0;
+    uint8_t *tmp = nullptr;
+    RFQ_HIP(hipMallocAsync(reinterpret_cast<void **>(&tmp), at_bytes + s2_bytes, s));
+    v4u *at = reinterpret_cast<v4u *>(tmp);
+    _Float16 *s2 = reinterpret_cast<_Float16 *>(tmp + at_bytes);
+    hipLaunchKernelGGL((arrange_a_kernel<FMT == RFQ_Q4_K>), dim3((unsigned)((tiles32 * nst + 3) / 4)), dim3(256), 0, s,
+                       reinterpret_cast<const _Float16 *>(a), at, s2, m, k, tiles32, nst);
+    hipLaunchKernelGGL((gemm_kq_kernel<FMT, OUT_F16>), dim3(tiles), dim3(256), LDS, s, w, at, s2, out, m, n, k);
     hipError_t launch_err = hipGetLastError();
-    if (s2) {
-        hipError_t free_err = hipFreeAsync(s2, s);
+    {
+        hipError_t free_err = hipFreeAsync(tmp, s);
         if (launch_err == hipSuccess) launch_err = free_err;
     }
     if (launch_err != hipSuccess) return hip_fail(launch_err, "gemm_kq_kernel");
