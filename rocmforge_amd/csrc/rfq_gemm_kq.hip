@@ -76,9 +76,12 @@ template <> struct Raw32<RFQ_Q4_0> {
     static constexpr bool TRIP_HEADER = false;
     static constexpr int ND = 5;
     uint32_t d[ND];
-    __device__ __forceinline__ void load(const uint8_t *row, int g)
+    // group 2*st + wh of the row at `base + row_off` (base and st are the
+    // same for the whole wavefront: the address is a scalar plus a 32-bit
+    // lane offset, without 64-bit vector arithmetic)
+    __device__ __forceinline__ void load(const uint8_t *base, uint32_t row_off, int st, int wh)
     {
-        const uint8_t *p = row + (size_t)g * 20;
+        const uint8_t *p = base + (size_t)st * 40 + (row_off + 20u * wh);
         d[0] = ld<uint32_t>(p);
         v4u q = ld<v4u>(p + 4);
         d[1] = q[0]; d[2] = q[1]; d[3] = q[2]; d[4] = q[3];
@@ -102,9 +105,9 @@ template <> struct Raw32<RFQ_Q8_0> {
     static constexpr bool TRIP_HEADER = false;
     static constexpr int ND = 9;
     uint32_t d[ND];
-    __device__ __forceinline__ void load(const uint8_t *row, int g)
+    __device__ __forceinline__ void load(const uint8_t *base, uint32_t row_off, int st, int wh)
     {
-        const uint8_t *p = row + (size_t)g * 36;
+        const uint8_t *p = base + (size_t)st * 72 + (row_off + 36u * wh);
         d[0] = ld<uint32_t>(p);
         v4u q0 = ld<v4u>(p + 4), q1 = ld<v4u>(p + 20);
         d[1] = q0[0]; d[2] = q0[1]; d[3] = q0[2]; d[4] = q0[3];
@@ -134,11 +137,10 @@ template <> struct Raw32<RFQ_Q4_K> {
     static constexpr bool TRIP_HEADER = true;                     // scales and mins are loaded once per super-block
     static constexpr int ND = 5;
     uint32_t d[ND];
-    __device__ __forceinline__ void load(const uint8_t *row, int g)
+    __device__ __forceinline__ void load(const uint8_t *base, uint32_t row_off, int st, int wh)
     {
-        const uint8_t *blk = row + (size_t)(g >> 3) * 256;
-        const int sb = g & 7;
-        v4u q = ld<v4u>(blk + 32 + 28 * sb);                      // (the scale comes with the super-block's header)
+        const uint8_t *blk = base + (size_t)(st >> 2) * 256 + 56 * (st & 3) + 32;
+        v4u q = ld<v4u>(blk + (row_off + 28u * wh));         // (the scale comes with the super-block's header)
         d[1] = q[0]; d[2] = q[1]; d[3] = q[2]; d[4] = q[3];
     }
     __device__ __forceinline__ void zero() { d[0] = d[1] = d[2] = d[3] = d[4] = 0; }
@@ -158,7 +160,10 @@ template <> struct Raw32<RFQ_Q4_K> {
         v2h s2, v;
         __builtin_memcpy(&s2, &d[0], 4);
         const uint32_t spread = __builtin_amdgcn_perm(0u, d[1 + c], 0x0C000C00u | (uint32_t)b | ((uint32_t)b << 16));
-        const uint32_t bits = (spread & 0x00F0000Fu) | 0x54006400u;
+        uint32_t mask = 0x00F0000Fu, magic = 0x54006400u;
+        asm("" : "+s"(mask));                                      // (register operands: and + or in one instruction)
+        asm("" : "+v"(magic));
+        const uint32_t bits = (spread & mask) | magic;
         __builtin_memcpy(&v, &bits, 4);
         v = (v + bias) * s2;
         h[c][2 * b] = v[0];
@@ -173,12 +178,11 @@ template <> struct Raw32<RFQ_Q6_K> {
     static constexpr bool TRIP_HEADER = false;
     static constexpr int ND = 7;
     uint32_t d[ND];
-    __device__ __forceinline__ void load(const uint8_t *row, int g)
+    __device__ __forceinline__ void load(const uint8_t *base, uint32_t row_off, int st, int wh)
     {
-        const uint8_t *blk = row + (size_t)(g >> 3) * 256;
-        const int s = g & 7;
-        d[0] = ld<uint32_t>(blk + 4 * s);
-        const uint8_t *p = blk + 32 + 24 * s;
+        const uint8_t *blk = base + (size_t)(st >> 2) * 256;
+        d[0] = ld<uint32_t>(blk + 8 * (st & 3) + (row_off + 4u * wh));
+        const uint8_t *p = blk + 32 + 48 * (st & 3) + (row_off + 24u * wh);
         v4u q = ld<v4u>(p);
         uint2 r = ld<uint2>(p + 16);
         d[1] = q[0]; d[2] = q[1]; d[3] = q[2]; d[4] = q[3]; d[5] = r.x; d[6] = r.y;
@@ -264,7 +268,9 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
 
     // Weights: thread t decodes group t%2 of row t/2 of each stage into LDS.
     const int wr = tid >> 1, wh = tid & 1;
-    const uint8_t *w_row = w + (size_t)(n0 + wr < N ? n0 + wr : N - 1) * row_bytes;
+    // (addresses are a wavefront-uniform pointer plus a 32-bit lane offset)
+    const uint8_t *w_tile = w + (size_t)n0 * row_bytes;
+    const uint32_t w_off = (uint32_t)((n0 + wr < N ? wr : N - 1 - n0) * (int)row_bytes);
     // Activations never pass through LDS: they arrive arranged in the order
     // the matrix instruction reads them (arrange_a_kernel), so each lane loads
     // its 4 x 16 bytes of a stage straight into the operand registers, and a
@@ -273,11 +279,16 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
     // instruction's k slots works as long as both operands use it); the
     // weight fragment is read from LDS at the same k.
     const int tiles32 = (M + 31) / 32;
-    const v4u *a_tile[TI];
+    // (buffer loads: a scalar descriptor per m tile, the stage as scalar
+    // offset, the lane as 32-bit vector offset; no 64-bit vector arithmetic)
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const uint32_t lane16 = lane * 16;
+    __amdgpu_buffer_rsrc_t a_tile[TI];
 #pragma unroll
     for (int i = 0; i < TI; i++) {
-        const int mt = m0 / 32 + wave * 2 + i;
-        a_tile[i] = at + (size_t)(mt < tiles32 ? mt : tiles32 - 1) * nstages * 256 + lane;
+        const int mt = m0 / 32 + wave_u * 2 + i;
+        a_tile[i] = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<v4u *>(at + (size_t)(mt < tiles32 ? mt : tiles32 - 1) * nstages * 256), 0, nstages * 4096, 0x00020000);
     }
 
     // Global loads run three stages ahead of the arithmetic through a ring of
@@ -302,11 +313,15 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
         else return ra3;
     };
     auto fetch_w = [&](auto slotc, int st) __attribute__((always_inline)) {
-        const int g = st * 2 + wh;
-        if (!(RFQ_KQ_SKIP & 2)) raw_of(slotc).load(w_row, g < groups ? g : groups - 1);
+        // the last stage of a row with an odd number of groups has no second
+        // group: both lanes of the row then read the first (zeroed when decoded)
+        const int sc = st < nstages ? st : nstages - 1;
+        const int whc = Fmt<FMT>::BE == 32 && sc * 2 + 1 >= groups ? 0 : wh;
+        if (!(RFQ_KQ_SKIP & 2)) raw_of(slotc).load(w_tile, w_off, sc, whc);
     };
     auto fetch_a = [&](auto slotc, int st, int i, int c) __attribute__((always_inline)) {
-        if (!(RFQ_KQ_SKIP & 1)) ra_of(slotc)[i][c] = a_tile[i][(size_t)(st < nstages ? st : nstages - 1) * 256 + c * 64];
+        const int sc = st < nstages ? st : nstages - 1;
+        if (!(RFQ_KQ_SKIP & 1)) ra_of(slotc)[i][c] = __builtin_amdgcn_raw_buffer_load_b128(a_tile[i], lane16 + c * 1024, sc * 4096, 0);
     };
     auto fetch_a_all = [&](auto slotc, int st) __attribute__((always_inline)) {
 #pragma unroll
@@ -372,7 +387,7 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
     v4u hs_ring = {0, 0, 0, 0}, hsA = {0, 0, 0, 0}, hsB = {0, 0, 0, 0};
     uint32_t hm_ring = 0, hmA = 0, hmB = 0;
     v4u sa_cur[TI], sa_ring[TI];
-    const v4u *s_tile[TI];
+    __amdgpu_buffer_rsrc_t s_tile[TI];
     v8h fm[TJ];
     constexpr int MNR = 48;                                       // bytes per row of the min area (32 used)
     uint8_t *mn_wr = lds + 4 * W_BYTES + wr * MNR + wh * 16;
@@ -380,14 +395,16 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
     if constexpr (FMT == RFQ_Q4_K) {
 #pragma unroll
         for (int i = 0; i < TI; i++) {
-            const int mt = m0 / 32 + wave * 2 + i;
-            s_tile[i] = reinterpret_cast<const v4u *>(s2) + (size_t)(mt < tiles32 ? mt : tiles32 - 1) * (K / 256) * 64 + lane;
+            const int mt = m0 / 32 + wave_u * 2 + i;
+            s_tile[i] = __builtin_amdgcn_make_buffer_rsrc(
+                const_cast<uint8_t *>(reinterpret_cast<const uint8_t *>(s2)) + (size_t)(mt < tiles32 ? mt : tiles32 - 1) * (K / 256) * 1024,
+                0, (K / 256) * 1024, 0x00020000);
         }
     }
     auto fetch_hdr = [&](int trip) __attribute__((always_inline)) {
         if constexpr (FMT == RFQ_Q4_K) {
             if (RFQ_KQ_SKIP & 2) return;
-            const uint8_t *blk = w_row + (size_t)(trip < K / 256 ? trip : K / 256 - 1) * 256;
+            const uint8_t *blk = w_tile + (size_t)(trip < K / 256 ? trip : K / 256 - 1) * 256 + w_off;
             hs_ring = ld<v4u>(blk);
             hm_ring = ld<uint32_t>(blk + 16 + 4 * wh);
         }
@@ -397,7 +414,7 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
             if (RFQ_KQ_SKIP & 32) return;
             const int t = trip < K / 256 ? trip : K / 256 - 1;
 #pragma unroll
-            for (int i = 0; i < TI; i++) sa_ring[i] = s_tile[i][(size_t)t * 64];
+            for (int i = 0; i < TI; i++) sa_ring[i] = __builtin_amdgcn_raw_buffer_load_b128(s_tile[i], lane16, t * 1024, 0);
         }
     };
     // 4 i8 mins -> 8 fp16 (each twice): 0x6400 | (min ^ 0x80) reads 1024 + 128 + min
@@ -436,8 +453,11 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
     // st%4) multiplies stage st (LDS buffer S, A registers of ring slot S):
     //   * weight fragments are read one k-step ahead, the last ones from the
     //     next stage's buffer (written during the previous iteration);
-    //   * slots 0..15 decode stage st+2 (ring slot S+2), slots 16..19 write it
-    //     to buffer S+2, slot 20 refills the slot's raw registers (stage st+6);
+    //   * decoding runs at an even pace, one piece (two weights) every other
+    //     slot: the second half of stage st+2 in slots 0..14, the first half
+    //     of stage st+3 in slots 16..30 (two sets of fp16 registers, by stage
+    //     parity); stage st+2 goes to LDS buffer S+2 in slots 17..23, and slot
+    //     25 refills its raw registers (stage st+6);
     //   * (Q4_K) slot 24 of a trip's first stage writes the min fragment, slots
     //     28..31 of its last stage read it;
     //   * the four matrix instructions that read an A chunk are followed by
@@ -445,18 +465,20 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
     // One barrier per stage: behind it stage st+2 is visible, and nobody still
     // reads the buffer the next iteration overwrites (st+3 = st-1 mod 4).
     v8h fw[2][TJ];
+    v8h hw_even[4], hw_odd[4];                                    // decoded weights of the even / odd stage in progress
     auto iter = [&](auto sc, int st) __attribute__((always_inline)) {
-        constexpr int S = decltype(sc)::value, S1 = (S + 1) & 3, S2 = (S + 2) & 3;
-        Raw32<FMT> &raw = raw_of(IC<S2>{});
+        constexpr int S = decltype(sc)::value, S1 = (S + 1) & 3, S2 = (S + 2) & 3, S3 = (S + 3) & 3;
+        Raw32<FMT> &raw_late = raw_of(IC<S2>{}), &raw_early = raw_of(IC<S3>{});
+        v8h (&hw_late)[4] = (S & 1) ? hw_odd : hw_even;
+        v8h (&hw_early)[4] = (S & 1) ? hw_even : hw_odd;
         v4u (&ra)[TI][4] = ra_of(sc);
-        v8h hw[4];
         if constexpr (FMT == RFQ_Q4_K) {
             if (S == 0) {                                          // this trip's sums arrived with stage st's A
 #pragma unroll
                 for (int i = 0; i < TI; i++) sa_cur[i] = sa_ring[i];
                 fetch_sums(st / 4 + 1);
             }
-            if (S == 2) {                                          // stage st+2 opens the next super-block
+            if (S == 1) {                                          // stage st+3 opens the next super-block
                 // (real moves: merged with hs_ring's registers, the copy would
                 // turn into one at the end of the loop body that waits for the
                 // refill issued below)
@@ -469,7 +491,6 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
                 asm volatile("v_mov_b32 %0, %1" : "=v"(hmB) : "v"(hm_ring));
             }
         }
-        settle(IC<S2>{}, st + 2, S < 2 ? hsA[S2] : hsB[S2]);       // stage st+2 is number S2 of its super-block
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int c = 0; c < 4; c++)
@@ -480,12 +501,16 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
                 __builtin_memcpy(&fa, &ra[i][c], 16);
                 acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[c & 1][j], fa, acc[j][i], 0, 0, 0);
                 if (t < 4) fw[(c + 1) & 1][t] = c < 3 ? read_frag(S, t, c + 1) : read_frag(S1, t, 0);
-                if (p < 16) {
-                    if (RFQ_KQ_SKIP & 16) { hw[p >> 2][2 * (p & 3)] = (_Float16)(float)raw.d[1]; hw[p >> 2][2 * (p & 3) + 1] = (_Float16)(float)raw.d[0]; }
-                    else raw.piece(p, hw);
+                if (!(RFQ_KQ_SKIP & 16)) {
+                    if (p < 16 && (p & 1) == 0) raw_late.piece(8 + p / 2, hw_late);
+                    if (p >= 16 && (p & 1) == 0) raw_early.piece((p - 16) / 2, hw_early);
                 }
-                else if (p < 20) stash(S2, p - 16, hw);
-                else if (p == 20) {
+#ifdef RFQ_KQ_THROTTLE
+                if (p == 15 || p == 31) __builtin_amdgcn_s_waitcnt((RFQ_KQ_THROTTLE & 15) | ((RFQ_KQ_THROTTLE >> 4) << 14) | 0x0F70);
+#endif
+                if (p == 15) settle(IC<S3>{}, st + 3, S == 0 ? hsA[3] : hsB[S3]);   // stage st+3 is number S3 of its super-block
+                if (p >= 17 && p <= 23 && (p & 1)) stash(S2, (p - 17) / 2, hw_late);
+                if (p == 25) {
                     fetch_w(IC<S2>{}, st + 6);
                     if (S == 2) fetch_hdr((st + 6) / 4);
                 }
@@ -501,6 +526,15 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
     };
     {
         v8h hw[4];
+        // (the loads the loop consumes first in each trip go out first here too:
+        // the wait counts of the loop are the smaller of those seen on the two
+        // ways into it)
+        fetch_hdr(1);
+        fetch_sums(0);
+        if constexpr (FMT == RFQ_Q4_K) {
+            hsA = ld<v4u>(w_tile + w_off);
+            hmA = ld<uint32_t>(w_tile + (w_off + 16 + 4 * wh));
+        }
         fetch_w(IC<0>{}, 0);
         fetch_a_all(IC<0>{}, 0);
         fetch_w(IC<1>{}, 1);
@@ -509,25 +543,24 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
         fetch_a_all(IC<2>{}, 2);
         fetch_w(IC<3>{}, 3);
         fetch_a_all(IC<3>{}, 3);
-        fetch_hdr(0);
-        fetch_sums(0);
-        hsA = hs_ring;
         // (a real move: the loop must not inherit a pending load on hmA, or its
         // first use in the loop body would wait for younger loads every trip)
-        asm volatile("v_mov_b32 %0, %1" : "=v"(hmA) : "v"(hm_ring));
+        asm volatile("v_mov_b32 %0, %1" : "=v"(hmA) : "v"(hmA));
         settle(IC<0>{}, 0, hsA[0]);
 #pragma unroll
         for (int p = 0; p < 16; p++) raw0.piece(p, hw);
 #pragma unroll
         for (int c = 0; c < 4; c++) stash(0, c, hw);
         fetch_w(IC<0>{}, 4);
-        fetch_hdr(1);
         settle(IC<1>{}, 1, hsA[1]);
 #pragma unroll
         for (int p = 0; p < 16; p++) raw1.piece(p, hw);
 #pragma unroll
         for (int c = 0; c < 4; c++) stash(1, c, hw);
         fetch_w(IC<1>{}, 5);
+        settle(IC<2>{}, 2, hsA[2]);
+#pragma unroll
+        for (int p = 0; p < 8; p++) raw2.piece(p, hw_even);
         lds_barrier();
 #pragma unroll
         for (int j = 0; j < TJ; j++) fw[0][j] = read_frag(0, j, 0);
