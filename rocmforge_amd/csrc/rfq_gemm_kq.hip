@@ -13,25 +13,42 @@
 // small q * scale: rounding the sum to fp16 would lose the small part's bits.
 // The two parts are therefore contracted separately:
 //   sum_k fp16(q_k * scale) * a_k  +  sum_sb min_sb * S_sb,   S_sb = sum of a over sub-block sb,
-// the second as a short extra k loop over (min, S) pairs with S split into
-// fp16 hi + lo (exact to 2^-22; min is exact in fp16).  S comes from a small
-// pass over A into a stream-ordered temporary of M * K / 16 fp16 values.
+// the second as one extra k-step per super-block over (min, S) pairs with S
+// split into fp16 hi + lo (exact to 2^-22; min is exact in fp16).
 //
-// Workgroup tile 256 (m) x 128 (n), k advances 64 per stage, two LDS stages.
-// 512 threads; thread t decodes 16 weights of a stage (row t/4, 32-element
-// group (t/2)%2, half t%2): half a Q4_0/Q8_0 block or half a Q4_K/Q6_K
-// sub-block.  Eight wavefronts in a 2 (n) x 4 (m) arrangement, two per SIMD
-// (one runs matrix instructions while the other decodes and moves data), each
-// 64 n x 64 m = 2 x 2 instruction tiles.  The weight fragment is the
-// instruction's first operand, so a lane ends up with 4 consecutive n of one
-// output row: 8- or 16-byte stores without a transpose.
+// Two kernels per call.  arrange_a_kernel rewrites the activations into the
+// order the matrix instruction reads them (and computes S for Q4_K), into a
+// temporary the library keeps per stream.  gemm_kq_kernel: workgroup tile 256
+// (m) x 128 (n), k advances 64 per stage, 256 threads = one wavefront per
+// SIMD, each 64 m x 128 n = 2 x 4 instruction tiles (the weight fragment is
+// the instruction's first operand, so a lane ends up with 4 consecutive n of
+// one output row).
+//   * Activations go global -> registers, straight into the operand registers:
+//     1 KiB of consecutive bytes per wavefront load, four stages ahead.  They
+//     never touch LDS, whose bandwidth the weight fragments need.
+//   * Weights: thread t decodes the 32-element group t%2 of row t/2 of a
+//     stage (a Q4_0/Q8_0 block, a Q4_K/Q6_K sub-block) from raw bytes loaded
+//     four stages ahead, two stages before its use, into one of four LDS
+//     buffers; every wavefront reads all four weight fragments of a k-step
+//     from there.
+//   * One wavefront per SIMD means nothing hides a stall: the body of a stage
+//     is laid out by hand, one matrix instruction per slot with its share of
+//     loads, decode steps and LDS traffic, and pinned in that order.
+// Measured on this layout: the matrix pipe alone (same instruction mix, no
+// other work) runs at about 35 clocks per instruction at a shader clock that
+// power management holds near 1.5-1.7 GHz under this load; the loop runs at
+// about 43.
 #include <mutex>
+#include <unordered_map>
+#include <type_traits>
 
 #include "rfq_common.hpp"
 
 // -DRFQ_KQ_SKIP=<mask> (tuning builds, results are wrong on purpose): leave out
 // 1 the A loads, 2 the W loads, 4 the LDS fragment reads, 8 the LDS writes,
-// 16 the weight decoding, to see what a stage's time is made of.
+// 16 the weight decoding, 32 the Q4_K group-sum loads, to see what a stage's
+// time is made of.  -DRFQ_KQ_TRACE=<workgroup> records that workgroup's loop
+// time in shader clocks and in 100 MHz ticks (rfq_kq_trace reads them back).
 #ifndef RFQ_KQ_SKIP
 #define RFQ_KQ_SKIP 0
 #endif
@@ -49,6 +66,7 @@ namespace {
 
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
+typedef uint32_t v2u __attribute__((ext_vector_type(2)));
 typedef uint32_t v4u __attribute__((ext_vector_type(4))); // 16 bytes in flight (a builtin vector: plain loads and stores)
 template <int N> struct IC { static constexpr int value = N; };
 
@@ -71,32 +89,46 @@ constexpr int W_BYTES = BN * LDR;                // one stage of decoded weights
 // ---- raw bytes of one 32-element group g of a row, and its f32 values --------
 template <int FMT> struct Raw32;
 
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+typedef __amdgpu_buffer_rsrc_t Rsrc;
+
+// Where element e (0..7) of an 8-element k chunk sits in the chunk as both
+// operands store it: [k0 k4 k1 k5 k2 k6 k3 k7].  Nibble pairs (k, k+4) of a
+// dword of packed 4-bit weights come out of one mask operation in that order;
+// the activations are arranged to match (any assignment of k to the matrix
+// instruction's k slots works as long as both operands use it).
+__device__ __forceinline__ constexpr int chunk_pos(int e) { return ((e & 3) << 1) | (e >> 2); }
+
+// Every format decodes a 32-element group in 12 steps (chunk c = T/3 of 8
+// elements, three steps each) so that the work can be spread evenly between
+// matrix instructions.  load() reads group 2*st + wh of the row at lane
+// offset row_off through a buffer descriptor of the weight tile: the stage
+// part of the address is scalar, the lane part a 32-bit offset.
+
 // src/kernels/quant/q4_0.rs:289-306: 20-byte block = f32 scale + 16 nibble bytes
 template <> struct Raw32<RFQ_Q4_0> {
     static constexpr bool TRIP_HEADER = false;
     static constexpr int ND = 5;
     uint32_t d[ND];
-    // group 2*st + wh of the row at `base + row_off` (base and st are the
-    // same for the whole wavefront: the address is a scalar plus a 32-bit
-    // lane offset, without 64-bit vector arithmetic)
-    __device__ __forceinline__ void load(const uint8_t *base, uint32_t row_off, int st, int wh)
+    __device__ __forceinline__ void load(Rsrc w, uint32_t row_off, int st, int wh)
     {
-        const uint8_t *p = base + (size_t)st * 40 + (row_off + 20u * wh);
-        d[0] = ld<uint32_t>(p);
-        v4u q = ld<v4u>(p + 4);
+        const uint32_t v = row_off + 20u * wh;
+        d[0] = __builtin_amdgcn_raw_buffer_load_b32(w, v, st * 40, 0);
+        v4u q = __builtin_amdgcn_raw_buffer_load_b128(w, v + 4, st * 40, 0);
         d[1] = q[0]; d[2] = q[1]; d[3] = q[2]; d[4] = q[3];
     }
     __device__ __forceinline__ void zero() { d[0] = 0; d[1] = d[2] = d[3] = d[4] = 0x88888888u; } // nibble 8 is 0.0
     __device__ __forceinline__ void settle(int, uint32_t) {}
-    // elements 2P and 2P+1 of the group (P = 0..15)
-    __device__ __forceinline__ void piece(int P, v8h (&h)[4]) const
+    __device__ __forceinline__ float value(int e) const            // element 2i = low nibble of byte i
     {
-        const float scale = __uint_as_float(d[0]);
+        uint32_t q = (d[1 + (e >> 3)] >> (4 * (e & 7))) & 15u;
+        return __uint_as_float(d[0]) * (float)((int)q - 8);
+    }
+    __device__ __forceinline__ void step(int T, v8h (&h)[4], v2h (&)[4]) const
+    {
+        const int c = T / 3, e0 = 3 * (T % 3), e1 = e0 + 3 < 8 ? e0 + 3 : 8;
 #pragma unroll
-        for (int e = 2 * P; e < 2 * P + 2; e++) {                  // element 2i = low nibble of byte i
-            uint32_t q = (d[1 + (e >> 3)] >> (4 * (e & 7))) & 15u;
-            h[e >> 3][e & 7] = (_Float16)(scale * (float)((int)q - 8));
-        }
+        for (int e = e0; e < e1; e++) h[c][chunk_pos(e)] = (_Float16)value(8 * c + e);
     }
 };
 
@@ -105,11 +137,12 @@ template <> struct Raw32<RFQ_Q8_0> {
     static constexpr bool TRIP_HEADER = false;
     static constexpr int ND = 9;
     uint32_t d[ND];
-    __device__ __forceinline__ void load(const uint8_t *base, uint32_t row_off, int st, int wh)
+    __device__ __forceinline__ void load(Rsrc w, uint32_t row_off, int st, int wh)
     {
-        const uint8_t *p = base + (size_t)st * 72 + (row_off + 36u * wh);
-        d[0] = ld<uint32_t>(p);
-        v4u q0 = ld<v4u>(p + 4), q1 = ld<v4u>(p + 20);
+        const uint32_t v = row_off + 36u * wh;
+        d[0] = __builtin_amdgcn_raw_buffer_load_b32(w, v, st * 72, 0);
+        v4u q0 = __builtin_amdgcn_raw_buffer_load_b128(w, v + 4, st * 72, 0);
+        v4u q1 = __builtin_amdgcn_raw_buffer_load_b128(w, v + 20, st * 72, 0);
         d[1] = q0[0]; d[2] = q0[1]; d[3] = q0[2]; d[4] = q0[3];
         d[5] = q1[0]; d[6] = q1[1]; d[7] = q1[2]; d[8] = q1[3];
     }
@@ -120,14 +153,16 @@ template <> struct Raw32<RFQ_Q8_0> {
         for (int i = 1; i < ND; i++) d[i] = 0x80808080u;
     }
     __device__ __forceinline__ void settle(int, uint32_t) {}
-    __device__ __forceinline__ void piece(int P, v8h (&h)[4]) const
+    __device__ __forceinline__ float value(int e) const
     {
-        const float scale = __uint_as_float(d[0]);
+        uint32_t b = (d[1 + (e >> 2)] >> (8 * (e & 3))) & 255u;
+        return ((float)b - 128.0f) * __uint_as_float(d[0]);
+    }
+    __device__ __forceinline__ void step(int T, v8h (&h)[4], v2h (&)[4]) const
+    {
+        const int c = T / 3, e0 = 3 * (T % 3), e1 = e0 + 3 < 8 ? e0 + 3 : 8;
 #pragma unroll
-        for (int e = 2 * P; e < 2 * P + 2; e++) {
-            uint32_t b = (d[1 + (e >> 2)] >> (8 * (e & 3))) & 255u;
-            h[e >> 3][e & 7] = (_Float16)(((float)b - 128.0f) * scale);
-        }
+        for (int e = e0; e < e1; e++) h[c][chunk_pos(e)] = (_Float16)value(8 * c + e);
     }
 };
 
@@ -137,10 +172,10 @@ template <> struct Raw32<RFQ_Q4_K> {
     static constexpr bool TRIP_HEADER = true;                     // scales and mins are loaded once per super-block
     static constexpr int ND = 5;
     uint32_t d[ND];
-    __device__ __forceinline__ void load(const uint8_t *base, uint32_t row_off, int st, int wh)
+    __device__ __forceinline__ void load(Rsrc w, uint32_t row_off, int st, int wh)
     {
-        const uint8_t *blk = base + (size_t)(st >> 2) * 256 + 56 * (st & 3) + 32;
-        v4u q = ld<v4u>(blk + (row_off + 28u * wh));         // (the scale comes with the super-block's header)
+        // (the scale comes with the super-block's header)
+        v4u q = __builtin_amdgcn_raw_buffer_load_b128(w, row_off + 28u * wh + 32, (st >> 2) * 256 + 56 * (st & 3), 0);
         d[1] = q[0]; d[2] = q[1]; d[3] = q[2]; d[4] = q[3];
     }
     __device__ __forceinline__ void zero() { d[0] = d[1] = d[2] = d[3] = d[4] = 0; }
@@ -150,24 +185,37 @@ template <> struct Raw32<RFQ_Q4_K> {
     // q * scale only: the min is contracted separately.  The product of the
     // integer q and the f16 scale is exact in f32, so rounding it to fp16 is
     // what a single fp16 multiplication returns: two weights per instruction.
-    // Byte P of the nibble stream holds elements 2P (low) and 2P+1 (high);
-    // 0x6400 | q reads 1024 + q, 0x5400 | (q << 4) reads 64 + q.
-    __device__ __forceinline__ void piece(int P, v8h (&h)[4]) const
+    // A dword holds nibbles k0..k7 of a chunk; 0x6400 | q reads 1024 + q and
+    // 0x5400 | (q << 4) reads 64 + q, so one and-or per pair (k0,k4), (k1,k5),
+    // and of the dword shifted by 8, (k2,k6), (k3,k7); then subtract the
+    // offset (exact) and multiply by the scale (one rounding).
+    __device__ __forceinline__ void step(int T, v8h (&h)[4], v2h (&t)[4]) const
     {
-        typedef _Float16 v2h __attribute__((ext_vector_type(2)));
-        const int c = P >> 2, b = P & 3;
-        const v2h bias = {(_Float16)-1024.0f, (_Float16)-64.0f};
-        v2h s2, v;
-        __builtin_memcpy(&s2, &d[0], 4);
-        const uint32_t spread = __builtin_amdgcn_perm(0u, d[1 + c], 0x0C000C00u | (uint32_t)b | ((uint32_t)b << 16));
-        uint32_t mask = 0x00F0000Fu, magic = 0x54006400u;
-        asm("" : "+s"(mask));                                      // (register operands: and + or in one instruction)
-        asm("" : "+v"(magic));
-        const uint32_t bits = (spread & mask) | magic;
-        __builtin_memcpy(&v, &bits, 4);
-        v = (v + bias) * s2;
-        h[c][2 * b] = v[0];
-        h[c][2 * b + 1] = v[1];
+        const int c = T / 3, ph = T % 3;
+        if (ph == 0) {
+            uint32_t m_lo = 0x000F000Fu, m_hi = 0x00F000F0u, g_lo = 0x64006400u, g_hi = 0x54005400u;
+            asm("" : "+s"(m_lo));                                  // (register operands: and + or in one instruction)
+            asm("" : "+s"(m_hi));
+            asm("" : "+v"(g_lo));
+            asm("" : "+v"(g_hi));
+            const uint32_t x = d[1 + c], y = x >> 8;
+            const uint32_t b[4] = {(x & m_lo) | g_lo, (x & m_hi) | g_hi, (y & m_lo) | g_lo, (y & m_hi) | g_hi};
+#pragma unroll
+            for (int q = 0; q < 4; q++) __builtin_memcpy(&t[q], &b[q], 4);
+        } else if (ph == 1) {
+            const v2h b_lo = {(_Float16)-1024.0f, (_Float16)-1024.0f}, b_hi = {(_Float16)-64.0f, (_Float16)-64.0f};
+#pragma unroll
+            for (int q = 0; q < 4; q++) t[q] = t[q] + ((q & 1) ? b_hi : b_lo);
+        } else {
+            v2h s2;
+            __builtin_memcpy(&s2, &d[0], 4);
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const v2h v = t[q] * s2;
+                h[c][2 * q] = v[0];
+                h[c][2 * q + 1] = v[1];
+            }
+        }
     }
 };
 
@@ -178,14 +226,14 @@ template <> struct Raw32<RFQ_Q6_K> {
     static constexpr bool TRIP_HEADER = false;
     static constexpr int ND = 7;
     uint32_t d[ND];
-    __device__ __forceinline__ void load(const uint8_t *base, uint32_t row_off, int st, int wh)
+    __device__ __forceinline__ void load(Rsrc w, uint32_t row_off, int st, int wh)
     {
-        const uint8_t *blk = base + (size_t)(st >> 2) * 256;
-        d[0] = ld<uint32_t>(blk + 8 * (st & 3) + (row_off + 4u * wh));
-        const uint8_t *p = blk + 32 + 48 * (st & 3) + (row_off + 24u * wh);
-        v4u q = ld<v4u>(p);
-        uint2 r = ld<uint2>(p + 16);
-        d[1] = q[0]; d[2] = q[1]; d[3] = q[2]; d[4] = q[3]; d[5] = r.x; d[6] = r.y;
+        const int blk = (st >> 2) * 256;
+        d[0] = __builtin_amdgcn_raw_buffer_load_b32(w, row_off + 4u * wh, blk + 8 * (st & 3), 0);
+        const uint32_t v = row_off + 24u * wh + 32;
+        v4u q = __builtin_amdgcn_raw_buffer_load_b128(w, v, blk + 48 * (st & 3), 0);
+        v2u r = __builtin_amdgcn_raw_buffer_load_b64(w, v + 16, blk + 48 * (st & 3), 0);
+        d[1] = q[0]; d[2] = q[1]; d[3] = q[2]; d[4] = q[3]; d[5] = r[0]; d[6] = r[1];
     }
     __device__ __forceinline__ void zero()
     {
@@ -193,23 +241,27 @@ template <> struct Raw32<RFQ_Q6_K> {
         for (int i = 0; i < ND; i++) d[i] = 0;
     }
     __device__ __forceinline__ void settle(int, uint32_t) {}
-    __device__ __forceinline__ void piece(int P, v8h (&h)[4]) const
+    __device__ __forceinline__ float value(int e) const
     {
+        const float scale = f16_bits_to_f32((uint16_t)((d[0] >> (16 * (e >> 4))) & 0xFFFFu));
+        const int bit = 6 * e, w = bit >> 5, o = bit & 31;
+        uint64_t two = (uint64_t)d[1 + w] | ((uint64_t)d[1 + (w < 5 ? w + 1 : w)] << 32);
+        return (float)sbfe6((uint32_t)(two >> o), 0) * scale;
+    }
+    __device__ __forceinline__ void step(int T, v8h (&h)[4], v2h (&)[4]) const
+    {
+        const int c = T / 3, e0 = 3 * (T % 3), e1 = e0 + 3 < 8 ? e0 + 3 : 8;
 #pragma unroll
-        for (int e = 2 * P; e < 2 * P + 2; e++) {
-            const float scale = f16_bits_to_f32((uint16_t)((d[0] >> (16 * (e >> 4))) & 0xFFFFu));
-            const int bit = 6 * e, w = bit >> 5, o = bit & 31;
-            uint64_t two = (uint64_t)d[1 + w] | ((uint64_t)d[1 + (w < 5 ? w + 1 : w)] << 32);
-            h[e >> 3][e & 7] = (_Float16)((float)sbfe6((uint32_t)(two >> o), 0) * scale);
-        }
+        for (int e = e0; e < e1; e++) h[c][chunk_pos(e)] = (_Float16)value(8 * c + e);
     }
 };
 
 // Activations in the order the matrix instruction reads them.  Unit (mt, st)
 // = 32 rows x 64 k; inside it chunk c (0..3) of lane (fr, fh) holds
-// A[32*mt + fr][64*st + 32*fh + 8*c .. +8]: at[((mt*nst + st)*4 + c)*64 + lane]
-// in 16-byte units, so that a wavefront's load of one chunk is 1 KiB of
-// consecutive bytes.  Rows past M and k past K are zero.
+// A[32*mt + fr][64*st + 32*fh + 8*c .. +8] in the order of chunk_pos():
+// at[((mt*nst + st)*4 + c)*64 + lane] in 16-byte units, so that a wavefront's
+// load of one chunk is 1 KiB of consecutive bytes.  Rows past M and k past K
+// are zero.
 // With SUMS (K a multiple of 256) also S[m, g] = sum of the 32 activations of
 // group g (fp32, in k order) as the fp16 pair (hi, lo) with hi + lo = S to
 // 2^-22, again in operand order: the 16 bytes of lane (fr, fh) in unit
@@ -219,19 +271,38 @@ __global__ void __launch_bounds__(256)
 arrange_a_kernel(const _Float16 *__restrict__ a, v4u *__restrict__ at, _Float16 *__restrict__ s2, int M, int K,
                  int tiles32, int nst)
 {
-    const int unit = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
-    if (unit >= tiles32 * nst) return;
-    const int mt = unit / nst, st = unit % nst, fr = lane & 31, fh = lane >> 5;
+    // A workgroup takes 32 rows x 256 k (four units): whole 512-byte row pieces
+    // come in with consecutive lanes on consecutive bytes, and a wavefront per
+    // unit reads its operand order back out of LDS.
+    constexpr int ROWB = 512 + 16;                                // row stride = 4 banks mod 32
+    __shared__ __attribute__((aligned(16))) uint8_t stage[32 * ROWB];
+    const int groups4 = (nst + 3) / 4;
+    const int mt = blockIdx.x / groups4, st0 = (blockIdx.x % groups4) * 4;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+        const int row = p * 8 + (tid >> 5), col = tid & 31;       // 16-byte column of the 512-byte piece
+        const int m = mt * 32 + row, k = st0 * 64 + col * 8;
+        v4u v = {0, 0, 0, 0};
+        if (m < M && k < K) v = *reinterpret_cast<const v4u *>(a + (size_t)m * K + k);
+        *reinterpret_cast<v4u *>(stage + row * ROWB + col * 16) = v;
+    }
+    __syncthreads();
+    const int st = st0 + wave;
+    if (st >= nst) return;
+    const int fr = lane & 31, fh = lane >> 5;
     const int m = mt * 32 + fr, k0 = st * 64 + fh * 32;
-    const bool ok = m < M && k0 < K;
+    const size_t unit = (size_t)mt * nst + st;
     v4u v[4];
 #pragma unroll
     for (int c = 0; c < 4; c++) {
-        v[c] = v4u{0, 0, 0, 0};
-        if (ok) v[c] = *reinterpret_cast<const v4u *>(a + (size_t)m * K + k0 + 8 * c);
-        at[((size_t)unit * 4 + c) * 64 + lane] = v[c];
+        v[c] = *reinterpret_cast<const v4u *>(stage + fr * ROWB + wave * 128 + fh * 64 + c * 16);
+        // dwords (k0 k1)(k2 k3)(k4 k5)(k6 k7) -> (k0 k4)(k1 k5)(k2 k6)(k3 k7)
+        const v4u p = {__builtin_amdgcn_perm(v[c][2], v[c][0], 0x05040100u), __builtin_amdgcn_perm(v[c][2], v[c][0], 0x07060302u),
+                       __builtin_amdgcn_perm(v[c][3], v[c][1], 0x05040100u), __builtin_amdgcn_perm(v[c][3], v[c][1], 0x07060302u)};
+        at[(unit * 4 + c) * 64 + lane] = p;
     }
-    if (SUMS && ok) {
+    if (SUMS && m < M && k0 < K) {
         float sum = 0.0f;
 #pragma unroll
         for (int c = 0; c < 4; c++) {
@@ -268,8 +339,10 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
 
     // Weights: thread t decodes group t%2 of row t/2 of each stage into LDS.
     const int wr = tid >> 1, wh = tid & 1;
-    // (addresses are a wavefront-uniform pointer plus a 32-bit lane offset)
-    const uint8_t *w_tile = w + (size_t)n0 * row_bytes;
+    // (a buffer descriptor from the tile's first row to the end of W, plus a 32-bit lane offset)
+    const size_t w_left = (size_t)(N - n0) * row_bytes;
+    const Rsrc w_tile = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(w) + (size_t)n0 * row_bytes, 0,
+                                                          w_left < 0xFFFFFFFFu ? (int)(uint32_t)w_left : -1, 0x00020000);
     const uint32_t w_off = (uint32_t)((n0 + wr < N ? wr : N - 1 - n0) * (int)row_bytes);
     // Activations never pass through LDS: they arrive arranged in the order
     // the matrix instruction reads them (arrange_a_kernel), so each lane loads
@@ -404,9 +477,9 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
     auto fetch_hdr = [&](int trip) __attribute__((always_inline)) {
         if constexpr (FMT == RFQ_Q4_K) {
             if (RFQ_KQ_SKIP & 2) return;
-            const uint8_t *blk = w_tile + (size_t)(trip < K / 256 ? trip : K / 256 - 1) * 256 + w_off;
-            hs_ring = ld<v4u>(blk);
-            hm_ring = ld<uint32_t>(blk + 16 + 4 * wh);
+            const int blk = (trip < K / 256 ? trip : K / 256 - 1) * 256;
+            hs_ring = __builtin_amdgcn_raw_buffer_load_b128(w_tile, w_off, blk, 0);
+            hm_ring = __builtin_amdgcn_raw_buffer_load_b32(w_tile, w_off + 16 + 4 * wh, blk, 0);
         }
     };
     auto fetch_sums = [&](int trip) __attribute__((always_inline)) {
@@ -453,9 +526,9 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
     // st%4) multiplies stage st (LDS buffer S, A registers of ring slot S):
     //   * weight fragments are read one k-step ahead, the last ones from the
     //     next stage's buffer (written during the previous iteration);
-    //   * decoding runs at an even pace, one piece (two weights) every other
-    //     slot: the second half of stage st+2 in slots 0..14, the first half
-    //     of stage st+3 in slots 16..30 (two sets of fp16 registers, by stage
+    //   * decoding runs at an even pace, six of a group's twelve steps in
+    //     slots 0..13 (second half of stage st+2) and six in slots 16..29
+    //     (first half of stage st+3; two sets of fp16 registers, by stage
     //     parity); stage st+2 goes to LDS buffer S+2 in slots 17..23, and slot
     //     25 refills its raw registers (stage st+6);
     //   * (Q4_K) slot 24 of a trip's first stage writes the min fragment, slots
@@ -466,6 +539,7 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
     // reads the buffer the next iteration overwrites (st+3 = st-1 mod 4).
     v8h fw[2][TJ];
     v8h hw_even[4], hw_odd[4];                                    // decoded weights of the even / odd stage in progress
+    v2h dec_tmp[4];                                               // a chunk between its decode steps
     auto iter = [&](auto sc, int st) __attribute__((always_inline)) {
         constexpr int S = decltype(sc)::value, S1 = (S + 1) & 3, S2 = (S + 2) & 3, S3 = (S + 3) & 3;
         Raw32<FMT> &raw_late = raw_of(IC<S2>{}), &raw_early = raw_of(IC<S3>{});
@@ -502,12 +576,13 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
                 acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[c & 1][j], fa, acc[j][i], 0, 0, 0);
                 if (t < 4) fw[(c + 1) & 1][t] = c < 3 ? read_frag(S, t, c + 1) : read_frag(S1, t, 0);
                 if (!(RFQ_KQ_SKIP & 16)) {
-                    if (p < 16 && (p & 1) == 0) raw_late.piece(8 + p / 2, hw_late);
-                    if (p >= 16 && (p & 1) == 0) raw_early.piece((p - 16) / 2, hw_early);
+                    constexpr int LATE[6] = {0, 3, 5, 8, 10, 13}, EARLY[6] = {16, 18, 20, 22, 26, 29};
+#pragma unroll
+                    for (int q = 0; q < 6; q++) {
+                        if (p == LATE[q]) raw_late.step(6 + q, hw_late, dec_tmp);
+                        if (p == EARLY[q]) raw_early.step(q, hw_early, dec_tmp);
+                    }
                 }
-#ifdef RFQ_KQ_THROTTLE
-                if (p == 15 || p == 31) __builtin_amdgcn_s_waitcnt((RFQ_KQ_THROTTLE & 15) | ((RFQ_KQ_THROTTLE >> 4) << 14) | 0x0F70);
-#endif
                 if (p == 15) settle(IC<S3>{}, st + 3, S == 0 ? hsA[3] : hsB[S3]);   // stage st+3 is number S3 of its super-block
                 if (p >= 17 && p <= 23 && (p & 1)) stash(S2, (p - 17) / 2, hw_late);
                 if (p == 25) {
@@ -532,8 +607,8 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
         fetch_hdr(1);
         fetch_sums(0);
         if constexpr (FMT == RFQ_Q4_K) {
-            hsA = ld<v4u>(w_tile + w_off);
-            hmA = ld<uint32_t>(w_tile + (w_off + 16 + 4 * wh));
+            hsA = __builtin_amdgcn_raw_buffer_load_b128(w_tile, w_off, 0, 0);
+            hmA = __builtin_amdgcn_raw_buffer_load_b32(w_tile, w_off + 16 + 4 * wh, 0, 0);
         }
         fetch_w(IC<0>{}, 0);
         fetch_a_all(IC<0>{}, 0);
@@ -548,19 +623,19 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
         asm volatile("v_mov_b32 %0, %1" : "=v"(hmA) : "v"(hmA));
         settle(IC<0>{}, 0, hsA[0]);
 #pragma unroll
-        for (int p = 0; p < 16; p++) raw0.piece(p, hw);
+        for (int T = 0; T < 12; T++) raw0.step(T, hw, dec_tmp);
 #pragma unroll
         for (int c = 0; c < 4; c++) stash(0, c, hw);
         fetch_w(IC<0>{}, 4);
         settle(IC<1>{}, 1, hsA[1]);
 #pragma unroll
-        for (int p = 0; p < 16; p++) raw1.piece(p, hw);
+        for (int T = 0; T < 12; T++) raw1.step(T, hw, dec_tmp);
 #pragma unroll
         for (int c = 0; c < 4; c++) stash(1, c, hw);
         fetch_w(IC<1>{}, 5);
         settle(IC<2>{}, 2, hsA[2]);
 #pragma unroll
-        for (int p = 0; p < 8; p++) raw2.piece(p, hw_even);
+        for (int T = 0; T < 6; T++) raw2.step(T, hw_even, dec_tmp);
         lds_barrier();
 #pragma unroll
         for (int j = 0; j < TJ; j++) fw[0][j] = read_frag(0, j, 0);
@@ -593,6 +668,51 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
 
     // Register r of tile (j, i): n = 8*(r/4) + 4*(lane/32) + r%4 within the
     // tile (four consecutive n per r/4), m = lane%32.
+    //
+    // Whole tiles leave through LDS (free now: the loop ended on a barrier),
+    // 32 rows of a wavefront at a time in an area of its own, so that each
+    // output row goes out as full 16-byte pieces of consecutive n instead of 8-
+    // or 16-byte pieces one row apart.
+    typedef typename std::conditional<OUT_F16, _Float16, float>::type OutT;
+    constexpr int ROWB = BN * (int)sizeof(OutT) + 16;             // bytes per staged row (row stride = 4 banks mod 32)
+    static_assert(4 * 32 * ROWB <= 4 * W_BYTES, "staging area");
+    if (m0 + BM <= M && n0 + BN <= N && (N * sizeof(OutT)) % 16 == 0 && (reinterpret_cast<uintptr_t>(outp) & 15u) == 0) {
+        uint8_t *area = lds + wave * (32 * ROWB);
+        constexpr int CPR = BN * (int)sizeof(OutT) / 16, RPI = 64 / CPR; // 16-byte chunks per row, rows per store instruction
+        const int chunk = lane % CPR, row_l = lane / CPR;
+#pragma unroll
+        for (int i = 0; i < TI; i++) {
+#pragma unroll
+            for (int j = 0; j < TJ; j++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    uint8_t *dst = area + fr * ROWB + (j * 32 + 8 * g + 4 * fh) * (int)sizeof(OutT);
+                    if (OUT_F16) {
+                        typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+                        *reinterpret_cast<v4h *>(dst) = v4h{(_Float16)acc[j][i][4 * g], (_Float16)acc[j][i][4 * g + 1],
+                                                            (_Float16)acc[j][i][4 * g + 2], (_Float16)acc[j][i][4 * g + 3]};
+                    } else {
+                        typedef float v4f __attribute__((ext_vector_type(4)));
+                        *reinterpret_cast<v4f *>(dst) = v4f{acc[j][i][4 * g], acc[j][i][4 * g + 1], acc[j][i][4 * g + 2], acc[j][i][4 * g + 3]};
+                    }
+                }
+            // (the area belongs to this wavefront alone, and a wavefront's LDS
+            // operations complete in order: no barrier between write and read)
+#pragma unroll
+            for (int it = 0; it < 32 / RPI; it++) {
+                const int row = it * RPI + row_l;
+                const v4u v = *reinterpret_cast<const v4u *>(area + row * ROWB + chunk * 16);
+                uint8_t *o = reinterpret_cast<uint8_t *>(outp) +
+                             ((size_t)(m0 + wave * 64 + i * 32 + row) * N + n0) * sizeof(OutT) + chunk * 16;
+                __builtin_nontemporal_store(v, reinterpret_cast<v4u *>(o));
+            }
+        }
+#ifdef RFQ_KQ_TRACE
+        __builtin_amdgcn_s_waitcnt(0);
+        if (tid == 0 && blockIdx.x == RFQ_KQ_TRACE) rfq_kq_trace_dev[4] = wall_clock64() - tr_w1;
+#endif
+        return;
+    }
     const bool vec_ok = (N % 4) == 0 && (reinterpret_cast<uintptr_t>(outp) & 15u) == 0;
 #pragma unroll
     for (int j = 0; j < TJ; j++)
@@ -630,6 +750,39 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
 #endif
 }
 
+// Temporary device memory for one call.  Up to WS_KEEP bytes it is a buffer
+// the library keeps per stream (calls on one stream run in order, so the next
+// call may overwrite it; different streams get different buffers) and frees
+// only when a larger one is needed: a stream-ordered allocation and release
+// around every call costs about 6 us of idle GPU between calls.  Larger
+// requests are allocated and released in stream order, per call.
+constexpr size_t WS_KEEP = (size_t)64 << 20;
+struct Kept { uint8_t *ptr; size_t bytes; int device; };
+std::mutex ws_mutex;
+std::unordered_map<hipStream_t, Kept> ws_kept;
+
+int workspace(hipStream_t s, size_t bytes, uint8_t **out, bool *transient)
+{
+    if (bytes > WS_KEEP) {
+        *transient = true;
+        RFQ_HIP(hipMallocAsync(reinterpret_cast<void **>(out), bytes, s));
+        return RFQ_OK;
+    }
+    *transient = false;
+    int device = 0;
+    RFQ_HIP(hipGetDevice(&device));
+    std::lock_guard<std::mutex> lock(ws_mutex);
+    Kept &kept = ws_kept[s];
+    if (kept.ptr == nullptr || kept.bytes < bytes || kept.device != device) {
+        if (kept.ptr != nullptr && kept.device == device) RFQ_HIP(hipFree(kept.ptr)); // (waits for the work that uses it)
+        kept = Kept{nullptr, 0, device};
+        RFQ_HIP(hipMalloc(reinterpret_cast<void **>(&kept.ptr), bytes));
+        kept.bytes = bytes;
+    }
+    *out = kept.ptr;
+    return RFQ_OK;
+}
+
 template <int FMT, bool OUT_F16>
 int launch_cfg(const uint8_t *w, const void *a, void *out, int m, int n, int k, hipStream_t s)
 {
@@ -643,20 +796,20 @@ int launch_cfg(const uint8_t *w, const void *a, void *out, int m, int n, int k, 
     });
     if (attr_err != hipSuccess) return hip_fail(attr_err, "hipFuncSetAttribute(gemm_kq_kernel)");
     const int tiles = ((m + BM - 1) / BM) * ((n + BN - 1) / BN);
-    // stream-ordered temporary (allocation and release are queued like the
-    // kernels): the arranged activations, then the Q4_K group sums
+    // the temporary: the arranged activations, then the Q4_K group sums
     const int tiles32 = (m + 31) / 32, nst = (k + BK - 1) / BK;
     const size_t at_bytes = (size_t)tiles32 * nst * 4096;
     const size_t s2_bytes = FMT == RFQ_Q4_K ? (size_t)tiles32 * (k / 256) * 1024 : 0;
     uint8_t *tmp = nullptr;
-    RFQ_HIP(hipMallocAsync(reinterpret_cast<void **>(&tmp), at_bytes + s2_bytes, s));
+    bool transient = false;
+    if (int rc = workspace(s, at_bytes + s2_bytes, &tmp, &transient)) return rc;
     v4u *at = reinterpret_cast<v4u *>(tmp);
     _Float16 *s2 = reinterpret_cast<_Float16 *>(tmp + at_bytes);
-    hipLaunchKernelGGL((arrange_a_kernel<FMT == RFQ_Q4_K>), dim3((unsigned)((tiles32 * nst + 3) / 4)), dim3(256), 0, s,
+    hipLaunchKernelGGL((arrange_a_kernel<FMT == RFQ_Q4_K>), dim3((unsigned)(tiles32 * ((nst + 3) / 4))), dim3(256), 0, s,
                        reinterpret_cast<const _Float16 *>(a), at, s2, m, k, tiles32, nst);
     hipLaunchKernelGGL((gemm_kq_kernel<FMT, OUT_F16>), dim3(tiles), dim3(256), LDS, s, w, at, s2, out, m, n, k);
     hipError_t launch_err = hipGetLastError();
-    {
+    if (transient) {
         hipError_t free_err = hipFreeAsync(tmp, s);
         if (launch_err == hipSuccess) launch_err = free_err;
     }
