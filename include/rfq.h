@@ -140,7 +140,10 @@ RFQ_API int rfq_matmul_host_weights(int fmt, const uint8_t *h_w, size_t w_bytes,
 /* d_out[m, n] = d_a[m, k] (fp16) . dequant(W)[n, k]^T on the fp16 matrix
  * cores with fp32 accumulation; out_dtype is RFQ_F32 or RFQ_F16.  Formats:
  * Q4_0, Q8_0, Q4_K, Q6_K.  k a multiple of 256 for the K-formats, of 32
- * otherwise.  The reference has no fused prefill GEMM (its matmul_q* hard-wire
+ * otherwise; d_a_f16 16-byte aligned, d_w 4-byte aligned.  Up to 64 MiB of
+ * temporary device memory (the activations in matrix-operand order) is kept
+ * per stream between calls; larger temporaries are allocated and released in
+ * stream order.  The reference has no fused prefill GEMM (its matmul_q* hard-wire
  * m = 1, src/kernels/matmul/quantized/q4_0.rs:169; larger m goes through
  * dequantise + hipBLAS SGEMM, src/tensor/matmul.rs:134-214); this is the same
  * contraction. */

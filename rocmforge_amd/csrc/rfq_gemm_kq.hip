@@ -833,6 +833,8 @@ int launch_gemm_f16(int fmt, const uint8_t *d_w, const void *d_a, void *d_out, i
         return fail(RFQ_E_BADARG, "rfq_gemm_f16: out_dtype %d (want RFQ_F32 or RFQ_F16)", out_dtype);
     if ((reinterpret_cast<uintptr_t>(d_a) & 15u) != 0 || k % 8 != 0)
         return fail(RFQ_E_BADARG, "rfq_gemm_f16: activations must be 16-byte aligned with k a multiple of 8");
+    if ((reinterpret_cast<uintptr_t>(d_w) & 3u) != 0)               // buffer loads of whole dwords
+        return fail(RFQ_E_BADARG, "rfq_gemm_f16: weights must be 4-byte aligned");
     switch (fmt) {
     case RFQ_Q4_0: return launch_fmt<RFQ_Q4_0>(d_w, d_a, d_out, out_dtype, m, n, k, s);
     case RFQ_Q8_0: return launch_fmt<RFQ_Q8_0>(d_w, d_a, d_out, out_dtype, m, n, k, s);
