@@ -57,6 +57,10 @@ int hip_fail(hipError_t e, const char *what);
     } while (0)
 
 int device_cu_count();
+// Temporary device memory for one call on stream s: a buffer the library keeps
+// per stream for modest sizes (*transient = false: leave it alone), a
+// stream-ordered allocation the caller releases with hipFreeAsync otherwise.
+int workspace(hipStream_t s, size_t bytes, uint8_t **out, bool *transient);
 
 // ---- launchers implemented per .hip file -----------------------------------
 int launch_dequant(int fmt, const uint8_t *d_in, size_t in_bytes, float *d_out, size_t n, hipStream_t s);

@@ -750,39 +750,6 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
 #endif
 }
 
-// Temporary device memory for one call.  Up to WS_KEEP bytes it is a buffer
-// the library keeps per stream (calls on one stream run in order, so the next
-// call may overwrite it; different streams get different buffers) and frees
-// only when a larger one is needed: a stream-ordered allocation and release
-// around every call costs about 6 us of idle GPU between calls.  Larger
-// requests are allocated and released in stream order, per call.
-constexpr size_t WS_KEEP = (size_t)64 << 20;
-struct Kept { uint8_t *ptr; size_t bytes; int device; };
-std::mutex ws_mutex;
-std::unordered_map<hipStream_t, Kept> ws_kept;
-
-int workspace(hipStream_t s, size_t bytes, uint8_t **out, bool *transient)
-{
-    if (bytes > WS_KEEP) {
-        *transient = true;
-        RFQ_HIP(hipMallocAsync(reinterpret_cast<void **>(out), bytes, s));
-        return RFQ_OK;
-    }
-    *transient = false;
-    int device = 0;
-    RFQ_HIP(hipGetDevice(&device));
-    std::lock_guard<std::mutex> lock(ws_mutex);
-    Kept &kept = ws_kept[s];
-    if (kept.ptr == nullptr || kept.bytes < bytes || kept.device != device) {
-        if (kept.ptr != nullptr && kept.device == device) RFQ_HIP(hipFree(kept.ptr)); // (waits for the work that uses it)
-        kept = Kept{nullptr, 0, device};
-        RFQ_HIP(hipMalloc(reinterpret_cast<void **>(&kept.ptr), bytes));
-        kept.bytes = bytes;
-    }
-    *out = kept.ptr;
-    return RFQ_OK;
-}
-
 template <int FMT, bool OUT_F16>
 int launch_cfg(const uint8_t *w, const void *a, void *out, int m, int n, int k, hipStream_t s)
 {
@@ -825,6 +792,41 @@ int launch_fmt(const uint8_t *w, const void *a, void *out, int out_dtype, int m,
 }
 
 } // namespace
+
+// Temporary device memory for one call.  Up to WS_KEEP bytes it is a buffer
+// the library keeps per stream (calls on one stream run in order, so the next
+// call may overwrite it; different streams get different buffers) and frees
+// only when a larger one is needed: a stream-ordered allocation and release
+// around every call costs about 6 us of idle GPU between calls.  Larger
+// requests are allocated and released in stream order, per call.
+namespace {
+constexpr size_t WS_KEEP = (size_t)64 << 20;
+struct Kept { uint8_t *ptr; size_t bytes; int device; };
+std::mutex ws_mutex;
+std::unordered_map<hipStream_t, Kept> ws_kept;
+} // namespace
+
+int workspace(hipStream_t s, size_t bytes, uint8_t **out, bool *transient)
+{
+    if (bytes > WS_KEEP) {
+        *transient = true;
+        RFQ_HIP(hipMallocAsync(reinterpret_cast<void **>(out), bytes, s));
+        return RFQ_OK;
+    }
+    *transient = false;
+    int device = 0;
+    RFQ_HIP(hipGetDevice(&device));
+    std::lock_guard<std::mutex> lock(ws_mutex);
+    Kept &kept = ws_kept[s];
+    if (kept.ptr == nullptr || kept.bytes < bytes || kept.device != device) {
+        if (kept.ptr != nullptr && kept.device == device) RFQ_HIP(hipFree(kept.ptr)); // (waits for the work that uses it)
+        kept = Kept{nullptr, 0, device};
+        RFQ_HIP(hipMalloc(reinterpret_cast<void **>(&kept.ptr), bytes));
+        kept.bytes = bytes;
+    }
+    *out = kept.ptr;
+    return RFQ_OK;
+}
 
 int launch_gemm_f16(int fmt, const uint8_t *d_w, const void *d_a, void *d_out, int out_dtype, int m, int n, int k,
                     hipStream_t s)

@@ -783,6 +783,158 @@ gemv_idot_batch_kernel(const uint8_t *__restrict__ w, const float *__restrict__ 
     }
 }
 
+// ---- 2 <= m <= 8, Q8_0: the batch through the matrix cores ----------------------
+//
+// With M vectors in registers the integer-dot kernel above needs more than 250
+// registers per lane, one wavefront per SIMD, and cannot keep enough loads in
+// flight to stream the matrix.  Here the M vectors are the rows of a matrix
+// operand instead: v_mfma_f32_16x16x32_f16 multiplies a 16 x 32 tile of
+// activations (vectors x one unit of k; rows 8..15 repeat rows 0..7 and their
+// results are dropped) with a 32 x 16 tile of weights (one unit of 16 rows).
+//
+// Exactness is kept as in the integer-dot scheme.  A small kernel first turns x
+// into block-fixed-point per unit and vector: a power of two s and integers
+// X_i = round(x_i / s), |X_i| <= 2^22, split as X = 2048 * hi + lo with
+// |hi| <= 2048 and 0 <= lo < 2048, both exact in fp16; the weights b - 128 are
+// exact in fp16 too, so every product and every 32-term sum is an exact
+// integer below 2^24 in the fp32 accumulator:
+//     sum_i (b_i - 128) x_i  =  s * (2048 * sum (b-128).hi + sum (b-128).lo).
+// Operand layout of the instruction: lane l holds row/column l % 16 and the
+// eight k values 8 * (l / 16) ..+8; the result's lane l holds column l % 16
+// (a weight row: the lane that loaded its bytes and its scale) and rows
+// 4 * (l / 16) ..+4 (vectors).
+//
+// A workgroup owns 16 weight rows; its 8 wavefronts take the units
+// w, w + 8, ... of those rows, sixteen at a time with all their loads issued up
+// front (64 KiB of weights in flight per CU), and add their partial results
+// through LDS.
+
+typedef _Float16 v8h_t __attribute__((ext_vector_type(8)));
+typedef _Float16 v2h_t __attribute__((ext_vector_type(2)));
+typedef float v4f_t __attribute__((ext_vector_type(4)));
+typedef uint32_t v2u_t __attribute__((ext_vector_type(2)));
+typedef uint32_t v4u_t __attribute__((ext_vector_type(4)));
+
+// parts: [unit][hi, lo][k octet 0..3][vector 0..7][8 fp16] (512 bytes per unit
+// and part; operand lane 16 * q + i reads octet q, vector i % 8); sx: [unit][8]
+// f32.  One workgroup per unit; thread t: vector t / 32, element t % 32.
+__global__ void __launch_bounds__(256)
+gemv_mfma_prep_kernel(const float *__restrict__ x, _Float16 *__restrict__ parts, float *__restrict__ sx, int m, int k)
+{
+    const int u = blockIdx.x, v = threadIdx.x >> 5, kk = threadIdx.x & 31, lane = threadIdx.x & 63;
+    const float xv = v < m ? x[(size_t)v * k + u * 32 + kk] : 0.0f;
+    float mx = fabsf(xv);
+    const bool bad = !(mx <= 3.40282347e+38f);
+    const unsigned long long bad_mask = __ballot(bad);
+    const bool any_bad = ((bad_mask >> (lane & 32)) & 0xFFFFFFFFull) != 0;
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 32));
+    const int e = (int)(__float_as_uint(mx) >> 23);   // biased exponent of the largest |x|
+    int ie = 275 - e;                                 // 1/s = 2^(21 - (e - 127))
+    if (ie > 254) ie = 254;
+    const float inv_s = __uint_as_float((uint32_t)ie << 23);
+    float sc = ie == 254 ? __uint_as_float(0x00400000u) : __uint_as_float((uint32_t)(254 - ie) << 23);
+    if (any_bad) sc = __uint_as_float(0x7FC00000u);   // a non-finite x poisons its unit, as it would a float sum
+    const int X = any_bad ? 0 : (int)(__float_as_uint(__builtin_fmaf(xv, inv_s, 12582912.0f)) - 0x4B400000u);
+    const int hi = X >> 11, lo = X & 2047;
+    const size_t at = ((size_t)u * 2 * 32 + (kk >> 3) * 8 + v) * 8 + (kk & 7);
+    parts[at] = (_Float16)(float)hi;
+    parts[at + 32 * 8] = (_Float16)(float)lo;
+    if (kk == 0) sx[u * 8 + v] = sc;
+}
+
+#ifndef RFQ_M8_SKIP
+#define RFQ_M8_SKIP 0
+#endif
+constexpr int MFMA_NB = 16;                           // units of a wavefront in flight together
+constexpr int MFMA_WAVES = 8;
+
+__global__ void __launch_bounds__(64 * MFMA_WAVES)
+gemv_mfma_q8_0_kernel(const uint8_t *__restrict__ w, const _Float16 *__restrict__ parts, const float *__restrict__ sx,
+                      float *__restrict__ y, int m, int n, int k)
+{
+    __shared__ float red[MFMA_WAVES * 16 * 8];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, j = lane & 15, q = lane >> 4;
+    const int units = k / 32, n0 = blockIdx.x * 16;
+    const int row = n0 + j < n ? n0 + j : n - 1;
+    const uint8_t *row_ptr = w + (size_t)row * units * 36;
+    // The weight bytes are fetched by four neighbouring lanes per row (32
+    // consecutive bytes: one request instead of four) and handed to the lane
+    // that holds them as an operand, lane 16 * q + j <- lane 4 * j + q.
+    const int row_c = n0 + (lane >> 2) < n ? n0 + (lane >> 2) : n - 1;
+    const uint8_t *row_ptr_c = w + (size_t)row_c * units * 36 + 4 + 8 * (lane & 3);
+    const int from_lane4 = 4 * (4 * j + q);
+    const v4u_t *parts_l = reinterpret_cast<const v4u_t *>(parts) + q * 8 + (j & 7);
+    const v2h_t bias = {(_Float16)-1152.0f, (_Float16)-1152.0f};
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int base = wave; base < units; base += MFMA_WAVES * MFMA_NB) {
+        v2u_t wq[MFMA_NB];
+        float ws[MFMA_NB];
+        v4u_t xh[MFMA_NB], xl[MFMA_NB];
+        v4f_t s4[MFMA_NB / 2];                          // (the x scales follow half a batch behind: registers)
+        auto load_s4 = [&](int b) {
+            const int u = base + MFMA_WAVES * b, uc = u < units ? u : units - 1;
+            s4[b % (MFMA_NB / 2)] = (RFQ_M8_SKIP & 4) ? v4f_t{1.f, 1.f, 1.f, 1.f} : *reinterpret_cast<const v4f_t *>(sx + uc * 8 + 4 * (q & 1));
+        };
+#pragma unroll
+        for (int b = 0; b < MFMA_NB; b++) {
+            const int u = base + MFMA_WAVES * b, uc = u < units ? u : units - 1; // (past the end: a valid unit, weight scale 0)
+            const uint8_t *blk = row_ptr + (size_t)uc * 36;
+            wq[b] = (RFQ_M8_SKIP & 1) ? v2u_t{(uint32_t)lane, (uint32_t)b} : ld<v2u_t>(row_ptr_c + (size_t)uc * 36);
+            ws[b] = (RFQ_M8_SKIP & 1) ? 1.0f : ld<float>(blk);                    // (no branch around a load: it would wait for the others)
+            xh[b] = (RFQ_M8_SKIP & 2) ? v4u_t{1u, 2u, 3u, (uint32_t)lane} : parts_l[(size_t)uc * 64];
+            xl[b] = (RFQ_M8_SKIP & 2) ? v4u_t{1u, 2u, 3u, (uint32_t)lane} : parts_l[(size_t)uc * 64 + 32];
+            if (b < MFMA_NB / 2) load_s4(b);
+        }
+        __builtin_amdgcn_sched_barrier(0);             // (every load of the batch is out before the first is used)
+#pragma unroll
+        for (int b = 0; b < MFMA_NB; b++) {
+            // bytes b0..b3 of a dword -> fp16 pairs (b0, b1), (b2, b3): 0x6400 | b reads 1024 + b
+            v4u_t wb;
+#pragma unroll
+            for (int d = 0; d < 2; d++) {
+                const uint32_t wd = (uint32_t)__builtin_amdgcn_ds_bpermute(from_lane4, (int)wq[b][d]);
+                const uint32_t p0 = __builtin_amdgcn_perm(0x64646464u, wd, 0x04010400u);
+                const uint32_t p1 = __builtin_amdgcn_perm(0x64646464u, wd, 0x04030402u);
+                v2h_t h0, h1;
+                __builtin_memcpy(&h0, &p0, 4);
+                __builtin_memcpy(&h1, &p1, 4);
+                h0 = h0 + bias;                        // 1024 + b - 1152 = b - 128
+                h1 = h1 + bias;
+                uint32_t o0, o1;
+                __builtin_memcpy(&o0, &h0, 4);
+                __builtin_memcpy(&o1, &h1, 4);
+                wb[2 * d] = o0;
+                wb[2 * d + 1] = o1;
+            }
+            v8h_t wf, ah, al;
+            __builtin_memcpy(&wf, &wb, 16);
+            __builtin_memcpy(&ah, &xh[b], 16);
+            __builtin_memcpy(&al, &xl[b], 16);
+            const v4f_t zero = {0.0f, 0.0f, 0.0f, 0.0f};
+            const v4f_t sh = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah, wf, zero, 0, 0, 0);
+            const v4f_t sl = __builtin_amdgcn_mfma_f32_16x16x32_f16(al, wf, zero, 0, 0, 0);
+            const float wsc = base + MFMA_WAVES * b < units ? ws[b] : 0.0f;
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                acc[r] = __builtin_fmaf(wsc * s4[b % (MFMA_NB / 2)][r], __builtin_fmaf(sh[r], 2048.0f, sl[r]), acc[r]);
+            if (b + MFMA_NB / 2 < MFMA_NB) load_s4(b + MFMA_NB / 2);
+        }
+    }
+    if (q < 2) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) red[(wave * 16 + j) * 8 + 4 * q + r] = acc[r];
+    }
+    __syncthreads();
+    if (tid < 128) {
+        const int jj = tid >> 3, v = tid & 7;
+        float sum = 0.0f;
+#pragma unroll
+        for (int wv = 0; wv < MFMA_WAVES; wv++) sum += red[(wv * 16 + jj) * 8 + v];
+        if (v < m && n0 + jj < n) y[(size_t)v * n + n0 + jj] = sum;
+    }
+}
+
 // ---- any m <= 8, any k: one row per wavefront ---------------------------------
 template <int FMT, int M>
 __global__ void __launch_bounds__(256)
@@ -984,6 +1136,26 @@ int run_generic(const uint8_t *w, const float *x, float *y, int n, int k, hipStr
     return RFQ_OK;
 }
 
+int run_mfma_q8_0(const uint8_t *w, const float *x, float *y, int m, int n, int k, hipStream_t s)
+{
+    const int units = k / 32;
+    const size_t parts_bytes = (size_t)units * 1024, sx_bytes = (size_t)units * 32;
+    uint8_t *tmp = nullptr;
+    bool transient = false;
+    if (int rc = workspace(s, parts_bytes + sx_bytes, &tmp, &transient)) return rc;
+    _Float16 *parts = reinterpret_cast<_Float16 *>(tmp);
+    float *sx = reinterpret_cast<float *>(tmp + parts_bytes);
+    hipLaunchKernelGGL(gemv_mfma_prep_kernel, dim3(units), dim3(256), 0, s, x, parts, sx, m, k);
+    hipLaunchKernelGGL(gemv_mfma_q8_0_kernel, dim3((n + 15) / 16), dim3(64 * MFMA_WAVES), 0, s, w, parts, sx, y, m, n, k);
+    hipError_t launch_err = hipGetLastError();
+    if (transient) {
+        hipError_t free_err = hipFreeAsync(tmp, s);
+        if (launch_err == hipSuccess) launch_err = free_err;
+    }
+    if (launch_err != hipSuccess) return hip_fail(launch_err, "gemv_mfma_q8_0_kernel");
+    return RFQ_OK;
+}
+
 template <int FMT>
 int run(const uint8_t *w, const float *x, float *y, int m, int n, int k, hipStream_t s)
 {
@@ -994,6 +1166,7 @@ int run(const uint8_t *w, const float *x, float *y, int m, int n, int k, hipStre
         if (ku <= 256) return run_idot<FMT, 2, 2>(w, x, y, n, k, s);
         if (ku <= 512) return run_idot<FMT, 2, 4>(w, x, y, n, k, s);
     }
+    if (FMT == RFQ_Q8_0 && m > 1 && (reinterpret_cast<uintptr_t>(w) & 3u) == 0) return run_mfma_q8_0(w, x, y, m, n, k, s);
     if (HasIdot<FMT>::value && m > 1 && ku > 32 && ku <= 256) {
         if (m <= 2) return run_idot_batch_k<FMT, 2>(w, x, y, m, n, k, s);
         if (m <= 4) return run_idot_batch_k<FMT, 4>(w, x, y, m, n, k, s);

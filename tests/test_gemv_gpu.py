@@ -54,6 +54,19 @@ def test_gemv_small_batches(fmt, m, oracle, cuda):
     assert_close(got, oracle.qmatmul_nk(fmt, w, x, m, n, k), f"{Q.NAMES[fmt]} m={m}")
 
 
+# Q8_0 batches run on the matrix cores: 16 rows per workgroup, 16 wavefronts
+# that take every 16th unit, eight units at a time: odd unit counts, more than
+# one trip, fewer units than wavefronts, a ragged last row tile.
+@pytest.mark.parametrize("m,n,k", [(2, 16, 96), (4, 50, 8224), (8, 33, 4096), (7, 1, 32)])
+def test_q8_0_batches_on_the_matrix_cores(m, n, k, oracle, cuda):
+    w = Q.make_weights(Q.Q8_0, n, k, seed=5100 + n)
+    x = x_for(m, k, 6100 + m)
+    x[0, ::7] *= 1000.0                                                   # outliers: per-unit scaling
+    x[m - 1, 5:40] = 0.0                                                  # an all-zero unit
+    got = gpu_gemv(Q.Q8_0, w, x, n, k, cuda)
+    assert_close(got, oracle.qmatmul_nk(Q.Q8_0, w, x, m, n, k), f"Q8_0 m={m} n={n} k={k}")
+
+
 @pytest.mark.parametrize("fmt", [Q.MXFP4, Q.MXFP6_E2M3])
 def test_gemv_mx_random_codes_and_clamp(fmt, oracle, cuda):
     # every code, exponents up to +6 so the +-8 / +-7.5 clamp is active
