@@ -72,6 +72,11 @@ typedef enum rfq_mx_kind { RFQ_MX_AUTO = 0, RFQ_MX_FP4 = 4, RFQ_MX_FP8 = 8 } rfq
 RFQ_API int rfq_version(void);
 /* Thread-local description of the last failure on this thread ("" if none). */
 RFQ_API const char *rfq_last_error(void);
+/* rfq_gemm_f16 and rfq_gemv (Q8_0, m > 1) keep up to 64 MiB of temporary
+ * device memory per stream between calls.  This frees all of it (it waits for
+ * the device first); the next call allocates again.  No counterpart in the
+ * reference, whose kernels take no temporaries. */
+RFQ_API int rfq_release_temporaries(void);
 /* Elements per block / bytes per block the decoders stride by
  * (GgufTensorType::block_size, src/loader/tensor_type.rs:77-88; strides at
  * src/kernels/quant/q4_0.rs:269, q8_0.rs:33, q4_k.rs:206, q6_k.rs:206,

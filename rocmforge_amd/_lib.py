@@ -30,6 +30,7 @@ _vp, _sz, _i = C.c_void_p, C.c_size_t, C.c_int
 _SIGNATURES = {
     "rfq_version": ([], _i),
     "rfq_last_error": ([], C.c_char_p),
+    "rfq_release_temporaries": ([], _i),
     "rfq_block_elems": ([_i], _sz),
     "rfq_block_bytes": ([_i], _sz),
     "rfq_packed_bytes": ([_i, _sz], _sz),

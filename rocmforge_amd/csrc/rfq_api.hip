@@ -79,6 +79,8 @@ int rfq_version(void) { return RFQ_VERSION; }
 
 const char *rfq_last_error(void) { return g_err; }
 
+int rfq_release_temporaries(void) { return rfq::release_workspaces(); }
+
 size_t rfq_block_elems(int fmt) { return (size_t)fmt_block_elems(fmt); }
 size_t rfq_block_bytes(int fmt) { return (size_t)fmt_block_bytes(fmt); }
 

@@ -61,6 +61,7 @@ int device_cu_count();
 // per stream for modest sizes (*transient = false: leave it alone), a
 // stream-ordered allocation the caller releases with hipFreeAsync otherwise.
 int workspace(hipStream_t s, size_t bytes, uint8_t **out, bool *transient);
+int release_workspaces();
 
 // ---- launchers implemented per .hip file -----------------------------------
 int launch_dequant(int fmt, const uint8_t *d_in, size_t in_bytes, float *d_out, size_t n, hipStream_t s);

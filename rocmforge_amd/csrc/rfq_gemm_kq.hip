@@ -828,6 +828,27 @@ int workspace(hipStream_t s, size_t bytes, uint8_t **out, bool *transient)
     return RFQ_OK;
 }
 
+int release_workspaces()
+{
+    std::lock_guard<std::mutex> lock(ws_mutex);
+    if (ws_kept.empty()) return RFQ_OK;
+    RFQ_HIP(hipDeviceSynchronize());
+    int current = 0;
+    RFQ_HIP(hipGetDevice(&current));
+    hipError_t first = hipSuccess;
+    for (auto &entry : ws_kept) {
+        if (entry.second.ptr == nullptr) continue;
+        hipError_t e = hipSetDevice(entry.second.device);
+        if (e == hipSuccess) e = hipFree(entry.second.ptr);
+        if (first == hipSuccess) first = e;
+    }
+    ws_kept.clear();
+    hipError_t back = hipSetDevice(current);
+    if (first == hipSuccess) first = back;
+    if (first != hipSuccess) return hip_fail(first, "rfq_release_temporaries");
+    return RFQ_OK;
+}
+
 int launch_gemm_f16(int fmt, const uint8_t *d_w, const void *d_a, void *d_out, int out_dtype, int m, int n, int k,
                     hipStream_t s)
 {

@@ -102,6 +102,12 @@ def test_weights_at_a_4_byte_offset_and_kept_temporary(oracle, cuda):
         assert_close(out.cpu().numpy(), oracle.qmatmul_nk(fmt, w, a.astype(np.float32), m, n, k), f"{m}x{n}x{k}")
         outs.append(out.cpu().numpy())
     assert np.array_equal(outs[0], outs[2])
+    from rocmforge_amd import _lib
+    assert _lib.lib().rfq_release_temporaries() == _lib.OK               # the next call allocates again
+    w, a = weights(fmt, 128, 512, 6), acts(64, 512, 7)
+    again = ops.gemm_f16(fmt, torch.from_numpy(w).to(cuda), torch.from_numpy(a).to(cuda), 128, 512, out_dtype=torch.float32)
+    torch.cuda.synchronize()
+    assert np.array_equal(again.cpu().numpy(), outs[0])
 
 
 def test_rejects_bad_arguments(cuda):
