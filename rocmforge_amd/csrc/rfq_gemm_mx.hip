@@ -94,9 +94,10 @@ template <int FMT> __device__ __forceinline__ void decode_block(const uint8_t *b
 template <> __device__ __forceinline__ void decode_block<RFQ_MXFP4>(const uint8_t *blk, float (&v)[32])
 {
     float scale = mx_scale((int)(int8_t)blk[0]);
+    const v4i q = ld<v4i>(blk + 1);                   // one 16-byte load (any alignment) instead of 16 byte loads
 #pragma unroll
     for (int j = 0; j < 16; j++) {
-        uint32_t b = blk[1 + j];
+        uint32_t b = ((uint32_t)q[j >> 2] >> (8 * (j & 3))) & 255u;
         v[2 * j] = clampf(scale * decode_e2m1(b >> 4), -8.0f, 8.0f);
         v[2 * j + 1] = clampf(scale * decode_e2m1(b & 15u), -8.0f, 8.0f);
     }

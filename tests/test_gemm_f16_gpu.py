@@ -110,6 +110,20 @@ def test_weights_at_a_4_byte_offset_and_kept_temporary(oracle, cuda):
     assert np.array_equal(again.cpu().numpy(), outs[0])
 
 
+def test_temporary_larger_than_the_kept_size(oracle, cuda):
+    """m * k * 2 bytes above 64 MiB: the arranged activations go to a stream-ordered
+    allocation that is released after the call."""
+    import torch
+    from rocmforge_amd import ops
+    fmt, m, n, k = Q.Q4_K, 4096, 128, 8448
+    w, a = weights(fmt, n, k, 8), acts(m, k, 9)
+    out = ops.gemm_f16(fmt, torch.from_numpy(w).to(cuda), torch.from_numpy(a).to(cuda), n, k, out_dtype=torch.float32)
+    torch.cuda.synchronize()
+    cols = np.array([0, 5, 31, 32, 100, 127])
+    want = oracle.qmatmul_nk(fmt, w, a.astype(np.float32), m, n, k, rows=cols)
+    assert_close(out[:, torch.from_numpy(cols).to(cuda)].cpu().numpy(), want, "large temporary")
+
+
 def test_rejects_bad_arguments(cuda):
     import torch
     from rocmforge_amd import _lib, ops
