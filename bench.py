@@ -45,7 +45,10 @@ def time_gemv(torch, fmt, n, k, m, copies, steps, warmup, Q, seed):
 
     from rocmforge_amd import _lib
     dev = torch.device("cuda:0")
-    w = Q.make_weights(fmt, n, k, seed=seed)
+    slab = 4008 if n > 32768 and n % 4008 == 0 else n   # a vocabulary-sized matrix: quantise a slab, repeat it down the rows
+    w = Q.make_weights(fmt, slab, k, seed=seed)
+    if slab != n:
+        w = np.tile(w, n // slab)
     rng = np.random.Generator(np.random.PCG64(seed + 1))
     x = rng.standard_normal((m, k), dtype=np.float32)
     dws = [torch.from_numpy(w).to(dev) for _ in range(copies)]
@@ -88,6 +91,30 @@ def time_dequant(torch, fmt, n, k, steps, warmup, Q, seed):
     _lib.check(L.rfq_bench_dequant(fmt, ptrs, copies, w.size, C.c_void_p(out.data_ptr()), n * k, 0, steps, stream,
                                    C.byref(ms)))
     return ms.value / 1e3 / steps, w.size + 4 * n * k
+
+
+def time_get_rows(torch, fmt, n_vocab, n_embd, n_tokens, Q):
+    """Embedding gather: n_tokens rows of a packed [n_vocab, n_embd] table, token ids on the device."""
+    import numpy as np
+
+    from rocmforge_amd import ops
+    dev = torch.device("cuda:0")
+    slab = 4008
+    tab = torch.from_numpy(np.tile(Q.make_weights(fmt, slab, n_embd, seed=20260033), n_vocab // slab)).to(dev)
+    rng = np.random.Generator(np.random.PCG64(20260034))
+    tok = torch.from_numpy(rng.integers(0, n_vocab, size=n_tokens).astype(np.int32)).to(dev)
+    for _ in range(5):
+        ops.get_rows(fmt, tab, tok, n_vocab, n_embd)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(50):
+        ops.get_rows(fmt, tab, tok, n_vocab, n_embd)
+    e1.record()
+    torch.cuda.synchronize()
+    t = e0.elapsed_time(e1) / 50 * 1e-3
+    b = n_tokens * (n_embd * 4 + Q.packed_bytes(fmt, n_embd))
+    return {"us": round(t * 1e6, 2), "GB/s": round(b / t / 1e9, 1), "rows/s": round(n_tokens / t)}
 
 
 def cpu_baseline(fmt, w, x, n, k, budget_s=12.0):
@@ -196,6 +223,12 @@ def main():
             b = algorithmic_bytes(f, n, k, m, Q)
             also[name] = {"GB/s": round(b / (d / 500) / 1e9, 1), "us": round(d / 500 * 1e6, 2),
                           "hbm_frac": round(b / (d / 500) / 1e9 / HBM_PEAK_GBS, 4)}
+        # the vocabulary projection, the largest GEMV of a decode step (525 MB: cold by size, one copy)
+        _, d, *_ = time_gemv(torch, Q.Q4_K, 128256, 4096, 1, 1, 50, 5, Q, 20260031)
+        b = algorithmic_bytes(Q.Q4_K, 128256, 4096, 1, Q)
+        also["Q4_K gemv 128256x4096 (LM head)"] = {"GB/s": round(b / (d / 50) / 1e9, 1), "us": round(d / 50 * 1e6, 2),
+                                                   "hbm_frac": round(b / (d / 50) / 1e9 / HBM_PEAK_GBS, 4)}
+        also["Q4_K get_rows 512 of 128256x4096"] = time_get_rows(torch, Q.Q4_K, 128256, 4096, 512, Q)
         for name, f, n, k, seed in (("Q4_0 dequant 4096x4096", Q.Q4_0, 4096, 4096, 20260021),
                                     ("Q4_K dequant 14336x4096", Q.Q4_K, N, K, 20260023),
                                     ("MXFP4 dequant 28672x8192", Q.MXFP4, 28672, 8192, 20260025)):

@@ -49,6 +49,8 @@ typedef enum rfq_format {
     RFQ_MXFP6_E2M3 = 21, /* 25 B / 32: i8 exponent + 24 packed bytes         */
     RFQ_MXFP6_E3M2 = 22  /* decoded exactly like E2M3 (src/loader/dequant.rs:693) */
 } rfq_format;
+/* rfq_get_rows also gathers from a plain f32 table (GgufTensorType F32 = 0). */
+#define RFQ_TABLE_F32 0
 
 typedef enum rfq_status {
     RFQ_OK = 0,
@@ -139,6 +141,20 @@ RFQ_API int rfq_matmul_q6_k(const float *d_act, const uint8_t *d_w, float *d_out
  * q6_k.rs:163-205, q8_0.rs:69-106).  d_out receives n_rows floats. */
 RFQ_API int rfq_matmul_host_weights(int fmt, const uint8_t *h_w, size_t w_bytes, const float *d_input,
                             size_t n_rows, size_t n_cols, float *d_out, void *stream);
+
+/* ---- embedding rows ---------------------------------------------------------- */
+
+/* d_out[i, :] = row d_tokens[i] of the [n_vocab, n_embd] table, dequantised
+ * (fmt = a block format, n_embd a multiple of its block) or copied (fmt =
+ * RFQ_TABLE_F32, n_embd a multiple of 4), for i < n_tokens.  Replaces
+ * get_rows (src/ggml/hip_backend/ops/get_rows.rs:6-53, RowMajor) and the
+ * token copy to the host in front of it (op_dispatch.rs:70-100): the ids are
+ * read on the device.  Where the reference fails with "Token ID exceeds vocab
+ * size" this leaves the row zero and, if d_status (a device int) is given,
+ * stores 1 + the smallest offending index there (0 when every id was valid);
+ * the call itself only enqueues.  d_out 16-byte aligned. */
+RFQ_API int rfq_get_rows(int fmt, const void *d_table, size_t table_bytes, int n_vocab, int n_embd,
+                         const uint32_t *d_tokens, int n_tokens, float *d_out, int *d_status, void *stream);
 
 /* ---- prefill GEMM ----------------------------------------------------------- */
 

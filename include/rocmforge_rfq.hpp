@@ -442,5 +442,35 @@ inline Status validate_matmul_q8_0(const std::vector<size_t> &ws, size_t wbytes,
     return validate_matmul("MatMulQ8_0", 36, ws, wbytes, is);
 }
 
+// ---- GetRows (src/ggml/hip_backend/ops/get_rows.rs) ----------------------------------
+// validate_token_ids (:55-65): the first id outside the vocabulary is an error.
+inline Status validate_token_ids(const std::vector<uint32_t> &tokens, size_t vocab_size)
+{
+    for (uint32_t t : tokens)
+        if ((size_t)t >= vocab_size)
+            return Status::Err("Token ID " + std::to_string(t) + " exceeds vocab size " + std::to_string(vocab_size));
+    return ok_status();
+}
+// get_rows (:6-53), RowMajor: output row i = table row tokens[i].  `format` is a
+// block format for a packed table or RFQ_TABLE_F32 for the f32 table the
+// reference holds; the ids go to the device once and are read there.
+inline Status get_rows(const HipBackend &b, const HipBuffer &weights, const std::vector<uint32_t> &tokens, size_t n_embd,
+                       size_t n_vocab, int format, const HipBuffer &output)
+{
+    Status ids = validate_token_ids(tokens, n_vocab);          // same error, same moment as the reference (:18-23)
+    if (!ids.ok) return ids;
+    if (output.size() < tokens.size() * n_embd * sizeof(float)) return Status::Err("get_rows: output buffer too small");
+    if (tokens.empty()) return ok_status();
+    auto dev_tokens = HipBuffer::create(tokens.size() * sizeof(uint32_t));
+    if (!dev_tokens.ok) return Status::Err(dev_tokens.error);
+    Status up = dev_tokens.value.copy_from_host(tokens);
+    if (!up.ok) return up;
+    int rc = rfq_get_rows(format, weights.as_ptr(), weights.size(), (int)n_vocab, (int)n_embd,
+                          (const uint32_t *)dev_tokens.value.as_ptr(), (int)tokens.size(), (float *)output.as_ptr(), nullptr,
+                          b.stream());
+    if (rc != RFQ_OK) return detail::from_rfq(rc, "get_rows");
+    return b.synchronize();                                    // the token buffer is dropped on return
+}
+
 } // namespace rocmforge
 #endif /* ROCMFORGE_RFQ_HPP */

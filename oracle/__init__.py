@@ -137,6 +137,30 @@ def qmatmul_nk(fmt: int, w_bytes, a: np.ndarray, m: int, n: int, k: int, rows=No
     return c
 
 
+def get_rows(fmt: int, table, tokens, n_vocab: int, n_embd: int):
+    """get_rows (src/ggml/hip_backend/ops/get_rows.rs:6-53, RowMajor) over a
+    table that is dequantised first (fmt != 0) or already f32 (fmt == 0):
+    out[i, :] = table[tokens[i], :].  Returns (out, bad) where bad is None or
+    the index of the first token id >= n_vocab; the reference stops with an
+    error there (:18-23), rows from that index on are returned as zero."""
+    tokens = np.asarray(tokens, dtype=np.int64)
+    if fmt == 0:
+        tab = np.ascontiguousarray(table, dtype=np.float32).reshape(n_vocab, n_embd)
+    else:
+        tab = None
+        d = _u8(table)
+        row_bytes = n_embd // block_elems(fmt) * block_bytes(fmt)
+    out = np.zeros((tokens.size, n_embd), dtype=np.float32)
+    bad = None
+    for i, t in enumerate(tokens):
+        if t >= n_vocab or t < 0:
+            if bad is None:
+                bad = i
+            continue
+        out[i] = tab[t] if tab is not None else dequantize(fmt, d[t * row_bytes:(t + 1) * row_bytes], n_embd)
+    return out, bad
+
+
 def pack_mxfp4(values: np.ndarray) -> np.ndarray:
     """MxfpBlock::pack_mxfp4 over consecutive 32-element blocks -> bytes."""
     v = np.ascontiguousarray(values, dtype=np.float32).ravel()

@@ -37,6 +37,7 @@ _SIGNATURES = {
     "rfq_dequant": ([_i, _vp, _sz, _vp, _sz, _vp], _i),
     "rfq_dequant_upload": ([_i, _vp, _sz, _vp, _sz, _vp], _i),
     "rfq_dequant_host": ([_i, _vp, _sz, _vp, _sz], _i),
+    "rfq_get_rows": ([_i, _vp, _sz, _i, _i, _vp, _i, _vp, _vp, _vp], _i),
     "rfq_gemv": ([_i, _vp, _sz, _vp, _vp, _i, _i, _i, _vp], _i),
     "rfq_matmul_q4_0": ([_vp, _vp, _vp, _i, _i, _i, _vp], _i),
     "rfq_matmul_q8_0": ([_vp, _vp, _vp, _i, _i, _i, _vp], _i),

@@ -100,6 +100,26 @@ int rfq_dequant(int fmt, const void *d_packed, size_t packed_bytes, float *d_out
     return launch_dequant(fmt, (const uint8_t *)d_packed, packed_bytes, d_out, n_elems, (hipStream_t)stream);
 }
 
+int rfq_get_rows(int fmt, const void *d_table, size_t table_bytes, int n_vocab, int n_embd, const uint32_t *d_tokens,
+                 int n_tokens, float *d_out, int *d_status, void *stream)
+{
+    const bool f32 = fmt == RFQ_TABLE_F32;
+    if (!f32 && !known_format(fmt)) return fail(RFQ_E_BADARG, "rfq_get_rows: unknown format %d", fmt);
+    if (n_vocab <= 0 || n_embd <= 0 || n_tokens < 0)
+        return fail(RFQ_E_BADARG, "rfq_get_rows: n_vocab=%d n_embd=%d n_tokens=%d", n_vocab, n_embd, n_tokens);
+    const int be = f32 ? 4 : fmt_block_elems(fmt);
+    if (n_embd % be != 0) return fail(RFQ_E_SIZE, "rfq_get_rows: n_embd=%d is not a multiple of %d", n_embd, be);
+    const size_t need = f32 ? (size_t)n_vocab * n_embd * 4 : (size_t)n_vocab * (n_embd / be) * fmt_block_bytes(fmt);
+    if (table_bytes != need)
+        return fail(RFQ_E_SIZE, "rfq_get_rows: table has %zu bytes, a %d x %d table needs %zu", table_bytes, n_vocab,
+                    n_embd, need);
+    if (n_tokens == 0) return RFQ_OK;
+    if (!d_table || !d_tokens || !d_out) return fail(RFQ_E_BADARG, "rfq_get_rows: null pointer");
+    if ((reinterpret_cast<uintptr_t>(d_out) & 15u) != 0 || (f32 && (reinterpret_cast<uintptr_t>(d_table) & 15u) != 0))
+        return fail(RFQ_E_BADARG, "rfq_get_rows: output (and an f32 table) must be 16-byte aligned");
+    return launch_get_rows(fmt, d_table, n_vocab, n_embd, d_tokens, n_tokens, d_out, d_status, (hipStream_t)stream);
+}
+
 int rfq_dequant_upload(int fmt, const uint8_t *h_packed, size_t packed_bytes, float *d_out, size_t n_elems,
                        void *stream)
 {

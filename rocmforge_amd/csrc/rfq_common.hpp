@@ -65,6 +65,8 @@ int release_workspaces();
 
 // ---- launchers implemented per .hip file -----------------------------------
 int launch_dequant(int fmt, const uint8_t *d_in, size_t in_bytes, float *d_out, size_t n, hipStream_t s);
+int launch_get_rows(int fmt, const void *d_table, int n_vocab, int n_embd, const uint32_t *d_tokens, int n_tokens,
+                    float *d_out, int *d_status, hipStream_t s);
 int launch_gemv(int fmt, const uint8_t *d_w, const float *d_x, float *d_y, int m, int n, int k, hipStream_t s);
 int launch_gemm_f16(int fmt, const uint8_t *d_w, const void *d_a, void *d_out, int out_dtype, int m, int n,
                     int k, hipStream_t s);

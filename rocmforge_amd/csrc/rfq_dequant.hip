@@ -202,6 +202,74 @@ dequant_checked_kernel(const uint8_t *__restrict__ in, size_t len, float *__rest
     if (idx < n) out[idx] = decode_checked<FMT>(in, len, idx);
 }
 
+// ---- GetRows: out[i, :] = dequant(row tokens[i]) -----------------------------
+//
+// The reference gathers embedding rows from an f32 table with one device copy
+// per token after copying the token ids to the host
+// (src/ggml/hip_backend/ops/get_rows.rs:6-53, op_dispatch.rs:70-100).  Here the
+// ids are read on the device and the table may stay packed: thread t decodes
+// quad t % (n_embd/4) of output row t / (n_embd/4).  An id outside the table
+// leaves its row zero and records 1 + the row's index in *status (the smallest
+// such index wins), where the reference returns "Token ID exceeds vocab size".
+template <int FMT>
+__global__ void __launch_bounds__(256)
+get_rows_kernel(const uint8_t *__restrict__ table, const uint32_t *__restrict__ tokens, float *__restrict__ out,
+                int n_vocab, int quads_per_row, size_t n_quads, int *status)
+{
+    constexpr int QPB = Fmt<FMT>::BE / 4;
+    const size_t t = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= n_quads) return;
+    const size_t i = t / quads_per_row;
+    const int qd = (int)(t % quads_per_row);
+    const uint32_t id = tokens[i];
+    float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if (id < (uint32_t)n_vocab) {
+        const size_t blk = (size_t)id * (quads_per_row / QPB) + qd / QPB;
+        v = decode_quad<FMT>(table + blk * Fmt<FMT>::BB, (qd % QPB) * 4);
+    } else if (status != nullptr && qd == 0) {
+        atomicMin(reinterpret_cast<unsigned *>(status), (unsigned)i + 1u);
+    }
+    *reinterpret_cast<float4 *>(out + t * 4) = v;
+}
+
+__global__ void __launch_bounds__(256)
+get_rows_f32_kernel(const float *__restrict__ table, const uint32_t *__restrict__ tokens, float *__restrict__ out,
+                    int n_vocab, int quads_per_row, size_t n_quads, int *status)
+{
+    const size_t t = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= n_quads) return;
+    const size_t i = t / quads_per_row;
+    const int qd = (int)(t % quads_per_row);
+    const uint32_t id = tokens[i];
+    float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if (id < (uint32_t)n_vocab) {
+        v = *reinterpret_cast<const float4 *>(table + ((size_t)id * quads_per_row + qd) * 4);
+    } else if (status != nullptr && qd == 0) {
+        atomicMin(reinterpret_cast<unsigned *>(status), (unsigned)i + 1u);
+    }
+    *reinterpret_cast<float4 *>(out + t * 4) = v;
+}
+
+// *status = "no bad id yet" (all ones), folded to 0 after the gather.
+__global__ void get_rows_status_kernel(int *status, int phase)
+{
+    if (phase == 0) *status = -1;
+    else if (*status == -1) *status = 0;
+}
+
+template <int FMT>
+int run_get_rows(const uint8_t *table, const uint32_t *tokens, float *out, int n_vocab, int n_embd, int n_tokens,
+                 int *status, hipStream_t s)
+{
+    const size_t n_quads = (size_t)n_tokens * (n_embd / 4);
+    const size_t grid = (n_quads + 255) / 256;
+    if (grid > 0x7fffffffu) return fail(RFQ_E_SIZE, "rfq_get_rows: %d rows of %d exceed one launch", n_tokens, n_embd);
+    hipLaunchKernelGGL((get_rows_kernel<FMT>), dim3((unsigned)grid), dim3(256), 0, s, table, tokens, out, n_vocab,
+                       n_embd / 4, n_quads, status);
+    RFQ_LAUNCH_CHECK("get_rows_kernel");
+    return RFQ_OK;
+}
+
 template <int FMT>
 int run(const uint8_t *d_in, size_t in_bytes, float *d_out, size_t n, hipStream_t s)
 {
@@ -241,6 +309,43 @@ int launch_dequant(int fmt, const uint8_t *d_in, size_t in_bytes, float *d_out, 
     case RFQ_MXFP6_E2M3: return run<RFQ_MXFP6_E2M3>(d_in, in_bytes, d_out, n, s);
     default: return fail(RFQ_E_BADARG, "rfq_dequant: unknown format %d", fmt);
     }
+}
+
+int launch_get_rows(int fmt, const void *d_table, int n_vocab, int n_embd, const uint32_t *d_tokens, int n_tokens,
+                    float *d_out, int *d_status, hipStream_t s)
+{
+    if (d_status) {
+        hipLaunchKernelGGL(get_rows_status_kernel, dim3(1), dim3(1), 0, s, d_status, 0);
+        RFQ_LAUNCH_CHECK("get_rows_status_kernel");
+    }
+    int rc;
+    const uint8_t *table = static_cast<const uint8_t *>(d_table);
+    switch (fmt) {
+    case RFQ_TABLE_F32: {
+        const size_t n_quads = (size_t)n_tokens * (n_embd / 4);
+        const size_t grid = (n_quads + 255) / 256;
+        if (grid > 0x7fffffffu) return fail(RFQ_E_SIZE, "rfq_get_rows: %d rows of %d exceed one launch", n_tokens, n_embd);
+        hipLaunchKernelGGL(get_rows_f32_kernel, dim3((unsigned)grid), dim3(256), 0, s, static_cast<const float *>(d_table),
+                           d_tokens, d_out, n_vocab, n_embd / 4, n_quads, d_status);
+        hipError_t e = hipGetLastError();
+        rc = e == hipSuccess ? RFQ_OK : hip_fail(e, "get_rows_f32_kernel");
+        break;
+    }
+    case RFQ_Q4_0: rc = run_get_rows<RFQ_Q4_0>(table, d_tokens, d_out, n_vocab, n_embd, n_tokens, d_status, s); break;
+    case RFQ_Q8_0: rc = run_get_rows<RFQ_Q8_0>(table, d_tokens, d_out, n_vocab, n_embd, n_tokens, d_status, s); break;
+    case RFQ_Q4_K: rc = run_get_rows<RFQ_Q4_K>(table, d_tokens, d_out, n_vocab, n_embd, n_tokens, d_status, s); break;
+    case RFQ_Q6_K: rc = run_get_rows<RFQ_Q6_K>(table, d_tokens, d_out, n_vocab, n_embd, n_tokens, d_status, s); break;
+    case RFQ_MXFP4: rc = run_get_rows<RFQ_MXFP4>(table, d_tokens, d_out, n_vocab, n_embd, n_tokens, d_status, s); break;
+    case RFQ_MXFP6_E2M3: case RFQ_MXFP6_E3M2:
+        rc = run_get_rows<RFQ_MXFP6_E2M3>(table, d_tokens, d_out, n_vocab, n_embd, n_tokens, d_status, s); break;
+    default: return fail(RFQ_E_BADARG, "rfq_get_rows: unknown format %d", fmt);
+    }
+    if (rc != RFQ_OK) return rc;
+    if (d_status) {
+        hipLaunchKernelGGL(get_rows_status_kernel, dim3(1), dim3(1), 0, s, d_status, 1);
+        RFQ_LAUNCH_CHECK("get_rows_status_kernel");
+    }
+    return RFQ_OK;
 }
 
 } // namespace rfq

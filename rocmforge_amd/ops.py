@@ -51,6 +51,24 @@ def gemv(fmt: int, w: torch.Tensor, x: torch.Tensor, n: int, k: int, out: torch.
     return out if x.dim() > 1 else out.view(n)
 
 
+def get_rows(fmt: int, table: torch.Tensor, tokens: torch.Tensor, n_vocab: int, n_embd: int,
+             status: torch.Tensor | None = None) -> torch.Tensor:
+    """out[i, :] = dequantised (fmt = block format) or copied (fmt = 0, f32 table) row tokens[i] of the table."""
+    if fmt == 0:
+        if table.dtype != torch.float32 or not table.is_contiguous():
+            raise ValueError("an f32 table must be a contiguous float32 tensor")
+        nbytes = table.numel() * 4
+    else:
+        table = _dev_u8(table)
+        nbytes = table.numel()
+    if tokens.dtype not in (torch.int32, torch.uint32) or not tokens.is_contiguous():
+        raise ValueError("tokens must be a contiguous int32/uint32 tensor")
+    out = torch.empty((tokens.numel(), n_embd), dtype=torch.float32, device=table.device)
+    check(lib().rfq_get_rows(fmt, _ptr(table), nbytes, n_vocab, n_embd, _ptr(tokens), tokens.numel(), _ptr(out),
+                             _ptr(status) if status is not None else None, _stream()))
+    return out
+
+
 def gemm_f16(fmt: int, w: torch.Tensor, a: torch.Tensor, n: int, k: int, out_dtype=torch.float16,
              out: torch.Tensor | None = None) -> torch.Tensor:
     """out[m, n] = a[m, k] (fp16) . dequant(W)[n, k]^T on the fp16 matrix cores."""

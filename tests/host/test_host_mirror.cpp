@@ -3,7 +3,8 @@
 // every value comes from the GPU kernels.  Vectors and names follow
 //   src/kernels/quant/q4_0.rs:317-438, q8_0.rs:78-183, q4_k.rs:280-368, q6_k.rs:273-399,
 //   src/loader/mxfp_tests.rs:97-187 and 424-464, src/loader/dequant.rs:440-470,
-//   src/kernels/matmul/quantized/q4_0.rs:318-338, src/ggml/hip_backend/op_dispatch.rs:951-1014.
+//   src/kernels/matmul/quantized/q4_0.rs:318-338, src/ggml/hip_backend/op_dispatch.rs:951-1014,
+//   src/ggml/hip_backend/ops/get_rows.rs:6-65.
 // Prints one line per test; exit status 0 only if all passed.
 #include <cmath>
 #include <cstdio>
@@ -267,6 +268,36 @@ static void test_matmul_validation_like_op_dispatch()
     EXPECT(bytes_per_element(QuantFormat::Q8_0) == 36.0f / 32.0f && std::string(name(QuantFormat::Q6_K)) == "Q6_K");
 }
 
+// get_rows.rs:6-65: rows are copied by token id; an id outside the vocabulary is an error
+static void test_get_rows_f32_and_packed_tables()
+{
+    auto be = HipBackend::create();
+    EXPECT(be.ok);
+    const size_t n_vocab = 5, n_embd = 32;
+    std::vector<float> table(n_vocab * n_embd);
+    for (size_t i = 0; i < table.size(); i++) table[i] = (float)i * 0.5f;
+    auto tab = HipBuffer::create(table.size() * 4), out = HipBuffer::create(3 * n_embd * 4);
+    EXPECT(tab.ok && out.ok && tab.value.copy_from_host(table).ok);
+    EXPECT(get_rows(be.value, tab.value, {4, 0, 4}, n_embd, n_vocab, RFQ_TABLE_F32, out.value).ok);
+    std::vector<float> got(3 * n_embd);
+    EXPECT(out.value.copy_to_host(got).ok);
+    for (size_t j = 0; j < n_embd; j++)
+        EXPECT(got[j] == table[4 * n_embd + j] && got[n_embd + j] == table[j] && got[2 * n_embd + j] == got[j]);
+    Status bad = get_rows(be.value, tab.value, {1, 5}, n_embd, n_vocab, RFQ_TABLE_F32, out.value);
+    EXPECT(!bad.ok && bad.error == "Token ID 5 exceeds vocab size 5");
+    // a Q4_0 table: row r = one block with scale r + 1 and every nibble 9 -> (9 - 8) * (r + 1)
+    bytes packed(n_vocab * 20);
+    for (size_t r = 0; r < n_vocab; r++) {
+        put_f32(packed, r * 20, (float)(r + 1));
+        for (size_t j = 0; j < 16; j++) packed[r * 20 + 4 + j] = 0x99;
+    }
+    auto ptab = HipBuffer::create(packed.size());
+    EXPECT(ptab.ok && ptab.value.copy_from_host(packed).ok);
+    EXPECT(get_rows(be.value, ptab.value, {2, 0, 3}, n_embd, n_vocab, RFQ_Q4_0, out.value).ok);
+    EXPECT(out.value.copy_to_host(got).ok);
+    EXPECT(all_eq(got, 0, 32, 3.0f) && all_eq(got, 32, 64, 1.0f) && all_eq(got, 64, 96, 4.0f));
+}
+
 int main()
 {
     struct T { const char *name; std::function<void()> fn; };
@@ -285,6 +316,7 @@ int main()
         {"test_dequantize_q4_0_kernel_cached_and_twins", test_dequantize_q4_0_kernel_cached_and_twins},
         {"test_matmul_q4_0_against_dequantized_weights", test_matmul_q4_0_against_dequantized_weights},
         {"test_matmul_validation_like_op_dispatch", test_matmul_validation_like_op_dispatch},
+        {"test_get_rows_f32_and_packed_tables", test_get_rows_f32_and_packed_tables},
     };
     for (const T &t : tests) {
         int before = failures;

@@ -28,5 +28,6 @@ def test_mirror_header_names_the_reference_surface():
                  "dequant_q6_k", "dequant_mxfp4", "dequant_mxfp6", "dequantize", "HipBuffer", "HipBackend",
                  "matmul_q4_0", "matmul_q8_0", "matmul_q4_k", "matmul_q6_k", "matmul_q4_0_gpu",
                  "dequantize_q4_0_kernel_cached", "dequantize_q4_k_gpu_kernel", "dequantize_q6_k_gpu_kernel",
-                 "QuantFormat", "QuantizedMatmulOp", "validate_matmul_q4_0", "validate_matmul_q8_0"):
+                 "QuantFormat", "QuantizedMatmulOp", "validate_matmul_q4_0", "validate_matmul_q8_0", "get_rows",
+                 "validate_token_ids"):
         assert name in text, name
