@@ -156,7 +156,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build is single-GPU (one MI355X per box); run with --gpus 1. "
-                 "The path shards by output rows with no exchange during compute; see DESIGN.md.")
+                 "The path shards by output rows with no exchange during compute.")
 
     import numpy as np
     import torch

@@ -77,7 +77,7 @@ def test_gemv_mx_random_codes_and_clamp(fmt, oracle, cuda):
     assert_close(gpu_gemv(fmt, w, x, n, k, cuda), oracle.qmatmul_nk(fmt, w, x, 1, n, k)[0], Q.NAMES[fmt])
 
 
-# BASELINE configs: Q4_0 4864x896; Q8_0 4096x4096 at m = 1 and 8; Q4_K and Q6_K 14336x4096.
+# The benchmark configurations: Q4_0 4864x896; Q8_0 4096x4096 at m = 1 and 8; Q4_K and Q6_K 14336x4096.
 @pytest.mark.parametrize("fmt,n,k,m,cfg", [(Q.Q4_0, 4864, 896, 1, 1), (Q.Q8_0, 4096, 4096, 1, 2),
                                            (Q.Q8_0, 4096, 4096, 8, 2), (Q.Q4_K, 14336, 4096, 1, 3),
                                            (Q.Q6_K, 14336, 4096, 1, 3)])
