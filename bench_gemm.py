@@ -34,15 +34,19 @@ def mx_gemm(torch, w_fmt, m=2048, n=28672, k=8192, steps=50, warmup=40):
     W = ops.MxOperand(w_fmt, w_dev, n, k)
 
     def prepare_us(fmt, raw, rows, kind):
-        # re-encoding into the matrix core's operand order, reported beside the GEMM, never inside it
-        import time
-        ops.MxOperand(fmt, raw, rows, k, kind)
+        # re-encoding into the matrix core's operand order, reported beside the GEMM, never inside it:
+        # device time of back-to-back calls that do not synchronise (8-bit kinds, and the 4-bit kind
+        # requested unchecked, which is how activations are prepared per prefill)
+        req = _lib.MX_FP4_UNCHECKED if kind == _lib.MX_FP4 else kind
+        ops.MxOperand(fmt, raw, rows, k, req)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(5):
-            ops.MxOperand(fmt, raw, rows, k, kind)
+        e0.record()
+        for _ in range(10):
+            ops.MxOperand(fmt, raw, rows, k, req)
+        e1.record()
         torch.cuda.synchronize()
-        return round((time.perf_counter() - t0) / 5 * 1e6, 1)
+        return round(e0.elapsed_time(e1) / 10 * 1e3, 1)
 
     prep = {"prepare_a_us": prepare_us(Q.MXFP4, a_dev, m, A.kind), "prepare_w_us": prepare_us(w_fmt, w_dev, n, W.kind)}
     out = torch.empty((m, n), dtype=torch.bfloat16, device=dev)

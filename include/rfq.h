@@ -67,7 +67,7 @@ typedef enum rfq_status {
 typedef enum rfq_dtype { RFQ_F32 = 0, RFQ_F16 = 1, RFQ_BF16 = 2 } rfq_dtype;
 
 /* Operand encodings of a prepared MXFP matrix (see rfq_mx_prepare). */
-typedef enum rfq_mx_kind { RFQ_MX_AUTO = 0, RFQ_MX_FP4 = 4, RFQ_MX_FP8 = 8 } rfq_mx_kind;
+typedef enum rfq_mx_kind { RFQ_MX_AUTO = 0, RFQ_MX_FP4 = 4, RFQ_MX_FP8 = 8, RFQ_MX_FP4_UNCHECKED = 0x104 } rfq_mx_kind;
 
 /* ---- library ------------------------------------------------------------ */
 
@@ -185,6 +185,13 @@ RFQ_API int rfq_gemm_f16(int fmt, const void *d_w, size_t w_bytes, const void *d
  *   (this reads one flag back and therefore synchronises the stream); FP8
  *   never synchronises; FP4 fails with RFQ_E_UNSUPPORTED (after a sync) when a
  *   block is not expressible.  *kind_out receives the encoding written.
+ *   FP4_UNCHECKED (a request only; the buffer's kind is FP4) is FP4 without
+ *   the read-back and the synchronisation, for activations re-encoded per
+ *   prefill: the caller vouches that every block fits, which holds for
+ *   whatever MxfpBlock::pack_mxfp4 (src/loader/mxfp.rs:118-161) produced (it
+ *   never emits the sign-only code, the one value below the four codes'
+ *   span); a block that does not fit is re-encoded wrongly without notice.
+ *   rfq_mx_prepared_bytes takes FP4 for it.
  * This is the one-time weight upload step (src/loader/gguf/gpu_upload.rs:57-125
  * does the analogous dequantise-at-load for the K formats). */
 RFQ_API size_t rfq_mx_prepared_bytes(int fmt, int kind, int rows, int k);

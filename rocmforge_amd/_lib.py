@@ -10,7 +10,7 @@ _SO = os.path.join(_HERE, "librfq.so")
 
 OK, E_BADARG, E_SIZE, E_UNSUPPORTED, E_HIP, E_NOMEM = 0, -1, -2, -3, -4, -5
 F32, F16, BF16 = 0, 1, 2
-MX_AUTO, MX_FP4, MX_FP8 = 0, 4, 8
+MX_AUTO, MX_FP4, MX_FP8, MX_FP4_UNCHECKED = 0, 4, 8, 0x104
 
 
 class RfqError(RuntimeError):

@@ -239,7 +239,7 @@ int rfq_mx_prepare(int fmt, int kind_req, const void *d_raw, size_t raw_bytes, i
     if (!d_raw || !d_prepared) return fail(RFQ_E_BADARG, "rfq_mx_prepare: null pointer");
     if (rows <= 0 || k <= 0) return fail(RFQ_E_BADARG, "rfq_mx_prepare: bad shape %d x %d", rows, k);
     if (k % 128 != 0) return fail(RFQ_E_SIZE, "rfq_mx_prepare: k=%d is not a multiple of 128", k);
-    if (kind_req != RFQ_MX_AUTO && kind_req != RFQ_MX_FP4 && kind_req != RFQ_MX_FP8)
+    if (kind_req != RFQ_MX_AUTO && kind_req != RFQ_MX_FP4 && kind_req != RFQ_MX_FP8 && kind_req != RFQ_MX_FP4_UNCHECKED)
         return fail(RFQ_E_BADARG, "rfq_mx_prepare: unknown kind %d", kind_req);
     size_t need = matrix_bytes(fmt, rows, k);
     if (raw_bytes != need)

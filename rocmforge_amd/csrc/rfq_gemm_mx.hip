@@ -49,6 +49,11 @@ __device__ unsigned long long *rfq_mx_trace;
 #endif
 // Ring depth (W slots in LDS = A fragment sets in registers) with 4-bit A
 // fragments; 8-bit A fragments take twice the registers and half the depth.
+// -DRFQ_MX_GENERAL_FP4=1: re-encode MXFP4 to 4-bit operands with the general
+// (float) kernel instead of the integer one, to compare the two.
+#ifndef RFQ_MX_GENERAL_FP4
+#define RFQ_MX_GENERAL_FP4 0
+#endif
 #ifndef RFQ_MX_RING
 #define RFQ_MX_RING 8
 #endif
@@ -219,12 +224,96 @@ mx_prepare_kernel(const uint8_t *__restrict__ raw, uint8_t *__restrict__ prep, M
     prep[L.data_bytes + ((size_t)rt * L.ks4 + (ks >> 2)) * 256 + (size_t)lane * 4 + (ks & 3)] = (uint8_t)E;
 }
 
-// Scale bytes (before the re-encoding overwrites them) and the status words.
-__global__ void mx_init_kernel(uint8_t *prep, MxLayout L)
+// MXFP4 -> 4-bit operand with integer arithmetic only (the general kernel
+// above goes through the 32 float values).  A raw code is sign | m with
+// magnitude 2^p(m) times the block's 2^e, p = -1 (m = 0 with the sign set),
+// 0, 0, 1, 1, 2, 2, 3 for m = 1..7, code 0 is 0.0
+// (MxfpBlock::decode_e2m1, src/loader/mxfp.rs:234-244); the +-8 clamp caps
+// the exponent e + p at 3.  The matrix core's E2M1 codes 1, 2, 4, 6 are 0.5,
+// 1, 2, 4: with the largest exponent of the block on code 6 (scale byte =
+// that exponent - 2) every other value is a code iff it is at most 3 octaves
+// below.  Which exponents occur is found with nibble-parallel arithmetic on the
+// four dwords, the code translation is two 8-entry byte tables (sign clear /
+// set) looked up with v_perm_b32, four codes per instruction.
+__global__ void __launch_bounds__(256)
+mx_prepare_fp4_kernel(const uint8_t *__restrict__ raw, uint8_t *__restrict__ prep, MxLayout L)
 {
     size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (g < L.scale_bytes) prep[L.data_bytes + g] = 127;
-    if (g < 4) reinterpret_cast<uint32_t *>(prep + L.data_bytes + L.scale_bytes)[g] = 0;
+    size_t npages = (size_t)L.rt * L.ks;
+    if (g >= npages * 64) return;
+    int lane = (int)(g & 63);
+    size_t page = g >> 6;
+    int rt = (int)(page / L.ks), ks = (int)(page % L.ks);
+    int row = rt * 32 + (lane & 31), kb = ks * 2 + (lane >> 5);
+    uint32_t *status = reinterpret_cast<uint32_t *>(prep + L.data_bytes + L.scale_bytes);
+
+    int E = 127;
+    uint32_t out[4] = {0u, 0u, 0u, 0u};
+    if (row < L.rows && ks < L.ks_real) {
+        const uint8_t *blk = raw + ((size_t)row * (L.k / 32) + kb) * 17;
+        const int e = (int)(int8_t)blk[0];
+        const v4i qi = ld<v4i>(blk + 1);
+        const uint32_t q[4] = {(uint32_t)qi[0], (uint32_t)qi[1], (uint32_t)qi[2], (uint32_t)qi[3]};
+        // bit 3 of a nibble of geN: that code has m >= N; cNN: m in that pair; neg0: m = 0 with the sign set
+        uint32_t ge7 = 0, c56 = 0, c34 = 0, c12 = 0, neg0 = 0;
+#pragma unroll
+        for (int d = 0; d < 4; d++) {
+            const uint32_t y = q[d] & 0x77777777u;
+            const uint32_t a1 = y + 0x77777777u, a3 = y + 0x55555555u, a5 = y + 0x33333333u, a7 = y + 0x11111111u;
+            ge7 |= a7;
+            c56 |= a5 & ~a7;
+            c34 |= a3 & ~a5;
+            c12 |= a1 & ~a3;
+            neg0 |= ~a1 & q[d];
+        }
+        const uint32_t M8 = 0x88888888u;
+        // bit p + 1 of `present`: an element with magnitude exponent p exists (2^-128 as the scale is 0.0: nothing does)
+        uint32_t present = ((neg0 & M8) ? 1u : 0u) | ((c12 & M8) ? 2u : 0u) | ((c34 & M8) ? 4u : 0u) |
+                           ((c56 & M8) ? 8u : 0u) | ((ge7 & M8) ? 16u : 0u);
+        if (e == -128) present = 0;
+        if (present != 0) {
+            const int pmax = 30 - __builtin_clz(present), pmin = __builtin_ctz(present) - 1;
+            const int cap = 3 - e;                                 // exponents above 3 are clamped to 3
+            auto ex = [&](int p) { return e + (p < cap ? p : cap); };
+            int Eu = ex(pmax) - 2;
+            if (Eu < -127) Eu = -127;
+            E = Eu + 127;
+            if (ex(pmin) - Eu < -1) status[0] = 1u;               // more than the four codes span
+            auto code = [&](int p) {                               // 0.5, 1, 2, 4 times the new scale
+                int kx = ex(p) - Eu;
+                kx = kx < -1 ? -1 : kx;
+                return (uint32_t)(kx < 0 ? 1 : 2 * kx + 2);
+            };
+            const uint32_t gm1 = code(-1), g0 = code(0), g1 = code(1), g2 = code(2), g3 = code(3);
+            const uint32_t t0_lo = (g0 << 8) | (g0 << 16) | (g1 << 24);          // m = 0 (with the sign clear: 0.0), 1, 2, 3
+            const uint32_t t0_hi = g1 | (g2 << 8) | (g2 << 16) | (g3 << 24);     // m = 4..7
+            const uint32_t t1_lo = t0_lo | 0x08080808u | gm1, t1_hi = t0_hi | 0x08080808u;
+#pragma unroll
+            for (int d = 0; d < 4; d++) {
+                // byte j of the raw dword: high nibble = element 2j, low nibble = element 2j+1;
+                // byte j of the operand dword: low nibble = element 2j, high nibble = element 2j+1
+                uint32_t r[2];
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    const uint32_t c = (h == 0 ? q[d] >> 4 : q[d]) & 0x0F0F0F0Fu;
+                    const uint32_t sel = c & 0x07070707u, s8 = c & 0x08080808u;
+                    const uint32_t plus = __builtin_amdgcn_perm(t0_hi, t0_lo, sel), minus = __builtin_amdgcn_perm(t1_hi, t1_lo, sel);
+                    const uint32_t neg = (s8 << 1) - (s8 >> 3);   // 0x0F in the bytes whose sign bit is set
+                    r[h] = (minus & neg) | (plus & ~neg);
+                }
+                out[d] = r[0] | (r[1] << 4);
+            }
+        }
+    }
+    uint4 *dst = reinterpret_cast<uint4 *>(prep + page * 1024 + (size_t)lane * 16);
+    *dst = make_uint4(out[0], out[1], out[2], out[3]);
+    prep[L.data_bytes + ((size_t)rt * L.ks4 + (ks >> 2)) * 256 + (size_t)lane * 4 + (ks & 3)] = (uint8_t)E;
+}
+
+// The status words (every page and every scale byte is written by the re-encoding kernels).
+__global__ void mx_init_kernel(uint8_t *prep, MxLayout L)
+{
+    if (threadIdx.x < 4) reinterpret_cast<uint32_t *>(prep + L.data_bytes + L.scale_bytes)[threadIdx.x] = 0;
 }
 
 // ---- GEMM ---------------------------------------------------------------------
@@ -832,11 +921,13 @@ template <int FMT, int KIND>
 int run_prepare(const uint8_t *raw, uint8_t *prep, const MxLayout &L, hipStream_t s)
 {
     size_t threads = (size_t)L.rt * L.ks * 64;
-    size_t init = L.scale_bytes > 4 ? L.scale_bytes : 4;
-    hipLaunchKernelGGL(mx_init_kernel, dim3((unsigned)((init + 255) / 256)), dim3(256), 0, s, prep, L);
+    hipLaunchKernelGGL(mx_init_kernel, dim3(1), dim3(64), 0, s, prep, L);
     RFQ_LAUNCH_CHECK("mx_init_kernel");
-    hipLaunchKernelGGL((mx_prepare_kernel<FMT, KIND>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, raw,
-                       prep, L);
+    if (FMT == RFQ_MXFP4 && KIND == RFQ_MX_FP4 && !RFQ_MX_GENERAL_FP4)
+        hipLaunchKernelGGL(mx_prepare_fp4_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, raw, prep, L);
+    else
+        hipLaunchKernelGGL((mx_prepare_kernel<FMT, KIND>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, raw,
+                           prep, L);
     RFQ_LAUNCH_CHECK("mx_prepare_kernel");
     return RFQ_OK;
 }
@@ -857,6 +948,8 @@ int launch_mx_prepare(int fmt, int kind_req, const uint8_t *d_raw, int rows, int
                       int *kind_out, hipStream_t s)
 {
     const bool is4 = fmt == RFQ_MXFP4;
+    const bool unchecked = kind_req == RFQ_MX_FP4_UNCHECKED;
+    if (unchecked) kind_req = RFQ_MX_FP4;
     if (kind_req == RFQ_MX_FP4 && !is4)
         return fail(RFQ_E_UNSUPPORTED, "rfq_mx_prepare: MXFP6 has no 4-bit re-encoding");
     uint8_t *prep = static_cast<uint8_t *>(d_prep);
@@ -870,6 +963,10 @@ int launch_mx_prepare(int fmt, int kind_req, const uint8_t *d_raw, int rows, int
             return fail(RFQ_E_SIZE, "rfq_mx_prepare: prepared buffer has %zu bytes, needs %zu", prep_bytes, need);
         int rc = run_prepare<RFQ_MXFP4, RFQ_MX_FP4>(d_raw, prep, L, s);
         if (rc != RFQ_OK) return rc;
+        if (unchecked) {                                         // the caller vouches for the data: no read-back, no sync
+            if (kind_out) *kind_out = RFQ_MX_FP4;
+            return RFQ_OK;
+        }
         uint32_t status = 0;
         RFQ_HIP(hipMemcpyAsync(&status, prep + L.data_bytes + L.scale_bytes, 4, hipMemcpyDeviceToHost, s));
         RFQ_HIP(hipStreamSynchronize(s));

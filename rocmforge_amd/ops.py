@@ -88,7 +88,7 @@ class MxOperand:
 
     def __init__(self, fmt: int, raw: torch.Tensor, rows: int, k: int, kind: int = _lib.MX_AUTO):
         raw = _dev_u8(raw)
-        nbytes = lib().rfq_mx_prepared_bytes(fmt, kind, rows, k)
+        nbytes = lib().rfq_mx_prepared_bytes(fmt, _lib.MX_FP4 if kind == _lib.MX_FP4_UNCHECKED else kind, rows, k)
         if nbytes == 0:
             raise ValueError(f"cannot size a prepared operand for fmt={fmt} rows={rows} k={k}")
         self.buf = torch.empty(nbytes, dtype=torch.uint8, device=raw.device)
