@@ -1160,7 +1160,7 @@ template <int FMT>
 int run(const uint8_t *w, const float *x, float *y, int m, int n, int k, hipStream_t s)
 {
     const int ku = k / 32;
-    if (m == 1 && ku > 32) {
+    if (m == 1 && ku > 16) {                                   // (shorter rows leave most of a wavefront's lanes without a unit)
         if (ku <= 64) return run_idot<FMT, 1, 1>(w, x, y, n, k, s);
         if (ku <= 128) return run_idot<FMT, 2, 1>(w, x, y, n, k, s);
         if (ku <= 256) return run_idot<FMT, 2, 2>(w, x, y, n, k, s);

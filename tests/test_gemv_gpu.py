@@ -29,11 +29,11 @@ def x_for(m, k, seed):
     return x[0] if m == 1 else x
 
 
-# k = 256..1024 takes the one-row-per-wavefront kernel, 2048 / 4096 / 8192 /
-# 14336 the register-resident one at 1, 2, 2x2 and 2x4 units per lane x
-# wavefronts per row, 32768 falls back again; n values exercise ragged teams.
+# k = 256 and 512 take the one-row-per-wavefront kernel, 768 ... 14336 the
+# register-resident one at 1, 2, 2x2 and 2x4 units per lane x wavefronts per
+# row, 32768 falls back again; n values exercise ragged teams.
 @pytest.mark.parametrize("fmt", FORMATS)
-@pytest.mark.parametrize("n,k", [(5, 256), (33, 1024), (64, 2048), (1001, 2048), (130, 4096), (257, 8192),
+@pytest.mark.parametrize("n,k", [(5, 256), (40, 512), (77, 768), (33, 1024), (64, 2048), (1001, 2048), (130, 4096), (257, 8192),
                                  (19, 14336), (9, 32768), (2048, 1536)])
 def test_gemv_m1_shapes(fmt, n, k, oracle, cuda):
     w = Q.make_weights(fmt, n, k, seed=3000 + fmt + n)
