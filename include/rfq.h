@@ -164,7 +164,8 @@ RFQ_API int rfq_get_rows(int fmt, const void *d_table, size_t table_bytes, int n
  * otherwise; d_a_f16 16-byte aligned, d_w 4-byte aligned.  Up to 64 MiB of
  * temporary device memory (the activations in matrix-operand order) is kept
  * per stream between calls; larger temporaries are allocated and released in
- * stream order.  The reference has no fused prefill GEMM (its matmul_q* hard-wire
+ * stream order.  (A stream's first call, or a larger shape than before,
+ * allocates: run the call once on the stream before capturing it into a graph.)  The reference has no fused prefill GEMM (its matmul_q* hard-wire
  * m = 1, src/kernels/matmul/quantized/q4_0.rs:169; larger m goes through
  * dequantise + hipBLAS SGEMM, src/tensor/matmul.rs:134-214); this is the same
  * contraction. */
