@@ -4,9 +4,10 @@ MXFP4 GEMM at M=2048, K=8192, N=28672 (bf16 out) and the MXFP6-weight variant,
 plus the Q4_K fp16 GEMM at M=512, K=4096, N=14336 when that kernel is built.
 FLOPs = 2*M*N*K; peaks: 10.1 PFLOP/s (FP4 scaled MFMA), 5.0 (FP8), 2.5 (fp16).
 
-Each configuration runs `warmup` untimed launches first (about 8 ms): the
-first launches after an idle period run 10-15 % slower than the steady state
-(the part's clocks ramp), and the timed launches should not include that.
+Each configuration runs `warmup` untimed launches first (20 to 30 ms): the
+launches of the first tens of milliseconds after an idle period run 5-15 %
+slower than the steady state (the part's clocks ramp), and the timed launches
+should not include that.
 """
 from __future__ import annotations
 
@@ -22,7 +23,7 @@ def _gauss(rows, k, seed, std):
     return rng.standard_normal((rows, k), dtype=np.float32) * np.float32(std)
 
 
-def mx_gemm(torch, w_fmt, m=2048, n=28672, k=8192, steps=50, warmup=40):
+def mx_gemm(torch, w_fmt, m=2048, n=28672, k=8192, steps=50, warmup=150):
     from rocmforge_amd import _lib, ops, quantize as Q
     dev = torch.device("cuda:0")
     a_raw = Q.pack_mxfp4(_gauss(m, k, 20260005, 1.0))
@@ -64,7 +65,7 @@ def mx_gemm(torch, w_fmt, m=2048, n=28672, k=8192, steps=50, warmup=40):
             "peak_TFLOP/s": peak / 1e12, "kinds": [A.kind, W.kind], **prep}
 
 
-def kq_gemm(torch, fmt, m=512, n=14336, k=4096, steps=100, warmup=80):
+def kq_gemm(torch, fmt, m=512, n=14336, k=4096, steps=100, warmup=300):
     """Q4_K / Q6_K prefill GEMM on the fp16 matrix cores, fp16 in and out."""
     from rocmforge_amd import _lib, quantize as Q
     dev = torch.device("cuda:0")
@@ -105,8 +106,8 @@ if __name__ == "__main__":
     import torch
     from rocmforge_amd import quantize as Q
     if a.only == "q4_k":
-        print(json.dumps(kq_gemm(torch, Q.Q4_K, steps=a.steps, warmup=40)))
+        print(json.dumps(kq_gemm(torch, Q.Q4_K, steps=a.steps)))
     elif a.only:
-        print(json.dumps(mx_gemm(torch, Q.MXFP4 if a.only == "mxfp4" else Q.MXFP6_E2M3, steps=a.steps, warmup=40)))
+        print(json.dumps(mx_gemm(torch, Q.MXFP4 if a.only == "mxfp4" else Q.MXFP6_E2M3, steps=a.steps)))
     else:
         print(json.dumps(run(torch)))
