@@ -156,6 +156,61 @@ RFQ_API int rfq_matmul_host_weights(int fmt, const uint8_t *h_w, size_t w_bytes,
 RFQ_API int rfq_get_rows(int fmt, const void *d_table, size_t table_bytes, int n_vocab, int n_embd,
                          const uint32_t *d_tokens, int n_tokens, float *d_out, int *d_status, void *stream);
 
+/* ---- neighbours of the matmul in a decoder layer ---------------------------- */
+
+/* d_out[r, j] = (d_x[r, j] / sqrt(mean_j d_x[r, j]^2 + eps)) * d_weight[j] for
+ * seq_len rows of hidden_size floats (hidden_size a multiple of 4, all three
+ * pointers 16-byte aligned).  Replaces rms_norm_gpu_kernel
+ * (src/mlp/kernels.rs:261-330, kernels/rms_norm.hip:40-84). */
+RFQ_API int rfq_rms_norm(const float *d_input, const float *d_weight, float *d_output, int seq_len, int hidden_size,
+                         float eps, void *stream);
+
+/* d_output[i] = d_gate[i] * (d_up[i] * sigmoid(d_up[i])) over seq_len *
+ * intermediate_size elements: the activation is applied to the UP projection,
+ * as the reference defines it.  Replaces swiglu_gpu_kernel
+ * (src/mlp/kernels.rs:177-240, kernels/swiglu.hip:40-62). */
+RFQ_API int rfq_swiglu(const float *d_gate, const float *d_up, float *d_output, int seq_len, int intermediate_size,
+                       void *stream);
+
+/* RMSNorm of rows that are still packed: d_packed holds seq_len rows of
+ * hidden_size elements in format fmt (hidden_size a multiple of the block), the
+ * rows are decoded on the fly and normalised as in rfq_rms_norm; no f32 copy
+ * of the input exists.  Replaces fused_q4_0_rmsnorm
+ * (src/ggml/hip_backend/ops/fused_ops.rs:149-160,
+ * kernels/fused_dequant_rmsnorm.hip:87-163), for every format. */
+RFQ_API int rfq_dequant_rms_norm(int fmt, const void *d_packed, size_t packed_bytes, const float *d_weight,
+                                 float *d_output, int seq_len, int hidden_size, float eps, void *stream);
+
+/* d_y[m, n] = RMSNorm(d_x[m, k]; d_norm_weight, eps) . dequant(W)[n, k]^T: the
+ * normalisation that precedes a projection in a decoder layer and the
+ * projection (rfq_gemv) in one call.  For m = 1 and 512 < k <= 16384 it is one
+ * launch and the normalised vector never exists in memory; other shapes run
+ * rfq_rms_norm into d_scratch (m * k floats, 16-byte aligned; may be NULL when
+ * the one-launch case applies) and then rfq_gemv.  The reference has the two
+ * steps only as separate f32 operations (kernels/rms_norm.hip, hipBLAS SGEMM:
+ * src/ggml/hip_backend/op_dispatch.rs:1001-1014). */
+RFQ_API int rfq_rms_norm_gemv(int fmt, const void *d_w, size_t w_bytes, const float *d_x, const float *d_norm_weight,
+                              float eps, float *d_y, int m, int n, int k, float *d_scratch, void *stream);
+
+/* The SwiGLU MLP of a decoder layer over quantised weights, 1 <= m <= 8 rows:
+ *   xn  = d_norm_weight ? RMSNorm(d_x; d_norm_weight, eps) : d_x      [m, hidden]
+ *   h   = swiglu(xn . dequant(gate)^T, xn . dequant(up)^T)            [m, inter]
+ *   out = h . dequant(down)^T                                         [m, hidden]
+ * gate and up are [inter, hidden] in fmt_gate_up (gate_up_bytes each), down is
+ * [hidden, inter] in fmt_down; rows are outputs, blocks run along k, as
+ * rfq_gemv takes them.  For m = 1 this is two launches: gate and up rows are
+ * walked together, normalisation and activation happen inside that kernel, and
+ * only h goes through d_scratch.  Replaces HipBackend::mlp_swiglu
+ * (src/backend/hip_backend/backend.rs:1153-1278: three f32 SGEMMs, a SwiGLU
+ * kernel and two synchronisations) for quantised weights.  d_scratch:
+ * rfq_mlp_scratch_bytes(m, hidden, inter) bytes, 16-byte aligned, owned by
+ * the caller; nothing is allocated and nothing synchronises. */
+RFQ_API size_t rfq_mlp_scratch_bytes(int m, int hidden_size, int intermediate_size);
+RFQ_API int rfq_mlp_swiglu(int fmt_gate_up, const void *d_gate_w, const void *d_up_w, size_t gate_up_bytes,
+                           int fmt_down, const void *d_down_w, size_t down_bytes, const float *d_x,
+                           const float *d_norm_weight, float eps, float *d_out, int m, int hidden_size,
+                           int intermediate_size, void *d_scratch, size_t scratch_bytes, void *stream);
+
 /* ---- prefill GEMM ----------------------------------------------------------- */
 
 /* d_out[m, n] = d_a[m, k] (fp16) . dequant(W)[n, k]^T on the fp16 matrix

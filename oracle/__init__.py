@@ -69,6 +69,11 @@ def lib() -> C.CDLL:
         L.rf_matmul_nk_f32.argtypes = [f32p, f32p, sz, sz, sz, f32p]
         L.rf_qmatmul_nk.argtypes = [C.c_int, u8p, sz, f32p, sz, sz, sz, C.c_void_p, sz, f32p]
         L.rf_qmatmul_nk.restype = C.c_int
+        L.rf_rms_norm.argtypes = [f32p, f32p, sz, sz, C.c_float, f32p]
+        L.rf_swiglu.argtypes = [f32p, f32p, sz, f32p]
+        L.rf_dequant_rms_norm.argtypes = [C.c_int, u8p, sz, f32p, sz, sz, C.c_float, f32p]
+        L.rf_mlp_swiglu_q.argtypes = [C.c_int, u8p, u8p, sz, C.c_int, u8p, sz, f32p, f32p, C.c_float, sz, sz, sz,
+                                      f32p, f32p]
         L.rf_qmatmul_nk_staged.argtypes = [C.c_int, u8p, sz, f32p, sz, sz, sz, f32p, f32p]
         L.rf_qmatmul_nk_staged.restype = C.c_int
         _lib = L
@@ -135,6 +140,57 @@ def qmatmul_nk(fmt: int, w_bytes, a: np.ndarray, m: int, n: int, k: int, rows=No
     if rc != 0:
         raise ValueError(f"rf_qmatmul_nk failed rc={rc}")
     return c
+
+
+def rms_norm(x: np.ndarray, weight: np.ndarray, eps: float) -> np.ndarray:
+    """RMSNorm over the last axis of x[rows, hidden] (src/mlp/rms_norm_tests.rs:44-73)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    w = np.ascontiguousarray(weight, dtype=np.float32)
+    rows, hidden = x.reshape(-1, x.shape[-1]).shape
+    assert w.size == hidden
+    out = np.empty_like(x)
+    lib().rf_rms_norm(_p(x), _p(w), rows, hidden, eps, _p(out))
+    return out
+
+
+def swiglu(gate: np.ndarray, up: np.ndarray) -> np.ndarray:
+    """gate * (up * sigmoid(up)), the reference's definition (src/mlp/swiglu_tests.rs:43-66)."""
+    g = np.ascontiguousarray(gate, dtype=np.float32)
+    u = np.ascontiguousarray(up, dtype=np.float32)
+    assert g.shape == u.shape
+    out = np.empty_like(g)
+    lib().rf_swiglu(_p(g), _p(u), g.size, _p(out))
+    return out
+
+
+def dequant_rms_norm(fmt: int, packed, weight: np.ndarray, rows: int, hidden: int, eps: float) -> np.ndarray:
+    """Dequantise packed[rows, hidden], then RMSNorm each row (src/ggml/hip_backend/ops/fused_ops.rs:149-160)."""
+    d = _u8(packed)
+    w = np.ascontiguousarray(weight, dtype=np.float32)
+    assert w.size == hidden
+    out = np.empty((rows, hidden), dtype=np.float32)
+    rc = lib().rf_dequant_rms_norm(fmt, _p(d), d.size, _p(w), rows, hidden, eps, _p(out))
+    if rc != 0:
+        raise ValueError(f"rf_dequant_rms_norm failed rc={rc}")
+    return out
+
+
+def mlp_swiglu_q(fmt_gu: int, wg, wu, fmt_d: int, wd, x: np.ndarray, norm_weight, eps: float, m: int, hidden: int,
+                 inter: int) -> np.ndarray:
+    """out[m, hidden] = swiglu(xn.Wg^T, xn.Wu^T).Wd^T with xn = rms_norm(x) when norm_weight is given, else x
+    (src/backend/hip_backend/backend.rs:1153-1278 over quantised [outputs, k] matrices)."""
+    wg, wu, wd = _u8(wg), _u8(wu), _u8(wd)
+    assert wg.size == wu.size
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    assert x.size == m * hidden
+    nw = None if norm_weight is None else np.ascontiguousarray(norm_weight, dtype=np.float32)
+    scratch = np.empty(m * (hidden + 3 * inter), dtype=np.float32)
+    out = np.empty((m, hidden), dtype=np.float32)
+    rc = lib().rf_mlp_swiglu_q(fmt_gu, _p(wg), _p(wu), wg.size, fmt_d, _p(wd), wd.size, _p(x),
+                               None if nw is None else _p(nw), eps, m, hidden, inter, _p(scratch), _p(out))
+    if rc != 0:
+        raise ValueError(f"rf_mlp_swiglu_q failed rc={rc}")
+    return out
 
 
 def get_rows(fmt: int, table, tokens, n_vocab: int, n_embd: int):

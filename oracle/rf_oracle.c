@@ -17,7 +17,10 @@
  *              rf_decode_e2m1, rf_decode_e2m3, rf_encode_e2m1, rf_encode_e2m3,
  *              rf_pack_6bit, rf_unpack_6bit, rf_pack_mxfp4, rf_pack_mxfp6,
  *              rf_unpack_mxfp4, rf_unpack_mxfp6, rf_cpu_matmul_f32,
- *              rf_f16_to_f32, rf_data_size
+ *              rf_f16_to_f32, rf_data_size, rf_rms_norm, rf_swiglu (the
+ *              reference's test properties and an independent float64
+ *              evaluation), rf_dequant_rms_norm, rf_mlp_swiglu_q (compositions
+ *              of pinned parts, checked against float64)
  *   parity unpinned (no reference vector, reasoned from compiler-rt source):
  *              rf_powi_f32 for exponent -128 only (returns 0.0), hence the
  *              MXFP scale byte 0x80; rf_e8m0_from_f32 when log2 lands on an
@@ -595,4 +598,78 @@ RF_API int rf_qmatmul_nk_staged(int type, const uint8_t *w, size_t w_len, const 
     if (r) return r;
     rf_matmul_nk_f32(a, wd, m, n, k, c);
     return 0;
+}
+
+/* ------------------------------------------------------------------ */
+/* neighbours of the quantised matmul in a decode step                 */
+/* ------------------------------------------------------------------ */
+
+/* RMSNorm as the reference's CPU check states it
+ * (rms_norm_cpu_reference, src/mlp/rms_norm_tests.rs:44-73; the GPU kernel
+ * kernels/rms_norm.hip:40-84 multiplies by rsqrtf instead of dividing):
+ * per row, sum of squares in ascending order, mean = sum / hidden,
+ * rms = sqrt(mean + eps), out = (x / rms) * weight.  */
+RF_API void rf_rms_norm(const float *x, const float *weight, size_t rows, size_t hidden, float eps, float *out)
+{
+    for (size_t r = 0; r < rows; r++) {
+        const float *row = x + r * hidden;
+        float sum_sq = 0.0f;
+        for (size_t j = 0; j < hidden; j++) sum_sq += row[j] * row[j];
+        float mean_sq = sum_sq / (float)hidden;
+        float rms = sqrtf(mean_sq + eps);
+        for (size_t j = 0; j < hidden; j++) out[r * hidden + j] = (row[j] / rms) * weight[j];
+    }
+}
+
+/* SwiGLU as the reference defines it: the activation is applied to the UP
+ * projection, out = gate * (up * (1 / (1 + exp(-up))))
+ * (swiglu_cpu_reference, src/mlp/swiglu_tests.rs:43-66; kernels/swiglu.hip:40-62). */
+RF_API void rf_swiglu(const float *gate, const float *up, size_t total, float *out)
+{
+    for (size_t i = 0; i < total; i++) {
+        float u = up[i];
+        float sigmoid_up = 1.0f / (1.0f + expf(-u));
+        float swish_up = u * sigmoid_up;
+        out[i] = gate[i] * swish_up;
+    }
+}
+
+/* Dequantise rows of a packed [rows, hidden] tensor, then RMSNorm them: the
+ * arithmetic of fused_q4_0_rmsnorm (src/ggml/hip_backend/ops/fused_ops.rs:149-160,
+ * kernels/fused_dequant_rmsnorm.hip:87-163) composed from its two unfused
+ * stages, for any format of the path.  */
+RF_API int rf_dequant_rms_norm(int type, const uint8_t *packed, size_t len, const float *weight, size_t rows,
+                               size_t hidden, float eps, float *out)
+{
+    float *tmp = (float *)__builtin_malloc(rows * hidden * sizeof(float));
+    if (!tmp) return -3;
+    int r = rf_dequantize(type, packed, len, rows * hidden, tmp);
+    if (r == 0) rf_rms_norm(tmp, weight, rows, hidden, eps, out);
+    __builtin_free(tmp);
+    return r;
+}
+
+/* The SwiGLU MLP of HipBackend::mlp_swiglu (src/backend/hip_backend/backend.rs:1153-1278:
+ * gate = x.Wg, up = x.Wu, h = swiglu(gate, up), out = h.Wd) with the three
+ * matrices quantised and stored [outputs, k] as the quantised matmuls take
+ * them (matmul_q4_0, src/kernels/matmul/quantized/q4_0.rs:139-148), each
+ * product being dequantise + naive matmul as in rf_qmatmul_nk.  norm_weight
+ * (optional) applies rf_rms_norm to x first, the step that precedes the MLP in
+ * a decoder layer.  scratch: m * (hidden + 3 * inter) floats.  */
+RF_API int rf_mlp_swiglu_q(int type_gu, const uint8_t *wg, const uint8_t *wu, size_t gu_len, int type_d,
+                           const uint8_t *wd, size_t d_len, const float *x, const float *norm_weight, float eps,
+                           size_t m, size_t hidden, size_t inter, float *scratch, float *out)
+{
+    float *xn = scratch, *g = xn + m * hidden, *u = g + m * inter, *h = u + m * inter;
+    const float *xin = x;
+    if (norm_weight) {
+        rf_rms_norm(x, norm_weight, m, hidden, eps, xn);
+        xin = xn;
+    }
+    int r = rf_qmatmul_nk(type_gu, wg, gu_len, xin, m, inter, hidden, NULL, 0, g);
+    if (r) return r;
+    r = rf_qmatmul_nk(type_gu, wu, gu_len, xin, m, inter, hidden, NULL, 0, u);
+    if (r) return r;
+    rf_swiglu(g, u, m * inter, h);
+    return rf_qmatmul_nk(type_d, wd, d_len, h, m, hidden, inter, NULL, 0, out);
 }

@@ -44,6 +44,12 @@ _SIGNATURES = {
     "rfq_matmul_q4_k": ([_vp, _vp, _vp, _i, _i, _i, _vp], _i),
     "rfq_matmul_q6_k": ([_vp, _vp, _vp, _i, _i, _i, _vp], _i),
     "rfq_matmul_host_weights": ([_i, _vp, _sz, _vp, _sz, _sz, _vp, _vp], _i),
+    "rfq_rms_norm": ([_vp, _vp, _vp, _i, _i, C.c_float, _vp], _i),
+    "rfq_swiglu": ([_vp, _vp, _vp, _i, _i, _vp], _i),
+    "rfq_dequant_rms_norm": ([_i, _vp, _sz, _vp, _vp, _i, _i, C.c_float, _vp], _i),
+    "rfq_rms_norm_gemv": ([_i, _vp, _sz, _vp, _vp, C.c_float, _vp, _i, _i, _i, _vp, _vp], _i),
+    "rfq_mlp_scratch_bytes": ([_i, _i, _i], _sz),
+    "rfq_mlp_swiglu": ([_i, _vp, _vp, _sz, _i, _vp, _sz, _vp, _vp, C.c_float, _vp, _i, _i, _i, _vp, _sz, _vp], _i),
     "rfq_gemm_f16": ([_i, _vp, _sz, _vp, _vp, _i, _i, _i, _i, _vp], _i),
     "rfq_mx_prepared_bytes": ([_i, _i, _i, _i], _sz),
     "rfq_mx_prepare": ([_i, _i, _vp, _sz, _i, _i, _vp, _sz, C.POINTER(C.c_int), _vp], _i),

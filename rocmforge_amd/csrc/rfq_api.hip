@@ -216,6 +216,129 @@ int rfq_matmul_host_weights(int fmt, const uint8_t *h_w, size_t w_bytes, const f
     return RFQ_OK;
 }
 
+static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int rfq_rms_norm(const float *d_input, const float *d_weight, float *d_output, int seq_len, int hidden_size, float eps,
+                 void *stream)
+{
+    if (seq_len < 0 || hidden_size <= 0)
+        return fail(RFQ_E_BADARG, "rfq_rms_norm: seq_len=%d hidden_size=%d", seq_len, hidden_size);
+    if (hidden_size % 4 != 0) return fail(RFQ_E_SIZE, "rfq_rms_norm: hidden_size=%d is not a multiple of 4", hidden_size);
+    if (seq_len == 0) return RFQ_OK;
+    if (!d_input || !d_weight || !d_output) return fail(RFQ_E_BADARG, "rfq_rms_norm: null pointer");
+    if (!aligned16(d_input) || !aligned16(d_weight) || !aligned16(d_output))
+        return fail(RFQ_E_BADARG, "rfq_rms_norm: input, weight and output must be 16-byte aligned");
+    return launch_rms_norm(RFQ_TABLE_F32, d_input, d_weight, d_output, seq_len, hidden_size, eps, (hipStream_t)stream);
+}
+
+int rfq_swiglu(const float *d_gate, const float *d_up, float *d_output, int seq_len, int intermediate_size, void *stream)
+{
+    if (seq_len < 0 || intermediate_size < 0)
+        return fail(RFQ_E_BADARG, "rfq_swiglu: seq_len=%d intermediate_size=%d", seq_len, intermediate_size);
+    const size_t total = (size_t)seq_len * (size_t)intermediate_size;
+    if (total == 0) return RFQ_OK;
+    if (!d_gate || !d_up || !d_output) return fail(RFQ_E_BADARG, "rfq_swiglu: null pointer");
+    return launch_swiglu(d_gate, d_up, d_output, total, (hipStream_t)stream);
+}
+
+int rfq_dequant_rms_norm(int fmt, const void *d_packed, size_t packed_bytes, const float *d_weight, float *d_output,
+                         int seq_len, int hidden_size, float eps, void *stream)
+{
+    if (!known_format(fmt)) return fail(RFQ_E_BADARG, "rfq_dequant_rms_norm: unknown format %d", fmt);
+    if (seq_len < 0 || hidden_size <= 0)
+        return fail(RFQ_E_BADARG, "rfq_dequant_rms_norm: seq_len=%d hidden_size=%d", seq_len, hidden_size);
+    const size_t need = matrix_bytes(fmt, seq_len > 0 ? seq_len : 1, hidden_size);
+    if (need == 0)
+        return fail(RFQ_E_SIZE, "rfq_dequant_rms_norm: hidden_size=%d is not a multiple of the %d-element block", hidden_size,
+                    fmt_block_elems(fmt));
+    if (seq_len == 0) return RFQ_OK;
+    if (packed_bytes != need)
+        return fail(RFQ_E_SIZE, "rfq_dequant_rms_norm: input has %zu bytes, [%d x %d] needs %zu", packed_bytes, seq_len,
+                    hidden_size, need);
+    if (!d_packed || !d_weight || !d_output) return fail(RFQ_E_BADARG, "rfq_dequant_rms_norm: null pointer");
+    if (!aligned16(d_weight) || !aligned16(d_output))
+        return fail(RFQ_E_BADARG, "rfq_dequant_rms_norm: weight and output must be 16-byte aligned");
+    return launch_rms_norm(fmt, d_packed, d_weight, d_output, seq_len, hidden_size, eps, (hipStream_t)stream);
+}
+
+int rfq_rms_norm_gemv(int fmt, const void *d_w, size_t w_bytes, const float *d_x, const float *d_norm_weight, float eps,
+                      float *d_y, int m, int n, int k, float *d_scratch, void *stream)
+{
+    int rc = check_gemv("rfq_rms_norm_gemv", fmt, d_w, w_bytes, true, d_x, d_y, m, n, k);
+    if (rc != RFQ_OK) return rc;
+    if (!d_norm_weight) return fail(RFQ_E_BADARG, "rfq_rms_norm_gemv: null norm weight");
+    if (m > 8) return fail(RFQ_E_UNSUPPORTED, "rfq_rms_norm_gemv: m=%d > 8", m);
+    hipStream_t s = (hipStream_t)stream;
+    if (m == 1) {
+        rc = launch_gemv_fused(fmt, (const uint8_t *)d_w, nullptr, d_x, d_norm_weight, eps, d_y, n, k, s);
+        if (rc != RFQ_E_UNSUPPORTED) return rc;
+    }
+    if (!d_scratch) return fail(RFQ_E_BADARG, "rfq_rms_norm_gemv: m=%d k=%d needs d_scratch (m * k floats)", m, k);
+    if (k % 4 != 0 || !aligned16(d_x) || !aligned16(d_norm_weight) || !aligned16(d_scratch))
+        return fail(RFQ_E_BADARG, "rfq_rms_norm_gemv: x, norm weight and scratch must be 16-byte aligned, k a multiple of 4");
+    rc = launch_rms_norm(RFQ_TABLE_F32, d_x, d_norm_weight, d_scratch, m, k, eps, s);
+    if (rc != RFQ_OK) return rc;
+    return launch_gemv(fmt, (const uint8_t *)d_w, d_scratch, d_y, m, n, k, s);
+}
+
+// scratch layout: h[m, inter] | xn[m, hidden] | gate[m, inter] | up[m, inter], each rounded to 16 bytes
+static size_t pad16(size_t b) { return (b + 15) & ~(size_t)15; }
+
+size_t rfq_mlp_scratch_bytes(int m, int hidden_size, int intermediate_size)
+{
+    if (m <= 0 || hidden_size <= 0 || intermediate_size <= 0) return 0;
+    return 3 * pad16((size_t)m * intermediate_size * 4) + pad16((size_t)m * hidden_size * 4);
+}
+
+int rfq_mlp_swiglu(int fmt_gate_up, const void *d_gate_w, const void *d_up_w, size_t gate_up_bytes, int fmt_down,
+                   const void *d_down_w, size_t down_bytes, const float *d_x, const float *d_norm_weight, float eps,
+                   float *d_out, int m, int hidden_size, int intermediate_size, void *d_scratch, size_t scratch_bytes,
+                   void *stream)
+{
+    int rc = check_gemv("rfq_mlp_swiglu (gate)", fmt_gate_up, d_gate_w, gate_up_bytes, true, d_x, d_out, m,
+                        intermediate_size, hidden_size);
+    if (rc != RFQ_OK) return rc;
+    rc = check_gemv("rfq_mlp_swiglu (up)", fmt_gate_up, d_up_w, gate_up_bytes, true, d_x, d_out, m, intermediate_size,
+                    hidden_size);
+    if (rc != RFQ_OK) return rc;
+    rc = check_gemv("rfq_mlp_swiglu (down)", fmt_down, d_down_w, down_bytes, true, d_x, d_out, m, hidden_size,
+                    intermediate_size);
+    if (rc != RFQ_OK) return rc;
+    if (m > 8) return fail(RFQ_E_UNSUPPORTED, "rfq_mlp_swiglu: m=%d > 8", m);
+    const size_t need = rfq_mlp_scratch_bytes(m, hidden_size, intermediate_size);
+    if (!d_scratch || scratch_bytes < need || !aligned16(d_scratch))
+        return fail(RFQ_E_SIZE, "rfq_mlp_swiglu: scratch of %zu bytes (16-byte aligned) needed, %zu given", need,
+                    scratch_bytes);
+    hipStream_t s = (hipStream_t)stream;
+    const size_t mi = pad16((size_t)m * intermediate_size * 4);
+    uint8_t *base = static_cast<uint8_t *>(d_scratch);
+    float *h = reinterpret_cast<float *>(base);
+    float *xn = reinterpret_cast<float *>(base + mi);
+    float *gate = reinterpret_cast<float *>(base + mi + pad16((size_t)m * hidden_size * 4));
+    float *up = reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(gate) + mi);
+    rc = RFQ_E_UNSUPPORTED;
+    if (m == 1)
+        rc = launch_gemv_fused(fmt_gate_up, (const uint8_t *)d_gate_w, (const uint8_t *)d_up_w, d_x, d_norm_weight, eps, h,
+                               intermediate_size, hidden_size, s);
+    if (rc == RFQ_E_UNSUPPORTED) {
+        const float *xin = d_x;
+        if (d_norm_weight) {
+            if (hidden_size % 4 != 0 || !aligned16(d_x) || !aligned16(d_norm_weight))
+                return fail(RFQ_E_BADARG, "rfq_mlp_swiglu: x and norm weight must be 16-byte aligned, hidden_size a multiple of 4");
+            rc = launch_rms_norm(RFQ_TABLE_F32, d_x, d_norm_weight, xn, m, hidden_size, eps, s);
+            if (rc != RFQ_OK) return rc;
+            xin = xn;
+        }
+        rc = launch_gemv(fmt_gate_up, (const uint8_t *)d_gate_w, xin, gate, m, intermediate_size, hidden_size, s);
+        if (rc != RFQ_OK) return rc;
+        rc = launch_gemv(fmt_gate_up, (const uint8_t *)d_up_w, xin, up, m, intermediate_size, hidden_size, s);
+        if (rc != RFQ_OK) return rc;
+        rc = launch_swiglu(gate, up, h, (size_t)m * intermediate_size, s);
+    }
+    if (rc != RFQ_OK) return rc;
+    return launch_gemv(fmt_down, (const uint8_t *)d_down_w, h, d_out, m, hidden_size, intermediate_size, s);
+}
+
 int rfq_gemm_f16(int fmt, const void *d_w, size_t w_bytes, const void *d_a_f16, void *d_out, int out_dtype, int m,
                  int n, int k, void *stream)
 {

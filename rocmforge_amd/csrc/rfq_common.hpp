@@ -67,7 +67,13 @@ int release_workspaces();
 int launch_dequant(int fmt, const uint8_t *d_in, size_t in_bytes, float *d_out, size_t n, hipStream_t s);
 int launch_get_rows(int fmt, const void *d_table, int n_vocab, int n_embd, const uint32_t *d_tokens, int n_tokens,
                     float *d_out, int *d_status, hipStream_t s);
+// src_fmt: RFQ_TABLE_F32 for f32 rows, else a packed format whose rows are decoded on the fly.
+int launch_rms_norm(int src_fmt, const void *d_x, const float *d_weight, float *d_out, int rows, int hidden, float eps,
+                    hipStream_t s);
+int launch_swiglu(const float *d_gate, const float *d_up, float *d_out, size_t total, hipStream_t s);
 int launch_gemv(int fmt, const uint8_t *d_w, const float *d_x, float *d_y, int m, int n, int k, hipStream_t s);
+int launch_gemv_fused(int fmt, const uint8_t *d_w, const uint8_t *d_w2, const float *d_x, const float *d_norm_w,
+                      float eps, float *d_y, int n, int k, hipStream_t s);
 int launch_gemm_f16(int fmt, const uint8_t *d_w, const void *d_a, void *d_out, int out_dtype, int m, int n,
                     int k, hipStream_t s);
 size_t mx_prepared_bytes(int fmt, int kind, int rows, int k);

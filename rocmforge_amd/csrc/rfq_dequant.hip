@@ -296,7 +296,109 @@ int run(const uint8_t *d_in, size_t in_bytes, float *d_out, size_t n, hipStream_
     return RFQ_OK;
 }
 
+// ---- neighbours of the matmul in a decoder layer --------------------------------
+//
+// RMSNorm (kernels/rms_norm.hip:40-84; CPU statement src/mlp/rms_norm_tests.rs:44-73):
+// out[r, j] = (x[r, j] / sqrt(mean_j x[r, j]^2 + eps)) * weight[j].  One workgroup
+// per row; the row is read twice (the second read is served by the cache).
+// SRC_FMT != 0 decodes the row from packed blocks instead of reading f32
+// (fused_q4_0_rmsnorm, src/ggml/hip_backend/ops/fused_ops.rs:149-160, for every format).
+
+__device__ __forceinline__ float block_sum_256(float v, float *lds4)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+    if ((threadIdx.x & 63) == 0) lds4[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return (lds4[0] + lds4[1]) + (lds4[2] + lds4[3]);
+}
+
+template <int SRC_FMT> __device__ __forceinline__ float4 norm_src_quad(const void *row, int q)
+{
+    if constexpr (SRC_FMT == RFQ_TABLE_F32) {
+        return *(reinterpret_cast<const float4 *>(row) + q);
+    } else {
+        constexpr int QPB = Fmt<SRC_FMT>::BE / 4;
+        return decode_quad<SRC_FMT>(static_cast<const uint8_t *>(row) + (size_t)(q / QPB) * Fmt<SRC_FMT>::BB, (q % QPB) * 4);
+    }
+}
+
+template <int SRC_FMT>
+__global__ void __launch_bounds__(256)
+rms_norm_kernel(const void *__restrict__ x, size_t row_stride_bytes, const float *__restrict__ weight,
+                float *__restrict__ out, int hidden, float eps)
+{
+    __shared__ float red[4];
+    const void *row = static_cast<const uint8_t *>(x) + (size_t)blockIdx.x * row_stride_bytes;
+    float *o = out + (size_t)blockIdx.x * hidden;
+    const int quads = hidden >> 2;
+    float ss = 0.0f;
+    for (int q = threadIdx.x; q < quads; q += 256) {
+        float4 v = norm_src_quad<SRC_FMT>(row, q);
+        ss += v.x * v.x; ss += v.y * v.y; ss += v.z * v.z; ss += v.w * v.w;
+    }
+    const float total = block_sum_256(ss, red);
+    const float rms = sqrtf(total / (float)hidden + eps);
+    for (int q = threadIdx.x; q < quads; q += 256) {
+        float4 v = norm_src_quad<SRC_FMT>(row, q);
+        float4 w = *(reinterpret_cast<const float4 *>(weight) + q);
+        float4 r;
+        r.x = (v.x / rms) * w.x; r.y = (v.y / rms) * w.y; r.z = (v.z / rms) * w.z; r.w = (v.w / rms) * w.w;
+        *(reinterpret_cast<float4 *>(o) + q) = r;
+    }
+}
+
+// SwiGLU as the reference defines it (kernels/swiglu.hip:40-62): the activation
+// is applied to the UP projection, out = gate * (up * 1 / (1 + exp(-up))).
+__global__ void __launch_bounds__(256)
+swiglu_kernel(const float *__restrict__ gate, const float *__restrict__ up, float *__restrict__ out, size_t total)
+{
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    float u = up[i];
+    float sigmoid_up = 1.0f / (1.0f + expf(-u));
+    out[i] = gate[i] * (u * sigmoid_up);
+}
+
+template <int SRC_FMT>
+int run_rms_norm(const void *x, size_t row_stride_bytes, const float *weight, float *out, int rows, int hidden, float eps,
+                 hipStream_t s)
+{
+    hipLaunchKernelGGL((rms_norm_kernel<SRC_FMT>), dim3((unsigned)rows), dim3(256), 0, s, x, row_stride_bytes, weight, out,
+                       hidden, eps);
+    RFQ_LAUNCH_CHECK("rms_norm_kernel");
+    return RFQ_OK;
+}
+
 } // namespace
+
+int launch_rms_norm(int src_fmt, const void *d_x, const float *d_weight, float *d_out, int rows, int hidden, float eps,
+                    hipStream_t s)
+{
+    if (rows == 0) return RFQ_OK;
+    const int be = src_fmt == RFQ_TABLE_F32 ? 4 : fmt_block_elems(src_fmt);
+    const size_t stride = src_fmt == RFQ_TABLE_F32 ? (size_t)hidden * 4 : (size_t)(hidden / be) * fmt_block_bytes(src_fmt);
+    switch (canonical_format(src_fmt)) {
+    case RFQ_TABLE_F32: return run_rms_norm<RFQ_TABLE_F32>(d_x, stride, d_weight, d_out, rows, hidden, eps, s);
+    case RFQ_Q4_0: return run_rms_norm<RFQ_Q4_0>(d_x, stride, d_weight, d_out, rows, hidden, eps, s);
+    case RFQ_Q8_0: return run_rms_norm<RFQ_Q8_0>(d_x, stride, d_weight, d_out, rows, hidden, eps, s);
+    case RFQ_Q4_K: return run_rms_norm<RFQ_Q4_K>(d_x, stride, d_weight, d_out, rows, hidden, eps, s);
+    case RFQ_Q6_K: return run_rms_norm<RFQ_Q6_K>(d_x, stride, d_weight, d_out, rows, hidden, eps, s);
+    case RFQ_MXFP4: return run_rms_norm<RFQ_MXFP4>(d_x, stride, d_weight, d_out, rows, hidden, eps, s);
+    case RFQ_MXFP6_E2M3: return run_rms_norm<RFQ_MXFP6_E2M3>(d_x, stride, d_weight, d_out, rows, hidden, eps, s);
+    default: return fail(RFQ_E_BADARG, "rms_norm: unknown source format %d", src_fmt);
+    }
+}
+
+int launch_swiglu(const float *d_gate, const float *d_up, float *d_out, size_t total, hipStream_t s)
+{
+    if (total == 0) return RFQ_OK;
+    const size_t grid = (total + 255) / 256;
+    if (grid > 0x7fffffffu) return fail(RFQ_E_SIZE, "rfq_swiglu: %zu elements exceed one launch", total);
+    hipLaunchKernelGGL(swiglu_kernel, dim3((unsigned)grid), dim3(256), 0, s, d_gate, d_up, d_out, total);
+    RFQ_LAUNCH_CHECK("swiglu_kernel");
+    return RFQ_OK;
+}
 
 int launch_dequant(int fmt, const uint8_t *d_in, size_t in_bytes, float *d_out, size_t n, hipStream_t s)
 {

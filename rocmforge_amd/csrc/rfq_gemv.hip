@@ -61,6 +61,12 @@ __device__ __forceinline__ float wave_sum(float v)
     return (r0 + r1) + (r2 + r3);
 }
 
+// The value of the neighbouring lane (lane ^ 1).
+__device__ __forceinline__ float dpp_xor1_f(float v)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true));
+}
+
 // ---- units: 32 consecutive k of one row -------------------------------------
 //
 // Unit<FMT>::load(row, u)  fetches unit u of the row starting at `row`.
@@ -285,6 +291,90 @@ __device__ __forceinline__ float sum32(const float (&x)[32])
     return (a + b) + (c + d);
 }
 
+// ---- optional fusion around the m == 1 kernels -------------------------------
+//
+// FUSE kernels take two run-time options.  norm_w != nullptr: the vector that
+// is multiplied is RMSNorm(x) * norm_w (kernels/rms_norm.hip:40-84) instead
+// of x; since the normalisation is one factor 1 / sqrt(mean(x^2) + eps) for the
+// whole vector, x * norm_w goes through the dot products and the factor is
+// applied to each result.  glu != 0: the n rows are an interleaving of two
+// matrices (row 2j = row j of w, row 2j+1 = row j of w2: gate and up
+// projections sharing x) and y[j] = swiglu(row 2j, row 2j+1) as the reference
+// defines it (kernels/swiglu.hip:40-62): gate * (up * sigmoid(up)).
+struct GemvFuse {
+    const uint8_t *w2;
+    const float *norm_w;
+    float eps;
+    int glu;
+};
+
+__device__ __forceinline__ float swiglu_ref(float gate, float up)
+{
+    return gate * (up * (1.0f / (1.0f + expf(-up))));
+}
+
+// Row r of the (possibly interleaved) matrix.
+template <bool FUSE>
+__device__ __forceinline__ const uint8_t *fused_row(const uint8_t *w, const GemvFuse &f, int r, size_t rb)
+{
+    if constexpr (FUSE) {
+        if (f.glu) return ((r & 1) ? f.w2 : w) + (size_t)(r >> 1) * rb;
+    }
+    return w + (size_t)r * rb;
+}
+
+// Results of one group of R rows (res[i] valid in every lane of each of the
+// team's WPR wavefronts) go to y.  `part` is [R][4] floats of LDS; with
+// WPR > 1 every wavefront of the block must call this the same number of times.
+template <int R, int WPR, bool FUSE>
+__device__ __forceinline__ void store_group(const float (&res)[R], float (*part)[4], float *__restrict__ y, int row_first,
+                                            int row_end, int lane, int wave, const GemvFuse &f, float rinv)
+{
+    const int team = wave / WPR, wit = wave % WPR;
+    if (WPR == 1) {
+        if (lane == 0) {
+            if (FUSE && f.glu) {
+#pragma unroll
+                for (int i = 0; i + 1 < R; i += 2) {
+                    int r = row_first + i;
+                    if (r < row_end) y[r >> 1] = swiglu_ref(res[i] * rinv, res[i + 1] * rinv);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < R; i++) {
+                    int r = row_first + i;
+                    if (r < row_end) y[r] = FUSE ? res[i] * rinv : res[i];
+                }
+            }
+        }
+    } else {
+        if (lane == 0) {
+#pragma unroll
+            for (int i = 0; i < R; i++) part[i][wave] = res[i];
+        }
+        __syncthreads();
+        if (wit == 0) {
+            const int li = lane < R ? lane : R - 1;
+            int r = row_first + li;
+            float t = 0.f;
+#pragma unroll
+            for (int q = 0; q < WPR; q++) t += part[li][team * WPR + q];
+            if (FUSE) {
+                t *= rinv;
+                float other = dpp_xor1_f(t);           // the up row's result sits in the odd neighbour lane
+                if (f.glu) {
+                    if (lane < R && (lane & 1) == 0 && r < row_end) y[r >> 1] = swiglu_ref(t, other);
+                } else if (lane < R && r < row_end) {
+                    y[r] = t;
+                }
+            } else if (lane < R && r < row_end) {
+                y[r] = t;
+            }
+        }
+        __syncthreads();
+    }
+}
+
 // ---- m == 1, x resident in registers ----------------------------------------
 //
 // Block = 4 wavefronts = 4 / WPR teams.  Lane `tl` of a team (0 .. 64*WPR-1)
@@ -297,10 +387,10 @@ __device__ __forceinline__ float sum32(const float (&x)[32])
 // their result is dropped; lanes past the end of a row do the same with the
 // row's last unit.  HBM latency, not bandwidth, bounds a wavefront that has a
 // single row in flight, hence the depth.
-template <int FMT, int UPL, int WPR, int R>
+template <int FMT, int UPL, int WPR, int R, bool FUSE>
 __global__ void __launch_bounds__(256)
 gemv_xreg_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ y, int n, int k,
-                 int groups)
+                 int groups, GemvFuse f)
 {
     constexpr int TEAMS = 4 / WPR, TL = 64 * WPR;
     constexpr int D = R < 3 ? R : 3;
@@ -320,6 +410,12 @@ gemv_xreg_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
         unit[j] = live[j] ? u : ku - 1;
         load_x32(x + (size_t)unit[j] * 32, xs[j]);
     }
+    const bool norm = FUSE && f.norm_w != nullptr;
+    float nws[FUSE ? UPL : 1][32];
+    if (norm) {
+#pragma unroll
+        for (int j = 0; j < UPL; j++) load_x32(f.norm_w + (size_t)unit[j] * 32, nws[FUSE ? j : 0]);
+    }
 
     __shared__ float part[R][4];
     const int rows_per_team = groups * R;
@@ -332,7 +428,7 @@ gemv_xreg_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
     auto load_row = [&](int slot, int i) {
         int r = row0 + i;
         if (r > row_last) r = row_last;
-        const uint8_t *row = w + (size_t)r * rb;
+        const uint8_t *row = fused_row<FUSE>(w, f, r, rb);
 #pragma unroll
         for (int j = 0; j < UPL; j++) buf[slot][j].load(row, unit[j]);
     };
@@ -340,6 +436,31 @@ gemv_xreg_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
     // weight loads are already in flight while the x sums are formed.
 #pragma unroll
     for (int d = 0; d < D; d++) load_row(d, d);
+    float rinv = 1.0f;
+    if (norm) {
+        // every team holds all of x: its own sum of squares, no exchange between teams
+        float ssq = 0.f;
+#pragma unroll
+        for (int j = 0; j < UPL; j++) {
+            float sj = 0.f;
+#pragma unroll
+            for (int i = 0; i < 32; i++) {
+                sj = __builtin_fmaf(xs[j][i], xs[j][i], sj);
+                xs[j][i] *= nws[FUSE ? j : 0][i];
+            }
+            ssq += live[j] ? sj : 0.f;
+        }
+        ssq = wave_sum(ssq);
+        if (WPR > 1) {
+            if (lane == 0) part[0][wave] = ssq;
+            __syncthreads();
+            ssq = 0.f;
+#pragma unroll
+            for (int q = 0; q < WPR; q++) ssq += part[0][team * WPR + q];
+            __syncthreads();
+        }
+        rinv = 1.0f / sqrtf(ssq / (float)k + f.eps);
+    }
 #pragma unroll
     for (int j = 0; j < UPL; j++) xsum[j] = Unit<FMT>::NEEDS_XSUM ? sum32(xs[j]) : 0.f;
 
@@ -361,31 +482,8 @@ gemv_xreg_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
             if (i + D < R) load_row(i % D, base + i + D); // the slot just consumed takes the row D further on
             res[i] = wave_sum(acc);
         }
-        if (WPR == 1) {
-            if (lane == 0) {
-#pragma unroll
-                for (int i = 0; i < R; i++) {
-                    int r = row0 + base + i;
-                    if (r < row_end) y[r] = res[i];
-                }
-            }
-        } else {
-            // `groups` is uniform over the block, so every wavefront reaches
-            // both barriers the same number of times.
-            if (lane == 0) {
-#pragma unroll
-                for (int i = 0; i < R; i++) part[i][wave] = res[i];
-            }
-            __syncthreads();
-            if (wit == 0 && lane < R) {
-                int r = row0 + base + lane;
-                float t = 0.f;
-#pragma unroll
-                for (int q = 0; q < WPR; q++) t += part[lane][team * WPR + q];
-                if (r < row_end) y[r] = t;
-            }
-            __syncthreads();
-        }
+        // (`groups` is uniform over the block: every wavefront stores the same number of groups)
+        store_group<R, WPR, FUSE>(res, part, y, row0 + base, row_end, lane, wave, f, rinv);
     }
 }
 
@@ -408,11 +506,6 @@ gemv_xreg_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
 // LDS holds, per unit, 24 limb dwords + s + sum(x) (stride 28 dwords).
 
 struct XPrep { uint32_t l[24]; float s, xsum; };
-
-__device__ __forceinline__ float dpp_xor1_f(float v)
-{
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true));
-}
 
 // Byte-transpose four 24-bit integers into (low, mid, top) limb dwords.
 __device__ __forceinline__ void limbs4(uint32_t x0, uint32_t x1, uint32_t x2, uint32_t x3, uint32_t *out3)
@@ -550,10 +643,10 @@ template <> struct IUnit<RFQ_Q8_0> : Unit<RFQ_Q8_0> {
 // accepts only so many outstanding requests and later loads just block issue.
 // Rows past the end re-read the team's last valid row (a cache hit) and their
 // result is dropped; so do lanes past the end of a row with the last unit.
-template <int FMT, int UPL, int WPR, int R>
+template <int FMT, int UPL, int WPR, int R, bool FUSE>
 __global__ void __launch_bounds__(256)
 gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ y, int n, int k,
-                 int groups)
+                 int groups, GemvFuse f)
 {
     RFQ_TS(0);
     using IU = IUnit<FMT>;
@@ -581,15 +674,19 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
     const int row_last = row_end > row0 ? row_end - 1 : (n - 1);
 
     // x goes first so that it also returns first.
-    float xv[16];
+    float xv[16], nv[FUSE ? 16 : 1];
     const bool prep0 = (int)threadIdx.x < 2 * ku;
+    const bool norm = FUSE && f.norm_w != nullptr;
     if (prep0) prep_load(x + (size_t)threadIdx.x * 16, xv);
+    if constexpr (FUSE) {
+        if (norm && prep0) prep_load(f.norm_w + (size_t)threadIdx.x * 16, nv);
+    }
 
     IU buf[D][UPL];
     auto load_row = [&](int slot, int i) {
         int r = row0 + i;
         if (r > row_last) r = row_last;
-        const uint8_t *row = w + (size_t)r * rb;
+        const uint8_t *row = fused_row<FUSE>(w, f, r, rb);
 #pragma unroll
         for (int j = 0; j < UPL; j++) buf[slot][j].load(row, unit[j]);
     };
@@ -598,14 +695,40 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
     RFQ_TS(1);
 
     // Cooperative conversion of x: 2*ku half-units over the 256 threads.
+    float ssq = 0.f;
+    if constexpr (FUSE) {
+        if (norm && prep0) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) { ssq = __builtin_fmaf(xv[i], xv[i], ssq); xv[i] *= nv[i]; }
+        }
+    }
     if (prep0) prep_convert<IU::NIBBLE, IU::TOPOFF>(xv, threadIdx.x & 1, xlds + (size_t)(threadIdx.x >> 1) * 28);
     for (int h = threadIdx.x + 256; h < 2 * ku; h += 256) {
         float xw[16];
         prep_load(x + (size_t)h * 16, xw);
+        if constexpr (FUSE) {
+            if (norm) {
+                float nw[16];
+                prep_load(f.norm_w + (size_t)h * 16, nw);
+#pragma unroll
+                for (int i = 0; i < 16; i++) { ssq = __builtin_fmaf(xw[i], xw[i], ssq); xw[i] *= nw[i]; }
+            }
+        }
         prep_convert<IU::NIBBLE, IU::TOPOFF>(xw, h & 1, xlds + (size_t)(h >> 1) * 28);
+    }
+    __shared__ float ssq_part[4];
+    if constexpr (FUSE) {
+        if (norm) {
+            ssq = wave_sum(ssq);
+            if (lane == 0) ssq_part[wave] = ssq;
+        }
     }
     RFQ_TS(2);
     __syncthreads();
+    float rinv = 1.0f;
+    if constexpr (FUSE) {
+        if (norm) rinv = 1.0f / sqrtf(((ssq_part[0] + ssq_part[1]) + (ssq_part[2] + ssq_part[3])) / (float)k + f.eps);
+    }
     XPrep xp[UPL];
 #pragma unroll
     for (int j = 0; j < UPL; j++) {
@@ -640,31 +763,8 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
             res[i] = wave_sum(acc);
         }
         RFQ_TS(4);
-        if (WPR == 1) {
-            if (lane == 0) {
-#pragma unroll
-                for (int i = 0; i < R; i++) {
-                    int r = row0 + base + i;
-                    if (r < row_end) y[r] = res[i];
-                }
-            }
-        } else {
-            // `groups` is uniform over the block, so every wavefront reaches
-            // both barriers the same number of times.
-            if (lane == 0) {
-#pragma unroll
-                for (int i = 0; i < R; i++) part[i][wave] = res[i];
-            }
-            __syncthreads();
-            if (wit == 0 && lane < R) {
-                int r = row0 + base + lane;
-                float t = 0.f;
-#pragma unroll
-                for (int q = 0; q < WPR; q++) t += part[lane][team * WPR + q];
-                if (r < row_end) y[r] = t;
-            }
-            __syncthreads();
-        }
+        // (`groups` is uniform over the block: every wavefront stores the same number of groups)
+        store_group<R, WPR, FUSE>(res, part, y, row0 + base, row_end, lane, wave, f, rinv);
     }
 }
 
@@ -973,7 +1073,7 @@ gemv_generic_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, 
 // with R from a small compiled set; the pair that wastes the fewest row slots
 // wins, the larger R on a tie.
 struct RowPlan { int r, groups, blocks; };
-inline RowPlan plan_rows(int n, int teams, int per_cu)
+inline RowPlan plan_rows(int n, int teams, int per_cu, bool even_only = false)
 {
     const int slots = device_cu_count() * per_cu;
     int want = (n + slots * teams - 1) / (slots * teams);
@@ -983,6 +1083,7 @@ inline RowPlan plan_rows(int n, int teams, int per_cu)
     long best_cost = -1;
     for (int idx = 0; idx < 6; idx++) {
         int r = RS[idx];
+        if (even_only && (r & 1)) continue;
         int groups = (want + r - 1) / r;
         int blocks = (n + teams * r * groups - 1) / (teams * r * groups);
         long waves_of_blocks = (blocks + slots - 1) / slots;
@@ -995,25 +1096,28 @@ inline RowPlan plan_rows(int n, int teams, int per_cu)
     return best;
 }
 
-template <int FMT, int UPL, int WPR, int R>
-int launch_xreg(const uint8_t *w, const float *x, float *y, int n, int k, const RowPlan &p, hipStream_t s)
+template <int FMT, int UPL, int WPR, int R, bool FUSE>
+int launch_xreg(const uint8_t *w, const float *x, float *y, int n, int k, const RowPlan &p, const GemvFuse &f,
+                hipStream_t s)
 {
-    hipLaunchKernelGGL((gemv_xreg_kernel<FMT, UPL, WPR, R>), dim3(p.blocks), dim3(256), 0, s, w, x, y, n, k, p.groups);
+    hipLaunchKernelGGL((gemv_xreg_kernel<FMT, UPL, WPR, R, FUSE>), dim3(p.blocks), dim3(256), 0, s, w, x, y, n, k,
+                       p.groups, f);
     RFQ_LAUNCH_CHECK("gemv_xreg_kernel");
     return RFQ_OK;
 }
 
-template <int FMT, int UPL, int WPR>
-int run_xreg(const uint8_t *w, const float *x, float *y, int n, int k, hipStream_t s)
+// FUSE launches with f.glu set need an even R: the two rows of a pair are reduced together.
+template <int FMT, int UPL, int WPR, bool FUSE>
+int run_xreg(const uint8_t *w, const float *x, float *y, int n, int k, const GemvFuse &f, hipStream_t s)
 {
-    const RowPlan p = plan_rows(n, 4 / WPR, 2); // (three blocks per CU fit for Q6_K but run slower)
+    const RowPlan p = plan_rows(n, 4 / WPR, 2, FUSE && f.glu); // (three blocks per CU fit for Q6_K but run slower)
     switch (p.r) {
-    case 2: return launch_xreg<FMT, UPL, WPR, 2>(w, x, y, n, k, p, s);
-    case 4: return launch_xreg<FMT, UPL, WPR, 4>(w, x, y, n, k, p, s);
-    case 5: return launch_xreg<FMT, UPL, WPR, 5>(w, x, y, n, k, p, s);
-    case 6: return launch_xreg<FMT, UPL, WPR, 6>(w, x, y, n, k, p, s);
-    case 7: return launch_xreg<FMT, UPL, WPR, 7>(w, x, y, n, k, p, s);
-    default: return launch_xreg<FMT, UPL, WPR, 8>(w, x, y, n, k, p, s);
+    case 2: return launch_xreg<FMT, UPL, WPR, 2, FUSE>(w, x, y, n, k, p, f, s);
+    case 4: return launch_xreg<FMT, UPL, WPR, 4, FUSE>(w, x, y, n, k, p, f, s);
+    case 5: return launch_xreg<FMT, UPL, WPR, 5, FUSE>(w, x, y, n, k, p, f, s);
+    case 6: return launch_xreg<FMT, UPL, WPR, 6, FUSE>(w, x, y, n, k, p, f, s);
+    case 7: return launch_xreg<FMT, UPL, WPR, 7, FUSE>(w, x, y, n, k, p, f, s);
+    default: return launch_xreg<FMT, UPL, WPR, 8, FUSE>(w, x, y, n, k, p, f, s);
     }
 }
 
@@ -1022,17 +1126,19 @@ template <> struct HasIdot<RFQ_Q4_K> { static constexpr bool value = true; };
 template <> struct HasIdot<RFQ_Q4_0> { static constexpr bool value = true; };
 template <> struct HasIdot<RFQ_Q8_0> { static constexpr bool value = true; };
 
-template <int FMT, int UPL, int WPR, int R>
-int launch_idot(const uint8_t *w, const float *x, float *y, int n, int k, int blocks, int groups, hipStream_t s)
+template <int FMT, int UPL, int WPR, int R, bool FUSE>
+int launch_idot(const uint8_t *w, const float *x, float *y, int n, int k, int blocks, int groups, const GemvFuse &f,
+                hipStream_t s)
 {
     size_t lds = (size_t)(k / 32) * 28 * sizeof(uint32_t);
-    hipLaunchKernelGGL((gemv_idot_kernel<FMT, UPL, WPR, R>), dim3(blocks), dim3(256), lds, s, w, x, y, n, k, groups);
+    hipLaunchKernelGGL((gemv_idot_kernel<FMT, UPL, WPR, R, FUSE>), dim3(blocks), dim3(256), lds, s, w, x, y, n, k, groups,
+                       f);
     RFQ_LAUNCH_CHECK("gemv_idot_kernel");
     return RFQ_OK;
 }
 
-template <int FMT, int UPL, int WPR>
-int run_idot(const uint8_t *w, const float *x, float *y, int n, int k, hipStream_t s)
+template <int FMT, int UPL, int WPR, bool FUSE>
+int run_idot(const uint8_t *w, const float *x, float *y, int n, int k, const GemvFuse &f, hipStream_t s)
 {
     if constexpr (HasIdot<FMT>::value) {
         constexpr int TEAMS = 4 / WPR;
@@ -1048,6 +1154,7 @@ int run_idot(const uint8_t *w, const float *x, float *y, int n, int k, hipStream
         long best_cost = -1;
         for (int idx = 0; idx < 4; idx++) {
             int r = RS[idx];
+            if (FUSE && f.glu && (r & 1)) continue;
             int groups = (want + r - 1) / r;
             int blocks = (n + TEAMS * r * groups - 1) / (TEAMS * r * groups);
             long waves_of_blocks = (blocks + slots - 1) / slots;
@@ -1057,13 +1164,13 @@ int run_idot(const uint8_t *w, const float *x, float *y, int n, int k, hipStream
             }
         }
         switch (best_r) {
-        case 2: return launch_idot<FMT, UPL, WPR, 2>(w, x, y, n, k, best_blocks, best_groups, s);
-        case 4: return launch_idot<FMT, UPL, WPR, 4>(w, x, y, n, k, best_blocks, best_groups, s);
-        case 7: return launch_idot<FMT, UPL, WPR, 7>(w, x, y, n, k, best_blocks, best_groups, s);
-        default: return launch_idot<FMT, UPL, WPR, 8>(w, x, y, n, k, best_blocks, best_groups, s);
+        case 2: return launch_idot<FMT, UPL, WPR, 2, FUSE>(w, x, y, n, k, best_blocks, best_groups, f, s);
+        case 4: return launch_idot<FMT, UPL, WPR, 4, FUSE>(w, x, y, n, k, best_blocks, best_groups, f, s);
+        case 7: return launch_idot<FMT, UPL, WPR, 7, FUSE>(w, x, y, n, k, best_blocks, best_groups, f, s);
+        default: return launch_idot<FMT, UPL, WPR, 8, FUSE>(w, x, y, n, k, best_blocks, best_groups, f, s);
         }
     } else {
-        return run_xreg<FMT, UPL, WPR>(w, x, y, n, k, s);
+        return run_xreg<FMT, UPL, WPR, FUSE>(w, x, y, n, k, f, s);
     }
 }
 
@@ -1156,16 +1263,23 @@ int run_mfma_q8_0(const uint8_t *w, const float *x, float *y, int m, int n, int 
     return RFQ_OK;
 }
 
+// m == 1, 16 < k / 32 <= 512: the kernels that keep x per lane.
+template <int FMT, bool FUSE>
+int run_rows(const uint8_t *w, const float *x, float *y, int n, int k, const GemvFuse &f, hipStream_t s)
+{
+    const int ku = k / 32;
+    if (ku <= 64) return run_idot<FMT, 1, 1, FUSE>(w, x, y, n, k, f, s);
+    if (ku <= 128) return run_idot<FMT, 2, 1, FUSE>(w, x, y, n, k, f, s);
+    if (ku <= 256) return run_idot<FMT, 2, 2, FUSE>(w, x, y, n, k, f, s);
+    return run_idot<FMT, 2, 4, FUSE>(w, x, y, n, k, f, s);
+}
+
 template <int FMT>
 int run(const uint8_t *w, const float *x, float *y, int m, int n, int k, hipStream_t s)
 {
     const int ku = k / 32;
-    if (m == 1 && ku > 16) {                                   // (shorter rows leave most of a wavefront's lanes without a unit)
-        if (ku <= 64) return run_idot<FMT, 1, 1>(w, x, y, n, k, s);
-        if (ku <= 128) return run_idot<FMT, 2, 1>(w, x, y, n, k, s);
-        if (ku <= 256) return run_idot<FMT, 2, 2>(w, x, y, n, k, s);
-        if (ku <= 512) return run_idot<FMT, 2, 4>(w, x, y, n, k, s);
-    }
+    if (m == 1 && ku > 16 && ku <= 512)                        // (shorter rows leave most of a wavefront's lanes without a unit)
+        return run_rows<FMT, false>(w, x, y, n, k, GemvFuse{nullptr, nullptr, 0.0f, 0}, s);
     if (FMT == RFQ_Q8_0 && m > 1 && (reinterpret_cast<uintptr_t>(w) & 3u) == 0) return run_mfma_q8_0(w, x, y, m, n, k, s);
     if (HasIdot<FMT>::value && m > 1 && ku > 32 && ku <= 256) {
         if (m <= 2) return run_idot_batch_k<FMT, 2>(w, x, y, m, n, k, s);
@@ -1197,6 +1311,30 @@ int launch_gemv(int fmt, const uint8_t *d_w, const float *d_x, float *d_y, int m
     case RFQ_MXFP4: return run<RFQ_MXFP4>(d_w, d_x, d_y, m, n, k, s);
     case RFQ_MXFP6_E2M3: return run<RFQ_MXFP6_E2M3>(d_w, d_x, d_y, m, n, k, s);
     default: return fail(RFQ_E_BADARG, "rfq_gemv: unknown format %d", fmt);
+    }
+}
+
+
+// One launch for RMSNorm -> GEMV (norm_w != nullptr) and / or two GEMVs sharing
+// x -> SwiGLU (w2 != nullptr: y[j] = swiglu(w row j . x, w2 row j . x), n counts
+// the rows of each matrix).  m == 1 only; RFQ_E_UNSUPPORTED (without an error
+// text) when the shape has no such kernel, so the caller can compose the steps.
+int launch_gemv_fused(int fmt, const uint8_t *d_w, const uint8_t *d_w2, const float *d_x, const float *d_norm_w,
+                      float eps, float *d_y, int n, int k, hipStream_t s)
+{
+    const int ku = k / 32;
+    if (k % 32 != 0 || ku <= 16 || ku > 512 || (d_w2 != nullptr && n > 0x3fffffff)) return RFQ_E_UNSUPPORTED;
+    if (k % fmt_block_elems(fmt) != 0) return RFQ_E_UNSUPPORTED;
+    const GemvFuse f{d_w2, d_norm_w, eps, d_w2 != nullptr ? 1 : 0};
+    const int rows = d_w2 != nullptr ? 2 * n : n;
+    switch (canonical_format(fmt)) {
+    case RFQ_Q4_0: return run_rows<RFQ_Q4_0, true>(d_w, d_x, d_y, rows, k, f, s);
+    case RFQ_Q8_0: return run_rows<RFQ_Q8_0, true>(d_w, d_x, d_y, rows, k, f, s);
+    case RFQ_Q4_K: return run_rows<RFQ_Q4_K, true>(d_w, d_x, d_y, rows, k, f, s);
+    case RFQ_Q6_K: return run_rows<RFQ_Q6_K, true>(d_w, d_x, d_y, rows, k, f, s);
+    case RFQ_MXFP4: return run_rows<RFQ_MXFP4, true>(d_w, d_x, d_y, rows, k, f, s);
+    case RFQ_MXFP6_E2M3: return run_rows<RFQ_MXFP6_E2M3, true>(d_w, d_x, d_y, rows, k, f, s);
+    default: return fail(RFQ_E_BADARG, "fused gemv: unknown format %d", fmt);
     }
 }
 

@@ -69,6 +69,73 @@ def get_rows(fmt: int, table: torch.Tensor, tokens: torch.Tensor, n_vocab: int, 
     return out
 
 
+def _f32(t: torch.Tensor, what: str) -> torch.Tensor:
+    if not (t.is_cuda and t.dtype == torch.float32 and t.is_contiguous()):
+        raise ValueError(f"{what} must be a contiguous float32 device tensor")
+    return t
+
+
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """RMSNorm over the last axis of x[seq_len, hidden] (src/mlp/kernels.rs:261-330)."""
+    x, weight = _f32(x, "x"), _f32(weight, "weight")
+    hidden = x.shape[-1]
+    out = torch.empty_like(x)
+    check(lib().rfq_rms_norm(_ptr(x), _ptr(weight), _ptr(out), x.numel() // hidden, hidden, eps, _stream()))
+    return out
+
+
+def swiglu(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """gate * (up * sigmoid(up)) elementwise (src/mlp/kernels.rs:177-240)."""
+    gate, up = _f32(gate, "gate"), _f32(up, "up")
+    if gate.shape != up.shape:
+        raise ValueError("gate and up differ in shape")
+    inter = gate.shape[-1] if gate.dim() else 1
+    out = torch.empty_like(gate)
+    check(lib().rfq_swiglu(_ptr(gate), _ptr(up), _ptr(out), gate.numel() // max(inter, 1), inter, _stream()))
+    return out
+
+
+def dequant_rms_norm(fmt: int, packed: torch.Tensor, weight: torch.Tensor, seq_len: int, hidden: int,
+                     eps: float) -> torch.Tensor:
+    """RMSNorm of packed rows, decoded on the fly (src/ggml/hip_backend/ops/fused_ops.rs:149-160)."""
+    packed, weight = _dev_u8(packed), _f32(weight, "weight")
+    out = torch.empty((seq_len, hidden), dtype=torch.float32, device=packed.device)
+    check(lib().rfq_dequant_rms_norm(fmt, _ptr(packed), packed.numel(), _ptr(weight), _ptr(out), seq_len, hidden, eps,
+                                     _stream()))
+    return out
+
+
+def rms_norm_gemv(fmt: int, w: torch.Tensor, x: torch.Tensor, norm_weight: torch.Tensor, eps: float, n: int,
+                  k: int, scratch: bool = True) -> torch.Tensor:
+    """y[m, n] = RMSNorm(x[m, k]) . dequant(W)[n, k]^T in one call."""
+    w, x, norm_weight = _dev_u8(w), _f32(x, "x"), _f32(norm_weight, "norm_weight")
+    m = 1 if x.dim() == 1 else x.shape[0]
+    out = torch.empty((m, n), dtype=torch.float32, device=x.device)
+    tmp = torch.empty((m, k), dtype=torch.float32, device=x.device) if scratch else None
+    check(lib().rfq_rms_norm_gemv(fmt, _ptr(w), w.numel(), _ptr(x), _ptr(norm_weight), eps, _ptr(out), m, n, k,
+                                  _ptr(tmp) if tmp is not None else None, _stream()))
+    return out if x.dim() > 1 else out.view(n)
+
+
+def mlp_swiglu(fmt_gate_up: int, gate_w: torch.Tensor, up_w: torch.Tensor, fmt_down: int, down_w: torch.Tensor,
+               x: torch.Tensor, norm_weight: torch.Tensor | None, eps: float, hidden: int, inter: int,
+               scratch: torch.Tensor | None = None) -> torch.Tensor:
+    """out[m, hidden] = swiglu(xn . gate^T, xn . up^T) . down^T over quantised weights
+    (src/backend/hip_backend/backend.rs:1153-1278); xn = RMSNorm(x) when norm_weight is given."""
+    gate_w, up_w, down_w, x = _dev_u8(gate_w), _dev_u8(up_w), _dev_u8(down_w), _f32(x, "x")
+    if gate_w.numel() != up_w.numel():
+        raise ValueError("gate and up weights differ in size")
+    m = 1 if x.dim() == 1 else x.shape[0]
+    need = lib().rfq_mlp_scratch_bytes(m, hidden, inter)
+    if scratch is None:
+        scratch = torch.empty(need, dtype=torch.uint8, device=x.device)
+    out = torch.empty((m, hidden), dtype=torch.float32, device=x.device)
+    check(lib().rfq_mlp_swiglu(fmt_gate_up, _ptr(gate_w), _ptr(up_w), gate_w.numel(), fmt_down, _ptr(down_w),
+                               down_w.numel(), _ptr(x), _ptr(_f32(norm_weight, "norm_weight")) if norm_weight is not None else None,
+                               eps, _ptr(out), m, hidden, inter, _ptr(scratch), scratch.numel(), _stream()))
+    return out if x.dim() > 1 else out.view(hidden)
+
+
 def gemm_f16(fmt: int, w: torch.Tensor, a: torch.Tensor, n: int, k: int, out_dtype=torch.float16,
              out: torch.Tensor | None = None) -> torch.Tensor:
     """out[m, n] = a[m, k] (fp16) . dequant(W)[n, k]^T on the fp16 matrix cores."""
