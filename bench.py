@@ -117,6 +117,48 @@ def time_get_rows(torch, fmt, n_vocab, n_embd, n_tokens, Q):
     return {"us": round(t * 1e6, 2), "GB/s": round(b / t / 1e9, 1), "rows/s": round(n_tokens / t)}
 
 
+def time_mlp(torch, fmt, hidden, inter, Q, steps=300, warmup=60):
+    """The SwiGLU MLP of one decode step (RMSNorm, gate and up projections, activation, down projection) over
+    rotating weight sets: rfq_mlp_swiglu (two launches) and the same arithmetic as five separate calls."""
+    import ctypes as C
+
+    import numpy as np
+
+    from rocmforge_amd import _lib
+    dev = torch.device("cuda:0")
+    L = _lib.lib()
+    gu_bytes, d_bytes = Q.packed_bytes(fmt, inter * hidden), Q.packed_bytes(fmt, hidden * inter)
+    copies = -(-int(2.5 * CACHE_BYTES) // (2 * gu_bytes + d_bytes))
+    slab = 1024                                                    # quantise a slab of rows, repeat it down the matrix
+    mats = []
+    for c in range(copies):
+        g = np.tile(Q.make_weights(fmt, slab, hidden, seed=20260040 + 3 * c), inter // slab)
+        u = np.tile(Q.make_weights(fmt, slab, hidden, seed=20260041 + 3 * c), inter // slab)
+        d = np.tile(Q.make_weights(fmt, slab, inter, seed=20260042 + 3 * c), hidden // slab)
+        mats.append(tuple(torch.from_numpy(a).to(dev) for a in (g, u, d)))
+    arr = [(C.c_void_p * copies)(*[m[i].data_ptr() for m in mats]) for i in range(3)]
+    rng = np.random.Generator(np.random.PCG64(20260049))
+    x = torch.from_numpy(rng.standard_normal(hidden, dtype=np.float32)).to(dev)
+    nw = torch.from_numpy(1.0 + 0.1 * rng.standard_normal(hidden, dtype=np.float32)).to(dev)
+    out = torch.empty(hidden, dtype=torch.float32, device=dev)
+    nscr = L.rfq_mlp_scratch_bytes(1, hidden, inter)
+    scratch = torch.empty(nscr, dtype=torch.uint8, device=dev)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    res = {}
+    for key, one_call in (("us", 1), ("five_calls_us", 0)):
+        ms = C.c_float(0)
+        for w_, s_ in ((warmup, 1), (0, steps)):
+            _lib.check(L.rfq_bench_mlp_swiglu(fmt, arr[0], arr[1], gu_bytes, fmt, arr[2], d_bytes, copies,
+                                              C.c_void_p(x.data_ptr()), C.c_void_p(nw.data_ptr()), 1e-5,
+                                              C.c_void_p(out.data_ptr()), 1, hidden, inter, C.c_void_p(scratch.data_ptr()),
+                                              nscr, one_call, w_, s_, stream, C.byref(ms)))
+        res[key] = round(ms.value / steps * 1e3, 2)
+    b = 2 * gu_bytes + d_bytes + 4 * (3 * hidden)                  # the three matrices, x, the norm weight, the output
+    res["GB/s"] = round(b / res["us"] / 1e3, 1)
+    res["hbm_frac"] = round(b / res["us"] / 1e3 / HBM_PEAK_GBS, 4)
+    return res
+
+
 def cpu_baseline(fmt, w, x, n, k, budget_s=12.0):
     """The CPU oracle (dequantise everything, then the sequential fp32 matmul)
     on one host thread, repeated until ~budget_s of CPU work."""
@@ -228,6 +270,7 @@ def main():
         b = algorithmic_bytes(Q.Q4_K, 128256, 4096, 1, Q)
         also["Q4_K gemv 128256x4096 (LM head)"] = {"GB/s": round(b / (d / 50) / 1e9, 1), "us": round(d / 50 * 1e6, 2),
                                                    "hbm_frac": round(b / (d / 50) / 1e9 / HBM_PEAK_GBS, 4)}
+        also["Q4_K mlp_swiglu 4096x14336 m1"] = time_mlp(torch, Q.Q4_K, 4096, 14336, Q)
         also["Q4_K get_rows 512 of 128256x4096"] = time_get_rows(torch, Q.Q4_K, 128256, 4096, 512, Q)
         for name, f, n, k, seed in (("Q4_0 dequant 4096x4096", Q.Q4_0, 4096, 4096, 20260021),
                                     ("Q4_K dequant 14336x4096", Q.Q4_K, N, K, 20260023),

@@ -36,6 +36,16 @@ RFQ_API int rfq_bench_gemm_mx(const void *d_a_prep, int a_kind, const void *d_w_
                               int out_dtype, int m, int n, int k, int warmup, int steps, void *stream,
                               float *elapsed_ms);
 
+/* Step i runs the MLP over weight set i % copies.  one_call != 0: rfq_mlp_swiglu;
+ * one_call == 0: the same arithmetic as five calls (rfq_rms_norm, rfq_gemv for
+ * gate and up, rfq_swiglu, rfq_gemv for down), for comparison. */
+RFQ_API int rfq_bench_mlp_swiglu(int fmt_gate_up, const void *const *d_gate_copies, const void *const *d_up_copies,
+                                 size_t gate_up_bytes, int fmt_down, const void *const *d_down_copies,
+                                 size_t down_bytes, int copies, const float *d_x, const float *d_norm_weight,
+                                 float eps, float *d_out, int m, int hidden_size, int intermediate_size,
+                                 void *d_scratch, size_t scratch_bytes, int one_call, int warmup, int steps,
+                                 void *stream, float *elapsed_ms);
+
 #ifdef __cplusplus
 }
 #endif

@@ -22,6 +22,13 @@
  *                         src/ggml/hip_backend/ops/batch_quantized.rs:20-90
  *   validate_matmul_q4_0 / q8_0 (the checks of execute_matmul_q4_0 / q8_0)
  *                         src/ggml/hip_backend/op_dispatch.rs:951-1083
+ *   get_rows, validate_token_ids
+ *                         src/ggml/hip_backend/ops/get_rows.rs:6-65
+ *   rms_norm_gpu_kernel, swiglu_gpu_kernel
+ *                         src/mlp/kernels.rs:261-330, 177-240
+ *   fused_q4_0_rmsnorm    src/ggml/hip_backend/ops/fused_ops.rs:149-160
+ *   DeviceTensor, mlp_swiglu (HipBackend::mlp_swiglu over quantised weights)
+ *                         src/backend/hip_backend/backend.rs:1385-1388, 1153-1278
  *
  * Rust's Result<T, E> becomes Result<T> below (ok / value / error text); no
  * exceptions cross the C ABI.  Everything computes on the GPU through librfq:
@@ -470,6 +477,70 @@ inline Status get_rows(const HipBackend &b, const HipBuffer &weights, const std:
                           b.stream());
     if (rc != RFQ_OK) return detail::from_rfq(rc, "get_rows");
     return b.synchronize();                                    // the token buffer is dropped on return
+}
+
+// ---- neighbours of the matmul in a decoder layer -------------------------------------
+// rms_norm_gpu_kernel (src/mlp/kernels.rs:261-330): raw device pointers, enqueue only; the
+// caller synchronises on the same backend, as the reference's doc comment demands.
+inline Status rms_norm_gpu_kernel(const HipBackend &b, const float *input, const float *weight, float *output,
+                                  uint32_t seq_len, uint32_t hidden_size, float eps)
+{
+    return detail::from_rfq(rfq_rms_norm(input, weight, output, (int)seq_len, (int)hidden_size, eps, b.stream()),
+                            "Failed to launch rms_norm kernel");
+}
+// swiglu_gpu_kernel (src/mlp/kernels.rs:177-240): output = gate * swish(up).
+inline Status swiglu_gpu_kernel(const HipBackend &b, const float *gate, const float *up, float *output, uint32_t seq_len,
+                                uint32_t intermediate_size)
+{
+    return detail::from_rfq(rfq_swiglu(gate, up, output, (int)seq_len, (int)intermediate_size, b.stream()),
+                            "Failed to launch swiglu kernel");
+}
+// fused_q4_0_rmsnorm (src/ggml/hip_backend/ops/fused_ops.rs:149-160): packed Q4_0 rows in, normalised f32 rows out.
+inline Status fused_q4_0_rmsnorm(const HipBackend &b, const uint8_t *q4_0_input, const float *weight, float *output,
+                                 uint32_t seq_len, uint32_t hidden_size, float eps)
+{
+    const size_t bytes = (size_t)seq_len * (hidden_size / 32) * 20;
+    return detail::from_rfq(rfq_dequant_rms_norm(RFQ_Q4_0, q4_0_input, bytes, weight, output, (int)seq_len, (int)hidden_size,
+                                                 eps, b.stream()),
+                            "Fused dequant+RMSNorm kernel failed");
+}
+
+// DeviceTensor (src/backend/hip_backend/backend.rs:1385-1388): a device buffer and its shape; `format` is
+// RFQ_TABLE_F32 for f32 data or the block format of packed data (the reference's tensors are f32 only).
+struct DeviceTensor {
+    HipBuffer buffer;
+    TensorShape shape;
+    int format = RFQ_TABLE_F32;
+};
+
+// HipBackend::mlp_swiglu (src/backend/hip_backend/backend.rs:1153-1278) with the three matrices quantised:
+// gate and up [intermediate_size, hidden_size], down [hidden_size, intermediate_size] (rows are outputs, as
+// the quantised matmuls store them), hidden_states and output f32 [seq_len, hidden_size], seq_len <= 8.
+// The reference's shape checks, in its order and wording; no temporaries are left behind and the call
+// synchronises before returning, as the reference does.
+inline Status mlp_swiglu(const HipBackend &b, const DeviceTensor &hidden_states, const DeviceTensor &gate_weight,
+                         const DeviceTensor &up_weight, const DeviceTensor &down_weight, DeviceTensor &output)
+{
+    const auto &hs = hidden_states.shape.dims(), &gs = gate_weight.shape.dims(), &us = up_weight.shape.dims(),
+               &ds = down_weight.shape.dims(), &os = output.shape.dims();
+    if (hs.size() != 2) return Status::Err("hidden_states must be 2D [seq_len, hidden_size]");
+    if (gs.size() != 2 || gs[1] != hs[1]) return Status::Err("gate_weight must be 2D [intermediate_size, hidden_size]");
+    if (us.size() != 2 || us[1] != hs[1]) return Status::Err("up_weight must be 2D [intermediate_size, hidden_size]");
+    if (ds.size() != 2 || ds[0] != hs[1]) return Status::Err("down_weight must be 2D [hidden_size, intermediate_size]");
+    if (os != hs) return Status::Err("output must match hidden_states shape [seq_len, hidden_size]");
+    const size_t seq_len = hs[0], hidden_size = hs[1], intermediate_size = gs[0];
+    if (us[0] != intermediate_size || ds[1] != intermediate_size) return Status::Err("All intermediate dimensions must match");
+    if (gate_weight.format != up_weight.format) return Status::Err("gate_weight and up_weight must share a format");
+    const size_t scratch_bytes = rfq_mlp_scratch_bytes((int)seq_len, (int)hidden_size, (int)intermediate_size);
+    auto scratch = HipBuffer::create(scratch_bytes);
+    if (!scratch.ok) return Status::Err("Failed to allocate SwiGLU buffer: " + scratch.error);
+    int rc = rfq_mlp_swiglu(gate_weight.format, gate_weight.buffer.as_ptr(), up_weight.buffer.as_ptr(),
+                            gate_weight.buffer.size(), down_weight.format, down_weight.buffer.as_ptr(),
+                            down_weight.buffer.size(), (const float *)hidden_states.buffer.as_ptr(), nullptr, 0.0f,
+                            (float *)output.buffer.as_ptr(), (int)seq_len, (int)hidden_size, (int)intermediate_size,
+                            scratch.value.as_ptr(), scratch_bytes, b.stream());
+    if (rc != RFQ_OK) return detail::from_rfq(rc, "mlp_swiglu");
+    return b.synchronize();
 }
 
 } // namespace rocmforge

@@ -74,4 +74,43 @@ int rfq_bench_gemm_mx(const void *d_a_prep, int a_kind, const void *d_w_prep, in
     });
 }
 
+int rfq_bench_mlp_swiglu(int fmt_gate_up, const void *const *d_gate_copies, const void *const *d_up_copies,
+                         size_t gate_up_bytes, int fmt_down, const void *const *d_down_copies, size_t down_bytes,
+                         int copies, const float *d_x, const float *d_norm_weight, float eps, float *d_out, int m,
+                         int hidden_size, int intermediate_size, void *d_scratch, size_t scratch_bytes, int one_call,
+                         int warmup, int steps, void *stream, float *elapsed_ms)
+{
+    if (!d_gate_copies || !d_up_copies || !d_down_copies || copies <= 0)
+        return rfq::fail(RFQ_E_BADARG, "rfq_bench_mlp_swiglu: no weight copies");
+    if (one_call)
+        return timed_loop(warmup, steps, stream, elapsed_ms, [&](int i) {
+            const int c = i % copies;
+            return rfq_mlp_swiglu(fmt_gate_up, d_gate_copies[c], d_up_copies[c], gate_up_bytes, fmt_down, d_down_copies[c],
+                                  down_bytes, d_x, d_norm_weight, eps, d_out, m, hidden_size, intermediate_size, d_scratch,
+                                  scratch_bytes, stream);
+        });
+    // the same arithmetic as five calls of the separate entry points
+    const size_t need = rfq_mlp_scratch_bytes(m, hidden_size, intermediate_size);
+    if (!d_scratch || scratch_bytes < need) return rfq::fail(RFQ_E_SIZE, "rfq_bench_mlp_swiglu: scratch too small");
+    const size_t mi = (((size_t)m * intermediate_size * 4) + 15) & ~(size_t)15;
+    const size_t mh = (((size_t)m * hidden_size * 4) + 15) & ~(size_t)15;
+    uint8_t *base = static_cast<uint8_t *>(d_scratch);
+    float *h = reinterpret_cast<float *>(base), *xn = reinterpret_cast<float *>(base + mi);
+    float *gate = reinterpret_cast<float *>(base + mi + mh), *up = reinterpret_cast<float *>(base + 2 * mi + mh);
+    return timed_loop(warmup, steps, stream, elapsed_ms, [&](int i) {
+        const int c = i % copies;
+        const float *xin = d_x;
+        int rc = RFQ_OK;
+        if (d_norm_weight) {
+            rc = rfq_rms_norm(d_x, d_norm_weight, xn, m, hidden_size, eps, stream);
+            xin = xn;
+        }
+        if (rc == RFQ_OK) rc = rfq_gemv(fmt_gate_up, d_gate_copies[c], gate_up_bytes, xin, gate, m, intermediate_size, hidden_size, stream);
+        if (rc == RFQ_OK) rc = rfq_gemv(fmt_gate_up, d_up_copies[c], gate_up_bytes, xin, up, m, intermediate_size, hidden_size, stream);
+        if (rc == RFQ_OK) rc = rfq_swiglu(gate, up, h, m, intermediate_size, stream);
+        if (rc == RFQ_OK) rc = rfq_gemv(fmt_down, d_down_copies[c], down_bytes, h, d_out, m, hidden_size, intermediate_size, stream);
+        return rc;
+    });
+}
+
 } // extern "C"

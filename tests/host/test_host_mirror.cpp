@@ -298,6 +298,76 @@ static void test_get_rows_f32_and_packed_tables()
     EXPECT(all_eq(got, 0, 32, 3.0f) && all_eq(got, 32, 64, 1.0f) && all_eq(got, 64, 96, 4.0f));
 }
 
+// src/mlp/rms_norm_tests.rs:211-251, src/mlp/swiglu_tests.rs:329-372, and an MLP whose result is known in closed form
+static void test_norm_swiglu_and_mlp()
+{
+    auto be = HipBackend::create();
+    EXPECT(be.ok);
+    const size_t hidden = 1024, inter = 512;
+    auto x = HipBuffer::create(hidden * 4), w = HipBuffer::create(hidden * 4), o = HipBuffer::create(hidden * 4);
+    EXPECT(x.ok && w.ok && o.ok);
+    std::vector<float> twos(hidden, 2.0f), ones(hidden, 1.0f), got(hidden);
+    EXPECT(x.value.copy_from_host(twos).ok && w.value.copy_from_host(ones).ok);
+    EXPECT(rms_norm_gpu_kernel(be.value, (const float *)x.value.as_ptr(), (const float *)w.value.as_ptr(),
+                               (float *)o.value.as_ptr(), 1, hidden, 1e-6f).ok && be.value.synchronize().ok);
+    EXPECT(o.value.copy_to_host(got).ok);
+    for (float v : got) EXPECT(std::fabs(v - 1.0f) < 0.01f);            // constant positive input -> ~1
+    std::vector<float> zeros(hidden, 0.0f);
+    EXPECT(x.value.copy_from_host(zeros).ok);
+    EXPECT(swiglu_gpu_kernel(be.value, (const float *)w.value.as_ptr(), (const float *)x.value.as_ptr(),
+                             (float *)o.value.as_ptr(), 1, hidden).ok && be.value.synchronize().ok);
+    EXPECT(o.value.copy_to_host(got).ok && all_eq(got, 0, hidden, 0.0f)); // up = 0 -> 0
+
+    // fused_q4_0_rmsnorm: one row of blocks with scale 2 and every nibble 9 decodes to 2.0 everywhere -> ~1 * weight
+    bytes row(hidden / 32 * 20);
+    for (size_t blk = 0; blk < hidden / 32; blk++) {
+        put_f32(row, blk * 20, 2.0f);
+        for (size_t j = 0; j < 16; j++) row[blk * 20 + 4 + j] = 0x99;
+    }
+    auto packed = HipBuffer::create(row.size());
+    EXPECT(packed.ok && packed.value.copy_from_host(row).ok);
+    std::vector<float> threes(hidden, 3.0f);
+    EXPECT(w.value.copy_from_host(threes).ok);
+    EXPECT(fused_q4_0_rmsnorm(be.value, (const uint8_t *)packed.value.as_ptr(), (const float *)w.value.as_ptr(),
+                              (float *)o.value.as_ptr(), 1, hidden, 1e-6f).ok && be.value.synchronize().ok);
+    EXPECT(o.value.copy_to_host(got).ok);
+    for (float v : got) EXPECT(std::fabs(v - 3.0f) < 0.01f);
+
+    // MLP with constant matrices: gate weights 1/64, up weights 1/32, down weights 1/8 (Q4_0: scale * (9 - 8)),
+    // x = 1: gate = 16, up = 32, h = 16 * 32 * sigmoid(32) = 512, out = 512 * 512 / 8 = 32768
+    auto constant = [&](size_t rows, size_t k, float value) {
+        bytes m(rows * (k / 32) * 20);
+        for (size_t blk = 0; blk < rows * (k / 32); blk++) {
+            put_f32(m, blk * 20, value);
+            for (size_t j = 0; j < 16; j++) m[blk * 20 + 4 + j] = 0x99;
+        }
+        DeviceTensor t;
+        auto buf = HipBuffer::create(m.size());
+        EXPECT(buf.ok && buf.value.copy_from_host(m).ok);
+        t.buffer = buf.value;
+        t.shape = TensorShape::from_dims({rows, k});
+        t.format = RFQ_Q4_0;
+        return t;
+    };
+    DeviceTensor gate = constant(inter, hidden, 1.0f / 64), up = constant(inter, hidden, 1.0f / 32),
+                 down = constant(hidden, inter, 1.0f / 8), hs, out;
+    EXPECT(x.value.copy_from_host(ones).ok);
+    hs.buffer = x.value; hs.shape = TensorShape::from_dims({1, hidden});
+    out.buffer = o.value; out.shape = TensorShape::from_dims({1, hidden});
+    Status st = mlp_swiglu(be.value, hs, gate, up, down, out);
+    EXPECT(st.ok);
+    EXPECT(o.value.copy_to_host(got).ok);
+    for (float v : got) EXPECT(std::fabs(v - 32768.0f) < 1.0f);
+    // the reference's shape checks
+    DeviceTensor bad = down;
+    bad.shape = TensorShape::from_dims({hidden, inter + 32});
+    Status e = mlp_swiglu(be.value, hs, gate, up, bad, out);
+    EXPECT(!e.ok && e.error == "All intermediate dimensions must match");
+    hs.shape = TensorShape::from_dims({hidden});
+    e = mlp_swiglu(be.value, hs, gate, up, down, out);
+    EXPECT(!e.ok && e.error == "hidden_states must be 2D [seq_len, hidden_size]");
+}
+
 int main()
 {
     struct T { const char *name; std::function<void()> fn; };
@@ -317,6 +387,7 @@ int main()
         {"test_matmul_q4_0_against_dequantized_weights", test_matmul_q4_0_against_dequantized_weights},
         {"test_matmul_validation_like_op_dispatch", test_matmul_validation_like_op_dispatch},
         {"test_get_rows_f32_and_packed_tables", test_get_rows_f32_and_packed_tables},
+        {"test_norm_swiglu_and_mlp", test_norm_swiglu_and_mlp},
     };
     for (const T &t : tests) {
         int before = failures;
