@@ -195,6 +195,8 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain elementwise copy of 256 MiB five times (for scaling HBM byte counters "
                          "of a profiler against a kernel of known traffic)")
+    ap.add_argument("--only-mlp", action="store_true", help="only the SwiGLU MLP line (profiling runs)")
+    ap.add_argument("--mlp-steps", type=int, default=300)
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build is single-GPU (one MI355X per box); run with --gpus 1. "
@@ -208,6 +210,10 @@ def main():
         sys.exit("bench.py: no GPU visible")
     import rocmforge_amd
     rocmforge_amd.lib()  # fail loudly if librfq.so is missing
+
+    if args.only_mlp:
+        print(json.dumps({"Q4_K mlp_swiglu 4096x14336 m1": time_mlp(torch, Q.Q4_K, 4096, 14336, Q, steps=args.mlp_steps)}))
+        return
 
     fmt = Q.Q4_K
     wbytes = Q.packed_bytes(fmt, N * K)
