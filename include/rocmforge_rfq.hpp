@@ -29,6 +29,8 @@
  *   fused_q4_0_rmsnorm    src/ggml/hip_backend/ops/fused_ops.rs:149-160
  *   DeviceTensor, mlp_swiglu (HipBackend::mlp_swiglu over quantised weights)
  *                         src/backend/hip_backend/backend.rs:1385-1388, 1153-1278
+ *   Op (the quantised matmuls), execute_matmul_quantized
+ *                         src/ggml/op.rs:4-30, src/ggml/hip_backend/op_dispatch.rs:951-1083
  *
  * Rust's Result<T, E> becomes Result<T> below (ok / value / error text); no
  * exceptions cross the C ABI.  Everything computes on the GPU through librfq:
@@ -541,6 +543,61 @@ inline Status mlp_swiglu(const HipBackend &b, const DeviceTensor &hidden_states,
                             scratch.value.as_ptr(), scratch_bytes, b.stream());
     if (rc != RFQ_OK) return detail::from_rfq(rc, "mlp_swiglu");
     return b.synchronize();
+}
+
+// ---- quantised matmul ops over device-resident weights ------------------------------------
+// Op (src/ggml/op.rs:4-30) has MatMulQ4_0 and MatMulQ8_0; the other four formats of this path get
+// ops of the same shape.  execute_matmul_q4_0 / q8_0 (src/ggml/hip_backend/op_dispatch.rs:951-1083)
+// copy the weights device -> host and hand them to matmul_q4_0, which uploads them again; here
+// the packed weights stay where they are.  Checks, order and wording follow the reference.
+enum class Op { MatMulQ4_0, MatMulQ8_0, MatMulQ4_K, MatMulQ6_K, MatMulMxfp4, MatMulMxfp6 };
+inline const char *name(Op op)
+{
+    switch (op) {
+    case Op::MatMulQ4_0: return "MatMulQ4_0";
+    case Op::MatMulQ8_0: return "MatMulQ8_0";
+    case Op::MatMulQ4_K: return "MatMulQ4_K";
+    case Op::MatMulQ6_K: return "MatMulQ6_K";
+    case Op::MatMulMxfp4: return "MatMulMxfp4";
+    default: return "MatMulMxfp6";
+    }
+}
+inline int rfq_format_of(Op op)
+{
+    switch (op) {
+    case Op::MatMulQ4_0: return RFQ_Q4_0;
+    case Op::MatMulQ8_0: return RFQ_Q8_0;
+    case Op::MatMulQ4_K: return RFQ_Q4_K;
+    case Op::MatMulQ6_K: return RFQ_Q6_K;
+    case Op::MatMulMxfp4: return RFQ_MXFP4;
+    default: return RFQ_MXFP6_E2M3;
+    }
+}
+// output[m, n_rows] = input[m, n_cols] . dequant(weights[n_rows, n_cols])^T; any m (rows go through the
+// decode kernels eight at a time).  Enqueue only.
+inline Status execute_matmul_quantized(const HipBackend &b, Op op, const DeviceTensor &weights, const DeviceTensor &input,
+                                       DeviceTensor &output)
+{
+    const std::string who = name(op);
+    const auto &ws = weights.shape.dims(), &is = input.shape.dims();
+    if (ws.size() != 2 || is.size() != 2) return Status::Err(who + " expects 2D tensors");
+    const int fmt = rfq_format_of(op);
+    const size_t n_rows = ws[0], n_cols = ws[1], be = rfq_block_elems(fmt), bb = rfq_block_bytes(fmt);
+    const size_t expected = ((n_rows * n_cols + be - 1) / be) * bb;
+    if (weights.buffer.size() != expected)
+        return Status::Err(who + " weights size mismatch: expected " + std::to_string(expected) + " bytes, got " +
+                           std::to_string(weights.buffer.size()));
+    if (is[1] != n_cols)
+        return Status::Err(who + " dimension mismatch: k=" + std::to_string(is[1]) + " weights_k=" + std::to_string(n_cols));
+    const size_t m = is[0];
+    if (output.buffer.size() < m * n_rows * sizeof(float)) return Status::Err(who + " output buffer too small");
+    for (size_t r0 = 0; r0 < m; r0 += 8) {
+        const size_t rows = m - r0 < 8 ? m - r0 : 8;
+        int rc = rfq_gemv(fmt, weights.buffer.as_ptr(), weights.buffer.size(), (const float *)input.buffer.as_ptr() + r0 * n_cols,
+                          (float *)output.buffer.as_ptr() + r0 * n_rows, (int)rows, (int)n_rows, (int)n_cols, b.stream());
+        if (rc != RFQ_OK) return detail::from_rfq(rc, name(op));
+    }
+    return ok_status();
 }
 
 } // namespace rocmforge

@@ -368,6 +368,62 @@ static void test_norm_swiglu_and_mlp()
     EXPECT(!e.ok && e.error == "hidden_states must be 2D [seq_len, hidden_size]");
 }
 
+// op_dispatch.rs:951-1083 without the round trip of the weights through the host: constant matrices, 11 input rows
+static void test_execute_matmul_quantized_ops()
+{
+    auto be = HipBackend::create();
+    EXPECT(be.ok);
+    const size_t n = 48, k = 512, m = 11;
+    struct Case { Op op; size_t block_elems, block_bytes; float weight; };
+    // every block decodes to one constant: Q4_0 scale 0.5, nibbles 9 -> 0.5; Q8_0 scale 0.25, bytes 130 -> 0.5;
+    // Q4_K scales 0.5 (f16 0x3800), mins 0, nibbles 1 -> 0.5; MXFP4 exponent 0, codes 2 -> 1.0
+    const Case cases[] = {{Op::MatMulQ4_0, 32, 20, 0.5f}, {Op::MatMulQ8_0, 32, 36, 0.5f}, {Op::MatMulQ4_K, 256, 256, 0.5f},
+                          {Op::MatMulMxfp4, 32, 17, 1.0f}};
+    std::vector<float> x(m * k);
+    for (size_t i = 0; i < m; i++)
+        for (size_t j = 0; j < k; j++) x[i * k + j] = (float)(i + 1) * ((j & 1) ? 0.25f : 0.5f);   // row sum = (i + 1) * 192
+    DeviceTensor in, out;
+    auto xb = HipBuffer::create(x.size() * 4), ob = HipBuffer::create(m * n * 4);
+    EXPECT(xb.ok && ob.ok && xb.value.copy_from_host(x).ok);
+    in.buffer = xb.value; in.shape = TensorShape::from_dims({m, k});
+    out.buffer = ob.value; out.shape = TensorShape::from_dims({m, n});
+    for (const Case &c : cases) {
+        bytes w(n * k / c.block_elems * c.block_bytes);
+        for (size_t blk = 0; blk < w.size() / c.block_bytes; blk++) {
+            uint8_t *p = w.data() + blk * c.block_bytes;
+            switch (c.op) {
+            case Op::MatMulQ4_0: put_f32(w, blk * 20, 0.5f); std::memset(p + 4, 0x99, 16); break;
+            case Op::MatMulQ8_0: put_f32(w, blk * 36, 0.25f); std::memset(p + 4, 130, 32); break;
+            case Op::MatMulQ4_K:
+                for (int sb = 0; sb < 8; sb++) put_f16(w, blk * 256 + 2 * sb, 0x3800);
+                std::memset(p + 16, 0, 16);
+                std::memset(p + 32, 0x11, 224);
+                break;
+            default: p[0] = 0; std::memset(p + 1, 0x22, 16); break;
+            }
+        }
+        DeviceTensor wt;
+        auto wb = HipBuffer::create(w.size());
+        EXPECT(wb.ok && wb.value.copy_from_host(w).ok);
+        wt.buffer = wb.value; wt.shape = TensorShape::from_dims({n, k});
+        Status st = execute_matmul_quantized(be.value, c.op, wt, in, out);
+        EXPECT(st.ok && be.value.synchronize().ok);
+        std::vector<float> got(m * n);
+        EXPECT(ob.value.copy_to_host(got).ok);
+        for (size_t i = 0; i < m; i++)
+            for (size_t j = 0; j < n; j++) EXPECT(std::fabs(got[i * n + j] - (float)(i + 1) * 192.0f * c.weight) < 1e-3f * (i + 1) * 192.0f);
+        // the reference's checks
+        DeviceTensor short_in = in;
+        short_in.shape = TensorShape::from_dims({m, k - 32});
+        Status e = execute_matmul_quantized(be.value, c.op, wt, short_in, out);
+        EXPECT(!e.ok && e.error == std::string(name(c.op)) + " dimension mismatch: k=" + std::to_string(k - 32) +
+                                       " weights_k=" + std::to_string(k));
+        wt.shape = TensorShape::from_dims({n + 1, k});
+        e = execute_matmul_quantized(be.value, c.op, wt, in, out);
+        EXPECT(!e.ok && e.error.find("weights size mismatch") != std::string::npos);
+    }
+}
+
 int main()
 {
     struct T { const char *name; std::function<void()> fn; };
@@ -388,6 +444,7 @@ int main()
         {"test_matmul_validation_like_op_dispatch", test_matmul_validation_like_op_dispatch},
         {"test_get_rows_f32_and_packed_tables", test_get_rows_f32_and_packed_tables},
         {"test_norm_swiglu_and_mlp", test_norm_swiglu_and_mlp},
+        {"test_execute_matmul_quantized_ops", test_execute_matmul_quantized_ops},
     };
     for (const T &t : tests) {
         int before = failures;
