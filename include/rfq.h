@@ -47,7 +47,18 @@ typedef enum rfq_format {
     RFQ_Q6_K = 14,       /* 256 B / 256: 16 f16 scales, 6-bit stream         */
     RFQ_MXFP4 = 20,      /* 17 B / 32: i8 exponent + 16 nibble bytes         */
     RFQ_MXFP6_E2M3 = 21, /* 25 B / 32: i8 exponent + 24 packed bytes         */
-    RFQ_MXFP6_E3M2 = 22  /* decoded exactly like E2M3 (src/loader/dequant.rs:693) */
+    RFQ_MXFP6_E3M2 = 22, /* decoded exactly like E2M3 (src/loader/dequant.rs:693) */
+    /* The block layouts of GGUF model files (public ggml definitions; 100 + the
+     * ggml type id).  ROCmForge has no decoder for them -- its loader sizes such
+     * tensors with its own layouts above (src/loader/gguf/tensor_info.rs:108-130,
+     * src/loader/gguf_tensor.rs:41-60) -- so there is no reference arithmetic to
+     * match: results follow ggml's dequantize_row_* (ggml-quants.c).  Accepted by
+     * rfq_dequant*, rfq_get_rows, rfq_dequant_rms_norm, rfq_gemv, rfq_matmul_host_weights,
+     * rfq_rms_norm_gemv and rfq_mlp_swiglu; rfq_gemm_f16 returns RFQ_E_UNSUPPORTED. */
+    RFQ_GGUF_Q4_0 = 102, /* 18 B / 32: f16 d, 16 bytes (low nibbles = elements 0-15, high = 16-31); d*(q-8) */
+    RFQ_GGUF_Q8_0 = 108, /* 34 B / 32: f16 d, 32 int8; d*q                                                 */
+    RFQ_GGUF_Q4_K = 112, /* 144 B / 256: f16 d, dmin, 12 B of 6-bit scales/mins, 128 nibble bytes          */
+    RFQ_GGUF_Q6_K = 114  /* 210 B / 256: 128 B low nibbles, 64 B high bit pairs, 16 i8 scales, f16 d       */
 } rfq_format;
 /* rfq_get_rows also gathers from a plain f32 table (GgufTensorType F32 = 0). */
 #define RFQ_TABLE_F32 0

@@ -21,6 +21,8 @@
  *              reference's test properties and an independent float64
  *              evaluation), rf_dequant_rms_norm, rf_mlp_swiglu_q (compositions
  *              of pinned parts, checked against float64)
+ *   parity unpinned (no counterpart in the reference; public ggml layouts):
+ *              rf_dequant_gguf_q4_0 / q8_0 / q4_k / q6_k
  *   parity unpinned (no reference vector, reasoned from compiler-rt source):
  *              rf_powi_f32 for exponent -128 only (returns 0.0), hence the
  *              MXFP scale byte 0x80; rf_e8m0_from_f32 when log2 lands on an
@@ -457,8 +459,110 @@ RF_API void rf_dequant_mxfp6(const uint8_t *data, size_t len, size_t n, float *o
 }
 
 /* GgufTensorType ids, src/loader/tensor_type.rs:16-32 */
+/* ------------------------------------------------------------------ */
+/* block layouts of GGUF model files (ggml)                            */
+/* ------------------------------------------------------------------ */
+/* PARITY UNPINNED against ROCmForge: nothing in the reference decodes these
+ * layouts (its Q4_0 / Q8_0 / Q4_K / Q6_K are the 20 / 36 / 256-byte layouts
+ * above).  They follow the public ggml definitions -- block_q4_0 {f16 d;
+ * u8 qs[16]}, block_q8_0 {f16 d; i8 qs[32]}, block_q4_K {f16 d, dmin;
+ * u8 scales[12]; u8 qs[128]}, block_q6_K {u8 ql[128]; u8 qh[64]; i8 scales[16];
+ * f16 d} and dequantize_row_q4_0 / q8_0 / q4_K / q6_K of ggml-quants.c -- in
+ * ggml's evaluation order, unfused.  They are pinned only by that published
+ * arithmetic: an independent numpy statement, hand-made blocks, and
+ * quantise -> dequantise error bounds in tests/.  Whole blocks only: decoding
+ * stops at the first block the input does not hold, the tail stays 0.0. */
+
+static float rd_f16le(const uint8_t *p) { return rf_f16_to_f32((uint16_t)(p[0] | (p[1] << 8))); }
+
+RF_API void rf_dequant_gguf_q4_0(const uint8_t *data, size_t len, size_t n, float *out)
+{
+    memset(out, 0, n * sizeof(float));
+    for (size_t b = 0; b * 32 + 32 <= n && b * 18 + 18 <= len; b++) {
+        const uint8_t *blk = data + b * 18;
+        float d = rd_f16le(blk);
+        for (int j = 0; j < 16; j++) {
+            int x0 = (blk[2 + j] & 0x0F) - 8, x1 = (blk[2 + j] >> 4) - 8;
+            out[b * 32 + j] = (float)x0 * d;
+            out[b * 32 + j + 16] = (float)x1 * d;
+        }
+    }
+}
+
+RF_API void rf_dequant_gguf_q8_0(const uint8_t *data, size_t len, size_t n, float *out)
+{
+    memset(out, 0, n * sizeof(float));
+    for (size_t b = 0; b * 32 + 32 <= n && b * 34 + 34 <= len; b++) {
+        const uint8_t *blk = data + b * 34;
+        float d = rd_f16le(blk);
+        for (int j = 0; j < 32; j++) out[b * 32 + j] = (float)(int8_t)blk[2 + j] * d;
+    }
+}
+
+/* get_scale_min_k4 of ggml-quants.c: 6-bit scale and min number j of 8, packed in 12 bytes */
+static void gguf_scale_min_k4(int j, const uint8_t *q, uint8_t *sc, uint8_t *m)
+{
+    if (j < 4) {
+        *sc = q[j] & 63;
+        *m = q[j + 4] & 63;
+    } else {
+        *sc = (uint8_t)((q[j + 4] & 0x0F) | ((q[j - 4] >> 6) << 4));
+        *m = (uint8_t)((q[j + 4] >> 4) | ((q[j] >> 6) << 4));
+    }
+}
+
+RF_API void rf_dequant_gguf_q4_k(const uint8_t *data, size_t len, size_t n, float *out)
+{
+    memset(out, 0, n * sizeof(float));
+    for (size_t b = 0; b * 256 + 256 <= n && b * 144 + 144 <= len; b++) {
+        const uint8_t *blk = data + b * 144;
+        float d = rd_f16le(blk), dmin = rd_f16le(blk + 2);
+        const uint8_t *scales = blk + 4, *q = blk + 16;
+        float *y = out + b * 256;
+        int is = 0;
+        for (int j = 0; j < 256; j += 64) {
+            uint8_t sc, m;
+            gguf_scale_min_k4(is + 0, scales, &sc, &m);
+            float d1 = d * (float)sc, m1 = dmin * (float)m;
+            gguf_scale_min_k4(is + 1, scales, &sc, &m);
+            float d2 = d * (float)sc, m2 = dmin * (float)m;
+            for (int l = 0; l < 32; l++) *y++ = d1 * (float)(q[l] & 0x0F) - m1;
+            for (int l = 0; l < 32; l++) *y++ = d2 * (float)(q[l] >> 4) - m2;
+            q += 32;
+            is += 2;
+        }
+    }
+}
+
+RF_API void rf_dequant_gguf_q6_k(const uint8_t *data, size_t len, size_t n, float *out)
+{
+    memset(out, 0, n * sizeof(float));
+    for (size_t b = 0; b * 256 + 256 <= n && b * 210 + 210 <= len; b++) {
+        const uint8_t *ql = data + b * 210, *qh = ql + 128;
+        const int8_t *sc = (const int8_t *)(ql + 192);
+        float d = rd_f16le(ql + 208);
+        float *y = out + b * 256;
+        for (int half = 0; half < 2; half++) {
+            for (int l = 0; l < 32; l++) {
+                int is = l / 16;
+                int q1 = (int8_t)((ql[l] & 0x0F) | (((qh[l] >> 0) & 3) << 4)) - 32;
+                int q2 = (int8_t)((ql[l + 32] & 0x0F) | (((qh[l] >> 2) & 3) << 4)) - 32;
+                int q3 = (int8_t)((ql[l] >> 4) | (((qh[l] >> 4) & 3) << 4)) - 32;
+                int q4 = (int8_t)((ql[l + 32] >> 4) | (((qh[l] >> 6) & 3) << 4)) - 32;
+                y[l] = d * (float)sc[is + 0] * (float)q1;
+                y[l + 32] = d * (float)sc[is + 2] * (float)q2;
+                y[l + 64] = d * (float)sc[is + 4] * (float)q3;
+                y[l + 96] = d * (float)sc[is + 6] * (float)q4;
+            }
+            y += 128; ql += 64; qh += 32; sc += 8;
+        }
+    }
+}
+
 enum { RF_F32 = 0, RF_F16 = 1, RF_Q4_0 = 2, RF_Q8_0 = 8, RF_Q4_K = 12, RF_Q6_K = 14,
-       RF_MXFP4 = 20, RF_MXFP6_E2M3 = 21, RF_MXFP6_E3M2 = 22 };
+       RF_MXFP4 = 20, RF_MXFP6_E2M3 = 21, RF_MXFP6_E3M2 = 22,
+       /* GGUF file layouts: 100 + the ggml type id */
+       RF_GGUF_Q4_0 = 102, RF_GGUF_Q8_0 = 108, RF_GGUF_Q4_K = 112, RF_GGUF_Q6_K = 114 };
 
 /* GgufTensor::data_size, src/loader/gguf_tensor.rs:41-75 (Q4_0 is sized
  * 36 bytes per block there although the decoder strides 20). */
@@ -486,6 +590,10 @@ RF_API size_t rf_block_bytes(int type)
     case RF_Q4_K: case RF_Q6_K: return 256;
     case RF_MXFP4: return 17;
     case RF_MXFP6_E2M3: case RF_MXFP6_E3M2: return 25;
+    case RF_GGUF_Q4_0: return 18;
+    case RF_GGUF_Q8_0: return 34;
+    case RF_GGUF_Q4_K: return 144;
+    case RF_GGUF_Q6_K: return 210;
     default: return 0;
     }
 }
@@ -509,6 +617,10 @@ RF_API int rf_dequantize(int type, const uint8_t *data, size_t len, size_t n, fl
     case RF_MXFP4: rf_dequant_mxfp4(data, len, n, out); return 0;
     case RF_MXFP6_E2M3:
     case RF_MXFP6_E3M2: rf_dequant_mxfp6(data, len, n, out); return 0;
+    case RF_GGUF_Q4_0: rf_dequant_gguf_q4_0(data, len, n, out); return 0;
+    case RF_GGUF_Q8_0: rf_dequant_gguf_q8_0(data, len, n, out); return 0;
+    case RF_GGUF_Q4_K: rf_dequant_gguf_q4_k(data, len, n, out); return 0;
+    case RF_GGUF_Q6_K: rf_dequant_gguf_q6_k(data, len, n, out); return 0;
     default: return -1;
     }
 }
@@ -560,7 +672,7 @@ RF_API int rf_qmatmul_nk(int type, const uint8_t *w, size_t w_len, const float *
                          size_t k, const int64_t *rows_sel, size_t n_sel, float *c)
 {
     size_t bb = rf_block_bytes(type);
-    size_t be = (type == RF_Q4_K || type == RF_Q6_K) ? 256 : 32;
+    size_t be = (type == RF_Q4_K || type == RF_Q6_K || type == RF_GGUF_Q4_K || type == RF_GGUF_Q6_K) ? 256 : 32;
     if (bb == 0 || k % be != 0) return -1;
     size_t row_bytes = (k / be) * bb;
     if (w_len < row_bytes * n) return -2;

@@ -16,6 +16,10 @@ template <> struct Fmt<RFQ_Q4_K> { static constexpr int BE = 256, BB = 256; };
 template <> struct Fmt<RFQ_Q6_K> { static constexpr int BE = 256, BB = 256; };
 template <> struct Fmt<RFQ_MXFP4> { static constexpr int BE = 32, BB = 17; };
 template <> struct Fmt<RFQ_MXFP6_E2M3> { static constexpr int BE = 32, BB = 25; };
+template <> struct Fmt<RFQ_GGUF_Q4_0> { static constexpr int BE = 32, BB = 18; };
+template <> struct Fmt<RFQ_GGUF_Q8_0> { static constexpr int BE = 32, BB = 34; };
+template <> struct Fmt<RFQ_GGUF_Q4_K> { static constexpr int BE = 256, BB = 144; };
+template <> struct Fmt<RFQ_GGUF_Q6_K> { static constexpr int BE = 256, BB = 210; };
 
 // MXFP6_E3M2 is decoded exactly like E2M3 by the reference
 // (src/loader/dequant.rs:693), so it shares every kernel.
@@ -25,7 +29,8 @@ inline int fmt_block_elems(int fmt)
 {
     switch (fmt) {
     case RFQ_Q4_0: case RFQ_Q8_0: case RFQ_MXFP4: case RFQ_MXFP6_E2M3: case RFQ_MXFP6_E3M2: return 32;
-    case RFQ_Q4_K: case RFQ_Q6_K: return 256;
+    case RFQ_GGUF_Q4_0: case RFQ_GGUF_Q8_0: return 32;
+    case RFQ_Q4_K: case RFQ_Q6_K: case RFQ_GGUF_Q4_K: case RFQ_GGUF_Q6_K: return 256;
     default: return 0;
     }
 }
@@ -37,6 +42,10 @@ inline int fmt_block_bytes(int fmt)
     case RFQ_Q4_K: case RFQ_Q6_K: return 256;
     case RFQ_MXFP4: return 17;
     case RFQ_MXFP6_E2M3: case RFQ_MXFP6_E3M2: return 25;
+    case RFQ_GGUF_Q4_0: return 18;
+    case RFQ_GGUF_Q8_0: return 34;
+    case RFQ_GGUF_Q4_K: return 144;
+    case RFQ_GGUF_Q6_K: return 210;
     default: return 0;
     }
 }
@@ -129,6 +138,18 @@ __device__ __forceinline__ float decode_e2m3(uint32_t q)
 
 // f32::clamp for finite bounds.
 __device__ __forceinline__ float clampf(float v, float lo, float hi) { return fminf(fmaxf(v, lo), hi); }
+
+// get_scale_min_k4 of ggml-quants.c: 6-bit scale (low 8 bits of the result) and
+// min (bits 8..15) number j of the 8 packed into 12 bytes, given as 3 dwords.
+__device__ __forceinline__ uint32_t gguf_scale_min_k4(int j, uint32_t s0, uint32_t s1, uint32_t s2)
+{
+    // bytes 0-3 = s0, 4-7 = s1, 8-11 = s2
+    const int sh = 8 * (j & 3);
+    const uint32_t a = (s0 >> sh) & 255u, b = (s1 >> sh) & 255u, c = (s2 >> sh) & 255u;
+    const uint32_t sc = j < 4 ? (a & 63u) : ((c & 15u) | ((a >> 6) << 4));
+    const uint32_t mn = j < 4 ? (b & 63u) : ((c >> 4) | ((b >> 6) << 4));
+    return sc | (mn << 8);
+}
 
 // Signed 6-bit field (two's complement) starting at bit `off` of w.
 __device__ __forceinline__ int sbfe6(uint32_t w, uint32_t off) { return ((int)(w << (26u - off))) >> 26; }

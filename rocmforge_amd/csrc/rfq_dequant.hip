@@ -109,6 +109,66 @@ template <> __device__ __forceinline__ float4 decode_quad<RFQ_MXFP6_E2M3>(const 
     return r;
 }
 
+// ---- GGUF file layouts (ggml-quants.c dequantize_row_q4_0 / q8_0 / q4_K / q6_K) ----
+// Blocks are only 2-byte aligned; the loads below are byte-exact copies.
+
+template <> __device__ __forceinline__ float4 decode_quad<RFQ_GGUF_Q4_0>(const uint8_t *blk, int e0)
+{
+    float d = f16_bits_to_f32(ld<uint16_t>(blk));
+    uint32_t w = ld<uint32_t>(blk + 2 + (e0 & 15));      // elements j and j + 16 share byte j
+    if (e0 & 16) w >>= 4;
+    float4 r;
+    r.x = (float)((int)(w & 15u) - 8) * d;
+    r.y = (float)((int)((w >> 8) & 15u) - 8) * d;
+    r.z = (float)((int)((w >> 16) & 15u) - 8) * d;
+    r.w = (float)((int)((w >> 24) & 15u) - 8) * d;
+    return r;
+}
+
+template <> __device__ __forceinline__ float4 decode_quad<RFQ_GGUF_Q8_0>(const uint8_t *blk, int e0)
+{
+    float d = f16_bits_to_f32(ld<uint16_t>(blk));
+    uint32_t w = ld<uint32_t>(blk + 2 + e0);
+    float4 r;
+    r.x = (float)(int8_t)(w & 255u) * d;
+    r.y = (float)(int8_t)((w >> 8) & 255u) * d;
+    r.z = (float)(int8_t)((w >> 16) & 255u) * d;
+    r.w = (float)(int8_t)(w >> 24) * d;
+    return r;
+}
+
+template <> __device__ __forceinline__ float4 decode_quad<RFQ_GGUF_Q4_K>(const uint8_t *blk, int e0)
+{
+    const float d = f16_bits_to_f32(ld<uint16_t>(blk)), dmin = f16_bits_to_f32(ld<uint16_t>(blk + 2));
+    const int c = e0 >> 6, h = (e0 >> 5) & 1, l = e0 & 31;   // chunk of 64, nibble half, byte
+    const uint32_t sm = gguf_scale_min_k4(2 * c + h, ld<uint32_t>(blk + 4), ld<uint32_t>(blk + 8), ld<uint32_t>(blk + 12));
+    const float d1 = d * (float)(sm & 255u), m1 = dmin * (float)(sm >> 8);
+    uint32_t w = ld<uint32_t>(blk + 16 + 32 * c + l) >> (4 * h);
+    float4 r;
+    r.x = d1 * (float)(w & 15u) - m1;
+    r.y = d1 * (float)((w >> 8) & 15u) - m1;
+    r.z = d1 * (float)((w >> 16) & 15u) - m1;
+    r.w = d1 * (float)((w >> 24) & 15u) - m1;
+    return r;
+}
+
+template <> __device__ __forceinline__ float4 decode_quad<RFQ_GGUF_Q6_K>(const uint8_t *blk, int e0)
+{
+    const int half = e0 >> 7, t = (e0 >> 5) & 3, l = e0 & 31;   // 128-element half, quarter, byte
+    const float d = f16_bits_to_f32(ld<uint16_t>(blk + 208));
+    const float sc = (float)(int8_t)blk[192 + 8 * half + 2 * t + (l >> 4)];
+    const uint32_t lo = (ld<uint32_t>(blk + 64 * half + 32 * (t & 1) + l) >> (4 * (t >> 1))) & 0x0F0F0F0Fu;
+    const uint32_t hi = (ld<uint32_t>(blk + 128 + 32 * half + l) >> (2 * t)) & 0x03030303u;
+    const uint32_t q = lo | (hi << 4);
+    const float ds = d * sc;
+    float4 r;
+    r.x = ds * (float)((int)(q & 255u) - 32);
+    r.y = ds * (float)((int)((q >> 8) & 255u) - 32);
+    r.z = ds * (float)((int)((q >> 16) & 255u) - 32);
+    r.w = ds * (float)((int)(q >> 24) - 32);
+    return r;
+}
+
 template <int FMT, bool ALIGNED16>
 __global__ void __launch_bounds__(256)
 dequant_blocks_kernel(const uint8_t *__restrict__ in, float *__restrict__ out, size_t n_quads)
@@ -252,6 +312,20 @@ template <> __device__ float decode_checked<RFQ_MXFP6_E2M3>(const uint8_t *in, s
     return clampf(mx_scale((int)(int8_t)in[off]) * decode_e2m3(q), -7.5f, 7.5f);
 }
 
+// GGUF layouts: a block the input does not hold completely decodes to 0.0.
+template <int FMT> __device__ float decode_checked_whole_blocks(const uint8_t *in, size_t len, size_t idx)
+{
+    const size_t b = idx / Fmt<FMT>::BE;
+    if ((b + 1) * Fmt<FMT>::BB > len) return 0.0f;
+    const int e = (int)(idx % Fmt<FMT>::BE);
+    const float4 q = decode_quad<FMT>(in + b * Fmt<FMT>::BB, e & ~3);
+    return (e & 3) == 0 ? q.x : ((e & 3) == 1 ? q.y : ((e & 3) == 2 ? q.z : q.w));
+}
+template <> __device__ float decode_checked<RFQ_GGUF_Q4_0>(const uint8_t *in, size_t len, size_t idx) { return decode_checked_whole_blocks<RFQ_GGUF_Q4_0>(in, len, idx); }
+template <> __device__ float decode_checked<RFQ_GGUF_Q8_0>(const uint8_t *in, size_t len, size_t idx) { return decode_checked_whole_blocks<RFQ_GGUF_Q8_0>(in, len, idx); }
+template <> __device__ float decode_checked<RFQ_GGUF_Q4_K>(const uint8_t *in, size_t len, size_t idx) { return decode_checked_whole_blocks<RFQ_GGUF_Q4_K>(in, len, idx); }
+template <> __device__ float decode_checked<RFQ_GGUF_Q6_K>(const uint8_t *in, size_t len, size_t idx) { return decode_checked_whole_blocks<RFQ_GGUF_Q6_K>(in, len, idx); }
+
 template <int FMT>
 __global__ void __launch_bounds__(256)
 dequant_checked_kernel(const uint8_t *__restrict__ in, size_t len, float *__restrict__ out, size_t first, size_t n)
@@ -351,7 +425,9 @@ int run(const uint8_t *d_in, size_t in_bytes, float *d_out, size_t n, hipStream_
     if (first < n) {
         size_t grid = (n - first + 255) / 256;
         if (grid > 0x7fffffffu) return fail(RFQ_E_SIZE, "rfq_dequant: ragged tail of %zu elements exceeds one launch", n - first);
-        hipLaunchKernelGGL((dequant_checked_kernel<FMT>), dim3((unsigned)grid), dim3(256), 0, s, d_in, in_bytes, d_out, first, n);
+        // (GGUF layouts decode whole blocks only: everything past the last whole block is 0.0)
+        const size_t reach = FMT >= RFQ_GGUF_Q4_0 ? full * BB : in_bytes;
+        hipLaunchKernelGGL((dequant_checked_kernel<FMT>), dim3((unsigned)grid), dim3(256), 0, s, d_in, reach, d_out, first, n);
         RFQ_LAUNCH_CHECK("dequant_checked_kernel");
     }
     return RFQ_OK;
@@ -447,6 +523,10 @@ int launch_rms_norm(int src_fmt, const void *d_x, const float *d_weight, float *
     case RFQ_Q6_K: return run_rms_norm<RFQ_Q6_K>(d_x, stride, d_weight, d_out, rows, hidden, eps, s);
     case RFQ_MXFP4: return run_rms_norm<RFQ_MXFP4>(d_x, stride, d_weight, d_out, rows, hidden, eps, s);
     case RFQ_MXFP6_E2M3: return run_rms_norm<RFQ_MXFP6_E2M3>(d_x, stride, d_weight, d_out, rows, hidden, eps, s);
+    case RFQ_GGUF_Q4_0: return run_rms_norm<RFQ_GGUF_Q4_0>(d_x, stride, d_weight, d_out, rows, hidden, eps, s);
+    case RFQ_GGUF_Q8_0: return run_rms_norm<RFQ_GGUF_Q8_0>(d_x, stride, d_weight, d_out, rows, hidden, eps, s);
+    case RFQ_GGUF_Q4_K: return run_rms_norm<RFQ_GGUF_Q4_K>(d_x, stride, d_weight, d_out, rows, hidden, eps, s);
+    case RFQ_GGUF_Q6_K: return run_rms_norm<RFQ_GGUF_Q6_K>(d_x, stride, d_weight, d_out, rows, hidden, eps, s);
     default: return fail(RFQ_E_BADARG, "rms_norm: unknown source format %d", src_fmt);
     }
 }
@@ -470,6 +550,10 @@ int launch_dequant(int fmt, const uint8_t *d_in, size_t in_bytes, float *d_out, 
     case RFQ_Q6_K: return run<RFQ_Q6_K>(d_in, in_bytes, d_out, n, s);
     case RFQ_MXFP4: return run<RFQ_MXFP4>(d_in, in_bytes, d_out, n, s);
     case RFQ_MXFP6_E2M3: return run<RFQ_MXFP6_E2M3>(d_in, in_bytes, d_out, n, s);
+    case RFQ_GGUF_Q4_0: return run<RFQ_GGUF_Q4_0>(d_in, in_bytes, d_out, n, s);
+    case RFQ_GGUF_Q8_0: return run<RFQ_GGUF_Q8_0>(d_in, in_bytes, d_out, n, s);
+    case RFQ_GGUF_Q4_K: return run<RFQ_GGUF_Q4_K>(d_in, in_bytes, d_out, n, s);
+    case RFQ_GGUF_Q6_K: return run<RFQ_GGUF_Q6_K>(d_in, in_bytes, d_out, n, s);
     default: return fail(RFQ_E_BADARG, "rfq_dequant: unknown format %d", fmt);
     }
 }
@@ -501,6 +585,10 @@ int launch_get_rows(int fmt, const void *d_table, int n_vocab, int n_embd, const
     case RFQ_MXFP4: rc = run_get_rows<RFQ_MXFP4>(table, d_tokens, d_out, n_vocab, n_embd, n_tokens, d_status, s); break;
     case RFQ_MXFP6_E2M3: case RFQ_MXFP6_E3M2:
         rc = run_get_rows<RFQ_MXFP6_E2M3>(table, d_tokens, d_out, n_vocab, n_embd, n_tokens, d_status, s); break;
+    case RFQ_GGUF_Q4_0: rc = run_get_rows<RFQ_GGUF_Q4_0>(table, d_tokens, d_out, n_vocab, n_embd, n_tokens, d_status, s); break;
+    case RFQ_GGUF_Q8_0: rc = run_get_rows<RFQ_GGUF_Q8_0>(table, d_tokens, d_out, n_vocab, n_embd, n_tokens, d_status, s); break;
+    case RFQ_GGUF_Q4_K: rc = run_get_rows<RFQ_GGUF_Q4_K>(table, d_tokens, d_out, n_vocab, n_embd, n_tokens, d_status, s); break;
+    case RFQ_GGUF_Q6_K: rc = run_get_rows<RFQ_GGUF_Q6_K>(table, d_tokens, d_out, n_vocab, n_embd, n_tokens, d_status, s); break;
     default: return fail(RFQ_E_BADARG, "rfq_get_rows: unknown format %d", fmt);
     }
     if (rc != RFQ_OK) return rc;

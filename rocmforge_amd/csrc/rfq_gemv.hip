@@ -269,6 +269,130 @@ template <> struct Unit<RFQ_MXFP6_E2M3> {
     }
 };
 
+// ---- GGUF file layouts (ggml block_q4_0 / q8_0 / q4_K / q6_K) -----------------
+// Blocks are 2-byte aligned only; loads are byte-exact copies.
+
+template <> struct Unit<RFQ_GGUF_Q4_0> {
+    static constexpr bool NEEDS_XSUM = true;
+    uint16_t d; U4 q;
+    __device__ __forceinline__ void load(const uint8_t *row, int u)
+    {
+        const uint8_t *p = row + (size_t)u * 18;
+        d = ld<uint16_t>(p);
+        q = ld<U4>(p + 2);
+    }
+    // element j = low nibble of byte j, element 16 + j = high nibble
+    __device__ __forceinline__ float dot(const float (&x)[32], float xsum) const
+    {
+        float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            uint32_t lo = q.v[w] & 0x0F0F0F0Fu, hi = (q.v[w] >> 4) & 0x0F0F0F0Fu;
+#pragma unroll
+            for (int b = 0; b < 4; b++) {
+                s0 = __builtin_fmaf(ub(lo, b), x[4 * w + b], s0);
+                s1 = __builtin_fmaf(ub(hi, b), x[16 + 4 * w + b], s1);
+            }
+        }
+        return f16_bits_to_f32(d) * __builtin_fmaf(-8.0f, xsum, s0 + s1);
+    }
+};
+
+template <> struct Unit<RFQ_GGUF_Q8_0> {
+    static constexpr bool NEEDS_XSUM = true;
+    uint16_t d; U8 q;
+    __device__ __forceinline__ void load(const uint8_t *row, int u)
+    {
+        const uint8_t *p = row + (size_t)u * 34;
+        d = ld<uint16_t>(p);
+        q = ld<U8>(p + 2);
+    }
+    // int8 q = (q ^ 0x80) - 128 with the left term read as an unsigned byte
+    __device__ __forceinline__ float dot(const float (&x)[32], float xsum) const
+    {
+        float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+        for (int w = 0; w < 8; w++) {
+            uint32_t v = q.v[w] ^ 0x80808080u;
+            s0 = __builtin_fmaf(ub(v, 0), x[4 * w], s0);
+            s1 = __builtin_fmaf(ub(v, 1), x[4 * w + 1], s1);
+            s0 = __builtin_fmaf(ub(v, 2), x[4 * w + 2], s0);
+            s1 = __builtin_fmaf(ub(v, 3), x[4 * w + 3], s1);
+        }
+        return f16_bits_to_f32(d) * __builtin_fmaf(-128.0f, xsum, s0 + s1);
+    }
+};
+
+// Unit u of a 144-byte super-block: chunk c = u >> 1 of 64 elements, half h = u & 1
+// (low or high nibbles of the chunk's 32 bytes); value = d * sc * q - dmin * m.
+template <> struct Unit<RFQ_GGUF_Q4_K> {
+    static constexpr bool NEEDS_XSUM = true;
+    uint32_t dd, s0, s1, s2; U8 q; int sub;
+    __device__ __forceinline__ void load(const uint8_t *row, int u)
+    {
+        const uint8_t *blk = row + (size_t)(u >> 3) * 144;
+        sub = u & 7;
+        dd = ld<uint32_t>(blk);
+        s0 = ld<uint32_t>(blk + 4); s1 = ld<uint32_t>(blk + 8); s2 = ld<uint32_t>(blk + 12);
+        q = ld<U8>(blk + 16 + 32 * (sub >> 1));
+    }
+    __device__ __forceinline__ float dot(const float (&x)[32], float xsum) const
+    {
+        const uint32_t sm = gguf_scale_min_k4(sub, s0, s1, s2);
+        const int sh = 4 * (sub & 1);
+        float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+        for (int w = 0; w < 8; w++) {
+            uint32_t v = (q.v[w] >> sh) & 0x0F0F0F0Fu;
+            a0 = __builtin_fmaf(ub(v, 0), x[4 * w], a0);
+            a1 = __builtin_fmaf(ub(v, 1), x[4 * w + 1], a1);
+            a0 = __builtin_fmaf(ub(v, 2), x[4 * w + 2], a0);
+            a1 = __builtin_fmaf(ub(v, 3), x[4 * w + 3], a1);
+        }
+        const float d1 = f16_bits_to_f32((uint16_t)(dd & 0xFFFFu)) * (float)(sm & 255u);
+        const float m1 = f16_bits_to_f32((uint16_t)(dd >> 16)) * (float)(sm >> 8);
+        return __builtin_fmaf(d1, a0 + a1, -m1 * xsum);
+    }
+};
+
+// Unit u of a 210-byte super-block: half n = (u >> 2) & 1 of 128 elements, quarter t = u & 3:
+// low nibbles from ql[64 n + 32 (t & 1) + l] (>> 4 for t >= 2), bits 4-5 from qh[32 n + l] >> 2 t,
+// scales sc[8 n + 2 t + l / 16]; value = d * sc * (q - 32).
+template <> struct Unit<RFQ_GGUF_Q6_K> {
+    static constexpr bool NEEDS_XSUM = true;
+    U8 ql, qh; uint16_t sc2, d; int t;
+    __device__ __forceinline__ void load(const uint8_t *row, int u)
+    {
+        const uint8_t *blk = row + (size_t)(u >> 3) * 210;
+        const int half = (u >> 2) & 1;
+        t = u & 3;
+        ql = ld<U8>(blk + 64 * half + 32 * (t & 1));
+        qh = ld<U8>(blk + 128 + 32 * half);
+        sc2 = ld<uint16_t>(blk + 192 + 8 * half + 2 * t);
+        d = ld<uint16_t>(blk + 208);
+    }
+    __device__ __forceinline__ float dot(const float (&x)[32], float xsum) const
+    {
+        const int shl = 4 * (t >> 1), shh = 2 * t;
+        float a[2] = {0.f, 0.f}, xs0 = 0.f;
+#pragma unroll
+        for (int w = 0; w < 8; w++) {
+            const uint32_t lo = (ql.v[w] >> shl) & 0x0F0F0F0Fu, hi = (qh.v[w] >> shh) & 0x03030303u;
+            const uint32_t v = lo | (hi << 4);
+            float s = a[w >> 2];
+            s = __builtin_fmaf(ub(v, 0), x[4 * w], s);
+            s = __builtin_fmaf(ub(v, 1), x[4 * w + 1], s);
+            s = __builtin_fmaf(ub(v, 2), x[4 * w + 2], s);
+            s = __builtin_fmaf(ub(v, 3), x[4 * w + 3], s);
+            a[w >> 2] = s;
+            if (w < 4) xs0 += (x[4 * w] + x[4 * w + 1]) + (x[4 * w + 2] + x[4 * w + 3]);
+        }
+        const float g0 = __builtin_fmaf(-32.0f, xs0, a[0]), g1 = __builtin_fmaf(-32.0f, xsum - xs0, a[1]);
+        const float c0 = (float)(int8_t)(sc2 & 255u), c1 = (float)(int8_t)(sc2 >> 8);
+        return f16_bits_to_f32(d) * __builtin_fmaf(c0, g0, c1 * g1);
+    }
+};
+
 template <int FMT> __host__ __device__ constexpr size_t row_bytes(int k)
 {
     return (size_t)(k / Fmt<FMT>::BE) * Fmt<FMT>::BB;
@@ -393,7 +517,11 @@ gemv_xreg_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
                  int groups, GemvFuse f)
 {
     constexpr int TEAMS = 4 / WPR, TL = 64 * WPR;
+#ifdef RFQ_XREG_D
+    constexpr int D = R < RFQ_XREG_D ? R : RFQ_XREG_D;
+#else
     constexpr int D = R < 3 ? R : 3;
+#endif
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int team = wave / WPR, wit = wave % WPR;
     const int tl = wit * 64 + lane;
@@ -1310,6 +1438,10 @@ int launch_gemv(int fmt, const uint8_t *d_w, const float *d_x, float *d_y, int m
     case RFQ_Q6_K: return run<RFQ_Q6_K>(d_w, d_x, d_y, m, n, k, s);
     case RFQ_MXFP4: return run<RFQ_MXFP4>(d_w, d_x, d_y, m, n, k, s);
     case RFQ_MXFP6_E2M3: return run<RFQ_MXFP6_E2M3>(d_w, d_x, d_y, m, n, k, s);
+    case RFQ_GGUF_Q4_0: return run<RFQ_GGUF_Q4_0>(d_w, d_x, d_y, m, n, k, s);
+    case RFQ_GGUF_Q8_0: return run<RFQ_GGUF_Q8_0>(d_w, d_x, d_y, m, n, k, s);
+    case RFQ_GGUF_Q4_K: return run<RFQ_GGUF_Q4_K>(d_w, d_x, d_y, m, n, k, s);
+    case RFQ_GGUF_Q6_K: return run<RFQ_GGUF_Q6_K>(d_w, d_x, d_y, m, n, k, s);
     default: return fail(RFQ_E_BADARG, "rfq_gemv: unknown format %d", fmt);
     }
 }
@@ -1334,6 +1466,10 @@ int launch_gemv_fused(int fmt, const uint8_t *d_w, const uint8_t *d_w2, const fl
     case RFQ_Q6_K: return run_rows<RFQ_Q6_K, true>(d_w, d_x, d_y, rows, k, f, s);
     case RFQ_MXFP4: return run_rows<RFQ_MXFP4, true>(d_w, d_x, d_y, rows, k, f, s);
     case RFQ_MXFP6_E2M3: return run_rows<RFQ_MXFP6_E2M3, true>(d_w, d_x, d_y, rows, k, f, s);
+    case RFQ_GGUF_Q4_0: return run_rows<RFQ_GGUF_Q4_0, true>(d_w, d_x, d_y, rows, k, f, s);
+    case RFQ_GGUF_Q8_0: return run_rows<RFQ_GGUF_Q8_0, true>(d_w, d_x, d_y, rows, k, f, s);
+    case RFQ_GGUF_Q4_K: return run_rows<RFQ_GGUF_Q4_K, true>(d_w, d_x, d_y, rows, k, f, s);
+    case RFQ_GGUF_Q6_K: return run_rows<RFQ_GGUF_Q6_K, true>(d_w, d_x, d_y, rows, k, f, s);
     default: return fail(RFQ_E_BADARG, "fused gemv: unknown format %d", fmt);
     }
 }

@@ -25,11 +25,17 @@ from __future__ import annotations
 import numpy as np
 
 Q4_0, Q8_0, Q4_K, Q6_K, MXFP4, MXFP6_E2M3, MXFP6_E3M2 = 2, 8, 12, 14, 20, 21, 22
+# the block layouts of GGUF model files (ggml), which ROCmForge does not decode: 100 + the ggml type id
+GGUF_Q4_0, GGUF_Q8_0, GGUF_Q4_K, GGUF_Q6_K = 102, 108, 112, 114
+GGUF_FORMATS = (GGUF_Q4_0, GGUF_Q8_0, GGUF_Q4_K, GGUF_Q6_K)
 
-BLOCK_ELEMS = {Q4_0: 32, Q8_0: 32, Q4_K: 256, Q6_K: 256, MXFP4: 32, MXFP6_E2M3: 32, MXFP6_E3M2: 32}
-BLOCK_BYTES = {Q4_0: 20, Q8_0: 36, Q4_K: 256, Q6_K: 256, MXFP4: 17, MXFP6_E2M3: 25, MXFP6_E3M2: 25}
+BLOCK_ELEMS = {Q4_0: 32, Q8_0: 32, Q4_K: 256, Q6_K: 256, MXFP4: 32, MXFP6_E2M3: 32, MXFP6_E3M2: 32,
+               GGUF_Q4_0: 32, GGUF_Q8_0: 32, GGUF_Q4_K: 256, GGUF_Q6_K: 256}
+BLOCK_BYTES = {Q4_0: 20, Q8_0: 36, Q4_K: 256, Q6_K: 256, MXFP4: 17, MXFP6_E2M3: 25, MXFP6_E3M2: 25,
+               GGUF_Q4_0: 18, GGUF_Q8_0: 34, GGUF_Q4_K: 144, GGUF_Q6_K: 210}
 NAMES = {Q4_0: "Q4_0", Q8_0: "Q8_0", Q4_K: "Q4_K", Q6_K: "Q6_K", MXFP4: "MXFP4",
-         MXFP6_E2M3: "MXFP6_E2M3", MXFP6_E3M2: "MXFP6_E3M2"}
+         MXFP6_E2M3: "MXFP6_E2M3", MXFP6_E3M2: "MXFP6_E3M2",
+         GGUF_Q4_0: "GGUF_Q4_0", GGUF_Q8_0: "GGUF_Q8_0", GGUF_Q4_K: "GGUF_Q4_K", GGUF_Q6_K: "GGUF_Q6_K"}
 
 
 def packed_bytes(fmt: int, n_elems: int) -> int:
@@ -203,10 +209,113 @@ def pack_mxfp6(values: np.ndarray) -> np.ndarray:
     return out.ravel()
 
 
+# ---- GGUF file layouts (public ggml block definitions) ---------------------------------
+#   GGUF_Q4_0  18 B / 32 : f16 d, 16 bytes; element j = low nibble of byte j, j + 16 = high nibble; d * (q - 8)
+#   GGUF_Q8_0  34 B / 32 : f16 d, 32 int8; d * q
+#   GGUF_Q4_K 144 B / 256: f16 d, f16 dmin, 12 bytes of 6-bit scales and mins (8 each), 128 nibble bytes; per
+#                          64 elements: low nibbles then high nibbles of 32 bytes; d * sc * q - dmin * m
+#   GGUF_Q6_K 210 B / 256: 128 bytes of low nibbles, 64 bytes of high bit pairs, 16 int8 scales, f16 d;
+#                          d * sc * (q - 32)
+# The quantisers below are simple decision rules (no search); they exist to produce valid inputs whose
+# dequantised values approximate w, not to match ggml's quantiser bit for bit.
+
+def _f16_bytes(x: np.ndarray) -> np.ndarray:
+    return np.ascontiguousarray(x, dtype="<f2").view(np.uint8)
+
+
+def quantize_gguf_q4_0(w: np.ndarray) -> np.ndarray:
+    b = _blocks(w, 32)
+    idx = np.argmax(np.abs(b), axis=1)
+    mx = b[np.arange(b.shape[0]), idx]
+    d = _f16_round(mx / -8.0)
+    inv = np.where(d != 0, 1.0 / np.where(d != 0, d, 1.0), 0.0).astype(np.float32)
+    q = np.clip(np.floor(b * inv[:, None] + 8.5), 0, 15).astype(np.uint8)
+    out = np.zeros((b.shape[0], 18), np.uint8)
+    out[:, 0:2] = _f16_bytes(d).reshape(-1, 2)
+    out[:, 2:] = q[:, :16] | (q[:, 16:] << 4)
+    return out.ravel()
+
+
+def quantize_gguf_q8_0(w: np.ndarray) -> np.ndarray:
+    b = _blocks(w, 32)
+    d = _f16_round(np.abs(b).max(axis=1) / 127.0)
+    inv = np.where(d != 0, 1.0 / np.where(d != 0, d, 1.0), 0.0).astype(np.float32)
+    q = np.clip(np.rint(b * inv[:, None]), -127, 127).astype(np.int8)
+    out = np.zeros((b.shape[0], 34), np.uint8)
+    out[:, 0:2] = _f16_bytes(d).reshape(-1, 2)
+    out[:, 2:] = q.view(np.uint8)
+    return out.ravel()
+
+
+def pack_scale_min_k4(sc: np.ndarray, mn: np.ndarray) -> np.ndarray:
+    """Eight 6-bit scales and eight 6-bit mins per block -> the 12 bytes get_scale_min_k4 reads."""
+    sc, mn = sc.astype(np.uint8), mn.astype(np.uint8)
+    out = np.zeros((sc.shape[0], 12), np.uint8)
+    out[:, 0:4] = (sc[:, 0:4] & 63) | ((sc[:, 4:8] >> 4) << 6)
+    out[:, 4:8] = (mn[:, 0:4] & 63) | ((mn[:, 4:8] >> 4) << 6)
+    out[:, 8:12] = (sc[:, 4:8] & 15) | ((mn[:, 4:8] & 15) << 4)
+    return out
+
+
+def quantize_gguf_q4_k(w: np.ndarray) -> np.ndarray:
+    b = _blocks(w, 256).reshape(-1, 8, 32)                        # sub-blocks of 32
+    lo = np.minimum(b.min(axis=2), 0.0)                           # value = scale * q - min, min >= 0
+    scale = (b.max(axis=2) - lo) / 15.0
+    d = _f16_round(scale.max(axis=1) / 63.0)
+    dmin = _f16_round((-lo).max(axis=1) / 63.0)
+    inv_d = np.where(d != 0, 1.0 / np.where(d != 0, d, 1.0), 0.0).astype(np.float32)
+    inv_m = np.where(dmin != 0, 1.0 / np.where(dmin != 0, dmin, 1.0), 0.0).astype(np.float32)
+    sc = np.clip(np.rint(scale * inv_d[:, None]), 0, 63)
+    mn = np.clip(np.rint(-lo * inv_m[:, None]), 0, 63)
+    eff_s = (d[:, None] * sc).astype(np.float32)
+    eff_m = (dmin[:, None] * mn).astype(np.float32)
+    inv_s = np.where(eff_s != 0, 1.0 / np.where(eff_s != 0, eff_s, 1.0), 0.0).astype(np.float32)
+    q = np.clip(np.rint((b + eff_m[:, :, None]) * inv_s[:, :, None]), 0, 15).astype(np.uint8)
+    out = np.zeros((b.shape[0], 144), np.uint8)
+    out[:, 0:2] = _f16_bytes(d).reshape(-1, 2)
+    out[:, 2:4] = _f16_bytes(dmin).reshape(-1, 2)
+    out[:, 4:16] = pack_scale_min_k4(sc, mn)
+    q = q.reshape(-1, 4, 2, 32)                                   # chunk of 64: low nibbles, then high nibbles
+    out[:, 16:] = (q[:, :, 0, :] | (q[:, :, 1, :] << 4)).reshape(-1, 128)
+    return out.ravel()
+
+
+def quantize_gguf_q6_k(w: np.ndarray) -> np.ndarray:
+    b = _blocks(w, 256).reshape(-1, 16, 16)                       # groups of 16
+    amax = np.abs(b).max(axis=2)
+    scale = amax / 31.0
+    d = _f16_round(scale.max(axis=1) / 127.0)
+    inv_d = np.where(d != 0, 1.0 / np.where(d != 0, d, 1.0), 0.0).astype(np.float32)
+    sc = np.clip(np.rint(scale * inv_d[:, None]), 0, 127).astype(np.int8)
+    eff = (d[:, None] * sc).astype(np.float32)
+    inv = np.where(eff != 0, 1.0 / np.where(eff != 0, eff, 1.0), 0.0).astype(np.float32)
+    q = (np.clip(np.rint(b * inv[:, :, None]), -32, 31) + 32).astype(np.uint8).reshape(-1, 2, 4, 32)   # half, quarter, l
+    out = np.zeros((b.shape[0], 210), np.uint8)
+    lo, hi = q & 15, q >> 4
+    ql = np.zeros((b.shape[0], 2, 64), np.uint8)
+    ql[:, :, 0:32] = lo[:, :, 0, :] | (lo[:, :, 2, :] << 4)
+    ql[:, :, 32:64] = lo[:, :, 1, :] | (lo[:, :, 3, :] << 4)
+    qh = hi[:, :, 0, :] | (hi[:, :, 1, :] << 2) | (hi[:, :, 2, :] << 4) | (hi[:, :, 3, :] << 6)
+    out[:, 0:128] = ql.reshape(-1, 128)
+    out[:, 128:192] = qh.reshape(-1, 64)
+    out[:, 192:208] = sc.view(np.uint8)
+    out[:, 208:210] = _f16_bytes(d).reshape(-1, 2)
+    return out.ravel()
+
+
 def random_blocks(fmt: int, n_blocks: int, rng: np.random.Generator, exp_range=(-20, 12)) -> np.ndarray:
     """Uniformly random payload bytes with sane scales, covering every code."""
     bb = BLOCK_BYTES[fmt]
     out = rng.integers(0, 256, (n_blocks, bb), dtype=np.uint8)
+    if fmt in GGUF_FORMATS:
+        d = (rng.standard_normal((n_blocks, 2)) * 0.01).astype("<f2").view(np.uint8).reshape(-1, 4)
+        if fmt in (GGUF_Q4_0, GGUF_Q8_0):
+            out[:, 0:2] = d[:, 0:2]
+        elif fmt == GGUF_Q4_K:
+            out[:, 0:4] = d
+        else:
+            out[:, 208:210] = d[:, 0:2]
+        return out.ravel()
     if fmt in (Q4_0, Q8_0):
         s = (rng.standard_normal(n_blocks) * 0.01).astype("<f4")
         out[:, 0:4] = s.view(np.uint8).reshape(-1, 4)
@@ -232,6 +341,9 @@ def make_weights(fmt: int, n: int, k: int, seed: int, std: float = 0.02) -> np.n
         return quantize_q8_0(w)
     if fmt == Q6_K:
         return quantize_q6_k(w, rng)
+    if fmt in GGUF_FORMATS:
+        return {GGUF_Q4_0: quantize_gguf_q4_0, GGUF_Q8_0: quantize_gguf_q8_0, GGUF_Q4_K: quantize_gguf_q4_k,
+                GGUF_Q6_K: quantize_gguf_q6_k}[fmt](w)
     if fmt == MXFP4:
         return pack_mxfp4(w)
     return pack_mxfp6(w)

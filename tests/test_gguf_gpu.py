@@ -1,0 +1,143 @@
+"""GPU parity for the GGUF block layouts (ggml block_q4_0 / q8_0 / q4_K / q6_K) against
+the oracle's restatement of ggml's decoders.  PARITY UNPINNED against ROCmForge: the
+reference does not decode these layouts; see tests/test_gguf_oracle.py for what pins the
+oracle."""
+import numpy as np
+import pytest
+
+from helpers import assert_bit_exact, assert_close
+from rocmforge_amd import quantize as Q
+
+pytestmark = pytest.mark.gpu
+F = Q.GGUF_FORMATS
+
+
+def dev(a, cuda):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).to(cuda)
+
+
+def host(t):
+    import torch
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def gauss(shape, seed, std=1.0):
+    rng = np.random.Generator(np.random.PCG64(seed))
+    return (rng.standard_normal(shape, dtype=np.float32) * np.float32(std)).astype(np.float32)
+
+
+@pytest.mark.parametrize("fmt", F)
+def test_dequant_random_blocks_bit_exact(fmt, oracle, cuda):
+    from rocmforge_amd import ops
+    rng = np.random.default_rng(1100 + fmt)
+    blocks = 4099                                           # odd: the last workgroup is ragged
+    data = Q.random_blocks(fmt, blocks, rng)
+    n = blocks * Q.BLOCK_ELEMS[fmt]
+    got = host(ops.dequant(fmt, dev(data, cuda), n))
+    assert_bit_exact(got, oracle.dequantize(fmt, data, n), Q.NAMES[fmt])
+
+
+@pytest.mark.parametrize("fmt", F)
+def test_dequant_quantised_weights_bit_exact(fmt, oracle, cuda):
+    from rocmforge_amd import ops
+    n, k = 512, 4096
+    data = Q.make_weights(fmt, n, k, seed=1110 + fmt)
+    got = host(ops.dequant(fmt, dev(data, cuda), n * k))
+    assert_bit_exact(got, oracle.dequantize(fmt, data, n * k), Q.NAMES[fmt])
+
+
+@pytest.mark.parametrize("fmt", F)
+def test_dequant_short_input_and_ragged_count(fmt, oracle, cuda):
+    from rocmforge_amd import ops
+    rng = np.random.default_rng(1120 + fmt)
+    be, bb = Q.BLOCK_ELEMS[fmt], Q.BLOCK_BYTES[fmt]
+    data = Q.random_blocks(fmt, 9, rng)
+    for cut_bytes, n in ((8 * bb + bb // 2, 9 * be), (9 * bb, 8 * be + 7), (bb - 1, be), (9 * bb, 9 * be)):
+        part = data[:cut_bytes]
+        got = host(ops.dequant(fmt, dev(part, cuda), n))
+        assert_bit_exact(got, oracle.dequantize(fmt, part, n), f"{Q.NAMES[fmt]} bytes={cut_bytes} n={n}")
+
+
+@pytest.mark.parametrize("fmt", F)
+def test_get_rows_and_dequant_rms_norm(fmt, oracle, cuda):
+    import torch
+    from rocmforge_amd import ops
+    n_vocab, n_embd = 300, 1024
+    tab = Q.make_weights(fmt, n_vocab, n_embd, seed=1130 + fmt)
+    tokens = np.array([299, 0, 17, 17, 5], dtype=np.int32)
+    got = host(ops.get_rows(fmt, dev(tab, cuda), dev(tokens, cuda), n_vocab, n_embd))
+    want, bad = oracle.get_rows(fmt, tab, tokens, n_vocab, n_embd)
+    assert bad is None
+    assert_bit_exact(got, want, f"get_rows {Q.NAMES[fmt]}")
+    w = (1.0 + 0.2 * gauss((n_embd,), 1131)).astype(np.float32)
+    rows = 7
+    packed = tab[:rows * Q.packed_bytes(fmt, n_embd)]
+    got = host(ops.dequant_rms_norm(fmt, dev(packed, cuda), dev(w, cuda), rows, n_embd, 1e-5))
+    assert_close(got, oracle.dequant_rms_norm(fmt, packed, w, rows, n_embd, 1e-5), f"rms {Q.NAMES[fmt]}", tol=1e-5)
+
+
+@pytest.mark.parametrize("fmt", F)
+@pytest.mark.parametrize("n,k", [(5, 256), (40, 512), (77, 768), (64, 2048), (1001, 2048), (130, 4096), (257, 8192),
+                                 (19, 14336), (9, 32768), (2048, 1536)])
+def test_gemv_m1_shapes(fmt, n, k, oracle, cuda):
+    from rocmforge_amd import ops
+    w = Q.make_weights(fmt, n, k, seed=1200 + fmt + n)
+    x = gauss((k,), 1210 + k)
+    got = host(ops.gemv(fmt, dev(w, cuda), dev(x, cuda), n, k))
+    assert_close(got, oracle.qmatmul_nk(fmt, w, x[None, :], 1, n, k)[0], f"{Q.NAMES[fmt]} n={n} k={k}")
+
+
+@pytest.mark.parametrize("fmt", F)
+def test_gemv_random_blocks(fmt, oracle, cuda):
+    # every code and scale pattern, not only what the quantisers emit
+    from rocmforge_amd import ops
+    n, k = 96, 2048
+    rng = np.random.default_rng(1220 + fmt)
+    w = Q.random_blocks(fmt, n * k // Q.BLOCK_ELEMS[fmt], rng)
+    x = gauss((k,), 1221)
+    got = host(ops.gemv(fmt, dev(w, cuda), dev(x, cuda), n, k))
+    assert_close(got, oracle.qmatmul_nk(fmt, w, x[None, :], 1, n, k)[0], f"{Q.NAMES[fmt]} random blocks")
+
+
+@pytest.mark.parametrize("fmt", F)
+@pytest.mark.parametrize("m", [2, 5, 8])
+def test_gemv_small_batches(fmt, m, oracle, cuda):
+    from rocmforge_amd import ops
+    n, k = 301, 2048
+    w = Q.make_weights(fmt, n, k, seed=1230 + fmt)
+    x = gauss((m, k), 1240 + m)
+    got = host(ops.gemv(fmt, dev(w, cuda), dev(x, cuda), n, k))
+    assert_close(got, oracle.qmatmul_nk(fmt, w, x, m, n, k), f"{Q.NAMES[fmt]} m={m}")
+
+
+@pytest.mark.parametrize("fmt", F)
+def test_rms_norm_gemv_and_mlp(fmt, oracle, cuda):
+    from rocmforge_amd import ops
+    hidden, inter = 2048, 2816
+    nw = (1.0 + 0.2 * gauss((hidden,), 1250)).astype(np.float32)
+    x = gauss((hidden,), 1251, 2.0)
+    w = Q.make_weights(fmt, 130, hidden, seed=1252 + fmt)
+    got = host(ops.rms_norm_gemv(fmt, dev(w, cuda), dev(x, cuda), dev(nw, cuda), 1e-5, 130, hidden))
+    assert_close(got, oracle.qmatmul_nk(fmt, w, oracle.rms_norm(x[None, :], nw, 1e-5), 1, 130, hidden)[0],
+                 f"rms_norm_gemv {Q.NAMES[fmt]}")
+    wg = Q.make_weights(fmt, inter, hidden, seed=1260 + fmt)
+    wu = Q.make_weights(fmt, inter, hidden, seed=1261 + fmt)
+    wd = Q.make_weights(fmt, hidden, inter, seed=1262 + fmt)
+    for m in (1, 3):
+        xm = gauss((m, hidden), 1263 + m)
+        got = host(ops.mlp_swiglu(fmt, dev(wg, cuda), dev(wu, cuda), fmt, dev(wd, cuda), dev(xm[0] if m == 1 else xm, cuda),
+                                  dev(nw, cuda), 1e-5, hidden, inter)).reshape(m, hidden)
+        assert_close(got, oracle.mlp_swiglu_q(fmt, wg, wu, fmt, wd, xm, nw, 1e-5, m, hidden, inter),
+                     f"mlp {Q.NAMES[fmt]} m={m}")
+
+
+def test_gemm_f16_has_no_kernel_for_gguf_layouts(cuda):
+    import torch
+    from rocmforge_amd import _lib, ops
+    w = dev(Q.make_weights(Q.GGUF_Q4_K, 128, 1024, seed=1), cuda)
+    a = torch.zeros((64, 1024), dtype=torch.float16, device=cuda)
+    with pytest.raises(_lib.RfqError) as e:
+        ops.gemm_f16(Q.GGUF_Q4_K, w, a, 128, 1024)
+    assert e.value.status == _lib.E_UNSUPPORTED
