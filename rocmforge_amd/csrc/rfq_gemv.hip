@@ -761,6 +761,79 @@ template <> struct IUnit<RFQ_Q8_0> : Unit<RFQ_Q8_0> {
     }
 };
 
+// GGUF layouts: x limbs in plain order (group g = elements 4g .. 4g+3).
+
+template <> struct IUnit<RFQ_GGUF_Q4_0> : Unit<RFQ_GGUF_Q4_0> {
+    static constexpr bool NIBBLE = false;
+    static constexpr uint32_t TOPOFF = 0;
+    // low nibbles of dword w are elements 4w .. 4w+3 (group w), high nibbles elements 16+4w .. (group 4+w)
+    __device__ __forceinline__ float idot(const XPrep &xp) const
+    {
+        uint32_t alo = 0, amid = 0;
+        int atop = 0;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            uint32_t lo = q.v[w] & 0x0F0F0F0Fu, hi = (q.v[w] >> 4) & 0x0F0F0F0Fu;
+            const uint32_t *L = &xp.l[w * 3], *H = &xp.l[(4 + w) * 3];
+            alo = __builtin_amdgcn_udot4(lo, L[0], alo, false);
+            amid = __builtin_amdgcn_udot4(lo, L[1], amid, false);
+            atop = __builtin_amdgcn_sdot4((int)lo, (int)L[2], atop, false);
+            alo = __builtin_amdgcn_udot4(hi, H[0], alo, false);
+            amid = __builtin_amdgcn_udot4(hi, H[1], amid, false);
+            atop = __builtin_amdgcn_sdot4((int)hi, (int)H[2], atop, false);
+        }
+        float S = __builtin_fmaf((float)atop, 65536.0f, __builtin_fmaf((float)amid, 256.0f, (float)alo));
+        return f16_bits_to_f32(d) * __builtin_fmaf(xp.s, S, -8.0f * xp.xsum);
+    }
+};
+
+template <> struct IUnit<RFQ_GGUF_Q8_0> : Unit<RFQ_GGUF_Q8_0> {
+    static constexpr bool NIBBLE = false;
+    static constexpr uint32_t TOPOFF = 0x400000u; // offset-binary weight bytes reach 255: keep every limb unsigned
+    __device__ __forceinline__ float idot(const XPrep &xp) const
+    {
+        uint32_t alo = 0, amid = 0, atop = 0, bsum = 0;
+#pragma unroll
+        for (int g = 0; g < 8; g++) {
+            const uint32_t v = q.v[g] ^ 0x80808080u;   // int8 q -> q + 128
+            const uint32_t *L = &xp.l[g * 3];
+            alo = __builtin_amdgcn_udot4(v, L[0], alo, false);
+            amid = __builtin_amdgcn_udot4(v, L[1], amid, false);
+            atop = __builtin_amdgcn_udot4(v, L[2], atop, false);
+            bsum = __builtin_amdgcn_udot4(v, 0x01010101u, bsum, false);
+        }
+        // top limbs carry +64: sum b*(top+64) - 64*sum b
+        float S = __builtin_fmaf((float)((int)atop - 64 * (int)bsum), 65536.0f,
+                                 __builtin_fmaf((float)amid, 256.0f, (float)alo));
+        return f16_bits_to_f32(d) * __builtin_fmaf(xp.s, S, -128.0f * xp.xsum);
+    }
+};
+
+template <> struct IUnit<RFQ_GGUF_Q4_K> : Unit<RFQ_GGUF_Q4_K> {
+    static constexpr bool NIBBLE = false;
+    static constexpr uint32_t TOPOFF = 0;
+    // byte l of the chunk holds element l of this unit in its low (even unit) or high (odd unit) nibble
+    __device__ __forceinline__ float idot(const XPrep &xp) const
+    {
+        const uint32_t sm = gguf_scale_min_k4(sub, s0, s1, s2);
+        const int sh = 4 * (sub & 1);
+        uint32_t alo = 0, amid = 0;
+        int atop = 0;
+#pragma unroll
+        for (int w = 0; w < 8; w++) {
+            const uint32_t v = (q.v[w] >> sh) & 0x0F0F0F0Fu;
+            const uint32_t *L = &xp.l[w * 3];
+            alo = __builtin_amdgcn_udot4(v, L[0], alo, false);
+            amid = __builtin_amdgcn_udot4(v, L[1], amid, false);
+            atop = __builtin_amdgcn_sdot4((int)v, (int)L[2], atop, false);
+        }
+        const float S = __builtin_fmaf((float)atop, 65536.0f, __builtin_fmaf((float)amid, 256.0f, (float)alo));
+        const float d1 = f16_bits_to_f32((uint16_t)(dd & 0xFFFFu)) * (float)(sm & 255u);
+        const float m1 = f16_bits_to_f32((uint16_t)(dd >> 16)) * (float)(sm >> 8);
+        return __builtin_fmaf(d1 * xp.s, S, -m1 * xp.xsum);
+    }
+};
+
 // Block = 4 wavefronts = 4 / WPR teams.  Lane `tl` of a team owns units
 // tl + j*64*WPR, j < UPL, of every row the team visits.  A team walks
 // `groups` groups of R consecutive rows; R is a compile-time constant so a
@@ -1253,6 +1326,11 @@ template <int FMT> struct HasIdot { static constexpr bool value = false; };
 template <> struct HasIdot<RFQ_Q4_K> { static constexpr bool value = true; };
 template <> struct HasIdot<RFQ_Q4_0> { static constexpr bool value = true; };
 template <> struct HasIdot<RFQ_Q8_0> { static constexpr bool value = true; };
+template <> struct HasIdot<RFQ_GGUF_Q4_0> { static constexpr bool value = true; };
+template <> struct HasIdot<RFQ_GGUF_Q8_0> { static constexpr bool value = true; };
+template <> struct HasIdot<RFQ_GGUF_Q4_K> { static constexpr bool value = true; };
+// (batches of the GGUF layouts go through the one-row-per-wavefront kernel)
+template <int FMT> struct HasIdotBatch { static constexpr bool value = HasIdot<FMT>::value && FMT < RFQ_GGUF_Q4_0; };
 
 template <int FMT, int UPL, int WPR, int R, bool FUSE>
 int launch_idot(const uint8_t *w, const float *x, float *y, int n, int k, int blocks, int groups, const GemvFuse &f,
@@ -1323,7 +1401,7 @@ int launch_idot_batch(const uint8_t *w, const float *x, float *y, int m, int n, 
 template <int FMT, int WPR, int M>
 int run_idot_batch(const uint8_t *w, const float *x, float *y, int m, int n, int k, hipStream_t s)
 {
-    if constexpr (HasIdot<FMT>::value) {
+    if constexpr (HasIdotBatch<FMT>::value) {
         constexpr int TEAMS = 4 / WPR;
         // one or two resident blocks per CU (LDS holds the M prepared vectors),
         // every team walking the same number of rows
@@ -1409,7 +1487,7 @@ int run(const uint8_t *w, const float *x, float *y, int m, int n, int k, hipStre
     if (m == 1 && ku > 16 && ku <= 512)                        // (shorter rows leave most of a wavefront's lanes without a unit)
         return run_rows<FMT, false>(w, x, y, n, k, GemvFuse{nullptr, nullptr, 0.0f, 0}, s);
     if (FMT == RFQ_Q8_0 && m > 1 && (reinterpret_cast<uintptr_t>(w) & 3u) == 0) return run_mfma_q8_0(w, x, y, m, n, k, s);
-    if (HasIdot<FMT>::value && m > 1 && ku > 32 && ku <= 256) {
+    if (HasIdotBatch<FMT>::value && m > 1 && ku > 32 && ku <= 256) {
         if (m <= 2) return run_idot_batch_k<FMT, 2>(w, x, y, m, n, k, s);
         if (m <= 4) return run_idot_batch_k<FMT, 4>(w, x, y, m, n, k, s);
         return run_idot_batch_k<FMT, 8>(w, x, y, m, n, k, s);
