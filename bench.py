@@ -276,6 +276,14 @@ def main():
         b = algorithmic_bytes(Q.Q4_K, 128256, 4096, 1, Q)
         also["Q4_K gemv 128256x4096 (LM head)"] = {"GB/s": round(b / (d / 50) / 1e9, 1), "us": round(d / 50 * 1e6, 2),
                                                    "hbm_frac": round(b / (d / 50) / 1e9 / HBM_PEAK_GBS, 4)}
+        # the block layouts of GGUF model files (no counterpart in the reference: reported beside, never as its parity)
+        for name, f, n, k, seed in (("GGUF_Q4_K gemv 14336x4096", Q.GGUF_Q4_K, N, K, 20260051),
+                                    ("GGUF_Q6_K gemv 14336x4096", Q.GGUF_Q6_K, N, K, 20260052)):
+            c = min(-(-int(2.5 * CACHE_BYTES) // Q.packed_bytes(f, n * k)), 64)
+            _, d, *_ = time_gemv(torch, f, n, k, 1, c, 500, 50, Q, seed)
+            b = algorithmic_bytes(f, n, k, 1, Q)
+            also[name] = {"GB/s": round(b / (d / 500) / 1e9, 1), "us": round(d / 500 * 1e6, 2),
+                          "hbm_frac": round(b / (d / 500) / 1e9 / HBM_PEAK_GBS, 4)}
         also["Q4_K mlp_swiglu 4096x14336 m1"] = time_mlp(torch, Q.Q4_K, 4096, 14336, Q)
         also["Q4_K get_rows 512 of 128256x4096"] = time_get_rows(torch, Q.Q4_K, 128256, 4096, 512, Q)
         for name, f, n, k, seed in (("Q4_0 dequant 4096x4096", Q.Q4_0, 4096, 4096, 20260021),

@@ -128,8 +128,10 @@ RFQ_API int rfq_dequant_host(int fmt, const uint8_t *h_packed, size_t packed_byt
 
 /* ---- decode GEMV (and small batches) -------------------------------------- */
 
-/* d_y[m, n] = d_x[m, k] . dequant(W)[n, k]^T, fp32 accumulation, 1 <= m <= 8,
- * k a multiple of the block size, w_bytes == n * (k / block_elems) * block_bytes.
+/* d_y[m, n] = d_x[m, k] . dequant(W)[n, k]^T, fp32 accumulation, k a multiple
+ * of the block size, w_bytes == n * (k / block_elems) * block_bytes.  Built for
+ * decode, 1 <= m <= 8 (one launch); larger m runs eight rows per launch and
+ * re-reads W each time -- a prefill belongs to rfq_gemm_f16 / rfq_gemm_mx.
  * Replaces matmul_q4_0_gpu (src/kernels/matmul/quantized/q4_0.rs:209-260) and
  * its q4_k / q6_k twins (q4_k.rs:221-268, q6_k.rs:211-258), for every format. */
 RFQ_API int rfq_gemv(int fmt, const void *d_w, size_t w_bytes, const float *d_x, float *d_y, int m, int n,

@@ -18,8 +18,8 @@
  *   matmul_q4_0_gpu       src/kernels/matmul/quantized/q4_0.rs:209-260
  *   dequantize_q4_0_kernel_cached, dequantize_q4_k_gpu_kernel, dequantize_q6_k_gpu_kernel
  *                         src/kernels/quant/q4_0.rs:107, q4_k.rs:99, q6_k.rs:102
- *   QuantFormat, QuantizedMatmulOp
- *                         src/ggml/hip_backend/ops/batch_quantized.rs:20-90
+ *   QuantFormat, QuantizedMatmulOp, BatchMatmulResult, BatchQuantizedMatmul
+ *                         src/ggml/hip_backend/ops/batch_quantized.rs:20-255
  *   validate_matmul_q4_0 / q8_0 (the checks of execute_matmul_q4_0 / q8_0)
  *                         src/ggml/hip_backend/op_dispatch.rs:951-1083
  *   get_rows, validate_token_ids
@@ -41,6 +41,7 @@
 
 #include <hip/hip_runtime_api.h>
 
+#include <chrono>
 #include <cstdint>
 #include <cstring>
 #include <limits>
@@ -384,7 +385,7 @@ inline Status matmul_q4_0_gpu(const HipBackend &b, const float *act, const uint8
     return detail::from_rfq(rfq_matmul_q4_0(act, w, out, (int)m, (int)n, (int)k, b.stream()), "matmul_q4_0_gpu");
 }
 
-// ---- batch description types (src/ggml/hip_backend/ops/batch_quantized.rs:20-90) --------
+// ---- batch description types (src/ggml/hip_backend/ops/batch_quantized.rs:20-255) --------
 enum class QuantFormat { Q4_0, Q4_K, Q6_K, Q8_0 };
 inline float bytes_per_element(QuantFormat f)
 {
@@ -424,6 +425,55 @@ struct QuantizedMatmulOp {
     {
         return matmul_host(rfq_format_of(format), name(format), b, weights, input, n, k, output);
     }
+};
+
+// BatchMatmulResult, BatchQuantizedMatmul (src/ggml/hip_backend/ops/batch_quantized.rs:92-255): a list of
+// quantised matmuls that share one input vector, run one after the other, each into an output it allocates.
+struct BatchMatmulResult {
+    std::vector<HipBuffer> outputs;
+    std::vector<float> timings_ms;
+    float total_time_ms = 0.0f;
+};
+class BatchQuantizedMatmul {
+public:
+    explicit BatchQuantizedMatmul(HipBackend backend) : backend_(backend) {}
+    BatchQuantizedMatmul with_profiling() const { BatchQuantizedMatmul b = *this; b.enable_profiling_ = true; return b; }
+    BatchQuantizedMatmul with_async() const { BatchQuantizedMatmul b = *this; b.enable_async_ = true; return b; }
+    // process_batch (:139-160)
+    Result<std::vector<HipBuffer>> process_batch(const HipBuffer &input, const std::vector<QuantizedMatmulOp> &ops) const
+    {
+        std::vector<HipBuffer> results;
+        results.reserve(ops.size());
+        for (const QuantizedMatmulOp &op : ops) {
+            auto out = HipBuffer::create(op.m * op.n * sizeof(float));
+            if (!out.ok) return Result<std::vector<HipBuffer>>::Err(out.error);
+            Status st = op.execute(backend_, input, out.value);
+            if (!st.ok) return Result<std::vector<HipBuffer>>::Err(std::string(name(op.format)) + " matmul failed: " + st.error);
+            results.push_back(out.value);
+        }
+        return Result<std::vector<HipBuffer>>::Ok(std::move(results));
+    }
+    // process_batch_profiled (:166-190): host wall-clock per operation (each operation synchronises)
+    Result<BatchMatmulResult> process_batch_profiled(const HipBuffer &input, const std::vector<QuantizedMatmulOp> &ops) const
+    {
+        BatchMatmulResult res;
+        const auto start = std::chrono::steady_clock::now();
+        for (const QuantizedMatmulOp &op : ops) {
+            auto out = HipBuffer::create(op.m * op.n * sizeof(float));
+            if (!out.ok) return Result<BatchMatmulResult>::Err(out.error);
+            const auto t0 = std::chrono::steady_clock::now();
+            Status st = op.execute(backend_, input, out.value);
+            if (!st.ok) return Result<BatchMatmulResult>::Err(std::string(name(op.format)) + " matmul failed: " + st.error);
+            res.timings_ms.push_back(std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - t0).count());
+            res.outputs.push_back(out.value);
+        }
+        res.total_time_ms = std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - start).count();
+        return Result<BatchMatmulResult>::Ok(std::move(res));
+    }
+
+private:
+    HipBackend backend_;
+    bool enable_profiling_ = false, enable_async_ = false;
 };
 
 // The shape checks of execute_matmul_q4_0 / q8_0 (src/ggml/hip_backend/op_dispatch.rs:951-1083):

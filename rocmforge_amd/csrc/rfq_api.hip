@@ -166,8 +166,12 @@ int rfq_gemv(int fmt, const void *d_w, size_t w_bytes, const float *d_x, float *
 {
     int rc = check_gemv("rfq_gemv", fmt, d_w, w_bytes, true, d_x, d_y, m, n, k);
     if (rc != RFQ_OK) return rc;
-    if (m > 8) return fail(RFQ_E_UNSUPPORTED, "rfq_gemv: m=%d > 8; use rfq_gemm_f16 for prefill", m);
-    return launch_gemv(fmt, (const uint8_t *)d_w, d_x, d_y, m, n, k, (hipStream_t)stream);
+    for (int r0 = 0; r0 < m; r0 += 8) {                 // the decode kernels take up to eight rows of x per launch
+        const int rows = m - r0 < 8 ? m - r0 : 8;
+        rc = launch_gemv(fmt, (const uint8_t *)d_w, d_x + (size_t)r0 * k, d_y + (size_t)r0 * n, rows, n, k, (hipStream_t)stream);
+        if (rc != RFQ_OK) return rc;
+    }
+    return RFQ_OK;
 }
 
 static int matmul_raw(const char *who, int fmt, const float *d_act, const uint8_t *d_w, float *d_out, int m, int n,

@@ -424,6 +424,37 @@ static void test_execute_matmul_quantized_ops()
     }
 }
 
+// batch_quantized.rs:139-190: ops sharing one input, one output buffer each
+static void test_batch_quantized_matmul()
+{
+    auto be = HipBackend::create();
+    EXPECT(be.ok);
+    const size_t k = 256;
+    std::vector<float> x(k, 1.0f);
+    auto xb = HipBuffer::create(k * 4);
+    EXPECT(xb.ok && xb.value.copy_from_host(x).ok);
+    std::vector<QuantizedMatmulOp> ops;
+    for (size_t n : {4u, 9u}) {                      // Q4_0 rows of scale (r + 1), nibbles 9: row sum = 256 * (r + 1)
+        bytes w(n * (k / 32) * 20);
+        for (size_t r = 0; r < n; r++)
+            for (size_t blk = 0; blk < k / 32; blk++) {
+                put_f32(w, (r * (k / 32) + blk) * 20, (float)(r + 1));
+                std::memset(w.data() + (r * (k / 32) + blk) * 20 + 4, 0x99, 16);
+            }
+        ops.emplace_back(w, n, k, QuantFormat::Q4_0);
+    }
+    BatchQuantizedMatmul batch(be.value);
+    auto res = batch.process_batch(xb.value, ops);
+    EXPECT(res.ok && res.value.size() == 2);
+    for (size_t i = 0; res.ok && i < 2; i++) {
+        std::vector<float> got(ops[i].n);
+        EXPECT(res.value[i].copy_to_host(got).ok);
+        for (size_t r = 0; r < ops[i].n; r++) EXPECT(got[r] == 256.0f * (float)(r + 1));
+    }
+    auto prof = batch.with_profiling().process_batch_profiled(xb.value, ops);
+    EXPECT(prof.ok && prof.value.outputs.size() == 2 && prof.value.timings_ms.size() == 2 && prof.value.total_time_ms > 0.0f);
+}
+
 int main()
 {
     struct T { const char *name; std::function<void()> fn; };
@@ -445,6 +476,7 @@ int main()
         {"test_get_rows_f32_and_packed_tables", test_get_rows_f32_and_packed_tables},
         {"test_norm_swiglu_and_mlp", test_norm_swiglu_and_mlp},
         {"test_execute_matmul_quantized_ops", test_execute_matmul_quantized_ops},
+        {"test_batch_quantized_matmul", test_batch_quantized_matmul},
     };
     for (const T &t : tests) {
         int before = failures;

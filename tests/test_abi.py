@@ -53,7 +53,8 @@ def test_validation_needs_no_device():
     assert L.rfq_gemv(12, one, 1024, one, one, 1, 4, 128, None) == _lib.E_SIZE  # k % 256
     assert L.rfq_gemv(2, one, 81, one, one, 1, 4, 32, None) == _lib.E_SIZE     # byte count
     assert b"needs 80" in L.rfq_last_error()
-    assert L.rfq_gemv(2, one, 80, one, one, 9, 4, 32, None) == _lib.E_UNSUPPORTED
+    assert L.rfq_matmul_q4_0(one, one, one, 9, 4, 32, None) == _lib.E_UNSUPPORTED   # the raw launch takes m <= 8
+    assert L.rfq_mlp_swiglu(2, one, one, 80, 2, one, 80, one, None, 0.0, one, 9, 32, 4, one, 1 << 20, None) == _lib.E_SIZE
     assert L.rfq_matmul_q4_0(one, one, one, 1, 0, 32, None) == _lib.E_BADARG
     assert L.rfq_matmul_host_weights(2, one, 80, one, 0, 32, one, None) == _lib.E_BADARG
     assert L.rfq_gemm_f16(12, one, 256, one, one, 2, 1, 1, 256, None) == _lib.E_BADARG  # bf16 out

@@ -134,3 +134,13 @@ def test_reference_signatures(oracle, cuda):
     # the all-0x88 Q4_0 weights of tests/q_dequant_tests.rs:396-489 give exactly zero
     w = np.zeros((n * k // 32, 20), np.uint8); w[:, 0:4] = np.frombuffer(np.float32(1.0).tobytes(), np.uint8); w[:, 4:] = 0x88
     assert np.all(np.abs(gpu_gemv(Q.Q4_0, w.ravel(), x, n, k, cuda)) < 1e-4)
+
+
+def test_gemv_more_than_eight_rows(oracle, cuda):
+    # eight rows of x per launch, any m
+    fmt, n, k, m = Q.Q4_K, 130, 2048, 19
+    w = Q.make_weights(fmt, n, k, seed=9100)
+    x = x_for(m, k, 9101)
+    got = gpu_gemv(fmt, w, x, n, k, cuda)
+    assert got.shape == (m, n)
+    assert_close(got, oracle.qmatmul_nk(fmt, w, x, m, n, k), "m=19")

@@ -30,5 +30,6 @@ def test_mirror_header_names_the_reference_surface():
                  "dequantize_q4_0_kernel_cached", "dequantize_q4_k_gpu_kernel", "dequantize_q6_k_gpu_kernel",
                  "QuantFormat", "QuantizedMatmulOp", "validate_matmul_q4_0", "validate_matmul_q8_0", "get_rows",
                  "validate_token_ids", "rms_norm_gpu_kernel", "swiglu_gpu_kernel", "fused_q4_0_rmsnorm", "DeviceTensor",
-                 "mlp_swiglu", "execute_matmul_quantized", "MatMulQ4_K", "MatMulMxfp4"):
+                 "mlp_swiglu", "execute_matmul_quantized", "MatMulQ4_K", "MatMulMxfp4", "BatchQuantizedMatmul",
+                 "BatchMatmulResult"):
         assert name in text, name
