@@ -141,14 +141,17 @@ __device__ __forceinline__ float clampf(float v, float lo, float hi) { return fm
 
 // get_scale_min_k4 of ggml-quants.c: 6-bit scale (low 8 bits of the result) and
 // min (bits 8..15) number j of the 8 packed into 12 bytes, given as 3 dwords.
+// Worked out for the pair (2c, 2c+1), c = j >> 1, as two bytes at a time, so that
+// the two sub-blocks of a 64-element chunk share everything but the last shift.
 __device__ __forceinline__ uint32_t gguf_scale_min_k4(int j, uint32_t s0, uint32_t s1, uint32_t s2)
 {
-    // bytes 0-3 = s0, 4-7 = s1, 8-11 = s2
-    const int sh = 8 * (j & 3);
-    const uint32_t a = (s0 >> sh) & 255u, b = (s1 >> sh) & 255u, c = (s2 >> sh) & 255u;
-    const uint32_t sc = j < 4 ? (a & 63u) : ((c & 15u) | ((a >> 6) << 4));
-    const uint32_t mn = j < 4 ? (b & 63u) : ((c >> 4) | ((b >> 6) << 4));
-    return sc | (mn << 8);
+    const int c = j >> 1, sh = 16 * (c & 1);
+    const uint32_t a = (s0 >> sh) & 0xFFFFu, b = (s1 >> sh) & 0xFFFFu, cc = (s2 >> sh) & 0xFFFFu;
+    // j < 4: sc = a & 63, m = b & 63;  j >= 4: sc = (cc & 15) | ((a >> 6) << 4), m = (cc >> 4) | ((b >> 6) << 4)
+    const uint32_t sc2 = c < 2 ? (a & 0x3F3Fu) : ((cc & 0x0F0Fu) | ((a >> 2) & 0x3030u));
+    const uint32_t mn2 = c < 2 ? (b & 0x3F3Fu) : (((cc >> 4) & 0x0F0Fu) | ((b >> 2) & 0x3030u));
+    const int hs = 8 * (j & 1);
+    return ((sc2 >> hs) & 255u) | (((mn2 >> hs) & 255u) << 8);
 }
 
 // Signed 6-bit field (two's complement) starting at bit `off` of w.

@@ -723,6 +723,7 @@ __device__ __forceinline__ float nib_idot(const U4 &q, const XPrep &xp)
 template <int FMT> struct IUnit;
 
 template <> struct IUnit<RFQ_Q4_K> : Unit<RFQ_Q4_K> {
+    static constexpr bool PAIR = false;
     static constexpr bool NIBBLE = true;
     static constexpr uint32_t TOPOFF = 0;
     __device__ __forceinline__ float idot(const XPrep &xp) const
@@ -732,6 +733,7 @@ template <> struct IUnit<RFQ_Q4_K> : Unit<RFQ_Q4_K> {
 };
 
 template <> struct IUnit<RFQ_Q4_0> : Unit<RFQ_Q4_0> {
+    static constexpr bool PAIR = false;
     static constexpr bool NIBBLE = true;
     static constexpr uint32_t TOPOFF = 0;
     __device__ __forceinline__ float idot(const XPrep &xp) const
@@ -741,6 +743,7 @@ template <> struct IUnit<RFQ_Q4_0> : Unit<RFQ_Q4_0> {
 };
 
 template <> struct IUnit<RFQ_Q8_0> : Unit<RFQ_Q8_0> {
+    static constexpr bool PAIR = false;
     static constexpr bool NIBBLE = false;
     static constexpr uint32_t TOPOFF = 0x400000u; // weight bytes reach 255: keep every limb unsigned
     __device__ __forceinline__ float idot(const XPrep &xp) const
@@ -764,6 +767,7 @@ template <> struct IUnit<RFQ_Q8_0> : Unit<RFQ_Q8_0> {
 // GGUF layouts: x limbs in plain order (group g = elements 4g .. 4g+3).
 
 template <> struct IUnit<RFQ_GGUF_Q4_0> : Unit<RFQ_GGUF_Q4_0> {
+    static constexpr bool PAIR = false;
     static constexpr bool NIBBLE = false;
     static constexpr uint32_t TOPOFF = 0;
     // low nibbles of dword w are elements 4w .. 4w+3 (group w), high nibbles elements 16+4w .. (group 4+w)
@@ -788,6 +792,7 @@ template <> struct IUnit<RFQ_GGUF_Q4_0> : Unit<RFQ_GGUF_Q4_0> {
 };
 
 template <> struct IUnit<RFQ_GGUF_Q8_0> : Unit<RFQ_GGUF_Q8_0> {
+    static constexpr bool PAIR = false;
     static constexpr bool NIBBLE = false;
     static constexpr uint32_t TOPOFF = 0x400000u; // offset-binary weight bytes reach 255: keep every limb unsigned
     __device__ __forceinline__ float idot(const XPrep &xp) const
@@ -812,6 +817,7 @@ template <> struct IUnit<RFQ_GGUF_Q8_0> : Unit<RFQ_GGUF_Q8_0> {
 template <> struct IUnit<RFQ_GGUF_Q4_K> : Unit<RFQ_GGUF_Q4_K> {
     static constexpr bool NIBBLE = false;
     static constexpr uint32_t TOPOFF = 0;
+    static constexpr bool PAIR = true;            // units 2p and 2p+1 read the same bytes: give both to one lane
     // byte l of the chunk holds element l of this unit in its low (even unit) or high (odd unit) nibble
     __device__ __forceinline__ float idot(const XPrep &xp) const
     {
@@ -862,11 +868,20 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
 
     bool live[UPL];
     int unit[UPL];
+    if constexpr (IU::PAIR && UPL == 2) {
+        // lane p owns units 2p and 2p+1 (the unit count of such a format is even: both live or both past the end)
+        const bool in = 2 * tl < ku;
+        const int p = in ? tl : (ku >> 1) - 1;
+        live[0] = live[1] = in;
+        unit[0] = 2 * p;
+        unit[1] = 2 * p + 1;
+    } else {
 #pragma unroll
-    for (int j = 0; j < UPL; j++) {
-        int u = tl + j * TL;
-        live[j] = u < ku;
-        unit[j] = live[j] ? u : ku - 1;
+        for (int j = 0; j < UPL; j++) {
+            int u = tl + j * TL;
+            live[j] = u < ku;
+            unit[j] = live[j] ? u : ku - 1;
+        }
     }
     const int rows_per_team = groups * R;
     const int row0 = (blockIdx.x * TEAMS + team) * rows_per_team;
@@ -888,8 +903,14 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
         int r = row0 + i;
         if (r > row_last) r = row_last;
         const uint8_t *row = fused_row<FUSE>(w, f, r, rb);
+        if constexpr (IU::PAIR && UPL == 2) {
+            buf[slot][0].load(row, unit[0]);          // one fetch serves both units of the pair
+            buf[slot][1] = buf[slot][0];
+            buf[slot][1].sub |= 1;
+        } else {
 #pragma unroll
-        for (int j = 0; j < UPL; j++) buf[slot][j].load(row, unit[j]);
+            for (int j = 0; j < UPL; j++) buf[slot][j].load(row, unit[j]);
+        }
     };
 #pragma unroll
     for (int d = 0; d < D; d++) load_row(d, d);

@@ -21,7 +21,8 @@ sys.path.insert(0, ROOT)
 import oracle  # noqa: E402
 from rocmforge_amd import quantize as Q  # noqa: E402
 
-FORMATS = [Q.Q4_0, Q.Q8_0, Q.Q4_K, Q.Q6_K, Q.MXFP4, Q.MXFP6_E2M3]
+FORMATS = [Q.Q4_0, Q.Q8_0, Q.Q4_K, Q.Q6_K, Q.MXFP4, Q.MXFP6_E2M3,
+           Q.GGUF_Q4_0, Q.GGUF_Q8_0, Q.GGUF_Q4_K, Q.GGUF_Q6_K]   # (GGUF layouts: ggml's arithmetic, not the reference's)
 
 
 def main():
@@ -39,6 +40,22 @@ def main():
             out[f"{name}.{tag}.dequant"] = oracle.dequantize(fmt, blob, n * k)
             out[f"{name}.{tag}.gemv"] = oracle.qmatmul_nk(fmt, blob, x, m, n, k)
         out[f"{name}.x"] = x
+    # the neighbours of the matmul: RMSNorm, SwiGLU, and the MLP over quantised weights (hidden 768, intermediate 256: the one-launch gate/up kernel applies)
+    hidden, inter = 768, 256
+    xm = rng.standard_normal((m, hidden), dtype=np.float32)
+    nw = (1.0 + 0.1 * rng.standard_normal(hidden, dtype=np.float32)).astype(np.float32)
+    g = rng.standard_normal((m, inter), dtype=np.float32) * np.float32(2.0)
+    u = rng.standard_normal((m, inter), dtype=np.float32) * np.float32(3.0)
+    out["mlp.x"], out["mlp.norm_weight"], out["swiglu.gate"], out["swiglu.up"] = xm, nw, g, u
+    out["rms_norm.out"] = oracle.rms_norm(xm, nw, 1e-5)
+    out["swiglu.out"] = oracle.swiglu(g, u)
+    for fmt in (Q.Q4_0, Q.GGUF_Q4_K):
+        name = Q.NAMES[fmt]
+        wg = Q.make_weights(fmt, inter, hidden, seed=20260200 + fmt)
+        wu = Q.make_weights(fmt, inter, hidden, seed=20260210 + fmt)
+        wd = Q.make_weights(fmt, hidden, inter, seed=20260220 + fmt)
+        out[f"mlp.{name}.gate"], out[f"mlp.{name}.up"], out[f"mlp.{name}.down"] = wg, wu, wd
+        out[f"mlp.{name}.out"] = oracle.mlp_swiglu_q(fmt, wg, wu, fmt, wd, xm, nw, 1e-5, m, hidden, inter)
     np.savez_compressed(os.path.join(os.path.dirname(os.path.abspath(__file__)), "vectors.npz"), **out)
     print("wrote", len(out), "arrays")
 
