@@ -90,6 +90,8 @@ def run(torch):
     res = {}
     res["Q4_K gemm 512x4096x14336 fp16"] = kq_gemm(torch, Q.Q4_K)
     res["Q6_K gemm 512x4096x14336 fp16"] = kq_gemm(torch, Q.Q6_K)
+    res["GGUF_Q4_K gemm 512x4096x14336 fp16"] = kq_gemm(torch, Q.GGUF_Q4_K)
+    res["GGUF_Q6_K gemm 512x4096x14336 fp16"] = kq_gemm(torch, Q.GGUF_Q6_K)
     res["MXFP4 gemm 2048x8192x28672 bf16"] = mx_gemm(torch, Q.MXFP4)
     res["MXFP6-weight gemm 2048x8192x28672 bf16"] = mx_gemm(torch, Q.MXFP6_E2M3)
     return res
@@ -100,13 +102,13 @@ if __name__ == "__main__":
     import os
     sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
     ap = argparse.ArgumentParser()
-    ap.add_argument("--only", choices=["mxfp4", "mxfp6", "q4_k"], help="one configuration (for profiling runs)")
+    ap.add_argument("--only", choices=["mxfp4", "mxfp6", "q4_k", "gguf_q4_k"], help="one configuration (for profiling runs)")
     ap.add_argument("--steps", type=int, default=50)
     a = ap.parse_args()
     import torch
     from rocmforge_amd import quantize as Q
-    if a.only == "q4_k":
-        print(json.dumps(kq_gemm(torch, Q.Q4_K, steps=a.steps)))
+    if a.only in ("q4_k", "gguf_q4_k"):
+        print(json.dumps(kq_gemm(torch, Q.Q4_K if a.only == "q4_k" else Q.GGUF_Q4_K, steps=a.steps)))
     elif a.only:
         print(json.dumps(mx_gemm(torch, Q.MXFP4 if a.only == "mxfp4" else Q.MXFP6_E2M3, steps=a.steps)))
     else:

@@ -54,7 +54,7 @@ typedef enum rfq_format {
      * src/loader/gguf_tensor.rs:41-60) -- so there is no reference arithmetic to
      * match: results follow ggml's dequantize_row_* (ggml-quants.c).  Accepted by
      * rfq_dequant*, rfq_get_rows, rfq_dequant_rms_norm, rfq_gemv, rfq_matmul_host_weights,
-     * rfq_rms_norm_gemv and rfq_mlp_swiglu; rfq_gemm_f16 returns RFQ_E_UNSUPPORTED. */
+     * rfq_rms_norm_gemv, rfq_mlp_swiglu and rfq_gemm_f16. */
     RFQ_GGUF_Q4_0 = 102, /* 18 B / 32: f16 d, 16 bytes (low nibbles = elements 0-15, high = 16-31); d*(q-8) */
     RFQ_GGUF_Q8_0 = 108, /* 34 B / 32: f16 d, 32 int8; d*q                                                 */
     RFQ_GGUF_Q4_K = 112, /* 144 B / 256: f16 d, dmin, 12 B of 6-bit scales/mins, 128 nibble bytes          */
@@ -228,8 +228,9 @@ RFQ_API int rfq_mlp_swiglu(int fmt_gate_up, const void *d_gate_w, const void *d_
 
 /* d_out[m, n] = d_a[m, k] (fp16) . dequant(W)[n, k]^T on the fp16 matrix
  * cores with fp32 accumulation; out_dtype is RFQ_F32 or RFQ_F16.  Formats:
- * Q4_0, Q8_0, Q4_K, Q6_K.  k a multiple of 256 for the K-formats, of 32
- * otherwise; d_a_f16 16-byte aligned, d_w 4-byte aligned.  Up to 64 MiB of
+ * Q4_0, Q8_0, Q4_K, Q6_K and the four GGUF file layouts (weights decoded to
+ * f32 as the format defines and rounded once to fp16).  k a multiple of 256
+ * for the K-formats, of 32 otherwise; d_a_f16 16-byte aligned, d_w 4-byte aligned.  Up to 64 MiB of
  * temporary device memory (the activations in matrix-operand order) is kept
  * per stream between calls; larger temporaries are allocated and released in
  * stream order.  (A stream's first call, or a larger shape than before,

@@ -256,6 +256,178 @@ template <> struct Raw32<RFQ_Q6_K> {
     }
 };
 
+// ---- the block layouts of GGUF model files (ggml-common.h, ggml-quants.c) --------
+// Blocks are 2-byte aligned only: the loads below land on any byte address.
+// Each format decodes with the generic step (f32 value, one rounding to fp16).
+
+// block_q4_0: f16 d, 16 bytes; low nibbles = elements 0..15, high = 16..31; d * (q - 8)
+template <> struct Raw32<RFQ_GGUF_Q4_0> {
+    static constexpr bool TRIP_HEADER = false;
+    static constexpr int ND = 5;
+    uint32_t d[ND];
+    __device__ __forceinline__ void load(Rsrc w, uint32_t row_off, int st, int wh)
+    {
+        const uint32_t v = row_off + 18u * wh;
+        d[0] = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(w, v, st * 36, 0);
+        v4u q = __builtin_amdgcn_raw_buffer_load_b128(w, v + 2, st * 36, 0);
+        d[1] = q[0]; d[2] = q[1]; d[3] = q[2]; d[4] = q[3];
+    }
+    __device__ __forceinline__ void zero() { d[0] = 0; d[1] = d[2] = d[3] = d[4] = 0x88888888u; }
+    // d[0] becomes the f32 scale
+    __device__ __forceinline__ void settle(int, uint32_t) { d[0] = __float_as_uint(f16_bits_to_f32((uint16_t)d[0])); }
+    __device__ __forceinline__ float value(int e) const
+    {
+        uint32_t q = (d[1 + ((e & 15) >> 2)] >> (8 * (e & 3) + 4 * (e >> 4))) & 15u;
+        return (float)((int)q - 8) * __uint_as_float(d[0]);
+    }
+    __device__ __forceinline__ void step(int T, v8h (&h)[4], v2h (&)[4]) const
+    {
+        const int c = T / 3, e0 = 3 * (T % 3), e1 = e0 + 3 < 8 ? e0 + 3 : 8;
+#pragma unroll
+        for (int e = e0; e < e1; e++) h[c][chunk_pos(e)] = (_Float16)value(8 * c + e);
+    }
+};
+
+// block_q8_0: f16 d, 32 int8; d * q
+template <> struct Raw32<RFQ_GGUF_Q8_0> {
+    static constexpr bool TRIP_HEADER = false;
+    static constexpr int ND = 9;
+    uint32_t d[ND];
+    __device__ __forceinline__ void load(Rsrc w, uint32_t row_off, int st, int wh)
+    {
+        const uint32_t v = row_off + 34u * wh;
+        d[0] = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(w, v, st * 68, 0);
+        v4u q0 = __builtin_amdgcn_raw_buffer_load_b128(w, v + 2, st * 68, 0);
+        v4u q1 = __builtin_amdgcn_raw_buffer_load_b128(w, v + 18, st * 68, 0);
+        d[1] = q0[0]; d[2] = q0[1]; d[3] = q0[2]; d[4] = q0[3];
+        d[5] = q1[0]; d[6] = q1[1]; d[7] = q1[2]; d[8] = q1[3];
+    }
+    __device__ __forceinline__ void zero()
+    {
+#pragma unroll
+        for (int i = 0; i < ND; i++) d[i] = 0;
+    }
+    __device__ __forceinline__ void settle(int, uint32_t) { d[0] = __float_as_uint(f16_bits_to_f32((uint16_t)d[0])); }
+    __device__ __forceinline__ float value(int e) const
+    {
+        const int b = (int)(int8_t)((d[1 + (e >> 2)] >> (8 * (e & 3))) & 255u);
+        return (float)b * __uint_as_float(d[0]);
+    }
+    __device__ __forceinline__ void step(int T, v8h (&h)[4], v2h (&)[4]) const
+    {
+        const int c = T / 3, e0 = 3 * (T % 3), e1 = e0 + 3 < 8 ? e0 + 3 : 8;
+#pragma unroll
+        for (int e = e0; e < e1; e++) h[c][chunk_pos(e)] = (_Float16)value(8 * c + e);
+    }
+};
+
+// block_q4_K (144 bytes): f16 d, f16 dmin, 12 bytes of 6-bit scales and mins, 128
+// nibble bytes.  Sub-block sb = 32 elements: chunk sb >> 1 of 32 bytes, low
+// (even sb) or high (odd sb) nibbles; value = (d * sc) * q - dmin * m.  The two
+// threads of a row read the same 32 bytes of a stage and take a nibble half each.
+// Unlike the 256-byte layout's integer mins, d * sc * q and dmin * m have the
+// same magnitude here (a real min/max quantisation), so the rounded fp16 value
+// of the whole expression carries the usual 2^-12 relative error.
+template <> struct Raw32<RFQ_GGUF_Q4_K> {
+    static constexpr bool TRIP_HEADER = false;
+    static constexpr int ND = 12;
+    uint32_t d[ND];
+    int sub;
+    __device__ __forceinline__ void load(Rsrc w, uint32_t row_off, int st, int wh)
+    {
+        const int blk = (st >> 2) * 144;
+        sub = ((st & 3) << 1) | wh;
+        v4u h = __builtin_amdgcn_raw_buffer_load_b128(w, row_off, blk, 0);
+        v4u q0 = __builtin_amdgcn_raw_buffer_load_b128(w, row_off + 16, blk + 32 * (st & 3), 0);
+        v4u q1 = __builtin_amdgcn_raw_buffer_load_b128(w, row_off + 32, blk + 32 * (st & 3), 0);
+        d[0] = h[0]; d[1] = h[1]; d[2] = h[2]; d[3] = h[3];
+        d[4] = q0[0]; d[5] = q0[1]; d[6] = q0[2]; d[7] = q0[3];
+        d[8] = q1[0]; d[9] = q1[1]; d[10] = q1[2]; d[11] = q1[3];
+    }
+    __device__ __forceinline__ void zero()
+    {
+#pragma unroll
+        for (int i = 0; i < ND; i++) d[i] = 0;
+        sub = 0;
+    }
+    // d[0] = d * sc, d[1] = dmin * m (f32); the nibbles of this half become bytes
+    __device__ __forceinline__ void settle(int, uint32_t)
+    {
+        const uint32_t sm = gguf_scale_min_k4(sub, d[1], d[2], d[3]);
+        const float d1 = f16_bits_to_f32((uint16_t)(d[0] & 0xFFFFu)) * (float)(sm & 255u);
+        const float m1 = f16_bits_to_f32((uint16_t)(d[0] >> 16)) * (float)(sm >> 8);
+        d[0] = __float_as_uint(d1);
+        d[1] = __float_as_uint(m1);
+        const int sh = 4 * (sub & 1);
+#pragma unroll
+        for (int i = 4; i < ND; i++) d[i] = (d[i] >> sh) & 0x0F0F0F0Fu;
+    }
+    __device__ __forceinline__ float value(int e) const
+    {
+        const uint32_t q = (d[4 + (e >> 2)] >> (8 * (e & 3))) & 255u;
+        return __uint_as_float(d[0]) * (float)q - __uint_as_float(d[1]);
+    }
+    __device__ __forceinline__ void step(int T, v8h (&h)[4], v2h (&)[4]) const
+    {
+        const int c = T / 3, e0 = 3 * (T % 3), e1 = e0 + 3 < 8 ? e0 + 3 : 8;
+#pragma unroll
+        for (int e = e0; e < e1; e++) h[c][chunk_pos(e)] = (_Float16)value(8 * c + e);
+    }
+};
+
+// block_q6_K (210 bytes): ql[128], qh[64], i8 scales[16], f16 d.  Sub-block sb =
+// 32 elements: half n = sb >> 2 of 128 elements, quarter t = sb & 3: low nibbles
+// from ql[64 n + 32 (t & 1) + l] (>> 4 for t >= 2), bits 4-5 from qh[32 n + l] >> 2 t,
+// scales sc[8 n + 2 t + l / 16]; value = (d * sc) * (q - 32).
+template <> struct Raw32<RFQ_GGUF_Q6_K> {
+    static constexpr bool TRIP_HEADER = false;
+    static constexpr int ND = 17;
+    uint32_t d[ND];
+    int sub;
+    __device__ __forceinline__ void load(Rsrc w, uint32_t row_off, int st, int wh)
+    {
+        const int blk = (st >> 2) * 210, half = (st & 3) >> 1, odd = st & 1;
+        sub = ((st & 3) << 1) | wh;
+        const uint32_t vq = row_off + 32u * wh;
+        v4u l0 = __builtin_amdgcn_raw_buffer_load_b128(w, vq, blk + 64 * half, 0);
+        v4u l1 = __builtin_amdgcn_raw_buffer_load_b128(w, vq + 16, blk + 64 * half, 0);
+        v4u h0 = __builtin_amdgcn_raw_buffer_load_b128(w, row_off, blk + 128 + 32 * half, 0);
+        v4u h1 = __builtin_amdgcn_raw_buffer_load_b128(w, row_off + 16, blk + 128 + 32 * half, 0);
+        const uint32_t sc = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(w, row_off + 2u * wh, blk + 192 + 8 * half + 4 * odd, 0);
+        const uint32_t dd = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(w, row_off, blk + 208, 0);
+        d[0] = l0[0]; d[1] = l0[1]; d[2] = l0[2]; d[3] = l0[3]; d[4] = l1[0]; d[5] = l1[1]; d[6] = l1[2]; d[7] = l1[3];
+        d[8] = h0[0]; d[9] = h0[1]; d[10] = h0[2]; d[11] = h0[3]; d[12] = h1[0]; d[13] = h1[1]; d[14] = h1[2]; d[15] = h1[3];
+        d[16] = sc | (dd << 16);
+    }
+    __device__ __forceinline__ void zero()
+    {
+#pragma unroll
+        for (int i = 0; i < ND; i++) d[i] = 0;
+        sub = 0;
+    }
+    // d[0..7] = the 6-bit codes as bytes, d[8] / d[9] = d * sc of the two 16-element halves (f32)
+    __device__ __forceinline__ void settle(int, uint32_t)
+    {
+        const int t = sub & 3, shl = 4 * (t >> 1), shh = 2 * t;
+#pragma unroll
+        for (int i = 0; i < 8; i++) d[i] = ((d[i] >> shl) & 0x0F0F0F0Fu) | (((d[8 + i] >> shh) & 0x03030303u) << 4);
+        const float dv = f16_bits_to_f32((uint16_t)(d[16] >> 16));
+        d[8] = __float_as_uint(dv * (float)(int)(int8_t)(d[16] & 255u));
+        d[9] = __float_as_uint(dv * (float)(int)(int8_t)((d[16] >> 8) & 255u));
+    }
+    __device__ __forceinline__ float value(int e) const
+    {
+        const uint32_t q = (d[e >> 2] >> (8 * (e & 3))) & 255u;
+        return __uint_as_float(d[8 + (e >> 4)]) * (float)((int)q - 32);
+    }
+    __device__ __forceinline__ void step(int T, v8h (&h)[4], v2h (&)[4]) const
+    {
+        const int c = T / 3, e0 = 3 * (T % 3), e1 = e0 + 3 < 8 ? e0 + 3 : 8;
+#pragma unroll
+        for (int e = e0; e < e1; e++) h[c][chunk_pos(e)] = (_Float16)value(8 * c + e);
+    }
+};
+
 // Activations in the order the matrix instruction reads them.  Unit (mt, st)
 // = 32 rows x 64 k; inside it chunk c (0..3) of lane (fr, fh) holds
 // A[32*mt + fr][64*st + 32*fh + 8*c .. +8] in the order of chunk_pos():
@@ -863,6 +1035,10 @@ int launch_gemm_f16(int fmt, const uint8_t *d_w, const void *d_a, void *d_out, i
     case RFQ_Q8_0: return launch_fmt<RFQ_Q8_0>(d_w, d_a, d_out, out_dtype, m, n, k, s);
     case RFQ_Q4_K: return launch_fmt<RFQ_Q4_K>(d_w, d_a, d_out, out_dtype, m, n, k, s);
     case RFQ_Q6_K: return launch_fmt<RFQ_Q6_K>(d_w, d_a, d_out, out_dtype, m, n, k, s);
+    case RFQ_GGUF_Q4_0: return launch_fmt<RFQ_GGUF_Q4_0>(d_w, d_a, d_out, out_dtype, m, n, k, s);
+    case RFQ_GGUF_Q8_0: return launch_fmt<RFQ_GGUF_Q8_0>(d_w, d_a, d_out, out_dtype, m, n, k, s);
+    case RFQ_GGUF_Q4_K: return launch_fmt<RFQ_GGUF_Q4_K>(d_w, d_a, d_out, out_dtype, m, n, k, s);
+    case RFQ_GGUF_Q6_K: return launch_fmt<RFQ_GGUF_Q6_K>(d_w, d_a, d_out, out_dtype, m, n, k, s);
     default: return fail(RFQ_E_UNSUPPORTED, "rfq_gemm_f16: no fp16 matrix-core kernel for format %d", fmt);
     }
 }
