@@ -118,11 +118,12 @@ template <> struct Raw32<RFQ_Q4_0> {
         d[1] = q[0]; d[2] = q[1]; d[3] = q[2]; d[4] = q[3];
     }
     __device__ __forceinline__ void zero() { d[0] = 0; d[1] = d[2] = d[3] = d[4] = 0x88888888u; } // nibble 8 is 0.0
-    __device__ __forceinline__ void settle(int, uint32_t) {}
+    __device__ __forceinline__ void settle(int, uint32_t, int) {}
     __device__ __forceinline__ float value(int e) const            // element 2i = low nibble of byte i
     {
         uint32_t q = (d[1 + (e >> 3)] >> (4 * (e & 7))) & 15u;
-        return __uint_as_float(d[0]) * (float)((int)q - 8);
+        // scale * (q - 8) as a fused multiply-add of q: 8 * scale is exact, so the one rounding is the product's
+        return __builtin_fmaf(__uint_as_float(d[0]), (float)q, -8.0f * __uint_as_float(d[0]));
     }
     __device__ __forceinline__ void step(int T, v8h (&h)[4], v2h (&)[4]) const
     {
@@ -152,11 +153,12 @@ template <> struct Raw32<RFQ_Q8_0> {
 #pragma unroll
         for (int i = 1; i < ND; i++) d[i] = 0x80808080u;
     }
-    __device__ __forceinline__ void settle(int, uint32_t) {}
+    __device__ __forceinline__ void settle(int, uint32_t, int) {}
     __device__ __forceinline__ float value(int e) const
     {
         uint32_t b = (d[1 + (e >> 2)] >> (8 * (e & 3))) & 255u;
-        return ((float)b - 128.0f) * __uint_as_float(d[0]);
+        // (b - 128) * scale as a fused multiply-add of b: 128 * scale is exact, so the one rounding is the product's
+        return __builtin_fmaf(__uint_as_float(d[0]), (float)b, -128.0f * __uint_as_float(d[0]));
     }
     __device__ __forceinline__ void step(int T, v8h (&h)[4], v2h (&)[4]) const
     {
@@ -181,7 +183,7 @@ template <> struct Raw32<RFQ_Q4_K> {
     __device__ __forceinline__ void zero() { d[0] = d[1] = d[2] = d[3] = d[4] = 0; }
     // d[0] becomes the f16 scale in both halves; `pair` is the header dword
     // that holds the scales of sub-blocks g & ~1 and g | 1.
-    __device__ __forceinline__ void settle(int g, uint32_t pair) { d[0] = ((pair >> (16 * (g & 1))) & 0xFFFFu) * 0x10001u; }
+    __device__ __forceinline__ void settle(int g, uint32_t pair, int) { d[0] = ((pair >> (16 * (g & 1))) & 0xFFFFu) * 0x10001u; }
     // q * scale only: the min is contracted separately.  The product of the
     // integer q and the f16 scale is exact in f32, so rounding it to fp16 is
     // what a single fp16 multiplication returns: two weights per instruction.
@@ -240,7 +242,7 @@ template <> struct Raw32<RFQ_Q6_K> {
 #pragma unroll
         for (int i = 0; i < ND; i++) d[i] = 0;
     }
-    __device__ __forceinline__ void settle(int, uint32_t) {}
+    __device__ __forceinline__ void settle(int, uint32_t, int) {}
     __device__ __forceinline__ float value(int e) const
     {
         const float scale = f16_bits_to_f32((uint16_t)((d[0] >> (16 * (e >> 4))) & 0xFFFFu));
@@ -274,11 +276,13 @@ template <> struct Raw32<RFQ_GGUF_Q4_0> {
     }
     __device__ __forceinline__ void zero() { d[0] = 0; d[1] = d[2] = d[3] = d[4] = 0x88888888u; }
     // d[0] becomes the f32 scale
-    __device__ __forceinline__ void settle(int, uint32_t) { d[0] = __float_as_uint(f16_bits_to_f32((uint16_t)d[0])); }
+    __device__ __forceinline__ void settle(int, uint32_t, int) { d[0] = __float_as_uint(f16_bits_to_f32((uint16_t)d[0])); }
+    // d * (q - 8) as a fused multiply-add of q (8 * d is exact: the same single rounding)
     __device__ __forceinline__ float value(int e) const
     {
         uint32_t q = (d[1 + ((e & 15) >> 2)] >> (8 * (e & 3) + 4 * (e >> 4))) & 15u;
-        return (float)((int)q - 8) * __uint_as_float(d[0]);
+        const float sc = __uint_as_float(d[0]);
+        return __builtin_fmaf(sc, (float)q, -8.0f * sc);
     }
     __device__ __forceinline__ void step(int T, v8h (&h)[4], v2h (&)[4]) const
     {
@@ -307,7 +311,7 @@ template <> struct Raw32<RFQ_GGUF_Q8_0> {
 #pragma unroll
         for (int i = 0; i < ND; i++) d[i] = 0;
     }
-    __device__ __forceinline__ void settle(int, uint32_t) { d[0] = __float_as_uint(f16_bits_to_f32((uint16_t)d[0])); }
+    __device__ __forceinline__ void settle(int, uint32_t, int) { d[0] = __float_as_uint(f16_bits_to_f32((uint16_t)d[0])); }
     __device__ __forceinline__ float value(int e) const
     {
         const int b = (int)(int8_t)((d[1 + (e >> 2)] >> (8 * (e & 3))) & 255u);
@@ -332,11 +336,9 @@ template <> struct Raw32<RFQ_GGUF_Q4_K> {
     static constexpr bool TRIP_HEADER = false;
     static constexpr int ND = 12;
     uint32_t d[ND];
-    int sub;
-    __device__ __forceinline__ void load(Rsrc w, uint32_t row_off, int st, int wh)
+    __device__ __forceinline__ void load(Rsrc w, uint32_t row_off, int st, int)
     {
         const int blk = (st >> 2) * 144;
-        sub = ((st & 3) << 1) | wh;
         v4u h = __builtin_amdgcn_raw_buffer_load_b128(w, row_off, blk, 0);
         v4u q0 = __builtin_amdgcn_raw_buffer_load_b128(w, row_off + 16, blk + 32 * (st & 3), 0);
         v4u q1 = __builtin_amdgcn_raw_buffer_load_b128(w, row_off + 32, blk + 32 * (st & 3), 0);
@@ -348,11 +350,13 @@ template <> struct Raw32<RFQ_GGUF_Q4_K> {
     {
 #pragma unroll
         for (int i = 0; i < ND; i++) d[i] = 0;
-        sub = 0;
     }
-    // d[0] = d * sc, d[1] = dmin * m (f32); the nibbles of this half become bytes
-    __device__ __forceinline__ void settle(int, uint32_t)
+    // d[0] = d * sc, d[1] = dmin * m (f32); the nibbles of this half become bytes.
+    // The stage's number c within its super-block (its 64-element chunk) is a
+    // compile-time constant where this is called, wh the thread's nibble half.
+    __device__ __forceinline__ void settle(int wh, uint32_t, int c)
     {
+        const int sub = 2 * c + wh;
         const uint32_t sm = gguf_scale_min_k4(sub, d[1], d[2], d[3]);
         const float d1 = f16_bits_to_f32((uint16_t)(d[0] & 0xFFFFu)) * (float)(sm & 255u);
         const float m1 = f16_bits_to_f32((uint16_t)(d[0] >> 16)) * (float)(sm >> 8);
@@ -383,11 +387,9 @@ template <> struct Raw32<RFQ_GGUF_Q6_K> {
     static constexpr bool TRIP_HEADER = false;
     static constexpr int ND = 17;
     uint32_t d[ND];
-    int sub;
     __device__ __forceinline__ void load(Rsrc w, uint32_t row_off, int st, int wh)
     {
         const int blk = (st >> 2) * 210, half = (st & 3) >> 1, odd = st & 1;
-        sub = ((st & 3) << 1) | wh;
         const uint32_t vq = row_off + 32u * wh;
         v4u l0 = __builtin_amdgcn_raw_buffer_load_b128(w, vq, blk + 64 * half, 0);
         v4u l1 = __builtin_amdgcn_raw_buffer_load_b128(w, vq + 16, blk + 64 * half, 0);
@@ -403,22 +405,27 @@ template <> struct Raw32<RFQ_GGUF_Q6_K> {
     {
 #pragma unroll
         for (int i = 0; i < ND; i++) d[i] = 0;
-        sub = 0;
     }
-    // d[0..7] = the 6-bit codes as bytes, d[8] / d[9] = d * sc of the two 16-element halves (f32)
-    __device__ __forceinline__ void settle(int, uint32_t)
+    // d[0..7] = the 6-bit codes as bytes, d[8] / d[9] = d * sc of the two 16-element halves (f32), d[10] / d[11] = -32 times those;
+    // c = the stage's number within its super-block (a compile-time constant at the call), wh = the thread's group
+    __device__ __forceinline__ void settle(int wh, uint32_t, int c)
     {
-        const int t = sub & 3, shl = 4 * (t >> 1), shh = 2 * t;
+        const int t = 2 * (c & 1) + wh, shl = 4 * (c & 1), shh = 2 * t;
 #pragma unroll
         for (int i = 0; i < 8; i++) d[i] = ((d[i] >> shl) & 0x0F0F0F0Fu) | (((d[8 + i] >> shh) & 0x03030303u) << 4);
         const float dv = f16_bits_to_f32((uint16_t)(d[16] >> 16));
-        d[8] = __float_as_uint(dv * (float)(int)(int8_t)(d[16] & 255u));
-        d[9] = __float_as_uint(dv * (float)(int)(int8_t)((d[16] >> 8) & 255u));
+        const float s0 = dv * (float)(int)(int8_t)(d[16] & 255u), s1 = dv * (float)(int)(int8_t)((d[16] >> 8) & 255u);
+        d[8] = __float_as_uint(s0);
+        d[9] = __float_as_uint(s1);
+        d[10] = __float_as_uint(-32.0f * s0);
+        d[11] = __float_as_uint(-32.0f * s1);
     }
+    // (d * sc) * (q - 32) as one fused multiply-add of q: 32 * (d * sc) is exact, so the
+    // single rounding of q * (d * sc) - 32 * (d * sc) is the rounding of the product.
     __device__ __forceinline__ float value(int e) const
     {
         const uint32_t q = (d[e >> 2] >> (8 * (e & 3))) & 255u;
-        return __uint_as_float(d[8 + (e >> 4)]) * (float)((int)q - 32);
+        return __builtin_fmaf(__uint_as_float(d[8 + (e >> 4)]), (float)q, __uint_as_float(d[10 + (e >> 4)]));
     }
     __device__ __forceinline__ void step(int T, v8h (&h)[4], v2h (&)[4]) const
     {
@@ -580,7 +587,7 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
         Raw32<FMT> &raw = raw_of(slotc);
         Raw32<FMT> z;
         z.zero();
-        raw.settle(wh, pair);                                     // (group 2*stage + wh has the parity of wh)
+        raw.settle(wh, pair, decltype(slotc)::value);             // (group 2*stage + wh has the parity of wh; ring slot = stage % 4)
 #pragma unroll
         for (int i = 0; i < Raw32<FMT>::ND; i++) raw.d[i] = st * 2 + wh < groups ? raw.d[i] : z.d[i];
     };
