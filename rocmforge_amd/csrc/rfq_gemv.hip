@@ -838,7 +838,43 @@ template <> struct IUnit<RFQ_GGUF_Q4_K> : Unit<RFQ_GGUF_Q4_K> {
         const float m1 = f16_bits_to_f32((uint16_t)(dd >> 16)) * (float)(sm >> 8);
         return __builtin_fmaf(d1 * xp.s, S, -m1 * xp.xsum);
     }
+    // Both units of a chunk (this one is the even one) from one fetch: low nibbles against
+    // xe, high nibbles against xo, the chunk's two scales and mins unpacked together.
+    __device__ __forceinline__ float idot_pair(const XPrep &xe, const XPrep &xo) const
+    {
+        const int c = sub >> 1, sh = 16 * (c & 1);
+        const uint32_t a = (s0 >> sh) & 0xFFFFu, b = (s1 >> sh) & 0xFFFFu, cc = (s2 >> sh) & 0xFFFFu;
+        const uint32_t sc2 = c < 2 ? (a & 0x3F3Fu) : ((cc & 0x0F0Fu) | ((a >> 2) & 0x3030u));
+        const uint32_t mn2 = c < 2 ? (b & 0x3F3Fu) : (((cc >> 4) & 0x0F0Fu) | ((b >> 2) & 0x3030u));
+        uint32_t elo = 0, emid = 0, olo = 0, omid = 0;
+        int etop = 0, otop = 0;
+#pragma unroll
+        for (int w = 0; w < 8; w++) {
+            const uint32_t lo = q.v[w] & 0x0F0F0F0Fu, hi = (q.v[w] >> 4) & 0x0F0F0F0Fu;
+            const uint32_t *E = &xe.l[w * 3], *O = &xo.l[w * 3];
+            elo = __builtin_amdgcn_udot4(lo, E[0], elo, false);
+            emid = __builtin_amdgcn_udot4(lo, E[1], emid, false);
+            etop = __builtin_amdgcn_sdot4((int)lo, (int)E[2], etop, false);
+            olo = __builtin_amdgcn_udot4(hi, O[0], olo, false);
+            omid = __builtin_amdgcn_udot4(hi, O[1], omid, false);
+            otop = __builtin_amdgcn_sdot4((int)hi, (int)O[2], otop, false);
+        }
+        const float Se = __builtin_fmaf((float)etop, 65536.0f, __builtin_fmaf((float)emid, 256.0f, (float)elo));
+        const float So = __builtin_fmaf((float)otop, 65536.0f, __builtin_fmaf((float)omid, 256.0f, (float)olo));
+        const float dv = f16_bits_to_f32((uint16_t)(dd & 0xFFFFu)), dm = f16_bits_to_f32((uint16_t)(dd >> 16));
+        const float pos = __builtin_fmaf((float)(sc2 & 255u) * xe.s, Se, (float)(sc2 >> 8) * xo.s * So);
+        const float neg = __builtin_fmaf((float)(mn2 & 255u), xe.xsum, (float)(mn2 >> 8) * xo.xsum);
+        return __builtin_fmaf(dv, pos, -dm * neg);
+    }
 };
+
+// The formats without paired units never call idot_pair.
+template <typename IU>
+__device__ __forceinline__ float idot_pair_of(const IU &u, const XPrep &xe, const XPrep &xo)
+{
+    if constexpr (IU::PAIR) return u.idot_pair(xe, xo);
+    else return 0.0f;
+}
 
 // Block = 4 wavefronts = 4 / WPR teams.  Lane `tl` of a team owns units
 // tl + j*64*WPR, j < UPL, of every row the team visits.  A team walks
@@ -905,8 +941,6 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
         const uint8_t *row = fused_row<FUSE>(w, f, r, rb);
         if constexpr (IU::PAIR && UPL == 2) {
             buf[slot][0].load(row, unit[0]);          // one fetch serves both units of the pair
-            buf[slot][1] = buf[slot][0];
-            buf[slot][1].sub |= 1;
         } else {
 #pragma unroll
             for (int j = 0; j < UPL; j++) buf[slot][j].load(row, unit[j]);
@@ -976,10 +1010,15 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
 #pragma unroll
         for (int i = 0; i < R; i++) {
             float acc = 0.f;
+            if constexpr (IU::PAIR && UPL == 2) {
+                const float t = idot_pair_of(buf[i % D][0], xp[0], xp[1]);
+                acc = live[0] ? t : 0.f;
+            } else {
 #pragma unroll
-            for (int j = 0; j < UPL; j++) {
-                float t = buf[i % D][j].idot(xp[j]);
-                acc += live[j] ? t : 0.f;
+                for (int j = 0; j < UPL; j++) {
+                    float t = buf[i % D][j].idot(xp[j]);
+                    acc += live[j] ? t : 0.f;
+                }
             }
             if (i + D < R) load_row(i % D, base + i + D);
             res[i] = wave_sum(acc);
