@@ -159,6 +159,42 @@ def time_mlp(torch, fmt, hidden, inter, Q, steps=300, warmup=60):
     return res
 
 
+def time_host_path(torch, fmt, w, x, n, k):
+    """The boundary with host-resident weights, as the reference's matmul_q4_k has it (the weights
+    cross the host link on every call): rfq_upload of the packed weights from pageable memory beside
+    the runtime's own pageable copy and a copy from pinned memory, and the whole rfq_matmul_host_weights."""
+    import ctypes as C
+    import numpy as np
+    from rocmforge_amd import _lib
+    L, dev = _lib.lib(), torch.device("cuda:0")
+    nb = int(w.size)
+    dst = torch.empty(nb, dtype=torch.uint8, device=dev)
+    pin = torch.empty(nb, dtype=torch.uint8, pin_memory=True)
+    pin.numpy()[:] = w
+    dx = torch.from_numpy(np.ascontiguousarray(x)).to(dev)
+    dy = torch.empty(n, dtype=torch.float32, device=dev)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def best(f, reps=5):
+        f()
+        torch.cuda.synchronize()
+        t = 1e9
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            f()
+            torch.cuda.synchronize()
+            t = min(t, time.perf_counter() - t0)
+        return t
+
+    t_up = best(lambda: _lib.check(L.rfq_upload(C.c_void_p(w.ctypes.data), nb, C.c_void_p(dst.data_ptr()), stream)))
+    t_page = best(lambda: dst.copy_(torch.from_numpy(w)))
+    t_pin = best(lambda: dst.copy_(pin, non_blocking=True))
+    t_mm = best(lambda: _lib.check(L.rfq_matmul_host_weights(fmt, C.c_void_p(w.ctypes.data), nb, C.c_void_p(dx.data_ptr()), n, k,
+                                                             C.c_void_p(dy.data_ptr()), stream)))
+    return {"MB": round(nb / 1e6, 1), "rfq_upload_GB/s": round(nb / t_up / 1e9, 1), "pageable_copy_GB/s": round(nb / t_page / 1e9, 1),
+            "pinned_copy_GB/s": round(nb / t_pin / 1e9, 1), "matmul_host_weights_ms": round(t_mm * 1e3, 3)}
+
+
 def cpu_baseline(fmt, w, x, n, k, budget_s=12.0):
     """The CPU oracle (dequantise everything, then the sequential fp32 matmul)
     on one host thread, repeated until ~budget_s of CPU work."""
@@ -292,6 +328,7 @@ def main():
             t, b = time_dequant(torch, f, n, k, 50, 5, Q, seed)
             also[name] = {"GB/s": round(b / t / 1e9, 1), "us": round(t * 1e6, 2), "hbm_frac": round(b / t / 1e9 / HBM_PEAK_GBS, 4),
                           "Gelem/s": round(n * k / t / 1e9, 1)}
+        also["Q4_K 14336x4096 weights from host memory"] = time_host_path(torch, fmt, w, x[0], N, K)
         try:
             import bench_gemm
             also.update(bench_gemm.run(torch))

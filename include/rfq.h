@@ -87,9 +87,23 @@ RFQ_API int rfq_version(void);
 RFQ_API const char *rfq_last_error(void);
 /* rfq_gemm_f16 and rfq_gemv (Q8_0, m > 1) keep up to 64 MiB of temporary
  * device memory per stream between calls.  This frees all of it (it waits for
- * the device first); the next call allocates again.  No counterpart in the
- * reference, whose kernels take no temporaries. */
+ * the device first), and rfq_upload's pinned staging slots; the next call
+ * allocates again.  No counterpart in the reference, whose kernels take no
+ * temporaries. */
 RFQ_API int rfq_release_temporaries(void);
+/* Host bytes (pageable: a slice of the memory-mapped model file) -> device
+ * memory, in stream order.  The bytes go through a ring of four pinned 8 MiB
+ * slots the library keeps per device: a few host threads fill a slot while the
+ * earlier slots' transfers are in flight.  On return the source may be
+ * released; the device copy completes in stream order (the call itself blocks
+ * only while it waits for a free slot).  Not for use under graph capture.
+ * Replaces the pageable hipMemcpy / hipMemcpyAsync of HipBuffer::copy_from_host
+ * (src/backend/hip_backend/memory.rs:135-170, 203-250) and
+ * AsyncLoader::upload_to_buffer / upload_to_buffer_offset
+ * (src/backend/hip_backend/async_ops.rs:66-180) as the loader uses them
+ * (src/loader/gguf/gpu_upload.rs:57-125); rfq_dequant_upload and
+ * rfq_matmul_host_weights upload through it too. */
+RFQ_API int rfq_upload(const void *h_src, size_t bytes, void *d_dst, void *stream);
 /* Elements per block / bytes per block the decoders stride by
  * (GgufTensorType::block_size, src/loader/tensor_type.rs:77-88; strides at
  * src/kernels/quant/q4_0.rs:269, q8_0.rs:33, q4_k.rs:206, q6_k.rs:206,

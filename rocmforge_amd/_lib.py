@@ -31,6 +31,7 @@ _SIGNATURES = {
     "rfq_version": ([], _i),
     "rfq_last_error": ([], C.c_char_p),
     "rfq_release_temporaries": ([], _i),
+    "rfq_upload": ([_vp, _sz, _vp, _vp], _i),
     "rfq_block_elems": ([_i], _sz),
     "rfq_block_bytes": ([_i], _sz),
     "rfq_packed_bytes": ([_i, _sz], _sz),

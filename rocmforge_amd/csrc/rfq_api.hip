@@ -79,7 +79,19 @@ int rfq_version(void) { return RFQ_VERSION; }
 
 const char *rfq_last_error(void) { return g_err; }
 
-int rfq_release_temporaries(void) { return rfq::release_workspaces(); }
+int rfq_release_temporaries(void)
+{
+    int rc = rfq::release_workspaces();
+    int rc2 = rfq::release_upload_rings();
+    return rc != RFQ_OK ? rc : rc2;
+}
+
+int rfq_upload(const void *h_src, size_t bytes, void *d_dst, void *stream)
+{
+    if (bytes == 0) return RFQ_OK;
+    if (!h_src || !d_dst) return fail(RFQ_E_BADARG, "rfq_upload: null pointer");
+    return upload_bytes(h_src, bytes, d_dst, (hipStream_t)stream);
+}
 
 size_t rfq_block_elems(int fmt) { return (size_t)fmt_block_elems(fmt); }
 size_t rfq_block_bytes(int fmt) { return (size_t)fmt_block_bytes(fmt); }
@@ -134,8 +146,7 @@ int rfq_dequant_upload(int fmt, const uint8_t *h_packed, size_t packed_bytes, fl
     void *d_in = nullptr;
     if (bytes) {
         RFQ_HIP(hipMalloc(&d_in, bytes));
-        hipError_t e = hipMemcpyAsync(d_in, h_packed, bytes, hipMemcpyHostToDevice, s);
-        if (e != hipSuccess) { (void)hipFree(d_in); return hip_fail(e, "hipMemcpyAsync(H2D)"); }
+        if (int up = upload_bytes(h_packed, bytes, d_in, s)) { (void)hipStreamSynchronize(s); (void)hipFree(d_in); return up; }
     }
     int rc = launch_dequant(fmt, (const uint8_t *)d_in, bytes, d_out, n_elems, s);
     hipError_t e = hipStreamSynchronize(s);
@@ -210,10 +221,9 @@ int rfq_matmul_host_weights(int fmt, const uint8_t *h_w, size_t w_bytes, const f
     hipStream_t s = (hipStream_t)stream;
     void *d_w = nullptr;
     RFQ_HIP(hipMalloc(&d_w, w_bytes));
-    hipError_t e = hipMemcpyAsync(d_w, h_w, w_bytes, hipMemcpyHostToDevice, s);
-    if (e != hipSuccess) { (void)hipFree(d_w); return hip_fail(e, "hipMemcpyAsync(H2D)"); }
+    if (int up = upload_bytes(h_w, w_bytes, d_w, s)) { (void)hipStreamSynchronize(s); (void)hipFree(d_w); return up; }
     rc = launch_gemv(fmt, (const uint8_t *)d_w, d_input, d_out, 1, (int)n_rows, (int)n_cols, s);
-    e = hipStreamSynchronize(s);
+    hipError_t e = hipStreamSynchronize(s);
     (void)hipFree(d_w);
     if (rc != RFQ_OK) return rc;
     if (e != hipSuccess) return hip_fail(e, "hipStreamSynchronize");

@@ -71,6 +71,9 @@ int device_cu_count();
 // stream-ordered allocation the caller releases with hipFreeAsync otherwise.
 int workspace(hipStream_t s, size_t bytes, uint8_t **out, bool *transient);
 int release_workspaces();
+// Host bytes -> device memory through the per-device ring of pinned slots (rfq_upload.hip).
+int upload_bytes(const void *h_src, size_t bytes, void *d_dst, hipStream_t s);
+int release_upload_rings();
 
 // ---- launchers implemented per .hip file -----------------------------------
 int launch_dequant(int fmt, const uint8_t *d_in, size_t in_bytes, float *d_out, size_t n, hipStream_t s);

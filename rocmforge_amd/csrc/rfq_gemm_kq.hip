@@ -107,7 +107,6 @@ __device__ __forceinline__ constexpr int chunk_pos(int e) { return ((e & 3) << 1
 
 // src/kernels/quant/q4_0.rs:289-306: 20-byte block = f32 scale + 16 nibble bytes
 template <> struct Raw32<RFQ_Q4_0> {
-    static constexpr bool TRIP_HEADER = false;
     static constexpr int ND = 5;
     uint32_t d[ND];
     __device__ __forceinline__ void load(Rsrc w, uint32_t row_off, int st, int wh)
@@ -135,7 +134,6 @@ template <> struct Raw32<RFQ_Q4_0> {
 
 // src/kernels/quant/q8_0.rs:55-59: 36-byte block = f32 scale + 32 offset-binary bytes
 template <> struct Raw32<RFQ_Q8_0> {
-    static constexpr bool TRIP_HEADER = false;
     static constexpr int ND = 9;
     uint32_t d[ND];
     __device__ __forceinline__ void load(Rsrc w, uint32_t row_off, int st, int wh)
@@ -171,7 +169,6 @@ template <> struct Raw32<RFQ_Q8_0> {
 // src/kernels/quant/q4_k.rs:222-268: sub-block sb of a 256-byte super-block:
 // f16 scale at 2*sb, i8 min at 16+sb, 16 nibble bytes at 32+28*sb
 template <> struct Raw32<RFQ_Q4_K> {
-    static constexpr bool TRIP_HEADER = true;                     // scales and mins are loaded once per super-block
     static constexpr int ND = 5;
     uint32_t d[ND];
     __device__ __forceinline__ void load(Rsrc w, uint32_t row_off, int st, int wh)
@@ -225,7 +222,6 @@ template <> struct Raw32<RFQ_Q4_K> {
 // 2*(i/16), signed 6-bit field at bit 6*i of the stream at +32.  32 elements =
 // two scales + 24 stream bytes.
 template <> struct Raw32<RFQ_Q6_K> {
-    static constexpr bool TRIP_HEADER = false;
     static constexpr int ND = 7;
     uint32_t d[ND];
     __device__ __forceinline__ void load(Rsrc w, uint32_t row_off, int st, int wh)
@@ -264,7 +260,6 @@ template <> struct Raw32<RFQ_Q6_K> {
 
 // block_q4_0: f16 d, 16 bytes; low nibbles = elements 0..15, high = 16..31; d * (q - 8)
 template <> struct Raw32<RFQ_GGUF_Q4_0> {
-    static constexpr bool TRIP_HEADER = false;
     static constexpr int ND = 5;
     uint32_t d[ND];
     __device__ __forceinline__ void load(Rsrc w, uint32_t row_off, int st, int wh)
@@ -294,7 +289,6 @@ template <> struct Raw32<RFQ_GGUF_Q4_0> {
 
 // block_q8_0: f16 d, 32 int8; d * q
 template <> struct Raw32<RFQ_GGUF_Q8_0> {
-    static constexpr bool TRIP_HEADER = false;
     static constexpr int ND = 9;
     uint32_t d[ND];
     __device__ __forceinline__ void load(Rsrc w, uint32_t row_off, int st, int wh)
@@ -333,7 +327,6 @@ template <> struct Raw32<RFQ_GGUF_Q8_0> {
 // same magnitude here (a real min/max quantisation), so the rounded fp16 value
 // of the whole expression carries the usual 2^-12 relative error.
 template <> struct Raw32<RFQ_GGUF_Q4_K> {
-    static constexpr bool TRIP_HEADER = false;
     static constexpr int ND = 12;
     uint32_t d[ND];
     __device__ __forceinline__ void load(Rsrc w, uint32_t row_off, int st, int)
@@ -384,7 +377,6 @@ template <> struct Raw32<RFQ_GGUF_Q4_K> {
 // from ql[64 n + 32 (t & 1) + l] (>> 4 for t >= 2), bits 4-5 from qh[32 n + l] >> 2 t,
 // scales sc[8 n + 2 t + l / 16]; value = (d * sc) * (q - 32).
 template <> struct Raw32<RFQ_GGUF_Q6_K> {
-    static constexpr bool TRIP_HEADER = false;
     static constexpr int ND = 17;
     uint32_t d[ND];
     __device__ __forceinline__ void load(Rsrc w, uint32_t row_off, int st, int wh)

@@ -30,6 +30,18 @@ def _dev_u8(t: torch.Tensor) -> torch.Tensor:
     return t
 
 
+def upload(host: "np.ndarray | bytes | memoryview", out: torch.Tensor | None = None) -> torch.Tensor:
+    """Host bytes -> a device uint8 tensor through the library's pinned staging ring (rfq_upload)."""
+    import numpy as np
+    h = np.frombuffer(host, dtype=np.uint8) if not isinstance(host, np.ndarray) else np.ascontiguousarray(host).view(np.uint8).reshape(-1)
+    if out is None:
+        out = torch.empty(h.size, dtype=torch.uint8, device="cuda")
+    if out.numel() != h.size or out.dtype != torch.uint8 or not out.is_contiguous():
+        raise ValueError("upload: out must be a contiguous uint8 device tensor of the source's size")
+    check(lib().rfq_upload(C.c_void_p(h.ctypes.data), h.size, _ptr(out), _stream()))
+    return out
+
+
 def dequant(fmt: int, packed: torch.Tensor, n_elems: int, out: torch.Tensor | None = None) -> torch.Tensor:
     """Packed device bytes -> f32 device tensor of n_elems."""
     packed = _dev_u8(packed)
