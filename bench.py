@@ -233,6 +233,7 @@ def main():
                          "of a profiler against a kernel of known traffic)")
     ap.add_argument("--only-mlp", action="store_true", help="only the SwiGLU MLP line (profiling runs)")
     ap.add_argument("--mlp-steps", type=int, default=300)
+    ap.add_argument("--only-gguf", action="store_true", help="only the GGUF-layout Q4_K GEMV line (profiling runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build is single-GPU (one MI355X per box); run with --gpus 1. "
@@ -249,6 +250,16 @@ def main():
 
     if args.only_mlp:
         print(json.dumps({"Q4_K mlp_swiglu 4096x14336 m1": time_mlp(torch, Q.Q4_K, 4096, 14336, Q, steps=args.mlp_steps)}))
+        return
+
+    if args.only_gguf:
+        f = Q.GGUF_Q4_K
+        c = min(-(-int(2.5 * CACHE_BYTES) // Q.packed_bytes(f, N * K)), 64)
+        _, d, *_ = time_gemv(torch, f, N, K, 1, c, args.steps, args.warmup, Q, 20260051)
+        b = algorithmic_bytes(f, N, K, 1, Q)
+        print(json.dumps({"GGUF_Q4_K gemv 14336x4096": {"GB/s": round(b / (d / args.steps) / 1e9, 1), "us": round(d / args.steps * 1e6, 2),
+                                                        "hbm_frac": round(b / (d / args.steps) / 1e9 / HBM_PEAK_GBS, 4),
+                                                        "algorithmic_bytes": b, "weight_copies": c}}))
         return
 
     fmt = Q.Q4_K

@@ -291,8 +291,18 @@ public:
     void *as_ptr() const { return inner_.get(); }
     template <typename T> Status copy_from_host(const std::vector<T> &src)
     {
-        if (src.size() * sizeof(T) > size_) return Status::Err("copy_from_host: source larger than the buffer");
-        hipError_t e = hipMemcpy(as_ptr(), src.data(), src.size() * sizeof(T), hipMemcpyHostToDevice);
+        const size_t bytes = src.size() * sizeof(T);
+        if (bytes > size_) return Status::Err("copy_from_host: source larger than the buffer");
+        hipError_t e = hipSuccess;
+        if (bytes >= ((size_t)1 << 20)) {
+            // large sources (tensor data) go through the library's pinned staging ring; the copy stays
+            // synchronous, as the reference's hipMemcpy is (src/backend/hip_backend/memory.rs:135-170)
+            Status up = detail::from_rfq(rfq_upload(src.data(), bytes, as_ptr(), nullptr), "copy_from_host");
+            if (!up.ok) return up;
+            e = hipStreamSynchronize(nullptr);
+        } else {
+            e = hipMemcpy(as_ptr(), src.data(), bytes, hipMemcpyHostToDevice);
+        }
         return e == hipSuccess ? ok_status() : Status::Err(std::string("hipMemcpy H2D failed: ") + hipGetErrorString(e));
     }
     template <typename T> Status copy_to_host(std::vector<T> &dst) const
