@@ -82,13 +82,15 @@ def time_dequant(torch, fmt, n, k, steps, warmup, Q, seed):
     copies = 4
     dws = [torch.from_numpy(w).to(dev) for _ in range(copies)]
     ptrs = (C.c_void_p * copies)(*[t.data_ptr() for t in dws])
-    out = torch.empty(n * k, dtype=torch.float32, device=dev)
+    # enough output buffers that a step's output lines are not the last step's, still in the last-level cache
+    out_copies = max(1, -(-int(2.5 * CACHE_BYTES) // (4 * n * k)))
+    out = torch.empty(out_copies * n * k, dtype=torch.float32, device=dev)
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     ms = C.c_float(0)
     L = _lib.lib()
-    _lib.check(L.rfq_bench_dequant(fmt, ptrs, copies, w.size, C.c_void_p(out.data_ptr()), n * k, 0, warmup, stream,
+    _lib.check(L.rfq_bench_dequant(fmt, ptrs, copies, w.size, C.c_void_p(out.data_ptr()), n * k, out_copies, 0, warmup, stream,
                                    C.byref(ms)))
-    _lib.check(L.rfq_bench_dequant(fmt, ptrs, copies, w.size, C.c_void_p(out.data_ptr()), n * k, 0, steps, stream,
+    _lib.check(L.rfq_bench_dequant(fmt, ptrs, copies, w.size, C.c_void_p(out.data_ptr()), n * k, out_copies, 0, steps, stream,
                                    C.byref(ms)))
     return ms.value / 1e3 / steps, w.size + 4 * n * k
 

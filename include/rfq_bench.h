@@ -25,8 +25,11 @@ RFQ_API int rfq_bench_gemv(int fmt, const void *const *d_w_copies, int copies, s
                            float *d_y, int m, int n, int k, int warmup, int steps, void *stream,
                            float *elapsed_ms);
 
+/* Step i reads input copy i % copies and writes the n_elems floats at
+ * d_out + (i % out_copies) * n_elems: with enough of both, neither the packed
+ * input nor the previous output of the same lines sits in the last-level cache. */
 RFQ_API int rfq_bench_dequant(int fmt, const void *const *d_in_copies, int copies, size_t packed_bytes, float *d_out,
-                              size_t n_elems, int warmup, int steps, void *stream, float *elapsed_ms);
+                              size_t n_elems, int out_copies, int warmup, int steps, void *stream, float *elapsed_ms);
 
 RFQ_API int rfq_bench_gemm_f16(int fmt, const void *d_w, size_t w_bytes, const void *d_a_f16, void *d_out,
                                int out_dtype, int m, int n, int k, int warmup, int steps, void *stream,

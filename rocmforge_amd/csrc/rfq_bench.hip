@@ -50,11 +50,11 @@ int rfq_bench_gemv(int fmt, const void *const *d_w_copies, int copies, size_t w_
 }
 
 int rfq_bench_dequant(int fmt, const void *const *d_in_copies, int copies, size_t packed_bytes, float *d_out,
-                      size_t n_elems, int warmup, int steps, void *stream, float *elapsed_ms)
+                      size_t n_elems, int out_copies, int warmup, int steps, void *stream, float *elapsed_ms)
 {
-    if (!d_in_copies || copies <= 0) return rfq::fail(RFQ_E_BADARG, "rfq_bench_dequant: no input copies");
+    if (!d_in_copies || copies <= 0 || out_copies <= 0) return rfq::fail(RFQ_E_BADARG, "rfq_bench_dequant: no copies");
     return timed_loop(warmup, steps, stream, elapsed_ms, [&](int i) {
-        return rfq_dequant(fmt, d_in_copies[i % copies], packed_bytes, d_out, n_elems, stream);
+        return rfq_dequant(fmt, d_in_copies[i % copies], packed_bytes, d_out + (size_t)(i % out_copies) * n_elems, n_elems, stream);
     });
 }
 

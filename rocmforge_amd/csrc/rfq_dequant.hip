@@ -169,6 +169,15 @@ template <> __device__ __forceinline__ float4 decode_quad<RFQ_GGUF_Q6_K>(const u
     return r;
 }
 
+// 16-byte store of decoded values.  The f32 output is four to eight times the packed input and is
+// written once: non-temporal stores keep it from displacing the input stream in the caches
+// (Q4_K 14336x4096: 53.7 -> 40.7 us, MXFP4 28672x8192: 232 -> 213 us).
+__device__ __forceinline__ void store_quad(float *o, const float4 &v)
+{
+    typedef float v4f_nt __attribute__((ext_vector_type(4)));
+    __builtin_nontemporal_store(v4f_nt{v.x, v.y, v.z, v.w}, reinterpret_cast<v4f_nt *>(o));
+}
+
 template <int FMT, bool ALIGNED16>
 __global__ void __launch_bounds__(256)
 dequant_blocks_kernel(const uint8_t *__restrict__ in, float *__restrict__ out, size_t n_quads)
@@ -181,7 +190,7 @@ dequant_blocks_kernel(const uint8_t *__restrict__ in, float *__restrict__ out, s
     float4 v = decode_quad<FMT>(in + b * Fmt<FMT>::BB, e0);
     float *o = out + t * 4;
     if (ALIGNED16) {
-        *reinterpret_cast<float4 *>(o) = v;
+        store_quad(o, v);
     } else {
         o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
     }
@@ -193,11 +202,8 @@ dequant_blocks_kernel(const uint8_t *__restrict__ in, float *__restrict__ out, s
 // (decode(b >> 4), decode(b & 15)), element 2j being the HIGH nibble of byte j
 // (src/loader/dequant.rs:53-77).  What remains per element is the multiply by
 // the block's power of two and the clamp.  A workgroup walks MX_LUT_TRIPS
-// consecutive chunks of 256 quads so the table is built once per 32 KiB written.
-// (With the input streamed beside it, the f32 output of every format goes out at
-// 4.2-4.6 TB/s, against 6.9 TB/s for a pure fill: mixed read/write traffic bounds
-// these kernels, not their instructions.)
-constexpr int MX_LUT_TRIPS = 8;
+// consecutive chunks of 256 quads so the table is built once per 12 KiB written.
+constexpr int MX_LUT_TRIPS = 3;   // measured 1..8, 16 at 28672x8192: 214, 181, 171, 186, 201, 201, 200, 203, 212 us
 
 __device__ __forceinline__ float4 mxfp4_quad_from_table(const float2 *lut, int exponent, uint32_t w)
 {
@@ -223,17 +229,23 @@ dequant_mxfp4_lut_kernel(const uint8_t *__restrict__ in, float *__restrict__ out
     const uint32_t code_off = 1u + ((threadIdx.x & 7u) << 1);
     float *o = out + (wg_first + threadIdx.x) * 4;
     if (wg_first + 256 * MX_LUT_TRIPS <= n_quads) {
-        // every load first (constant offsets from one address), then table, scale, clamp, store
-        int ex[MX_LUT_TRIPS];
-        uint32_t w[MX_LUT_TRIPS];
+        // Every load first (constant offsets from one address), then table, scale, clamp, store.
+        // One dword per lane and trip: lane j of a block's eight reads bytes 2j .. 2j+3 (its two code
+        // bytes are bytes 1 and 2 of the dword; the last lane starts one byte earlier so as not to
+        // read past the block), and lane 0's byte 0 is the block's exponent, handed to the other
+        // seven through the LDS crossbar -- half the load instructions of a byte and a halfword each.
+        const int j = threadIdx.x & 7, last = j == 7;
+        const uint8_t *dw_ptr = blk0 + 2 * j - last;
+        const int code_shift = 8 + 8 * last;
+        const int from_lane0 = (int)((threadIdx.x & 63u & ~7u) << 2);
+        uint32_t dw[MX_LUT_TRIPS];
+#pragma unroll
+        for (int trip = 0; trip < MX_LUT_TRIPS; trip++) dw[trip] = ld<uint32_t>(dw_ptr + trip * 32 * 17);
 #pragma unroll
         for (int trip = 0; trip < MX_LUT_TRIPS; trip++) {
-            ex[trip] = (int)(int8_t)blk0[trip * 32 * 17];
-            w[trip] = ld<uint16_t>(blk0 + trip * 32 * 17 + code_off);
+            const int ex = (int)(int8_t)(__builtin_amdgcn_ds_bpermute(from_lane0, (int)dw[trip]) & 255);
+            store_quad(o + (size_t)trip * 1024, mxfp4_quad_from_table(lut, ex, (dw[trip] >> code_shift) & 0xFFFFu));
         }
-#pragma unroll
-        for (int trip = 0; trip < MX_LUT_TRIPS; trip++)
-            *reinterpret_cast<float4 *>(o + (size_t)trip * 1024) = mxfp4_quad_from_table(lut, ex[trip], w[trip]);
     } else {
         for (int trip = 0; trip < MX_LUT_TRIPS; trip++) {
             if (wg_first + threadIdx.x + (size_t)trip * 256 < n_quads) {

@@ -16,7 +16,6 @@
 #include <mutex>
 #include <thread>
 #include <unordered_map>
-#include <vector>
 
 #include "rfq_common.hpp"
 
@@ -63,14 +62,20 @@ void fill_slot(uint8_t *dst, const uint8_t *src, size_t bytes)
     }
     const int parts = (int)std::min<size_t>(COPY_THREADS, bytes / THREAD_MIN);
     const size_t per = ((bytes / parts) + 4095) & ~(size_t)4095;
-    std::vector<std::thread> helpers;
-    helpers.reserve(parts - 1);
+    // (no exception may leave through the C ABI: a part whose thread cannot be started is copied here)
+    std::thread helpers[COPY_THREADS];
+    int started = 0;
     for (int p = 1; p < parts; p++) {
         const size_t at = per * p, len = p == parts - 1 ? bytes - at : per;
-        helpers.emplace_back([=] { std::memcpy(dst + at, src + at, len); });
+        try {
+            helpers[started] = std::thread([=] { std::memcpy(dst + at, src + at, len); });
+            started++;
+        } catch (...) {
+            std::memcpy(dst + at, src + at, len);
+        }
     }
     std::memcpy(dst, src, per);
-    for (auto &t : helpers) t.join();
+    for (int i = 0; i < started; i++) helpers[i].join();
 }
 
 } // namespace
