@@ -199,6 +199,25 @@ template <> struct Unit<RFQ_Q6_K> {
 // clamp(scale * v, +-L) == scale * clamp(v, +-L/scale) for a power-of-two
 // scale, so the clamp is applied to the decoded code and the scale once per
 // unit.  The bound only bites for exponents >= 1 (|code value| <= 8).
+// MXFP4: decoding a code (zero test, sign, exponent) costs more than its multiply-add, so the
+// two values of a code byte come from a 256-entry table in LDS, entry b = (decode(b >> 4),
+// decode(b & 15)); the kernels that dot MXFP4 units fill it first (unit_tables_init).
+__device__ __forceinline__ float2 *mxfp4_lut()
+{
+    __shared__ float2 lut[256];
+    return lut;
+}
+
+template <int FMT> __device__ __forceinline__ void unit_tables_init()
+{
+    if constexpr (FMT == RFQ_MXFP4) {
+        float2 *lut = mxfp4_lut();
+        for (int i = threadIdx.x; i < 256; i += blockDim.x)
+            lut[i] = make_float2(decode_e2m1((uint32_t)i >> 4), decode_e2m1((uint32_t)i & 15u));
+        __syncthreads();
+    }
+}
+
 template <> struct Unit<RFQ_MXFP4> {
     static constexpr bool NEEDS_XSUM = false;
     int e; U4 q;
@@ -212,15 +231,15 @@ template <> struct Unit<RFQ_MXFP4> {
     {
         // bound on |code value|: 8 / 2^e when e >= 1 (exact, 2^(3-e)), else 8.
         float bound = e >= 1 ? __uint_as_float((uint32_t)(130 - e) << 23) : 8.0f;
+        const float2 *lut = mxfp4_lut();
         float s0 = 0.f, s1 = 0.f;
 #pragma unroll
         for (int d = 0; d < 4; d++) {
 #pragma unroll
             for (int b = 0; b < 4; b++) {
-                uint32_t byte = (q.v[d] >> (8 * b)) & 255u;
-                float hi = decode_e2m1(byte >> 4), lo = decode_e2m1(byte & 15u); // element 2j = high nibble
-                hi = __builtin_amdgcn_fmed3f(hi, -bound, bound);
-                lo = __builtin_amdgcn_fmed3f(lo, -bound, bound);
+                const float2 v = lut[(q.v[d] >> (8 * b)) & 255u];                // element 2j = high nibble
+                const float hi = __builtin_amdgcn_fmed3f(v.x, -bound, bound);
+                const float lo = __builtin_amdgcn_fmed3f(v.y, -bound, bound);
                 s0 = __builtin_fmaf(hi, x[8 * d + 2 * b], s0);
                 s1 = __builtin_fmaf(lo, x[8 * d + 2 * b + 1], s1);
             }
@@ -545,6 +564,7 @@ gemv_xreg_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
         for (int j = 0; j < UPL; j++) load_x32(f.norm_w + (size_t)unit[j] * 32, nws[FUSE ? j : 0]);
     }
 
+    unit_tables_init<FMT>();
     __shared__ float part[R][4];
     const int rows_per_team = groups * R;
     const int row0 = (blockIdx.x * TEAMS + team) * rows_per_team;
@@ -1305,6 +1325,7 @@ gemv_generic_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, 
     const int ku = k >> 5;
     const size_t rb = row_bytes<FMT>(k);
     const int waves_total = gridDim.x * 4;
+    unit_tables_init<FMT>();
     for (int r = blockIdx.x * 4 + wave; r < n; r += waves_total) {
         const uint8_t *row = w + (size_t)r * rb;
         float acc[M];
