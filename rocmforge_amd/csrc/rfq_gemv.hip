@@ -208,12 +208,24 @@ __device__ __forceinline__ float2 *mxfp4_lut()
     return lut;
 }
 
+// MXFP6 likewise: 64 decoded codes.
+__device__ __forceinline__ float *mxfp6_lut()
+{
+    __shared__ float lut[64];
+    return lut;
+}
+
 template <int FMT> __device__ __forceinline__ void unit_tables_init()
 {
     if constexpr (FMT == RFQ_MXFP4) {
         float2 *lut = mxfp4_lut();
         for (int i = threadIdx.x; i < 256; i += blockDim.x)
             lut[i] = make_float2(decode_e2m1((uint32_t)i >> 4), decode_e2m1((uint32_t)i & 15u));
+        __syncthreads();
+    }
+    if constexpr (FMT == RFQ_MXFP6_E2M3) {
+        float *lut = mxfp6_lut();
+        if (threadIdx.x < 64) lut[threadIdx.x] = decode_e2m3(threadIdx.x);
         __syncthreads();
     }
 }
@@ -261,6 +273,7 @@ template <> struct Unit<RFQ_MXFP6_E2M3> {
     {
         // 7.5 * 2^-e for e >= 1: 7.5 = 0x40F00000 (biased exponent 129).
         float bound = e >= 1 ? __uint_as_float(0x40F00000u - ((uint32_t)e << 23)) : 7.5f;
+        const float *lut = mxfp6_lut();
         float s0 = 0.f, s1 = 0.f;
         // group j: bytes b[3j..3j+3]; see the extraction table in rfq_dequant.hip.
 #pragma unroll
@@ -270,9 +283,9 @@ template <> struct Unit<RFQ_MXFP6_E2M3> {
             uint32_t w = (sh == 0) ? q.v[d]
                                    : __builtin_amdgcn_alignbit(d + 1 < 6 ? q.v[d + 1] : 0u, q.v[d], sh);
             uint32_t b0 = w & 255u, b1 = (w >> 8) & 255u, b2 = (w >> 16) & 255u, b3 = w >> 24;
-            float v0 = decode_e2m3(b1 >> 2);
-            float v1 = decode_e2m3((b0 >> 4) | ((b1 & 3u) << 4));
-            float v2 = decode_e2m3((b1 >> 6) | ((b2 & 15u) << 2));
+            float v0 = lut[b1 >> 2];
+            float v1 = lut[(b0 >> 4) | ((b1 & 3u) << 4)];
+            float v2 = lut[(b1 >> 6) | ((b2 & 15u) << 2)];
             v0 = __builtin_amdgcn_fmed3f(v0, -bound, bound);
             v1 = __builtin_amdgcn_fmed3f(v1, -bound, bound);
             v2 = __builtin_amdgcn_fmed3f(v2, -bound, bound);
@@ -280,7 +293,7 @@ template <> struct Unit<RFQ_MXFP6_E2M3> {
             s1 = __builtin_fmaf(v1, x[4 * j + 1], s1);
             s0 = __builtin_fmaf(v2, x[4 * j + 2], s0);
             if (j < 7) { // element 31 is never written by the reference: weight 0
-                float v3 = __builtin_amdgcn_fmed3f(decode_e2m3(b3 & 63u), -bound, bound);
+                float v3 = __builtin_amdgcn_fmed3f(lut[b3 & 63u], -bound, bound);
                 s1 = __builtin_fmaf(v3, x[4 * j + 3], s1);
             }
         }
