@@ -664,9 +664,9 @@ gemv_xreg_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
 // value, and the final scaling).  A non-finite x value poisons its unit's s
 // with NaN, as it would poison the float sum.
 //
-// LDS holds, per unit, 24 limb dwords + s + sum(x) (stride 28 dwords).
+// LDS holds, per unit, 24 limb dwords + s + sum(x) + the sums of its two halves (stride 28 dwords).
 
-struct XPrep { uint32_t l[24]; float s, xsum; };
+struct XPrep { uint32_t l[24]; float s, xsum, xh0, xh1; };   // xh0, xh1: sums of elements 0..15 and 16..31
 
 // Byte-transpose four 24-bit integers into (low, mid, top) limb dwords.
 __device__ __forceinline__ void limbs4(uint32_t x0, uint32_t x1, uint32_t x2, uint32_t x3, uint32_t *out3)
@@ -704,6 +704,7 @@ __device__ __forceinline__ void prep_convert(const float (&xv)[16], int half, ui
     bool bad = false;
 #pragma unroll
     for (int i = 0; i < 16; i++) bad |= !(fabsf(xv[i]) <= 3.40282347e+38f);
+    const float half_sum = sum;
     m = fmaxf(m, dpp_xor1_f(m));
     sum += dpp_xor1_f(sum);
     bad |= __builtin_amdgcn_update_dpp(0, (int)bad, 0xB1, 0xF, 0xF, true) != 0;
@@ -732,6 +733,7 @@ __device__ __forceinline__ void prep_convert(const float (&xv)[16], int half, ui
         lds_unit[24] = __float_as_uint(sc);
         lds_unit[25] = __float_as_uint(sum);
     }
+    lds_unit[26 + half] = __float_as_uint(half_sum);
 }
 
 // sum_i nibble_i * X_i for 16 weight bytes in low-nibble-first order.
@@ -901,6 +903,34 @@ template <> struct IUnit<RFQ_GGUF_Q4_K> : Unit<RFQ_GGUF_Q4_K> {
     }
 };
 
+// A 6-bit code is a byte once its nibble and its bit pair are joined (five instructions per
+// four weights), which is what the byte dot products take; the two int8 scales of the unit
+// get a sum each, and the offset of 32 goes through the sums of x over the two halves.
+template <> struct IUnit<RFQ_GGUF_Q6_K> : Unit<RFQ_GGUF_Q6_K> {
+    static constexpr bool PAIR = false;
+    static constexpr bool NIBBLE = false;
+    static constexpr uint32_t TOPOFF = 0;
+    __device__ __forceinline__ float idot(const XPrep &xp) const
+    {
+        const int shl = 4 * (t >> 1), shh = 2 * t;
+        uint32_t alo[2] = {0, 0}, amid[2] = {0, 0};
+        int atop[2] = {0, 0};
+#pragma unroll
+        for (int w = 0; w < 8; w++) {
+            const uint32_t v = ((ql.v[w] >> shl) & 0x0F0F0F0Fu) | (((qh.v[w] >> shh) & 0x03030303u) << 4);
+            const uint32_t *L = &xp.l[w * 3];
+            alo[w >> 2] = __builtin_amdgcn_udot4(v, L[0], alo[w >> 2], false);
+            amid[w >> 2] = __builtin_amdgcn_udot4(v, L[1], amid[w >> 2], false);
+            atop[w >> 2] = __builtin_amdgcn_sdot4((int)v, (int)L[2], atop[w >> 2], false);
+        }
+        const float S0 = __builtin_fmaf((float)atop[0], 65536.0f, __builtin_fmaf((float)amid[0], 256.0f, (float)alo[0]));
+        const float S1 = __builtin_fmaf((float)atop[1], 65536.0f, __builtin_fmaf((float)amid[1], 256.0f, (float)alo[1]));
+        const float sc0 = (float)(int)(int8_t)(sc2 & 255u), sc1 = (float)(int)(int8_t)(sc2 >> 8);
+        const float h0 = __builtin_fmaf(xp.s, S0, -32.0f * xp.xh0), h1 = __builtin_fmaf(xp.s, S1, -32.0f * xp.xh1);
+        return f16_bits_to_f32(d) * __builtin_fmaf(sc0, h0, sc1 * h1);
+    }
+};
+
 // The formats without paired units never call idot_pair.
 template <typename IU>
 __device__ __forceinline__ float idot_pair_of(const IU &u, const XPrep &xe, const XPrep &xo)
@@ -1029,6 +1059,8 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
         }
         xp[j].s = __uint_as_float(src[24]);
         xp[j].xsum = __uint_as_float(src[25]);
+        xp[j].xh0 = __uint_as_float(src[26]);
+        xp[j].xh1 = __uint_as_float(src[27]);
     }
     RFQ_TS(3);
 
@@ -1122,6 +1154,8 @@ gemv_idot_batch_kernel(const uint8_t *__restrict__ w, const float *__restrict__ 
         }
         xp[v].s = __uint_as_float(src[24]);
         xp[v].xsum = __uint_as_float(src[25]);
+        xp[v].xh0 = __uint_as_float(src[26]);
+        xp[v].xh1 = __uint_as_float(src[27]);
     }
 
     __shared__ float part[R * M][4];
@@ -1423,6 +1457,7 @@ template <> struct HasIdot<RFQ_Q8_0> { static constexpr bool value = true; };
 template <> struct HasIdot<RFQ_GGUF_Q4_0> { static constexpr bool value = true; };
 template <> struct HasIdot<RFQ_GGUF_Q8_0> { static constexpr bool value = true; };
 template <> struct HasIdot<RFQ_GGUF_Q4_K> { static constexpr bool value = true; };
+template <> struct HasIdot<RFQ_GGUF_Q6_K> { static constexpr bool value = true; };
 // (batches of the GGUF layouts go through the one-row-per-wavefront kernel)
 template <int FMT> struct HasIdotBatch { static constexpr bool value = HasIdot<FMT>::value && FMT < RFQ_GGUF_Q4_0; };
 
