@@ -1277,20 +1277,25 @@ gemv_mfma_prep_kernel(const float *__restrict__ x, _Float16 *__restrict__ parts,
 constexpr int MFMA_NB = 16;                           // units of a wavefront in flight together
 constexpr int MFMA_WAVES = 8;
 
+// FMT: RFQ_Q8_0 (36-byte blocks: f32 scale, offset-binary bytes) or RFQ_GGUF_Q8_0 (34-byte
+// blocks: f16 scale, int8 bytes, flipped to offset binary with one XOR per dword).
+template <int FMT>
 __global__ void __launch_bounds__(64 * MFMA_WAVES)
 gemv_mfma_q8_0_kernel(const uint8_t *__restrict__ w, const _Float16 *__restrict__ parts, const float *__restrict__ sx,
                       float *__restrict__ y, int m, int n, int k)
 {
+    constexpr int BB = Fmt<FMT>::BB, DOFF = FMT == RFQ_Q8_0 ? 4 : 2;
+    constexpr uint32_t FLIP = FMT == RFQ_Q8_0 ? 0u : 0x80808080u;
     __shared__ float red[MFMA_WAVES * 16 * 8];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, j = lane & 15, q = lane >> 4;
     const int units = k / 32, n0 = blockIdx.x * 16;
     const int row = n0 + j < n ? n0 + j : n - 1;
-    const uint8_t *row_ptr = w + (size_t)row * units * 36;
+    const uint8_t *row_ptr = w + (size_t)row * units * BB;
     // The weight bytes are fetched by four neighbouring lanes per row (32
     // consecutive bytes: one request instead of four) and handed to the lane
     // that holds them as an operand, lane 16 * q + j <- lane 4 * j + q.
     const int row_c = n0 + (lane >> 2) < n ? n0 + (lane >> 2) : n - 1;
-    const uint8_t *row_ptr_c = w + (size_t)row_c * units * 36 + 4 + 8 * (lane & 3);
+    const uint8_t *row_ptr_c = w + (size_t)row_c * units * BB + DOFF + 8 * (lane & 3);
     const int from_lane4 = 4 * (4 * j + q);
     const v4u_t *parts_l = reinterpret_cast<const v4u_t *>(parts) + q * 8 + (j & 7);
     const v2h_t bias = {(_Float16)-1152.0f, (_Float16)-1152.0f};
@@ -1307,9 +1312,9 @@ gemv_mfma_q8_0_kernel(const uint8_t *__restrict__ w, const _Float16 *__restrict_
 #pragma unroll
         for (int b = 0; b < MFMA_NB; b++) {
             const int u = base + MFMA_WAVES * b, uc = u < units ? u : units - 1; // (past the end: a valid unit, weight scale 0)
-            const uint8_t *blk = row_ptr + (size_t)uc * 36;
-            wq[b] = (RFQ_M8_SKIP & 1) ? v2u_t{(uint32_t)lane, (uint32_t)b} : ld<v2u_t>(row_ptr_c + (size_t)uc * 36);
-            ws[b] = (RFQ_M8_SKIP & 1) ? 1.0f : ld<float>(blk);                    // (no branch around a load: it would wait for the others)
+            const uint8_t *blk = row_ptr + (size_t)uc * BB;
+            wq[b] = (RFQ_M8_SKIP & 1) ? v2u_t{(uint32_t)lane, (uint32_t)b} : ld<v2u_t>(row_ptr_c + (size_t)uc * BB);
+            ws[b] = (RFQ_M8_SKIP & 1) ? 1.0f : (FMT == RFQ_Q8_0 ? ld<float>(blk) : f16_bits_to_f32(ld<uint16_t>(blk)));                    // (no branch around a load: it would wait for the others)
             xh[b] = (RFQ_M8_SKIP & 2) ? v4u_t{1u, 2u, 3u, (uint32_t)lane} : parts_l[(size_t)uc * 64];
             xl[b] = (RFQ_M8_SKIP & 2) ? v4u_t{1u, 2u, 3u, (uint32_t)lane} : parts_l[(size_t)uc * 64 + 32];
             if (b < MFMA_NB / 2) load_s4(b);
@@ -1321,7 +1326,7 @@ gemv_mfma_q8_0_kernel(const uint8_t *__restrict__ w, const _Float16 *__restrict_
             v4u_t wb;
 #pragma unroll
             for (int d = 0; d < 2; d++) {
-                const uint32_t wd = (uint32_t)__builtin_amdgcn_ds_bpermute(from_lane4, (int)wq[b][d]);
+                const uint32_t wd = (uint32_t)__builtin_amdgcn_ds_bpermute(from_lane4, (int)wq[b][d]) ^ FLIP;
                 const uint32_t p0 = __builtin_amdgcn_perm(0x64646464u, wd, 0x04010400u);
                 const uint32_t p1 = __builtin_amdgcn_perm(0x64646464u, wd, 0x04030402u);
                 v2h_t h0, h1;
@@ -1458,8 +1463,7 @@ template <> struct HasIdot<RFQ_GGUF_Q4_0> { static constexpr bool value = true; 
 template <> struct HasIdot<RFQ_GGUF_Q8_0> { static constexpr bool value = true; };
 template <> struct HasIdot<RFQ_GGUF_Q4_K> { static constexpr bool value = true; };
 template <> struct HasIdot<RFQ_GGUF_Q6_K> { static constexpr bool value = true; };
-// (batches of the GGUF layouts go through the one-row-per-wavefront kernel)
-template <int FMT> struct HasIdotBatch { static constexpr bool value = HasIdot<FMT>::value && FMT < RFQ_GGUF_Q4_0; };
+template <int FMT> struct HasIdotBatch { static constexpr bool value = HasIdot<FMT>::value; };
 
 template <int FMT, int UPL, int WPR, int R, bool FUSE>
 int launch_idot(const uint8_t *w, const float *x, float *y, int n, int k, int blocks, int groups, const GemvFuse &f,
@@ -1578,6 +1582,7 @@ int run_generic(const uint8_t *w, const float *x, float *y, int n, int k, hipStr
     return RFQ_OK;
 }
 
+template <int FMT>
 int run_mfma_q8_0(const uint8_t *w, const float *x, float *y, int m, int n, int k, hipStream_t s)
 {
     const int units = k / 32;
@@ -1588,7 +1593,7 @@ int run_mfma_q8_0(const uint8_t *w, const float *x, float *y, int m, int n, int 
     _Float16 *parts = reinterpret_cast<_Float16 *>(tmp);
     float *sx = reinterpret_cast<float *>(tmp + parts_bytes);
     hipLaunchKernelGGL(gemv_mfma_prep_kernel, dim3(units), dim3(256), 0, s, x, parts, sx, m, k);
-    hipLaunchKernelGGL(gemv_mfma_q8_0_kernel, dim3((n + 15) / 16), dim3(64 * MFMA_WAVES), 0, s, w, parts, sx, y, m, n, k);
+    hipLaunchKernelGGL(gemv_mfma_q8_0_kernel<FMT>, dim3((n + 15) / 16), dim3(64 * MFMA_WAVES), 0, s, w, parts, sx, y, m, n, k);
     hipError_t launch_err = hipGetLastError();
     if (transient) {
         hipError_t free_err = hipFreeAsync(tmp, s);
@@ -1615,11 +1620,26 @@ int run(const uint8_t *w, const float *x, float *y, int m, int n, int k, hipStre
     const int ku = k / 32;
     if (m == 1 && ku > 16 && ku <= 512)                        // (shorter rows leave most of a wavefront's lanes without a unit)
         return run_rows<FMT, false>(w, x, y, n, k, GemvFuse{nullptr, nullptr, 0.0f, 0}, s);
-    if (FMT == RFQ_Q8_0 && m > 1 && (reinterpret_cast<uintptr_t>(w) & 3u) == 0) return run_mfma_q8_0(w, x, y, m, n, k, s);
+    if constexpr (FMT == RFQ_Q8_0 || FMT == RFQ_GGUF_Q8_0) {
+        if (m > 1 && (reinterpret_cast<uintptr_t>(w) & (FMT == RFQ_Q8_0 ? 3u : 1u)) == 0) return run_mfma_q8_0<FMT>(w, x, y, m, n, k, s);
+    }
     if (HasIdotBatch<FMT>::value && m > 1 && ku > 32 && ku <= 256) {
-        if (m <= 2) return run_idot_batch_k<FMT, 2>(w, x, y, m, n, k, s);
-        if (m <= 4) return run_idot_batch_k<FMT, 4>(w, x, y, m, n, k, s);
-        return run_idot_batch_k<FMT, 8>(w, x, y, m, n, k, s);
+        // the prepared vectors of a launch live in LDS (112 bytes per unit and vector): a batch that
+        // does not fit goes out as launches of four or two vectors
+        const size_t lds_limit = 160 * 1024 - 4096;
+        int mb = m <= 2 ? 2 : (m <= 4 ? 4 : 8);
+        while (mb > 2 && (size_t)mb * ku * 112 > lds_limit) mb /= 2;
+        for (int v0 = 0; v0 < m; v0 += mb) {
+            const int mv = m - v0 < mb ? m - v0 : mb;
+            const float *xv = x + (size_t)v0 * k;
+            float *yv = y + (size_t)v0 * n;
+            int rc;
+            if (mb == 2) rc = run_idot_batch_k<FMT, 2>(w, xv, yv, mv, n, k, s);
+            else if (mb == 4) rc = run_idot_batch_k<FMT, 4>(w, xv, yv, mv, n, k, s);
+            else rc = run_idot_batch_k<FMT, 8>(w, xv, yv, mv, n, k, s);
+            if (rc != RFQ_OK) return rc;
+        }
+        return RFQ_OK;
     }
     switch (m) {
     case 1: return run_generic<FMT, 1>(w, x, y, n, k, s);

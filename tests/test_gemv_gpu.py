@@ -57,14 +57,26 @@ def test_gemv_small_batches(fmt, m, oracle, cuda):
 # Q8_0 batches run on the matrix cores: 16 rows per workgroup, 16 wavefronts
 # that take every 16th unit, eight units at a time: odd unit counts, more than
 # one trip, fewer units than wavefronts, a ragged last row tile.
+@pytest.mark.parametrize("fmt", [Q.Q8_0, Q.GGUF_Q8_0])
 @pytest.mark.parametrize("m,n,k", [(2, 16, 96), (4, 50, 8224), (8, 33, 4096), (7, 1, 32)])
-def test_q8_0_batches_on_the_matrix_cores(m, n, k, oracle, cuda):
-    w = Q.make_weights(Q.Q8_0, n, k, seed=5100 + n)
+def test_q8_0_batches_on_the_matrix_cores(fmt, m, n, k, oracle, cuda):
+    w = Q.make_weights(fmt, n, k, seed=5100 + n)
     x = x_for(m, k, 6100 + m)
     x[0, ::7] *= 1000.0                                                   # outliers: per-unit scaling
     x[m - 1, 5:40] = 0.0                                                  # an all-zero unit
-    got = gpu_gemv(Q.Q8_0, w, x, n, k, cuda)
-    assert_close(got, oracle.qmatmul_nk(Q.Q8_0, w, x, m, n, k), f"Q8_0 m={m} n={n} k={k}")
+    got = gpu_gemv(fmt, w, x, n, k, cuda)
+    assert_close(got, oracle.qmatmul_nk(fmt, w, x, m, n, k), f"{Q.NAMES[fmt]} m={m} n={n} k={k}")
+
+
+@pytest.mark.parametrize("fmt", [Q.Q4_0, Q.Q4_K])
+@pytest.mark.parametrize("m,k", [(8, 4096), (8, 8192), (5, 8192), (3, 8192)])
+def test_batches_whose_prepared_vectors_exceed_lds(fmt, m, k, oracle, cuda):
+    """Eight prepared vectors of k = 8192 need 229 KB of LDS: the batch goes out as launches of four."""
+    n = 150
+    w = Q.make_weights(fmt, n, k, seed=5200 + fmt)
+    x = x_for(m, k, 6200 + m)
+    got = gpu_gemv(fmt, w, x, n, k, cuda)
+    assert_close(got, oracle.qmatmul_nk(fmt, w, x, m, n, k), f"{Q.NAMES[fmt]} m={m} k={k}")
 
 
 @pytest.mark.parametrize("fmt", [Q.MXFP4, Q.MXFP6_E2M3])

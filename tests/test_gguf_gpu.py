@@ -102,10 +102,12 @@ def test_gemv_random_blocks(fmt, oracle, cuda):
 
 
 @pytest.mark.parametrize("fmt", F)
-@pytest.mark.parametrize("m", [2, 5, 8])
-def test_gemv_small_batches(fmt, m, oracle, cuda):
+@pytest.mark.parametrize("m,k", [(2, 2048), (5, 2048), (8, 2048), (3, 4096), (8, 4096), (4, 8192), (8, 8192), (8, 1024)])
+def test_gemv_small_batches(fmt, m, k, oracle, cuda):
+    """Batches of 2..8 vectors: one, two and four wavefronts per row in the batch kernels, and a row too
+    short for them (k = 1024: the one-row-per-wavefront kernel)."""
     from rocmforge_amd import ops
-    n, k = 301, 2048
+    n = 301
     w = Q.make_weights(fmt, n, k, seed=1230 + fmt)
     x = gauss((m, k), 1240 + m)
     got = host(ops.gemv(fmt, dev(w, cuda), dev(x, cuda), n, k))
