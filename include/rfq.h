@@ -43,7 +43,10 @@ extern "C" {
 typedef enum rfq_format {
     RFQ_Q4_0 = 2,        /* 20 B / 32: f32 scale + 16 nibble bytes           */
     RFQ_Q8_0 = 8,        /* 36 B / 32: f32 scale + 32 offset-binary bytes    */
+    RFQ_Q2_K = 10,       /* 256 B / 256: 16 f16 scales, 16 f16 mins, 2-bit codes (+ one high bit); rfq_dequant* only */
+    RFQ_Q3_K = 11,       /* 256 B / 256: 16 f16 scales, 3-bit codes (+ high bits), q - 4;          rfq_dequant* only */
     RFQ_Q4_K = 12,       /* 256 B / 256: 8 f16 scales, 8 i8 mins, nibbles    */
+    RFQ_Q5_K = 13,       /* 256 B / 256: 16 f16 scales, 16 i8 mins, 5-bit codes;                    rfq_dequant* only */
     RFQ_Q6_K = 14,       /* 256 B / 256: 16 f16 scales, 6-bit stream         */
     RFQ_MXFP4 = 20,      /* 17 B / 32: i8 exponent + 16 nibble bytes         */
     RFQ_MXFP6_E2M3 = 21, /* 25 B / 32: i8 exponent + 24 packed bytes         */

@@ -222,6 +222,19 @@ inline std::vector<float> dequant_q6_k(const std::vector<uint8_t> &data, size_t 
 {
     return detail_::through_gpu(RFQ_Q6_K, data.data(), data.size(), n_elements);
 }
+// dequant_q5_k / dequant_q3_k / dequant_q2_k (src/loader/dequant.rs:150-225, 243-320, 326-420)
+inline Result<std::vector<float>> dequant_q5_k(const GgufTensor &t)
+{
+    return Result<std::vector<float>>::Ok(detail_::through_gpu(RFQ_Q5_K, t.data.data(), t.data.size(), t.total_elements()));
+}
+inline Result<std::vector<float>> dequant_q3_k(const GgufTensor &t)
+{
+    return Result<std::vector<float>>::Ok(detail_::through_gpu(RFQ_Q3_K, t.data.data(), t.data.size(), t.total_elements()));
+}
+inline Result<std::vector<float>> dequant_q2_k(const GgufTensor &t)
+{
+    return Result<std::vector<float>>::Ok(detail_::through_gpu(RFQ_Q2_K, t.data.data(), t.data.size(), t.total_elements()));
+}
 inline Result<std::vector<float>> dequant_mxfp4(const GgufTensor &t)
 {
     return Result<std::vector<float>>::Ok(detail_::through_gpu(RFQ_MXFP4, t.data.data(), t.data.size(), t.total_elements()));
@@ -266,6 +279,9 @@ inline Result<std::vector<float>> dequantize(const GgufTensor &t)
     case GgufTensorType::Q8_0: return R::Ok(dequant_q8_0(t.data, t.total_elements()));
     case GgufTensorType::Q4_K: return R::Ok(dequant_q4_k(t.data, t.total_elements()));
     case GgufTensorType::Q6_K: return R::Ok(dequant_q6_k(t.data, t.total_elements()));
+    case GgufTensorType::Q2_K: return dequant_q2_k(t);
+    case GgufTensorType::Q3_K: return dequant_q3_k(t);
+    case GgufTensorType::Q5_K: return dequant_q5_k(t);
     case GgufTensorType::Mxfp4: return dequant_mxfp4(t);
     case GgufTensorType::Mxfp6E2m3: case GgufTensorType::Mxfp6E3m2: return dequant_mxfp6(t);
     default: return R::Err(std::string("dequantize: ") + to_string(t.tensor_type) + " is outside this library's path");

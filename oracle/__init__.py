@@ -89,7 +89,7 @@ def _p(a: np.ndarray):
 
 
 def block_elems(fmt: int) -> int:
-    return 256 if fmt in (Q4_K, Q6_K, 112, 114) else 32
+    return 256 if fmt in (10, 11, Q4_K, 13, Q6_K, 112, 114) else 32
 
 
 def block_bytes(fmt: int) -> int:

@@ -13,7 +13,7 @@
  *
  * Parity status per function:
  *   pinned   : rf_dequant_q4_0, rf_dequant_q8_0, rf_dequant_q4_k,
- *              rf_dequant_q6_k, rf_dequant_mxfp4, rf_dequant_mxfp6,
+ *              rf_dequant_q6_k, rf_dequant_q2_k, rf_dequant_q3_k, rf_dequant_q5_k, rf_dequant_mxfp4, rf_dequant_mxfp6,
  *              rf_decode_e2m1, rf_decode_e2m3, rf_encode_e2m1, rf_encode_e2m3,
  *              rf_pack_6bit, rf_unpack_6bit, rf_pack_mxfp4, rf_pack_mxfp6,
  *              rf_unpack_mxfp4, rf_unpack_mxfp6, rf_cpu_matmul_f32,
@@ -559,7 +559,95 @@ RF_API void rf_dequant_gguf_q6_k(const uint8_t *data, size_t len, size_t n, floa
     }
 }
 
-enum { RF_F32 = 0, RF_F16 = 1, RF_Q4_0 = 2, RF_Q8_0 = 8, RF_Q4_K = 12, RF_Q6_K = 14,
+/* The loader's other K-type decoders (src/loader/dequant.rs): ROCmForge's own 256-byte
+ * layouts of 16 sub-blocks x 16 elements, f16 scale at 2 * sub.  A block the input
+ * does not hold completely ends the loop; elements past n are not written. */
+static inline uint32_t rd_u16le(const uint8_t *p) { return (uint32_t)p[0] | ((uint32_t)p[1] << 8); }
+
+/* dequant_q5_k, src/loader/dequant.rs:150-225: i8 min at 32 + sub, 5-bit codes LSB first
+ * at 48 + 10 * sub, read through a 16-bit window; min + q * scale */
+RF_API void rf_dequant_q5_k(const uint8_t *data, size_t len, size_t n, float *out)
+{
+    size_t blocks = (n + 255) / 256;
+    for (size_t i = 0; i < n; i++) out[i] = 0.0f;
+    for (size_t b = 0; b < blocks; b++) {
+        size_t bs = b * 256;
+        if (bs + 256 > len) break;
+        for (size_t sub = 0; sub < 16; sub++) {
+            float scale = rf_f16_to_f32((uint16_t)rd_u16le(data + bs + sub * 2));
+            float mn = (float)(int8_t)data[bs + 32 + sub];
+            for (size_t i = 0; i < 16; i++) {
+                size_t idx = b * 256 + sub * 16 + i;
+                if (idx >= n) break;
+                size_t bit = i * 5, off = bs + 48 + sub * 10 + bit / 8;
+                uint32_t q = 0;
+                if (off + 2 <= len) q = (rd_u16le(data + off) >> (bit % 8)) & 31u;
+                out[idx] = mn + (float)q * scale;
+            }
+        }
+    }
+}
+
+/* dequant_q3_k, src/loader/dequant.rs:243-320: two high bits per sub-block at 32 + sub / 4
+ * (shift 2 * (sub % 4)), 3-bit codes LSB first at 36 + 6 * sub; bit i of the pair is bit 3
+ * of element i for i < 8 (so only elements 0 and 1 can carry one); (q - 4) * scale */
+RF_API void rf_dequant_q3_k(const uint8_t *data, size_t len, size_t n, float *out)
+{
+    size_t blocks = (n + 255) / 256;
+    for (size_t i = 0; i < n; i++) out[i] = 0.0f;
+    for (size_t b = 0; b < blocks; b++) {
+        size_t bs = b * 256;
+        if (bs + 256 > len) break;
+        for (size_t sub = 0; sub < 16; sub++) {
+            float scale = rf_f16_to_f32((uint16_t)rd_u16le(data + bs + sub * 2));
+            uint32_t qh = (data[bs + 32 + sub / 4] >> ((sub % 4) * 2)) & 3u;
+            for (size_t i = 0; i < 16; i++) {
+                size_t idx = b * 256 + sub * 16 + i;
+                if (idx >= n) break;
+                size_t bit = i * 3, off = bs + 36 + sub * 6 + bit / 8;
+                float q = 0.0f;
+                if (off + 1 < len) {
+                    uint32_t low = (rd_u16le(data + off) >> (bit % 8)) & 7u;
+                    uint32_t high = i < 8 ? (qh >> i) & 1u : 0u;
+                    q = (float)(int8_t)(low | (high << 3)) - 4.0f;
+                }
+                out[idx] = q * scale;
+            }
+        }
+    }
+}
+
+/* dequant_q2_k, src/loader/dequant.rs:326-420: f16 min at 32 + 2 * sub, one high bit per
+ * sub-block at 64 + sub / 8 (shift sub % 8), 2-bit codes LSB first at 68 + 4 * sub; the
+ * high bit is bit 2 of element 0 only; min + q * scale */
+RF_API void rf_dequant_q2_k(const uint8_t *data, size_t len, size_t n, float *out)
+{
+    size_t blocks = (n + 255) / 256;
+    for (size_t i = 0; i < n; i++) out[i] = 0.0f;
+    for (size_t b = 0; b < blocks; b++) {
+        size_t bs = b * 256;
+        if (bs + 256 > len) break;
+        for (size_t sub = 0; sub < 16; sub++) {
+            float scale = rf_f16_to_f32((uint16_t)rd_u16le(data + bs + sub * 2));
+            float mn = rf_f16_to_f32((uint16_t)rd_u16le(data + bs + 32 + sub * 2));
+            uint32_t qh = (data[bs + 64 + sub / 8] >> (sub % 8)) & 1u;
+            for (size_t i = 0; i < 16; i++) {
+                size_t idx = b * 256 + sub * 16 + i;
+                if (idx >= n) break;
+                size_t bit = i * 2, off = bs + 68 + sub * 4 + bit / 8;
+                float q = 0.0f;
+                if (off + 1 < len) {
+                    uint32_t low = (rd_u16le(data + off) >> (bit % 8)) & 3u;
+                    uint32_t high = i < 8 ? (qh >> i) & 1u : 0u;
+                    q = (float)(int8_t)(low | (high << 2));
+                }
+                out[idx] = mn + q * scale;
+            }
+        }
+    }
+}
+
+enum { RF_F32 = 0, RF_F16 = 1, RF_Q4_0 = 2, RF_Q8_0 = 8, RF_Q2_K = 10, RF_Q3_K = 11, RF_Q4_K = 12, RF_Q5_K = 13, RF_Q6_K = 14,
        RF_MXFP4 = 20, RF_MXFP6_E2M3 = 21, RF_MXFP6_E3M2 = 22,
        /* GGUF file layouts: 100 + the ggml type id */
        RF_GGUF_Q4_0 = 102, RF_GGUF_Q8_0 = 108, RF_GGUF_Q4_K = 112, RF_GGUF_Q6_K = 114 };
@@ -573,7 +661,7 @@ RF_API size_t rf_data_size(int type, size_t n)
     case RF_F16: return n * 2;
     case RF_Q4_0: return ((n + 31) / 32) * 36;
     case RF_Q8_0: return ((n + 31) / 32) * 36;
-    case 10: case 11: case RF_Q4_K: case 13: case RF_Q6_K: return ((n + 255) / 256) * 256;
+    case RF_Q2_K: case RF_Q3_K: case RF_Q4_K: case RF_Q5_K: case RF_Q6_K: return ((n + 255) / 256) * 256;
     case RF_MXFP4: return ((n + 31) / 32) * 17;
     case RF_MXFP6_E2M3: case RF_MXFP6_E3M2: return ((n + 31) / 32) * 25;
     default: return 0;
@@ -587,7 +675,7 @@ RF_API size_t rf_block_bytes(int type)
     switch (type) {
     case RF_Q4_0: return 20;
     case RF_Q8_0: return 36;
-    case RF_Q4_K: case RF_Q6_K: return 256;
+    case RF_Q2_K: case RF_Q3_K: case RF_Q4_K: case RF_Q5_K: case RF_Q6_K: return 256;
     case RF_MXFP4: return 17;
     case RF_MXFP6_E2M3: case RF_MXFP6_E3M2: return 25;
     case RF_GGUF_Q4_0: return 18;
@@ -614,6 +702,9 @@ RF_API int rf_dequantize(int type, const uint8_t *data, size_t len, size_t n, fl
     case RF_Q8_0: rf_dequant_q8_0(data, len, n, out); return 0;
     case RF_Q4_K: rf_dequant_q4_k(data, len, n, out); return 0;
     case RF_Q6_K: rf_dequant_q6_k(data, len, n, out); return 0;
+    case RF_Q2_K: rf_dequant_q2_k(data, len, n, out); return 0;
+    case RF_Q3_K: rf_dequant_q3_k(data, len, n, out); return 0;
+    case RF_Q5_K: rf_dequant_q5_k(data, len, n, out); return 0;
     case RF_MXFP4: rf_dequant_mxfp4(data, len, n, out); return 0;
     case RF_MXFP6_E2M3:
     case RF_MXFP6_E3M2: rf_dequant_mxfp6(data, len, n, out); return 0;

@@ -58,6 +58,7 @@ static int check_gemv(const char *who, int fmt, const void *w, size_t w_bytes, b
                       const void *y, int m, int n, int k)
 {
     if (!known_format(fmt)) return fail(RFQ_E_BADARG, "%s: unknown format %d", who, fmt);
+    if (fmt_dequant_only(fmt)) return fail(RFQ_E_UNSUPPORTED, "%s: format %d is decoded by rfq_dequant only", who, fmt);
     if (!w || !x || !y) return fail(RFQ_E_BADARG, "%s: null pointer", who);
     if (m <= 0 || n <= 0 || k <= 0)
         return fail(RFQ_E_BADARG, "%s: dimensions must be positive (m=%d n=%d k=%d)", who, m, n, k);
@@ -117,6 +118,7 @@ int rfq_get_rows(int fmt, const void *d_table, size_t table_bytes, int n_vocab, 
 {
     const bool f32 = fmt == RFQ_TABLE_F32;
     if (!f32 && !known_format(fmt)) return fail(RFQ_E_BADARG, "rfq_get_rows: unknown format %d", fmt);
+    if (fmt_dequant_only(fmt)) return fail(RFQ_E_UNSUPPORTED, "rfq_get_rows: format %d is decoded by rfq_dequant only", fmt);
     if (n_vocab <= 0 || n_embd <= 0 || n_tokens < 0)
         return fail(RFQ_E_BADARG, "rfq_get_rows: n_vocab=%d n_embd=%d n_tokens=%d", n_vocab, n_embd, n_tokens);
     const int be = f32 ? 4 : fmt_block_elems(fmt);
@@ -259,6 +261,7 @@ int rfq_dequant_rms_norm(int fmt, const void *d_packed, size_t packed_bytes, con
                          int seq_len, int hidden_size, float eps, void *stream)
 {
     if (!known_format(fmt)) return fail(RFQ_E_BADARG, "rfq_dequant_rms_norm: unknown format %d", fmt);
+    if (fmt_dequant_only(fmt)) return fail(RFQ_E_UNSUPPORTED, "rfq_dequant_rms_norm: format %d is decoded by rfq_dequant only", fmt);
     if (seq_len < 0 || hidden_size <= 0)
         return fail(RFQ_E_BADARG, "rfq_dequant_rms_norm: seq_len=%d hidden_size=%d", seq_len, hidden_size);
     const size_t need = matrix_bytes(fmt, seq_len > 0 ? seq_len : 1, hidden_size);

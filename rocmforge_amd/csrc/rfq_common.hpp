@@ -14,6 +14,9 @@ template <> struct Fmt<RFQ_Q4_0> { static constexpr int BE = 32, BB = 20; };
 template <> struct Fmt<RFQ_Q8_0> { static constexpr int BE = 32, BB = 36; };
 template <> struct Fmt<RFQ_Q4_K> { static constexpr int BE = 256, BB = 256; };
 template <> struct Fmt<RFQ_Q6_K> { static constexpr int BE = 256, BB = 256; };
+template <> struct Fmt<RFQ_Q2_K> { static constexpr int BE = 256, BB = 256; };
+template <> struct Fmt<RFQ_Q3_K> { static constexpr int BE = 256, BB = 256; };
+template <> struct Fmt<RFQ_Q5_K> { static constexpr int BE = 256, BB = 256; };
 template <> struct Fmt<RFQ_MXFP4> { static constexpr int BE = 32, BB = 17; };
 template <> struct Fmt<RFQ_MXFP6_E2M3> { static constexpr int BE = 32, BB = 25; };
 template <> struct Fmt<RFQ_GGUF_Q4_0> { static constexpr int BE = 32, BB = 18; };
@@ -31,15 +34,18 @@ inline int fmt_block_elems(int fmt)
     case RFQ_Q4_0: case RFQ_Q8_0: case RFQ_MXFP4: case RFQ_MXFP6_E2M3: case RFQ_MXFP6_E3M2: return 32;
     case RFQ_GGUF_Q4_0: case RFQ_GGUF_Q8_0: return 32;
     case RFQ_Q4_K: case RFQ_Q6_K: case RFQ_GGUF_Q4_K: case RFQ_GGUF_Q6_K: return 256;
+    case RFQ_Q2_K: case RFQ_Q3_K: case RFQ_Q5_K: return 256;
     default: return 0;
     }
 }
+// The loader's other K types (src/loader/dequant.rs:150-420): decoded by rfq_dequant*, on no matmul path.
+inline bool fmt_dequant_only(int fmt) { return fmt == RFQ_Q2_K || fmt == RFQ_Q3_K || fmt == RFQ_Q5_K; }
 inline int fmt_block_bytes(int fmt)
 {
     switch (fmt) {
     case RFQ_Q4_0: return 20;
     case RFQ_Q8_0: return 36;
-    case RFQ_Q4_K: case RFQ_Q6_K: return 256;
+    case RFQ_Q4_K: case RFQ_Q6_K: case RFQ_Q2_K: case RFQ_Q3_K: case RFQ_Q5_K: return 256;
     case RFQ_MXFP4: return 17;
     case RFQ_MXFP6_E2M3: case RFQ_MXFP6_E3M2: return 25;
     case RFQ_GGUF_Q4_0: return 18;

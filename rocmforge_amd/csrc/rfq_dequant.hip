@@ -169,6 +169,58 @@ template <> __device__ __forceinline__ float4 decode_quad<RFQ_GGUF_Q6_K>(const u
     return r;
 }
 
+// The loader's other K types (src/loader/dequant.rs): 256-byte blocks of 16 sub-blocks x 16
+// elements, f16 scale at 2 * sub; the codes of a sub-block are an LSB-first bit stream that the
+// reference reads through 16-bit windows.  Four consecutive elements never leave a sub-block.
+
+// dequant_q5_k, src/loader/dequant.rs:150-225: i8 min at 32 + sub, 5-bit codes at 48 + 10 * sub
+template <> __device__ __forceinline__ float4 decode_quad<RFQ_Q5_K>(const uint8_t *blk, int e0)
+{
+    const int sub = e0 >> 4, bit = (e0 & 15) * 5;
+    const float scale = f16_bits_to_f32(ld<uint16_t>(blk + 2 * sub));
+    const float mn = (float)(int8_t)blk[32 + sub];
+    const uint32_t w = ld<uint32_t>(blk + 48 + 10 * sub + (bit >> 3)) >> (bit & 7);   // 20 bits from bit 0 or 4
+    float4 r;
+    r.x = mn + (float)(w & 31u) * scale;
+    r.y = mn + (float)((w >> 5) & 31u) * scale;
+    r.z = mn + (float)((w >> 10) & 31u) * scale;
+    r.w = mn + (float)((w >> 15) & 31u) * scale;
+    return r;
+}
+
+// dequant_q3_k, src/loader/dequant.rs:243-320: two high bits per sub-block at 32 + sub / 4, 3-bit
+// codes at 36 + 6 * sub; high bit i is bit 3 of element i (elements 0 and 1 only); (q - 4) * scale
+template <> __device__ __forceinline__ float4 decode_quad<RFQ_Q3_K>(const uint8_t *blk, int e0)
+{
+    const int sub = e0 >> 4, i0 = e0 & 15, bit = i0 * 3;
+    const float scale = f16_bits_to_f32(ld<uint16_t>(blk + 2 * sub));
+    const uint32_t qh = i0 == 0 ? ((uint32_t)blk[32 + (sub >> 2)] >> ((sub & 3) * 2)) & 3u : 0u;
+    const uint32_t w = ld<uint16_t>(blk + 36 + 6 * sub + (bit >> 3)) >> (bit & 7);    // 12 bits from bit 0 or 4
+    float4 r;
+    r.x = ((float)(int)((w & 7u) | ((qh & 1u) << 3)) - 4.0f) * scale;
+    r.y = ((float)(int)(((w >> 3) & 7u) | ((qh >> 1) << 3)) - 4.0f) * scale;
+    r.z = ((float)(int)((w >> 6) & 7u) - 4.0f) * scale;
+    r.w = ((float)(int)((w >> 9) & 7u) - 4.0f) * scale;
+    return r;
+}
+
+// dequant_q2_k, src/loader/dequant.rs:326-420: f16 min at 32 + 2 * sub, one high bit per sub-block at
+// 64 + sub / 8 (bit 2 of element 0 only), 2-bit codes at 68 + 4 * sub; min + q * scale
+template <> __device__ __forceinline__ float4 decode_quad<RFQ_Q2_K>(const uint8_t *blk, int e0)
+{
+    const int sub = e0 >> 4, i0 = e0 & 15;
+    const float scale = f16_bits_to_f32(ld<uint16_t>(blk + 2 * sub));
+    const float mn = f16_bits_to_f32(ld<uint16_t>(blk + 32 + 2 * sub));
+    const uint32_t qh = i0 == 0 ? ((uint32_t)blk[64 + (sub >> 3)] >> (sub & 7)) & 1u : 0u;
+    const uint32_t w = blk[68 + 4 * sub + (i0 >> 2)];
+    float4 r;
+    r.x = mn + (float)((w & 3u) | (qh << 2)) * scale;
+    r.y = mn + (float)((w >> 2) & 3u) * scale;
+    r.z = mn + (float)((w >> 4) & 3u) * scale;
+    r.w = mn + (float)(w >> 6) * scale;
+    return r;
+}
+
 // 16-byte store of decoded values.  The f32 output is four to eight times the packed input and is
 // written once: non-temporal stores keep it from displacing the input stream in the caches
 // (Q4_K 14336x4096: 53.7 -> 40.7 us, MXFP4 28672x8192: 232 -> 213 us).
@@ -297,6 +349,19 @@ template <> __device__ float decode_checked<RFQ_Q6_K>(const uint8_t *in, size_t 
     int l = (int)(idx & 3);
     return l == 0 ? v.x : l == 1 ? v.y : l == 2 ? v.z : v.w;
 }
+
+// (src/loader/dequant.rs:158-160, 251-253, 334-336: a block the input does not hold completely ends the loop)
+template <int FMT> __device__ float decode_checked_k256(const uint8_t *in, size_t len, size_t idx)
+{
+    size_t off = (idx / 256) * 256;
+    if (off + 256 > len) return 0.0f;
+    float4 v = decode_quad<FMT>(in + off, (int)(idx % 256) & ~3);
+    int l = (int)(idx & 3);
+    return l == 0 ? v.x : l == 1 ? v.y : l == 2 ? v.z : v.w;
+}
+template <> __device__ float decode_checked<RFQ_Q2_K>(const uint8_t *in, size_t len, size_t idx) { return decode_checked_k256<RFQ_Q2_K>(in, len, idx); }
+template <> __device__ float decode_checked<RFQ_Q3_K>(const uint8_t *in, size_t len, size_t idx) { return decode_checked_k256<RFQ_Q3_K>(in, len, idx); }
+template <> __device__ float decode_checked<RFQ_Q5_K>(const uint8_t *in, size_t len, size_t idx) { return decode_checked_k256<RFQ_Q5_K>(in, len, idx); }
 
 template <> __device__ float decode_checked<RFQ_MXFP4>(const uint8_t *in, size_t len, size_t idx)
 {
@@ -560,6 +625,9 @@ int launch_dequant(int fmt, const uint8_t *d_in, size_t in_bytes, float *d_out, 
     case RFQ_Q8_0: return run<RFQ_Q8_0>(d_in, in_bytes, d_out, n, s);
     case RFQ_Q4_K: return run<RFQ_Q4_K>(d_in, in_bytes, d_out, n, s);
     case RFQ_Q6_K: return run<RFQ_Q6_K>(d_in, in_bytes, d_out, n, s);
+    case RFQ_Q2_K: return run<RFQ_Q2_K>(d_in, in_bytes, d_out, n, s);
+    case RFQ_Q3_K: return run<RFQ_Q3_K>(d_in, in_bytes, d_out, n, s);
+    case RFQ_Q5_K: return run<RFQ_Q5_K>(d_in, in_bytes, d_out, n, s);
     case RFQ_MXFP4: return run<RFQ_MXFP4>(d_in, in_bytes, d_out, n, s);
     case RFQ_MXFP6_E2M3: return run<RFQ_MXFP6_E2M3>(d_in, in_bytes, d_out, n, s);
     case RFQ_GGUF_Q4_0: return run<RFQ_GGUF_Q4_0>(d_in, in_bytes, d_out, n, s);

@@ -25,15 +25,18 @@ from __future__ import annotations
 import numpy as np
 
 Q4_0, Q8_0, Q4_K, Q6_K, MXFP4, MXFP6_E2M3, MXFP6_E3M2 = 2, 8, 12, 14, 20, 21, 22
+# the loader's other K types (src/loader/dequant.rs:150-420): dequantisation only
+Q2_K, Q3_K, Q5_K = 10, 11, 13
+DEQUANT_ONLY_FORMATS = (Q2_K, Q3_K, Q5_K)
 # the block layouts of GGUF model files (ggml), which ROCmForge does not decode: 100 + the ggml type id
 GGUF_Q4_0, GGUF_Q8_0, GGUF_Q4_K, GGUF_Q6_K = 102, 108, 112, 114
 GGUF_FORMATS = (GGUF_Q4_0, GGUF_Q8_0, GGUF_Q4_K, GGUF_Q6_K)
 
-BLOCK_ELEMS = {Q4_0: 32, Q8_0: 32, Q4_K: 256, Q6_K: 256, MXFP4: 32, MXFP6_E2M3: 32, MXFP6_E3M2: 32,
+BLOCK_ELEMS = {Q2_K: 256, Q3_K: 256, Q5_K: 256, Q4_0: 32, Q8_0: 32, Q4_K: 256, Q6_K: 256, MXFP4: 32, MXFP6_E2M3: 32, MXFP6_E3M2: 32,
                GGUF_Q4_0: 32, GGUF_Q8_0: 32, GGUF_Q4_K: 256, GGUF_Q6_K: 256}
-BLOCK_BYTES = {Q4_0: 20, Q8_0: 36, Q4_K: 256, Q6_K: 256, MXFP4: 17, MXFP6_E2M3: 25, MXFP6_E3M2: 25,
+BLOCK_BYTES = {Q2_K: 256, Q3_K: 256, Q5_K: 256, Q4_0: 20, Q8_0: 36, Q4_K: 256, Q6_K: 256, MXFP4: 17, MXFP6_E2M3: 25, MXFP6_E3M2: 25,
                GGUF_Q4_0: 18, GGUF_Q8_0: 34, GGUF_Q4_K: 144, GGUF_Q6_K: 210}
-NAMES = {Q4_0: "Q4_0", Q8_0: "Q8_0", Q4_K: "Q4_K", Q6_K: "Q6_K", MXFP4: "MXFP4",
+NAMES = {Q2_K: "Q2_K", Q3_K: "Q3_K", Q5_K: "Q5_K", Q4_0: "Q4_0", Q8_0: "Q8_0", Q4_K: "Q4_K", Q6_K: "Q6_K", MXFP4: "MXFP4",
          MXFP6_E2M3: "MXFP6_E2M3", MXFP6_E3M2: "MXFP6_E3M2",
          GGUF_Q4_0: "GGUF_Q4_0", GGUF_Q8_0: "GGUF_Q8_0", GGUF_Q4_K: "GGUF_Q4_K", GGUF_Q6_K: "GGUF_Q6_K"}
 
@@ -321,9 +324,12 @@ def random_blocks(fmt: int, n_blocks: int, rng: np.random.Generator, exp_range=(
         out[:, 0:4] = s.view(np.uint8).reshape(-1, 4)
     elif fmt == Q4_K:
         return synth_q4_k(n_blocks, rng)
-    elif fmt == Q6_K:
+    elif fmt in (Q6_K, Q3_K, Q5_K):
         s = (rng.standard_normal((n_blocks, 16)) * 0.01).astype(np.float16)
         out[:, 0:32] = s.view(np.uint8).reshape(-1, 32)
+    elif fmt == Q2_K:                                     # f16 scales, then f16 mins
+        s = (rng.standard_normal((n_blocks, 32)) * 0.01).astype(np.float16)
+        out[:, 0:64] = s.view(np.uint8).reshape(-1, 64)
     else:
         out[:, 0] = rng.integers(exp_range[0], exp_range[1] + 1, n_blocks).astype(np.int8).view(np.uint8)
     return out.ravel()

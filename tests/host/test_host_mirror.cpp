@@ -190,8 +190,44 @@ static void test_dequantize_dispatch_f32_f16()
     put_f16(h.data, 0, 0x3C00); put_f16(h.data, 2, 0x4000); put_f16(h.data, 4, 0xC000); put_f16(h.data, 6, 0x0001);
     r = loader::dequantize(h);
     EXPECT(r.ok && r.value[0] == 1.0f && r.value[1] == 2.0f && r.value[2] == -2.0f && r.value[3] == std::ldexp(1.0f, -24));
-    GgufTensor q2("q", TensorShape::from_dims({256}), GgufTensorType::Q2_K, 0);
-    EXPECT(!loader::dequantize(q2).ok);
+}
+// src/loader/dequant.rs:440-665 (Q5_K, Q3_K, Q2_K through the dispatcher)
+static void test_dequantize_other_k_types()
+{
+    auto one_block = [](GgufTensorType t, size_t n) {
+        GgufTensor g("q", TensorShape::from_dims({n}), t, 0);
+        g.data.assign(256, 0);
+        put_f16(g.data, 0, 0x3C00);               // sub-block 0: scale 1.0
+        return g;
+    };
+    GgufTensor q5 = one_block(GgufTensorType::Q5_K, 256);
+    q5.data[48] = 0x01;
+    auto r = loader::dequantize(q5);
+    EXPECT(r.ok && r.value.size() == 256 && r.value[0] == 1.0f && r.value[1] == 0.0f && r.value[15] == 0.0f);
+    GgufTensor q5p = one_block(GgufTensorType::Q5_K, 100);
+    r = loader::dequant_q5_k(q5p);
+    EXPECT(r.ok && r.value.size() == 100 && r.value[0] == 0.0f && r.value[99] == 0.0f);
+    GgufTensor q5m("q", TensorShape::from_dims({512}), GgufTensorType::Q5_K, 0);
+    q5m.data.assign(512, 0);
+    put_f16(q5m.data, 0, 0x3C00); put_f16(q5m.data, 256, 0x4000);
+    q5m.data[256 + 48] = 0xFF; q5m.data[256 + 49] = 0x80;
+    r = loader::dequantize(q5m);
+    EXPECT(r.ok && r.value[0] == 0.0f && r.value[255] == 0.0f && r.value[256] == 62.0f);
+    GgufTensor q3 = one_block(GgufTensorType::Q3_K, 256);
+    r = loader::dequantize(q3);
+    EXPECT(r.ok && r.value[0] == -4.0f && r.value[15] == -4.0f);
+    q3.data[36] = 0x01;
+    r = loader::dequant_q3_k(q3);
+    EXPECT(r.ok && r.value[0] == -3.0f && r.value[1] == -4.0f);
+    GgufTensor q2 = one_block(GgufTensorType::Q2_K, 256);
+    r = loader::dequantize(q2);
+    EXPECT(r.ok && r.value[0] == 0.0f && r.value[15] == 0.0f);
+    q2.data[68] = 0x01;
+    r = loader::dequant_q2_k(q2);
+    EXPECT(r.ok && r.value[0] == 1.0f);
+    GgufTensor q2p = one_block(GgufTensorType::Q2_K, 100);
+    r = loader::dequantize(q2p);
+    EXPECT(r.ok && r.value.size() == 100 && r.value[0] == 0.0f);
 }
 
 // ---- device buffers and matmul ------------------------------------------------------
@@ -466,6 +502,7 @@ int main()
         {"test_dequantize_q4_k_single_block", test_dequantize_q4_k_single_block},
         {"test_dequantize_q4_k_partial_block_and_mins", test_dequantize_q4_k_partial_block_and_mins},
         {"test_dequantize_q6_k_vectors", test_dequantize_q6_k_vectors},
+        {"test_dequantize_other_k_types", test_dequantize_other_k_types},
         {"test_mxfp4_block_of_twos_and_clamp", test_mxfp4_block_of_twos_and_clamp},
         {"test_mxfp6_block_size_clamp_and_last_element", test_mxfp6_block_size_clamp_and_last_element},
         {"test_tensor_types_and_sizes", test_tensor_types_and_sizes},
