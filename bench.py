@@ -236,6 +236,7 @@ def main():
     ap.add_argument("--only-mlp", action="store_true", help="only the SwiGLU MLP line (profiling runs)")
     ap.add_argument("--mlp-steps", type=int, default=300)
     ap.add_argument("--only-gguf", action="store_true", help="only the GGUF-layout Q4_K GEMV line (profiling runs)")
+    ap.add_argument("--only-dequant", action="store_true", help="only the dequantisation lines (profiling runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build is single-GPU (one MI355X per box); run with --gpus 1. "
@@ -252,6 +253,16 @@ def main():
 
     if args.only_mlp:
         print(json.dumps({"Q4_K mlp_swiglu 4096x14336 m1": time_mlp(torch, Q.Q4_K, 4096, 14336, Q, steps=args.mlp_steps)}))
+        return
+
+    if args.only_dequant:
+        res = {}
+        for name, f, n, k, seed in (("Q4_K dequant 14336x4096", Q.Q4_K, N, K, 20260023),
+                                    ("MXFP4 dequant 28672x8192", Q.MXFP4, 28672, 8192, 20260025)):
+            t, b = time_dequant(torch, f, n, k, min(args.steps, 50), min(args.warmup, 5), Q, seed)
+            res[name] = {"GB/s": round(b / t / 1e9, 1), "us": round(t * 1e6, 2), "hbm_frac": round(b / t / 1e9 / HBM_PEAK_GBS, 4),
+                         "algorithmic_bytes": b}
+        print(json.dumps(res))
         return
 
     if args.only_gguf:
@@ -328,11 +339,14 @@ def main():
         also["Q4_K gemv 128256x4096 (LM head)"] = {"GB/s": round(b / (d / 50) / 1e9, 1), "us": round(d / 50 * 1e6, 2),
                                                    "hbm_frac": round(b / (d / 50) / 1e9 / HBM_PEAK_GBS, 4)}
         # the block layouts of GGUF model files (no counterpart in the reference: reported beside, never as its parity)
-        for name, f, n, k, seed in (("GGUF_Q4_K gemv 14336x4096", Q.GGUF_Q4_K, N, K, 20260051),
-                                    ("GGUF_Q6_K gemv 14336x4096", Q.GGUF_Q6_K, N, K, 20260052)):
+        for name, f, n, k, m, seed in (("GGUF_Q4_K gemv 14336x4096", Q.GGUF_Q4_K, N, K, 1, 20260051),
+                                       ("GGUF_Q6_K gemv 14336x4096", Q.GGUF_Q6_K, N, K, 1, 20260052),
+                                       ("GGUF_Q8_0 gemv 4096x4096 m1", Q.GGUF_Q8_0, 4096, 4096, 1, 20260053),
+                                       ("GGUF_Q8_0 gemv 4096x4096 m8", Q.GGUF_Q8_0, 4096, 4096, 8, 20260053),
+                                       ("GGUF_Q4_0 gemv 4864x896", Q.GGUF_Q4_0, 4864, 896, 1, 20260054)):
             c = min(-(-int(2.5 * CACHE_BYTES) // Q.packed_bytes(f, n * k)), 64)
-            _, d, *_ = time_gemv(torch, f, n, k, 1, c, 500, 50, Q, seed)
-            b = algorithmic_bytes(f, n, k, 1, Q)
+            _, d, *_ = time_gemv(torch, f, n, k, m, c, 500, 50, Q, seed)
+            b = algorithmic_bytes(f, n, k, m, Q)
             also[name] = {"GB/s": round(b / (d / 500) / 1e9, 1), "us": round(d / 500 * 1e6, 2),
                           "hbm_frac": round(b / (d / 500) / 1e9 / HBM_PEAK_GBS, 4)}
         also["Q4_K mlp_swiglu 4096x14336 m1"] = time_mlp(torch, Q.Q4_K, 4096, 14336, Q)
