@@ -480,10 +480,10 @@ __device__ __forceinline__ const uint8_t *fused_row(const uint8_t *w, const Gemv
 }
 
 // Results of one group of R rows (res[i] valid in every lane of each of the
-// team's WPR wavefronts) go to y.  `part` is [R][4] floats of LDS; with
+// team's WPR wavefronts) go to y.  `part` is [R][WAVES] floats of LDS; with
 // WPR > 1 every wavefront of the block must call this the same number of times.
-template <int R, int WPR, bool FUSE>
-__device__ __forceinline__ void store_group(const float (&res)[R], float (*part)[4], float *__restrict__ y, int row_first,
+template <int R, int WPR, bool FUSE, int WAVES = 4>
+__device__ __forceinline__ void store_group(const float (&res)[R], float (*part)[WAVES], float *__restrict__ y, int row_first,
                                             int row_end, int lane, int wave, const GemvFuse &f, float rinv)
 {
     const int team = wave / WPR, wit = wave % WPR;
@@ -736,6 +736,67 @@ __device__ __forceinline__ void prep_convert(const float (&xv)[16], int half, ui
     lds_unit[26 + half] = __float_as_uint(half_sum);
 }
 
+// The same conversion with four threads per unit (neighbouring lanes), eight consecutive x each:
+// a quarter is two limb groups in either order, so thread q of a unit writes limb dwords 6q .. 6q+5.
+__device__ __forceinline__ float dpp_xor2_f(float v)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true));
+}
+
+__device__ __forceinline__ void prep_load8(const float *xp, float (&xv)[8])
+{
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        float4 v = ld<float4>(reinterpret_cast<const uint8_t *>(xp + 4 * i));
+        xv[4 * i] = v.x; xv[4 * i + 1] = v.y; xv[4 * i + 2] = v.z; xv[4 * i + 3] = v.w;
+    }
+}
+
+template <bool NIBBLE, uint32_t TOPOFF>
+__device__ __forceinline__ void prep_convert_quarter(const float (&xv)[8], int quarter, uint32_t *lds_unit)
+{
+    float m = 0.f, sum = 0.f;
+    uint32_t top = 0;                                 // largest |x| bit pattern: at or above 0x7F800000 means inf or NaN
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        m = fmaxf(m, fabsf(xv[i]));
+        sum += xv[i];
+        const uint32_t a = __float_as_uint(xv[i]) & 0x7FFFFFFFu;
+        top = a > top ? a : top;
+    }
+    bool bad = top >= 0x7F800000u;
+    m = fmaxf(m, dpp_xor1_f(m));
+    sum += dpp_xor1_f(sum);
+    bad |= __builtin_amdgcn_update_dpp(0, (int)bad, 0xB1, 0xF, 0xF, true) != 0;
+    const float half_sum = sum;
+    m = fmaxf(m, dpp_xor2_f(m));
+    sum += dpp_xor2_f(sum);
+    bad |= __builtin_amdgcn_update_dpp(0, (int)bad, 0x4E, 0xF, 0xF, true) != 0;
+    int e = (int)(__float_as_uint(m) >> 23);          // biased exponent of the largest |x|
+    int ie = 275 - e;                                 // 1/s = 2^(21 - (e - 127))
+    if (ie > 254) ie = 254;
+    float inv_s = __uint_as_float((uint32_t)ie << 23);
+    float sc = ie == 254 ? __uint_as_float(0x00400000u) : __uint_as_float((uint32_t)(254 - ie) << 23);
+    if (bad) sc = __uint_as_float(0x7FC00000u);
+    uint32_t X[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+        X[i] = __float_as_uint(__builtin_fmaf(xv[i], inv_s, 12582912.0f)) - 0x4B400000u + TOPOFF;
+    uint32_t *o = lds_unit + quarter * 6;
+    if (NIBBLE) {
+        limbs4(X[0], X[2], X[4], X[6], o);
+        limbs4(X[1], X[3], X[5], X[7], o + 3);
+    } else {
+        limbs4(X[0], X[1], X[2], X[3], o);
+        limbs4(X[4], X[5], X[6], X[7], o + 3);
+    }
+    if (quarter == 0) {
+        lds_unit[24] = __float_as_uint(sc);
+        lds_unit[25] = __float_as_uint(sum);
+    }
+    if ((quarter & 1) == 0) lds_unit[26 + (quarter >> 1)] = __float_as_uint(half_sum);
+}
+
 // sum_i nibble_i * X_i for 16 weight bytes in low-nibble-first order.
 __device__ __forceinline__ float nib_idot(const U4 &q, const XPrep &xp)
 {
@@ -949,14 +1010,18 @@ __device__ __forceinline__ float idot_pair_of(const IU &u, const XPrep &xe, cons
 // accepts only so many outstanding requests and later loads just block issue.
 // Rows past the end re-read the team's last valid row (a cache hit) and their
 // result is dropped; so do lanes past the end of a row with the last unit.
+// Wavefronts per block of the integer-dot kernel: one block per CU, so that x is converted once per CU and
+// each thread converts a quarter unit.
+constexpr int IDOT_WAVES = 8;
+
 template <int FMT, int UPL, int WPR, int R, bool FUSE>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(64 * IDOT_WAVES)
 gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ y, int n, int k,
                  int groups, GemvFuse f)
 {
     RFQ_TS(0);
     using IU = IUnit<FMT>;
-    constexpr int TEAMS = 4 / WPR, TL = 64 * WPR;
+    constexpr int WAVES = IDOT_WAVES, TEAMS = WAVES / WPR, TL = 64 * WPR, THREADS = 64 * WAVES;
     constexpr int D = R < 3 ? R : 3;
     extern __shared__ __attribute__((aligned(16))) uint32_t xlds[]; // [units][28]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -989,12 +1054,12 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
     const int row_last = row_end > row0 ? row_end - 1 : (n - 1);
 
     // x goes first so that it also returns first.
-    float xv[16], nv[FUSE ? 16 : 1];
-    const bool prep0 = (int)threadIdx.x < 2 * ku;
+    float xv[8], nv[FUSE ? 8 : 1];
+    const bool prep0 = (int)threadIdx.x < 4 * ku;
     const bool norm = FUSE && f.norm_w != nullptr;
-    if (prep0) prep_load(x + (size_t)threadIdx.x * 16, xv);
+    if (prep0) prep_load8(x + (size_t)threadIdx.x * 8, xv);
     if constexpr (FUSE) {
-        if (norm && prep0) prep_load(f.norm_w + (size_t)threadIdx.x * 16, nv);
+        if (norm && prep0) prep_load8(f.norm_w + (size_t)threadIdx.x * 8, nv);
     }
 
     IU buf[D][UPL];
@@ -1013,29 +1078,29 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
     for (int d = 0; d < D; d++) load_row(d, d);
     RFQ_TS(1);
 
-    // Cooperative conversion of x: 2*ku half-units over the 256 threads.
+    // Cooperative conversion of x: 4*ku quarter-units (eight values each) over the block's threads.
     float ssq = 0.f;
     if constexpr (FUSE) {
         if (norm && prep0) {
 #pragma unroll
-            for (int i = 0; i < 16; i++) { ssq = __builtin_fmaf(xv[i], xv[i], ssq); xv[i] *= nv[i]; }
+            for (int i = 0; i < 8; i++) { ssq = __builtin_fmaf(xv[i], xv[i], ssq); xv[i] *= nv[i]; }
         }
     }
-    if (prep0) prep_convert<IU::NIBBLE, IU::TOPOFF>(xv, threadIdx.x & 1, xlds + (size_t)(threadIdx.x >> 1) * 28);
-    for (int h = threadIdx.x + 256; h < 2 * ku; h += 256) {
-        float xw[16];
-        prep_load(x + (size_t)h * 16, xw);
+    if (prep0) prep_convert_quarter<IU::NIBBLE, IU::TOPOFF>(xv, threadIdx.x & 3, xlds + (size_t)(threadIdx.x >> 2) * 28);
+    for (int h = threadIdx.x + THREADS; h < 4 * ku; h += THREADS) {
+        float xw[8];
+        prep_load8(x + (size_t)h * 8, xw);
         if constexpr (FUSE) {
             if (norm) {
-                float nw[16];
-                prep_load(f.norm_w + (size_t)h * 16, nw);
+                float nw[8];
+                prep_load8(f.norm_w + (size_t)h * 8, nw);
 #pragma unroll
-                for (int i = 0; i < 16; i++) { ssq = __builtin_fmaf(xw[i], xw[i], ssq); xw[i] *= nw[i]; }
+                for (int i = 0; i < 8; i++) { ssq = __builtin_fmaf(xw[i], xw[i], ssq); xw[i] *= nw[i]; }
             }
         }
-        prep_convert<IU::NIBBLE, IU::TOPOFF>(xw, h & 1, xlds + (size_t)(h >> 1) * 28);
+        prep_convert_quarter<IU::NIBBLE, IU::TOPOFF>(xw, h & 3, xlds + (size_t)(h >> 2) * 28);
     }
-    __shared__ float ssq_part[4];
+    __shared__ float ssq_part[WAVES];
     if constexpr (FUSE) {
         if (norm) {
             ssq = wave_sum(ssq);
@@ -1046,7 +1111,12 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
     __syncthreads();
     float rinv = 1.0f;
     if constexpr (FUSE) {
-        if (norm) rinv = 1.0f / sqrtf(((ssq_part[0] + ssq_part[1]) + (ssq_part[2] + ssq_part[3])) / (float)k + f.eps);
+        if (norm) {
+            float total = 0.0f;
+#pragma unroll
+            for (int q = 0; q < WAVES; q++) total += ssq_part[q];
+            rinv = 1.0f / sqrtf(total / (float)k + f.eps);
+        }
     }
     XPrep xp[UPL];
 #pragma unroll
@@ -1064,7 +1134,7 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
     }
     RFQ_TS(3);
 
-    __shared__ float part[R][4];
+    __shared__ float part[R][WAVES];
     for (int g = 0; g < groups; g++) {
         const int base = g * R;
         if (g > 0) {
@@ -1090,7 +1160,7 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
         }
         RFQ_TS(4);
         // (`groups` is uniform over the block: every wavefront stores the same number of groups)
-        store_group<R, WPR, FUSE>(res, part, y, row0 + base, row_end, lane, wave, f, rinv);
+        store_group<R, WPR, FUSE, WAVES>(res, part, y, row0 + base, row_end, lane, wave, f, rinv);
     }
 }
 
@@ -1470,7 +1540,7 @@ int launch_idot(const uint8_t *w, const float *x, float *y, int n, int k, int bl
                 hipStream_t s)
 {
     size_t lds = (size_t)(k / 32) * 28 * sizeof(uint32_t);
-    hipLaunchKernelGGL((gemv_idot_kernel<FMT, UPL, WPR, R, FUSE>), dim3(blocks), dim3(256), lds, s, w, x, y, n, k, groups,
+    hipLaunchKernelGGL((gemv_idot_kernel<FMT, UPL, WPR, R, FUSE>), dim3(blocks), dim3(64 * IDOT_WAVES), lds, s, w, x, y, n, k, groups,
                        f);
     RFQ_LAUNCH_CHECK("gemv_idot_kernel");
     return RFQ_OK;
@@ -1480,12 +1550,12 @@ template <int FMT, int UPL, int WPR, bool FUSE>
 int run_idot(const uint8_t *w, const float *x, float *y, int n, int k, const GemvFuse &f, hipStream_t s)
 {
     if constexpr (HasIdot<FMT>::value) {
-        constexpr int TEAMS = 4 / WPR;
-        // Aim at two resident blocks per CU, every team walking the same number
+        constexpr int TEAMS = IDOT_WAVES / WPR;
+        // Aim at eight resident wavefronts per CU, every team walking the same number
         // of rows (a straggler is expensive on a ~10 us kernel).  Rows per team
         // = groups * R with R from a small compiled set; take the pair that
         // wastes the fewest row slots, the larger R on a tie.
-        const int slots = device_cu_count() * 2;
+        const int slots = device_cu_count() * 8 / IDOT_WAVES;
         int want = (n + slots * TEAMS - 1) / (slots * TEAMS);
         if (want < 1) want = 1;
         static const int RS[4] = {2, 4, 7, 8};
