@@ -26,10 +26,26 @@ def weights(fmt, n, k, seed):
     return Q.make_weights(fmt, n, k, seed=seed)
 
 
+def gguf_q4_k_fused(w, n, k):
+    """GGUF Q4_K values as the kernel forms them: (d * sc) * q - dmin * m as ONE fused multiply-add in f32
+    (the float64 expression below is exact, so its f32 rounding is the fused result)."""
+    b = np.frombuffer(bytes(w), np.uint8).reshape(-1, 144)
+    d = b[:, 0:2].copy().view("<f2").astype(np.float32)
+    dmin = b[:, 2:4].copy().view("<f2").astype(np.float32)
+    s = b[:, 4:16].astype(np.uint32)
+    sc = np.concatenate([s[:, 0:4] & 63, (s[:, 8:12] & 15) | ((s[:, 0:4] >> 6) << 4)], axis=1).astype(np.float32)
+    mn = np.concatenate([s[:, 4:8] & 63, (s[:, 8:12] >> 4) | ((s[:, 4:8] >> 6) << 4)], axis=1).astype(np.float32)
+    qs = b[:, 16:].reshape(-1, 4, 32)
+    q = np.stack([qs & 15, qs >> 4], axis=2).reshape(-1, 8, 32).astype(np.float64)
+    d1 = (d * sc).astype(np.float32).astype(np.float64)[:, :, None]
+    m1 = (dmin * mn).astype(np.float32).astype(np.float64)[:, :, None]
+    return (d1 * q - m1).astype(np.float32).reshape(n, k)
+
+
 def rounded_weight_product(oracle, fmt, w, a, n, k):
     """What the kernel is built to compute: the contraction of the weights rounded once to fp16 (float64 sums)."""
-    w16 = oracle.dequantize(fmt, w, n * k).reshape(n, k).astype(np.float16).astype(np.float64)
-    return a.astype(np.float64) @ w16.T
+    w32 = gguf_q4_k_fused(w, n, k) if fmt == Q.GGUF_Q4_K else oracle.dequantize(fmt, w, n * k).reshape(n, k)
+    return a.astype(np.float64) @ w32.astype(np.float16).astype(np.float64).T
 
 
 # The one rounding of each weight to fp16 (the matrix instruction's operand type) is the whole error budget:
