@@ -412,7 +412,7 @@ def test_dispatcher_f32_f16_and_e3m2(oracle):
     d = np.random.default_rng(2).integers(0, 256, 50, dtype=np.uint8); d[0] = 1; d[25] = 255
     assert np.array_equal(oracle.dequantize(21, d, 64), oracle.dequantize(22, d, 64))
     with pytest.raises(ValueError):
-        oracle.dequantize(13, d, 64)
+        oracle.dequantize(3, d, 64)                                   # ids 3, 6, 7 are rejected (src/loader/tensor_type.rs:16-56)
 
 
 def test_cpu_matmul_vectors(oracle):
