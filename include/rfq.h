@@ -124,7 +124,9 @@ RFQ_API size_t rfq_packed_bytes(int fmt, size_t n_elems);
  * Replaces the kernel launches inside dequantize_q4_0_kernel_cached
  * (src/kernels/quant/q4_0.rs:107-153), dequantize_q4_k_gpu_kernel
  * (q4_k.rs:99-148), dequantize_q6_k_gpu_kernel (q6_k.rs:102-149) and the
- * unused mxfp/q8_0 dequant kernels (kernels/mxfp_dequant.hip, q8_0_dequant.hip). */
+ * unused mxfp/q8_0 dequant kernels (kernels/mxfp_dequant.hip, q8_0_dequant.hip);
+ * for Q2_K / Q3_K / Q5_K, the CPU loops dequant_q2_k / q3_k / q5_k
+ * (src/loader/dequant.rs:150-420) that loader::dequantize dispatches to. */
 RFQ_API int rfq_dequant(int fmt, const void *d_packed, size_t packed_bytes, float *d_out, size_t n_elems,
                 void *stream);
 
