@@ -307,7 +307,7 @@ def main():
                    "algorithmic_bytes_per_step": abytes, "weight_copies": copies},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
-                     "kernel": "gemv_idot_kernel<Q4_K,2,1,7>", "avg_launch_us": round(dev_s / args.steps * 1e6, 3),
+                     "kernel": "gemv_idot_kernel<Q4_K,1,2,7>", "avg_launch_us": round(dev_s / args.steps * 1e6, 3),
                      "warm_cache_gbs": round(abytes / (dev_w / args.steps) / 1e9, 1) if dev_w else None},
     }
 
