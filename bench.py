@@ -28,8 +28,8 @@ N, K = 14336, 4096
 CACHE_BYTES = 256 << 20
 # HBM bytes one launch of the headline kernel moves, from FETCH_SIZE / WRITE_SIZE
 # profiler counters scaled by a copy kernel of known size
-# (profiles/gemv_q4k_14336x4096_hbm_counters.txt): 57,615.6 KiB read + 56.0 KiB written.
-MEASURED_TRAFFIC_BYTES = 59055736
+# (profiles/gemv_q4k_14336x4096_hbm_counters.txt): 57,584.4 KiB read + 64.0 KiB written.
+MEASURED_TRAFFIC_BYTES = 59031938
 
 
 def algorithmic_bytes(fmt, n, k, m, Q):
