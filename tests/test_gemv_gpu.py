@@ -156,3 +156,13 @@ def test_gemv_more_than_eight_rows(oracle, cuda):
     got = gpu_gemv(fmt, w, x, n, k, cuda)
     assert got.shape == (m, n)
     assert_close(got, oracle.qmatmul_nk(fmt, w, x, m, n, k), "m=19")
+
+
+@pytest.mark.parametrize("n,k", [(14336, 4096), (14413, 4096), (15001, 2304), (20000, 2560), (14337, 3840)])
+def test_q4_k_long_matrices_one_unit_per_lane(n, k, oracle, cuda):
+    """Q4_K with rows of 65..128 units and at least seven rows per team runs with one unit per lane and two
+    wavefronts per row: ragged row counts, rows that end inside the second wavefront."""
+    w = Q.make_weights(Q.Q4_K, n, k, seed=5300 + n)
+    x = x_for(1, k, 6300 + k)
+    got = gpu_gemv(Q.Q4_K, w, x, n, k, cuda)
+    assert_close(got, oracle.qmatmul_nk(Q.Q4_K, w, x, 1, n, k), f"Q4_K {n}x{k}")
