@@ -549,11 +549,10 @@ gemv_xreg_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
                  int groups, GemvFuse f)
 {
     constexpr int TEAMS = 4 / WPR, TL = 64 * WPR;
-#ifdef RFQ_XREG_D
-    constexpr int D = R < RFQ_XREG_D ? R : RFQ_XREG_D;
-#else
-    constexpr int D = R < 3 ? R : 3;
-#endif
+    // rows in flight per lane: three, or five in the form with one unit per lane and two wavefronts per row
+    // (Q6_K 14336 x 4096 in that form: 14.6 us with three, 13.8 us with five)
+    constexpr int DW = (UPL == 1 && WPR == 2) ? 5 : 3;
+    constexpr int D = R < DW ? R : DW;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int team = wave / WPR, wit = wave % WPR;
     const int tl = wit * 64 + lane;
@@ -1517,7 +1516,9 @@ int launch_xreg(const uint8_t *w, const float *x, float *y, int n, int k, const 
 template <int FMT, int UPL, int WPR, bool FUSE>
 int run_xreg(const uint8_t *w, const float *x, float *y, int n, int k, const GemvFuse &f, hipStream_t s)
 {
-    const RowPlan p = plan_rows(n, 4 / WPR, 2, FUSE && f.glu); // (three blocks per CU fit for Q6_K but run slower)
+    // two blocks of four wavefronts per CU (three fit for Q6_K in the two-units-per-lane form but run slower);
+    // four in the form with one unit per lane and two wavefronts per row, which is light on registers
+    const RowPlan p = plan_rows(n, 4 / WPR, (UPL == 1 && WPR == 2) ? 4 : 2, FUSE && f.glu);
     switch (p.r) {
     case 2: return launch_xreg<FMT, UPL, WPR, 2, FUSE>(w, x, y, n, k, p, f, s);
     case 4: return launch_xreg<FMT, UPL, WPR, 4, FUSE>(w, x, y, n, k, p, f, s);
@@ -1685,6 +1686,11 @@ int run_rows(const uint8_t *w, const float *x, float *y, int n, int k, const Gem
     if (ku <= 64) return run_idot<FMT, 1, 1, FUSE>(w, x, y, n, k, f, s);
     // Q4_K rows of 65..128 units with at least seven rows per team in that form: one unit per lane, two
     // wavefronts per row, sixteen wavefronts per CU (14336 x 4096: 11.67 -> 11.30 us; 4096 rows would lose 6 %)
+    // The float formats likewise (their kernels are bound by instructions and gain most from sixteen wavefronts
+    // per CU: Q6_K 14336 x 4096 16.5 -> 13.8 us).
+    if constexpr (!HasIdot<FMT>::value && !FUSE) {
+        if (ku > 64 && ku <= 128 && n >= device_cu_count() * 56) return run_xreg<FMT, 1, 2, FUSE>(w, x, y, n, k, f, s);
+    }
     // (the plain GEMV only: the fused gate/up form measured slower this way, 22.5 -> 25 us)
     if constexpr (FMT == RFQ_Q4_K && !FUSE) {
         if (ku > 64 && ku <= 128 && n >= device_cu_count() * 56) return run_idot<FMT, 1, 2, FUSE>(w, x, y, n, k, f, s);

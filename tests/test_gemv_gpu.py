@@ -158,11 +158,12 @@ def test_gemv_more_than_eight_rows(oracle, cuda):
     assert_close(got, oracle.qmatmul_nk(fmt, w, x, m, n, k), "m=19")
 
 
+@pytest.mark.parametrize("fmt", [Q.Q4_K, Q.Q6_K, Q.MXFP4, Q.MXFP6_E2M3])
 @pytest.mark.parametrize("n,k", [(14336, 4096), (14413, 4096), (15001, 2304), (20000, 2560), (14337, 3840)])
-def test_q4_k_long_matrices_one_unit_per_lane(n, k, oracle, cuda):
-    """Q4_K with rows of 65..128 units and at least seven rows per team runs with one unit per lane and two
-    wavefronts per row: ragged row counts, rows that end inside the second wavefront."""
-    w = Q.make_weights(Q.Q4_K, n, k, seed=5300 + n)
+def test_long_matrices_one_unit_per_lane(fmt, n, k, oracle, cuda):
+    """Q4_K and the float-path formats with rows of 65..128 units and at least seven rows per team run with one
+    unit per lane and two wavefronts per row: ragged row counts, rows that end inside the second wavefront."""
+    w = Q.make_weights(fmt, n, k, seed=5300 + n + fmt)
     x = x_for(1, k, 6300 + k)
-    got = gpu_gemv(Q.Q4_K, w, x, n, k, cuda)
-    assert_close(got, oracle.qmatmul_nk(Q.Q4_K, w, x, 1, n, k), f"Q4_K {n}x{k}")
+    got = gpu_gemv(fmt, w, x, n, k, cuda)
+    assert_close(got, oracle.qmatmul_nk(fmt, w, x, 1, n, k), f"{Q.NAMES[fmt]} {n}x{k}")
