@@ -1684,7 +1684,7 @@ int run_rows(const uint8_t *w, const float *x, float *y, int n, int k, const Gem
 {
     const int ku = k / 32;
     if (ku <= 64) return run_idot<FMT, 1, 1, FUSE>(w, x, y, n, k, f, s);
-    // Q4_K rows of 65..128 units with at least seven rows per team in that form: one unit per lane, two
+    // Rows of 65..128 units with at least seven rows per team in that form: one unit per lane, two
     // wavefronts per row, sixteen wavefronts per CU (14336 x 4096: 11.67 -> 11.30 us; 4096 rows would lose 6 %)
     // The float formats likewise (their kernels are bound by instructions and gain most from sixteen wavefronts
     // per CU: Q6_K 14336 x 4096 16.5 -> 13.8 us).
@@ -1692,7 +1692,9 @@ int run_rows(const uint8_t *w, const float *x, float *y, int n, int k, const Gem
         if (ku > 64 && ku <= 128 && n >= device_cu_count() * 56) return run_xreg<FMT, 1, 2, FUSE>(w, x, y, n, k, f, s);
     }
     // (the plain GEMV only: the fused gate/up form measured slower this way, 22.5 -> 25 us)
-    if constexpr (FMT == RFQ_Q4_K && !FUSE) {
+    // (all integer-dot formats but the two GGUF K-layouts: GGUF_Q4_K needs two units per lane for its shared
+    // bytes, GGUF_Q6_K measured slower this way, 17.1 -> 17.7 us; Q8_0 13.7 -> 12.9 us, the 4-bit ones 1 %)
+    if constexpr (HasIdot<FMT>::value && FMT != RFQ_GGUF_Q4_K && FMT != RFQ_GGUF_Q6_K && !FUSE) {
         if (ku > 64 && ku <= 128 && n >= device_cu_count() * 56) return run_idot<FMT, 1, 2, FUSE>(w, x, y, n, k, f, s);
     }
     if (ku <= 128) return run_idot<FMT, 2, 1, FUSE>(w, x, y, n, k, f, s);
