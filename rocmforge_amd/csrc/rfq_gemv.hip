@@ -1688,8 +1688,9 @@ int run_rows(const uint8_t *w, const float *x, float *y, int n, int k, const Gem
     // wavefronts per row, sixteen wavefronts per CU (14336 x 4096: 11.67 -> 11.30 us; 4096 rows would lose 6 %)
     // The float formats likewise (their kernels are bound by instructions and gain most from sixteen wavefronts
     // per CU: Q6_K 14336 x 4096 16.5 -> 13.8 us).
+    // (from 32 rows per CU on: Q6_K 11008 x 4096 14.6 -> 11.8 us, 8192 x 4096 the same either way)
     if constexpr (!HasIdot<FMT>::value && !FUSE) {
-        if (ku > 64 && ku <= 128 && n >= device_cu_count() * 56) return run_xreg<FMT, 1, 2, FUSE>(w, x, y, n, k, f, s);
+        if (ku > 64 && ku <= 128 && n >= device_cu_count() * 32) return run_xreg<FMT, 1, 2, FUSE>(w, x, y, n, k, f, s);
     }
     // (the plain GEMV only: the fused gate/up form measured slower this way, 22.5 -> 25 us)
     // (all integer-dot formats but the two GGUF K-layouts: GGUF_Q4_K needs two units per lane for its shared

@@ -159,7 +159,7 @@ def test_gemv_more_than_eight_rows(oracle, cuda):
 
 
 @pytest.mark.parametrize("fmt", [Q.Q4_K, Q.Q6_K, Q.MXFP4, Q.MXFP6_E2M3, Q.Q4_0, Q.Q8_0, Q.GGUF_Q4_0, Q.GGUF_Q8_0])
-@pytest.mark.parametrize("n,k", [(14336, 4096), (14413, 4096), (15001, 2304), (20000, 2560), (14337, 3840)])
+@pytest.mark.parametrize("n,k", [(14336, 4096), (14413, 4096), (15001, 2304), (20000, 2560), (14337, 3840), (8192, 4096), (8201, 2304), (11008, 4096)])
 def test_long_matrices_one_unit_per_lane(fmt, n, k, oracle, cuda):
     """Q4_K and the float-path formats with rows of 65..128 units and at least seven rows per team run with one
     unit per lane and two wavefronts per row: ragged row counts, rows that end inside the second wavefront."""
