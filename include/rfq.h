@@ -61,7 +61,22 @@ typedef enum rfq_format {
     RFQ_GGUF_Q4_0 = 102, /* 18 B / 32: f16 d, 16 bytes (low nibbles = elements 0-15, high = 16-31); d*(q-8) */
     RFQ_GGUF_Q8_0 = 108, /* 34 B / 32: f16 d, 32 int8; d*q                                                 */
     RFQ_GGUF_Q4_K = 112, /* 144 B / 256: f16 d, dmin, 12 B of 6-bit scales/mins, 128 nibble bytes          */
-    RFQ_GGUF_Q6_K = 114  /* 210 B / 256: 128 B low nibbles, 64 B high bit pairs, 16 i8 scales, f16 d       */
+    RFQ_GGUF_Q6_K = 114, /* 210 B / 256: 128 B low nibbles, 64 B high bit pairs, 16 i8 scales, f16 d       */
+    /* The decoders the matmul module carries beside the loader's
+     * (src/kernels/matmul/quantized/; 200 + the id of the format they are a
+     * variant of).  They are what matmul_q8_0 and the *_cpu_fallback paths feed
+     * to the f32 matmul, and they read the same bytes differently from the
+     * formats above.  Accepted by rfq_dequant*, rfq_gemv, rfq_gemv_kn and
+     * rfq_matmul_host_weights*.  (That module's dequantize_q4_0, q4_0.rs:89-134,
+     * is RFQ_Q4_0 itself: same bytes, same arithmetic.) */
+    RFQ_MM_Q8_0 = 208,   /* 36 B / 32: f32 scale + 32 two's-complement int8 bytes; scale * q
+                            (quantized/q8_0.rs:18-56)                                                      */
+    RFQ_MM_Q4_K = 212,   /* 256 B / 256: as RFQ_Q4_K but the nibbles of sub-block sb start at 32 + 20 * sb,
+                            and the f16 scale is widened by f16_to_f32_cpu (quantized/common.rs:44-60,
+                            which reads exponent field 0 as 2^-15 * (1 + m/1024) and field 31 as
+                            2^16 * (1 + m/1024)); min + q * scale (quantized/q4_k.rs:90-148)               */
+    RFQ_MM_Q6_K = 214    /* 256 B / 256: the RFQ_Q6_K stream with the scales widened by f16_to_f32_cpu
+                            (quantized/q6_k.rs:90-148)                                                     */
 } rfq_format;
 /* rfq_get_rows also gathers from a plain f32 table (GgufTensorType F32 = 0). */
 #define RFQ_TABLE_F32 0
@@ -88,11 +103,19 @@ typedef enum rfq_mx_kind { RFQ_MX_AUTO = 0, RFQ_MX_FP4 = 4, RFQ_MX_FP8 = 8, RFQ_
 RFQ_API int rfq_version(void);
 /* Thread-local description of the last failure on this thread ("" if none). */
 RFQ_API const char *rfq_last_error(void);
-/* rfq_gemm_f16 and rfq_gemv (Q8_0, m > 1) keep up to 64 MiB of temporary
- * device memory per stream between calls.  This frees all of it (it waits for
- * the device first), and rfq_upload's pinned staging slots; the next call
- * allocates again.  No counterpart in the reference, whose kernels take no
- * temporaries. */
+/* rfq_gemm_f16, rfq_gemv_kn and rfq_gemv (Q8_0, m > 1) keep up to 64 MiB of
+ * temporary device memory per stream between calls (a stream's first call, or
+ * a larger shape than before, allocates; a larger request replaces the
+ * buffer).  Under stream capture such a call uses the buffer the stream
+ * already has and fails with RFQ_E_UNSUPPORTED if it would have to allocate or
+ * grow: run the call once on the stream before capturing.  A captured graph
+ * holds the buffer's address, so the library never frees a buffer it handed
+ * out during a capture when it grows -- only this function does: it frees
+ * every kept buffer (it waits for the device first) and rfq_upload's pinned
+ * staging slots, and thereby invalidates graphs captured earlier; the next
+ * call allocates again.  Buffers are kept per stream handle: call this after
+ * destroying streams that used the library.  No counterpart in the
+ * reference, whose kernels take no temporaries. */
 RFQ_API int rfq_release_temporaries(void);
 /* Host bytes (pageable: a slice of the memory-mapped model file) -> device
  * memory, in stream order.  The bytes go through a ring of four pinned 8 MiB
@@ -156,11 +179,33 @@ RFQ_API int rfq_dequant_host(int fmt, const uint8_t *h_packed, size_t packed_byt
 RFQ_API int rfq_gemv(int fmt, const void *d_w, size_t w_bytes, const float *d_x, float *d_y, int m, int n,
              int k, void *stream);
 
+/* The other orientation: d_y[m, n] = d_x[m, k] . Wd[k, n], where Wd is the
+ * packed stream decoded as ONE flat array of n * k elements and element
+ * (l, j) is Wd[l * n + j] -- the blocks run along n.  This is what the
+ * reference computes on the bytes it is handed, whatever the doc comments of
+ * its wrappers say about [n_rows, n_cols]: the fused kernel indexes
+ * weight_linear_idx = k_idx * n + col (kernels/q4_0_matmul.hip:207, q4_k_matmul.hip:270, reached
+ * through matmul_q4_0_gpu, src/kernels/matmul/quantized/q4_0.rs:209-260), and
+ * the fallback hands the flat dequantised buffer to the f32 matmul as b[k, n]
+ * (matmul_q4_0_cpu_fallback, q4_0.rs:274-311; cpu_matmul_f32,
+ * src/tensor/matmul.rs:219-233: b[l * n + j]).  The same weight bytes give
+ * different numbers through rfq_gemv (rows of k) and through this call.
+ * n * k a multiple of the block size, w_bytes == n * k / block_elems *
+ * block_bytes, any m >= 1 (one pass over W per row of x).  The sum over l is
+ * split over workgroups in a fixed order (the result does not vary from run
+ * to run); the partial sums live in the temporary memory described at
+ * rfq_release_temporaries (at most 8 MiB). */
+RFQ_API int rfq_gemv_kn(int fmt, const void *d_w, size_t w_bytes, const float *d_x, float *d_y, int m, int n,
+                        int k, void *stream);
+
 /* The reference's raw-pointer launch signatures, argument order
  * (activations, weights, output, m, n, k) as in matmul_q4_0_gpu
  * (src/kernels/matmul/quantized/q4_0.rs:209-217) and the kernels' own
  * parameter lists (kernels/q4_0_matmul.hip:153-160).  The byte size of the
- * weights is implied by n and k. */
+ * weights is implied by n and k.  These read W as [n, k], rows of k -- the
+ * layout the reference documents (q4_0.rs:139-148) -- and are rfq_gemv under
+ * another argument order; what the reference's kernel computes on the same
+ * buffer is rfq_gemv_kn. */
 RFQ_API int rfq_matmul_q4_0(const float *d_act, const uint8_t *d_w, float *d_out, int m, int n, int k, void *stream);
 RFQ_API int rfq_matmul_q8_0(const float *d_act, const uint8_t *d_w, float *d_out, int m, int n, int k, void *stream);
 RFQ_API int rfq_matmul_q4_k(const float *d_act, const uint8_t *d_w, float *d_out, int m, int n, int k, void *stream);
@@ -173,6 +218,14 @@ RFQ_API int rfq_matmul_q6_k(const float *d_act, const uint8_t *d_w, float *d_out
  * q6_k.rs:163-205, q8_0.rs:69-106).  d_out receives n_rows floats. */
 RFQ_API int rfq_matmul_host_weights(int fmt, const uint8_t *h_w, size_t w_bytes, const float *d_input,
                             size_t n_rows, size_t n_cols, float *d_out, void *stream);
+/* The same call in the orientation of rfq_gemv_kn: d_out[j] = sum_l
+ * d_input[l] * Wd[l * n_rows + j], the numbers matmul_q4_0_cpu_fallback
+ * (src/kernels/matmul/quantized/q4_0.rs:274-311, fmt = RFQ_Q4_0) and matmul_q8_0
+ * (quantized/q8_0.rs:69-106, fmt = RFQ_MM_Q8_0) produce: they dequantise on the
+ * CPU (fmt = RFQ_MM_Q4_K / RFQ_MM_Q6_K for that module's K decoders), upload
+ * the f32 array and multiply with m = 1, k = n_cols, n = n_rows. */
+RFQ_API int rfq_matmul_host_weights_kn(int fmt, const uint8_t *h_w, size_t w_bytes, const float *d_input,
+                                       size_t n_rows, size_t n_cols, float *d_out, void *stream);
 
 /* ---- embedding rows ---------------------------------------------------------- */
 

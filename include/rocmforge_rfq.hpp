@@ -411,6 +411,54 @@ inline Status matmul_q4_0_gpu(const HipBackend &b, const float *act, const uint8
     return detail::from_rfq(rfq_matmul_q4_0(act, w, out, (int)m, (int)n, (int)k, b.stream()), "matmul_q4_0_gpu");
 }
 
+// ---- what the reference computes on the bytes (the other orientation, the module's own decoders) ----
+// The wrappers above read W as [n_rows, n_cols], the layout the reference documents
+// (src/kernels/matmul/quantized/q4_0.rs:139-148).  Its code does something else with the same buffer: the fused
+// kernel indexes k_idx * n + col (kernels/q4_0_matmul.hip:207) and the CPU paths hand the flat dequantised array
+// to the f32 matmul as b[k, n] (cpu_matmul_f32, src/tensor/matmul.rs:219-233), so out[j] = sum_l in[l] * Wd[l * n_rows + j].
+// These reproduce those numbers; `layout` selects between the two readings.
+enum class WeightLayout { RowsOfK /* documented */, FlatKN /* computed */ };
+
+// matmul_q4_0_cpu_fallback (src/kernels/matmul/quantized/q4_0.rs:274-311): dequantize_q4_0 (same file, :89-134: the
+// loader's arithmetic), then the f32 matmul with m = 1, k = n_cols, n = n_rows over the flat array.
+inline Status matmul_q4_0_cpu_fallback(const HipBackend &b, const std::vector<uint8_t> &w, const HipBuffer &in,
+                                       size_t n_rows, size_t n_cols, const HipBuffer &out)
+{
+    if (in.size() < n_cols * sizeof(float)) return Status::Err("matmul_q4_0_cpu_fallback: input buffer too small");
+    if (out.size() < n_rows * sizeof(float)) return Status::Err("matmul_q4_0_cpu_fallback: output buffer too small");
+    return detail::from_rfq(rfq_matmul_host_weights_kn(RFQ_Q4_0, w.data(), w.size(), (const float *)in.as_ptr(), n_rows, n_cols,
+                                                       (float *)out.as_ptr(), b.stream()),
+                            "matmul_q4_0_cpu_fallback");
+}
+// The body of matmul_q8_0 as the reference has it (quantized/q8_0.rs:69-106): its own dequantize_q8_0 (:18-56, the
+// bytes as two's-complement int8), then the same f32 matmul over the flat array.
+inline Status matmul_q8_0_as_computed(const HipBackend &b, const std::vector<uint8_t> &w, const HipBuffer &in, size_t n_rows,
+                                      size_t n_cols, const HipBuffer &out)
+{
+    if (in.size() < n_cols * sizeof(float)) return Status::Err("matmul_q8_0: input buffer too small");
+    if (out.size() < n_rows * sizeof(float)) return Status::Err("matmul_q8_0: output buffer too small");
+    return detail::from_rfq(rfq_matmul_host_weights_kn(RFQ_MM_Q8_0, w.data(), w.size(), (const float *)in.as_ptr(), n_rows,
+                                                       n_cols, (float *)out.as_ptr(), b.stream()),
+                            "matmul_q8_0");
+}
+// matmul_q4_0_gpu with the indexing of the kernel it launches (quantized/q4_0.rs:209-260, kernels/q4_0_matmul.hip:207).
+inline Status matmul_q4_0_gpu(const HipBackend &b, const float *act, const uint8_t *w, float *out, size_t m, size_t n,
+                              size_t k, WeightLayout layout)
+{
+    if (layout == WeightLayout::RowsOfK) return matmul_q4_0_gpu(b, act, w, out, m, n, k);
+    return detail::from_rfq(rfq_gemv_kn(RFQ_Q4_0, w, detail::checked_mul(n, k) / 32 * 20, act, out, (int)m, (int)n, (int)k, b.stream()),
+                            "matmul_q4_0_gpu");
+}
+// The module's CPU decoders, evaluated on the GPU (bit-exact): dequantize_q8_0 / dequantize_q4_k / dequantize_q6_k of
+// src/kernels/matmul/quantized/ (q8_0.rs:18-56, q4_k.rs:90-148, q6_k.rs:90-148); dequantize_q4_0 (q4_0.rs:89-134) is
+// loader::dequant_q4_0.
+namespace matmul_quantized {
+inline std::vector<float> dequantize_q4_0(const std::vector<uint8_t> &d, size_t n) { return loader::dequant_q4_0(d, n); }
+inline std::vector<float> dequantize_q8_0(const std::vector<uint8_t> &d, size_t n) { return loader::detail_::through_gpu(RFQ_MM_Q8_0, d.data(), d.size(), n); }
+inline std::vector<float> dequantize_q4_k(const std::vector<uint8_t> &d, size_t n) { return loader::detail_::through_gpu(RFQ_MM_Q4_K, d.data(), d.size(), n); }
+inline std::vector<float> dequantize_q6_k(const std::vector<uint8_t> &d, size_t n) { return loader::detail_::through_gpu(RFQ_MM_Q6_K, d.data(), d.size(), n); }
+} // namespace matmul_quantized
+
 // ---- batch description types (src/ggml/hip_backend/ops/batch_quantized.rs:20-255) --------
 enum class QuantFormat { Q4_0, Q4_K, Q6_K, Q8_0 };
 inline float bytes_per_element(QuantFormat f)

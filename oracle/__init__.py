@@ -15,6 +15,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "librf_oracle.so")
 
 F32, F16, Q4_0, Q8_0, Q4_K, Q6_K, MXFP4, MXFP6_E2M3, MXFP6_E3M2 = 0, 1, 2, 8, 12, 14, 20, 21, 22
+# the decoders of src/kernels/matmul/quantized/ (q8_0.rs:18-56, q4_k.rs:90-148, q6_k.rs:90-148)
+MM_Q8_0, MM_Q4_K, MM_Q6_K = 208, 212, 214
 
 
 def build(force: bool = False) -> str:
@@ -35,7 +37,7 @@ def lib() -> C.CDLL:
             build()
         L = C.CDLL(_SO)
         u8p, f32p, sz = C.c_void_p, C.c_void_p, C.c_size_t
-        for name in ("q4_0", "q8_0", "q4_k", "q6_k", "mxfp4", "mxfp6"):
+        for name in ("q4_0", "q8_0", "q4_k", "q6_k", "mxfp4", "mxfp6", "mm_q8_0", "mm_q4_k", "mm_q6_k"):
             fn = getattr(L, "rf_dequant_" + name)
             fn.argtypes = [u8p, sz, sz, f32p]
             fn.restype = None
@@ -43,6 +45,10 @@ def lib() -> C.CDLL:
         L.rf_dequantize.restype = C.c_int
         L.rf_f16_to_f32.argtypes = [C.c_uint16]
         L.rf_f16_to_f32.restype = C.c_float
+        L.rf_f16_to_f32_mm.argtypes = [C.c_uint16]
+        L.rf_f16_to_f32_mm.restype = C.c_float
+        L.rf_qmatmul_kn.argtypes = [C.c_int, u8p, sz, f32p, sz, sz, sz, f32p, f32p]
+        L.rf_qmatmul_kn.restype = C.c_int
         L.rf_powi_f32.argtypes = [C.c_float, C.c_int]
         L.rf_powi_f32.restype = C.c_float
         for name in ("rf_decode_e2m1", "rf_decode_e2m3"):
@@ -89,7 +95,7 @@ def _p(a: np.ndarray):
 
 
 def block_elems(fmt: int) -> int:
-    return 256 if fmt in (10, 11, Q4_K, 13, Q6_K, 112, 114) else 32
+    return 256 if fmt in (10, 11, Q4_K, 13, Q6_K, 112, 114, MM_Q4_K, MM_Q6_K) else 32
 
 
 def block_bytes(fmt: int) -> int:
@@ -139,6 +145,21 @@ def qmatmul_nk(fmt: int, w_bytes, a: np.ndarray, m: int, n: int, k: int, rows=No
         rc = lib().rf_qmatmul_nk(fmt, _p(w), w.size, _p(a), m, n, k, _p(r), r.size, _p(c))
     if rc != 0:
         raise ValueError(f"rf_qmatmul_nk failed rc={rc}")
+    return c
+
+
+def qmatmul_kn(fmt: int, w_bytes, a: np.ndarray, m: int, n: int, k: int) -> np.ndarray:
+    """c[m, n] = a[m, k] . Wd[k, n] where Wd is the packed stream dequantised as one flat array of n * k
+    elements and read as b[l * n + j]: what matmul_q4_0_cpu_fallback and the fused kernel compute
+    (src/kernels/matmul/quantized/q4_0.rs:274-311, src/tensor/matmul.rs:219-233)."""
+    w = _u8(w_bytes)
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    assert a.size == m * k
+    wd = np.empty(n * k, dtype=np.float32)
+    c = np.empty((m, n), dtype=np.float32)
+    rc = lib().rf_qmatmul_kn(fmt, _p(w), w.size, _p(a), m, n, k, _p(wd), _p(c))
+    if rc != 0:
+        raise ValueError(f"rf_qmatmul_kn failed rc={rc}")
     return c
 
 

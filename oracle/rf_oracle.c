@@ -21,6 +21,18 @@
  *              reference's test properties and an independent float64
  *              evaluation), rf_dequant_rms_norm, rf_mlp_swiglu_q (compositions
  *              of pinned parts, checked against float64)
+ *   pinned   : rf_dequant_mm_q8_0 (the reference's vector at
+ *              src/kernels/matmul/quantized/q8_0.rs:113-131 and an independent
+ *              numpy statement), rf_dequant_mm_q4_k, rf_dequant_mm_q6_k
+ *              (independent whole-array numpy statements on random blocks; the
+ *              canonical decoders on the inputs where the two must agree),
+ *              rf_f16_to_f32_mm for the 61 440 normal binary16 patterns (equals
+ *              IEEE widening), rf_qmatmul_kn (rf_cpu_matmul_f32 on the flat
+ *              dequantised stream; the recipe of quantized/q4_0.rs:343-435)
+ *   parity unpinned (no reference vector; follows from reading the code):
+ *              rf_f16_to_f32_mm for exponent field 0 (zero, subnormals) and 31
+ *              (inf, NaN), where the reference's `exp <= 0` test can never hold
+ *              and the value is 2^(e-15) * (1 + m/1024) for every pattern
  *   parity unpinned (no counterpart in the reference; public ggml layouts):
  *              rf_dequant_gguf_q4_0 / q8_0 / q4_k / q6_k
  *   parity unpinned (no reference vector, reasoned from compiler-rt source):
@@ -458,7 +470,118 @@ RF_API void rf_dequant_mxfp6(const uint8_t *data, size_t len, size_t n, float *o
     }
 }
 
-/* GgufTensorType ids, src/loader/tensor_type.rs:16-32 */
+/* ------------------------------------------------------------------ */
+/* the matmul module's own decoders (src/kernels/matmul/quantized/):    */
+/* what matmul_q8_0 and the *_cpu_fallback paths really compute.  They   */
+/* differ from the canonical decoders above in layout or arithmetic.     */
+/* ------------------------------------------------------------------ */
+
+/* f16_to_f32_cpu, src/kernels/matmul/quantized/common.rs:44-60.  `exp` already
+ * carries the f32 bias (field + 112 >= 112), so the `exp <= 0` branch that
+ * was meant for zero and subnormals is never taken: every pattern decodes as
+ * sign | (field + 112) << 23 | mantissa << 13.  Normal numbers come out
+ * exact; field 0 reads 2^-15 * (1 + m/1024) (0x0000 -> 2^-15), field 31 reads
+ * 2^16 * (1 + m/1024).  The branch is kept as written. */
+RF_API float rf_f16_to_f32_mm(uint16_t bits)
+{
+    uint32_t sign = (bits & 0x8000u) != 0 ? (1u << 31) : 0u;
+    int32_t exp = (int32_t)((bits & 0x7C00u) >> 10) - 15 + 127;
+    uint32_t mant = (uint32_t)(bits & 0x03FFu) << 13;
+    uint32_t out;
+    if (exp <= 0) {
+        if ((bits & 0x7FFFu) == 0) out = sign;
+        else return 0.0f;
+    } else {
+        out = sign | ((uint32_t)exp << 23) | mant;
+    }
+    float f;
+    memcpy(&f, &out, 4);
+    return f;
+}
+
+/* dequantize_q8_0, src/kernels/matmul/quantized/q8_0.rs:18-56: the bytes are
+ * two's-complement int8, value = scale * (byte as i8). */
+RF_API void rf_dequant_mm_q8_0(const uint8_t *data, size_t len, size_t n, float *out)
+{
+    size_t n_blocks = (n + 31) / 32;
+    for (size_t i = 0; i < n; i++) out[i] = 0.0f;
+    for (size_t b = 0; b < n_blocks; b++) {
+        size_t off = b * 36;
+        if (off + 4 > len) break;
+        float scale = rd_f32le(data + off);
+        size_t ds = off + 4, base = b * 32;
+        for (size_t i = 0; i < 32; i++) {
+            size_t idx = ds + i;
+            if (idx >= len) break;
+            size_t e = base + i;
+            if (e < n) out[e] = scale * (float)(int8_t)data[idx];
+        }
+    }
+}
+
+/* dequantize_q4_k, src/kernels/matmul/quantized/q4_k.rs:90-148: the nibbles of
+ * sub-block sb start at 32 + 20 * sb (the canonical decoder strides 28), the
+ * scale goes through rf_f16_to_f32_mm, a super-block needs only its first 32
+ * bytes to be present. */
+RF_API void rf_dequant_mm_q4_k(const uint8_t *data, size_t len, size_t n, float *out)
+{
+    size_t nsb = (n + 255) / 256;
+    for (size_t i = 0; i < n; i++) out[i] = 0.0f;
+    for (size_t s = 0; s < nsb; s++) {
+        size_t so = s * 256;
+        if (so + 32 > len) break;
+        for (size_t sub = 0; sub < 8; sub++) {
+            size_t base = s * 256 + sub * 32;
+            size_t sc_off = so + sub * 2;
+            if (sc_off + 2 > len) break;
+            float scale = rf_f16_to_f32_mm((uint16_t)(data[sc_off] | (data[sc_off + 1] << 8)));
+            size_t mn_off = so + 16 + sub;
+            if (mn_off >= len) break;
+            float mn = (float)(int8_t)data[mn_off];
+            size_t qb = so + 32 + sub * 20;
+            for (size_t i = 0; i < 32; i++) {
+                size_t e = base + i;
+                if (e >= n) break;
+                size_t bit_pos = i * 4, byte_idx = bit_pos / 8;
+                unsigned bit_offset = (unsigned)(bit_pos % 8);
+                size_t qi = qb + byte_idx;
+                if (qi + 1 >= len) break;
+                uint16_t combined = (uint16_t)(((uint16_t)data[qi + 1] << 8) | data[qi]);
+                float quant = (float)((combined >> bit_offset) & 0x0F);
+                out[e] = mn + (quant * scale);
+            }
+        }
+    }
+}
+
+/* dequantize_q6_k, src/kernels/matmul/quantized/q6_k.rs:90-148: the canonical
+ * bit stream, but the scale goes through rf_f16_to_f32_mm and a block needs
+ * only its first 32 bytes to be present. */
+RF_API void rf_dequant_mm_q6_k(const uint8_t *data, size_t len, size_t n, float *out)
+{
+    size_t nb = (n + 255) / 256;
+    for (size_t i = 0; i < n; i++) out[i] = 0.0f;
+    for (size_t b = 0; b < nb; b++) {
+        size_t bo = b * 256;
+        if (bo + 32 > len) break;
+        for (size_t i = 0; i < 256; i++) {
+            size_t e = b * 256 + i;
+            if (e >= n) break;
+            size_t sc_off = bo + (i / 16) * 2;
+            if (sc_off + 2 > len) break;
+            float scale = rf_f16_to_f32_mm((uint16_t)(data[sc_off] | (data[sc_off + 1] << 8)));
+            size_t bit_pos = i * 6, byte_idx = bit_pos / 8;
+            unsigned bit_offset = (unsigned)(bit_pos % 8);
+            size_t qi = bo + 32 + byte_idx;
+            if (qi + 1 >= len) break;
+            uint16_t combined = (uint16_t)(((uint16_t)data[qi + 1] << 8) | data[qi]);
+            int quant = (int)((combined >> bit_offset) & 0x3F);
+            int sv = quant >= 32 ? quant - 64 : quant;
+            out[e] = (float)sv * scale;
+        }
+    }
+}
+
 /* ------------------------------------------------------------------ */
 /* block layouts of GGUF model files (ggml)                            */
 /* ------------------------------------------------------------------ */
@@ -647,10 +770,13 @@ RF_API void rf_dequant_q2_k(const uint8_t *data, size_t len, size_t n, float *ou
     }
 }
 
+/* GgufTensorType ids, src/loader/tensor_type.rs:16-32 */
 enum { RF_F32 = 0, RF_F16 = 1, RF_Q4_0 = 2, RF_Q8_0 = 8, RF_Q2_K = 10, RF_Q3_K = 11, RF_Q4_K = 12, RF_Q5_K = 13, RF_Q6_K = 14,
        RF_MXFP4 = 20, RF_MXFP6_E2M3 = 21, RF_MXFP6_E3M2 = 22,
        /* GGUF file layouts: 100 + the ggml type id */
-       RF_GGUF_Q4_0 = 102, RF_GGUF_Q8_0 = 108, RF_GGUF_Q4_K = 112, RF_GGUF_Q6_K = 114 };
+       RF_GGUF_Q4_0 = 102, RF_GGUF_Q8_0 = 108, RF_GGUF_Q4_K = 112, RF_GGUF_Q6_K = 114,
+       /* the matmul module's decoders: 200 + the id of the format they are a variant of */
+       RF_MM_Q8_0 = 208, RF_MM_Q4_K = 212, RF_MM_Q6_K = 214 };
 
 /* GgufTensor::data_size, src/loader/gguf_tensor.rs:41-75 (Q4_0 is sized
  * 36 bytes per block there although the decoder strides 20). */
@@ -682,6 +808,8 @@ RF_API size_t rf_block_bytes(int type)
     case RF_GGUF_Q8_0: return 34;
     case RF_GGUF_Q4_K: return 144;
     case RF_GGUF_Q6_K: return 210;
+    case RF_MM_Q8_0: return 36;
+    case RF_MM_Q4_K: case RF_MM_Q6_K: return 256;
     default: return 0;
     }
 }
@@ -712,6 +840,9 @@ RF_API int rf_dequantize(int type, const uint8_t *data, size_t len, size_t n, fl
     case RF_GGUF_Q8_0: rf_dequant_gguf_q8_0(data, len, n, out); return 0;
     case RF_GGUF_Q4_K: rf_dequant_gguf_q4_k(data, len, n, out); return 0;
     case RF_GGUF_Q6_K: rf_dequant_gguf_q6_k(data, len, n, out); return 0;
+    case RF_MM_Q8_0: rf_dequant_mm_q8_0(data, len, n, out); return 0;
+    case RF_MM_Q4_K: rf_dequant_mm_q4_k(data, len, n, out); return 0;
+    case RF_MM_Q6_K: rf_dequant_mm_q6_k(data, len, n, out); return 0;
     default: return -1;
     }
 }
@@ -763,7 +894,8 @@ RF_API int rf_qmatmul_nk(int type, const uint8_t *w, size_t w_len, const float *
                          size_t k, const int64_t *rows_sel, size_t n_sel, float *c)
 {
     size_t bb = rf_block_bytes(type);
-    size_t be = (type == RF_Q4_K || type == RF_Q6_K || type == RF_GGUF_Q4_K || type == RF_GGUF_Q6_K) ? 256 : 32;
+    size_t be = (type == RF_Q4_K || type == RF_Q6_K || type == RF_GGUF_Q4_K || type == RF_GGUF_Q6_K || type == RF_MM_Q4_K ||
+                 type == RF_MM_Q6_K) ? 256 : 32;
     if (bb == 0 || k % be != 0) return -1;
     size_t row_bytes = (k / be) * bb;
     if (w_len < row_bytes * n) return -2;
@@ -800,6 +932,34 @@ RF_API int rf_qmatmul_nk_staged(int type, const uint8_t *w, size_t w_len, const 
     int r = rf_dequantize(type, w, w_len, n * k, wd);
     if (r) return r;
     rf_matmul_nk_f32(a, wd, m, n, k, c);
+    return 0;
+}
+
+/* What the reference's quantised matmuls compute on the bytes they are given
+ * (matmul_q4_0_cpu_fallback, src/kernels/matmul/quantized/q4_0.rs:274-311, and
+ * matmul_q8_0, q8_0.rs:69-106; the fused kernel indexes the same way,
+ * kernels/q4_0_matmul.hip: weight_linear_idx = k_idx * n + col): the packed
+ * stream is dequantised as ONE flat array of n * k elements, and that array is
+ * handed to the f32 matmul as b[k, n] (cpu_matmul_f32, src/tensor/matmul.rs:219-233,
+ * b[l * n + j]):  c[i, j] = sum_{l ascending} a[i, l] * Wd[l * n + j].
+ * The blocks therefore run along j.  Each output is the same sequential fp32
+ * sum as rf_cpu_matmul_f32 (the loops are reordered i-l-j for the cache; every
+ * c[i, j] still adds its l terms in ascending order, product rounded first).
+ * wd: n * k floats of scratch. */
+RF_API int rf_qmatmul_kn(int type, const uint8_t *w, size_t w_len, const float *a, size_t m, size_t n, size_t k,
+                         float *wd, float *c)
+{
+    int r = rf_dequantize(type, w, w_len, n * k, wd);
+    if (r) return r;
+    for (size_t i = 0; i < m; i++) {
+        float *ci = c + i * n;
+        for (size_t j = 0; j < n; j++) ci[j] = 0.0f;
+        for (size_t l = 0; l < k; l++) {
+            const float al = a[i * k + l];
+            const float *row = wd + l * n;
+            for (size_t j = 0; j < n; j++) ci[j] += al * row[j];
+        }
+    }
     return 0;
 }
 

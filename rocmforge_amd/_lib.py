@@ -40,11 +40,13 @@ _SIGNATURES = {
     "rfq_dequant_host": ([_i, _vp, _sz, _vp, _sz], _i),
     "rfq_get_rows": ([_i, _vp, _sz, _i, _i, _vp, _i, _vp, _vp, _vp], _i),
     "rfq_gemv": ([_i, _vp, _sz, _vp, _vp, _i, _i, _i, _vp], _i),
+    "rfq_gemv_kn": ([_i, _vp, _sz, _vp, _vp, _i, _i, _i, _vp], _i),
     "rfq_matmul_q4_0": ([_vp, _vp, _vp, _i, _i, _i, _vp], _i),
     "rfq_matmul_q8_0": ([_vp, _vp, _vp, _i, _i, _i, _vp], _i),
     "rfq_matmul_q4_k": ([_vp, _vp, _vp, _i, _i, _i, _vp], _i),
     "rfq_matmul_q6_k": ([_vp, _vp, _vp, _i, _i, _i, _vp], _i),
     "rfq_matmul_host_weights": ([_i, _vp, _sz, _vp, _sz, _sz, _vp, _vp], _i),
+    "rfq_matmul_host_weights_kn": ([_i, _vp, _sz, _vp, _sz, _sz, _vp, _vp], _i),
     "rfq_rms_norm": ([_vp, _vp, _vp, _i, _i, C.c_float, _vp], _i),
     "rfq_swiglu": ([_vp, _vp, _vp, _i, _i, _vp], _i),
     "rfq_dequant_rms_norm": ([_i, _vp, _sz, _vp, _vp, _i, _i, C.c_float, _vp], _i),

@@ -55,10 +55,12 @@ static size_t matrix_bytes(int fmt, int n, int k)
 }
 
 static int check_gemv(const char *who, int fmt, const void *w, size_t w_bytes, bool have_bytes, const void *x,
-                      const void *y, int m, int n, int k)
+                      const void *y, int m, int n, int k, bool mm_ok = false)
 {
     if (!known_format(fmt)) return fail(RFQ_E_BADARG, "%s: unknown format %d", who, fmt);
     if (fmt_dequant_only(fmt)) return fail(RFQ_E_UNSUPPORTED, "%s: format %d is decoded by rfq_dequant only", who, fmt);
+    if (fmt_mm_variant(fmt) && !mm_ok)
+        return fail(RFQ_E_UNSUPPORTED, "%s: format %d (a decoder of the matmul module) is taken by rfq_dequant*, rfq_gemv, rfq_gemv_kn and rfq_matmul_host_weights* only", who, fmt);
     if (!w || !x || !y) return fail(RFQ_E_BADARG, "%s: null pointer", who);
     if (m <= 0 || n <= 0 || k <= 0)
         return fail(RFQ_E_BADARG, "%s: dimensions must be positive (m=%d n=%d k=%d)", who, m, n, k);
@@ -118,7 +120,8 @@ int rfq_get_rows(int fmt, const void *d_table, size_t table_bytes, int n_vocab, 
 {
     const bool f32 = fmt == RFQ_TABLE_F32;
     if (!f32 && !known_format(fmt)) return fail(RFQ_E_BADARG, "rfq_get_rows: unknown format %d", fmt);
-    if (fmt_dequant_only(fmt)) return fail(RFQ_E_UNSUPPORTED, "rfq_get_rows: format %d is decoded by rfq_dequant only", fmt);
+    if (fmt_dequant_only(fmt) || fmt_mm_variant(fmt))
+        return fail(RFQ_E_UNSUPPORTED, "rfq_get_rows: format %d is decoded by rfq_dequant only", fmt);
     if (n_vocab <= 0 || n_embd <= 0 || n_tokens < 0)
         return fail(RFQ_E_BADARG, "rfq_get_rows: n_vocab=%d n_embd=%d n_tokens=%d", n_vocab, n_embd, n_tokens);
     const int be = f32 ? 4 : fmt_block_elems(fmt);
@@ -177,7 +180,7 @@ int rfq_dequant_host(int fmt, const uint8_t *h_packed, size_t packed_bytes, floa
 int rfq_gemv(int fmt, const void *d_w, size_t w_bytes, const float *d_x, float *d_y, int m, int n, int k,
              void *stream)
 {
-    int rc = check_gemv("rfq_gemv", fmt, d_w, w_bytes, true, d_x, d_y, m, n, k);
+    int rc = check_gemv("rfq_gemv", fmt, d_w, w_bytes, true, d_x, d_y, m, n, k, true);
     if (rc != RFQ_OK) return rc;
     for (int r0 = 0; r0 < m; r0 += 8) {                 // the decode kernels take up to eight rows of x per launch
         const int rows = m - r0 < 8 ? m - r0 : 8;
@@ -218,13 +221,61 @@ int rfq_matmul_host_weights(int fmt, const uint8_t *h_w, size_t w_bytes, const f
 {
     if (n_rows == 0 || n_cols == 0 || n_rows > 0x7fffffffu || n_cols > 0x7fffffffu)
         return fail(RFQ_E_BADARG, "rfq_matmul_host_weights: bad shape %zu x %zu", n_rows, n_cols);
-    int rc = check_gemv("rfq_matmul_host_weights", fmt, h_w, w_bytes, true, d_input, d_out, 1, (int)n_rows, (int)n_cols);
+    int rc = check_gemv("rfq_matmul_host_weights", fmt, h_w, w_bytes, true, d_input, d_out, 1, (int)n_rows, (int)n_cols, true);
     if (rc != RFQ_OK) return rc;
     hipStream_t s = (hipStream_t)stream;
     void *d_w = nullptr;
     RFQ_HIP(hipMalloc(&d_w, w_bytes));
     if (int up = upload_bytes(h_w, w_bytes, d_w, s)) { (void)hipStreamSynchronize(s); (void)hipFree(d_w); return up; }
     rc = launch_gemv(fmt, (const uint8_t *)d_w, d_input, d_out, 1, (int)n_rows, (int)n_cols, s);
+    hipError_t e = hipStreamSynchronize(s);
+    (void)hipFree(d_w);
+    if (rc != RFQ_OK) return rc;
+    if (e != hipSuccess) return hip_fail(e, "hipStreamSynchronize");
+    return RFQ_OK;
+}
+
+// Shape and size checks of the flat-stream orientation: n * k elements in whole blocks.
+static int check_gemv_kn(const char *who, int fmt, const void *w, size_t w_bytes, const void *x, const void *y, int m,
+                         int n, int k)
+{
+    if (!known_format(fmt)) return fail(RFQ_E_BADARG, "%s: unknown format %d", who, fmt);
+    if (fmt_dequant_only(fmt)) return fail(RFQ_E_UNSUPPORTED, "%s: format %d is decoded by rfq_dequant only", who, fmt);
+    if (!w || !x || !y) return fail(RFQ_E_BADARG, "%s: null pointer", who);
+    if (m <= 0 || n <= 0 || k <= 0)
+        return fail(RFQ_E_BADARG, "%s: dimensions must be positive (m=%d n=%d k=%d)", who, m, n, k);
+    const size_t elems = (size_t)n * (size_t)k, be = (size_t)fmt_block_elems(fmt);
+    if (elems % be != 0)
+        return fail(RFQ_E_SIZE, "%s: n * k = %zu is not a multiple of the %zu-element block", who, elems, be);
+    const size_t need = elems / be * (size_t)fmt_block_bytes(fmt);
+    if (w_bytes != need)
+        return fail(RFQ_E_SIZE, "%s: weight buffer has %zu bytes, %d x %d elements need %zu", who, w_bytes, k, n, need);
+    return RFQ_OK;
+}
+
+int rfq_gemv_kn(int fmt, const void *d_w, size_t w_bytes, const float *d_x, float *d_y, int m, int n, int k, void *stream)
+{
+    int rc = check_gemv_kn("rfq_gemv_kn", fmt, d_w, w_bytes, d_x, d_y, m, n, k);
+    if (rc != RFQ_OK) return rc;
+    for (int i = 0; i < m; i++) {
+        rc = launch_gemv_kn(fmt, (const uint8_t *)d_w, d_x + (size_t)i * k, d_y + (size_t)i * n, n, k, (hipStream_t)stream);
+        if (rc != RFQ_OK) return rc;
+    }
+    return RFQ_OK;
+}
+
+int rfq_matmul_host_weights_kn(int fmt, const uint8_t *h_w, size_t w_bytes, const float *d_input, size_t n_rows,
+                               size_t n_cols, float *d_out, void *stream)
+{
+    if (n_rows == 0 || n_cols == 0 || n_rows > 0x7fffffffu || n_cols > 0x7fffffffu)
+        return fail(RFQ_E_BADARG, "rfq_matmul_host_weights_kn: bad shape %zu x %zu", n_rows, n_cols);
+    int rc = check_gemv_kn("rfq_matmul_host_weights_kn", fmt, h_w, w_bytes, d_input, d_out, 1, (int)n_rows, (int)n_cols);
+    if (rc != RFQ_OK) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    void *d_w = nullptr;
+    RFQ_HIP(hipMalloc(&d_w, w_bytes));
+    if (int up = upload_bytes(h_w, w_bytes, d_w, s)) { (void)hipStreamSynchronize(s); (void)hipFree(d_w); return up; }
+    rc = launch_gemv_kn(fmt, (const uint8_t *)d_w, d_input, d_out, (int)n_rows, (int)n_cols, s);
     hipError_t e = hipStreamSynchronize(s);
     (void)hipFree(d_w);
     if (rc != RFQ_OK) return rc;
@@ -261,7 +312,8 @@ int rfq_dequant_rms_norm(int fmt, const void *d_packed, size_t packed_bytes, con
                          int seq_len, int hidden_size, float eps, void *stream)
 {
     if (!known_format(fmt)) return fail(RFQ_E_BADARG, "rfq_dequant_rms_norm: unknown format %d", fmt);
-    if (fmt_dequant_only(fmt)) return fail(RFQ_E_UNSUPPORTED, "rfq_dequant_rms_norm: format %d is decoded by rfq_dequant only", fmt);
+    if (fmt_dequant_only(fmt) || fmt_mm_variant(fmt))
+        return fail(RFQ_E_UNSUPPORTED, "rfq_dequant_rms_norm: format %d is decoded by rfq_dequant only", fmt);
     if (seq_len < 0 || hidden_size <= 0)
         return fail(RFQ_E_BADARG, "rfq_dequant_rms_norm: seq_len=%d hidden_size=%d", seq_len, hidden_size);
     const size_t need = matrix_bytes(fmt, seq_len > 0 ? seq_len : 1, hidden_size);

@@ -23,6 +23,9 @@ template <> struct Fmt<RFQ_GGUF_Q4_0> { static constexpr int BE = 32, BB = 18; }
 template <> struct Fmt<RFQ_GGUF_Q8_0> { static constexpr int BE = 32, BB = 34; };
 template <> struct Fmt<RFQ_GGUF_Q4_K> { static constexpr int BE = 256, BB = 144; };
 template <> struct Fmt<RFQ_GGUF_Q6_K> { static constexpr int BE = 256, BB = 210; };
+template <> struct Fmt<RFQ_MM_Q8_0> { static constexpr int BE = 32, BB = 36; };
+template <> struct Fmt<RFQ_MM_Q4_K> { static constexpr int BE = 256, BB = 256; };
+template <> struct Fmt<RFQ_MM_Q6_K> { static constexpr int BE = 256, BB = 256; };
 
 // MXFP6_E3M2 is decoded exactly like E2M3 by the reference
 // (src/loader/dequant.rs:693), so it shares every kernel.
@@ -32,20 +35,22 @@ inline int fmt_block_elems(int fmt)
 {
     switch (fmt) {
     case RFQ_Q4_0: case RFQ_Q8_0: case RFQ_MXFP4: case RFQ_MXFP6_E2M3: case RFQ_MXFP6_E3M2: return 32;
-    case RFQ_GGUF_Q4_0: case RFQ_GGUF_Q8_0: return 32;
-    case RFQ_Q4_K: case RFQ_Q6_K: case RFQ_GGUF_Q4_K: case RFQ_GGUF_Q6_K: return 256;
+    case RFQ_GGUF_Q4_0: case RFQ_GGUF_Q8_0: case RFQ_MM_Q8_0: return 32;
+    case RFQ_Q4_K: case RFQ_Q6_K: case RFQ_GGUF_Q4_K: case RFQ_GGUF_Q6_K: case RFQ_MM_Q4_K: case RFQ_MM_Q6_K: return 256;
     case RFQ_Q2_K: case RFQ_Q3_K: case RFQ_Q5_K: return 256;
     default: return 0;
     }
 }
 // The loader's other K types (src/loader/dequant.rs:150-420): decoded by rfq_dequant*, on no matmul path.
 inline bool fmt_dequant_only(int fmt) { return fmt == RFQ_Q2_K || fmt == RFQ_Q3_K || fmt == RFQ_Q5_K; }
+// The matmul module's own decoders (src/kernels/matmul/quantized/): dequantisation and the two GEMV orientations.
+inline bool fmt_mm_variant(int fmt) { return fmt == RFQ_MM_Q8_0 || fmt == RFQ_MM_Q4_K || fmt == RFQ_MM_Q6_K; }
 inline int fmt_block_bytes(int fmt)
 {
     switch (fmt) {
     case RFQ_Q4_0: return 20;
-    case RFQ_Q8_0: return 36;
-    case RFQ_Q4_K: case RFQ_Q6_K: case RFQ_Q2_K: case RFQ_Q3_K: case RFQ_Q5_K: return 256;
+    case RFQ_Q8_0: case RFQ_MM_Q8_0: return 36;
+    case RFQ_Q4_K: case RFQ_Q6_K: case RFQ_Q2_K: case RFQ_Q3_K: case RFQ_Q5_K: case RFQ_MM_Q4_K: case RFQ_MM_Q6_K: return 256;
     case RFQ_MXFP4: return 17;
     case RFQ_MXFP6_E2M3: case RFQ_MXFP6_E3M2: return 25;
     case RFQ_GGUF_Q4_0: return 18;
@@ -90,6 +95,8 @@ int launch_rms_norm(int src_fmt, const void *d_x, const float *d_weight, float *
                     hipStream_t s);
 int launch_swiglu(const float *d_gate, const float *d_up, float *d_out, size_t total, hipStream_t s);
 int launch_gemv(int fmt, const uint8_t *d_w, const float *d_x, float *d_y, int m, int n, int k, hipStream_t s);
+// y[n] = sum_l x[l] * Wd[l * n + j] over the flat stream of n * k elements (one row of x).
+int launch_gemv_kn(int fmt, const uint8_t *d_w, const float *d_x, float *d_y, int n, int k, hipStream_t s);
 int launch_gemv_fused(int fmt, const uint8_t *d_w, const uint8_t *d_w2, const float *d_x, const float *d_norm_w,
                       float eps, float *d_y, int n, int k, hipStream_t s);
 int launch_gemm_f16(int fmt, const uint8_t *d_w, const void *d_a, void *d_out, int out_dtype, int m, int n,
@@ -161,6 +168,15 @@ __device__ __forceinline__ uint32_t gguf_scale_min_k4(int j, uint32_t s0, uint32
     const uint32_t mn2 = c < 2 ? (b & 0x3F3Fu) : (((cc >> 4) & 0x0F0Fu) | ((b >> 2) & 0x3030u));
     const int hs = 8 * (j & 1);
     return ((sc2 >> hs) & 255u) | (((mn2 >> hs) & 255u) << 8);
+}
+
+// f16_to_f32_cpu of the matmul module (src/kernels/matmul/quantized/common.rs:44-60): its test for zero and
+// subnormals compares the already re-biased exponent with 0 and never holds, so every pattern widens as
+// sign | (field + 112) << 23 | mantissa << 13 (exact for normal numbers only).
+__device__ __forceinline__ float f16_bits_to_f32_mm(uint16_t h)
+{
+    const uint32_t b = h;
+    return __uint_as_float(((b & 0x8000u) << 16) | ((((b >> 10) & 31u) + 112u) << 23) | ((b & 0x3FFu) << 13));
 }
 
 // Signed 6-bit field (two's complement) starting at bit `off` of w.

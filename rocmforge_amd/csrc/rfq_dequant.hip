@@ -169,6 +169,50 @@ template <> __device__ __forceinline__ float4 decode_quad<RFQ_GGUF_Q6_K>(const u
     return r;
 }
 
+// ---- the matmul module's own decoders (src/kernels/matmul/quantized/) -------------
+
+// quantized/q8_0.rs:34-52: two's-complement bytes, scale * q
+template <> __device__ __forceinline__ float4 decode_quad<RFQ_MM_Q8_0>(const uint8_t *blk, int e0)
+{
+    float scale = ld<float>(blk);
+    uint32_t w = ld<uint32_t>(blk + 4 + e0);
+    float4 r;
+    r.x = scale * (float)(int8_t)(w & 255u);
+    r.y = scale * (float)(int8_t)((w >> 8) & 255u);
+    r.z = scale * (float)(int8_t)((w >> 16) & 255u);
+    r.w = scale * (float)(int8_t)(w >> 24);
+    return r;
+}
+
+// quantized/q4_k.rs:101-143: nibbles of sub-block sb at 32 + 20 * sb, scale through f16_to_f32_cpu
+template <> __device__ __forceinline__ float4 decode_quad<RFQ_MM_Q4_K>(const uint8_t *blk, int e0)
+{
+    int sb = e0 >> 5, i = e0 & 31;
+    float scale = f16_bits_to_f32_mm(ld<uint16_t>(blk + 2 * sb));
+    float mn = (float)(int8_t)blk[16 + sb];
+    uint32_t w = ld<uint16_t>(blk + 32 + 20 * sb + (i >> 1));
+    float4 r;
+    r.x = mn + (float)(w & 15u) * scale;
+    r.y = mn + (float)((w >> 4) & 15u) * scale;
+    r.z = mn + (float)((w >> 8) & 15u) * scale;
+    r.w = mn + (float)((w >> 12) & 15u) * scale;
+    return r;
+}
+
+// quantized/q6_k.rs:101-143: the canonical stream, scale through f16_to_f32_cpu
+template <> __device__ __forceinline__ float4 decode_quad<RFQ_MM_Q6_K>(const uint8_t *blk, int e0)
+{
+    float scale = f16_bits_to_f32_mm(ld<uint16_t>(blk + 2 * (e0 >> 4)));
+    const uint8_t *p = blk + 32 + 3 * (e0 >> 2);
+    uint32_t w = (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16);
+    float4 r;
+    r.x = (float)sbfe6(w, 0) * scale;
+    r.y = (float)sbfe6(w, 6) * scale;
+    r.z = (float)sbfe6(w, 12) * scale;
+    r.w = (float)sbfe6(w, 18) * scale;
+    return r;
+}
+
 // The loader's other K types (src/loader/dequant.rs): 256-byte blocks of 16 sub-blocks x 16
 // elements, f16 scale at 2 * sub; the codes of a sub-block are an LSB-first bit stream that the
 // reference reads through 16-bit windows.  Four consecutive elements never leave a sub-block.
@@ -389,6 +433,41 @@ template <> __device__ float decode_checked<RFQ_MXFP6_E2M3>(const uint8_t *in, s
     return clampf(mx_scale((int)(int8_t)in[off]) * decode_e2m3(q), -7.5f, 7.5f);
 }
 
+// The matmul module's decoders reach into an incomplete last block as far as its bytes go.
+template <> __device__ float decode_checked<RFQ_MM_Q8_0>(const uint8_t *in, size_t len, size_t idx)
+{
+    size_t off = (idx / 32) * 36;
+    if (off + 4 > len) return 0.0f;             // quantized/q8_0.rs:24-26
+    size_t p = off + 4 + idx % 32;
+    if (p >= len) return 0.0f;                  // q8_0.rs:42-44
+    return ld<float>(in + off) * (float)(int8_t)in[p];
+}
+
+template <> __device__ float decode_checked<RFQ_MM_Q4_K>(const uint8_t *in, size_t len, size_t idx)
+{
+    size_t off = (idx / 256) * 256;
+    if (off + 32 > len) return 0.0f;            // quantized/q4_k.rs:96-98 (scales and mins are then present)
+    int e = (int)(idx % 256), sb = e >> 5, i = e & 31;
+    size_t qi = off + 32 + 20 * sb + (i >> 1);
+    if (qi + 1 >= len) return 0.0f;             // q4_k.rs:135-137
+    uint32_t q = (i & 1) ? (in[qi] >> 4) : (in[qi] & 15u);
+    float scale = f16_bits_to_f32_mm(ld<uint16_t>(in + off + 2 * sb));
+    return (float)(int8_t)in[off + 16 + sb] + (float)q * scale;
+}
+
+template <> __device__ float decode_checked<RFQ_MM_Q6_K>(const uint8_t *in, size_t len, size_t idx)
+{
+    size_t off = (idx / 256) * 256;
+    if (off + 32 > len) return 0.0f;            // quantized/q6_k.rs:96-98
+    int i = (int)(idx % 256);
+    size_t qi = off + 32 + (size_t)(i * 6) / 8;
+    if (qi + 1 >= len) return 0.0f;             // q6_k.rs:128-130
+    uint32_t combined = (uint32_t)in[qi] | ((uint32_t)in[qi + 1] << 8);
+    int q = (int)((combined >> ((i * 6) % 8)) & 63u);
+    float scale = f16_bits_to_f32_mm(ld<uint16_t>(in + off + 2 * (i >> 4)));
+    return (float)(q >= 32 ? q - 64 : q) * scale;
+}
+
 // GGUF layouts: a block the input does not hold completely decodes to 0.0.
 template <int FMT> __device__ float decode_checked_whole_blocks(const uint8_t *in, size_t len, size_t idx)
 {
@@ -503,9 +582,97 @@ int run(const uint8_t *d_in, size_t in_bytes, float *d_out, size_t n, hipStream_
         size_t grid = (n - first + 255) / 256;
         if (grid > 0x7fffffffu) return fail(RFQ_E_SIZE, "rfq_dequant: ragged tail of %zu elements exceeds one launch", n - first);
         // (GGUF layouts decode whole blocks only: everything past the last whole block is 0.0)
-        const size_t reach = FMT >= RFQ_GGUF_Q4_0 ? full * BB : in_bytes;
+        const size_t reach = (FMT >= RFQ_GGUF_Q4_0 && FMT < RFQ_MM_Q8_0) ? full * BB : in_bytes;
         hipLaunchKernelGGL((dequant_checked_kernel<FMT>), dim3((unsigned)grid), dim3(256), 0, s, d_in, reach, d_out, first, n);
         RFQ_LAUNCH_CHECK("dequant_checked_kernel");
+    }
+    return RFQ_OK;
+}
+
+// ---- the orientation the reference computes: y[j] = sum_l x[l] * Wd[l * n + j] -----------
+//
+// Wd is the packed stream decoded as one flat array of n * k elements (blocks run along j):
+// kernels/q4_0_matmul.hip:207 (weight_linear_idx = k_idx * n + col) and
+// matmul_q4_0_cpu_fallback + cpu_matmul_f32 (src/kernels/matmul/quantized/q4_0.rs:274-311,
+// src/tensor/matmul.rs:219-233).  A thread owns VEC consecutive columns (4 when n is a multiple of 4: a
+// decoded quad never straddles two rows of Wd then; else 1) and walks the rows l of its split, so a
+// wavefront reads consecutive bytes of one row of Wd per step and the stream is read once.  The k rows are
+// split over blockIdx.y; split s writes its partial sums to part[s * n + j], and a second kernel adds the
+// splits in ascending order (fixed summation order: the result does not change from run to run).
+template <int FMT, int VEC>
+__global__ void __launch_bounds__(256)
+gemv_kn_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ part, int n, int k,
+               int rows_per_split)
+{
+    constexpr size_t BE = Fmt<FMT>::BE, BB = Fmt<FMT>::BB;
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    const int groups = VEC == 4 ? n / 4 : n;
+    if (c >= groups) return;
+    const int l0 = blockIdx.y * rows_per_split;
+    int l1 = l0 + rows_per_split;
+    if (l1 > k) l1 = k;
+    float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    size_t e = (size_t)l0 * n + (size_t)c * VEC;
+#pragma unroll 4
+    for (int l = l0; l < l1; l++, e += n) {
+        const int eo = (int)(e % BE);
+        const float4 v = decode_quad<FMT>(w + (e / BE) * BB, eo & ~3);
+        const float xl = x[l];
+        if (VEC == 4) {
+            acc.x = __builtin_fmaf(xl, v.x, acc.x);
+            acc.y = __builtin_fmaf(xl, v.y, acc.y);
+            acc.z = __builtin_fmaf(xl, v.z, acc.z);
+            acc.w = __builtin_fmaf(xl, v.w, acc.w);
+        } else {
+            const int r = eo & 3;
+            acc.x = __builtin_fmaf(xl, r == 0 ? v.x : (r == 1 ? v.y : (r == 2 ? v.z : v.w)), acc.x);
+        }
+    }
+    float *o = part + (size_t)blockIdx.y * n + (size_t)c * VEC;
+    o[0] = acc.x;
+    if (VEC == 4) { o[1] = acc.y; o[2] = acc.z; o[3] = acc.w; }
+}
+
+__global__ void __launch_bounds__(256)
+gemv_kn_reduce_kernel(const float *__restrict__ part, float *__restrict__ y, int n, int splits)
+{
+    const int j = blockIdx.x * 256 + threadIdx.x;
+    if (j >= n) return;
+    float sum = 0.0f;
+    for (int s = 0; s < splits; s++) sum += part[(size_t)s * n + j];
+    y[j] = sum;
+}
+
+constexpr size_t KN_PART_MAX = (size_t)8 << 20;   // bytes of partial sums at most
+
+template <int FMT>
+int run_gemv_kn(const uint8_t *w, const float *x, float *y, int n, int k, hipStream_t s)
+{
+    const bool vec = n % 4 == 0;
+    const int groups = vec ? n / 4 : n;
+    const int bx = (groups + 255) / 256;
+    // about four workgroups per CU, at least 16 rows per split, partial sums within KN_PART_MAX
+    int splits = (4 * device_cu_count() + bx - 1) / bx;
+    if (splits > k / 16) splits = k / 16;
+    const size_t by_bytes = KN_PART_MAX / ((size_t)n * 4);
+    if ((size_t)splits > by_bytes) splits = (int)by_bytes;
+    if (splits < 1) splits = 1;
+    if (splits > 65535) splits = 65535;
+    const int rows_per_split = (k + splits - 1) / splits;
+    splits = (k + rows_per_split - 1) / rows_per_split;
+    float *part = y;
+    if (splits > 1) {
+        uint8_t *tmp = nullptr;
+        bool transient = false;
+        if (int rc = workspace(s, (size_t)splits * n * 4, &tmp, &transient)) return rc;   // (never transient: <= 8 MiB)
+        part = reinterpret_cast<float *>(tmp);
+    }
+    if (vec) hipLaunchKernelGGL((gemv_kn_kernel<FMT, 4>), dim3(bx, splits), dim3(256), 0, s, w, x, part, n, k, rows_per_split);
+    else hipLaunchKernelGGL((gemv_kn_kernel<FMT, 1>), dim3(bx, splits), dim3(256), 0, s, w, x, part, n, k, rows_per_split);
+    RFQ_LAUNCH_CHECK("gemv_kn_kernel");
+    if (splits > 1) {
+        hipLaunchKernelGGL(gemv_kn_reduce_kernel, dim3((n + 255) / 256), dim3(256), 0, s, part, y, n, splits);
+        RFQ_LAUNCH_CHECK("gemv_kn_reduce_kernel");
     }
     return RFQ_OK;
 }
@@ -634,7 +801,30 @@ int launch_dequant(int fmt, const uint8_t *d_in, size_t in_bytes, float *d_out, 
     case RFQ_GGUF_Q8_0: return run<RFQ_GGUF_Q8_0>(d_in, in_bytes, d_out, n, s);
     case RFQ_GGUF_Q4_K: return run<RFQ_GGUF_Q4_K>(d_in, in_bytes, d_out, n, s);
     case RFQ_GGUF_Q6_K: return run<RFQ_GGUF_Q6_K>(d_in, in_bytes, d_out, n, s);
+    case RFQ_MM_Q8_0: return run<RFQ_MM_Q8_0>(d_in, in_bytes, d_out, n, s);
+    case RFQ_MM_Q4_K: return run<RFQ_MM_Q4_K>(d_in, in_bytes, d_out, n, s);
+    case RFQ_MM_Q6_K: return run<RFQ_MM_Q6_K>(d_in, in_bytes, d_out, n, s);
     default: return fail(RFQ_E_BADARG, "rfq_dequant: unknown format %d", fmt);
+    }
+}
+
+int launch_gemv_kn(int fmt, const uint8_t *d_w, const float *d_x, float *d_y, int n, int k, hipStream_t s)
+{
+    switch (canonical_format(fmt)) {
+    case RFQ_Q4_0: return run_gemv_kn<RFQ_Q4_0>(d_w, d_x, d_y, n, k, s);
+    case RFQ_Q8_0: return run_gemv_kn<RFQ_Q8_0>(d_w, d_x, d_y, n, k, s);
+    case RFQ_Q4_K: return run_gemv_kn<RFQ_Q4_K>(d_w, d_x, d_y, n, k, s);
+    case RFQ_Q6_K: return run_gemv_kn<RFQ_Q6_K>(d_w, d_x, d_y, n, k, s);
+    case RFQ_MXFP4: return run_gemv_kn<RFQ_MXFP4>(d_w, d_x, d_y, n, k, s);
+    case RFQ_MXFP6_E2M3: return run_gemv_kn<RFQ_MXFP6_E2M3>(d_w, d_x, d_y, n, k, s);
+    case RFQ_GGUF_Q4_0: return run_gemv_kn<RFQ_GGUF_Q4_0>(d_w, d_x, d_y, n, k, s);
+    case RFQ_GGUF_Q8_0: return run_gemv_kn<RFQ_GGUF_Q8_0>(d_w, d_x, d_y, n, k, s);
+    case RFQ_GGUF_Q4_K: return run_gemv_kn<RFQ_GGUF_Q4_K>(d_w, d_x, d_y, n, k, s);
+    case RFQ_GGUF_Q6_K: return run_gemv_kn<RFQ_GGUF_Q6_K>(d_w, d_x, d_y, n, k, s);
+    case RFQ_MM_Q8_0: return run_gemv_kn<RFQ_MM_Q8_0>(d_w, d_x, d_y, n, k, s);
+    case RFQ_MM_Q4_K: return run_gemv_kn<RFQ_MM_Q4_K>(d_w, d_x, d_y, n, k, s);
+    case RFQ_MM_Q6_K: return run_gemv_kn<RFQ_MM_Q6_K>(d_w, d_x, d_y, n, k, s);
+    default: return fail(RFQ_E_BADARG, "rfq_gemv_kn: unknown format %d", fmt);
     }
 }
 

@@ -40,26 +40,10 @@
 // about 43.
 #include <mutex>
 #include <unordered_map>
+#include <vector>
 #include <type_traits>
 
 #include "rfq_common.hpp"
-
-// -DRFQ_KQ_SKIP=<mask> (tuning builds, results are wrong on purpose): leave out
-// 1 the A loads, 2 the W loads, 4 the LDS fragment reads, 8 the LDS writes,
-// 16 the weight decoding, 32 the Q4_K group-sum loads, to see what a stage's
-// time is made of.  -DRFQ_KQ_TRACE=<workgroup> records that workgroup's loop
-// time in shader clocks and in 100 MHz ticks (rfq_kq_trace reads them back).
-#ifndef RFQ_KQ_SKIP
-#define RFQ_KQ_SKIP 0
-#endif
-
-#ifdef RFQ_KQ_TRACE
-__device__ long long rfq_kq_trace_dev[8];
-extern "C" __attribute__((visibility("default"))) int rfq_kq_trace(long long *out)
-{
-    return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(rfq_kq_trace_dev), sizeof(long long) * 8);
-}
-#endif
 
 namespace rfq {
 namespace {
@@ -465,7 +449,7 @@ arrange_a_kernel(const _Float16 *__restrict__ a, v4u *__restrict__ at, _Float16 
     const int st = st0 + wave;
     if (st >= nst) return;
     const int fr = lane & 31, fh = lane >> 5;
-    const int m = mt * 32 + fr, k0 = st * 64 + fh * 32;
+    const int k0 = st * 64 + fh * 32;
     const size_t unit = (size_t)mt * nst + st;
     v4u v[4];
 #pragma unroll
@@ -476,7 +460,7 @@ arrange_a_kernel(const _Float16 *__restrict__ a, v4u *__restrict__ at, _Float16 
                        __builtin_amdgcn_perm(v[c][3], v[c][1], 0x05040100u), __builtin_amdgcn_perm(v[c][3], v[c][1], 0x07060302u)};
         at[(unit * 4 + c) * 64 + lane] = p;
     }
-    if (SUMS && m < M && k0 < K) {
+    if (SUMS && k0 < K) {                                         // (rows past M were staged as zeros: their sums are zero)
         float sum = 0.0f;
 #pragma unroll
         for (int c = 0; c < 4; c++) {
@@ -499,9 +483,6 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
                void *__restrict__ outp, int M, int N, int K)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-#ifdef RFQ_KQ_TRACE
-    const long long tr_e = wall_clock64();
-#endif
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int fr = lane & 31, fh = lane >> 5;                     // fragment row, k half
     const int tiles_m = (M + BM - 1) / BM;
@@ -564,11 +545,11 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
         // group: both lanes of the row then read the first (zeroed when decoded)
         const int sc = st < nstages ? st : nstages - 1;
         const int whc = Fmt<FMT>::BE == 32 && sc * 2 + 1 >= groups ? 0 : wh;
-        if (!(RFQ_KQ_SKIP & 2)) raw_of(slotc).load(w_tile, w_off, sc, whc);
+        raw_of(slotc).load(w_tile, w_off, sc, whc);
     };
     auto fetch_a = [&](auto slotc, int st, int i, int c) __attribute__((always_inline)) {
         const int sc = st < nstages ? st : nstages - 1;
-        if (!(RFQ_KQ_SKIP & 1)) ra_of(slotc)[i][c] = __builtin_amdgcn_raw_buffer_load_b128(a_tile[i], lane16 + c * 1024, sc * 4096, 0);
+        ra_of(slotc)[i][c] = __builtin_amdgcn_raw_buffer_load_b128(a_tile[i], lane16 + c * 1024, sc * 4096, 0);
     };
     auto fetch_a_all = [&](auto slotc, int st) __attribute__((always_inline)) {
 #pragma unroll
@@ -593,20 +574,9 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
     const uint8_t *rd_base[2] = {lds + fr * LDR + fh * 64, lds + 2 * W_BYTES + fr * LDR + fh * 64};
     uint8_t *wr_base[2] = {lds + wr * LDR + wh * 64, lds + 2 * W_BYTES + wr * LDR + wh * 64};
     auto read_frag = [&](int buf, int j, int c) __attribute__((always_inline)) -> v8h {
-        if (RFQ_KQ_SKIP & 4) {
-            v8h r;
-#pragma unroll
-            for (int e = 0; e < 8; e++) r[e] = (_Float16)(float)(lane + e);
-            return r;
-        }
         return *reinterpret_cast<const v8h *>(rd_base[buf >> 1] + (buf & 1) * W_BYTES + j * 32 * LDR + c * 16);
     };
     auto stash = [&](int buf, int c, const v8h (&hw)[4]) __attribute__((always_inline)) {
-        if (RFQ_KQ_SKIP & 8) {
-            if ((float)hw[c][0] + (float)hw[c][1] + (float)hw[c][2] + (float)hw[c][3] + (float)hw[c][4] + (float)hw[c][5] + (float)hw[c][6] + (float)hw[c][7] == 1.2345e-30f)
-                *reinterpret_cast<v8h *>(wr_base[0]) = hw[c];
-            return;
-        }
         *reinterpret_cast<v8h *>(wr_base[buf >> 1] + (buf & 1) * W_BYTES + c * 16) = hw[c];
     };
 
@@ -650,7 +620,6 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
     }
     auto fetch_hdr = [&](int trip) __attribute__((always_inline)) {
         if constexpr (FMT == RFQ_Q4_K) {
-            if (RFQ_KQ_SKIP & 2) return;
             const int blk = (trip < K / 256 ? trip : K / 256 - 1) * 256;
             hs_ring = __builtin_amdgcn_raw_buffer_load_b128(w_tile, w_off, blk, 0);
             hm_ring = __builtin_amdgcn_raw_buffer_load_b32(w_tile, w_off + 16 + 4 * wh, blk, 0);
@@ -658,7 +627,6 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
     };
     auto fetch_sums = [&](int trip) __attribute__((always_inline)) {
         if constexpr (FMT == RFQ_Q4_K) {
-            if (RFQ_KQ_SKIP & 32) return;
             const int t = trip < K / 256 ? trip : K / 256 - 1;
 #pragma unroll
             for (int i = 0; i < TI; i++) sa_ring[i] = __builtin_amdgcn_raw_buffer_load_b128(s_tile[i], lane16, t * 1024, 0);
@@ -749,7 +717,7 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
                 __builtin_memcpy(&fa, &ra[i][c], 16);
                 acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[c & 1][j], fa, acc[j][i], 0, 0, 0);
                 if (t < 4) fw[(c + 1) & 1][t] = c < 3 ? read_frag(S, t, c + 1) : read_frag(S1, t, 0);
-                if (!(RFQ_KQ_SKIP & 16)) {
+                {
                     constexpr int LATE[6] = {0, 3, 5, 8, 10, 13}, EARLY[6] = {16, 18, 20, 22, 26, 29};
 #pragma unroll
                     for (int q = 0; q < 6; q++) {
@@ -814,9 +782,6 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
 #pragma unroll
         for (int j = 0; j < TJ; j++) fw[0][j] = read_frag(0, j, 0);
     }
-#ifdef RFQ_KQ_TRACE
-    const long long tr_c0 = clock64(), tr_w0 = wall_clock64();
-#endif
     // Whole trips through the ring only (no branch between the four bodies);
     // stages past the end multiply zero weights.
     for (int st = 0; st < nstages; st += 4) {
@@ -830,15 +795,6 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
             hmA = hmB;
         }
     }
-#ifdef RFQ_KQ_TRACE
-    if (tid == 0 && blockIdx.x == RFQ_KQ_TRACE) {
-        rfq_kq_trace_dev[0] = clock64() - tr_c0;
-        rfq_kq_trace_dev[1] = wall_clock64() - tr_w0;
-        rfq_kq_trace_dev[2] = nstages;
-        rfq_kq_trace_dev[3] = tr_w0 - tr_e;
-    }
-    const long long tr_w1 = wall_clock64();
-#endif
 
     // Register r of tile (j, i): n = 8*(r/4) + 4*(lane/32) + r%4 within the
     // tile (four consecutive n per r/4), m = lane%32.
@@ -881,10 +837,6 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
                 __builtin_nontemporal_store(v, reinterpret_cast<v4u *>(o));
             }
         }
-#ifdef RFQ_KQ_TRACE
-        __builtin_amdgcn_s_waitcnt(0);
-        if (tid == 0 && blockIdx.x == RFQ_KQ_TRACE) rfq_kq_trace_dev[4] = wall_clock64() - tr_w1;
-#endif
         return;
     }
     const bool vec_ok = (N % 4) == 0 && (reinterpret_cast<uintptr_t>(outp) & 15u) == 0;
@@ -918,10 +870,6 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
                 }
             }
         }
-#ifdef RFQ_KQ_TRACE
-    __builtin_amdgcn_s_waitcnt(0);
-    if (tid == 0 && blockIdx.x == RFQ_KQ_TRACE) rfq_kq_trace_dev[4] = wall_clock64() - tr_w1;
-#endif
 }
 
 template <int FMT, bool OUT_F16>
@@ -969,20 +917,31 @@ int launch_fmt(const uint8_t *w, const void *a, void *out, int out_dtype, int m,
 
 // Temporary device memory for one call.  Up to WS_KEEP bytes it is a buffer
 // the library keeps per stream (calls on one stream run in order, so the next
-// call may overwrite it; different streams get different buffers) and frees
+// call may overwrite it; different streams get different buffers) and replaces
 // only when a larger one is needed: a stream-ordered allocation and release
 // around every call costs about 6 us of idle GPU between calls.  Larger
 // requests are allocated and released in stream order, per call.
+// While the stream is being captured nothing is allocated or freed: the call
+// gets the stream's buffer if it is large enough and an error otherwise.  A
+// buffer handed out under capture is baked into the graph, so when a later
+// call outgrows it the old buffer is retired (kept allocated) instead of
+// freed; only release_workspaces() frees retired buffers.
 namespace {
 constexpr size_t WS_KEEP = (size_t)64 << 20;
-struct Kept { uint8_t *ptr; size_t bytes; int device; };
+struct Kept { uint8_t *ptr; size_t bytes; int device; bool captured; };
 std::mutex ws_mutex;
 std::unordered_map<hipStream_t, Kept> ws_kept;
+std::vector<Kept> ws_retired;
 } // namespace
 
 int workspace(hipStream_t s, size_t bytes, uint8_t **out, bool *transient)
 {
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    RFQ_HIP(hipStreamIsCapturing(s, &cap));
+    const bool capturing = cap != hipStreamCaptureStatusNone;
     if (bytes > WS_KEEP) {
+        if (capturing)
+            return fail(RFQ_E_UNSUPPORTED, "%zu bytes of temporary memory exceed what the library keeps per stream and cannot be allocated while the stream is being captured", bytes);
         *transient = true;
         RFQ_HIP(hipMallocAsync(reinterpret_cast<void **>(out), bytes, s));
         return RFQ_OK;
@@ -993,11 +952,18 @@ int workspace(hipStream_t s, size_t bytes, uint8_t **out, bool *transient)
     std::lock_guard<std::mutex> lock(ws_mutex);
     Kept &kept = ws_kept[s];
     if (kept.ptr == nullptr || kept.bytes < bytes || kept.device != device) {
-        if (kept.ptr != nullptr && kept.device == device) RFQ_HIP(hipFree(kept.ptr)); // (waits for the work that uses it)
-        kept = Kept{nullptr, 0, device};
+        if (capturing)
+            return fail(RFQ_E_UNSUPPORTED, "the call needs %zu bytes of temporary memory and the stream being captured holds %zu: run the call once on this stream before capturing it",
+                        bytes, kept.device == device ? kept.bytes : (size_t)0);
+        if (kept.ptr != nullptr) {
+            if (kept.captured || kept.device != device) ws_retired.push_back(kept);   // a graph (or another device's stream) may hold it
+            else RFQ_HIP(hipFree(kept.ptr));                                          // (waits for the work that uses it)
+        }
+        kept = Kept{nullptr, 0, device, false};
         RFQ_HIP(hipMalloc(reinterpret_cast<void **>(&kept.ptr), bytes));
         kept.bytes = bytes;
     }
+    if (capturing) kept.captured = true;
     *out = kept.ptr;
     return RFQ_OK;
 }
@@ -1005,18 +971,20 @@ int workspace(hipStream_t s, size_t bytes, uint8_t **out, bool *transient)
 int release_workspaces()
 {
     std::lock_guard<std::mutex> lock(ws_mutex);
-    if (ws_kept.empty()) return RFQ_OK;
+    if (ws_kept.empty() && ws_retired.empty()) return RFQ_OK;
     RFQ_HIP(hipDeviceSynchronize());
     int current = 0;
     RFQ_HIP(hipGetDevice(&current));
     hipError_t first = hipSuccess;
-    for (auto &entry : ws_kept) {
-        if (entry.second.ptr == nullptr) continue;
-        hipError_t e = hipSetDevice(entry.second.device);
-        if (e == hipSuccess) e = hipFree(entry.second.ptr);
+    for (auto &entry : ws_kept) ws_retired.push_back(entry.second);
+    ws_kept.clear();
+    for (const Kept &k : ws_retired) {
+        if (k.ptr == nullptr) continue;
+        hipError_t e = hipSetDevice(k.device);
+        if (e == hipSuccess) e = hipFree(k.ptr);
         if (first == hipSuccess) first = e;
     }
-    ws_kept.clear();
+    ws_retired.clear();
     hipError_t back = hipSetDevice(current);
     if (first == hipSuccess) first = back;
     if (first != hipSuccess) return hip_fail(first, "rfq_release_temporaries");

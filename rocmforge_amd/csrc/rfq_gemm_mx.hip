@@ -29,34 +29,9 @@
 
 #include "rfq_common.hpp"
 
-// -DRFQ_MX_TRACE (tuning builds): every workgroup records wall-clock stamps
-// (100 MHz) at kernel entry, loop entry, loop exit and exit.
-#ifdef RFQ_MX_TRACE
-__device__ unsigned long long *rfq_mx_trace;
-#define RFQ_MX_STAMP(slot)                                                                                     \
-    do {                                                                                                       \
-        if (threadIdx.x == 0 && rfq_mx_trace) rfq_mx_trace[(size_t)blockIdx.x * 4 + (slot)] = wall_clock64(); \
-    } while (0)
-#else
-#define RFQ_MX_STAMP(slot) do { } while (0)
-#endif
-// -DRFQ_MX_SKIP=<mask> (tuning builds, results are wrong on purpose): leave out
-// 1 the A loads, 2 the W copies, 4 the LDS fragment reads, 8 the output stores,
-// to see what the loop time is made of.  No address depends on loaded data,
-// so the skipped parts change timing only.
-#ifndef RFQ_MX_SKIP
-#define RFQ_MX_SKIP 0
-#endif
 // Ring depth (W slots in LDS = A fragment sets in registers) with 4-bit A
 // fragments; 8-bit A fragments take twice the registers and half the depth.
-// -DRFQ_MX_GENERAL_FP4=1: re-encode MXFP4 to 4-bit operands with the general
-// (float) kernel instead of the integer one, to compare the two.
-#ifndef RFQ_MX_GENERAL_FP4
-#define RFQ_MX_GENERAL_FP4 0
-#endif
-#ifndef RFQ_MX_RING
-#define RFQ_MX_RING 8
-#endif
+constexpr int RFQ_MX_RING = 8;
 
 namespace rfq {
 namespace {
@@ -418,7 +393,6 @@ __global__ void __launch_bounds__(256)
 gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, void *__restrict__ outp, int M, int N,
                MxLayout LA, MxLayout LB)
 {
-    RFQ_MX_STAMP(0);
     using C = GemmCfg<BK_, TJ, RING>;
     constexpr int TI = C::TI, PA = Pg<AK>::BYTES;
     constexpr int NMMA = TI * TJ;
@@ -431,7 +405,7 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
     // among themselves, so "at most this many operations outstanding" proves
     // that stage s+1 has arrived; stores in flight (from a tile's epilogue)
     // can only make the wait longer, never too short.
-    constexpr int NA_CNT = (RFQ_MX_SKIP & 1) ? 0 : NA_OPS, ND_CNT = (RFQ_MX_SKIP & 2) ? 0 : C::ND;
+    constexpr int NA_CNT = NA_OPS, ND_CNT = C::ND;
     // (the counter has 6 bits; a smaller number only waits for more than necessary)
     constexpr int HANDOVER_EXACT = (RING - 2) * (NA_CNT + ND_CNT);
     constexpr int PROLOGUE_EXACT = (RING - 1) * ND_CNT + (RING - 2) * NA_CNT;
@@ -535,7 +509,6 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
     // uses M0).
     auto dma_piece = [&](auto slotc, int i) {
         constexpr int SLOT = decltype(slotc)::value;
-        if (RFQ_MX_SKIP & 2) return;
         const uint32_t voff = i == C::ND - 1 ? voffWL : voffW;
         const uint8_t *base = pf_w[i];
         const int doff = dst_off[i] + (int)lds0;
@@ -554,7 +527,6 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
     // fragment) stays with compiler-tracked loads.
     auto a_piece = [&](auto setc, int piece) {
         constexpr int SET = decltype(setc)::value;
-        if (RFQ_MX_SKIP & 1) return;
         if (piece < TI * 2 * A_PER_FRAG) {
             const int f = piece / A_PER_FRAG, half = piece % A_PER_FRAG, i = f >> 1, ksl = f & 1;
             if (AK == RFQ_MX_FP4) {
@@ -656,7 +628,6 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
     asm volatile("" : "+v"(wf1), "+v"(wf2), "+v"(ws1), "+v"(ws2));
     static_assert(C::RING_BYTES <= 3 * 65536, "LDS windows");
     auto read_b = [&](int slot, int ksl, int j, WFrag (&fb)[TJ]) {
-        if (RFQ_MX_SKIP & 4) return;
         const int off = slot * C::STAGE + (j * 2 + ksl) * C::PB;
         lds_u8_ptr w = (off >> 16) == 0 ? wf0 : (off >> 16) == 1 ? wf1 : wf2;
         v4i lo = *reinterpret_cast<lds_v4i_ptr>(w + (off & 65535));
@@ -670,18 +641,12 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
     };
     // Scale dword of lane l for row tile j sits at (j*64 + l)*4 of the scale part.
     auto read_bscale = [&](int slot, int j, int (&xb)[TJ]) {
-        if (RFQ_MX_SKIP & 4) return;
         const int off = slot * C::STAGE + C::B_STAGE + j * 256;
         lds_u8_ptr w = (off >> 16) == 0 ? ws0 : (off >> 16) == 1 ? ws1 : ws2;
         xb[j] = *reinterpret_cast<lds_i32_ptr>(w + (off & 65535));
     };
 #pragma unroll
     for (int j = 0; j < TJ; j++) {
-        if (RFQ_MX_SKIP & 4) {
-#pragma unroll
-            for (int e = 0; e < (BK_ == RFQ_MX_FP4 ? 4 : 8); e++) fb0[j][e] = fb1[j][e] = 0x22222222 + lane + j;
-            sb[0][j] = sb[1][j] = 0x7f7f7f7f;
-        }
         read_b(0, 0, j, fb0);
         read_bscale(0, j, sb[0]);
     }
@@ -778,18 +743,6 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
         const int m_base = tmi * C::BM + wave * TI * 32, n_base = tn * C::BN;
         const bool interior = m_base + TI * 32 <= M && n_base + TJ * 32 <= N && ((size_t)N * ES) % 16 == 0 &&
                               (reinterpret_cast<uintptr_t>(outp) & 15u) == 0;
-        if (RFQ_MX_SKIP & 8) {
-            // keep the accumulators alive without storing them (the test is never true for finite sums of products)
-            float keep = 0.0f;
-#pragma unroll
-            for (int i = 0; i < TI; i++)
-#pragma unroll
-                for (int j = 0; j < TJ; j++)
-#pragma unroll
-                    for (int r = 0; r < 16; r++) keep += acc[i][j][r];
-            if (keep == 1.2345e-30f) reinterpret_cast<float *>(outp)[lane] = keep;
-            return;
-        }
         typedef __attribute__((address_space(3))) uint8_t *lds_w8_ptr;
         lds_w8_ptr stage3 = (lds_w8_ptr)lds + C::RING_BYTES + wave * RB * ROW_STRIDE;
         // this lane's accumulator elements: rows 4*(lane/32) + {0..3, 8..11, 16..19, 24..27}, column lane%32 of a tile
@@ -853,7 +806,6 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
             }
     };
 
-    RFQ_MX_STAMP(1);
     for (int idx = idx0; tile_valid(idx); idx += G8) {
         // past the last tile the streams fetch the start of the last tile again
         // (into registers / LDS nobody reads): every stage issues the same
@@ -875,7 +827,6 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
     // The trailing prefetches still write LDS slots and registers: drain them
     // before the wavefront ends.
     wait_vmcnt<0>();
-    RFQ_MX_STAMP(3);
 }
 
 template <int AK, int BK_, bool OUT_BF16, int TJ, int RING>
@@ -923,7 +874,7 @@ int run_prepare(const uint8_t *raw, uint8_t *prep, const MxLayout &L, hipStream_
     size_t threads = (size_t)L.rt * L.ks * 64;
     hipLaunchKernelGGL(mx_init_kernel, dim3(1), dim3(64), 0, s, prep, L);
     RFQ_LAUNCH_CHECK("mx_init_kernel");
-    if (FMT == RFQ_MXFP4 && KIND == RFQ_MX_FP4 && !RFQ_MX_GENERAL_FP4)
+    if (FMT == RFQ_MXFP4 && KIND == RFQ_MX_FP4)
         hipLaunchKernelGGL(mx_prepare_fp4_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, raw, prep, L);
     else
         hipLaunchKernelGGL((mx_prepare_kernel<FMT, KIND>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, raw,

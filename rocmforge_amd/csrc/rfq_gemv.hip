@@ -22,19 +22,6 @@
 
 #include "rfq_common.hpp"
 
-// Per-wavefront phase timestamps for tuning builds (-DRFQ_GEMV_TRACE); compiled
-// out of the library.
-#ifdef RFQ_GEMV_TRACE
-__device__ unsigned long long *rfq_trace_buf;
-#define RFQ_TS(slot)                                                                                   \
-    do {                                                                                               \
-        if ((threadIdx.x & 63) == 0 && rfq_trace_buf)                                                  \
-            rfq_trace_buf[((size_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * 8 + (slot)] = wall_clock64(); \
-    } while (0)
-#else
-#define RFQ_TS(slot) do { } while (0)
-#endif
-
 namespace rfq {
 namespace {
 
@@ -422,6 +409,59 @@ template <> struct Unit<RFQ_GGUF_Q6_K> {
         const float g0 = __builtin_fmaf(-32.0f, xs0, a[0]), g1 = __builtin_fmaf(-32.0f, xsum - xs0, a[1]);
         const float c0 = (float)(int8_t)(sc2 & 255u), c1 = (float)(int8_t)(sc2 >> 8);
         return f16_bits_to_f32(d) * __builtin_fmaf(c0, g0, c1 * g1);
+    }
+};
+
+// ---- the matmul module's own decoders (src/kernels/matmul/quantized/) -------------
+// Multiplied by the one-row-per-wavefront kernel only (the reference multiplies them in the other orientation,
+// see gemv_kn_kernel).
+
+template <> struct Unit<RFQ_MM_Q8_0> {                 // quantized/q8_0.rs:34-52: scale * (byte as i8)
+    static constexpr bool NEEDS_XSUM = false;
+    float scale; U8 q;
+    __device__ __forceinline__ void load(const uint8_t *row, int u)
+    {
+        const uint8_t *p = row + (size_t)u * 36;
+        scale = ld<float>(p);
+        q = ld<U8>(p + 4);
+    }
+    __device__ __forceinline__ float dot(const float (&x)[32], float) const
+    {
+        float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+        for (int d = 0; d < 8; d++) {
+            s0 = __builtin_fmaf((float)(int8_t)(q.v[d] & 255u), x[4 * d], s0);
+            s1 = __builtin_fmaf((float)(int8_t)((q.v[d] >> 8) & 255u), x[4 * d + 1], s1);
+            s0 = __builtin_fmaf((float)(int8_t)((q.v[d] >> 16) & 255u), x[4 * d + 2], s0);
+            s1 = __builtin_fmaf((float)(int8_t)(q.v[d] >> 24), x[4 * d + 3], s1);
+        }
+        return scale * (s0 + s1);
+    }
+};
+
+template <> struct Unit<RFQ_MM_Q4_K> {                 // quantized/q4_k.rs:101-143: nibbles at 32 + 20 * sb
+    static constexpr bool NEEDS_XSUM = true;
+    uint16_t sc; int8_t mn; U4 q;
+    __device__ __forceinline__ void load(const uint8_t *row, int u)
+    {
+        const uint8_t *blk = row + (size_t)(u >> 3) * 256;
+        int sb = u & 7;
+        sc = ld<uint16_t>(blk + 2 * sb);
+        mn = (int8_t)blk[16 + sb];
+        q = ld<U4>(blk + 32 + 20 * sb);
+    }
+    __device__ __forceinline__ float dot(const float (&x)[32], float xsum) const
+    {
+        return __builtin_fmaf(f16_bits_to_f32_mm(sc), nib_dot_lo_first(q, x), (float)mn * xsum);
+    }
+};
+
+template <> struct Unit<RFQ_MM_Q6_K> : Unit<RFQ_Q6_K> { // quantized/q6_k.rs:101-143: scales through f16_to_f32_cpu
+    __device__ __forceinline__ float dot(const float (&x)[32], float) const
+    {
+        float a = dot16(q.v[0], q.v[1], q.v[2], &x[0]);
+        float b = dot16(q.v[3], q.v[4], q.v[5], &x[16]);
+        return __builtin_fmaf(f16_bits_to_f32_mm((uint16_t)(sc2 & 0xFFFFu)), a, f16_bits_to_f32_mm((uint16_t)(sc2 >> 16)) * b);
     }
 };
 
@@ -1018,7 +1058,6 @@ __global__ void __launch_bounds__(64 * IDOT_WAVES)
 gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ y, int n, int k,
                  int groups, GemvFuse f)
 {
-    RFQ_TS(0);
     using IU = IUnit<FMT>;
     constexpr int WAVES = IDOT_WAVES, TEAMS = WAVES / WPR, TL = 64 * WPR, THREADS = 64 * WAVES;
     // rows in flight per lane: three, or five in the form with one unit per lane (its registers allow it;
@@ -1078,7 +1117,6 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
     };
 #pragma unroll
     for (int d = 0; d < D; d++) load_row(d, d);
-    RFQ_TS(1);
 
     // Cooperative conversion of x: 4*ku quarter-units (eight values each) over the block's threads.
     float ssq = 0.f;
@@ -1109,7 +1147,6 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
             if (lane == 0) ssq_part[wave] = ssq;
         }
     }
-    RFQ_TS(2);
     __syncthreads();
     float rinv = 1.0f;
     if constexpr (FUSE) {
@@ -1134,7 +1171,6 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
         xp[j].xh0 = __uint_as_float(src[26]);
         xp[j].xh1 = __uint_as_float(src[27]);
     }
-    RFQ_TS(3);
 
     __shared__ float part[R][WAVES];
     for (int g = 0; g < groups; g++) {
@@ -1160,7 +1196,6 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
             if (i + D < R) load_row(i % D, base + i + D);
             res[i] = wave_sum(acc);
         }
-        RFQ_TS(4);
         // (`groups` is uniform over the block: every wavefront stores the same number of groups)
         store_group<R, WPR, FUSE, WAVES>(res, part, y, row0 + base, row_end, lane, wave, f, rinv);
     }
@@ -1343,9 +1378,6 @@ gemv_mfma_prep_kernel(const float *__restrict__ x, _Float16 *__restrict__ parts,
     if (kk == 0) sx[u * 8 + v] = sc;
 }
 
-#ifndef RFQ_M8_SKIP
-#define RFQ_M8_SKIP 0
-#endif
 constexpr int MFMA_NB = 16;                           // units of a wavefront in flight together
 constexpr int MFMA_WAVES = 8;
 
@@ -1379,16 +1411,16 @@ gemv_mfma_q8_0_kernel(const uint8_t *__restrict__ w, const _Float16 *__restrict_
         v4f_t s4[MFMA_NB / 2];                          // (the x scales follow half a batch behind: registers)
         auto load_s4 = [&](int b) {
             const int u = base + MFMA_WAVES * b, uc = u < units ? u : units - 1;
-            s4[b % (MFMA_NB / 2)] = (RFQ_M8_SKIP & 4) ? v4f_t{1.f, 1.f, 1.f, 1.f} : *reinterpret_cast<const v4f_t *>(sx + uc * 8 + 4 * (q & 1));
+            s4[b % (MFMA_NB / 2)] = *reinterpret_cast<const v4f_t *>(sx + uc * 8 + 4 * (q & 1));
         };
 #pragma unroll
         for (int b = 0; b < MFMA_NB; b++) {
             const int u = base + MFMA_WAVES * b, uc = u < units ? u : units - 1; // (past the end: a valid unit, weight scale 0)
             const uint8_t *blk = row_ptr + (size_t)uc * BB;
-            wq[b] = (RFQ_M8_SKIP & 1) ? v2u_t{(uint32_t)lane, (uint32_t)b} : ld<v2u_t>(row_ptr_c + (size_t)uc * BB);
-            ws[b] = (RFQ_M8_SKIP & 1) ? 1.0f : (FMT == RFQ_Q8_0 ? ld<float>(blk) : f16_bits_to_f32(ld<uint16_t>(blk)));                    // (no branch around a load: it would wait for the others)
-            xh[b] = (RFQ_M8_SKIP & 2) ? v4u_t{1u, 2u, 3u, (uint32_t)lane} : parts_l[(size_t)uc * 64];
-            xl[b] = (RFQ_M8_SKIP & 2) ? v4u_t{1u, 2u, 3u, (uint32_t)lane} : parts_l[(size_t)uc * 64 + 32];
+            wq[b] = ld<v2u_t>(row_ptr_c + (size_t)uc * BB);
+            ws[b] = FMT == RFQ_Q8_0 ? ld<float>(blk) : f16_bits_to_f32(ld<uint16_t>(blk));                    // (no branch around a load: it would wait for the others)
+            xh[b] = parts_l[(size_t)uc * 64];
+            xl[b] = parts_l[(size_t)uc * 64 + 32];
             if (b < MFMA_NB / 2) load_s4(b);
         }
         __builtin_amdgcn_sched_barrier(0);             // (every load of the batch is out before the first is used)
@@ -1704,6 +1736,22 @@ int run_rows(const uint8_t *w, const float *x, float *y, int n, int k, const Gem
 }
 
 template <int FMT>
+int run_generic_m(const uint8_t *w, const float *x, float *y, int m, int n, int k, hipStream_t s)
+{
+    switch (m) {
+    case 1: return run_generic<FMT, 1>(w, x, y, n, k, s);
+    case 2: return run_generic<FMT, 2>(w, x, y, n, k, s);
+    case 3: return run_generic<FMT, 3>(w, x, y, n, k, s);
+    case 4: return run_generic<FMT, 4>(w, x, y, n, k, s);
+    case 5: return run_generic<FMT, 5>(w, x, y, n, k, s);
+    case 6: return run_generic<FMT, 6>(w, x, y, n, k, s);
+    case 7: return run_generic<FMT, 7>(w, x, y, n, k, s);
+    case 8: return run_generic<FMT, 8>(w, x, y, n, k, s);
+    default: return fail(RFQ_E_BADARG, "rfq_gemv: m=%d outside 1..8", m);
+    }
+}
+
+template <int FMT>
 int run(const uint8_t *w, const float *x, float *y, int m, int n, int k, hipStream_t s)
 {
     const int ku = k / 32;
@@ -1730,17 +1778,7 @@ int run(const uint8_t *w, const float *x, float *y, int m, int n, int k, hipStre
         }
         return RFQ_OK;
     }
-    switch (m) {
-    case 1: return run_generic<FMT, 1>(w, x, y, n, k, s);
-    case 2: return run_generic<FMT, 2>(w, x, y, n, k, s);
-    case 3: return run_generic<FMT, 3>(w, x, y, n, k, s);
-    case 4: return run_generic<FMT, 4>(w, x, y, n, k, s);
-    case 5: return run_generic<FMT, 5>(w, x, y, n, k, s);
-    case 6: return run_generic<FMT, 6>(w, x, y, n, k, s);
-    case 7: return run_generic<FMT, 7>(w, x, y, n, k, s);
-    case 8: return run_generic<FMT, 8>(w, x, y, n, k, s);
-    default: return fail(RFQ_E_BADARG, "rfq_gemv: m=%d outside 1..8", m);
-    }
+    return run_generic_m<FMT>(w, x, y, m, n, k, s);
 }
 
 } // namespace
@@ -1758,6 +1796,9 @@ int launch_gemv(int fmt, const uint8_t *d_w, const float *d_x, float *d_y, int m
     case RFQ_GGUF_Q8_0: return run<RFQ_GGUF_Q8_0>(d_w, d_x, d_y, m, n, k, s);
     case RFQ_GGUF_Q4_K: return run<RFQ_GGUF_Q4_K>(d_w, d_x, d_y, m, n, k, s);
     case RFQ_GGUF_Q6_K: return run<RFQ_GGUF_Q6_K>(d_w, d_x, d_y, m, n, k, s);
+    case RFQ_MM_Q8_0: return run_generic_m<RFQ_MM_Q8_0>(d_w, d_x, d_y, m, n, k, s);
+    case RFQ_MM_Q4_K: return run_generic_m<RFQ_MM_Q4_K>(d_w, d_x, d_y, m, n, k, s);
+    case RFQ_MM_Q6_K: return run_generic_m<RFQ_MM_Q6_K>(d_w, d_x, d_y, m, n, k, s);
     default: return fail(RFQ_E_BADARG, "rfq_gemv: unknown format %d", fmt);
     }
 }

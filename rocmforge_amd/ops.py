@@ -63,6 +63,23 @@ def gemv(fmt: int, w: torch.Tensor, x: torch.Tensor, n: int, k: int, out: torch.
     return out if x.dim() > 1 else out.view(n)
 
 
+def gemv_kn(fmt: int, w: torch.Tensor, x: torch.Tensor, n: int, k: int, out: torch.Tensor | None = None) -> torch.Tensor:
+    """y[m, n] = x[m, k] . Wd[k, n] with Wd[l, j] = element l * n + j of the packed stream decoded as one flat
+    array: the orientation the reference's kernel and CPU fallback compute (kernels/q4_0_matmul.hip:207,
+    src/kernels/matmul/quantized/q4_0.rs:274-311)."""
+    w = _dev_u8(w)
+    x = _f32(x, "x")
+    m = 1 if x.dim() == 1 else x.shape[0]
+    if x.shape[-1] != k:
+        raise ValueError(f"x has {x.shape[-1]} columns, k = {k}")
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float32, device=x.device)
+    elif not (out.is_cuda and out.dtype == torch.float32 and out.is_contiguous() and out.numel() == m * n):
+        raise ValueError("out must be a contiguous float32 device tensor of m * n elements")
+    check(lib().rfq_gemv_kn(fmt, _ptr(w), w.numel(), _ptr(x), _ptr(out), m, n, k, _stream()))
+    return out if x.dim() > 1 else out.view(n)
+
+
 def get_rows(fmt: int, table: torch.Tensor, tokens: torch.Tensor, n_vocab: int, n_embd: int,
              status: torch.Tensor | None = None) -> torch.Tensor:
     """out[i, :] = dequantised (fmt = block format) or copied (fmt = 0, f32 table) row tokens[i] of the table."""

@@ -31,14 +31,20 @@ DEQUANT_ONLY_FORMATS = (Q2_K, Q3_K, Q5_K)
 # the block layouts of GGUF model files (ggml), which ROCmForge does not decode: 100 + the ggml type id
 GGUF_Q4_0, GGUF_Q8_0, GGUF_Q4_K, GGUF_Q6_K = 102, 108, 112, 114
 GGUF_FORMATS = (GGUF_Q4_0, GGUF_Q8_0, GGUF_Q4_K, GGUF_Q6_K)
+# what the decoders of src/kernels/matmul/quantized/ read (q8_0.rs:18-56: int8 bytes; q4_k.rs:90-148: nibbles at
+# 32 + 20 * sub-block; q6_k.rs:90-148: the canonical stream; the K scales through common.rs:44-60): 200 + the id
+# of the format they are a variant of
+MM_Q8_0, MM_Q4_K, MM_Q6_K = 208, 212, 214
+MM_FORMATS = (MM_Q8_0, MM_Q4_K, MM_Q6_K)
 
 BLOCK_ELEMS = {Q2_K: 256, Q3_K: 256, Q5_K: 256, Q4_0: 32, Q8_0: 32, Q4_K: 256, Q6_K: 256, MXFP4: 32, MXFP6_E2M3: 32, MXFP6_E3M2: 32,
-               GGUF_Q4_0: 32, GGUF_Q8_0: 32, GGUF_Q4_K: 256, GGUF_Q6_K: 256}
+               GGUF_Q4_0: 32, GGUF_Q8_0: 32, GGUF_Q4_K: 256, GGUF_Q6_K: 256, MM_Q8_0: 32, MM_Q4_K: 256, MM_Q6_K: 256}
 BLOCK_BYTES = {Q2_K: 256, Q3_K: 256, Q5_K: 256, Q4_0: 20, Q8_0: 36, Q4_K: 256, Q6_K: 256, MXFP4: 17, MXFP6_E2M3: 25, MXFP6_E3M2: 25,
-               GGUF_Q4_0: 18, GGUF_Q8_0: 34, GGUF_Q4_K: 144, GGUF_Q6_K: 210}
+               GGUF_Q4_0: 18, GGUF_Q8_0: 34, GGUF_Q4_K: 144, GGUF_Q6_K: 210, MM_Q8_0: 36, MM_Q4_K: 256, MM_Q6_K: 256}
 NAMES = {Q2_K: "Q2_K", Q3_K: "Q3_K", Q5_K: "Q5_K", Q4_0: "Q4_0", Q8_0: "Q8_0", Q4_K: "Q4_K", Q6_K: "Q6_K", MXFP4: "MXFP4",
          MXFP6_E2M3: "MXFP6_E2M3", MXFP6_E3M2: "MXFP6_E3M2",
-         GGUF_Q4_0: "GGUF_Q4_0", GGUF_Q8_0: "GGUF_Q8_0", GGUF_Q4_K: "GGUF_Q4_K", GGUF_Q6_K: "GGUF_Q6_K"}
+         GGUF_Q4_0: "GGUF_Q4_0", GGUF_Q8_0: "GGUF_Q8_0", GGUF_Q4_K: "GGUF_Q4_K", GGUF_Q6_K: "GGUF_Q6_K",
+         MM_Q8_0: "MM_Q8_0", MM_Q4_K: "MM_Q4_K", MM_Q6_K: "MM_Q6_K"}
 
 
 def packed_bytes(fmt: int, n_elems: int) -> int:
@@ -83,6 +89,21 @@ def quantize_q8_0(w: np.ndarray) -> np.ndarray:
     out[:, 0:4] = d.astype("<f4").view(np.uint8).reshape(-1, 4)
     out[:, 4:36] = q.astype(np.uint8)
     return out.ravel()
+
+
+def quantize_mm_q8_0(w: np.ndarray) -> np.ndarray:
+    """The same decision rule with the bytes as two's-complement int8, which is how
+    src/kernels/matmul/quantized/q8_0.rs:18-56 reads them."""
+    out = quantize_q8_0(w).reshape(-1, 36).copy()
+    out[:, 4:36] ^= 0x80                                  # offset binary -> two's complement
+    return out.ravel()
+
+
+def synth_mm_q4_k(n_superblocks: int, rng: np.random.Generator) -> np.ndarray:
+    """Random super-blocks for the stride-20 reading (src/kernels/matmul/quantized/q4_k.rs:90-148): the same
+    scales and mins as synth_q4_k; every other byte is random, so the nibble bytes are random wherever they
+    are taken from."""
+    return synth_q4_k(n_superblocks, rng)
 
 
 def pack6_lsb(codes: np.ndarray) -> np.ndarray:
@@ -319,12 +340,12 @@ def random_blocks(fmt: int, n_blocks: int, rng: np.random.Generator, exp_range=(
         else:
             out[:, 208:210] = d[:, 0:2]
         return out.ravel()
-    if fmt in (Q4_0, Q8_0):
+    if fmt in (Q4_0, Q8_0, MM_Q8_0):
         s = (rng.standard_normal(n_blocks) * 0.01).astype("<f4")
         out[:, 0:4] = s.view(np.uint8).reshape(-1, 4)
-    elif fmt == Q4_K:
+    elif fmt in (Q4_K, MM_Q4_K):
         return synth_q4_k(n_blocks, rng)
-    elif fmt in (Q6_K, Q3_K, Q5_K):
+    elif fmt in (Q6_K, Q3_K, Q5_K, MM_Q6_K):
         s = (rng.standard_normal((n_blocks, 16)) * 0.01).astype(np.float16)
         out[:, 0:32] = s.view(np.uint8).reshape(-1, 32)
     elif fmt == Q2_K:                                     # f16 scales, then f16 mins
@@ -338,9 +359,13 @@ def random_blocks(fmt: int, n_blocks: int, rng: np.random.Generator, exp_range=(
 def make_weights(fmt: int, n: int, k: int, seed: int, std: float = 0.02) -> np.ndarray:
     """Seeded W[n,k] ~ N(0, std) quantised to ``fmt`` (Q4_K: synthetic blocks)."""
     rng = np.random.Generator(np.random.PCG64(seed))
-    if fmt == Q4_K:
+    if fmt in (Q4_K, MM_Q4_K):
         return synth_q4_k(n * k // 256, rng)
     w = (rng.standard_normal((n, k), dtype=np.float32) * np.float32(std))
+    if fmt == MM_Q8_0:
+        return quantize_mm_q8_0(w)
+    if fmt == MM_Q6_K:
+        return quantize_q6_k(w, rng)
     if fmt == Q4_0:
         return quantize_q4_0(w)
     if fmt == Q8_0:

@@ -17,23 +17,58 @@ def assert_bit_exact(got, want, what=""):
             f"got {np.asarray(got).ravel()[i]!r} (0x{g[i]:08x}) want {np.asarray(want).ravel()[i]!r} (0x{w[i]:08x})")
 
 
-# GEMV / GEMM tolerance: "max relative error 1e-3 with fp32 accumulation".
-# The error of element j is taken relative to max(|ref_j|, rms(ref)): plain
-# relative error wherever the reference is at least of typical size, and
-# relative to the typical size for the (arbitrarily small) outputs near zero,
-# where a pure ratio is meaningless for any summation order.
+# GEMV / GEMM tolerance: "max relative error 1e-3 with fp32 accumulation".  Three figures are computed:
+#   rel_err        max_j |y_j - ref_j| / max(|ref_j|, rms(ref)): plain relative error wherever the reference is
+#                  at least of typical size, relative to the typical size for outputs near zero;
+#   rel_err_plain  max_j |y_j - ref_j| / |ref_j| over the outputs with |ref_j| > rms(ref) / 10;
+#   rel_err_floor  max_j |y_j - ref_j| / max(|ref_j|, 1e-3 * rms(ref)): the same ratio with a floor a thousand
+#                  times lower.  Reported, not gated: among 10^4 outputs the smallest |ref_j| are about
+#                  1e-4 * rms, and there two fp32 summation orders of the SAME products already differ by several
+#                  1e-3 under this figure (the reference's own sequential fp32 sum is about sqrt(k) * 2^-24 * rms
+#                  away from the exact sum; tests/test_oracle_kat.py::test_tolerance_floor_of_fp32_summation
+#                  measures it), so it cannot tell a correct kernel from a wrong one.
+# A result passes when rel_err <= 1e-3 and rel_err_plain <= 1e-3.
 REL_TOL = 1e-3
 
 
+def _flat64(a):
+    return np.asarray(a, dtype=np.float64).ravel()
+
+
 def rel_err(got, ref):
-    got = np.asarray(got, dtype=np.float64).ravel()
-    ref = np.asarray(ref, dtype=np.float64).ravel()
-    rms = float(np.sqrt(np.mean(ref * ref))) if ref.size else 0.0
+    got, ref = _flat64(got), _flat64(ref)
+    if not ref.size:
+        return 0.0
+    rms = float(np.sqrt(np.mean(ref * ref)))
     den = np.maximum(np.abs(ref), rms if rms > 0 else 1.0)
-    return float(np.max(np.abs(got - ref) / den)) if ref.size else 0.0
+    return float(np.max(np.abs(got - ref) / den))
+
+
+def rel_err_plain(got, ref):
+    got, ref = _flat64(got), _flat64(ref)
+    if not ref.size:
+        return 0.0
+    rms = float(np.sqrt(np.mean(ref * ref)))
+    sel = np.abs(ref) > rms / 10 if rms > 0 else np.zeros(ref.shape, bool)
+    return float(np.max(np.abs(got[sel] - ref[sel]) / np.abs(ref[sel]))) if sel.any() else 0.0
+
+
+def rel_err_floor(got, ref):
+    got, ref = _flat64(got), _flat64(ref)
+    if not ref.size:
+        return 0.0
+    rms = float(np.sqrt(np.mean(ref * ref)))
+    den = np.maximum(np.abs(ref), 1e-3 * rms if rms > 0 else 1.0)
+    return float(np.max(np.abs(got - ref) / den))
+
+
+def error_report(got, ref):
+    return (f"max rel err {rel_err(got, ref):.2e} (floor rms), {rel_err_plain(got, ref):.2e} (plain, |ref| > rms/10), "
+            f"{rel_err_floor(got, ref):.2e} (floor 1e-3 rms, reported only)")
 
 
 def assert_close(got, ref, what="", tol=REL_TOL):
-    e = rel_err(got, ref)
+    e, p = rel_err(got, ref), rel_err_plain(got, ref)
     assert e <= tol, f"{what}: max relative error {e:.3e} > {tol:.1e}"
+    assert p <= tol, f"{what}: max plain relative error over |ref| > rms/10 is {p:.3e} > {tol:.1e}"
     return e

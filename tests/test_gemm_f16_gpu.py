@@ -5,7 +5,7 @@ reference's sequential fp32 matmul over the fp16 activations widened to f32)."""
 import numpy as np
 import pytest
 
-from helpers import assert_close
+from helpers import assert_close, error_report
 from rocmforge_amd import quantize as Q
 
 pytestmark = pytest.mark.gpu
@@ -111,6 +111,7 @@ def test_full_size_sampled(fmt, oracle, cuda):
     want = oracle.qmatmul_nk(fmt, w, a.astype(np.float32), m, n, k, rows=cols)
     got = f32[:, torch.from_numpy(cols).to(cuda)].cpu().numpy()
     assert_close(got, want, "sampled fp32")
+    print(f"{Q.NAMES[fmt]} 512x14336x4096, {cols.size} sampled columns, fp32 out: {error_report(got, want)}")
     got16 = f16[:, torch.from_numpy(cols).to(cuda)].float().cpu().numpy()
     assert_close(got16, want, "sampled fp16", tol=1e-3 + 2.0 ** -11)      # one fp16 rounding on top
     wsum = oracle.dequantize(fmt, w, n * k).reshape(n, k).astype(np.float64).sum(axis=0)

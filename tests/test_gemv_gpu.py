@@ -5,7 +5,7 @@ import ctypes as C
 import numpy as np
 import pytest
 
-from helpers import assert_close
+from helpers import assert_close, error_report
 from rocmforge_amd import quantize as Q
 
 pytestmark = pytest.mark.gpu
@@ -98,8 +98,35 @@ def test_gemv_baseline_configs(fmt, n, k, m, cfg, oracle, cuda):
     x = x_for(m, k, 20260100 + cfg)
     got = gpu_gemv(fmt, w, x, n, k, cuda)
     want = oracle.qmatmul_nk(fmt, w, x, m, n, k)
-    e = assert_close(got.reshape(m, n), want, f"config {cfg} {Q.NAMES[fmt]} m={m}")
-    print(f"config {cfg} {Q.NAMES[fmt]} m={m}: max rel err {e:.2e}")
+    assert_close(got.reshape(m, n), want, f"config {cfg} {Q.NAMES[fmt]} m={m}")
+    print(f"config {cfg} {Q.NAMES[fmt]} m={m}: {error_report(got.reshape(m, n), want)}")
+
+
+# The vocabulary projection (LM head), the largest GEMV of a decode step: 128256 x 4096 (525 MB as Q4_K).  Sampled
+# rows against the oracle (first and last rows of the matrix, of a team's and a workgroup's range, and random ones)
+# and a checksum over every output: sum_n y[n] = x . sum_n W[n, :], the column sums taken from the oracle's dequantisation.
+@pytest.mark.timeout(600)
+@pytest.mark.parametrize("fmt", [Q.Q4_K, Q.GGUF_Q4_K])
+def test_lm_head_shape_sampled(fmt, oracle, cuda):
+    n, k = 128256, 4096
+    rng = np.random.default_rng(20260200 + fmt)
+    w = Q.random_blocks(fmt, n * k // 256, rng)
+    x = x_for(1, k, 20260201)
+    got = gpu_gemv(fmt, w, x, n, k, cuda)
+    rows = np.unique(np.concatenate([np.arange(0, 40), np.arange(n - 40, n), np.arange(62600, 62680),
+                                     rng.integers(0, n, 400)]))
+    want = oracle.qmatmul_nk(fmt, w, x, 1, n, k, rows=rows)[0]
+    assert_close(got[rows], want, f"{Q.NAMES[fmt]} LM head, {rows.size} sampled rows")
+    print(f"{Q.NAMES[fmt]} 128256x4096, {rows.size} rows: {error_report(got[rows], want)}")
+    rb = Q.BLOCK_BYTES[fmt] * k // 256
+    colsum = np.zeros(k, np.float64)
+    step = 8016                                               # 16 chunks of rows
+    for r0 in range(0, n, step):
+        r1 = min(n, r0 + step)
+        colsum += oracle.dequantize(fmt, w[r0 * rb:r1 * rb], (r1 - r0) * k).reshape(-1, k).astype(np.float64).sum(axis=0)
+    total, want_total = float(got.astype(np.float64).sum()), float(x.astype(np.float64) @ colsum)
+    scale = float(np.sqrt(n) * np.sqrt(np.mean(got.astype(np.float64) ** 2)))   # size of a sum of n outputs
+    assert abs(total - want_total) <= 1e-4 * scale, (total, want_total, scale)
 
 
 def test_q4_k_onesided_real_data(oracle, cuda):

@@ -80,3 +80,44 @@ def test_prefill_gemms_replay(cuda):
         step()
         torch.cuda.synchronize()
         assert torch.equal(got, out) and torch.equal(got_mx, out_mx)
+
+
+def test_capture_refuses_to_allocate_temporaries(cuda):
+    """A stream that has never run the call has no kept temporary: under capture the call must fail with
+    RFQ_E_UNSUPPORTED instead of allocating (or growing, which would free memory an earlier graph holds)."""
+    import torch
+    from rocmforge_amd import _lib, ops
+    m, n, k = 64, 128, 512
+    w = torch.from_numpy(Q.make_weights(Q.Q4_K, n, k, seed=8)).to(cuda)
+    a = torch.zeros((m, k), dtype=torch.float16, device=cuda)
+    a2 = torch.zeros((4 * m, k), dtype=torch.float16, device=cuda)
+    out = torch.empty((m, n), dtype=torch.float16, device=cuda)
+    out2 = torch.empty((4 * m, n), dtype=torch.float16, device=cuda)
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        ops.gemm_f16(Q.Q4_K, w, a, n, k, out=out)          # the stream now keeps a temporary for m = 64
+        torch.cuda.synchronize()
+        refused = None
+        with torch.cuda.graph(graph, stream=side):
+            ops.gemm_f16(Q.Q4_K, w, a, n, k, out=out)      # fits: captured
+            try:
+                ops.gemm_f16(Q.Q4_K, w, a2, n, k, out=out2)  # four times the rows: would have to grow
+            except _lib.RfqError as e:
+                refused = e
+    assert refused is not None and refused.status == _lib.E_UNSUPPORTED and "captur" in refused.message
+    a.copy_(torch.from_numpy(np.random.default_rng(9).standard_normal((m, k)).astype(np.float16)))
+    torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    got = out.clone()
+    # growing afterwards (eagerly) must leave the captured graph's buffer alive: replay again and compare
+    with torch.cuda.stream(side):
+        ops.gemm_f16(Q.Q4_K, w, a2, n, k, out=out2)
+        torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(out, got)
+    want = ops.gemm_f16(Q.Q4_K, w, a, n, k)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)

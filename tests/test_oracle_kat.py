@@ -552,3 +552,20 @@ def test_dequant_rms_norm_and_mlp_are_compositions(oracle):
             got = oracle.mlp_swiglu_q(fmt, wg, wu, fmt, wd, x, norm, 1e-5, 2, hidden, inter)
             scale = np.sqrt((ref * ref).mean())
             assert np.max(np.abs(got - ref)) / scale < 1e-4
+
+
+def test_tolerance_floor_of_fp32_summation(oracle):
+    """What the error figures of tests/helpers.py read for the reference's own arithmetic: the sequential fp32 sum
+    of cpu_matmul_f32 (src/tensor/matmul.rs:219-233) against the exact (float64) sum of the same f32 products, at
+    the headline shape's k.  Relative to max(|y|, rms) the reference is ~1e-6 from the exact result; with the floor
+    lowered to 1e-3 * rms the same deviation reads above 1e-3 on the outputs nearest zero, so that figure cannot
+    serve as a pass criterion for any fp32 implementation that sums in another order."""
+    from helpers import rel_err, rel_err_floor, rel_err_plain
+    rng = np.random.default_rng(2026)
+    n, k = 14336, 4096
+    w = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
+    x = rng.standard_normal(k).astype(np.float32)
+    seq = oracle.matmul_nk_f32(x, w, 1, n, k)[0]
+    exact = w.astype(np.float64) @ x.astype(np.float64)
+    assert rel_err(seq, exact) < 2e-5 and rel_err_plain(seq, exact) < 1e-4
+    assert rel_err_floor(seq, exact) > 1e-3
