@@ -313,6 +313,22 @@ RFQ_API int rfq_mlp_swiglu(int fmt_gate_up, const void *d_gate_w, const void *d_
 RFQ_API int rfq_gemm_f16(int fmt, const void *d_w, size_t w_bytes, const void *d_a_f16, void *d_out,
                  int out_dtype, int m, int n, int k, void *stream);
 
+/* rfq_gemm_f16 for callers that cannot allocate device memory: code under
+ * stream capture, tight serving loops, harnesses that forbid hipMalloc.  No
+ * counterpart in the reference.  Same arguments, same kernels and bit-identical
+ * results, but the temporaries (the activations in matrix-operand order, the
+ * Q4_K group sums) live in a 16 MiB array that is part of the library's device
+ * image, one copy per GPU, held until the process ends; the call allocates
+ * and frees nothing.  Shapes whose temporaries exceed the array fail with
+ * RFQ_E_SIZE: ceil(m / 32) * ceil(k / 64) * 4096 bytes, plus ceil(m / 32) * k * 4
+ * for RFQ_Q4_K (m * k up to about 7.8 million elements; 512 x 4096 takes 4.25 MiB).
+ * Every call on a GPU shares that GPU's array: calls that may overlap on one
+ * GPU (different streams, different threads) race; calls on one stream do not.
+ * The first call on each device looks the array's address up (make that call
+ * outside stream capture). */
+RFQ_API int rfq_gemm_f16_static(int fmt, const void *d_w, size_t w_bytes, const void *d_a_f16, void *d_out,
+                                int out_dtype, int m, int n, int k, void *stream);
+
 /* MXFP matrices feed the gfx950 block-scaled matrix instruction, whose element
  * and scale encodings differ from the bytes ROCmForge stores (signed exponent
  * byte, its own E2M1/E2M3 value tables, a +-8 / +-7.5 clamp).  A matrix

@@ -54,6 +54,7 @@ _SIGNATURES = {
     "rfq_mlp_scratch_bytes": ([_i, _i, _i], _sz),
     "rfq_mlp_swiglu": ([_i, _vp, _vp, _sz, _i, _vp, _sz, _vp, _vp, C.c_float, _vp, _i, _i, _i, _vp, _sz, _vp], _i),
     "rfq_gemm_f16": ([_i, _vp, _sz, _vp, _vp, _i, _i, _i, _i, _vp], _i),
+    "rfq_gemm_f16_static": ([_i, _vp, _sz, _vp, _vp, _i, _i, _i, _i, _vp], _i),
     "rfq_mx_prepared_bytes": ([_i, _i, _i, _i], _sz),
     "rfq_mx_prepare": ([_i, _i, _vp, _sz, _i, _i, _vp, _sz, C.POINTER(C.c_int), _vp], _i),
     "rfq_gemm_mx": ([_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _vp], _i),

@@ -415,7 +415,17 @@ int rfq_gemm_f16(int fmt, const void *d_w, size_t w_bytes, const void *d_a_f16, 
     if (rc != RFQ_OK) return rc;
     if (out_dtype != RFQ_F32 && out_dtype != RFQ_F16)
         return fail(RFQ_E_BADARG, "rfq_gemm_f16: out_dtype %d is neither F32 nor F16", out_dtype);
-    return launch_gemm_f16(fmt, (const uint8_t *)d_w, d_a_f16, d_out, out_dtype, m, n, k, (hipStream_t)stream);
+    return launch_gemm_f16(fmt, (const uint8_t *)d_w, d_a_f16, d_out, out_dtype, m, n, k, false, (hipStream_t)stream);
+}
+
+int rfq_gemm_f16_static(int fmt, const void *d_w, size_t w_bytes, const void *d_a_f16, void *d_out, int out_dtype, int m,
+                        int n, int k, void *stream)
+{
+    int rc = check_gemv("rfq_gemm_f16_static", fmt, d_w, w_bytes, true, d_a_f16, d_out, m, n, k);
+    if (rc != RFQ_OK) return rc;
+    if (out_dtype != RFQ_F32 && out_dtype != RFQ_F16)
+        return fail(RFQ_E_BADARG, "rfq_gemm_f16_static: out_dtype %d is neither F32 nor F16", out_dtype);
+    return launch_gemm_f16(fmt, (const uint8_t *)d_w, d_a_f16, d_out, out_dtype, m, n, k, true, (hipStream_t)stream);
 }
 
 size_t rfq_mx_prepared_bytes(int fmt, int kind, int rows, int k)

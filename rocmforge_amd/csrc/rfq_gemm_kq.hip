@@ -45,6 +45,13 @@
 
 #include "rfq_common.hpp"
 
+// Temporary memory of rfq_gemm_f16_static, the entry point for callers that cannot allocate (stream capture,
+// serving loops): the arranged activations and the Q4_K group sums of one call.  Every GPU the library runs on
+// holds its own copy of this array until the process ends.  Host code never uses the array's name as an address:
+// static_scratch() resolves the copy of the current device once and hands out that pointer.
+constexpr size_t RFQ_STATIC_SCRATCH_BYTES = (size_t)16 << 20;
+static __device__ __align__(256) uint8_t scratch[RFQ_STATIC_SCRATCH_BYTES];
+
 namespace rfq {
 namespace {
 
@@ -873,7 +880,7 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
 }
 
 template <int FMT, bool OUT_F16>
-int launch_cfg(const uint8_t *w, const void *a, void *out, int m, int n, int k, hipStream_t s)
+int launch_cfg(const uint8_t *w, const void *a, void *out, int m, int n, int k, uint8_t *static_tmp, hipStream_t s)
 {
     constexpr int LDS = 4 * W_BYTES + BN * 48;                  // four weight stages + the Q4_K min fragment
     static_assert(LDS <= 160 * 1024, "LDS budget");
@@ -889,9 +896,15 @@ int launch_cfg(const uint8_t *w, const void *a, void *out, int m, int n, int k, 
     const int tiles32 = (m + 31) / 32, nst = (k + BK - 1) / BK;
     const size_t at_bytes = (size_t)tiles32 * nst * 4096;
     const size_t s2_bytes = FMT == RFQ_Q4_K ? (size_t)tiles32 * (k / 256) * 1024 : 0;
-    uint8_t *tmp = nullptr;
+    uint8_t *tmp = static_tmp;
     bool transient = false;
-    if (int rc = workspace(s, at_bytes + s2_bytes, &tmp, &transient)) return rc;
+    if (static_tmp != nullptr) {
+        if (at_bytes + s2_bytes > RFQ_STATIC_SCRATCH_BYTES)
+            return fail(RFQ_E_SIZE, "rfq_gemm_f16_static: m=%d k=%d needs %zu bytes of temporary memory, the static buffer holds %zu",
+                        m, k, at_bytes + s2_bytes, RFQ_STATIC_SCRATCH_BYTES);
+    } else if (int rc = workspace(s, at_bytes + s2_bytes, &tmp, &transient)) {
+        return rc;
+    }
     v4u *at = reinterpret_cast<v4u *>(tmp);
     _Float16 *s2 = reinterpret_cast<_Float16 *>(tmp + at_bytes);
     hipLaunchKernelGGL((arrange_a_kernel<FMT == RFQ_Q4_K>), dim3((unsigned)(tiles32 * ((nst + 3) / 4))), dim3(256), 0, s,
@@ -907,10 +920,30 @@ int launch_cfg(const uint8_t *w, const void *a, void *out, int m, int n, int k, 
 }
 
 template <int FMT>
-int launch_fmt(const uint8_t *w, const void *a, void *out, int out_dtype, int m, int n, int k, hipStream_t s)
+int launch_fmt(const uint8_t *w, const void *a, void *out, int out_dtype, int m, int n, int k, uint8_t *static_tmp,
+               hipStream_t s)
 {
-    return out_dtype == RFQ_F16 ? launch_cfg<FMT, true>(w, a, out, m, n, k, s)
-                                : launch_cfg<FMT, false>(w, a, out, m, n, k, s);
+    return out_dtype == RFQ_F16 ? launch_cfg<FMT, true>(w, a, out, m, n, k, static_tmp, s)
+                                : launch_cfg<FMT, false>(w, a, out, m, n, k, static_tmp, s);
+}
+
+// The address of this device's copy of `scratch`, resolved on the first call on each device.
+int static_scratch(uint8_t **out)
+{
+    static std::mutex mu;
+    static uint8_t *ptrs[64];
+    int dev = 0;
+    RFQ_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= 64) return fail(RFQ_E_BADARG, "rfq_gemm_f16_static: device %d outside 0..63", dev);
+    std::lock_guard<std::mutex> lock(mu);
+    if (ptrs[dev] == nullptr) {
+        void *p = nullptr;
+        RFQ_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (p == nullptr) return fail(RFQ_E_HIP, "rfq_gemm_f16_static: the static buffer has no device address");
+        ptrs[dev] = static_cast<uint8_t *>(p);
+    }
+    *out = ptrs[dev];
+    return RFQ_OK;
 }
 
 } // namespace
@@ -992,8 +1025,12 @@ int release_workspaces()
 }
 
 int launch_gemm_f16(int fmt, const uint8_t *d_w, const void *d_a, void *d_out, int out_dtype, int m, int n, int k,
-                    hipStream_t s)
+                    bool use_static_scratch, hipStream_t s)
 {
+    uint8_t *st = nullptr;
+    if (use_static_scratch) {
+        if (int rc = static_scratch(&st)) return rc;
+    }
     if (out_dtype != RFQ_F16 && out_dtype != RFQ_F32)
         return fail(RFQ_E_BADARG, "rfq_gemm_f16: out_dtype %d (want RFQ_F32 or RFQ_F16)", out_dtype);
     if ((reinterpret_cast<uintptr_t>(d_a) & 15u) != 0 || k % 8 != 0)
@@ -1001,14 +1038,14 @@ int launch_gemm_f16(int fmt, const uint8_t *d_w, const void *d_a, void *d_out, i
     if ((reinterpret_cast<uintptr_t>(d_w) & 3u) != 0)               // buffer loads of whole dwords
         return fail(RFQ_E_BADARG, "rfq_gemm_f16: weights must be 4-byte aligned");
     switch (fmt) {
-    case RFQ_Q4_0: return launch_fmt<RFQ_Q4_0>(d_w, d_a, d_out, out_dtype, m, n, k, s);
-    case RFQ_Q8_0: return launch_fmt<RFQ_Q8_0>(d_w, d_a, d_out, out_dtype, m, n, k, s);
-    case RFQ_Q4_K: return launch_fmt<RFQ_Q4_K>(d_w, d_a, d_out, out_dtype, m, n, k, s);
-    case RFQ_Q6_K: return launch_fmt<RFQ_Q6_K>(d_w, d_a, d_out, out_dtype, m, n, k, s);
-    case RFQ_GGUF_Q4_0: return launch_fmt<RFQ_GGUF_Q4_0>(d_w, d_a, d_out, out_dtype, m, n, k, s);
-    case RFQ_GGUF_Q8_0: return launch_fmt<RFQ_GGUF_Q8_0>(d_w, d_a, d_out, out_dtype, m, n, k, s);
-    case RFQ_GGUF_Q4_K: return launch_fmt<RFQ_GGUF_Q4_K>(d_w, d_a, d_out, out_dtype, m, n, k, s);
-    case RFQ_GGUF_Q6_K: return launch_fmt<RFQ_GGUF_Q6_K>(d_w, d_a, d_out, out_dtype, m, n, k, s);
+    case RFQ_Q4_0: return launch_fmt<RFQ_Q4_0>(d_w, d_a, d_out, out_dtype, m, n, k, st, s);
+    case RFQ_Q8_0: return launch_fmt<RFQ_Q8_0>(d_w, d_a, d_out, out_dtype, m, n, k, st, s);
+    case RFQ_Q4_K: return launch_fmt<RFQ_Q4_K>(d_w, d_a, d_out, out_dtype, m, n, k, st, s);
+    case RFQ_Q6_K: return launch_fmt<RFQ_Q6_K>(d_w, d_a, d_out, out_dtype, m, n, k, st, s);
+    case RFQ_GGUF_Q4_0: return launch_fmt<RFQ_GGUF_Q4_0>(d_w, d_a, d_out, out_dtype, m, n, k, st, s);
+    case RFQ_GGUF_Q8_0: return launch_fmt<RFQ_GGUF_Q8_0>(d_w, d_a, d_out, out_dtype, m, n, k, st, s);
+    case RFQ_GGUF_Q4_K: return launch_fmt<RFQ_GGUF_Q4_K>(d_w, d_a, d_out, out_dtype, m, n, k, st, s);
+    case RFQ_GGUF_Q6_K: return launch_fmt<RFQ_GGUF_Q6_K>(d_w, d_a, d_out, out_dtype, m, n, k, st, s);
     default: return fail(RFQ_E_UNSUPPORTED, "rfq_gemm_f16: no fp16 matrix-core kernel for format %d", fmt);
     }
 }

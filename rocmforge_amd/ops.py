@@ -179,6 +179,21 @@ def gemm_f16(fmt: int, w: torch.Tensor, a: torch.Tensor, n: int, k: int, out_dty
     return out
 
 
+def gemm_f16_static(fmt: int, w: torch.Tensor, a: torch.Tensor, n: int, k: int, out: torch.Tensor,
+                    out_dtype=torch.float16) -> torch.Tensor:
+    """rfq_gemm_f16 with its temporaries in the library's static device array: the call allocates nothing, so the
+    caller passes ``out``."""
+    w = _dev_u8(w)
+    if not (a.is_cuda and a.dtype == torch.float16 and a.is_contiguous() and a.dim() == 2 and a.shape[1] == k):
+        raise ValueError("a must be a contiguous [m, k] float16 device tensor")
+    m = a.shape[0]
+    code = {torch.float32: _lib.F32, torch.float16: _lib.F16}[out_dtype]
+    if not (out.is_cuda and out.dtype == out_dtype and out.is_contiguous() and out.numel() == m * n):
+        raise ValueError("out must be a contiguous device tensor of m * n elements of out_dtype")
+    check(lib().rfq_gemm_f16_static(fmt, _ptr(w), w.numel(), _ptr(a), _ptr(out), code, m, n, k, _stream()))
+    return out
+
+
 class MxOperand:
     """A [rows, k] MXFP matrix re-encoded for the block-scaled matrix core."""
 
