@@ -7,9 +7,14 @@ enough distinct weight copies that the 256 MB last-level cache cannot hold
 them, so every step streams its 58.7 MB from HBM ("cold").  The metric is
 algorithmic bytes (packed W as stored + x + y) per second.
 
-Prints ONE JSON line.  Extra keys: `roofline` (HIP-event timing of the same
-launches against the 8 TB/s HBM peak), `cpu_baseline` (the CPU oracle timed on
-this host), `also` (the other configurations, one short run each).
+Prints ONE JSON line.  `value` and `roofline.achieved` come from one clock: HIP
+events recorded on the launch stream around the K timed launches (the host's
+wall clock around the same region, which adds the final synchronisation's
+wake-up -- tens of microseconds, as much as the work itself at K = 20 -- is
+reported as `wall_ms_per_step`).  Extra keys: `roofline` (with the name of the
+kernel the dispatch took, read back from the library, and the time of a kernel
+that only reads the same bytes), `cpu_baseline` (the CPU oracle timed on this
+host), `also` (the other configurations, one short run each).
 """
 from __future__ import annotations
 
@@ -30,6 +35,9 @@ CACHE_BYTES = 256 << 20
 # profiler counters scaled by a copy kernel of known size
 # (profiles/gemv_q4k_14336x4096_hbm_counters.txt): 57,584.4 KiB read + 64.0 KiB written.
 MEASURED_TRAFFIC_BYTES = 59031938
+TRAFFIC_SOURCE = "profiles/gemv_q4k_14336x4096_hbm_counters.txt"
+# launch shapes of the read-only kernel that the floor is taken over (workgroups, threads, loads in flight, non-temporal)
+READ_FLOOR_SHAPES = ((256, 1024, 8, 1), (256, 1024, 16, 1), (512, 512, 8, 1), (256, 1024, 8, 0))
 
 
 def algorithmic_bytes(fmt, n, k, m, Q):
@@ -58,16 +66,35 @@ def time_gemv(torch, fmt, n, k, m, copies, steps, warmup, Q, seed):
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     ms = C.c_float(0)
     L = _lib.lib()
-    # untimed warm-up (also loads the code object), then barrier
-    _lib.check(L.rfq_bench_gemv(fmt, ptrs, copies, w.size, C.c_void_p(dx.data_ptr()), C.c_void_p(y.data_ptr()),
-                                m, n, k, 0, max(warmup, 1), stream, C.byref(ms)))
+    # the warm-up launches and the timed ones are one native loop: the rotation through the weight copies
+    # continues across the boundary, so the first timed steps do not meet copies the warm-up touched last
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     _lib.check(L.rfq_bench_gemv(fmt, ptrs, copies, w.size, C.c_void_p(dx.data_ptr()), C.c_void_p(y.data_ptr()),
-                                m, n, k, 0, steps, stream, C.byref(ms)))
+                                m, n, k, max(warmup, 1), steps, stream, C.byref(ms)))
     torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
+    wall = (time.perf_counter() - t0) * steps / (steps + max(warmup, 1))
     return wall, ms.value / 1e3, w, x, y.cpu().numpy()
+
+
+def read_floor(torch, nbytes, copies, steps, warmup):
+    """Device seconds per launch of a kernel that only reads `nbytes` (rotating copies, back-to-back launches like
+    the GEMV): the floor of a one-launch step over the same bytes.  The best of a few launch shapes."""
+    import ctypes as C
+
+    from rocmforge_amd import _lib
+    dev = torch.device("cuda:0")
+    bufs = [torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device=dev) for _ in range(copies)]
+    ptrs = (C.c_void_p * copies)(*[b.data_ptr() for b in bufs])
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    ms, best = C.c_float(0), None
+    for blocks, threads, depth, nt in READ_FLOOR_SHAPES:
+        _lib.check(_lib.lib().rfq_bench_read_floor(ptrs, copies, nbytes, blocks, threads, nt, depth, warmup, steps, stream,
+                                                   C.byref(ms)))
+        t = ms.value / 1e3 / steps
+        if best is None or t < best[0]:
+            best = (t, f"{blocks} x {threads} threads, {depth} loads in flight, {'non-temporal' if nt else 'plain'}")
+    return best
 
 
 def time_dequant(torch, fmt, n, k, steps, warmup, Q, seed):
@@ -197,7 +224,12 @@ def time_host_path(torch, fmt, w, x, n, k):
             "pinned_copy_GB/s": round(nb / t_pin / 1e9, 1), "matmul_host_weights_ms": round(t_mm * 1e3, 3)}
 
 
-def cpu_baseline(fmt, w, x, n, k, budget_s=12.0):
+def _omp_threads(nthreads):
+    import ctypes as C
+    C.CDLL("libgomp.so.1").omp_set_num_threads(int(nthreads))
+
+
+def cpu_baseline(fmt, w, x, n, k, budget_s=8.0):
     """The CPU oracle (dequantise everything, then the sequential fp32 matmul)
     on one host thread, repeated until ~budget_s of CPU work."""
     import ctypes as C
@@ -206,8 +238,7 @@ def cpu_baseline(fmt, w, x, n, k, budget_s=12.0):
 
     import oracle
     L = oracle.lib()
-    gomp = C.CDLL("libgomp.so.1")
-    gomp.omp_set_num_threads(1)
+    _omp_threads(1)
     wd = np.empty(n * k, np.float32)
     c = np.empty(n, np.float32)
     reps, spent = 0, 0.0
@@ -218,8 +249,69 @@ def cpu_baseline(fmt, w, x, n, k, budget_s=12.0):
         assert rc == 0
         spent += time.perf_counter() - t
         reps += 1
-    gomp.omp_set_num_threads(os.cpu_count() or 1)
+    _omp_threads(os.cpu_count() or 1)
     return spent / reps, reps, c
+
+
+def cpu_baseline_more(Q, fmt, w, x, n, k, threads):
+    """The other legs of the CPU baseline, each a few repetitions (about 10 s together):
+      * the headline GEMV with `threads` OpenMP threads (rows spread over threads, each row dequantised and
+        multiplied by its thread; the reference itself is single-threaded);
+      * dequantisation alone of a 4096 x 4096 tensor in Q4_0 and Q8_0, one thread, beside the figures the reference
+        publishes for exactly that (benchmarks/baselines/rdna3-baseline.json:187-237: 12.8 ms and 15.2 ms);
+      * the two prefill GEMMs at M = 1 and M = 4 rows (dequantise all of W once, then the sequential fp32 matmul
+        per row, one thread), with the linear extrapolation to their full M labelled as such."""
+    import ctypes as C
+
+    import numpy as np
+
+    import oracle
+    L = oracle.lib()
+    p = lambda a: a.ctypes.data_as(C.c_void_p)
+
+    def best_of(f, reps):
+        t = 1e30
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            f()
+            t = min(t, time.perf_counter() - t0)
+        return t
+
+    out = {}
+    _omp_threads(threads)
+    y = np.empty(n, np.float32)
+    t = best_of(lambda: L.rf_qmatmul_nk(fmt, p(w), w.size, p(x), 1, n, k, None, 0, p(y)), 5)
+    out["gemv_all_threads"] = {"threads": threads, "ms_per_step": round(t * 1e3, 2),
+                               "GB/s": round((w.size + 4 * k + 4 * n) / t / 1e9, 2),
+                               "what": "the same GEMV, rows spread over OpenMP threads (per-row dequantise + dot)"}
+    _omp_threads(1)
+    for name, f, ref_ms in (("Q4_0", Q.Q4_0, 12.8), ("Q8_0", Q.Q8_0, 15.2)):
+        wq = Q.make_weights(f, 4096, 4096, seed=20260021)
+        dst = np.empty(4096 * 4096, np.float32)
+        t = best_of(lambda: L.rf_dequantize(f, p(wq), wq.size, dst.size, p(dst)), 5)
+        out[f"dequant_{name}_4096x4096"] = {"ms": round(t * 1e3, 2), "Gelem/s": round(dst.size / t / 1e9, 2), "threads": 1,
+                                            "reference_published_ms": ref_ms}
+    rng = np.random.Generator(np.random.PCG64(20260061))
+    for name, f, gm, gn, gk in (("Q4_K_gemm_512x4096x14336", Q.Q4_K, 512, 14336, 4096),
+                                ("MXFP4_gemm_2048x8192x28672", Q.MXFP4, 2048, 28672, 8192)):
+        slab = Q.make_weights(f, 4096 if gn % 4096 == 0 else gn, gk, seed=20260062)
+        wq = np.tile(slab, gn // 4096) if gn % 4096 == 0 else slab
+        wd = np.empty(gn * gk, np.float32)
+        res = {}
+        for m in (1, 4):
+            a = rng.standard_normal((m, gk), dtype=np.float32)
+            c = np.empty(m * gn, np.float32)
+            t = best_of(lambda: L.rf_qmatmul_nk_staged(f, p(wq), wq.size, p(a), m, gn, gk, p(wd), p(c)), 1 if gn > 20000 else 2)
+            res[f"m{m}_ms"] = round(t * 1e3, 1)
+        per_row = (res["m4_ms"] - res["m1_ms"]) / 3.0
+        fixed = res["m1_ms"] - per_row
+        res["extrapolated_full_m_ms"] = round(fixed + per_row * gm, 1)
+        res["extrapolation"] = f"linear in M from M = 1 and M = 4 (dequantise once + {gm} rows of the fp32 matmul), not measured"
+        res["extrapolated_GFLOP/s"] = round(2.0 * gm * gn * gk / (res["extrapolated_full_m_ms"] * 1e-3) / 1e9, 2)
+        res["threads"] = 1
+        out[name] = res
+    _omp_threads(os.cpu_count() or 1)
+    return out
 
 
 def main():
@@ -280,9 +372,12 @@ def main():
     copies = -(-int(2.5 * CACHE_BYTES) // wbytes)          # 11 copies, 646 MB > 2.5x the last-level cache
     abytes = algorithmic_bytes(fmt, N, K, 1, Q)
     wall, dev_s, w, x, y = time_gemv(torch, fmt, N, K, 1, copies, args.steps, args.warmup, Q, 20260003)
-    ms_per_step = wall / args.steps * 1e3
-    value = abytes / (wall / args.steps) / 1e9
+    from rocmforge_amd import _lib
+    kernel_name = _lib.lib().rfq_bench_last_gemv_kernel().decode()
+    ms_per_step = dev_s / args.steps * 1e3
     achieved = abytes / (dev_s / args.steps) / 1e9
+    value = achieved
+    floor_s, floor_shape = read_floor(torch, wbytes, copies, min(args.steps, 500), min(args.warmup, 50))
 
     # warm variant (one copy, cache-resident) for the record
     dev_w = None
@@ -297,6 +392,8 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 6),
+        "wall_ms_per_step": round(wall / args.steps * 1e3, 6),
+        "value_clock": "HIP events on the launch stream around the timed launches (roofline.achieved is the same figure)",
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -307,7 +404,10 @@ def main():
                    "algorithmic_bytes_per_step": abytes, "weight_copies": copies},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
-                     "kernel": "gemv_idot_kernel<Q4_K,1,2,7>", "avg_launch_us": round(dev_s / args.steps * 1e6, 3),
+                     "traffic_source": TRAFFIC_SOURCE,
+                     "kernel": kernel_name, "avg_launch_us": round(dev_s / args.steps * 1e6, 3),
+                     "read_only_kernel_us": round(floor_s * 1e6, 3), "read_only_kernel": floor_shape,
+                     "over_read_only_kernel": round(dev_s / args.steps / floor_s - 1.0, 4),
                      "warm_cache_gbs": round(abytes / (dev_w / args.steps) / 1e9, 1) if dev_w else None},
     }
 
@@ -370,10 +470,13 @@ def main():
         ref = c.astype(np.float64)
         rms = float(np.sqrt(np.mean(ref * ref)))
         err = float(np.max(np.abs(y[0] - ref) / np.maximum(np.abs(ref), rms)))
+        threads = min(os.cpu_count() or 1, 16)
         out["cpu_baseline"] = {"value": round(abytes / t_cpu / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
                                "sample": f"the full 14336x4096 GEMV (dequantise all weights to f32, then the sequential "
                                          f"fp32 matmul), {reps} repetitions on one host thread",
-                               "ms_per_step": round(t_cpu * 1e3, 2), "gpu_vs_cpu_max_rel_err": float(f"{err:.3e}")}
+                               "ms_per_step": round(t_cpu * 1e3, 2), "gpu_vs_cpu_max_rel_err": float(f"{err:.3e}"),
+                               "host_cpus": os.cpu_count(), "compiler_flags": "gcc -O2 -ffp-contract=off -fno-fast-math -fopenmp",
+                               "more": cpu_baseline_more(Q, fmt, w, x[0], N, K, threads)}
     print(json.dumps(out), flush=True)
 
 

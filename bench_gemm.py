@@ -4,10 +4,12 @@ MXFP4 GEMM at M=2048, K=8192, N=28672 (bf16 out) and the MXFP6-weight variant,
 plus the Q4_K fp16 GEMM at M=512, K=4096, N=14336 when that kernel is built.
 FLOPs = 2*M*N*K; peaks: 10.1 PFLOP/s (FP4 scaled MFMA), 5.0 (FP8), 2.5 (fp16).
 
-Each configuration runs `warmup` untimed launches first (20 to 30 ms): the
-launches of the first tens of milliseconds after an idle period run 5-15 %
-slower than the steady state (the part's clocks ramp), and the timed launches
-should not include that.
+Each configuration runs at most 40 untimed launches, then `steps` timed ones; the figure is the average over
+all timed launches (the launches of the first tens of milliseconds after an idle period run 5-15 % slower than
+the steady state: the part's clocks ramp, and the timed region is long enough to carry that).  The MXFP4 GEMM
+is reported three ways: on operands from the reference's packer (which emits only codes {0, 1, 8, 9}), on
+full-entropy operands (every code of a four-octave window, both signs), and as a prefill step that re-encodes
+the raw activations for the matrix core before every GEMM.
 """
 from __future__ import annotations
 
@@ -23,49 +25,68 @@ def _gauss(rows, k, seed, std):
     return rng.standard_normal((rows, k), dtype=np.float32) * np.float32(std)
 
 
-def mx_gemm(torch, w_fmt, m=2048, n=28672, k=8192, steps=50, warmup=150):
+def mx_gemm(torch, w_fmt, m=2048, n=28672, k=8192, steps=200, warmup=40, data="packer"):
     from rocmforge_amd import _lib, ops, quantize as Q
     dev = torch.device("cuda:0")
-    a_raw = Q.pack_mxfp4(_gauss(m, k, 20260005, 1.0))
     slab_rows = 4096
-    pack = Q.pack_mxfp4 if w_fmt == Q.MXFP4 else Q.pack_mxfp6
-    w_raw = np.tile(pack(_gauss(slab_rows, k, 20260015 + w_fmt, 0.02)), n // slab_rows)
+    if data == "packer":
+        a_raw = Q.pack_mxfp4(_gauss(m, k, 20260005, 1.0))
+        pack = Q.pack_mxfp4 if w_fmt == Q.MXFP4 else Q.pack_mxfp6
+        w_raw = np.tile(pack(_gauss(slab_rows, k, 20260015 + w_fmt, 0.02)), n // slab_rows)
+    else:                                                     # every code of a four-octave window, random exponents
+        rng = np.random.Generator(np.random.PCG64(20260065))
+        a_raw = Q.mxfp4_window_blocks(rng, m * k // 32, (-3, 3), zero_blocks=0.0)
+        w_raw = Q.mxfp4_window_blocks(rng, n * k // 32, (-9, -3), zero_blocks=0.0)
     a_dev, w_dev = torch.from_numpy(a_raw).to(dev), torch.from_numpy(w_raw).to(dev)
     A = ops.MxOperand(Q.MXFP4, a_dev, m, k)
     W = ops.MxOperand(w_fmt, w_dev, n, k)
-
-    def prepare_us(fmt, raw, rows, kind):
-        # re-encoding into the matrix core's operand order, reported beside the GEMM, never inside it:
-        # device time of back-to-back calls that do not synchronise (8-bit kinds, and the 4-bit kind
-        # requested unchecked, which is how activations are prepared per prefill)
-        req = _lib.MX_FP4_UNCHECKED if kind == _lib.MX_FP4 else kind
-        ops.MxOperand(fmt, raw, rows, k, req)
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        torch.cuda.synchronize()
-        e0.record()
-        for _ in range(10):
-            ops.MxOperand(fmt, raw, rows, k, req)
-        e1.record()
-        torch.cuda.synchronize()
-        return round(e0.elapsed_time(e1) / 10 * 1e3, 1)
-
-    prep = {"prepare_a_us": prepare_us(Q.MXFP4, a_dev, m, A.kind), "prepare_w_us": prepare_us(w_fmt, w_dev, n, W.kind)}
     out = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
     ms = C.c_float(0)
     L = _lib.lib()
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def prepare_us(fmt, raw, rows, kind, reps=20):
+        # re-encoding into the matrix core's operand order: device time of back-to-back rfq_mx_prepare calls into one
+        # buffer that do not synchronise (8-bit kinds, and the 4-bit kind requested unchecked, which is how
+        # activations are prepared per prefill)
+        req = _lib.MX_FP4_UNCHECKED if kind == _lib.MX_FP4 else kind
+        nbytes = L.rfq_mx_prepared_bytes(fmt, kind, rows, k)
+        buf = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        got = C.c_int(0)
+        call = lambda: _lib.check(L.rfq_mx_prepare(fmt, req, C.c_void_p(raw.data_ptr()), raw.numel(), rows, k,
+                                                   C.c_void_p(buf.data_ptr()), nbytes, C.byref(got), stream))
+        call()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(reps):
+            call()
+        e1.record()
+        torch.cuda.synchronize()
+        return round(e0.elapsed_time(e1) / reps * 1e3, 1)
+
+    prep = {"prepare_a_us": prepare_us(Q.MXFP4, a_dev, m, A.kind), "prepare_w_us": prepare_us(w_fmt, w_dev, n, W.kind, reps=5)}
     args = (C.c_void_p(A.buf.data_ptr()), A.kind, C.c_void_p(W.buf.data_ptr()), W.kind, C.c_void_p(out.data_ptr()),
             _lib.BF16, m, n, k)
-    _lib.check(L.rfq_bench_gemm_mx(*args, 0, warmup, stream, C.byref(ms)))
-    _lib.check(L.rfq_bench_gemm_mx(*args, 0, steps, stream, C.byref(ms)))
+    _lib.check(L.rfq_bench_gemm_mx(*args, warmup, steps, stream, C.byref(ms)))
     t = ms.value / 1e3 / steps
     flops = 2.0 * m * n * k
     peak = 10.1e15 if (A.kind == _lib.MX_FP4 and W.kind == _lib.MX_FP4) else 5.0e15
-    return {"TFLOP/s": round(flops / t / 1e12, 1), "us": round(t * 1e6, 1), "mfma_frac": round(flops / t / peak, 4),
-            "peak_TFLOP/s": peak / 1e12, "kinds": [A.kind, W.kind], **prep}
+    res = {"TFLOP/s": round(flops / t / 1e12, 1), "us": round(t * 1e6, 1), "mfma_frac": round(flops / t / peak, 4),
+           "peak_TFLOP/s": peak / 1e12, "kinds": [A.kind, W.kind], "warmup_launches": warmup, "timed_launches": steps,
+           "operands": "reference packer (codes 0, 1, 8, 9)" if data == "packer" else "every code of a four-octave window", **prep}
+    if A.kind == _lib.MX_FP4 and data == "packer":
+        # the prefill step end to end: raw MXFP4 activations re-encoded before every GEMM
+        _lib.check(L.rfq_bench_gemm_mx_prefill(C.c_void_p(a_dev.data_ptr()), a_dev.numel(), C.c_void_p(A.buf.data_ptr()),
+                                               A.buf.numel(), C.c_void_p(W.buf.data_ptr()), W.kind, C.c_void_p(out.data_ptr()),
+                                               _lib.BF16, m, n, k, warmup, steps, stream, C.byref(ms)))
+        te = ms.value / 1e3 / steps
+        res["prefill_step"] = {"us": round(te * 1e6, 1), "TFLOP/s": round(flops / te / 1e12, 1), "mfma_frac": round(flops / te / peak, 4),
+                               "what": "rfq_mx_prepare(A, unchecked) + rfq_gemm_mx per step"}
+    return res
 
 
-def kq_gemm(torch, fmt, m=512, n=14336, k=4096, steps=100, warmup=300):
+def kq_gemm(torch, fmt, m=512, n=14336, k=4096, steps=300, warmup=40):
     """Q4_K / Q6_K prefill GEMM on the fp16 matrix cores, fp16 in and out."""
     from rocmforge_amd import _lib, quantize as Q
     dev = torch.device("cuda:0")
@@ -77,12 +98,11 @@ def kq_gemm(torch, fmt, m=512, n=14336, k=4096, steps=100, warmup=300):
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     args = (fmt, C.c_void_p(w.data_ptr()), w.numel(), C.c_void_p(a.data_ptr()), C.c_void_p(out.data_ptr()), _lib.F16,
             m, n, k)
-    _lib.check(L.rfq_bench_gemm_f16(*args, 0, warmup, stream, C.byref(ms)))
-    _lib.check(L.rfq_bench_gemm_f16(*args, 0, steps, stream, C.byref(ms)))
+    _lib.check(L.rfq_bench_gemm_f16(*args, warmup, steps, stream, C.byref(ms)))
     t = ms.value / 1e3 / steps
     flops = 2.0 * m * n * k
     return {"TFLOP/s": round(flops / t / 1e12, 1), "us": round(t * 1e6, 1), "mfma_frac": round(flops / t / 2.5e15, 4),
-            "peak_TFLOP/s": 2500.0}
+            "peak_TFLOP/s": 2500.0, "warmup_launches": warmup, "timed_launches": steps}
 
 
 def run(torch):
@@ -93,6 +113,7 @@ def run(torch):
     res["GGUF_Q4_K gemm 512x4096x14336 fp16"] = kq_gemm(torch, Q.GGUF_Q4_K)
     res["GGUF_Q6_K gemm 512x4096x14336 fp16"] = kq_gemm(torch, Q.GGUF_Q6_K)
     res["MXFP4 gemm 2048x8192x28672 bf16"] = mx_gemm(torch, Q.MXFP4)
+    res["MXFP4 gemm 2048x8192x28672 bf16, full-entropy operands"] = mx_gemm(torch, Q.MXFP4, data="window")
     res["MXFP6-weight gemm 2048x8192x28672 bf16"] = mx_gemm(torch, Q.MXFP6_E2M3)
     return res
 
@@ -103,13 +124,14 @@ if __name__ == "__main__":
     sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
     ap = argparse.ArgumentParser()
     ap.add_argument("--only", choices=["mxfp4", "mxfp6", "q4_k", "gguf_q4_k"], help="one configuration (for profiling runs)")
-    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--data", choices=["packer", "window"], default="packer", help="MXFP4 operands: the reference packer's, or full-entropy")
     a = ap.parse_args()
     import torch
     from rocmforge_amd import quantize as Q
     if a.only in ("q4_k", "gguf_q4_k"):
         print(json.dumps(kq_gemm(torch, Q.Q4_K if a.only == "q4_k" else Q.GGUF_Q4_K, steps=a.steps)))
     elif a.only:
-        print(json.dumps(mx_gemm(torch, Q.MXFP4 if a.only == "mxfp4" else Q.MXFP6_E2M3, steps=a.steps)))
+        print(json.dumps(mx_gemm(torch, Q.MXFP4 if a.only == "mxfp4" else Q.MXFP6_E2M3, steps=a.steps, data=a.data)))
     else:
         print(json.dumps(run(torch)))

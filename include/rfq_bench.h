@@ -31,6 +31,18 @@ RFQ_API int rfq_bench_gemv(int fmt, const void *const *d_w_copies, int copies, s
 RFQ_API int rfq_bench_dequant(int fmt, const void *const *d_in_copies, int copies, size_t packed_bytes, float *d_out,
                               size_t n_elems, int out_copies, int warmup, int steps, void *stream, float *elapsed_ms);
 
+/* Name and template arguments of the kernel that the calling thread's last rfq_gemv / rfq_rms_norm_gemv /
+ * rfq_mlp_swiglu launch took ("" before the first), e.g. "gemv_idot_kernel<Q4_K,1,2,7>": lets the driver name the
+ * kernel it timed from the dispatch actually taken instead of a constant. */
+RFQ_API const char *rfq_bench_last_gemv_kernel(void);
+
+/* The floor of a one-launch step that has to fetch `bytes` from HBM: a kernel that only reads copy i % copies
+ * (16-byte loads, consecutive lanes on consecutive addresses, `depth` = 4, 8 or 16 loads of a thread in flight at
+ * once, non-temporal when nt != 0), folds the words into one value and stores nothing, launched back to back like the
+ * GEMV it is compared with: `blocks` workgroups of `threads` (a multiple of 64, at most 1024). */
+RFQ_API int rfq_bench_read_floor(const void *const *d_copies, int copies, size_t bytes, int blocks, int threads, int nt,
+                                 int depth, int warmup, int steps, void *stream, float *elapsed_ms);
+
 RFQ_API int rfq_bench_gemm_f16(int fmt, const void *d_w, size_t w_bytes, const void *d_a_f16, void *d_out,
                                int out_dtype, int m, int n, int k, int warmup, int steps, void *stream,
                                float *elapsed_ms);
@@ -38,6 +50,13 @@ RFQ_API int rfq_bench_gemm_f16(int fmt, const void *d_w, size_t w_bytes, const v
 RFQ_API int rfq_bench_gemm_mx(const void *d_a_prep, int a_kind, const void *d_w_prep, int w_kind, void *d_out,
                               int out_dtype, int m, int n, int k, int warmup, int steps, void *stream,
                               float *elapsed_ms);
+
+/* A prefill step as a caller that holds raw MXFP4 activations runs it: re-encode A for the matrix core
+ * (rfq_mx_prepare, RFQ_MX_FP4_UNCHECKED: no read-back, no synchronisation) into d_a_prep, then rfq_gemm_mx
+ * against the weights prepared once at upload. */
+RFQ_API int rfq_bench_gemm_mx_prefill(const void *d_a_raw, size_t a_raw_bytes, void *d_a_prep, size_t a_prep_bytes,
+                                      const void *d_w_prep, int w_kind, void *d_out, int out_dtype, int m, int n, int k,
+                                      int warmup, int steps, void *stream, float *elapsed_ms);
 
 /* Step i runs the MLP over weight set i % copies.  one_call != 0: rfq_mlp_swiglu;
  * one_call == 0: the same arithmetic as five calls (rfq_rms_norm, rfq_gemv for

@@ -36,9 +36,58 @@ int timed_loop(int warmup, int steps, void *stream, float *elapsed_ms, Step step
     return RFQ_OK;
 }
 
+// Reads n16 16-byte words and keeps nothing: thread t takes words t, t + T, t + 2T, ... (T = all threads), D at a
+// time in flight.  The store can never happen (a 32-bit fold of arbitrary data equal to a value the host picks at
+// random per launch would be needed), but the compiler cannot know that, so the loads stay.
+template <bool NT, int D>
+__global__ void __launch_bounds__(1024)
+read_floor_kernel(const uint8_t *__restrict__ p, size_t n16, uint32_t never, uint32_t *sink)
+{
+    typedef uint32_t v4_t __attribute__((ext_vector_type(4)));
+    const size_t T = (size_t)gridDim.x * blockDim.x, t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const v4_t *w = reinterpret_cast<const v4_t *>(p);
+    uint32_t acc = 0;
+    for (size_t i = t; i < n16; i += D * T) {
+        v4_t v[D];
+#pragma unroll
+        for (int d = 0; d < D; d++) {
+            const size_t j = i + d * T < n16 ? i + d * T : t;       // (past the end: re-read the first word, a cache hit)
+            v[d] = NT ? __builtin_nontemporal_load(w + j) : w[j];
+        }
+#pragma unroll
+        for (int d = 0; d < D; d++) acc += (v[d][0] ^ v[d][1]) + (v[d][2] ^ v[d][3]);
+    }
+    if (acc == never && never != 0) sink[t & 63] = acc;
+}
+
 } // namespace
 
 extern "C" {
+
+int rfq_bench_read_floor(const void *const *d_copies, int copies, size_t bytes, int blocks, int threads, int nt, int depth,
+                         int warmup, int steps, void *stream, float *elapsed_ms)
+{
+    if (!d_copies || copies <= 0 || bytes < 16 || blocks <= 0 || threads <= 0 || threads > 1024 || threads % 64 != 0 ||
+        (depth != 4 && depth != 8 && depth != 16))
+        return rfq::fail(RFQ_E_BADARG, "rfq_bench_read_floor: bad arguments");
+    static uint32_t *sink = nullptr;                        // 64 words, never written
+    if (!sink) RFQ_HIP(hipMalloc(reinterpret_cast<void **>(&sink), 256));
+    hipStream_t s = (hipStream_t)stream;
+    return timed_loop(warmup, steps, stream, elapsed_ms, [&](int i) {
+        const uint8_t *p = static_cast<const uint8_t *>(d_copies[i % copies]);
+        const uint32_t never = 0x9E3779B9u * (uint32_t)(i + 1) | 1u;
+        const dim3 g(blocks), b(threads);
+        const size_t n16 = bytes / 16;
+        if (nt && depth == 4) hipLaunchKernelGGL((read_floor_kernel<true, 4>), g, b, 0, s, p, n16, never, sink);
+        else if (nt && depth == 8) hipLaunchKernelGGL((read_floor_kernel<true, 8>), g, b, 0, s, p, n16, never, sink);
+        else if (nt) hipLaunchKernelGGL((read_floor_kernel<true, 16>), g, b, 0, s, p, n16, never, sink);
+        else if (depth == 4) hipLaunchKernelGGL((read_floor_kernel<false, 4>), g, b, 0, s, p, n16, never, sink);
+        else if (depth == 8) hipLaunchKernelGGL((read_floor_kernel<false, 8>), g, b, 0, s, p, n16, never, sink);
+        else hipLaunchKernelGGL((read_floor_kernel<false, 16>), g, b, 0, s, p, n16, never, sink);
+        RFQ_LAUNCH_CHECK("read_floor_kernel");
+        return (int)RFQ_OK;
+    });
+}
 
 int rfq_bench_gemv(int fmt, const void *const *d_w_copies, int copies, size_t w_bytes, const float *d_x, float *d_y,
                    int m, int n, int k, int warmup, int steps, void *stream, float *elapsed_ms)
@@ -71,6 +120,18 @@ int rfq_bench_gemm_mx(const void *d_a_prep, int a_kind, const void *d_w_prep, in
 {
     return timed_loop(warmup, steps, stream, elapsed_ms, [&](int) {
         return rfq_gemm_mx(d_a_prep, a_kind, d_w_prep, w_kind, d_out, out_dtype, m, n, k, stream);
+    });
+}
+
+int rfq_bench_gemm_mx_prefill(const void *d_a_raw, size_t a_raw_bytes, void *d_a_prep, size_t a_prep_bytes,
+                              const void *d_w_prep, int w_kind, void *d_out, int out_dtype, int m, int n, int k, int warmup,
+                              int steps, void *stream, float *elapsed_ms)
+{
+    return timed_loop(warmup, steps, stream, elapsed_ms, [&](int) {
+        int kind = 0;
+        int rc = rfq_mx_prepare(RFQ_MXFP4, RFQ_MX_FP4_UNCHECKED, d_a_raw, a_raw_bytes, m, k, d_a_prep, a_prep_bytes, &kind, stream);
+        if (rc != RFQ_OK) return rc;
+        return rfq_gemm_mx(d_a_prep, kind, d_w_prep, w_kind, d_out, out_dtype, m, n, k, stream);
     });
 }
 

@@ -120,6 +120,38 @@ template <typename T> __device__ __forceinline__ T ld(const uint8_t *p)
     return v;
 }
 
+// The same with the non-temporal hint, for the nibble bytes of the 256-byte Q4_K layouts: a lane takes 16 of every 28
+// (or 20) bytes there in ONE load, the rest of the line is never wanted, and keeping such lines out of the caches
+// leaves them to what is reused -- x, the block headers neighbouring lanes share (Q4_K 14336 x 4096 GEMV: 11.33 ->
+// 10.84 us, 128256 x 4096: 93.4 -> 82.6 us; with the hint on the 2-byte scale and 1-byte min loads as well the gain
+// is gone).  Not for layouts whose cache lines are consumed by two load instructions of a lane or by neighbouring
+// lanes in turn -- there the second access finds the line gone: measured with the hint, Q6_K 13.9 -> 16.4 us,
+// GGUF_Q4_K 8.0 -> 9.1 us, GGUF_Q8_0 6.1 -> 6.5 us; Q4_0 and Q8_0 no change.
+template <typename T> __device__ __forceinline__ T ld_once(const uint8_t *p)
+{
+    static_assert(sizeof(T) % 4 == 0, "whole dwords");
+    constexpr int N = sizeof(T) / 4;
+    typedef uint32_t v4_t __attribute__((ext_vector_type(4), aligned(1)));
+    typedef uint32_t v2_t __attribute__((ext_vector_type(2), aligned(1)));
+    typedef uint32_t v1_t __attribute__((aligned(1)));
+    uint32_t w[N];
+    int i = 0;
+#pragma unroll
+    for (; i + 4 <= N; i += 4) {
+        const v4_t v = __builtin_nontemporal_load(reinterpret_cast<const v4_t *>(p + 4 * i));
+        w[i] = v[0]; w[i + 1] = v[1]; w[i + 2] = v[2]; w[i + 3] = v[3];
+    }
+    if (i + 2 <= N) {
+        const v2_t v = __builtin_nontemporal_load(reinterpret_cast<const v2_t *>(p + 4 * i));
+        w[i] = v[0]; w[i + 1] = v[1];
+        i += 2;
+    }
+    if (i < N) w[i] = __builtin_nontemporal_load(reinterpret_cast<const v1_t *>(p + 4 * i));
+    T out;
+    __builtin_memcpy(&out, w, sizeof(T));
+    return out;
+}
+
 __device__ __forceinline__ float f16_bits_to_f32(uint16_t h)
 {
     _Float16 v;

@@ -493,7 +493,11 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int fr = lane & 31, fh = lane >> 5;                     // fragment row, k half
     const int tiles_m = (M + BM - 1) / BM;
-    const int tm = blockIdx.x % tiles_m, tn = blockIdx.x / tiles_m; // the m tiles of one W tile are neighbours
+    // Workgroups are dealt round-robin to the 8 XCDs (blockIdx.x % 8), each with an L2 of its own: hand every XCD a
+    // contiguous run of tiles, so that the m tiles of one W tile meet in one L2 and W comes from HBM once.
+    const int nwg = gridDim.x;
+    const int tile = nwg % 8 == 0 ? (int)(blockIdx.x % 8) * (nwg / 8) + (int)(blockIdx.x / 8) : (int)blockIdx.x;
+    const int tm = tile % tiles_m, tn = tile / tiles_m;             // the m tiles of one W tile are neighbours
     const int m0 = tm * BM, n0 = tn * BN;
     const int groups = K / 32;                                    // 32-element groups per row
     const size_t row_bytes = (size_t)(K / Fmt<FMT>::BE) * Fmt<FMT>::BB;

@@ -109,15 +109,28 @@ __device__ __forceinline__ int exponent_of(float a)
 // One thread per (row, block).  Thread g: lane = g & 63, page = g >> 6.
 // status[0] is set to 1 if an FP4 re-encoding met a block it cannot express.
 
+// The scale bytes of k-steps 4j .. 4j+3 of a row tile are the four bytes of one dword per lane.  A workgroup's four
+// wavefronts re-encode exactly those four pages (the padded k-step count is a multiple of 4 and so is a
+// workgroup's first page), so the bytes meet in LDS and leave as one coalesced dword store per lane instead of
+// four byte stores from four wavefronts into the same dword.
+__device__ __forceinline__ void store_scales(uint8_t *prep, const MxLayout &L, int rt, int ks, int lane, int E)
+{
+    __shared__ uint8_t sc[4][64];
+    sc[ks & 3][lane] = (uint8_t)E;
+    __syncthreads();
+    if ((ks & 3) == 0) {
+        const uint32_t w = (uint32_t)sc[0][lane] | ((uint32_t)sc[1][lane] << 8) | ((uint32_t)sc[2][lane] << 16) | ((uint32_t)sc[3][lane] << 24);
+        *reinterpret_cast<uint32_t *>(prep + L.data_bytes + ((size_t)rt * L.ks4 + (ks >> 2)) * 256 + (size_t)lane * 4) = w;
+    }
+}
+
 template <int FMT, int KIND>
 __global__ void __launch_bounds__(256)
 mx_prepare_kernel(const uint8_t *__restrict__ raw, uint8_t *__restrict__ prep, MxLayout L)
 {
     constexpr int BB = Fmt<FMT>::BB;
     size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
-    size_t npages = (size_t)L.rt * L.ks;
-    if (g >= npages * 64) return;
-    int lane = (int)(g & 63);
+    int lane = (int)(g & 63);                                  // (the grid is exactly rt * ks pages: no thread is past the end)
     size_t page = g >> 6;
     int rt = (int)(page / L.ks), ks = (int)(page % L.ks);
     int row = rt * 32 + (lane & 31), kb = ks * 2 + (lane >> 5);
@@ -196,7 +209,7 @@ mx_prepare_kernel(const uint8_t *__restrict__ raw, uint8_t *__restrict__ prep, M
         *reinterpret_cast<uint4 *>(dst) = make_uint4(out[0], out[1], out[2], out[3]);
         *reinterpret_cast<uint4 *>(dst + 512) = make_uint4(out[4], out[5], out[6], out[7]);
     }
-    prep[L.data_bytes + ((size_t)rt * L.ks4 + (ks >> 2)) * 256 + (size_t)lane * 4 + (ks & 3)] = (uint8_t)E;
+    store_scales(prep, L, rt, ks, lane, E);
 }
 
 // MXFP4 -> 4-bit operand with integer arithmetic only (the general kernel
@@ -214,9 +227,7 @@ __global__ void __launch_bounds__(256)
 mx_prepare_fp4_kernel(const uint8_t *__restrict__ raw, uint8_t *__restrict__ prep, MxLayout L)
 {
     size_t g = (size_t)blockIdx.x * 256 + threadIdx.x;
-    size_t npages = (size_t)L.rt * L.ks;
-    if (g >= npages * 64) return;
-    int lane = (int)(g & 63);
+    int lane = (int)(g & 63);                                  // (the grid is exactly rt * ks pages: no thread is past the end)
     size_t page = g >> 6;
     int rt = (int)(page / L.ks), ks = (int)(page % L.ks);
     int row = rt * 32 + (lane & 31), kb = ks * 2 + (lane >> 5);
@@ -282,7 +293,7 @@ mx_prepare_fp4_kernel(const uint8_t *__restrict__ raw, uint8_t *__restrict__ pre
     }
     uint4 *dst = reinterpret_cast<uint4 *>(prep + page * 1024 + (size_t)lane * 16);
     *dst = make_uint4(out[0], out[1], out[2], out[3]);
-    prep[L.data_bytes + ((size_t)rt * L.ks4 + (ks >> 2)) * 256 + (size_t)lane * 4 + (ks & 3)] = (uint8_t)E;
+    store_scales(prep, L, rt, ks, lane, E);
 }
 
 // The status words (every page and every scale byte is written by the re-encoding kernels).
@@ -869,11 +880,13 @@ int run_gemm(const uint8_t *a, const uint8_t *b, void *out, int m, int n, int k,
 }
 
 template <int FMT, int KIND>
-int run_prepare(const uint8_t *raw, uint8_t *prep, const MxLayout &L, hipStream_t s)
+int run_prepare(const uint8_t *raw, uint8_t *prep, const MxLayout &L, bool clear_status, hipStream_t s)
 {
-    size_t threads = (size_t)L.rt * L.ks * 64;
-    hipLaunchKernelGGL(mx_init_kernel, dim3(1), dim3(64), 0, s, prep, L);
-    RFQ_LAUNCH_CHECK("mx_init_kernel");
+    size_t threads = (size_t)L.rt * L.ks * 64;                  // a multiple of 1024: ks is padded to a multiple of 16
+    if (clear_status) {                                         // (an unchecked request never reads the status words)
+        hipLaunchKernelGGL(mx_init_kernel, dim3(1), dim3(64), 0, s, prep, L);
+        RFQ_LAUNCH_CHECK("mx_init_kernel");
+    }
     if (FMT == RFQ_MXFP4 && KIND == RFQ_MX_FP4)
         hipLaunchKernelGGL(mx_prepare_fp4_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, raw, prep, L);
     else
@@ -912,7 +925,7 @@ int launch_mx_prepare(int fmt, int kind_req, const uint8_t *d_raw, int rows, int
         size_t need = kind_req == RFQ_MX_AUTO ? mx_layout(RFQ_MX_FP8, rows, k).total() : L.total();
         if (prep_bytes < need)
             return fail(RFQ_E_SIZE, "rfq_mx_prepare: prepared buffer has %zu bytes, needs %zu", prep_bytes, need);
-        int rc = run_prepare<RFQ_MXFP4, RFQ_MX_FP4>(d_raw, prep, L, s);
+        int rc = run_prepare<RFQ_MXFP4, RFQ_MX_FP4>(d_raw, prep, L, !unchecked, s);
         if (rc != RFQ_OK) return rc;
         if (unchecked) {                                         // the caller vouches for the data: no read-back, no sync
             if (kind_out) *kind_out = RFQ_MX_FP4;
@@ -932,8 +945,8 @@ int launch_mx_prepare(int fmt, int kind_req, const uint8_t *d_raw, int rows, int
     MxLayout L = mx_layout(RFQ_MX_FP8, rows, k);
     if (prep_bytes < L.total())
         return fail(RFQ_E_SIZE, "rfq_mx_prepare: prepared buffer has %zu bytes, needs %zu", prep_bytes, L.total());
-    int rc = is4 ? run_prepare<RFQ_MXFP4, RFQ_MX_FP8>(d_raw, prep, L, s)
-                 : run_prepare<RFQ_MXFP6_E2M3, RFQ_MX_FP8>(d_raw, prep, L, s);
+    int rc = is4 ? run_prepare<RFQ_MXFP4, RFQ_MX_FP8>(d_raw, prep, L, true, s)
+                 : run_prepare<RFQ_MXFP6_E2M3, RFQ_MX_FP8>(d_raw, prep, L, true, s);
     if (rc != RFQ_OK) return rc;
     if (kind_out) *kind_out = RFQ_MX_FP8;
     return RFQ_OK;

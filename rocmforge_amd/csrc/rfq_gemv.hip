@@ -18,12 +18,20 @@
 //                the units and read x through the L1/L2 caches.
 // Reduction: DPP butterflies inside each row of 16 lanes, v_readlane across
 // the four rows; an LDS hop only when a row is split over several wavefronts.
+#include <stdio.h>
+
 #include <mutex>
 
 #include "rfq_common.hpp"
 
 namespace rfq {
 namespace {
+
+// Which kernel the last GEMV launch of this thread took (name and template arguments), for the benchmark
+// driver's report: plain stores on the launch path, formatted only when asked for.
+struct LastKernel { const char *name; int fmt, a, b, c; };
+thread_local LastKernel g_last_kernel = {"", 0, 0, 0, 0};
+inline void note_kernel(const char *name, int fmt, int a, int b, int c) { g_last_kernel = LastKernel{name, fmt, a, b, c}; }
 
 // ---- wavefront reduction -----------------------------------------------------
 
@@ -86,6 +94,44 @@ __device__ __forceinline__ float nib_dot_lo_first(const U4 &q, const float (&x)[
 
 template <int FMT> struct Unit;
 
+// ---- pieces that do not start on a multiple of 4 ------------------------------------------
+// A 16-byte load from an address that is not a multiple of 4 runs at a fraction of the aligned rate on this part
+// (17-byte blocks streamed as stored, a byte and 16 bytes per lane: 9.2 us for 31 MB; through aligned windows of whole
+// dwords: 6.8 us).  For the units whose kernels are bound by their instructions the byte permutes that move a window
+// into place cost more than the loads gain (measured: MXFP4 / MXFP6 / GGUF_Q4_0 / GGUF_Q8_0 GEMV 1..5 % slower with
+// windows); the 210-byte GGUF_Q6_K block, two 32-byte pieces per unit at 2-byte alignment, gains 3 %.
+template <int NW> __device__ __forceinline__ void load_dwords_a4(const uint8_t *a, uint32_t (&d)[NW])
+{
+    typedef uint32_t v4a4 __attribute__((ext_vector_type(4), aligned(4)));
+    int i = 0;
+#pragma unroll
+    for (; i + 4 <= NW; i += 4) {
+        const v4a4 v = *reinterpret_cast<const v4a4 *>(a + 4 * i);
+        d[i] = v[0]; d[i + 1] = v[1]; d[i + 2] = v[2]; d[i + 3] = v[3];
+    }
+#pragma unroll
+    for (; i < NW; i++) d[i] = *reinterpret_cast<const uint32_t *>(a + 4 * i);
+}
+
+// 32 bytes at a 2-byte aligned address inside a larger block: the window of 9 dwords from the multiple of 4 at or
+// before it, moved into place with byte permutes.  The 4 bytes read behind the piece belong to the same block; the
+// up to 2 bytes read before it stay inside the tensor as long as the tensor starts on a multiple of 4, which the
+// launcher checks (a tensor at another address takes the byte-exact load_bytes in the generic kernel).
+__device__ __forceinline__ U8 load32_a2(const uint8_t *c)
+{
+    const uint8_t *a = reinterpret_cast<const uint8_t *>(reinterpret_cast<uintptr_t>(c) & ~(uintptr_t)3);
+    const uint32_t sel = 0x03020100u + 0x01010101u * (uint32_t)(reinterpret_cast<uintptr_t>(c) & 3u);
+    uint32_t d[9];
+    load_dwords_a4<9>(a, d);
+    U8 r;
+#pragma unroll
+    for (int i = 0; i < 8; i++) r.v[i] = __builtin_amdgcn_perm(d[i + 1], d[i], sel);
+    return r;
+}
+
+template <int FMT> struct NeedsAlignedTensor { static constexpr bool value = false; };
+template <> struct NeedsAlignedTensor<RFQ_GGUF_Q6_K> { static constexpr bool value = true; };
+
 template <> struct Unit<RFQ_Q4_0> {
     static constexpr bool NEEDS_XSUM = true;
     float scale; U4 q;
@@ -133,7 +179,7 @@ template <> struct Unit<RFQ_Q4_K> {
         int sb = u & 7;
         sc = ld<uint16_t>(blk + 2 * sb);
         mn = (int8_t)blk[16 + sb];
-        q = ld<U4>(blk + 32 + 28 * sb);
+        q = ld_once<U4>(blk + 32 + 28 * sb);
     }
     __device__ __forceinline__ float dot(const float (&x)[32], float xsum) const
     {
@@ -385,6 +431,16 @@ template <> struct Unit<RFQ_GGUF_Q6_K> {
         const uint8_t *blk = row + (size_t)(u >> 3) * 210;
         const int half = (u >> 2) & 1;
         t = u & 3;
+        ql = load32_a2(blk + 64 * half + 32 * (t & 1));
+        qh = load32_a2(blk + 128 + 32 * half);
+        sc2 = ld<uint16_t>(blk + 192 + 8 * half + 2 * t);
+        d = ld<uint16_t>(blk + 208);
+    }
+    __device__ __forceinline__ void load_bytes(const uint8_t *row, int u)
+    {
+        const uint8_t *blk = row + (size_t)(u >> 3) * 210;
+        const int half = (u >> 2) & 1;
+        t = u & 3;
         ql = ld<U8>(blk + 64 * half + 32 * (t & 1));
         qh = ld<U8>(blk + 128 + 32 * half);
         sc2 = ld<uint16_t>(blk + 192 + 8 * half + 2 * t);
@@ -448,7 +504,7 @@ template <> struct Unit<RFQ_MM_Q4_K> {                 // quantized/q4_k.rs:101-
         int sb = u & 7;
         sc = ld<uint16_t>(blk + 2 * sb);
         mn = (int8_t)blk[16 + sb];
-        q = ld<U4>(blk + 32 + 20 * sb);
+        q = ld_once<U4>(blk + 32 + 20 * sb);
     }
     __device__ __forceinline__ float dot(const float (&x)[32], float xsum) const
     {
@@ -586,7 +642,7 @@ __device__ __forceinline__ void store_group(const float (&res)[R], float (*part)
 template <int FMT, int UPL, int WPR, int R, bool FUSE>
 __global__ void __launch_bounds__(256)
 gemv_xreg_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ y, int n, int k,
-                 int groups, GemvFuse f)
+                 int groups, GemvFuse f, int xstage)
 {
     constexpr int TEAMS = 4 / WPR, TL = 64 * WPR;
     // rows in flight per lane: three, or five in the form with one unit per lane and two wavefronts per row
@@ -607,11 +663,36 @@ gemv_xreg_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
         int u = tl + j * TL;
         live[j] = u < ku;
         unit[j] = live[j] ? u : ku - 1;
-        load_x32(x + (size_t)unit[j] * 32, xs[j]);
     }
     const bool norm = FUSE && f.norm_w != nullptr;
-    float nws[FUSE ? UPL : 1][32];
-    if (norm) {
+
+    // x reaches the lanes through LDS (xstage != 0: the launcher gave the block k floats of dynamic LDS): the block
+    // fetches it once with consecutive lanes on consecutive 16-byte pieces, and a lane then reads its units from
+    // LDS.  Every lane fetching its own 128-byte unit from memory instead costs a wavefront eight load
+    // instructions that each touch 64 different cache lines -- with sixteen short-lived wavefronts per CU that
+    // address traffic, not the weight stream, set the kernel's time (Q6_K 14336 x 4096: 6.4 us of 13.9).
+    // LDS layout: 16-byte piece q (0..7) of unit u at ((q * ku + u) * 16), so consecutive lanes read consecutive pieces.
+    extern __shared__ __attribute__((aligned(16))) float xstage_lds[];
+    constexpr int XQ = 4;                                         // pieces a thread holds in registers while the first rows are requested
+    const int pieces = ku * 8;
+    float4 xq[XQ], nq[FUSE ? XQ : 1];
+    if (xstage) {
+#pragma unroll
+        for (int i = 0; i < XQ; i++) {
+            const int p = threadIdx.x + 256 * i;
+            if (p < pieces) {
+                xq[i] = ld<float4>(reinterpret_cast<const uint8_t *>(x + (size_t)p * 4));
+                if constexpr (FUSE) {
+                    if (norm) nq[i] = ld<float4>(reinterpret_cast<const uint8_t *>(f.norm_w + (size_t)p * 4));
+                }
+            }
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < UPL; j++) load_x32(x + (size_t)unit[j] * 32, xs[j]);
+    }
+    float nws[(FUSE ? UPL : 1)][32];
+    if (norm && !xstage) {
 #pragma unroll
         for (int j = 0; j < UPL; j++) load_x32(f.norm_w + (size_t)unit[j] * 32, nws[FUSE ? j : 0]);
     }
@@ -633,11 +714,56 @@ gemv_xreg_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
         for (int j = 0; j < UPL; j++) buf[slot][j].load(row, unit[j]);
     };
     // x first, then the first rows, and only then the first use of x: the
-    // weight loads are already in flight while the x sums are formed.
+    // weight loads are already in flight while x is staged and its sums are formed.
 #pragma unroll
     for (int d = 0; d < D; d++) load_row(d, d);
     float rinv = 1.0f;
-    if (norm) {
+    if (xstage) {
+        float ssq = 0.f;
+        auto put = [&](int p, float4 v, float4 nv) {
+            if constexpr (FUSE) {
+                if (norm) {
+                    ssq = __builtin_fmaf(v.x, v.x, ssq); ssq = __builtin_fmaf(v.y, v.y, ssq);
+                    ssq = __builtin_fmaf(v.z, v.z, ssq); ssq = __builtin_fmaf(v.w, v.w, ssq);
+                    v.x *= nv.x; v.y *= nv.y; v.z *= nv.z; v.w *= nv.w;
+                }
+            }
+            *reinterpret_cast<float4 *>(xstage_lds + ((size_t)(p & 7) * ku + (p >> 3)) * 4) = v;
+        };
+#pragma unroll
+        for (int i = 0; i < XQ; i++) {
+            const int p = threadIdx.x + 256 * i;
+            if (p < pieces) put(p, xq[i], nq[FUSE ? i : 0]);
+        }
+        for (int p = threadIdx.x + 256 * XQ; p < pieces; p += 256) {  // (longer rows: the rest, behind the first rows' loads)
+            float4 v = ld<float4>(reinterpret_cast<const uint8_t *>(x + (size_t)p * 4)), nv = v;
+            if constexpr (FUSE) {
+                if (norm) nv = ld<float4>(reinterpret_cast<const uint8_t *>(f.norm_w + (size_t)p * 4));
+            }
+            put(p, v, nv);
+        }
+        if constexpr (FUSE) {
+            if (norm) {
+                ssq = wave_sum(ssq);
+                if (lane == 0) part[0][wave] = ssq;
+            }
+        }
+        __syncthreads();
+        if constexpr (FUSE) {
+            if (norm) rinv = 1.0f / sqrtf(((part[0][0] + part[0][1]) + (part[0][2] + part[0][3])) / (float)k + f.eps);
+        }
+#pragma unroll
+        for (int j = 0; j < UPL; j++) {
+#pragma unroll
+            for (int q = 0; q < 8; q++) {
+                const float4 v = *reinterpret_cast<const float4 *>(xstage_lds + ((size_t)q * ku + unit[j]) * 4);
+                xs[j][4 * q] = v.x; xs[j][4 * q + 1] = v.y; xs[j][4 * q + 2] = v.z; xs[j][4 * q + 3] = v.w;
+            }
+        }
+        if constexpr (FUSE) {
+            if (norm) __syncthreads();                            // part[0] is reused by the first group's results
+        }
+    } else if (norm) {
         // every team holds all of x: its own sum of squares, no exchange between teams
         float ssq = 0.f;
 #pragma unroll
@@ -1473,7 +1599,8 @@ gemv_mfma_q8_0_kernel(const uint8_t *__restrict__ w, const _Float16 *__restrict_
 }
 
 // ---- any m <= 8, any k: one row per wavefront ---------------------------------
-template <int FMT, int M>
+// BYTES: fetch blocks byte-exactly (a tensor that does not start on a multiple of 4, see load32_a2).
+template <int FMT, int M, bool BYTES = false>
 __global__ void __launch_bounds__(256)
 gemv_generic_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ y, int n, int k)
 {
@@ -1489,7 +1616,8 @@ gemv_generic_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, 
         for (int mi = 0; mi < M; mi++) acc[mi] = 0.f;
         for (int u = lane; u < ku; u += 64) {
             Unit<FMT> un;
-            un.load(row, u);
+            if constexpr (BYTES) un.load_bytes(row, u);            // (only instantiated for units that have it)
+            else un.load(row, u);
 #pragma unroll
             for (int mi = 0; mi < M; mi++) {
                 float xv[32];
@@ -1538,8 +1666,13 @@ template <int FMT, int UPL, int WPR, int R, bool FUSE>
 int launch_xreg(const uint8_t *w, const float *x, float *y, int n, int k, const RowPlan &p, const GemvFuse &f,
                 hipStream_t s)
 {
-    hipLaunchKernelGGL((gemv_xreg_kernel<FMT, UPL, WPR, R, FUSE>), dim3(p.blocks), dim3(256), 0, s, w, x, y, n, k,
-                       p.groups, f);
+    note_kernel(FUSE ? "gemv_xreg_kernel<%s,%d,%d,%d,fused>" : "gemv_xreg_kernel<%s,%d,%d,%d>", FMT, UPL, WPR, R);
+    // x goes through k floats of LDS when that stays well inside the default limit beside the decode tables
+    // (and its address is one 16-byte loads accept); longer rows fetch it per lane
+    const size_t xbytes = (size_t)k * 4;
+    const int xstage = xbytes <= 32 * 1024 && (reinterpret_cast<uintptr_t>(x) & 3u) == 0 ? 1 : 0;
+    hipLaunchKernelGGL((gemv_xreg_kernel<FMT, UPL, WPR, R, FUSE>), dim3(p.blocks), dim3(256), xstage ? xbytes : 0, s, w, x, y,
+                       n, k, p.groups, f, xstage);
     RFQ_LAUNCH_CHECK("gemv_xreg_kernel");
     return RFQ_OK;
 }
@@ -1576,6 +1709,7 @@ int launch_idot(const uint8_t *w, const float *x, float *y, int n, int k, int bl
                 hipStream_t s)
 {
     size_t lds = (size_t)(k / 32) * 28 * sizeof(uint32_t);
+    note_kernel(FUSE ? "gemv_idot_kernel<%s,%d,%d,%d,fused>" : "gemv_idot_kernel<%s,%d,%d,%d>", FMT, UPL, WPR, R);
     hipLaunchKernelGGL((gemv_idot_kernel<FMT, UPL, WPR, R, FUSE>), dim3(blocks), dim3(64 * IDOT_WAVES), lds, s, w, x, y, n, k, groups,
                        f);
     RFQ_LAUNCH_CHECK("gemv_idot_kernel");
@@ -1632,6 +1766,7 @@ int launch_idot_batch(const uint8_t *w, const float *x, float *y, int m, int n, 
                                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 4096);
     });
     if (attr_err != hipSuccess) return hip_fail(attr_err, "hipFuncSetAttribute(gemv_idot_batch_kernel)");
+    note_kernel("gemv_idot_batch_kernel<%s,%d,%d,%d>", FMT, WPR, R, M);
     hipLaunchKernelGGL((gemv_idot_batch_kernel<FMT, WPR, R, M>), dim3(blocks), dim3(256), lds, s, w, x, y, n, k, groups,
                        m);
     RFQ_LAUNCH_CHECK("gemv_idot_batch_kernel");
@@ -1678,12 +1813,27 @@ int run_idot_batch_k(const uint8_t *w, const float *x, float *y, int m, int n, i
     return run_idot_batch<FMT, 4, M>(w, x, y, m, n, k, s);
 }
 
+// Windowed loads read whole dwords around a piece: the tensor must start on a multiple of 4.
+template <int FMT> bool tensor_aligned(const uint8_t *w, int, int)
+{
+    return (reinterpret_cast<uintptr_t>(w) & 3u) == 0;
+}
+
 template <int FMT, int M>
 int run_generic(const uint8_t *w, const float *x, float *y, int n, int k, hipStream_t s)
 {
     int blocks = (n + 3) / 4;
     int cap = device_cu_count() * 8;
     if (blocks > cap) blocks = cap;
+    if constexpr (NeedsAlignedTensor<FMT>::value) {
+        if (!tensor_aligned<FMT>(w, n, k)) {
+            note_kernel("gemv_generic_kernel<%s,%d,bytes>", FMT, M, 0, 0);
+            hipLaunchKernelGGL((gemv_generic_kernel<FMT, M, true>), dim3(blocks), dim3(256), 0, s, w, x, y, n, k);
+            RFQ_LAUNCH_CHECK("gemv_generic_kernel");
+            return RFQ_OK;
+        }
+    }
+    note_kernel("gemv_generic_kernel<%s,%d>", FMT, M, 0, 0);
     hipLaunchKernelGGL((gemv_generic_kernel<FMT, M>), dim3(blocks), dim3(256), 0, s, w, x, y, n, k);
     RFQ_LAUNCH_CHECK("gemv_generic_kernel");
     return RFQ_OK;
@@ -1699,6 +1849,7 @@ int run_mfma_q8_0(const uint8_t *w, const float *x, float *y, int m, int n, int 
     if (int rc = workspace(s, parts_bytes + sx_bytes, &tmp, &transient)) return rc;
     _Float16 *parts = reinterpret_cast<_Float16 *>(tmp);
     float *sx = reinterpret_cast<float *>(tmp + parts_bytes);
+    note_kernel("gemv_mfma_prep_kernel + gemv_mfma_q8_0_kernel<%s>", FMT, 0, 0, 0);
     hipLaunchKernelGGL(gemv_mfma_prep_kernel, dim3(units), dim3(256), 0, s, x, parts, sx, m, k);
     hipLaunchKernelGGL(gemv_mfma_q8_0_kernel<FMT>, dim3((n + 15) / 16), dim3(64 * MFMA_WAVES), 0, s, w, parts, sx, y, m, n, k);
     hipError_t launch_err = hipGetLastError();
@@ -1755,6 +1906,9 @@ template <int FMT>
 int run(const uint8_t *w, const float *x, float *y, int m, int n, int k, hipStream_t s)
 {
     const int ku = k / 32;
+    if constexpr (NeedsAlignedTensor<FMT>::value) {
+        if (!tensor_aligned<FMT>(w, n, k)) return run_generic_m<FMT>(w, x, y, m, n, k, s);
+    }
     if (m == 1 && ku > 16 && ku <= 512)                        // (shorter rows leave most of a wavefront's lanes without a unit)
         return run_rows<FMT, false>(w, x, y, n, k, GemvFuse{nullptr, nullptr, 0.0f, 0}, s);
     if constexpr (FMT == RFQ_Q8_0 || FMT == RFQ_GGUF_Q8_0) {
@@ -1816,6 +1970,11 @@ int launch_gemv_fused(int fmt, const uint8_t *d_w, const uint8_t *d_w2, const fl
     if (k % fmt_block_elems(fmt) != 0) return RFQ_E_UNSUPPORTED;
     const GemvFuse f{d_w2, d_norm_w, eps, d_w2 != nullptr ? 1 : 0};
     const int rows = d_w2 != nullptr ? 2 * n : n;
+    // (GGUF_Q6_K pieces are fetched through aligned windows: both matrices must start on a multiple of 4, else the
+    // caller composes the separate steps, which take the byte-exact kernel)
+    if (canonical_format(fmt) == RFQ_GGUF_Q6_K &&
+        ((reinterpret_cast<uintptr_t>(d_w) | (d_w2 ? reinterpret_cast<uintptr_t>(d_w2) : 0)) & 3u) != 0)
+        return RFQ_E_UNSUPPORTED;
     switch (canonical_format(fmt)) {
     case RFQ_Q4_0: return run_rows<RFQ_Q4_0, true>(d_w, d_x, d_y, rows, k, f, s);
     case RFQ_Q8_0: return run_rows<RFQ_Q8_0, true>(d_w, d_x, d_y, rows, k, f, s);
@@ -1832,3 +1991,28 @@ int launch_gemv_fused(int fmt, const uint8_t *d_w, const uint8_t *d_w2, const fl
 }
 
 } // namespace rfq
+
+extern "C" RFQ_API const char *rfq_bench_last_gemv_kernel(void)
+{
+    static thread_local char text[128];
+    const rfq::LastKernel &k = rfq::g_last_kernel;
+    const char *f = "?";
+    switch (k.fmt) {
+    case RFQ_Q4_0: f = "Q4_0"; break;
+    case RFQ_Q8_0: f = "Q8_0"; break;
+    case RFQ_Q4_K: f = "Q4_K"; break;
+    case RFQ_Q6_K: f = "Q6_K"; break;
+    case RFQ_MXFP4: f = "MXFP4"; break;
+    case RFQ_MXFP6_E2M3: f = "MXFP6"; break;
+    case RFQ_GGUF_Q4_0: f = "GGUF_Q4_0"; break;
+    case RFQ_GGUF_Q8_0: f = "GGUF_Q8_0"; break;
+    case RFQ_GGUF_Q4_K: f = "GGUF_Q4_K"; break;
+    case RFQ_GGUF_Q6_K: f = "GGUF_Q6_K"; break;
+    case RFQ_MM_Q8_0: f = "MM_Q8_0"; break;
+    case RFQ_MM_Q4_K: f = "MM_Q4_K"; break;
+    case RFQ_MM_Q6_K: f = "MM_Q6_K"; break;
+    default: break;
+    }
+    snprintf(text, sizeof text, k.name, f, k.a, k.b, k.c);
+    return text;
+}

@@ -327,6 +327,23 @@ def quantize_gguf_q6_k(w: np.ndarray) -> np.ndarray:
     return out.ravel()
 
 
+def mxfp4_window_blocks(rng: np.random.Generator, nblk: int, exp_range=(-6, 1), zero_blocks: float = 0.05) -> np.ndarray:
+    """Random MXFP4 blocks whose values span at most the four octaves a 4-bit matrix-core operand holds: every
+    code of a window of exponents -1..2 or 0..3, zeros, both signs (the reference's packer only ever produces codes
+    {0, 1, 8, 9} of the second window).  Full-entropy input for the 4-bit path of the prefill GEMM."""
+    p_of_m = np.array([-1, 0, 0, 1, 1, 2, 2, 3])
+    raw = np.zeros((nblk, 17), dtype=np.uint8)
+    raw[:, 0] = rng.integers(exp_range[0], exp_range[1] + 1, size=nblk).astype(np.int8).view(np.uint8)
+    codes = rng.integers(0, 16, size=(nblk, 32))
+    lo = rng.integers(-1, 1, size=nblk)[:, None]
+    p = p_of_m[codes & 7]
+    codes = np.where((codes != 0) & ((p < lo) | (p > lo + 3)), 0, codes)
+    if zero_blocks > 0:
+        codes[rng.random(nblk) < zero_blocks] = 0                              # some all-zero blocks
+    raw[:, 1:] = ((codes[:, 0::2] << 4) | codes[:, 1::2]).astype(np.uint8)     # element 2j in the high nibble
+    return raw.reshape(-1)
+
+
 def random_blocks(fmt: int, n_blocks: int, rng: np.random.Generator, exp_range=(-20, 12)) -> np.ndarray:
     """Uniformly random payload bytes with sane scales, covering every code."""
     bb = BLOCK_BYTES[fmt]

@@ -294,6 +294,72 @@ static void test_matmul_q4_0_against_dequantized_weights()
     bytes shorter(w.begin(), w.end() - 20);
     EXPECT(!matmul_q4_0(be.value, shorter, in.value, n_rows, n_cols, out.value).ok);
 }
+// What the reference computes on the bytes (src/kernels/matmul/quantized/q4_0.rs:274-311 + src/tensor/matmul.rs:219-233,
+// kernels/q4_0_matmul.hip:207): the flat dequantised array read as b[k, n], and the module's own int8 decoder
+// (quantized/q8_0.rs:18-56; its unit-test vector :113-131).
+static void test_matmul_as_the_reference_computes_it()
+{
+    const size_t n_rows = 8, n_cols = 64;
+    bytes w(n_rows * n_cols / 32 * 20);
+    for (size_t b = 0; b < w.size() / 20; b++) {
+        put_f32(w, b * 20, 0.25f * (float)(b % 5 + 1));
+        for (int i = 0; i < 16; i++) w[b * 20 + 4 + i] = (uint8_t)((b * 37 + i * 11) & 0xFF);
+    }
+    std::vector<float> x(n_cols);
+    for (size_t i = 0; i < n_cols; i++) x[i] = 0.125f * (float)((int)(i % 9) - 4);
+    auto be = HipBackend::create();
+    auto in = HipBuffer::create(n_cols * 4), out = HipBuffer::create(n_rows * 4), out2 = HipBuffer::create(n_rows * 4);
+    EXPECT(in.value.copy_from_host(x).ok);
+    EXPECT(matmul_q4_0_cpu_fallback(be.value, w, in.value, n_rows, n_cols, out.value).ok);
+    std::vector<float> y(n_rows), y2(n_rows), deq = matmul_quantized::dequantize_q4_0(w, n_rows * n_cols);
+    EXPECT(out.value.copy_to_host(y).ok);
+    bool close = true, differs = false;
+    for (size_t j = 0; j < n_rows; j++) {
+        float s = 0.0f, s_rows = 0.0f;
+        for (size_t l = 0; l < n_cols; l++) s += x[l] * deq[l * n_rows + j];          // cpu_matmul_f32: b[l * n + j]
+        for (size_t l = 0; l < n_cols; l++) s_rows += x[l] * deq[j * n_cols + l];
+        if (std::fabs(y[j] - s) > 1e-3f * std::fmax(std::fabs(s), 1.0f)) close = false;
+        if (std::fabs(s - s_rows) > 1e-2f) differs = true;
+    }
+    EXPECT(close);
+    EXPECT(differs);                                                                   // the two readings are different numbers
+    auto dw = HipBuffer::create(w.size());
+    EXPECT(dw.value.copy_from_host(w).ok);
+    EXPECT(matmul_q4_0_gpu(be.value, (const float *)in.value.as_ptr(), (const uint8_t *)dw.value.as_ptr(),
+                           (float *)out2.value.as_ptr(), 1, n_rows, n_cols, WeightLayout::FlatKN).ok);
+    EXPECT(be.value.synchronize().ok && out2.value.copy_to_host(y2).ok && y2 == y);
+    // int8 decoder: scale 1.0, bytes (i - 16) as u8 -> i - 16
+    bytes q8(36);
+    put_f32(q8, 0, 1.0f);
+    for (int i = 0; i < 32; i++) q8[4 + i] = (uint8_t)(int8_t)(i - 16);
+    auto v = matmul_quantized::dequantize_q8_0(q8, 32);
+    bool exact = true;
+    for (int i = 0; i < 32; i++) if (v[i] != (float)(i - 16)) exact = false;
+    EXPECT(exact);
+    // matmul_q8_0 as its body computes it: 32 rows x 1 column of that block, x = 1 -> the sum of the 32 values... over l:
+    // n_rows = 1, n_cols = 32: out[0] = sum_l x[l] * deq[l]
+    std::vector<float> ones(32, 1.0f);
+    auto in8 = HipBuffer::create(32 * 4), out8 = HipBuffer::create(4);
+    EXPECT(in8.value.copy_from_host(ones).ok);
+    EXPECT(matmul_q8_0_as_computed(be.value, q8, in8.value, 1, 32, out8.value).ok);
+    std::vector<float> y8(1);
+    EXPECT(out8.value.copy_to_host(y8).ok && y8[0] == -16.0f);                          // sum of -16 .. 15
+    // the K decoders of the module: normal scales decode like the loader's Q6_K; Q4_K reads other bytes
+    bytes k6(256, 0);
+    for (int g = 0; g < 16; g++) put_f16(k6, 2 * g, 0x3C00);                           // 1.0
+    for (int i = 32; i < 224; i++) k6[i] = (uint8_t)(i * 7);
+    EXPECT(matmul_quantized::dequantize_q6_k(k6, 256) == loader::dequant_q6_k(k6, 256));
+    bytes k4(256, 0);
+    for (int sb = 0; sb < 8; sb++) put_f16(k4, 2 * sb, 0x3C00);
+    for (int i = 32; i < 256; i++) k4[i] = (uint8_t)(i * 5 + 1);
+    auto a4 = matmul_quantized::dequantize_q4_k(k4, 256), c4 = loader::dequant_q4_k(k4, 256);
+    bool sb0_same = true, rest_differs = false;
+    for (int i = 0; i < 32; i++) if (a4[i] != c4[i]) sb0_same = false;
+    for (int i = 32; i < 256; i++) if (a4[i] != c4[i]) rest_differs = true;
+    EXPECT(sb0_same && rest_differs);
+    EXPECT(a4[32] == (float)(k4[32 + 20] & 15));                                      // sub-block 1 starts at byte 52
+}
+
 static void test_matmul_validation_like_op_dispatch()
 {
     EXPECT(validate_matmul_q4_0({8, 64}, 8 * 2 * 20, {1, 64}).ok);
@@ -509,6 +575,7 @@ int main()
         {"test_dequantize_dispatch_f32_f16", test_dequantize_dispatch_f32_f16},
         {"test_dequantize_q4_0_kernel_cached_and_twins", test_dequantize_q4_0_kernel_cached_and_twins},
         {"test_matmul_q4_0_against_dequantized_weights", test_matmul_q4_0_against_dequantized_weights},
+        {"test_matmul_as_the_reference_computes_it", test_matmul_as_the_reference_computes_it},
         {"test_matmul_validation_like_op_dispatch", test_matmul_validation_like_op_dispatch},
         {"test_get_rows_f32_and_packed_tables", test_get_rows_f32_and_packed_tables},
         {"test_norm_swiglu_and_mlp", test_norm_swiglu_and_mlp},

@@ -194,3 +194,28 @@ def test_long_matrices_one_unit_per_lane(fmt, n, k, oracle, cuda):
     x = x_for(1, k, 6300 + k)
     got = gpu_gemv(fmt, w, x, n, k, cuda)
     assert_close(got, oracle.qmatmul_nk(fmt, w, x, 1, n, k), f"{Q.NAMES[fmt]} {n}x{k}")
+
+
+# The 17-, 25-, 18-, 34- and 210-byte layouts are read in place at whatever alignment their blocks have (the 210-byte
+# one through aligned windows of whole dwords when the tensor starts on a multiple of 4, byte-exactly otherwise):
+# weights at odd device addresses, and tensors whose byte count is not a multiple of 4, must agree with the oracle.
+@pytest.mark.parametrize("fmt", [Q.MXFP4, Q.MXFP6_E2M3, Q.GGUF_Q4_0, Q.GGUF_Q8_0, Q.GGUF_Q6_K])
+def test_gemv_windowed_layouts_at_any_address(fmt, oracle, cuda):
+    import torch
+    from rocmforge_amd import _lib
+    L = _lib.lib()
+    be = Q.BLOCK_ELEMS[fmt]
+    for (m, n, k) in [(1, 130, 4096), (1, 3, 3 * be), (4, 33, 2048), (1, 5, 5 * be)]:
+        rng = np.random.default_rng(9000 + fmt + n)
+        w = Q.random_blocks(fmt, n * k // be, rng, exp_range=(-9, 3))
+        x = rng.standard_normal((m, k)).astype(np.float32)
+        want = oracle.qmatmul_nk(fmt, w, x, m, n, k)
+        dx = torch.from_numpy(x).to(cuda)
+        for off in (0, 1, 2, 3):
+            buf = torch.zeros(w.size + 8, dtype=torch.uint8, device=cuda)
+            buf[off:off + w.size] = torch.from_numpy(w).to(cuda)
+            y = torch.empty((m, n), dtype=torch.float32, device=cuda)
+            _lib.check(L.rfq_gemv(fmt, C.c_void_p(buf.data_ptr() + off), w.size, C.c_void_p(dx.data_ptr()),
+                                  C.c_void_p(y.data_ptr()), m, n, k, None))
+            torch.cuda.synchronize()
+            assert_close(y.cpu().numpy(), want, f"{Q.NAMES[fmt]} m={m} n={n} k={k} offset {off}")
