@@ -4,9 +4,10 @@ MXFP4 GEMM at M=2048, K=8192, N=28672 (bf16 out) and the MXFP6-weight variant,
 plus the Q4_K fp16 GEMM at M=512, K=4096, N=14336 when that kernel is built.
 FLOPs = 2*M*N*K; peaks: 10.1 PFLOP/s (FP4 scaled MFMA), 5.0 (FP8), 2.5 (fp16).
 
-Each configuration runs at most 40 untimed launches, then `steps` timed ones; the figure is the average over
-all timed launches (the launches of the first tens of milliseconds after an idle period run 5-15 % slower than
-the steady state: the part's clocks ramp, and the timed region is long enough to carry that).  The MXFP4 GEMM
+The launches of the first tens of milliseconds after an idle period run 5-15 % slower than the steady state (the
+part's clocks ramp).  The MXFP4 configurations run 40 untimed launches (7 ms), then 200 timed ones, and report the
+average over all timed launches, ramp included; the fp16 K-quant configurations run 300 untimed launches (20 ms)
+and 300 timed ones (`warmup_launches` / `timed_launches` in each line say which).  The MXFP4 GEMM
 is reported three ways: on operands from the reference's packer (which emits only codes {0, 1, 8, 9}), on
 full-entropy operands (every code of a four-octave window, both signs), and as a prefill step that re-encodes
 the raw activations for the matrix core before every GEMM.
@@ -86,7 +87,7 @@ def mx_gemm(torch, w_fmt, m=2048, n=28672, k=8192, steps=200, warmup=40, data="p
     return res
 
 
-def kq_gemm(torch, fmt, m=512, n=14336, k=4096, steps=300, warmup=40):
+def kq_gemm(torch, fmt, m=512, n=14336, k=4096, steps=300, warmup=300):
     """Q4_K / Q6_K prefill GEMM on the fp16 matrix cores, fp16 in and out."""
     from rocmforge_amd import _lib, quantize as Q
     dev = torch.device("cuda:0")
