@@ -158,6 +158,33 @@ def time_get_rows(torch, fmt, n_vocab, n_embd, n_tokens, Q):
     return {"us": round(t * 1e6, 2), "GB/s": round(b / t / 1e9, 1), "rows/s": round(n_tokens / t)}
 
 
+def time_gemv_kn(torch, fmt, n, k, Q, copies=6, reps=10):
+    """The reference's own orientation (y[j] = sum_l x[l] * Wd[l * n + j] over the flat dequantised stream) on the
+    same bytes as the headline, rotating weight copies."""
+    import numpy as np
+
+    from rocmforge_amd import ops
+    dev = torch.device("cuda:0")
+    w = torch.from_numpy(Q.make_weights(fmt, n, k, seed=20260003)).to(dev)
+    ws = [w.clone() for _ in range(copies)]
+    rng = np.random.Generator(np.random.PCG64(20260036))
+    x = torch.from_numpy(rng.standard_normal(k, dtype=np.float32)).to(dev)
+    out = torch.empty((1, n), dtype=torch.float32, device=dev)
+    for wc in ws:
+        ops.gemv_kn(fmt, wc, x, n, k, out=out)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(reps):
+        for wc in ws:
+            ops.gemv_kn(fmt, wc, x, n, k, out=out)
+    e1.record()
+    torch.cuda.synchronize()
+    t = e0.elapsed_time(e1) / (reps * copies) * 1e-3
+    b = algorithmic_bytes(fmt, n, k, 1, Q)
+    return {"us": round(t * 1e6, 2), "GB/s": round(b / t / 1e9, 1), "hbm_frac": round(b / t / 1e9 / HBM_PEAK_GBS, 4)}
+
+
 def time_mlp(torch, fmt, hidden, inter, Q, steps=300, warmup=60):
     """The SwiGLU MLP of one decode step (RMSNorm, gate and up projections, activation, down projection) over
     rotating weight sets: rfq_mlp_swiglu (two launches) and the same arithmetic as five separate calls."""
@@ -473,6 +500,7 @@ def main():
             b = algorithmic_bytes(f, n, k, m, Q)
             also[name] = {"GB/s": round(b / (d / 500) / 1e9, 1), "us": round(d / 500 * 1e6, 2),
                           "hbm_frac": round(b / (d / 500) / 1e9 / HBM_PEAK_GBS, 4)}
+        also["Q4_K gemv_kn n=14336 k=4096 (the orientation the reference computes)"] = time_gemv_kn(torch, Q.Q4_K, N, K, Q)
         also["Q4_K mlp_swiglu 4096x14336 m1"] = time_mlp(torch, Q.Q4_K, 4096, 14336, Q)
         also["Q4_K get_rows 512 of 128256x4096"] = time_get_rows(torch, Q.Q4_K, 128256, 4096, 512, Q)
         for name, f, n, k, seed in (("Q4_0 dequant 4096x4096", Q.Q4_0, 4096, 4096, 20260021),
