@@ -67,8 +67,8 @@ def mx_gemm(torch, w_fmt, m=2048, n=28672, k=8192, steps=200, warmup=40, data="p
         return round(e0.elapsed_time(e1) / reps * 1e3, 1)
 
     prep = {"prepare_a_us": prepare_us(Q.MXFP4, a_dev, m, A.kind), "prepare_w_us": prepare_us(w_fmt, w_dev, n, W.kind, reps=5)}
-    args = (C.c_void_p(A.buf.data_ptr()), A.kind, C.c_void_p(W.buf.data_ptr()), W.kind, C.c_void_p(out.data_ptr()),
-            _lib.BF16, m, n, k)
+    args = (C.c_void_p(A.buf.data_ptr()), A.buf.numel(), A.kind, C.c_void_p(W.buf.data_ptr()), W.buf.numel(), W.kind,
+            C.c_void_p(out.data_ptr()), _lib.BF16, m, n, k)
     _lib.check(L.rfq_bench_gemm_mx(*args, warmup, steps, stream, C.byref(ms)))
     t = ms.value / 1e3 / steps
     flops = 2.0 * m * n * k
@@ -79,7 +79,7 @@ def mx_gemm(torch, w_fmt, m=2048, n=28672, k=8192, steps=200, warmup=40, data="p
     if A.kind == _lib.MX_FP4 and data == "packer":
         # the prefill step end to end: raw MXFP4 activations re-encoded before every GEMM
         _lib.check(L.rfq_bench_gemm_mx_prefill(C.c_void_p(a_dev.data_ptr()), a_dev.numel(), C.c_void_p(A.buf.data_ptr()),
-                                               A.buf.numel(), C.c_void_p(W.buf.data_ptr()), W.kind, C.c_void_p(out.data_ptr()),
+                                               A.buf.numel(), C.c_void_p(W.buf.data_ptr()), W.buf.numel(), W.kind, C.c_void_p(out.data_ptr()),
                                                _lib.BF16, m, n, k, warmup, steps, stream, C.byref(ms)))
         te = ms.value / 1e3 / steps
         res["prefill_step"] = {"us": round(te * 1e6, 1), "TFLOP/s": round(flops / te / 1e12, 1), "mfma_frac": round(flops / te / peak, 4),

@@ -358,9 +358,14 @@ RFQ_API int rfq_mx_prepare(int fmt, int kind_req, const void *d_raw, size_t raw_
 
 /* d_out[m, n] = A[m, k] . W[n, k]^T from two prepared operands, fp32
  * accumulation in the matrix core, out_dtype RFQ_F32 or RFQ_BF16.
- * m, n multiples of 32 are not required; k a multiple of 128 is. */
-RFQ_API int rfq_gemm_mx(const void *d_a_prep, int a_kind, const void *d_w_prep, int w_kind, void *d_out,
-                int out_dtype, int m, int n, int k, void *stream);
+ * m, n multiples of 32 are not required; k a multiple of 128 is.
+ * a_prep_bytes / w_prep_bytes are the sizes of the two prepared buffers: each
+ * must be at least what rfq_mx_prepared_bytes gives for (a_kind, m, k) and
+ * (w_kind, n, k) -- a buffer sized for RFQ_MX_AUTO that came out as FP4 is larger --
+ * so a shape beyond what was prepared is refused (RFQ_E_SIZE) instead of read
+ * out of bounds. */
+RFQ_API int rfq_gemm_mx(const void *d_a_prep, size_t a_prep_bytes, int a_kind, const void *d_w_prep,
+                size_t w_prep_bytes, int w_kind, void *d_out, int out_dtype, int m, int n, int k, void *stream);
 
 #ifdef __cplusplus
 }

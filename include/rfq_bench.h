@@ -47,16 +47,16 @@ RFQ_API int rfq_bench_gemm_f16(int fmt, const void *d_w, size_t w_bytes, const v
                                int out_dtype, int m, int n, int k, int warmup, int steps, void *stream,
                                float *elapsed_ms);
 
-RFQ_API int rfq_bench_gemm_mx(const void *d_a_prep, int a_kind, const void *d_w_prep, int w_kind, void *d_out,
-                              int out_dtype, int m, int n, int k, int warmup, int steps, void *stream,
-                              float *elapsed_ms);
+RFQ_API int rfq_bench_gemm_mx(const void *d_a_prep, size_t a_prep_bytes, int a_kind, const void *d_w_prep,
+                              size_t w_prep_bytes, int w_kind, void *d_out, int out_dtype, int m, int n, int k,
+                              int warmup, int steps, void *stream, float *elapsed_ms);
 
 /* A prefill step as a caller that holds raw MXFP4 activations runs it: re-encode A for the matrix core
  * (rfq_mx_prepare, RFQ_MX_FP4_UNCHECKED: no read-back, no synchronisation) into d_a_prep, then rfq_gemm_mx
  * against the weights prepared once at upload. */
 RFQ_API int rfq_bench_gemm_mx_prefill(const void *d_a_raw, size_t a_raw_bytes, void *d_a_prep, size_t a_prep_bytes,
-                                      const void *d_w_prep, int w_kind, void *d_out, int out_dtype, int m, int n, int k,
-                                      int warmup, int steps, void *stream, float *elapsed_ms);
+                                      const void *d_w_prep, size_t w_prep_bytes, int w_kind, void *d_out, int out_dtype,
+                                      int m, int n, int k, int warmup, int steps, void *stream, float *elapsed_ms);
 
 /* Step i runs the MLP over weight set i % copies.  one_call != 0: rfq_mlp_swiglu;
  * one_call == 0: the same arithmetic as five calls (rfq_rms_norm, rfq_gemv for

@@ -450,8 +450,8 @@ int rfq_mx_prepare(int fmt, int kind_req, const void *d_raw, size_t raw_bytes, i
                              (hipStream_t)stream);
 }
 
-int rfq_gemm_mx(const void *d_a_prep, int a_kind, const void *d_w_prep, int w_kind, void *d_out, int out_dtype, int m,
-                int n, int k, void *stream)
+int rfq_gemm_mx(const void *d_a_prep, size_t a_prep_bytes, int a_kind, const void *d_w_prep, size_t w_prep_bytes,
+                int w_kind, void *d_out, int out_dtype, int m, int n, int k, void *stream)
 {
     if (!d_a_prep || !d_w_prep || !d_out) return fail(RFQ_E_BADARG, "rfq_gemm_mx: null pointer");
     if (m <= 0 || n <= 0 || k <= 0) return fail(RFQ_E_BADARG, "rfq_gemm_mx: bad shape m=%d n=%d k=%d", m, n, k);
@@ -460,6 +460,15 @@ int rfq_gemm_mx(const void *d_a_prep, int a_kind, const void *d_w_prep, int w_ki
         return fail(RFQ_E_BADARG, "rfq_gemm_mx: operand kinds must be FP4 or FP8 (a=%d w=%d)", a_kind, w_kind);
     if (out_dtype != RFQ_F32 && out_dtype != RFQ_BF16)
         return fail(RFQ_E_BADARG, "rfq_gemm_mx: out_dtype %d is neither F32 nor BF16", out_dtype);
+    // (the layout of a prepared operand depends on its kind and shape only; an FP4 operand is always MXFP4)
+    const size_t a_need = mx_prepared_bytes(a_kind == RFQ_MX_FP4 ? RFQ_MXFP4 : RFQ_MXFP6_E2M3, a_kind, m, k);
+    const size_t w_need = mx_prepared_bytes(w_kind == RFQ_MX_FP4 ? RFQ_MXFP4 : RFQ_MXFP6_E2M3, w_kind, n, k);
+    if (a_need == 0 || a_prep_bytes < a_need)
+        return fail(RFQ_E_SIZE, "rfq_gemm_mx: prepared A has %zu bytes, [%d x %d] of kind %d needs %zu", a_prep_bytes, m, k,
+                    a_kind, a_need);
+    if (w_need == 0 || w_prep_bytes < w_need)
+        return fail(RFQ_E_SIZE, "rfq_gemm_mx: prepared W has %zu bytes, [%d x %d] of kind %d needs %zu", w_prep_bytes, n, k,
+                    w_kind, w_need);
     return launch_gemm_mx(d_a_prep, a_kind, d_w_prep, w_kind, d_out, out_dtype, m, n, k, (hipStream_t)stream);
 }
 

@@ -115,23 +115,24 @@ int rfq_bench_gemm_f16(int fmt, const void *d_w, size_t w_bytes, const void *d_a
     });
 }
 
-int rfq_bench_gemm_mx(const void *d_a_prep, int a_kind, const void *d_w_prep, int w_kind, void *d_out, int out_dtype,
-                      int m, int n, int k, int warmup, int steps, void *stream, float *elapsed_ms)
+int rfq_bench_gemm_mx(const void *d_a_prep, size_t a_prep_bytes, int a_kind, const void *d_w_prep, size_t w_prep_bytes,
+                      int w_kind, void *d_out, int out_dtype, int m, int n, int k, int warmup, int steps, void *stream,
+                      float *elapsed_ms)
 {
     return timed_loop(warmup, steps, stream, elapsed_ms, [&](int) {
-        return rfq_gemm_mx(d_a_prep, a_kind, d_w_prep, w_kind, d_out, out_dtype, m, n, k, stream);
+        return rfq_gemm_mx(d_a_prep, a_prep_bytes, a_kind, d_w_prep, w_prep_bytes, w_kind, d_out, out_dtype, m, n, k, stream);
     });
 }
 
 int rfq_bench_gemm_mx_prefill(const void *d_a_raw, size_t a_raw_bytes, void *d_a_prep, size_t a_prep_bytes,
-                              const void *d_w_prep, int w_kind, void *d_out, int out_dtype, int m, int n, int k, int warmup,
-                              int steps, void *stream, float *elapsed_ms)
+                              const void *d_w_prep, size_t w_prep_bytes, int w_kind, void *d_out, int out_dtype, int m,
+                              int n, int k, int warmup, int steps, void *stream, float *elapsed_ms)
 {
     return timed_loop(warmup, steps, stream, elapsed_ms, [&](int) {
         int kind = 0;
         int rc = rfq_mx_prepare(RFQ_MXFP4, RFQ_MX_FP4_UNCHECKED, d_a_raw, a_raw_bytes, m, k, d_a_prep, a_prep_bytes, &kind, stream);
         if (rc != RFQ_OK) return rc;
-        return rfq_gemm_mx(d_a_prep, kind, d_w_prep, w_kind, d_out, out_dtype, m, n, k, stream);
+        return rfq_gemm_mx(d_a_prep, a_prep_bytes, kind, d_w_prep, w_prep_bytes, w_kind, d_out, out_dtype, m, n, k, stream);
     });
 }
 

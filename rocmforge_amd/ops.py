@@ -30,6 +30,31 @@ def _dev_u8(t: torch.Tensor) -> torch.Tensor:
     return t
 
 
+def _f32(t: torch.Tensor, what: str) -> torch.Tensor:
+    if not (t.is_cuda and t.dtype == torch.float32 and t.is_contiguous()):
+        raise ValueError(f"{what} must be a contiguous float32 device tensor")
+    return t
+
+
+def _rows_of(x: torch.Tensor, k: int, what: str) -> int:
+    """Rows of x[m, k] (or of a single vector x[k]); the last axis must be k."""
+    if x.dim() not in (1, 2) or x.shape[-1] != k:
+        raise ValueError(f"{what} has shape {tuple(x.shape)}, expected [m, {k}] or [{k}]")
+    return 1 if x.dim() == 1 else x.shape[0]
+
+
+def _out(out: torch.Tensor | None, shape, dtype, like: torch.Tensor) -> torch.Tensor:
+    """The caller's output buffer, checked, or a new one on the device of `like`."""
+    if out is None:
+        return torch.empty(shape, dtype=dtype, device=like.device)
+    n = 1
+    for d in shape:
+        n *= d
+    if not (out.is_cuda and out.device == like.device and out.dtype == dtype and out.is_contiguous() and out.numel() == n):
+        raise ValueError(f"out must be a contiguous {dtype} tensor of {n} elements on {like.device}")
+    return out
+
+
 def upload(host: "np.ndarray | bytes | memoryview", out: torch.Tensor | None = None) -> torch.Tensor:
     """Host bytes -> a device uint8 tensor through the library's pinned staging ring (rfq_upload)."""
     import numpy as np
@@ -45,20 +70,18 @@ def upload(host: "np.ndarray | bytes | memoryview", out: torch.Tensor | None = N
 def dequant(fmt: int, packed: torch.Tensor, n_elems: int, out: torch.Tensor | None = None) -> torch.Tensor:
     """Packed device bytes -> f32 device tensor of n_elems."""
     packed = _dev_u8(packed)
-    if out is None:
-        out = torch.empty(n_elems, dtype=torch.float32, device=packed.device)
+    if n_elems < 0:
+        raise ValueError("n_elems is negative")
+    out = _out(out, (n_elems,), torch.float32, packed)
     check(lib().rfq_dequant(fmt, _ptr(packed), packed.numel(), _ptr(out), n_elems, _stream()))
     return out
 
 
 def gemv(fmt: int, w: torch.Tensor, x: torch.Tensor, n: int, k: int, out: torch.Tensor | None = None) -> torch.Tensor:
     """y[m, n] = x[m, k] . dequant(W)[n, k]^T (m <= 8), fp32."""
-    w = _dev_u8(w)
-    if x.dtype != torch.float32 or not x.is_contiguous():
-        raise ValueError("x must be contiguous float32")
-    m = 1 if x.dim() == 1 else x.shape[0]
-    if out is None:
-        out = torch.empty((m, n), dtype=torch.float32, device=x.device)
+    w, x = _dev_u8(w), _f32(x, "x")
+    m = _rows_of(x, k, "x")
+    out = _out(out, (m, n), torch.float32, x)
     check(lib().rfq_gemv(fmt, _ptr(w), w.numel(), _ptr(x), _ptr(out), m, n, k, _stream()))
     return out if x.dim() > 1 else out.view(n)
 
@@ -67,15 +90,9 @@ def gemv_kn(fmt: int, w: torch.Tensor, x: torch.Tensor, n: int, k: int, out: tor
     """y[m, n] = x[m, k] . Wd[k, n] with Wd[l, j] = element l * n + j of the packed stream decoded as one flat
     array: the orientation the reference's kernel and CPU fallback compute (kernels/q4_0_matmul.hip:207,
     src/kernels/matmul/quantized/q4_0.rs:274-311)."""
-    w = _dev_u8(w)
-    x = _f32(x, "x")
-    m = 1 if x.dim() == 1 else x.shape[0]
-    if x.shape[-1] != k:
-        raise ValueError(f"x has {x.shape[-1]} columns, k = {k}")
-    if out is None:
-        out = torch.empty((m, n), dtype=torch.float32, device=x.device)
-    elif not (out.is_cuda and out.dtype == torch.float32 and out.is_contiguous() and out.numel() == m * n):
-        raise ValueError("out must be a contiguous float32 device tensor of m * n elements")
+    w, x = _dev_u8(w), _f32(x, "x")
+    m = _rows_of(x, k, "x")
+    out = _out(out, (m, n), torch.float32, x)
     check(lib().rfq_gemv_kn(fmt, _ptr(w), w.numel(), _ptr(x), _ptr(out), m, n, k, _stream()))
     return out if x.dim() > 1 else out.view(n)
 
@@ -84,30 +101,29 @@ def get_rows(fmt: int, table: torch.Tensor, tokens: torch.Tensor, n_vocab: int, 
              status: torch.Tensor | None = None) -> torch.Tensor:
     """out[i, :] = dequantised (fmt = block format) or copied (fmt = 0, f32 table) row tokens[i] of the table."""
     if fmt == 0:
-        if table.dtype != torch.float32 or not table.is_contiguous():
-            raise ValueError("an f32 table must be a contiguous float32 tensor")
+        table = _f32(table, "an f32 table")
         nbytes = table.numel() * 4
     else:
         table = _dev_u8(table)
         nbytes = table.numel()
-    if tokens.dtype not in (torch.int32, torch.uint32) or not tokens.is_contiguous():
-        raise ValueError("tokens must be a contiguous int32/uint32 tensor")
+    if not (tokens.is_cuda and tokens.device == table.device and tokens.dtype in (torch.int32, torch.uint32)
+            and tokens.is_contiguous()):
+        raise ValueError("tokens must be a contiguous int32/uint32 tensor on the table's device")
+    if status is not None and not (status.is_cuda and status.device == table.device and status.dtype == torch.int32
+                                   and status.numel() >= 1):
+        raise ValueError("status must be an int32 tensor on the table's device")
     out = torch.empty((tokens.numel(), n_embd), dtype=torch.float32, device=table.device)
     check(lib().rfq_get_rows(fmt, _ptr(table), nbytes, n_vocab, n_embd, _ptr(tokens), tokens.numel(), _ptr(out),
                              _ptr(status) if status is not None else None, _stream()))
     return out
 
 
-def _f32(t: torch.Tensor, what: str) -> torch.Tensor:
-    if not (t.is_cuda and t.dtype == torch.float32 and t.is_contiguous()):
-        raise ValueError(f"{what} must be a contiguous float32 device tensor")
-    return t
-
-
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     """RMSNorm over the last axis of x[seq_len, hidden] (src/mlp/kernels.rs:261-330)."""
     x, weight = _f32(x, "x"), _f32(weight, "weight")
     hidden = x.shape[-1]
+    if weight.numel() != hidden:
+        raise ValueError(f"weight has {weight.numel()} elements, hidden = {hidden}")
     out = torch.empty_like(x)
     check(lib().rfq_rms_norm(_ptr(x), _ptr(weight), _ptr(out), x.numel() // hidden, hidden, eps, _stream()))
     return out
@@ -128,6 +144,8 @@ def dequant_rms_norm(fmt: int, packed: torch.Tensor, weight: torch.Tensor, seq_l
                      eps: float) -> torch.Tensor:
     """RMSNorm of packed rows, decoded on the fly (src/ggml/hip_backend/ops/fused_ops.rs:149-160)."""
     packed, weight = _dev_u8(packed), _f32(weight, "weight")
+    if weight.numel() != hidden:
+        raise ValueError(f"weight has {weight.numel()} elements, hidden = {hidden}")
     out = torch.empty((seq_len, hidden), dtype=torch.float32, device=packed.device)
     check(lib().rfq_dequant_rms_norm(fmt, _ptr(packed), packed.numel(), _ptr(weight), _ptr(out), seq_len, hidden, eps,
                                      _stream()))
@@ -138,7 +156,9 @@ def rms_norm_gemv(fmt: int, w: torch.Tensor, x: torch.Tensor, norm_weight: torch
                   k: int, scratch: bool = True) -> torch.Tensor:
     """y[m, n] = RMSNorm(x[m, k]) . dequant(W)[n, k]^T in one call."""
     w, x, norm_weight = _dev_u8(w), _f32(x, "x"), _f32(norm_weight, "norm_weight")
-    m = 1 if x.dim() == 1 else x.shape[0]
+    m = _rows_of(x, k, "x")
+    if norm_weight.numel() != k:
+        raise ValueError(f"norm_weight has {norm_weight.numel()} elements, k = {k}")
     out = torch.empty((m, n), dtype=torch.float32, device=x.device)
     tmp = torch.empty((m, k), dtype=torch.float32, device=x.device) if scratch else None
     check(lib().rfq_rms_norm_gemv(fmt, _ptr(w), w.numel(), _ptr(x), _ptr(norm_weight), eps, _ptr(out), m, n, k,
@@ -154,10 +174,14 @@ def mlp_swiglu(fmt_gate_up: int, gate_w: torch.Tensor, up_w: torch.Tensor, fmt_d
     gate_w, up_w, down_w, x = _dev_u8(gate_w), _dev_u8(up_w), _dev_u8(down_w), _f32(x, "x")
     if gate_w.numel() != up_w.numel():
         raise ValueError("gate and up weights differ in size")
-    m = 1 if x.dim() == 1 else x.shape[0]
+    m = _rows_of(x, hidden, "x")
+    if norm_weight is not None and _f32(norm_weight, "norm_weight").numel() != hidden:
+        raise ValueError(f"norm_weight has {norm_weight.numel()} elements, hidden = {hidden}")
     need = lib().rfq_mlp_scratch_bytes(m, hidden, inter)
     if scratch is None:
         scratch = torch.empty(need, dtype=torch.uint8, device=x.device)
+    elif not (scratch.is_cuda and scratch.device == x.device and scratch.dtype == torch.uint8 and scratch.is_contiguous()):
+        raise ValueError("scratch must be a contiguous uint8 tensor on x's device")
     out = torch.empty((m, hidden), dtype=torch.float32, device=x.device)
     check(lib().rfq_mlp_swiglu(fmt_gate_up, _ptr(gate_w), _ptr(up_w), gate_w.numel(), fmt_down, _ptr(down_w),
                                down_w.numel(), _ptr(x), _ptr(_f32(norm_weight, "norm_weight")) if norm_weight is not None else None,
@@ -169,12 +193,11 @@ def gemm_f16(fmt: int, w: torch.Tensor, a: torch.Tensor, n: int, k: int, out_dty
              out: torch.Tensor | None = None) -> torch.Tensor:
     """out[m, n] = a[m, k] (fp16) . dequant(W)[n, k]^T on the fp16 matrix cores."""
     w = _dev_u8(w)
-    if a.dtype != torch.float16 or not a.is_contiguous() or a.dim() != 2:
-        raise ValueError("a must be a contiguous [m, k] float16 tensor")
+    if not (a.is_cuda and a.dtype == torch.float16 and a.is_contiguous() and a.dim() == 2 and a.shape[1] == k):
+        raise ValueError(f"a must be a contiguous [m, {k}] float16 device tensor")
     m = a.shape[0]
     code = {torch.float32: _lib.F32, torch.float16: _lib.F16}[out_dtype]
-    if out is None:
-        out = torch.empty((m, n), dtype=out_dtype, device=a.device)
+    out = _out(out, (m, n), out_dtype, a)
     check(lib().rfq_gemm_f16(fmt, _ptr(w), w.numel(), _ptr(a), _ptr(out), code, m, n, k, _stream()))
     return out
 
@@ -188,8 +211,7 @@ def gemm_f16_static(fmt: int, w: torch.Tensor, a: torch.Tensor, n: int, k: int, 
         raise ValueError("a must be a contiguous [m, k] float16 device tensor")
     m = a.shape[0]
     code = {torch.float32: _lib.F32, torch.float16: _lib.F16}[out_dtype]
-    if not (out.is_cuda and out.dtype == out_dtype and out.is_contiguous() and out.numel() == m * n):
-        raise ValueError("out must be a contiguous device tensor of m * n elements of out_dtype")
+    out = _out(out, (m, n), out_dtype, a)
     check(lib().rfq_gemm_f16_static(fmt, _ptr(w), w.numel(), _ptr(a), _ptr(out), code, m, n, k, _stream()))
     return out
 
@@ -214,9 +236,9 @@ def gemm_mx(a: MxOperand, w: MxOperand, out_dtype=torch.bfloat16, out: torch.Ten
     if a.k != w.k:
         raise ValueError("inner dimensions differ")
     code = {torch.float32: _lib.F32, torch.bfloat16: _lib.BF16}[out_dtype]
-    if out is None:
-        out = torch.empty((a.rows, w.rows), dtype=out_dtype, device=a.buf.device)
-    check(lib().rfq_gemm_mx(_ptr(a.buf), a.kind, _ptr(w.buf), w.kind, _ptr(out), code, a.rows, w.rows, a.k, _stream()))
+    out = _out(out, (a.rows, w.rows), out_dtype, a.buf)
+    check(lib().rfq_gemm_mx(_ptr(a.buf), a.buf.numel(), a.kind, _ptr(w.buf), w.buf.numel(), w.kind, _ptr(out), code, a.rows, w.rows,
+                            a.k, _stream()))
     return out
 
 

@@ -120,9 +120,9 @@ extern "C" {
     pub fn rfq_mx_prepare(fmt: c_int, kind_req: c_int, d_raw: *const c_void, raw_bytes: usize, rows: c_int, k: c_int,
                           d_prepared: *mut c_void, prepared_bytes: usize, kind_out: *mut c_int,
                           stream: *mut c_void) -> c_int;
-    pub fn rfq_gemm_mx(d_a_prep: *const c_void, a_kind: c_int, d_w_prep: *const c_void, w_kind: c_int,
-                       d_out: *mut c_void, out_dtype: c_int, m: c_int, n: c_int, k: c_int,
-                       stream: *mut c_void) -> c_int;
+    pub fn rfq_gemm_mx(d_a_prep: *const c_void, a_prep_bytes: usize, a_kind: c_int, d_w_prep: *const c_void,
+                       w_prep_bytes: usize, w_kind: c_int, d_out: *mut c_void, out_dtype: c_int, m: c_int, n: c_int,
+                       k: c_int, stream: *mut c_void) -> c_int;
 }
 
 /// Text of the last failure on this thread (`""` if none).

@@ -60,5 +60,10 @@ def test_validation_needs_no_device():
     assert L.rfq_gemm_f16(12, one, 256, one, one, 2, 1, 1, 256, None) == _lib.E_BADARG  # bf16 out
     assert L.rfq_mx_prepare(12, 0, one, 17, 1, 128, one, 64, None, None) == _lib.E_BADARG
     assert L.rfq_mx_prepare(20, 0, one, 68, 1, 100, one, 64, None, None) == _lib.E_SIZE
-    assert L.rfq_gemm_mx(one, 4, one, 4, one, 1, 32, 32, 128, None) == _lib.E_BADARG     # f16 out
-    assert L.rfq_gemm_mx(one, 5, one, 4, one, 0, 32, 32, 128, None) == _lib.E_BADARG
+    pb = L.rfq_mx_prepared_bytes(20, 4, 32, 128)
+    assert L.rfq_gemm_mx(one, pb, 4, one, pb, 4, one, 1, 32, 32, 128, None) == _lib.E_BADARG     # f16 out
+    assert L.rfq_gemm_mx(one, pb, 5, one, pb, 4, one, 0, 32, 32, 128, None) == _lib.E_BADARG
+    assert L.rfq_gemm_mx(one, pb, 4, one, pb, 4, one, 0, 64, 32, 128, None) == _lib.E_SIZE       # A was prepared for 32 rows
+    assert b"prepared A" in L.rfq_last_error()
+    assert L.rfq_gemm_mx(one, pb, 4, one, pb - 16, 4, one, 0, 32, 32, 128, None) == _lib.E_SIZE
+    assert b"prepared W" in L.rfq_last_error()
