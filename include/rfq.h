@@ -113,10 +113,14 @@ RFQ_API const char *rfq_last_error(void);
  * out during a capture when it grows -- only this function does: it frees
  * every kept buffer (it waits for the device first) and rfq_upload's pinned
  * staging slots, and thereby invalidates graphs captured earlier; the next
- * call allocates again.  Buffers are kept per stream handle: call this after
- * destroying streams that used the library.  No counterpart in the
- * reference, whose kernels take no temporaries. */
+ * call allocates again.  Buffers are kept per stream handle:
+ * rfq_release_stream_temporaries(stream) gives up the one of a stream that is
+ * about to be destroyed (it frees the buffer once the stream's work is done;
+ * a buffer that a capture used stays allocated until rfq_release_temporaries),
+ * so that a later stream with the same handle value does not inherit it.
+ * No counterpart in the reference, whose kernels take no temporaries. */
 RFQ_API int rfq_release_temporaries(void);
+RFQ_API int rfq_release_stream_temporaries(void *stream);
 /* Host bytes (pageable: a slice of the memory-mapped model file) -> device
  * memory, in stream order.  The bytes go through a ring of four pinned 8 MiB
  * slots the library keeps per device: a few host threads fill a slot while the

@@ -57,6 +57,7 @@ _SIGNATURES = {
     "rfq_gemm_f16_static": ([_i, _vp, _sz, _vp, _vp, _i, _i, _i, _i, _vp], _i),
     "rfq_mx_prepared_bytes": ([_i, _i, _i, _i], _sz),
     "rfq_mx_prepare": ([_i, _i, _vp, _sz, _i, _i, _vp, _sz, C.POINTER(C.c_int), _vp], _i),
+    "rfq_release_stream_temporaries": ([_vp], _i),
     "rfq_gemm_mx": ([_vp, _sz, _i, _vp, _sz, _i, _vp, _i, _i, _i, _i, _vp], _i),
     # include/rfq_bench.h
     "rfq_bench_gemv": ([_i, _vp, _i, _sz, _vp, _vp, _i, _i, _i, _i, _i, _vp, C.POINTER(C.c_float)], _i),

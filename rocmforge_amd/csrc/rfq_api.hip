@@ -89,6 +89,8 @@ int rfq_release_temporaries(void)
     return rc != RFQ_OK ? rc : rc2;
 }
 
+int rfq_release_stream_temporaries(void *stream) { return rfq::release_stream_workspace((hipStream_t)stream); }
+
 int rfq_upload(const void *h_src, size_t bytes, void *d_dst, void *stream)
 {
     if (bytes == 0) return RFQ_OK;

@@ -82,6 +82,7 @@ int device_cu_count();
 // stream-ordered allocation the caller releases with hipFreeAsync otherwise.
 int workspace(hipStream_t s, size_t bytes, uint8_t **out, bool *transient);
 int release_workspaces();
+int release_stream_workspace(hipStream_t s);
 // Host bytes -> device memory through the per-device ring of pinned slots (rfq_upload.hip).
 int upload_bytes(const void *h_src, size_t bytes, void *d_dst, hipStream_t s);
 int release_upload_rings();

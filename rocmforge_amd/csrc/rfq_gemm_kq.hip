@@ -1005,6 +1005,30 @@ int workspace(hipStream_t s, size_t bytes, uint8_t **out, bool *transient)
     return RFQ_OK;
 }
 
+// The buffer kept for one stream, before the caller destroys the stream: the handle's entry is erased (a later
+// stream that gets the same handle value starts without a buffer).  A buffer a capture used stays allocated.
+int release_stream_workspace(hipStream_t s)
+{
+    std::lock_guard<std::mutex> lock(ws_mutex);
+    auto it = ws_kept.find(s);
+    if (it == ws_kept.end()) return RFQ_OK;
+    const Kept kept = it->second;
+    ws_kept.erase(it);
+    if (kept.ptr == nullptr) return RFQ_OK;
+    if (kept.captured) {
+        ws_retired.push_back(kept);
+        return RFQ_OK;
+    }
+    int current = 0;
+    RFQ_HIP(hipGetDevice(&current));
+    hipError_t e = hipSetDevice(kept.device);
+    if (e == hipSuccess) e = hipFree(kept.ptr);                                       // (waits for the work that uses it)
+    const hipError_t back = hipSetDevice(current);
+    if (e == hipSuccess) e = back;
+    if (e != hipSuccess) return hip_fail(e, "rfq_release_stream_temporaries");
+    return RFQ_OK;
+}
+
 int release_workspaces()
 {
     std::lock_guard<std::mutex> lock(ws_mutex);

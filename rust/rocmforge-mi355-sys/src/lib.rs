@@ -56,6 +56,7 @@ extern "C" {
     pub fn rfq_version() -> c_int;
     pub fn rfq_last_error() -> *const c_char;
     pub fn rfq_release_temporaries() -> c_int;
+    pub fn rfq_release_stream_temporaries(stream: *mut c_void) -> c_int;
     pub fn rfq_upload(h_src: *const c_void, bytes: usize, d_dst: *mut c_void, stream: *mut c_void) -> c_int;
     pub fn rfq_block_elems(fmt: c_int) -> usize;
     pub fn rfq_block_bytes(fmt: c_int) -> usize;

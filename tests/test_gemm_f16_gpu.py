@@ -143,6 +143,22 @@ def test_weights_at_a_4_byte_offset_and_kept_temporary(oracle, cuda):
     again = ops.gemm_f16(fmt, torch.from_numpy(w).to(cuda), torch.from_numpy(a).to(cuda), 128, 512, out_dtype=torch.float32)
     torch.cuda.synchronize()
     assert np.array_equal(again.cpu().numpy(), outs[0])
+    # a stream gives up its own buffer before it is destroyed; the default stream's stays
+    side = torch.cuda.Stream()
+    wd, ad = torch.from_numpy(w).to(cuda), torch.from_numpy(a).to(cuda)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        on_side = ops.gemm_f16(fmt, wd, ad, 128, 512, out_dtype=torch.float32)
+    side.synchronize()
+    assert np.array_equal(on_side.cpu().numpy(), outs[0])
+    import ctypes as C
+    assert _lib.lib().rfq_release_stream_temporaries(C.c_void_p(side.cuda_stream)) == _lib.OK
+    assert _lib.lib().rfq_release_stream_temporaries(C.c_void_p(side.cuda_stream)) == _lib.OK   # nothing left: still fine
+    with torch.cuda.stream(side):
+        on_side = ops.gemm_f16(fmt, wd, ad, 128, 512, out_dtype=torch.float32)      # allocates again
+    side.synchronize()
+    assert np.array_equal(on_side.cpu().numpy(), outs[0])
+    assert np.array_equal(ops.gemm_f16(fmt, wd, ad, 128, 512, out_dtype=torch.float32).cpu().numpy(), outs[0])
 
 
 def test_temporary_larger_than_the_kept_size(oracle, cuda):
