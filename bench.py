@@ -477,7 +477,10 @@ def main():
                                        ("Q8_0 gemv 4096x4096 m8", Q.Q8_0, 4096, 4096, 8, 20260002),
                                        ("Q4_0 gemv 4864x896", Q.Q4_0, 4864, 896, 1, 20260001),
                                        ("MXFP4 gemv 14336x4096", Q.MXFP4, N, K, 1, 20260041),
-                                       ("MXFP6 gemv 14336x4096", Q.MXFP6_E2M3, N, K, 1, 20260042)):
+                                       ("MXFP6 gemv 14336x4096", Q.MXFP6_E2M3, N, K, 1, 20260042),
+                                       # the matmul module's own decoders (nibble stride 20; bytes as int8)
+                                       ("MM_Q4_K gemv 14336x4096", Q.MM_Q4_K, N, K, 1, 20260043),
+                                       ("MM_Q8_0 gemv 4096x4096 m1", Q.MM_Q8_0, 4096, 4096, 1, 20260044)):
             c = -(-int(2.5 * CACHE_BYTES) // Q.packed_bytes(f, n * k))
             c = min(c, 64)
             _, d, *_ = time_gemv(torch, f, n, k, m, c, 500, 50, Q, seed)

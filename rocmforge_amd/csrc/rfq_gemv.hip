@@ -1025,6 +1025,40 @@ template <> struct IUnit<RFQ_Q8_0> : Unit<RFQ_Q8_0> {
     }
 };
 
+// The matmul module's variants of the two integer formats: the same sums, the f16 scale widened the module's own
+// way (Q4_K), the bytes read as int8 (Q8_0: one XOR per dword makes them the offset-binary bytes of the sum above).
+template <> struct IUnit<RFQ_MM_Q4_K> : Unit<RFQ_MM_Q4_K> {
+    static constexpr bool PAIR = false;
+    static constexpr bool NIBBLE = true;
+    static constexpr uint32_t TOPOFF = 0;
+    __device__ __forceinline__ float idot(const XPrep &xp) const
+    {
+        return __builtin_fmaf(f16_bits_to_f32_mm(sc) * xp.s, nib_idot(q, xp), (float)mn * xp.xsum);
+    }
+};
+
+template <> struct IUnit<RFQ_MM_Q8_0> : Unit<RFQ_MM_Q8_0> {
+    static constexpr bool PAIR = false;
+    static constexpr bool NIBBLE = false;
+    static constexpr uint32_t TOPOFF = 0x400000u;
+    __device__ __forceinline__ float idot(const XPrep &xp) const
+    {
+        uint32_t alo = 0, amid = 0, atop = 0, bsum = 0;
+#pragma unroll
+        for (int g = 0; g < 8; g++) {
+            const uint32_t *L = &xp.l[g * 3];
+            const uint32_t b = q.v[g] ^ 0x80808080u;               // int8 + 128
+            alo = __builtin_amdgcn_udot4(b, L[0], alo, false);
+            amid = __builtin_amdgcn_udot4(b, L[1], amid, false);
+            atop = __builtin_amdgcn_udot4(b, L[2], atop, false);
+            bsum = __builtin_amdgcn_udot4(b, 0x01010101u, bsum, false);
+        }
+        float S = __builtin_fmaf((float)((int)atop - 64 * (int)bsum), 65536.0f,
+                                 __builtin_fmaf((float)amid, 256.0f, (float)alo));
+        return scale * __builtin_fmaf(xp.s, S, -128.0f * xp.xsum);
+    }
+};
+
 // GGUF layouts: x limbs in plain order (group g = elements 4g .. 4g+3).
 
 template <> struct IUnit<RFQ_GGUF_Q4_0> : Unit<RFQ_GGUF_Q4_0> {
@@ -1702,6 +1736,8 @@ template <> struct HasIdot<RFQ_GGUF_Q4_0> { static constexpr bool value = true; 
 template <> struct HasIdot<RFQ_GGUF_Q8_0> { static constexpr bool value = true; };
 template <> struct HasIdot<RFQ_GGUF_Q4_K> { static constexpr bool value = true; };
 template <> struct HasIdot<RFQ_GGUF_Q6_K> { static constexpr bool value = true; };
+template <> struct HasIdot<RFQ_MM_Q4_K> { static constexpr bool value = true; };
+template <> struct HasIdot<RFQ_MM_Q8_0> { static constexpr bool value = true; };
 template <int FMT> struct HasIdotBatch { static constexpr bool value = HasIdot<FMT>::value; };
 
 template <int FMT, int UPL, int WPR, int R, bool FUSE>
@@ -1935,6 +1971,16 @@ int run(const uint8_t *w, const float *x, float *y, int m, int n, int k, hipStre
     return run_generic_m<FMT>(w, x, y, m, n, k, s);
 }
 
+// The matmul module's variants: the decode GEMV (m == 1) through the kernels of their canonical twins, batches
+// and odd shapes through the one-row-per-wavefront kernel.
+template <int FMT>
+int run_mm(const uint8_t *w, const float *x, float *y, int m, int n, int k, hipStream_t s)
+{
+    const int ku = k / 32;
+    if (m == 1 && ku > 16 && ku <= 512) return run_rows<FMT, false>(w, x, y, n, k, GemvFuse{nullptr, nullptr, 0.0f, 0}, s);
+    return run_generic_m<FMT>(w, x, y, m, n, k, s);
+}
+
 } // namespace
 
 int launch_gemv(int fmt, const uint8_t *d_w, const float *d_x, float *d_y, int m, int n, int k, hipStream_t s)
@@ -1950,9 +1996,9 @@ int launch_gemv(int fmt, const uint8_t *d_w, const float *d_x, float *d_y, int m
     case RFQ_GGUF_Q8_0: return run<RFQ_GGUF_Q8_0>(d_w, d_x, d_y, m, n, k, s);
     case RFQ_GGUF_Q4_K: return run<RFQ_GGUF_Q4_K>(d_w, d_x, d_y, m, n, k, s);
     case RFQ_GGUF_Q6_K: return run<RFQ_GGUF_Q6_K>(d_w, d_x, d_y, m, n, k, s);
-    case RFQ_MM_Q8_0: return run_generic_m<RFQ_MM_Q8_0>(d_w, d_x, d_y, m, n, k, s);
-    case RFQ_MM_Q4_K: return run_generic_m<RFQ_MM_Q4_K>(d_w, d_x, d_y, m, n, k, s);
-    case RFQ_MM_Q6_K: return run_generic_m<RFQ_MM_Q6_K>(d_w, d_x, d_y, m, n, k, s);
+    case RFQ_MM_Q8_0: return run_mm<RFQ_MM_Q8_0>(d_w, d_x, d_y, m, n, k, s);
+    case RFQ_MM_Q4_K: return run_mm<RFQ_MM_Q4_K>(d_w, d_x, d_y, m, n, k, s);
+    case RFQ_MM_Q6_K: return run_mm<RFQ_MM_Q6_K>(d_w, d_x, d_y, m, n, k, s);
     default: return fail(RFQ_E_BADARG, "rfq_gemv: unknown format %d", fmt);
     }
 }
