@@ -272,7 +272,7 @@ template <> struct Unit<RFQ_MXFP4> {
         e = (int)(int8_t)p[0];
         q = ld<U4>(p + 1);
     }
-    __device__ __forceinline__ float dot(const float (&x)[32], float) const
+    template <bool CLAMP> __device__ __forceinline__ float dot_as(const float (&x)[32]) const
     {
         // bound on |code value|: 8 / 2^e when e >= 1 (exact, 2^(3-e)), else 8.
         float bound = e >= 1 ? __uint_as_float((uint32_t)(130 - e) << 23) : 8.0f;
@@ -283,13 +283,19 @@ template <> struct Unit<RFQ_MXFP4> {
 #pragma unroll
             for (int b = 0; b < 4; b++) {
                 const float2 v = lut[(q.v[d] >> (8 * b)) & 255u];                // element 2j = high nibble
-                const float hi = __builtin_amdgcn_fmed3f(v.x, -bound, bound);
-                const float lo = __builtin_amdgcn_fmed3f(v.y, -bound, bound);
+                const float hi = CLAMP ? __builtin_amdgcn_fmed3f(v.x, -bound, bound) : v.x;
+                const float lo = CLAMP ? __builtin_amdgcn_fmed3f(v.y, -bound, bound) : v.y;
                 s0 = __builtin_fmaf(hi, x[8 * d + 2 * b], s0);
                 s1 = __builtin_fmaf(lo, x[8 * d + 2 * b + 1], s1);
             }
         }
         return mx_scale(e) * (s0 + s1);
+    }
+    __device__ __forceinline__ float dot(const float (&x)[32], float) const
+    {
+        // (the clamp only bites for exponents >= 1, which weights below 1 never have: a wavefront without such a
+        // unit skips the 32 clamps)
+        return __builtin_amdgcn_ballot_w64(e >= 1) != 0 ? dot_as<true>(x) : dot_as<false>(x);
     }
 };
 
@@ -302,7 +308,7 @@ template <> struct Unit<RFQ_MXFP6_E2M3> {
         e = (int)(int8_t)p[0];
         q = ld<U6>(p + 1);
     }
-    __device__ __forceinline__ float dot(const float (&x)[32], float) const
+    template <bool CLAMP> __device__ __forceinline__ float dot_as(const float (&x)[32]) const
     {
         // 7.5 * 2^-e for e >= 1: 7.5 = 0x40F00000 (biased exponent 129).
         float bound = e >= 1 ? __uint_as_float(0x40F00000u - ((uint32_t)e << 23)) : 7.5f;
@@ -319,18 +325,25 @@ template <> struct Unit<RFQ_MXFP6_E2M3> {
             float v0 = lut[b1 >> 2];
             float v1 = lut[(b0 >> 4) | ((b1 & 3u) << 4)];
             float v2 = lut[(b1 >> 6) | ((b2 & 15u) << 2)];
-            v0 = __builtin_amdgcn_fmed3f(v0, -bound, bound);
-            v1 = __builtin_amdgcn_fmed3f(v1, -bound, bound);
-            v2 = __builtin_amdgcn_fmed3f(v2, -bound, bound);
+            if (CLAMP) {
+                v0 = __builtin_amdgcn_fmed3f(v0, -bound, bound);
+                v1 = __builtin_amdgcn_fmed3f(v1, -bound, bound);
+                v2 = __builtin_amdgcn_fmed3f(v2, -bound, bound);
+            }
             s0 = __builtin_fmaf(v0, x[4 * j], s0);
             s1 = __builtin_fmaf(v1, x[4 * j + 1], s1);
             s0 = __builtin_fmaf(v2, x[4 * j + 2], s0);
             if (j < 7) { // element 31 is never written by the reference: weight 0
-                float v3 = __builtin_amdgcn_fmed3f(lut[b3 & 63u], -bound, bound);
+                float v3 = lut[b3 & 63u];
+                if (CLAMP) v3 = __builtin_amdgcn_fmed3f(v3, -bound, bound);
                 s1 = __builtin_fmaf(v3, x[4 * j + 3], s1);
             }
         }
         return mx_scale(e) * (s0 + s1);
+    }
+    __device__ __forceinline__ float dot(const float (&x)[32], float) const
+    {
+        return __builtin_amdgcn_ballot_w64(e >= 1) != 0 ? dot_as<true>(x) : dot_as<false>(x);
     }
 };
 
