@@ -368,6 +368,7 @@ def main():
     ap.add_argument("--mlp-steps", type=int, default=300)
     ap.add_argument("--only-gguf", action="store_true", help="only the GGUF-layout Q4_K GEMV line (profiling runs)")
     ap.add_argument("--only-dequant", action="store_true", help="only the dequantisation lines (profiling runs)")
+    ap.add_argument("--only-gemv", metavar="FMT:NxK:M", help="only one decode GEMV, e.g. MXFP4:14336x4096:1 (profiling runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build is single-GPU (one MI355X per box); run with --gpus 1. "
@@ -394,6 +395,21 @@ def main():
             res[name] = {"GB/s": round(b / t / 1e9, 1), "us": round(t * 1e6, 2), "hbm_frac": round(b / t / 1e9 / HBM_PEAK_GBS, 4),
                          "algorithmic_bytes": b}
         print(json.dumps(res))
+        return
+
+    if args.only_gemv:
+        name, shape, mm = args.only_gemv.split(":")
+        f = {v: k_ for k_, v in Q.NAMES.items()}[name]
+        n_, k_ = (int(t) for t in shape.split("x"))
+        m_ = int(mm)
+        c = min(-(-int(2.5 * CACHE_BYTES) // Q.packed_bytes(f, n_ * k_)), 64)
+        _, d, *_ = time_gemv(torch, f, n_, k_, m_, c, args.steps, args.warmup, Q, 20260060)
+        b = algorithmic_bytes(f, n_, k_, m_, Q)
+        from rocmforge_amd import _lib
+        print(json.dumps({f"{name} gemv {n_}x{k_} m{m_}": {
+            "GB/s": round(b / (d / args.steps) / 1e9, 1), "us": round(d / args.steps * 1e6, 2),
+            "hbm_frac": round(b / (d / args.steps) / 1e9 / HBM_PEAK_GBS, 4), "algorithmic_bytes": b, "weight_copies": c,
+            "kernel": _lib.lib().rfq_bench_last_gemv_kernel().decode()}}))
         return
 
     if args.only_gguf:
