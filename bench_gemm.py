@@ -87,7 +87,7 @@ def mx_gemm(torch, w_fmt, m=2048, n=28672, k=8192, steps=200, warmup=40, data="p
     return res
 
 
-def kq_gemm(torch, fmt, m=512, n=14336, k=4096, steps=300, warmup=300):
+def kq_gemm(torch, fmt, m=512, n=14336, k=4096, steps=300, warmup=300, arranged=False):
     """Q4_K / Q6_K prefill GEMM on the fp16 matrix cores, fp16 in and out."""
     from rocmforge_amd import _lib, quantize as Q
     dev = torch.device("cuda:0")
@@ -102,14 +102,25 @@ def kq_gemm(torch, fmt, m=512, n=14336, k=4096, steps=300, warmup=300):
     _lib.check(L.rfq_bench_gemm_f16(*args, warmup, steps, stream, C.byref(ms)))
     t = ms.value / 1e3 / steps
     flops = 2.0 * m * n * k
-    return {"TFLOP/s": round(flops / t / 1e12, 1), "us": round(t * 1e6, 1), "mfma_frac": round(flops / t / 2.5e15, 4),
-            "peak_TFLOP/s": 2500.0, "warmup_launches": warmup, "timed_launches": steps}
+    res = {"TFLOP/s": round(flops / t / 1e12, 1), "us": round(t * 1e6, 1), "mfma_frac": round(flops / t / 2.5e15, 4),
+           "peak_TFLOP/s": 2500.0, "warmup_launches": warmup, "timed_launches": steps}
+    if arranged:
+        # the same GEMM on activations arranged once (the second and third projection of one input)
+        from rocmforge_amd import ops
+        A = ops.ArrangedA(a)
+        _lib.check(L.rfq_bench_gemm_f16_arranged(fmt, C.c_void_p(w.data_ptr()), w.numel(), C.c_void_p(A.buf.data_ptr()), A.buf.numel(),
+                                                 C.c_void_p(out.data_ptr()), _lib.F16, m, n, k, warmup, steps, stream, C.byref(ms)))
+        ta = ms.value / 1e3 / steps
+        res["activations_arranged_once"] = {"us": round(ta * 1e6, 1), "TFLOP/s": round(flops / ta / 1e12, 1),
+                                            "mfma_frac": round(flops / ta / 2.5e15, 4),
+                                            "what": "rfq_gemm_f16_arranged per step, rfq_gemm_f16_arrange before the loop"}
+    return res
 
 
 def run(torch):
     from rocmforge_amd import quantize as Q
     res = {}
-    res["Q4_K gemm 512x4096x14336 fp16"] = kq_gemm(torch, Q.Q4_K)
+    res["Q4_K gemm 512x4096x14336 fp16"] = kq_gemm(torch, Q.Q4_K, arranged=True)
     res["Q6_K gemm 512x4096x14336 fp16"] = kq_gemm(torch, Q.Q6_K)
     res["GGUF_Q4_K gemm 512x4096x14336 fp16"] = kq_gemm(torch, Q.GGUF_Q4_K)
     res["GGUF_Q6_K gemm 512x4096x14336 fp16"] = kq_gemm(torch, Q.GGUF_Q6_K)
@@ -131,7 +142,7 @@ if __name__ == "__main__":
     import torch
     from rocmforge_amd import quantize as Q
     if a.only in ("q4_k", "gguf_q4_k"):
-        print(json.dumps(kq_gemm(torch, Q.Q4_K if a.only == "q4_k" else Q.GGUF_Q4_K, steps=a.steps)))
+        print(json.dumps(kq_gemm(torch, Q.Q4_K if a.only == "q4_k" else Q.GGUF_Q4_K, steps=a.steps, arranged=True)))
     elif a.only:
         print(json.dumps(mx_gemm(torch, Q.MXFP4 if a.only == "mxfp4" else Q.MXFP6_E2M3, steps=a.steps, data=a.data)))
     else:

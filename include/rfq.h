@@ -333,6 +333,25 @@ RFQ_API int rfq_gemm_f16(int fmt, const void *d_w, size_t w_bytes, const void *d
 RFQ_API int rfq_gemm_f16_static(int fmt, const void *d_w, size_t w_bytes, const void *d_a_f16, void *d_out,
                                 int out_dtype, int m, int n, int k, void *stream);
 
+/* The same GEMM with the re-ordering of the activations taken out of the call,
+ * for several projections of one input (the Q, K and V weights of a layer,
+ * gate and up): rfq_gemm_f16_arrange writes A[m, k] (fp16, 16-byte aligned, k a
+ * multiple of 8) once, in matrix-operand order plus the per-group sums the
+ * RFQ_Q4_K kernel wants, into a caller's buffer of
+ * rfq_gemm_f16_arranged_bytes(m, k) bytes (16-byte aligned; 0 = bad shape);
+ * rfq_gemm_f16_arranged multiplies any of the formats of rfq_gemm_f16 with it.
+ * Results are bit-identical to rfq_gemm_f16 on the same A.  Neither call
+ * allocates or keeps anything, so both may be recorded under stream capture.
+ * The reference has no fused prefill GEMM (see rfq_gemm_f16); its
+ * counterpart is the shared input of the three SGEMMs of
+ * HipBackend::mlp_swiglu (src/backend/hip_backend/backend.rs:1153-1278). */
+RFQ_API size_t rfq_gemm_f16_arranged_bytes(int m, int k);
+RFQ_API int rfq_gemm_f16_arrange(const void *d_a_f16, int m, int k, void *d_arranged, size_t arranged_bytes,
+                                 void *stream);
+RFQ_API int rfq_gemm_f16_arranged(int fmt, const void *d_w, size_t w_bytes, const void *d_arranged,
+                                  size_t arranged_bytes, void *d_out, int out_dtype, int m, int n, int k,
+                                  void *stream);
+
 /* MXFP matrices feed the gfx950 block-scaled matrix instruction, whose element
  * and scale encodings differ from the bytes ROCmForge stores (signed exponent
  * byte, its own E2M1/E2M3 value tables, a +-8 / +-7.5 clamp).  A matrix

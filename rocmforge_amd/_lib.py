@@ -58,6 +58,9 @@ _SIGNATURES = {
     "rfq_mx_prepared_bytes": ([_i, _i, _i, _i], _sz),
     "rfq_mx_prepare": ([_i, _i, _vp, _sz, _i, _i, _vp, _sz, C.POINTER(C.c_int), _vp], _i),
     "rfq_release_stream_temporaries": ([_vp], _i),
+    "rfq_gemm_f16_arranged_bytes": ([_i, _i], _sz),
+    "rfq_gemm_f16_arrange": ([_vp, _i, _i, _vp, _sz, _vp], _i),
+    "rfq_gemm_f16_arranged": ([_i, _vp, _sz, _vp, _sz, _vp, _i, _i, _i, _i, _vp], _i),
     "rfq_gemm_mx": ([_vp, _sz, _i, _vp, _sz, _i, _vp, _i, _i, _i, _i, _vp], _i),
     # include/rfq_bench.h
     "rfq_bench_gemv": ([_i, _vp, _i, _sz, _vp, _vp, _i, _i, _i, _i, _i, _vp, C.POINTER(C.c_float)], _i),
@@ -68,6 +71,7 @@ _SIGNATURES = {
     "rfq_bench_last_gemv_kernel": ([], C.c_char_p),
     "rfq_bench_read_floor": ([_vp, _i, _sz, _i, _i, _i, _i, _i, _i, _vp, C.POINTER(C.c_float)], _i),
     "rfq_bench_gemm_mx_prefill": ([_vp, _sz, _vp, _sz, _vp, _sz, _i, _vp, _i, _i, _i, _i, _i, _i, _vp, C.POINTER(C.c_float)], _i),
+    "rfq_bench_gemm_f16_arranged": ([_i, _vp, _sz, _vp, _sz, _vp, _i, _i, _i, _i, _i, _i, _vp, C.POINTER(C.c_float)], _i),
     "rfq_bench_gemm_mx": ([_vp, _sz, _i, _vp, _sz, _i, _vp, _i, _i, _i, _i, _i, _i, _vp, C.POINTER(C.c_float)], _i),
 }
 

@@ -417,7 +417,7 @@ int rfq_gemm_f16(int fmt, const void *d_w, size_t w_bytes, const void *d_a_f16, 
     if (rc != RFQ_OK) return rc;
     if (out_dtype != RFQ_F32 && out_dtype != RFQ_F16)
         return fail(RFQ_E_BADARG, "rfq_gemm_f16: out_dtype %d is neither F32 nor F16", out_dtype);
-    return launch_gemm_f16(fmt, (const uint8_t *)d_w, d_a_f16, d_out, out_dtype, m, n, k, false, (hipStream_t)stream);
+    return launch_gemm_f16(fmt, (const uint8_t *)d_w, d_a_f16, d_out, out_dtype, m, n, k, false, nullptr, (hipStream_t)stream);
 }
 
 int rfq_gemm_f16_static(int fmt, const void *d_w, size_t w_bytes, const void *d_a_f16, void *d_out, int out_dtype, int m,
@@ -427,7 +427,35 @@ int rfq_gemm_f16_static(int fmt, const void *d_w, size_t w_bytes, const void *d_
     if (rc != RFQ_OK) return rc;
     if (out_dtype != RFQ_F32 && out_dtype != RFQ_F16)
         return fail(RFQ_E_BADARG, "rfq_gemm_f16_static: out_dtype %d is neither F32 nor F16", out_dtype);
-    return launch_gemm_f16(fmt, (const uint8_t *)d_w, d_a_f16, d_out, out_dtype, m, n, k, true, (hipStream_t)stream);
+    return launch_gemm_f16(fmt, (const uint8_t *)d_w, d_a_f16, d_out, out_dtype, m, n, k, true, nullptr, (hipStream_t)stream);
+}
+
+size_t rfq_gemm_f16_arranged_bytes(int m, int k) { return gemm_f16_arranged_bytes(m, k); }
+
+int rfq_gemm_f16_arrange(const void *d_a_f16, int m, int k, void *d_arranged, size_t arranged_bytes, void *stream)
+{
+    if (!d_a_f16 || !d_arranged) return fail(RFQ_E_BADARG, "rfq_gemm_f16_arrange: null pointer");
+    if (m <= 0 || k <= 0) return fail(RFQ_E_BADARG, "rfq_gemm_f16_arrange: bad shape m=%d k=%d", m, k);
+    const size_t need = gemm_f16_arranged_bytes(m, k);
+    if (need == 0) return fail(RFQ_E_SIZE, "rfq_gemm_f16_arrange: k=%d is not a multiple of 8", k);
+    if (arranged_bytes < need)
+        return fail(RFQ_E_SIZE, "rfq_gemm_f16_arrange: the buffer has %zu bytes, [%d x %d] needs %zu", arranged_bytes, m, k, need);
+    return launch_arrange_a(d_a_f16, m, k, (uint8_t *)d_arranged, (hipStream_t)stream);
+}
+
+int rfq_gemm_f16_arranged(int fmt, const void *d_w, size_t w_bytes, const void *d_arranged, size_t arranged_bytes,
+                          void *d_out, int out_dtype, int m, int n, int k, void *stream)
+{
+    int rc = check_gemv("rfq_gemm_f16_arranged", fmt, d_w, w_bytes, true, d_arranged, d_out, m, n, k);
+    if (rc != RFQ_OK) return rc;
+    if (out_dtype != RFQ_F32 && out_dtype != RFQ_F16)
+        return fail(RFQ_E_BADARG, "rfq_gemm_f16_arranged: out_dtype %d is neither F32 nor F16", out_dtype);
+    const size_t need = gemm_f16_arranged_bytes(m, k);
+    if (need == 0 || arranged_bytes < need)
+        return fail(RFQ_E_SIZE, "rfq_gemm_f16_arranged: the arranged activations have %zu bytes, [%d x %d] needs %zu",
+                    arranged_bytes, m, k, need);
+    return launch_gemm_f16(fmt, (const uint8_t *)d_w, nullptr, d_out, out_dtype, m, n, k, false, (const uint8_t *)d_arranged,
+                           (hipStream_t)stream);
 }
 
 size_t rfq_mx_prepared_bytes(int fmt, int kind, int rows, int k)

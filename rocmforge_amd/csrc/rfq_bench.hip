@@ -115,6 +115,15 @@ int rfq_bench_gemm_f16(int fmt, const void *d_w, size_t w_bytes, const void *d_a
     });
 }
 
+int rfq_bench_gemm_f16_arranged(int fmt, const void *d_w, size_t w_bytes, const void *d_arranged, size_t arranged_bytes,
+                                void *d_out, int out_dtype, int m, int n, int k, int warmup, int steps, void *stream,
+                                float *elapsed_ms)
+{
+    return timed_loop(warmup, steps, stream, elapsed_ms, [&](int) {
+        return rfq_gemm_f16_arranged(fmt, d_w, w_bytes, d_arranged, arranged_bytes, d_out, out_dtype, m, n, k, stream);
+    });
+}
+
 int rfq_bench_gemm_mx(const void *d_a_prep, size_t a_prep_bytes, int a_kind, const void *d_w_prep, size_t w_prep_bytes,
                       int w_kind, void *d_out, int out_dtype, int m, int n, int k, int warmup, int steps, void *stream,
                       float *elapsed_ms)

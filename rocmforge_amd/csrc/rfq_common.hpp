@@ -101,8 +101,11 @@ int launch_gemv_kn(int fmt, const uint8_t *d_w, const float *d_x, float *d_y, in
 int launch_gemv_fused(int fmt, const uint8_t *d_w, const uint8_t *d_w2, const float *d_x, const float *d_norm_w,
                       float eps, float *d_y, int n, int k, hipStream_t s);
 // use_static_scratch: the temporaries live in the library's static device array instead of workspace().
+size_t gemm_f16_arranged_bytes(int m, int k);
+int launch_arrange_a(const void *d_a, int m, int k, uint8_t *d_arranged, hipStream_t s);
+// d_arranged != nullptr: activations already in operand order (launch_arrange_a); d_a is not read.
 int launch_gemm_f16(int fmt, const uint8_t *d_w, const void *d_a, void *d_out, int out_dtype, int m, int n,
-                    int k, bool use_static_scratch, hipStream_t s);
+                    int k, bool use_static_scratch, const uint8_t *d_arranged, hipStream_t s);
 size_t mx_prepared_bytes(int fmt, int kind, int rows, int k);
 int launch_mx_prepare(int fmt, int kind_req, const uint8_t *d_raw, int rows, int k, void *d_prep,
                       size_t prep_bytes, int *kind_out, hipStream_t s);

@@ -883,8 +883,15 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
         }
 }
 
+// Bytes of the arranged activations of an [m, k] matrix, and of the group sums that follow them when k is whole
+// super-blocks (the Q4_K kernel reads them; the others ignore them).
+size_t arranged_at_bytes(int m, int k) { return (size_t)((m + 31) / 32) * ((k + BK - 1) / BK) * 4096; }
+size_t arranged_s2_bytes(int m, int k) { return k % 256 == 0 ? (size_t)((m + 31) / 32) * (k / 256) * 1024 : 0; }
+
+// `arranged` != nullptr: the caller's buffer from launch_arrange_a (activations and sums); a is not read.
 template <int FMT, bool OUT_F16>
-int launch_cfg(const uint8_t *w, const void *a, void *out, int m, int n, int k, uint8_t *static_tmp, hipStream_t s)
+int launch_cfg(const uint8_t *w, const void *a, void *out, int m, int n, int k, uint8_t *static_tmp, const uint8_t *arranged,
+               hipStream_t s)
 {
     constexpr int LDS = 4 * W_BYTES + BN * 48;                  // four weight stages + the Q4_K min fragment
     static_assert(LDS <= 160 * 1024, "LDS budget");
@@ -896,6 +903,13 @@ int launch_cfg(const uint8_t *w, const void *a, void *out, int m, int n, int k, 
     });
     if (attr_err != hipSuccess) return hip_fail(attr_err, "hipFuncSetAttribute(gemm_kq_kernel)");
     const int tiles = ((m + BM - 1) / BM) * ((n + BN - 1) / BN);
+    if (arranged != nullptr) {
+        const v4u *at = reinterpret_cast<const v4u *>(arranged);
+        const _Float16 *s2 = reinterpret_cast<const _Float16 *>(arranged + arranged_at_bytes(m, k));
+        hipLaunchKernelGGL((gemm_kq_kernel<FMT, OUT_F16>), dim3(tiles), dim3(256), LDS, s, w, at, s2, out, m, n, k);
+        RFQ_LAUNCH_CHECK("gemm_kq_kernel");
+        return RFQ_OK;
+    }
     // the temporary: the arranged activations, then the Q4_K group sums
     const int tiles32 = (m + 31) / 32, nst = (k + BK - 1) / BK;
     const size_t at_bytes = (size_t)tiles32 * nst * 4096;
@@ -925,10 +939,10 @@ int launch_cfg(const uint8_t *w, const void *a, void *out, int m, int n, int k, 
 
 template <int FMT>
 int launch_fmt(const uint8_t *w, const void *a, void *out, int out_dtype, int m, int n, int k, uint8_t *static_tmp,
-               hipStream_t s)
+               const uint8_t *arranged, hipStream_t s)
 {
-    return out_dtype == RFQ_F16 ? launch_cfg<FMT, true>(w, a, out, m, n, k, static_tmp, s)
-                                : launch_cfg<FMT, false>(w, a, out, m, n, k, static_tmp, s);
+    return out_dtype == RFQ_F16 ? launch_cfg<FMT, true>(w, a, out, m, n, k, static_tmp, arranged, s)
+                                : launch_cfg<FMT, false>(w, a, out, m, n, k, static_tmp, arranged, s);
 }
 
 // The address of this device's copy of `scratch`, resolved on the first call on each device.
@@ -1052,8 +1066,32 @@ int release_workspaces()
     return RFQ_OK;
 }
 
+size_t gemm_f16_arranged_bytes(int m, int k)
+{
+    if (m <= 0 || k <= 0 || k % 8 != 0) return 0;
+    return arranged_at_bytes(m, k) + arranged_s2_bytes(m, k);
+}
+
+int launch_arrange_a(const void *d_a, int m, int k, uint8_t *d_arranged, hipStream_t s)
+{
+    if ((reinterpret_cast<uintptr_t>(d_a) & 15u) != 0 || k % 8 != 0)
+        return fail(RFQ_E_BADARG, "rfq_gemm_f16_arrange: activations must be 16-byte aligned with k a multiple of 8");
+    if ((reinterpret_cast<uintptr_t>(d_arranged) & 15u) != 0)
+        return fail(RFQ_E_BADARG, "rfq_gemm_f16_arrange: the arranged buffer must be 16-byte aligned");
+    const int tiles32 = (m + 31) / 32, nst = (k + BK - 1) / BK;
+    v4u *at = reinterpret_cast<v4u *>(d_arranged);
+    _Float16 *s2 = reinterpret_cast<_Float16 *>(d_arranged + arranged_at_bytes(m, k));
+    const dim3 grid((unsigned)(tiles32 * ((nst + 3) / 4)));
+    if (k % 256 == 0)
+        hipLaunchKernelGGL((arrange_a_kernel<true>), grid, dim3(256), 0, s, reinterpret_cast<const _Float16 *>(d_a), at, s2, m, k, tiles32, nst);
+    else
+        hipLaunchKernelGGL((arrange_a_kernel<false>), grid, dim3(256), 0, s, reinterpret_cast<const _Float16 *>(d_a), at, s2, m, k, tiles32, nst);
+    RFQ_LAUNCH_CHECK("arrange_a_kernel");
+    return RFQ_OK;
+}
+
 int launch_gemm_f16(int fmt, const uint8_t *d_w, const void *d_a, void *d_out, int out_dtype, int m, int n, int k,
-                    bool use_static_scratch, hipStream_t s)
+                    bool use_static_scratch, const uint8_t *d_arranged, hipStream_t s)
 {
     uint8_t *st = nullptr;
     if (use_static_scratch) {
@@ -1061,19 +1099,22 @@ int launch_gemm_f16(int fmt, const uint8_t *d_w, const void *d_a, void *d_out, i
     }
     if (out_dtype != RFQ_F16 && out_dtype != RFQ_F32)
         return fail(RFQ_E_BADARG, "rfq_gemm_f16: out_dtype %d (want RFQ_F32 or RFQ_F16)", out_dtype);
-    if ((reinterpret_cast<uintptr_t>(d_a) & 15u) != 0 || k % 8 != 0)
+    if (d_arranged != nullptr) {
+        if ((reinterpret_cast<uintptr_t>(d_arranged) & 15u) != 0 || k % 8 != 0)
+            return fail(RFQ_E_BADARG, "rfq_gemm_f16_arranged: the arranged buffer must be 16-byte aligned with k a multiple of 8");
+    } else if ((reinterpret_cast<uintptr_t>(d_a) & 15u) != 0 || k % 8 != 0)
         return fail(RFQ_E_BADARG, "rfq_gemm_f16: activations must be 16-byte aligned with k a multiple of 8");
     if ((reinterpret_cast<uintptr_t>(d_w) & 3u) != 0)               // buffer loads of whole dwords
         return fail(RFQ_E_BADARG, "rfq_gemm_f16: weights must be 4-byte aligned");
     switch (fmt) {
-    case RFQ_Q4_0: return launch_fmt<RFQ_Q4_0>(d_w, d_a, d_out, out_dtype, m, n, k, st, s);
-    case RFQ_Q8_0: return launch_fmt<RFQ_Q8_0>(d_w, d_a, d_out, out_dtype, m, n, k, st, s);
-    case RFQ_Q4_K: return launch_fmt<RFQ_Q4_K>(d_w, d_a, d_out, out_dtype, m, n, k, st, s);
-    case RFQ_Q6_K: return launch_fmt<RFQ_Q6_K>(d_w, d_a, d_out, out_dtype, m, n, k, st, s);
-    case RFQ_GGUF_Q4_0: return launch_fmt<RFQ_GGUF_Q4_0>(d_w, d_a, d_out, out_dtype, m, n, k, st, s);
-    case RFQ_GGUF_Q8_0: return launch_fmt<RFQ_GGUF_Q8_0>(d_w, d_a, d_out, out_dtype, m, n, k, st, s);
-    case RFQ_GGUF_Q4_K: return launch_fmt<RFQ_GGUF_Q4_K>(d_w, d_a, d_out, out_dtype, m, n, k, st, s);
-    case RFQ_GGUF_Q6_K: return launch_fmt<RFQ_GGUF_Q6_K>(d_w, d_a, d_out, out_dtype, m, n, k, st, s);
+    case RFQ_Q4_0: return launch_fmt<RFQ_Q4_0>(d_w, d_a, d_out, out_dtype, m, n, k, st, d_arranged, s);
+    case RFQ_Q8_0: return launch_fmt<RFQ_Q8_0>(d_w, d_a, d_out, out_dtype, m, n, k, st, d_arranged, s);
+    case RFQ_Q4_K: return launch_fmt<RFQ_Q4_K>(d_w, d_a, d_out, out_dtype, m, n, k, st, d_arranged, s);
+    case RFQ_Q6_K: return launch_fmt<RFQ_Q6_K>(d_w, d_a, d_out, out_dtype, m, n, k, st, d_arranged, s);
+    case RFQ_GGUF_Q4_0: return launch_fmt<RFQ_GGUF_Q4_0>(d_w, d_a, d_out, out_dtype, m, n, k, st, d_arranged, s);
+    case RFQ_GGUF_Q8_0: return launch_fmt<RFQ_GGUF_Q8_0>(d_w, d_a, d_out, out_dtype, m, n, k, st, d_arranged, s);
+    case RFQ_GGUF_Q4_K: return launch_fmt<RFQ_GGUF_Q4_K>(d_w, d_a, d_out, out_dtype, m, n, k, st, d_arranged, s);
+    case RFQ_GGUF_Q6_K: return launch_fmt<RFQ_GGUF_Q6_K>(d_w, d_a, d_out, out_dtype, m, n, k, st, d_arranged, s);
     default: return fail(RFQ_E_UNSUPPORTED, "rfq_gemm_f16: no fp16 matrix-core kernel for format %d", fmt);
     }
 }

@@ -216,6 +216,31 @@ def gemm_f16_static(fmt: int, w: torch.Tensor, a: torch.Tensor, n: int, k: int, 
     return out
 
 
+class ArrangedA:
+    """Activations a[m, k] (fp16) in matrix-operand order, written once for several gemm_f16_arranged calls."""
+
+    def __init__(self, a: torch.Tensor):
+        if not (a.is_cuda and a.dtype == torch.float16 and a.is_contiguous() and a.dim() == 2):
+            raise ValueError("a must be a contiguous [m, k] float16 device tensor")
+        self.m, self.k = a.shape
+        nbytes = lib().rfq_gemm_f16_arranged_bytes(self.m, self.k)
+        if nbytes == 0:
+            raise ValueError(f"cannot arrange activations of shape {tuple(a.shape)} (k must be a multiple of 8)")
+        self.buf = torch.empty(nbytes, dtype=torch.uint8, device=a.device)
+        check(lib().rfq_gemm_f16_arrange(_ptr(a), self.m, self.k, _ptr(self.buf), nbytes, _stream()))
+
+
+def gemm_f16_arranged(fmt: int, w: torch.Tensor, a: ArrangedA, n: int, out_dtype=torch.float16,
+                      out: torch.Tensor | None = None) -> torch.Tensor:
+    """out[m, n] = a . dequant(W)[n, k]^T with activations arranged beforehand (bit-identical to gemm_f16)."""
+    w = _dev_u8(w)
+    code = {torch.float32: _lib.F32, torch.float16: _lib.F16}[out_dtype]
+    out = _out(out, (a.m, n), out_dtype, a.buf)
+    check(lib().rfq_gemm_f16_arranged(fmt, _ptr(w), w.numel(), _ptr(a.buf), a.buf.numel(), _ptr(out), code, a.m, n, a.k,
+                                      _stream()))
+    return out
+
+
 class MxOperand:
     """A [rows, k] MXFP matrix re-encoded for the block-scaled matrix core."""
 

@@ -117,6 +117,12 @@ extern "C" {
     pub fn rfq_gemm_f16_static(fmt: c_int, d_w: *const c_void, w_bytes: usize, d_a_f16: *const c_void,
                                d_out: *mut c_void, out_dtype: c_int, m: c_int, n: c_int, k: c_int,
                                stream: *mut c_void) -> c_int;
+    pub fn rfq_gemm_f16_arranged_bytes(m: c_int, k: c_int) -> usize;
+    pub fn rfq_gemm_f16_arrange(d_a_f16: *const c_void, m: c_int, k: c_int, d_arranged: *mut c_void,
+                                arranged_bytes: usize, stream: *mut c_void) -> c_int;
+    pub fn rfq_gemm_f16_arranged(fmt: c_int, d_w: *const c_void, w_bytes: usize, d_arranged: *const c_void,
+                                 arranged_bytes: usize, d_out: *mut c_void, out_dtype: c_int, m: c_int, n: c_int,
+                                 k: c_int, stream: *mut c_void) -> c_int;
     pub fn rfq_mx_prepared_bytes(fmt: c_int, kind: c_int, rows: c_int, k: c_int) -> usize;
     pub fn rfq_mx_prepare(fmt: c_int, kind_req: c_int, d_raw: *const c_void, raw_bytes: usize, rows: c_int, k: c_int,
                           d_prepared: *mut c_void, prepared_bytes: usize, kind_out: *mut c_int,

@@ -199,3 +199,57 @@ def test_gguf_blocks_at_a_2_byte_phase(fmt, oracle, cuda):
     w, a = weights(fmt, n, k, 41), acts(m, k, 42)
     out = run(fmt, w, a, n, k, cuda, torch.float32).cpu().numpy()
     assert_close(out, oracle.qmatmul_nk(fmt, w, a.astype(np.float32), m, n, k), f"{Q.NAMES[fmt]} odd block count")
+
+
+# Activations arranged once for several projections: the same kernels, bit-identical results; nothing is
+# allocated or kept, so the pair may be recorded into a graph without a call beforehand.
+@pytest.mark.parametrize("fmt", [Q.Q4_0, Q.Q8_0, Q.Q4_K, Q.Q6_K, Q.GGUF_Q4_K, Q.GGUF_Q6_K])
+@pytest.mark.parametrize("m,n,k", [(64, 128, 512), (300, 259, 768), (33, 130, 1024), (512, 256, 4096)])
+def test_arranged_activations_give_the_same_bits(fmt, m, n, k, cuda):
+    import torch
+    from rocmforge_amd import ops
+    w = torch.from_numpy(weights(fmt, n, k, 31)).to(cuda)
+    a = torch.from_numpy(acts(m, k, 32)).to(cuda)
+    A = ops.ArrangedA(a)
+    for dt in (torch.float32, torch.float16):
+        want = ops.gemm_f16(fmt, w, a, n, k, out_dtype=dt)
+        got = ops.gemm_f16_arranged(fmt, w, A, n, out_dtype=dt)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), f"{Q.NAMES[fmt]} {m}x{n}x{k} {dt}"
+    w2 = torch.from_numpy(weights(fmt, n, k, 33)).to(cuda)                  # a second projection of the same input
+    assert torch.equal(ops.gemm_f16_arranged(fmt, w2, A, n), ops.gemm_f16(fmt, w2, a, n, k))
+
+
+def test_arranged_activations_in_a_graph_and_bad_sizes(cuda):
+    import ctypes as C
+    import torch
+    from rocmforge_amd import _lib, ops
+    fmt, m, n, k = Q.Q4_K, 96, 256, 1024
+    w = torch.from_numpy(weights(fmt, n, k, 41)).to(cuda)
+    a = torch.from_numpy(acts(m, k, 42)).to(cuda)
+    want = ops.gemm_f16(fmt, w, a, n, k)
+    L = _lib.lib()
+    nbytes = L.rfq_gemm_f16_arranged_bytes(m, k)
+    assert nbytes == 3 * 16 * 4096 + 3 * 4 * 1024 and L.rfq_gemm_f16_arranged_bytes(m, 1020) == 0
+    buf = torch.empty(nbytes, dtype=torch.uint8, device=cuda)
+    out = torch.empty((m, n), dtype=torch.float16, device=cuda)
+    side = torch.cuda.Stream()                                              # a stream the library has never seen
+    side.wait_stream(torch.cuda.current_stream())
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=side):
+        s = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+        _lib.check(L.rfq_gemm_f16_arrange(C.c_void_p(a.data_ptr()), m, k, C.c_void_p(buf.data_ptr()), nbytes, s))
+        _lib.check(L.rfq_gemm_f16_arranged(fmt, C.c_void_p(w.data_ptr()), w.numel(), C.c_void_p(buf.data_ptr()), nbytes,
+                                           C.c_void_p(out.data_ptr()), _lib.F16, m, n, k, s))
+    for _ in range(3):
+        out.zero_()
+        buf.zero_()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want)
+    one = C.c_void_p(buf.data_ptr())
+    assert L.rfq_gemm_f16_arrange(C.c_void_p(a.data_ptr()), m, k, one, nbytes - 1, None) == _lib.E_SIZE
+    assert L.rfq_gemm_f16_arranged(fmt, C.c_void_p(w.data_ptr()), w.numel(), one, nbytes - 1, C.c_void_p(out.data_ptr()),
+                                   _lib.F16, m, n, k, None) == _lib.E_SIZE
+    assert L.rfq_gemm_f16_arranged(fmt, C.c_void_p(w.data_ptr()), w.numel(), one, nbytes, C.c_void_p(out.data_ptr()),
+                                   _lib.BF16, m, n, k, None) == _lib.E_BADARG
