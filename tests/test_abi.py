@@ -67,3 +67,16 @@ def test_validation_needs_no_device():
     assert b"prepared A" in L.rfq_last_error()
     assert L.rfq_gemm_mx(one, pb, 4, one, pb - 16, 4, one, 0, 32, 32, 128, None) == _lib.E_SIZE
     assert b"prepared W" in L.rfq_last_error()
+
+
+def test_empty_inputs_are_accepted_without_touching_the_device():
+    """Zero elements / zero tokens: the reference's loops run zero times (dequantize_q4_0_cpu with n = 0 returns an
+    empty vector, src/kernels/quant/q4_0.rs:266-310); here the calls return before any device work."""
+    L = _lib.lib()
+    for fmt in (2, 8, 12, 14, 20, 21, 102, 112, 208, 212):
+        assert L.rfq_dequant(fmt, None, 0, None, 0, None) == _lib.OK
+        assert L.rfq_dequant_host(fmt, None, 0, None, 0) == _lib.OK
+        assert L.rfq_dequant_upload(fmt, None, 0, None, 0, None) == _lib.OK
+    assert L.rfq_get_rows(12, None, 256 * 16, 1, 4096, None, 0, None, None, None) == _lib.OK
+    assert L.rfq_upload(None, 0, None, None) == _lib.OK
+    assert L.rfq_packed_bytes(12, 0) == 0
