@@ -298,6 +298,7 @@ def cpu_baseline_more(Q, fmt, w, x, n, k, threads):
         multiplied by its thread; the reference itself is single-threaded);
       * dequantisation alone of a 4096 x 4096 tensor in Q4_0 and Q8_0, one thread, beside the figures the reference
         publishes for exactly that (benchmarks/baselines/rdna3-baseline.json:187-237: 12.8 ms and 15.2 ms);
+      * the Q4_0 and Q8_0 decode configurations (4864 x 896; 4096 x 4096 at m = 1 and 8) in full, one thread;
       * the two prefill GEMMs at M = 1 and M = 4 rows (dequantise all of W once, then the sequential fp32 matmul
         per row, one thread), with the linear extrapolation to their full M labelled as such."""
     import ctypes as C
@@ -330,7 +331,16 @@ def cpu_baseline_more(Q, fmt, w, x, n, k, threads):
         t = best_of(lambda: L.rf_dequantize(f, p(wq), wq.size, dst.size, p(dst)), 5)
         out[f"dequant_{name}_4096x4096"] = {"ms": round(t * 1e3, 2), "Gelem/s": round(dst.size / t / 1e9, 2), "threads": 1,
                                             "reference_published_ms": ref_ms}
+    # the two other decode configurations, measured in full: dequantise all weights, then the sequential matmul
     rng = np.random.Generator(np.random.PCG64(20260061))
+    for name, f, gm, gn, gk in (("Q4_0_gemv_4864x896_m1", Q.Q4_0, 1, 4864, 896), ("Q8_0_gemv_4096x4096_m1", Q.Q8_0, 1, 4096, 4096),
+                                ("Q8_0_gemv_4096x4096_m8", Q.Q8_0, 8, 4096, 4096)):
+        wq = Q.make_weights(f, gn, gk, seed=20260063)
+        wd = np.empty(gn * gk, np.float32)
+        a = rng.standard_normal((gm, gk), dtype=np.float32)
+        c = np.empty(gm * gn, np.float32)
+        t = best_of(lambda: L.rf_qmatmul_nk_staged(f, p(wq), wq.size, p(a), gm, gn, gk, p(wd), p(c)), 3)
+        out[name] = {"ms": round(t * 1e3, 2), "GB/s": round((wq.size + 4 * gm * gk + 4 * gm * gn) / t / 1e9, 3), "threads": 1}
     for name, f, gm, gn, gk in (("Q4_K_gemm_512x4096x14336", Q.Q4_K, 512, 14336, 4096),
                                 ("MXFP4_gemm_2048x8192x28672", Q.MXFP4, 2048, 28672, 8192)):
         slab = Q.make_weights(f, 4096 if gn % 4096 == 0 else gn, gk, seed=20260062)
