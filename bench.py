@@ -144,16 +144,16 @@ def time_get_rows(torch, fmt, n_vocab, n_embd, n_tokens, Q):
     tab = torch.from_numpy(np.tile(Q.make_weights(fmt, slab, n_embd, seed=20260033), n_vocab // slab)).to(dev)
     rng = np.random.Generator(np.random.PCG64(20260034))
     tok = torch.from_numpy(rng.integers(0, n_vocab, size=n_tokens).astype(np.int32)).to(dev)
-    for _ in range(5):
-        ops.get_rows(fmt, tab, tok, n_vocab, n_embd)
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    torch.cuda.synchronize()
-    e0.record()
-    for _ in range(50):
-        ops.get_rows(fmt, tab, tok, n_vocab, n_embd)
-    e1.record()
-    torch.cuda.synchronize()
-    t = e0.elapsed_time(e1) / 50 * 1e-3
+    import ctypes as C
+
+    from rocmforge_amd import _lib
+    out_copies = 32                                            # 268 MB of outputs: none is rewritten while still cached
+    out = torch.empty((out_copies, n_tokens, n_embd), dtype=torch.float32, device=dev)
+    ms = C.c_float(0)
+    _lib.check(_lib.lib().rfq_bench_get_rows(fmt, C.c_void_p(tab.data_ptr()), tab.numel(), n_vocab, n_embd,
+                                             C.c_void_p(tok.data_ptr()), n_tokens, C.c_void_p(out.data_ptr()), out_copies, 20, 200,
+                                             C.c_void_p(torch.cuda.current_stream().cuda_stream), C.byref(ms)))
+    t = ms.value / 200 * 1e-3
     b = n_tokens * (n_embd * 4 + Q.packed_bytes(fmt, n_embd))
     return {"us": round(t * 1e6, 2), "GB/s": round(b / t / 1e9, 1), "rows/s": round(n_tokens / t)}
 

@@ -31,6 +31,11 @@ RFQ_API int rfq_bench_gemv(int fmt, const void *const *d_w_copies, int copies, s
 RFQ_API int rfq_bench_dequant(int fmt, const void *const *d_in_copies, int copies, size_t packed_bytes, float *d_out,
                               size_t n_elems, int out_copies, int warmup, int steps, void *stream, float *elapsed_ms);
 
+/* rfq_get_rows in a native loop (step i gathers into d_out + (i % out_copies) * n_tokens * n_embd). */
+RFQ_API int rfq_bench_get_rows(int fmt, const void *d_table, size_t table_bytes, int n_vocab, int n_embd,
+                               const uint32_t *d_tokens, int n_tokens, float *d_out, int out_copies, int warmup,
+                               int steps, void *stream, float *elapsed_ms);
+
 /* Name and template arguments of the kernel that the calling thread's last rfq_gemv / rfq_rms_norm_gemv /
  * rfq_mlp_swiglu launch took ("" before the first), e.g. "gemv_idot_kernel<Q4_K,1,2,7>": lets the driver name the
  * kernel it timed from the dispatch actually taken instead of a constant. */

@@ -71,6 +71,7 @@ _SIGNATURES = {
     "rfq_bench_last_gemv_kernel": ([], C.c_char_p),
     "rfq_bench_read_floor": ([_vp, _i, _sz, _i, _i, _i, _i, _i, _i, _vp, C.POINTER(C.c_float)], _i),
     "rfq_bench_gemm_mx_prefill": ([_vp, _sz, _vp, _sz, _vp, _sz, _i, _vp, _i, _i, _i, _i, _i, _i, _vp, C.POINTER(C.c_float)], _i),
+    "rfq_bench_get_rows": ([_i, _vp, _sz, _i, _i, _vp, _i, _vp, _i, _i, _i, _vp, C.POINTER(C.c_float)], _i),
     "rfq_bench_gemm_f16_arranged": ([_i, _vp, _sz, _vp, _sz, _vp, _i, _i, _i, _i, _i, _i, _vp, C.POINTER(C.c_float)], _i),
     "rfq_bench_gemm_mx": ([_vp, _sz, _i, _vp, _sz, _i, _vp, _i, _i, _i, _i, _i, _i, _vp, C.POINTER(C.c_float)], _i),
 }

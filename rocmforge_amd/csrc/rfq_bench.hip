@@ -107,6 +107,16 @@ int rfq_bench_dequant(int fmt, const void *const *d_in_copies, int copies, size_
     });
 }
 
+int rfq_bench_get_rows(int fmt, const void *d_table, size_t table_bytes, int n_vocab, int n_embd, const uint32_t *d_tokens,
+                       int n_tokens, float *d_out, int out_copies, int warmup, int steps, void *stream, float *elapsed_ms)
+{
+    if (out_copies <= 0) return rfq::fail(RFQ_E_BADARG, "rfq_bench_get_rows: no output copies");
+    return timed_loop(warmup, steps, stream, elapsed_ms, [&](int i) {
+        return rfq_get_rows(fmt, d_table, table_bytes, n_vocab, n_embd, d_tokens, n_tokens,
+                            d_out + (size_t)(i % out_copies) * n_tokens * n_embd, nullptr, stream);
+    });
+}
+
 int rfq_bench_gemm_f16(int fmt, const void *d_w, size_t w_bytes, const void *d_a_f16, void *d_out, int out_dtype,
                        int m, int n, int k, int warmup, int steps, void *stream, float *elapsed_ms)
 {
