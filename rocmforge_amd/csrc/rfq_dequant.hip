@@ -633,21 +633,214 @@ gemv_kn_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, float
     if (VEC == 4) { o[1] = acc.y; o[2] = acc.z; o[3] = acc.w; }
 }
 
+// The same contraction for the reference's own four layouts when n is a multiple of 32: a lane owns one unit of 32
+// consecutive columns and fetches it with one wide load per row of Wd (16 to 32 bytes plus the scale) instead of
+// eight quads of two or three small loads each; what the 32 values of a unit share (a minimum, a code offset) is
+// summed once per row instead of per value.  The four
+// wavefronts of a workgroup take the rows l0 + w, l0 + w + 4, ... of the split and add their 32 sums per lane
+// through LDS in a fixed order.
+template <int FMT> struct KnUnit;
+
+// add(xl, acc, off): acc[i] += xl * (the part of value i that varies with i); off collects what all 32 values of the
+// unit share (the Q4_K minimum, the -8 and -128 of the code offsets), times xl; finish() puts it back.
+template <> struct KnUnit<RFQ_Q4_0> {                   // src/kernels/quant/q4_0.rs:289-306: scale * (nibble - 8)
+    float scale; uint4 q;
+    __device__ __forceinline__ void load(const uint8_t *w, size_t u)
+    {
+        const uint8_t *blk = w + u * 20;
+        scale = ld<float>(blk);
+        q = ld<uint4>(blk + 4);
+    }
+    __device__ __forceinline__ void add(float xl, float (&acc)[32], float &off) const
+    {
+        const float xs = xl * scale;
+        off = __builtin_fmaf(-8.0f, xs, off);
+        // nibbles 0, 2, 4, 6 of a dword become the bytes of one register, 1, 3, 5, 7 of another: a byte converts to
+        // float in one instruction
+#pragma unroll
+        for (int d = 0; d < 4; d++) {
+            const uint32_t lo = (&q.x)[d] & 0x0F0F0F0Fu, hi = ((&q.x)[d] >> 4) & 0x0F0F0F0Fu;
+#pragma unroll
+            for (int b = 0; b < 4; b++) {
+                acc[8 * d + 2 * b] = __builtin_fmaf((float)((lo >> (8 * b)) & 255u), xs, acc[8 * d + 2 * b]);
+                acc[8 * d + 2 * b + 1] = __builtin_fmaf((float)((hi >> (8 * b)) & 255u), xs, acc[8 * d + 2 * b + 1]);
+            }
+        }
+    }
+};
+
+template <> struct KnUnit<RFQ_Q8_0> {                   // src/kernels/quant/q8_0.rs:55-59: (byte - 128) * scale
+    float scale; uint4 q0, q1;
+    __device__ __forceinline__ void load(const uint8_t *w, size_t u)
+    {
+        const uint8_t *blk = w + u * 36;
+        scale = ld<float>(blk);
+        q0 = ld<uint4>(blk + 4);
+        q1 = ld<uint4>(blk + 20);
+    }
+    __device__ __forceinline__ void add(float xl, float (&acc)[32], float &off) const
+    {
+        const float xs = xl * scale;
+        off = __builtin_fmaf(-128.0f, xs, off);
+#pragma unroll
+        for (int i = 0; i < 32; i++) {
+            const uint32_t d = i < 16 ? (&q0.x)[i >> 2] : (&q1.x)[(i - 16) >> 2];
+            acc[i] = __builtin_fmaf((float)((d >> (8 * (i & 3))) & 255u), xs, acc[i]);
+        }
+    }
+};
+
+template <> struct KnUnit<RFQ_Q4_K> {                   // src/kernels/quant/q4_k.rs:222-268: min + nibble * scale
+    float scale, mn; uint4 q;
+    __device__ __forceinline__ void load(const uint8_t *w, size_t u)
+    {
+        const uint8_t *blk = w + (u >> 3) * 256;
+        const int sb = (int)(u & 7);
+        scale = f16_bits_to_f32(ld<uint16_t>(blk + 2 * sb));
+        mn = (float)(int8_t)blk[16 + sb];
+        q = ld<uint4>(blk + 32 + 28 * sb);
+    }
+    __device__ __forceinline__ void add(float xl, float (&acc)[32], float &off) const
+    {
+        const float xs = xl * scale;
+        off = __builtin_fmaf(xl, mn, off);
+        // nibbles 0, 2, 4, 6 of a dword become the bytes of one register, 1, 3, 5, 7 of another: a byte converts to
+        // float in one instruction
+#pragma unroll
+        for (int d = 0; d < 4; d++) {
+            const uint32_t lo = (&q.x)[d] & 0x0F0F0F0Fu, hi = ((&q.x)[d] >> 4) & 0x0F0F0F0Fu;
+#pragma unroll
+            for (int b = 0; b < 4; b++) {
+                acc[8 * d + 2 * b] = __builtin_fmaf((float)((lo >> (8 * b)) & 255u), xs, acc[8 * d + 2 * b]);
+                acc[8 * d + 2 * b + 1] = __builtin_fmaf((float)((hi >> (8 * b)) & 255u), xs, acc[8 * d + 2 * b + 1]);
+            }
+        }
+    }
+};
+
+template <> struct KnUnit<RFQ_Q6_K> {                   // src/kernels/quant/q6_k.rs:221-261: signed 6-bit code * scale of its 16
+    uint32_t sc2; uint32_t q[6];
+    __device__ __forceinline__ void load(const uint8_t *w, size_t u)
+    {
+        const uint8_t *blk = w + (u >> 3) * 256;
+        const int g = (int)(u & 7);
+        sc2 = ld<uint32_t>(blk + 4 * g);
+        const uint2 a = ld<uint2>(blk + 32 + 24 * g);
+        const uint4 b = ld<uint4>(blk + 32 + 24 * g + 8);
+        q[0] = a.x; q[1] = a.y; q[2] = b.x; q[3] = b.y; q[4] = b.z; q[5] = b.w;
+    }
+    __device__ __forceinline__ void add(float xl, float (&acc)[32], float &) const
+    {
+        const float xs0 = xl * f16_bits_to_f32((uint16_t)(sc2 & 0xFFFFu)), xs1 = xl * f16_bits_to_f32((uint16_t)(sc2 >> 16));
+#pragma unroll
+        for (int i = 0; i < 32; i++) {
+            const int bit = 6 * i, d = bit >> 5, sh = bit & 31;
+            const uint32_t lo = q[d] >> sh;
+            const uint32_t v = sh > 26 ? (lo | (q[d + 1] << (32 - sh))) : lo;     // a code that straddles two dwords
+            acc[i] = __builtin_fmaf((float)sbfe6(v, 0), i < 16 ? xs0 : xs1, acc[i]);
+        }
+    }
+};
+
+template <int FMT>
+__global__ void __launch_bounds__(256)
+gemv_kn_unit_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ part, int n, int k,
+                    int rows_per_split)
+{
+    __shared__ float red[4 * 32 * 64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int units_per_row = n >> 5;
+    const int c = blockIdx.x * 64 + lane;
+    const bool live = c < units_per_row;
+    const int cc = live ? c : units_per_row - 1;
+    const int l0 = blockIdx.y * rows_per_split;
+    int l1 = l0 + rows_per_split;
+    if (l1 > k) l1 = k;
+    float acc[32], off = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 32; i++) acc[i] = 0.0f;
+    // eight rows per trip: every load of the trip is issued before the first value is used (rows past the split's
+    // end repeat its last row with x taken as 0)
+    for (int lb = l0 + wave; lb < l1; lb += 32) {
+        KnUnit<FMT> un[8];
+        float xl[8];
+#pragma unroll
+        for (int r = 0; r < 8; r++) {
+            const int l = lb + 4 * r, lc = l < l1 ? l : l1 - 1;
+            un[r].load(w, (size_t)lc * units_per_row + cc);
+            xl[r] = l < l1 ? x[lc] : 0.0f;
+        }
+#pragma unroll
+        for (int r = 0; r < 8; r++) un[r].add(xl[r], acc, off);
+    }
+#pragma unroll
+    for (int i = 0; i < 32; i++) red[(wave * 32 + i) * 64 + lane] = acc[i] + off;
+    __syncthreads();
+    if (wave == 0 && live) {
+        float *o = part + (size_t)blockIdx.y * n + (size_t)c * 32;
+#pragma unroll
+        for (int i = 0; i < 32; i++)
+            o[i] = ((red[i * 64 + lane] + red[(32 + i) * 64 + lane]) + red[(64 + i) * 64 + lane]) + red[(96 + i) * 64 + lane];
+    }
+}
+
+// 64 columns per workgroup; wavefront g adds the splits g, g + 4, ... in ascending order and the four sums are
+// added in a fixed order: the result does not depend on timing.
 __global__ void __launch_bounds__(256)
 gemv_kn_reduce_kernel(const float *__restrict__ part, float *__restrict__ y, int n, int splits)
 {
-    const int j = blockIdx.x * 256 + threadIdx.x;
-    if (j >= n) return;
+    __shared__ float red[4][64];
+    const int lane = threadIdx.x & 63, g = threadIdx.x >> 6;
+    const int j = blockIdx.x * 64 + lane;
     float sum = 0.0f;
-    for (int s = 0; s < splits; s++) sum += part[(size_t)s * n + j];
-    y[j] = sum;
+    if (j < n) {
+#pragma unroll 8
+        for (int s = g; s < splits; s += 4) sum += part[(size_t)s * n + j];
+    }
+    red[g][lane] = sum;
+    __syncthreads();
+    if (g == 0 && j < n) y[j] = (red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane]);
 }
 
 constexpr size_t KN_PART_MAX = (size_t)8 << 20;   // bytes of partial sums at most
 
+template <int FMT> struct HasKnUnit { static constexpr bool value = FMT == RFQ_Q4_0 || FMT == RFQ_Q8_0 || FMT == RFQ_Q4_K || FMT == RFQ_Q6_K; };
+
+template <int FMT>
+int run_gemv_kn_units(const uint8_t *w, const float *x, float *y, int n, int k, hipStream_t s)
+{
+    const int bx = (n / 32 + 63) / 64;
+    // about four workgroups per CU, at least 16 rows per split (four per wavefront), partial sums within KN_PART_MAX
+    int splits = (4 * device_cu_count() + bx - 1) / bx;
+    if (splits > k / 16) splits = k / 16;
+    const size_t by_bytes = KN_PART_MAX / ((size_t)n * 4);
+    if ((size_t)splits > by_bytes) splits = (int)by_bytes;
+    if (splits < 1) splits = 1;
+    if (splits > 65535) splits = 65535;
+    const int rows_per_split = (k + splits - 1) / splits;
+    splits = (k + rows_per_split - 1) / rows_per_split;
+    float *part = y;
+    if (splits > 1) {
+        uint8_t *tmp = nullptr;
+        bool transient = false;
+        if (int rc = workspace(s, (size_t)splits * n * 4, &tmp, &transient)) return rc;   // (never transient: <= 8 MiB)
+        part = reinterpret_cast<float *>(tmp);
+    }
+    hipLaunchKernelGGL((gemv_kn_unit_kernel<FMT>), dim3(bx, splits), dim3(256), 0, s, w, x, part, n, k, rows_per_split);
+    RFQ_LAUNCH_CHECK("gemv_kn_unit_kernel");
+    if (splits > 1) {
+        hipLaunchKernelGGL(gemv_kn_reduce_kernel, dim3((n + 63) / 64), dim3(256), 0, s, part, y, n, splits);
+        RFQ_LAUNCH_CHECK("gemv_kn_reduce_kernel");
+    }
+    return RFQ_OK;
+}
+
 template <int FMT>
 int run_gemv_kn(const uint8_t *w, const float *x, float *y, int n, int k, hipStream_t s)
 {
+    if constexpr (HasKnUnit<FMT>::value) {
+        if (n % 32 == 0 && (reinterpret_cast<uintptr_t>(w) & 3u) == 0) return run_gemv_kn_units<FMT>(w, x, y, n, k, s);
+    }
     const bool vec = n % 4 == 0;
     const int groups = vec ? n / 4 : n;
     const int bx = (groups + 255) / 256;
@@ -671,7 +864,7 @@ int run_gemv_kn(const uint8_t *w, const float *x, float *y, int n, int k, hipStr
     else hipLaunchKernelGGL((gemv_kn_kernel<FMT, 1>), dim3(bx, splits), dim3(256), 0, s, w, x, part, n, k, rows_per_split);
     RFQ_LAUNCH_CHECK("gemv_kn_kernel");
     if (splits > 1) {
-        hipLaunchKernelGGL(gemv_kn_reduce_kernel, dim3((n + 255) / 256), dim3(256), 0, s, part, y, n, splits);
+        hipLaunchKernelGGL(gemv_kn_reduce_kernel, dim3((n + 63) / 64), dim3(256), 0, s, part, y, n, splits);
         RFQ_LAUNCH_CHECK("gemv_kn_reduce_kernel");
     }
     return RFQ_OK;
