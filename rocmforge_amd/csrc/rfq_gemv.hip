@@ -1497,8 +1497,9 @@ gemv_idot_batch_kernel(const uint8_t *__restrict__ w, const float *__restrict__ 
 // registers per lane, one wavefront per SIMD, and cannot keep enough loads in
 // flight to stream the matrix.  Here the M vectors are the rows of a matrix
 // operand instead: v_mfma_f32_16x16x32_f16 multiplies a 16 x 32 tile of
-// activations (vectors x one unit of k; rows 8..15 repeat rows 0..7 and their
-// results are dropped) with a 32 x 16 tile of weights (one unit of 16 rows).
+// activations (one unit of k; rows 0..7 are the high parts of the eight
+// vectors, rows 8..15 their low parts, see below) with a 32 x 16 tile of
+// weights (one unit of 16 rows).
 //
 // Exactness is kept as in the integer-dot scheme.  A small kernel first turns x
 // into block-fixed-point per unit and vector: a power of two s and integers
@@ -1523,9 +1524,10 @@ typedef float v4f_t __attribute__((ext_vector_type(4)));
 typedef uint32_t v2u_t __attribute__((ext_vector_type(2)));
 typedef uint32_t v4u_t __attribute__((ext_vector_type(4)));
 
-// parts: [unit][hi, lo][k octet 0..3][vector 0..7][8 fp16] (512 bytes per unit
-// and part; operand lane 16 * q + i reads octet q, vector i % 8); sx: [unit][8]
-// f32.  One workgroup per unit; thread t: vector t / 32, element t % 32.
+// parts: [unit][k octet 0..3][row 0..15][8 fp16] (1 KiB per unit; row i < 8 is
+// the high part of vector i, row i >= 8 the low part of vector i - 8; operand lane
+// 16 * q + i reads octet q, row i); sx: [unit][8] f32.  One workgroup per unit;
+// thread t: vector t / 32, element t % 32.
 __global__ void __launch_bounds__(256)
 gemv_mfma_prep_kernel(const float *__restrict__ x, _Float16 *__restrict__ parts, float *__restrict__ sx, int m, int k)
 {
@@ -1545,9 +1547,9 @@ gemv_mfma_prep_kernel(const float *__restrict__ x, _Float16 *__restrict__ parts,
     if (any_bad) sc = __uint_as_float(0x7FC00000u);   // a non-finite x poisons its unit, as it would a float sum
     const int X = any_bad ? 0 : (int)(__float_as_uint(__builtin_fmaf(xv, inv_s, 12582912.0f)) - 0x4B400000u);
     const int hi = X >> 11, lo = X & 2047;
-    const size_t at = ((size_t)u * 2 * 32 + (kk >> 3) * 8 + v) * 8 + (kk & 7);
+    const size_t at = ((size_t)u * 64 + (kk >> 3) * 16 + v) * 8 + (kk & 7);
     parts[at] = (_Float16)(float)hi;
-    parts[at + 32 * 8] = (_Float16)(float)lo;
+    parts[at + 8 * 8] = (_Float16)(float)lo;
     if (kk == 0) sx[u * 8 + v] = sc;
 }
 
@@ -1563,9 +1565,10 @@ gemv_mfma_q8_0_kernel(const uint8_t *__restrict__ w, const _Float16 *__restrict_
 {
     constexpr int BB = Fmt<FMT>::BB, DOFF = FMT == RFQ_Q8_0 ? 4 : 2;
     constexpr uint32_t FLIP = FMT == RFQ_Q8_0 ? 0u : 0x80808080u;
-    __shared__ float red[MFMA_WAVES * 16 * 8];
+    __shared__ float red[MFMA_WAVES * 2 * 16 * 8];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, j = lane & 15, q = lane >> 4;
     const int units = k / 32, n0 = blockIdx.x * 16;
+
     const int row = n0 + j < n ? n0 + j : n - 1;
     const uint8_t *row_ptr = w + (size_t)row * units * BB;
     // The weight bytes are fetched by four neighbouring lanes per row (32
@@ -1574,13 +1577,13 @@ gemv_mfma_q8_0_kernel(const uint8_t *__restrict__ w, const _Float16 *__restrict_
     const int row_c = n0 + (lane >> 2) < n ? n0 + (lane >> 2) : n - 1;
     const uint8_t *row_ptr_c = w + (size_t)row_c * units * BB + DOFF + 8 * (lane & 3);
     const int from_lane4 = 4 * (4 * j + q);
-    const v4u_t *parts_l = reinterpret_cast<const v4u_t *>(parts) + q * 8 + (j & 7);
+    const v4u_t *parts_l = reinterpret_cast<const v4u_t *>(parts) + lane;     // (octet q, row j: 16 bytes per lane)
     const v2h_t bias = {(_Float16)-1152.0f, (_Float16)-1152.0f};
     float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     for (int base = wave; base < units; base += MFMA_WAVES * MFMA_NB) {
         v2u_t wq[MFMA_NB];
         float ws[MFMA_NB];
-        v4u_t xh[MFMA_NB], xl[MFMA_NB];
+        v4u_t xa[MFMA_NB];
         v4f_t s4[MFMA_NB / 2];                          // (the x scales follow half a batch behind: registers)
         auto load_s4 = [&](int b) {
             const int u = base + MFMA_WAVES * b, uc = u < units ? u : units - 1;
@@ -1592,8 +1595,7 @@ gemv_mfma_q8_0_kernel(const uint8_t *__restrict__ w, const _Float16 *__restrict_
             const uint8_t *blk = row_ptr + (size_t)uc * BB;
             wq[b] = ld<v2u_t>(row_ptr_c + (size_t)uc * BB);
             ws[b] = FMT == RFQ_Q8_0 ? ld<float>(blk) : f16_bits_to_f32(ld<uint16_t>(blk));                    // (no branch around a load: it would wait for the others)
-            xh[b] = parts_l[(size_t)uc * 64];
-            xl[b] = parts_l[(size_t)uc * 64 + 32];
+            xa[b] = parts_l[(size_t)uc * 64];
             if (b < MFMA_NB / 2) load_s4(b);
         }
         __builtin_amdgcn_sched_barrier(0);             // (every load of the batch is out before the first is used)
@@ -1617,31 +1619,31 @@ gemv_mfma_q8_0_kernel(const uint8_t *__restrict__ w, const _Float16 *__restrict_
                 wb[2 * d] = o0;
                 wb[2 * d + 1] = o1;
             }
-            v8h_t wf, ah, al;
+            v8h_t wf, ax;
             __builtin_memcpy(&wf, &wb, 16);
-            __builtin_memcpy(&ah, &xh[b], 16);
-            __builtin_memcpy(&al, &xl[b], 16);
+            __builtin_memcpy(&ax, &xa[b], 16);
             const v4f_t zero = {0.0f, 0.0f, 0.0f, 0.0f};
-            const v4f_t sh = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah, wf, zero, 0, 0, 0);
-            const v4f_t sl = __builtin_amdgcn_mfma_f32_16x16x32_f16(al, wf, zero, 0, 0, 0);
+            // this lane's four results: weight row j times the high (q < 2) or low parts of vectors 4 (q & 1) ..+4
+            const v4f_t sp = __builtin_amdgcn_mfma_f32_16x16x32_f16(ax, wf, zero, 0, 0, 0);
             const float wsc = base + MFMA_WAVES * b < units ? ws[b] : 0.0f;
 #pragma unroll
-            for (int r = 0; r < 4; r++)
-                acc[r] = __builtin_fmaf(wsc * s4[b % (MFMA_NB / 2)][r], __builtin_fmaf(sh[r], 2048.0f, sl[r]), acc[r]);
+            for (int r = 0; r < 4; r++) acc[r] = __builtin_fmaf(wsc * s4[b % (MFMA_NB / 2)][r], sp[r], acc[r]);
             if (b + MFMA_NB / 2 < MFMA_NB) load_s4(b + MFMA_NB / 2);
         }
     }
-    if (q < 2) {
+    // red[wavefront][part: 0 high, 1 low][weight row][vector]
 #pragma unroll
-        for (int r = 0; r < 4; r++) red[(wave * 16 + j) * 8 + 4 * q + r] = acc[r];
-    }
+    for (int r = 0; r < 4; r++) red[((wave * 2 + (q >> 1)) * 16 + j) * 8 + 4 * (q & 1) + r] = acc[r];
     __syncthreads();
     if (tid < 128) {
         const int jj = tid >> 3, v = tid & 7;
-        float sum = 0.0f;
+        float hi = 0.0f, lo = 0.0f;
 #pragma unroll
-        for (int wv = 0; wv < MFMA_WAVES; wv++) sum += red[(wv * 16 + jj) * 8 + v];
-        if (v < m && n0 + jj < n) y[(size_t)v * n + n0 + jj] = sum;
+        for (int wv = 0; wv < MFMA_WAVES; wv++) {
+            hi += red[((wv * 2 + 0) * 16 + jj) * 8 + v];
+            lo += red[((wv * 2 + 1) * 16 + jj) * 8 + v];
+        }
+        if (v < m && n0 + jj < n) y[(size_t)v * n + n0 + jj] = __builtin_fmaf(hi, 2048.0f, lo);
     }
 }
 
