@@ -1348,9 +1348,11 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
     }
 
     // With R = D a row's slot is the same in every group, and the ring of rows in flight runs on across the groups:
-    // the slot a row leaves takes the same row of the next group.  Otherwise a group starts by requesting its first
-    // D rows with nothing in flight.  (Only the group size that long walks choose is compiled this way: the extra
-    // conditional load makes the short forms slower, 5.2 -> 5.5 us for Q8_0 4096 x 4096.)
+    // the slot a row leaves takes the same row of the next group (past the last group: the team's last row again,
+    // a cache hit whose result is never used).  Otherwise a group starts by requesting its first D rows with nothing
+    // in flight.  The ring's loads are unconditional: a load under a condition makes the compiler wait for every
+    // load in flight behind it.  Only the group size that long walks choose is compiled this way (the same ring
+    // measured on the other forms and on the float kernel gained 0..2 % or lost).
     constexpr bool RING = R == 5 && D == 5;
     __shared__ float part[2][R][WAVES];
     for (int g = 0; g < groups; g++) {
@@ -1374,7 +1376,7 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
                 }
             }
             if (i + D < R) load_row(i % D, base + i + D);
-            else if (RING && g + 1 < groups) load_row(i % D, base + i + D);
+            else if (RING) load_row(i % D, base + i + D);
             res[i] = wave_sum(acc);
         }
         // (`groups` is uniform over the block: every wavefront stores the same number of groups)
@@ -1796,9 +1798,9 @@ int run_idot(const uint8_t *w, const float *x, float *y, int n, int k, const Gem
         long best_cost = -1;
         for (int idx = 0; idx < 5; idx++) {
             int r = RS[idx];
-            if (r == 5 && !FIVE) continue;
             if (FUSE && f.glu && (r & 1)) continue;
             int groups = (want + r - 1) / r;
+            if (r == 5 && !(FIVE && groups > 1)) continue;
             int blocks = (n + TEAMS * r * groups - 1) / (TEAMS * r * groups);
             long waves_of_blocks = (blocks + slots - 1) / slots;
             long cost = waves_of_blocks * r * groups * (r == 5 && groups > 1 ? 19 : 20);

@@ -106,19 +106,20 @@ def test_gemv_baseline_configs(fmt, n, k, m, cfg, oracle, cuda):
 # rows against the oracle (first and last rows of the matrix, of a team's and a workgroup's range, and random ones)
 # and a checksum over every output: sum_n y[n] = x . sum_n W[n, :], the column sums taken from the oracle's dequantisation.
 @pytest.mark.timeout(600)
-@pytest.mark.parametrize("fmt", [Q.Q4_K, Q.GGUF_Q4_K])
+@pytest.mark.parametrize("fmt", [Q.Q4_K, Q.GGUF_Q4_K, Q.Q6_K, Q.GGUF_Q6_K, Q.Q8_0, Q.MXFP4])
 def test_lm_head_shape_sampled(fmt, oracle, cuda):
     n, k = 128256, 4096
     rng = np.random.default_rng(20260200 + fmt)
-    w = Q.random_blocks(fmt, n * k // 256, rng)
+    w = Q.random_blocks(fmt, n * k // Q.BLOCK_ELEMS[fmt], rng)
     x = x_for(1, k, 20260201)
     got = gpu_gemv(fmt, w, x, n, k, cuda)
-    rows = np.unique(np.concatenate([np.arange(0, 40), np.arange(n - 40, n), np.arange(62600, 62680),
+    # (a team walks its rows in groups of 5..8 with loads running on from group to group: whole teams' ranges)
+    rows = np.unique(np.concatenate([np.arange(0, 140), np.arange(n - 140, n), np.arange(62600, 62740),
                                      rng.integers(0, n, 400)]))
     want = oracle.qmatmul_nk(fmt, w, x, 1, n, k, rows=rows)[0]
     assert_close(got[rows], want, f"{Q.NAMES[fmt]} LM head, {rows.size} sampled rows")
     print(f"{Q.NAMES[fmt]} 128256x4096, {rows.size} rows: {error_report(got[rows], want)}")
-    rb = Q.BLOCK_BYTES[fmt] * k // 256
+    rb = Q.BLOCK_BYTES[fmt] * k // Q.BLOCK_ELEMS[fmt]
     colsum = np.zeros(k, np.float64)
     step = 8016                                               # 16 chunks of rows
     for r0 in range(0, n, step):
