@@ -34,7 +34,7 @@ CACHE_BYTES = 256 << 20
 # HBM bytes one launch of the headline kernel moves, from FETCH_SIZE / WRITE_SIZE
 # profiler counters scaled by a copy kernel of known size
 # (profiles/gemv_q4k_14336x4096_hbm_counters.txt): 57,576.4 KiB read + 64.0 KiB written.
-MEASURED_TRAFFIC_BYTES = 59023772
+MEASURED_TRAFFIC_BYTES = 59033935
 TRAFFIC_SOURCE = "profiles/gemv_q4k_14336x4096_hbm_counters.txt"
 # launch shapes of the read-only kernel that the floor is taken over (workgroups, threads, loads in flight, non-temporal)
 PREHEAT_MS = 30.0
