@@ -688,7 +688,10 @@ gemv_xreg_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
     // address traffic, not the weight stream, set the kernel's time (Q6_K 14336 x 4096: 6.4 us of 13.9).
     // LDS layout: 16-byte piece q (0..7) of unit u at ((q * ku + u) * 16), so consecutive lanes read consecutive pieces.
     extern __shared__ __attribute__((aligned(16))) float xstage_lds[];
-    constexpr int XQ = 4;                                         // pieces a thread holds in registers while the first rows are requested
+    // pieces a thread requests before the first rows' weights: all of x for the rows this form takes, up to the 8192
+    // values that are staged this way (a piece requested behind the weights would be served behind them, and the
+    // barrier below would hold every wavefront's first dot until then)
+    constexpr int XQ = 2 * UPL * WPR < 8 ? (2 * UPL * WPR < 4 ? 4 : 2 * UPL * WPR) : 8;
     const int pieces = ku * 8;
     float4 xq[XQ], nq[FUSE ? XQ : 1];
     if (xstage) {
@@ -1269,13 +1272,22 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
     if (row_end > n) row_end = n;
     const int row_last = row_end > row0 ? row_end - 1 : (n - 1);
 
-    // x goes first so that it also returns first.
-    float xv[8], nv[FUSE ? 8 : 1];
-    const bool prep0 = (int)threadIdx.x < 4 * ku;
+    // x goes first so that it also returns first: all of it, NX quarter units (eight values each) per thread for the
+    // longest row this form takes.  A CU serves its loads in the order they were issued, so a piece of x requested
+    // behind the first rows' weights would hold the barrier below, and with it every wavefront's first dot, until
+    // those rows had arrived (Q4_K 4096 x 14336: 12.2 -> 11.5 us, 8192 x 8192: 14.0 -> 12.8 us).
+    constexpr int NX = (4 * 64 * WPR * UPL + THREADS - 1) / THREADS;
+    float xv[NX][8], nv[FUSE ? NX : 1][8];
+    bool prep[NX];
     const bool norm = FUSE && f.norm_w != nullptr;
-    if (prep0) prep_load8(x + (size_t)threadIdx.x * 8, xv);
-    if constexpr (FUSE) {
-        if (norm && prep0) prep_load8(f.norm_w + (size_t)threadIdx.x * 8, nv);
+#pragma unroll
+    for (int i = 0; i < NX; i++) {
+        const int h = threadIdx.x + i * THREADS;
+        prep[i] = h < 4 * ku;
+        if (prep[i]) prep_load8(x + (size_t)h * 8, xv[i]);
+        if constexpr (FUSE) {
+            if (norm && prep[i]) prep_load8(f.norm_w + (size_t)h * 8, nv[i]);
+        }
     }
 
     IU buf[D][UPL];
@@ -1295,25 +1307,16 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
 
     // Cooperative conversion of x: 4*ku quarter-units (eight values each) over the block's threads.
     float ssq = 0.f;
-    if constexpr (FUSE) {
-        if (norm && prep0) {
 #pragma unroll
-            for (int i = 0; i < 8; i++) { ssq = __builtin_fmaf(xv[i], xv[i], ssq); xv[i] *= nv[i]; }
-        }
-    }
-    if (prep0) prep_convert_quarter<IU::NIBBLE, IU::TOPOFF>(xv, threadIdx.x & 3, xlds + (size_t)(threadIdx.x >> 2) * 28);
-    for (int h = threadIdx.x + THREADS; h < 4 * ku; h += THREADS) {
-        float xw[8];
-        prep_load8(x + (size_t)h * 8, xw);
+    for (int c = 0; c < NX; c++) {
+        const int h = threadIdx.x + c * THREADS;
         if constexpr (FUSE) {
-            if (norm) {
-                float nw[8];
-                prep_load8(f.norm_w + (size_t)h * 8, nw);
+            if (norm && prep[c]) {
 #pragma unroll
-                for (int i = 0; i < 8; i++) { ssq = __builtin_fmaf(xw[i], xw[i], ssq); xw[i] *= nw[i]; }
+                for (int i = 0; i < 8; i++) { ssq = __builtin_fmaf(xv[c][i], xv[c][i], ssq); xv[c][i] *= nv[c][i]; }
             }
         }
-        prep_convert_quarter<IU::NIBBLE, IU::TOPOFF>(xw, h & 3, xlds + (size_t)(h >> 2) * 28);
+        if (prep[c]) prep_convert_quarter<IU::NIBBLE, IU::TOPOFF>(xv[c], h & 3, xlds + (size_t)(h >> 2) * 28);
     }
     __shared__ float ssq_part[WAVES];
     if constexpr (FUSE) {
