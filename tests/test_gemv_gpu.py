@@ -34,7 +34,7 @@ def x_for(m, k, seed):
 # row, 32768 falls back again; n values exercise ragged teams.
 @pytest.mark.parametrize("fmt", FORMATS)
 @pytest.mark.parametrize("n,k", [(5, 256), (40, 512), (77, 768), (33, 1024), (64, 2048), (1001, 2048), (130, 4096), (257, 8192),
-                                 (19, 14336), (9, 32768), (2048, 1536)])
+                                 (19, 14336), (9, 32768), (2048, 1536), (21, 16384), (300, 12288)])
 def test_gemv_m1_shapes(fmt, n, k, oracle, cuda):
     w = Q.make_weights(fmt, n, k, seed=3000 + fmt + n)
     x = x_for(1, k, 4000 + k)
@@ -187,10 +187,12 @@ def test_gemv_more_than_eight_rows(oracle, cuda):
 
 
 @pytest.mark.parametrize("fmt", [Q.Q4_K, Q.Q6_K, Q.MXFP4, Q.MXFP6_E2M3, Q.Q4_0, Q.Q8_0, Q.GGUF_Q4_0, Q.GGUF_Q8_0])
-@pytest.mark.parametrize("n,k", [(14336, 4096), (14413, 4096), (15001, 2304), (20000, 2560), (14337, 3840), (8192, 4096), (8201, 2304), (11008, 4096)])
+@pytest.mark.parametrize("n,k", [(14336, 4096), (14413, 4096), (15001, 2304), (20000, 2560), (14337, 3840), (8192, 4096), (8201, 2304), (11008, 4096),
+                                 (50000, 4096), (51203, 2304)])
 def test_long_matrices_one_unit_per_lane(fmt, n, k, oracle, cuda):
     """Q4_K and the float-path formats with rows of 65..128 units and at least seven rows per team run with one
-    unit per lane and two wavefronts per row: ragged row counts, rows that end inside the second wavefront."""
+    unit per lane and two wavefronts per row: ragged row counts, rows that end inside the second wavefront; at 50000 rows
+    a team walks several groups of five rows with its loads carrying on from group to group."""
     w = Q.make_weights(fmt, n, k, seed=5300 + n + fmt)
     x = x_for(1, k, 6300 + k)
     got = gpu_gemv(fmt, w, x, n, k, cuda)
