@@ -119,7 +119,9 @@ template <int NW> __device__ __forceinline__ void load_dwords_a4(const uint8_t *
 // launcher checks (a tensor at another address takes the byte-exact load_bytes in the generic kernel).
 __device__ __forceinline__ U8 load32_a2(const uint8_t *c)
 {
-    const uint8_t *a = reinterpret_cast<const uint8_t *>(reinterpret_cast<uintptr_t>(c) & ~(uintptr_t)3);
+    // (stepping back from c rather than building a pointer from the masked integer: the loads stay global loads
+    // instead of flat ones, which also count against the LDS counter)
+    const uint8_t *a = c - (reinterpret_cast<uintptr_t>(c) & 3u);
     const uint32_t sel = 0x03020100u + 0x01010101u * (uint32_t)(reinterpret_cast<uintptr_t>(c) & 3u);
     uint32_t d[9];
     load_dwords_a4<9>(a, d);
@@ -1190,12 +1192,15 @@ template <> struct IUnit<RFQ_GGUF_Q6_K> : Unit<RFQ_GGUF_Q6_K> {
     static constexpr uint32_t TOPOFF = 0;
     __device__ __forceinline__ float idot(const XPrep &xp) const
     {
-        const int shl = 4 * (t >> 1), shh = 2 * t;
+        // bits 4-5 of a code: the bit pair at 2t of its qh byte, brought to bits 4-5 by one rotation (what it drags in
+        // from the neighbouring bytes is masked away)
+        const int shl = 4 * (t >> 1), rot = (2 * t + 28) & 31;
         uint32_t alo[2] = {0, 0}, amid[2] = {0, 0};
         int atop[2] = {0, 0};
 #pragma unroll
         for (int w = 0; w < 8; w++) {
-            const uint32_t v = ((ql.v[w] >> shl) & 0x0F0F0F0Fu) | (((qh.v[w] >> shh) & 0x03030303u) << 4);
+            const uint32_t h4 = __builtin_amdgcn_alignbit(qh.v[w], qh.v[w], rot);
+            const uint32_t v = (h4 & 0x30303030u) | ((ql.v[w] >> shl) & 0x0F0F0F0Fu);
             const uint32_t *L = &xp.l[w * 3];
             alo[w >> 2] = __builtin_amdgcn_udot4(v, L[0], alo[w >> 2], false);
             amid[w >> 2] = __builtin_amdgcn_udot4(v, L[1], amid[w >> 2], false);
