@@ -548,16 +548,23 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
                 else
                     asm volatile("global_load_dwordx4 %0, %1, %2 offset:1024" : "=v"(areg4[SET][i][1]) : "v"(voff), "s"(base) : "memory");
             } else {
-                uint4 v = *reinterpret_cast<const uint4 *>(pf_a[i] + voffA + ksl * PA + half * 1024);
-                areg[SET][i][ksl][4 * half + 0] = (int)v.x; areg[SET][i][ksl][4 * half + 1] = (int)v.y;
-                areg[SET][i][ksl][4 * half + 2] = (int)v.z; areg[SET][i][ksl][4 * half + 3] = (int)v.w;
+                // (the bases were rebuilt from scalar integers: naming the global address space keeps these global
+                // loads; as flat loads they would also count against the LDS counter)
+                typedef int v4i_g __attribute__((ext_vector_type(4)));
+                typedef const __attribute__((address_space(1))) v4i_g *GlobalV4;
+                const v4i_g v = *reinterpret_cast<GlobalV4>(reinterpret_cast<uintptr_t>(pf_a[i] + voffA + ksl * PA + half * 1024));
+                areg[SET][i][ksl][4 * half + 0] = v[0]; areg[SET][i][ksl][4 * half + 1] = v[1];
+                areg[SET][i][ksl][4 * half + 2] = v[2]; areg[SET][i][ksl][4 * half + 3] = v[3];
             }
         } else {
             const int i = piece - TI * 2 * A_PER_FRAG;
             const uint8_t *base = pf_as[i];
             const uint32_t voff = voffAS;
             if (AK == RFQ_MX_FP4) asm volatile("global_load_dword %0, %1, %2" : "=v"(ascl[SET][i]) : "v"(voff), "s"(base) : "memory");
-            else ascl[SET][i] = *reinterpret_cast<const int *>(base + voff);
+            else {
+                typedef const __attribute__((address_space(1))) int *GlobalI;
+                ascl[SET][i] = *reinterpret_cast<GlobalI>(reinterpret_cast<uintptr_t>(base + voff));
+            }
         }
     };
     auto a_frag = [&](auto setc, int i, int ksl) -> v8i {
