@@ -56,6 +56,46 @@ __device__ __forceinline__ float wave_sum(float v)
     return (r0 + r1) + (r2 + r3);
 }
 
+// Sums of M values per lane over the 16 lanes of each row, M = 2, 4 or 8: instead of M separate reductions, lanes that
+// differ in one bit exchange half of what they hold (the lane keeps the value whose index has that bit like its own
+// number and adds the partner's copy of it), so after log2(M) steps a lane holds a single partial sum, of value number
+// lane % M, and the remaining steps are one addition each.  Afterwards lane l holds the sum of value l % M over its
+// row of 16 lanes.  25 instructions for M = 8 where eight wave_sum take about 90.
+template <int CTRL> __device__ __forceinline__ float dpp_get(float v)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+// the value of lane ^ 4: lanes 4..7 and 12..15 of a row take it from four lanes down, the others from four lanes up
+__device__ __forceinline__ float dpp_xor4(float v)
+{
+    int r = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x114, 0xF, 0xA, false);          // row_shr:4 into banks 1, 3
+    r = __builtin_amdgcn_update_dpp(r, __float_as_int(v), 0x104, 0xF, 0x5, false);              // row_shl:4 into banks 0, 2
+    return __int_as_float(r);
+}
+template <int M> __device__ __forceinline__ float rows16_sum_of(const float (&a)[M], int lane)
+{
+    static_assert(M == 2 || M == 4 || M == 8, "two, four or eight values");
+    const bool b0 = lane & 1, b1 = lane & 2, b2 = lane & 4;
+    float w[M / 2];
+#pragma unroll
+    for (int p = 0; p < M / 2; p++) w[p] = (b0 ? a[2 * p + 1] : a[2 * p]) + dpp_get<0xB1>(b0 ? a[2 * p] : a[2 * p + 1]);
+    float f;
+    if constexpr (M == 2) {
+        f = w[0] + dpp_get<0x4E>(w[0]);
+        f += dpp_xor4(f);
+    } else {
+        float z[M / 4];
+#pragma unroll
+        for (int q = 0; q < M / 4; q++) z[q] = (b1 ? w[2 * q + 1] : w[2 * q]) + dpp_get<0x4E>(b1 ? w[2 * q] : w[2 * q + 1]);
+        if constexpr (M == 4) {
+            f = z[0] + dpp_xor4(z[0]);
+        } else {
+            f = (b2 ? z[1] : z[0]) + dpp_xor4(b2 ? z[0] : z[1]);
+        }
+    }
+    return f + dpp_get<0x128>(f);                                                              // row_ror:8
+}
+
 // The value of the neighbouring lane (lane ^ 1).
 __device__ __forceinline__ float dpp_xor1_f(float v)
 {
@@ -1456,14 +1496,15 @@ gemv_idot_batch_kernel(const uint8_t *__restrict__ w, const float *__restrict__ 
         xp[v].xh1 = __uint_as_float(src[27]);
     }
 
-    __shared__ float part[R * M][4];
+    // The M sums of a row are reduced together (rows16_sum_of) and the four 16-lane rows of each of the team's
+    // wavefronts meet in LDS: part[row * M + vector][4 * wavefront + lane row].
+    __shared__ float part[R * M][16];
     for (int g = 0; g < groups; g++) {
         const int base = g * R;
         if (g > 0) {
 #pragma unroll
             for (int d = 0; d < D; d++) load_row(d, base + d);
         }
-        float res[R][M];
 #pragma unroll
         for (int i = 0; i < R; i++) {
             float acc[M];
@@ -1473,39 +1514,21 @@ gemv_idot_batch_kernel(const uint8_t *__restrict__ w, const float *__restrict__ 
                 acc[v] = live ? t : 0.f;
             }
             if (i + D < R) load_row(i % D, base + i + D);
-#pragma unroll
-            for (int v = 0; v < M; v++) res[i][v] = wave_sum(acc[v]);
+            const float f = rows16_sum_of<M>(acc, lane);
+            if ((lane & 15) < M) part[i * M + (lane & 15)][wave * 4 + (lane >> 4)] = f;
         }
-        if (WPR == 1) {
-            if (lane == 0) {
+        // `groups` is uniform over the block, so every wavefront reaches both barriers the same number of times
+        // (a team of one wavefront reads back what it wrote itself: its LDS operations complete in order).
+        if (WPR > 1) __syncthreads();
+        if (wit == 0 && lane < R * M) {
+            const int i = lane / M, v = lane % M;
+            const int r = row0 + base + i;
+            float t = 0.f;
 #pragma unroll
-                for (int i = 0; i < R; i++) {
-                    int r = row0 + base + i;
-#pragma unroll
-                    for (int v = 0; v < M; v++)
-                        if (r < row_end && v < m_valid) y[(size_t)v * n + r] = res[i][v];
-                }
-            }
-        } else {
-            // `groups` is uniform over the block, so every wavefront reaches
-            // both barriers the same number of times.
-            if (lane == 0) {
-#pragma unroll
-                for (int i = 0; i < R; i++)
-#pragma unroll
-                    for (int v = 0; v < M; v++) part[i * M + v][wave] = res[i][v];
-            }
-            __syncthreads();
-            if (wit == 0 && lane < R * M) {
-                const int i = lane / M, v = lane % M;
-                const int r = row0 + base + i;
-                float t = 0.f;
-#pragma unroll
-                for (int q = 0; q < WPR; q++) t += part[lane][team * WPR + q];
-                if (r < row_end && v < m_valid) y[(size_t)v * n + r] = t;
-            }
-            __syncthreads();
+            for (int q = 0; q < 4 * WPR; q++) t += part[lane][team * WPR * 4 + q];
+            if (r < row_end && v < m_valid) y[(size_t)v * n + r] = t;
         }
+        if (WPR > 1) __syncthreads();
     }
 }
 
