@@ -2031,6 +2031,17 @@ int run(const uint8_t *w, const float *x, float *y, int m, int n, int k, hipStre
         }
         return RFQ_OK;
     }
+    // No batch kernel for this format or row length (the float-path formats; integer formats beyond 256 units per
+    // row): from eight million weights on, one decode launch per vector beats the one-row-per-wavefront kernel,
+    // although it reads the weights m times (Q6_K, m = 8: 14336 x 4096 321 -> 91 us, 4096 x 4096 80 -> 37 us; at
+    // 1024 x 2048 the single launch is the faster one, 11 against 22 us).
+    if (m > 1 && ku > 16 && ku <= 512 && (size_t)n * (size_t)k >= ((size_t)1 << 23)) {
+        for (int v = 0; v < m; v++) {
+            const int rc = run_rows<FMT, false>(w, x + (size_t)v * k, y + (size_t)v * n, n, k, GemvFuse{nullptr, nullptr, 0.0f, 0}, s);
+            if (rc != RFQ_OK) return rc;
+        }
+        return RFQ_OK;
+    }
     return run_generic_m<FMT>(w, x, y, m, n, k, s);
 }
 

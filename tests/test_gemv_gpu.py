@@ -54,6 +54,19 @@ def test_gemv_small_batches(fmt, m, oracle, cuda):
     assert_close(got, oracle.qmatmul_nk(fmt, w, x, m, n, k), f"{Q.NAMES[fmt]} m={m}")
 
 
+# Batches of a format or row length without a batch kernel go out as one decode launch per vector once the matrix has
+# eight million weights (below that the one-row-per-wavefront kernel takes the whole batch).
+@pytest.mark.parametrize("fmt,n,k", [(Q.Q6_K, 2100, 4096), (Q.MXFP4, 2100, 4096), (Q.MXFP6_E2M3, 2049, 4096),
+                                     (Q.Q4_K, 700, 12288), (Q.Q4_0, 513, 16384), (Q.Q6_K, 1100, 8192)])
+@pytest.mark.parametrize("m", [2, 5, 8])
+def test_gemv_batches_as_decode_launches(fmt, n, k, m, oracle, cuda):
+    w = Q.make_weights(fmt, n, k, seed=5100 + fmt + n)
+    x = x_for(m, k, 6100 + m)
+    got = gpu_gemv(fmt, w, x, n, k, cuda)
+    assert got.shape == (m, n)
+    assert_close(got, oracle.qmatmul_nk(fmt, w, x, m, n, k), f"{Q.NAMES[fmt]} {n}x{k} m={m}")
+
+
 # Q8_0 batches run on the matrix cores: 16 rows per workgroup, 16 wavefronts
 # that take every 16th unit, eight units at a time: odd unit counts, more than
 # one trip, fewer units than wavefronts, a ragged last row tile.
