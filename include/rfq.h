@@ -30,7 +30,9 @@
 extern "C" {
 #endif
 
-#define RFQ_VERSION 100 /* 0.1.0 */
+/* Raised whenever an exported signature or the meaning of a format changes: a caller compares
+ * rfq_version() with the RFQ_VERSION it was built against before its first call. */
+#define RFQ_VERSION 102 /* 0.1.2 */
 
 #if defined(_WIN32)
 #define RFQ_API
@@ -72,9 +74,10 @@ typedef enum rfq_format {
     RFQ_MM_Q8_0 = 208,   /* 36 B / 32: f32 scale + 32 two's-complement int8 bytes; scale * q
                             (quantized/q8_0.rs:18-56)                                                      */
     RFQ_MM_Q4_K = 212,   /* 256 B / 256: as RFQ_Q4_K but the nibbles of sub-block sb start at 32 + 20 * sb,
-                            and the f16 scale is widened by f16_to_f32_cpu (quantized/common.rs:44-60,
-                            which reads exponent field 0 as 2^-15 * (1 + m/1024) and field 31 as
-                            2^16 * (1 + m/1024)); min + q * scale (quantized/q4_k.rs:90-148)               */
+                            and the f16 scale is widened by f16_to_f32_cpu (quantized/common.rs:44-60:
+                            its mantissa shift runs in 16 bits and its zero/subnormal branch is dead, so
+                            a pattern b reads +-2^(field - 15) * (1 + (b & 7) / 1024) -- 0x3E00 is 1.0,
+                            0x0000 is 2^-15); min + q * scale (quantized/q4_k.rs:90-148)                   */
     RFQ_MM_Q6_K = 214    /* 256 B / 256: the RFQ_Q6_K stream with the scales widened by f16_to_f32_cpu
                             (quantized/q6_k.rs:90-148)                                                     */
 } rfq_format;

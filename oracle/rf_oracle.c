@@ -26,13 +26,15 @@
  *              numpy statement), rf_dequant_mm_q4_k, rf_dequant_mm_q6_k
  *              (independent whole-array numpy statements on random blocks; the
  *              canonical decoders on the inputs where the two must agree),
- *              rf_f16_to_f32_mm for the 61 440 normal binary16 patterns (equals
- *              IEEE widening), rf_qmatmul_kn (rf_cpu_matmul_f32 on the flat
- *              dequantised stream; the recipe of quantized/q4_0.rs:343-435)
+ *              rf_f16_to_f32_mm for all 65 536 patterns (an independent
+ *              statement in 16-bit numpy integers of the shift the reference
+ *              performs in u16, and hand values), rf_qmatmul_kn
+ *              (rf_cpu_matmul_f32 on the flat dequantised stream; the recipe of
+ *              quantized/q4_0.rs:343-435)
  *   parity unpinned (no reference vector; follows from reading the code):
- *              rf_f16_to_f32_mm for exponent field 0 (zero, subnormals) and 31
- *              (inf, NaN), where the reference's `exp <= 0` test can never hold
- *              and the value is 2^(e-15) * (1 + m/1024) for every pattern
+ *              that the `exp <= 0` branch of f16_to_f32_cpu is dead (exponent
+ *              fields 0 and 31 of rf_f16_to_f32_mm take the same closed form as
+ *              every other field)
  *   parity unpinned (no counterpart in the reference; public ggml layouts):
  *              rf_dequant_gguf_q4_0 / q8_0 / q4_k / q6_k
  *   parity unpinned (no reference vector, reasoned from compiler-rt source):
@@ -476,17 +478,26 @@ RF_API void rf_dequant_mxfp6(const uint8_t *data, size_t len, size_t n, float *o
 /* differ from the canonical decoders above in layout or arithmetic.     */
 /* ------------------------------------------------------------------ */
 
-/* f16_to_f32_cpu, src/kernels/matmul/quantized/common.rs:44-60.  `exp` already
- * carries the f32 bias (field + 112 >= 112), so the `exp <= 0` branch that
- * was meant for zero and subnormals is never taken: every pattern decodes as
- * sign | (field + 112) << 23 | mantissa << 13.  Normal numbers come out
- * exact; field 0 reads 2^-15 * (1 + m/1024) (0x0000 -> 2^-15), field 31 reads
- * 2^16 * (1 + m/1024).  The branch is kept as written. */
+/* f16_to_f32_cpu, src/kernels/matmul/quantized/common.rs:44-60, token by
+ * token with Rust's integer widths.  Two things make it differ from IEEE
+ * widening:
+ *  - line 47 is `((bits & 0x03FF) << 13) as u32` with `bits: u16`: the shift
+ *    happens in 16 bits (a shift count below the width never panics, the bits
+ *    shifted out are dropped) and only then is the result widened, so mantissa
+ *    bits 3..9 are lost and the mantissa term is `(bits & 7) << 13`;
+ *  - `exp` already carries the f32 bias (field + 112 >= 112), so the
+ *    `exp <= 0` branch meant for zero and subnormals is never taken.
+ * Every pattern therefore decodes as sign | (field + 112) << 23 | (bits & 7) << 13
+ * = +-2^(field - 15) * (1 + (bits & 7) / 1024): 0x3E00 (1.5) reads 1.0, 0x2E66
+ * (0.1) reads 0.062866..., 0x0000 reads 2^-15.  Only patterns whose mantissa
+ * bits 3..9 are zero (powers of two among them: 0x3C00 -> 1.0, 0x4000 -> 2.0)
+ * come out as IEEE.  The branch is kept as written. */
 RF_API float rf_f16_to_f32_mm(uint16_t bits)
 {
     uint32_t sign = (bits & 0x8000u) != 0 ? (1u << 31) : 0u;
     int32_t exp = (int32_t)((bits & 0x7C00u) >> 10) - 15 + 127;
-    uint32_t mant = (uint32_t)(bits & 0x03FFu) << 13;
+    uint16_t mant16 = (uint16_t)((bits & 0x03FFu) << 13);   /* u16 << 13: Rust shifts before `as u32` */
+    uint32_t mant = (uint32_t)mant16;
     uint32_t out;
     if (exp <= 0) {
         if ((bits & 0x7FFFu) == 0) out = sign;

@@ -207,13 +207,14 @@ __device__ __forceinline__ uint32_t gguf_scale_min_k4(int j, uint32_t s0, uint32
     return ((sc2 >> hs) & 255u) | (((mn2 >> hs) & 255u) << 8);
 }
 
-// f16_to_f32_cpu of the matmul module (src/kernels/matmul/quantized/common.rs:44-60): its test for zero and
-// subnormals compares the already re-biased exponent with 0 and never holds, so every pattern widens as
-// sign | (field + 112) << 23 | mantissa << 13 (exact for normal numbers only).
+// f16_to_f32_cpu of the matmul module (src/kernels/matmul/quantized/common.rs:44-60).  Its mantissa term is
+// `((bits & 0x03FF) << 13) as u32` on a u16: the shift is done in 16 bits, so only mantissa bits 0..2 survive
+// (as bits 13..15); its test for zero and subnormals compares the already re-biased exponent with 0 and never
+// holds.  Every pattern widens as sign | (field + 112) << 23 | (bits & 7) << 13.
 __device__ __forceinline__ float f16_bits_to_f32_mm(uint16_t h)
 {
     const uint32_t b = h;
-    return __uint_as_float(((b & 0x8000u) << 16) | ((((b >> 10) & 31u) + 112u) << 23) | ((b & 0x3FFu) << 13));
+    return __uint_as_float(((b & 0x8000u) << 16) | ((((b >> 10) & 31u) + 112u) << 23) | ((b & 7u) << 13));
 }
 
 // Signed 6-bit field (two's complement) starting at bit `off` of w.

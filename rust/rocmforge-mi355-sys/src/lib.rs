@@ -48,7 +48,7 @@ pub const RFQ_MX_FP4: c_int = 4;
 pub const RFQ_MX_FP8: c_int = 8;
 pub const RFQ_MX_FP4_UNCHECKED: c_int = 0x104;
 
-pub const RFQ_VERSION: c_int = 100;
+pub const RFQ_VERSION: c_int = 102;
 
 #[link(name = "rfq")]
 extern "C" {

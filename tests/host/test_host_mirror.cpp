@@ -344,11 +344,17 @@ static void test_matmul_as_the_reference_computes_it()
     EXPECT(matmul_q8_0_as_computed(be.value, q8, in8.value, 1, 32, out8.value).ok);
     std::vector<float> y8(1);
     EXPECT(out8.value.copy_to_host(y8).ok && y8[0] == -16.0f);                          // sum of -16 .. 15
-    // the K decoders of the module: normal scales decode like the loader's Q6_K; Q4_K reads other bytes
+    // the K decoders of the module: a scale whose mantissa bits 3..9 are clear decodes like the loader's Q6_K; Q4_K reads
+    // other bytes
     bytes k6(256, 0);
     for (int g = 0; g < 16; g++) put_f16(k6, 2 * g, 0x3C00);                           // 1.0
     for (int i = 32; i < 224; i++) k6[i] = (uint8_t)(i * 7);
     EXPECT(matmul_quantized::dequantize_q6_k(k6, 256) == loader::dequant_q6_k(k6, 256));
+    // f16_to_f32_cpu (quantized/common.rs:47) shifts the mantissa within 16 bits: 0x3E00 (1.5) widens to 1.0 there
+    bytes k6b = k6;
+    for (int g = 0; g < 16; g++) put_f16(k6b, 2 * g, 0x3E00);
+    EXPECT(matmul_quantized::dequantize_q6_k(k6b, 256) == matmul_quantized::dequantize_q6_k(k6, 256));
+    EXPECT(loader::dequant_q6_k(k6b, 256) != loader::dequant_q6_k(k6, 256));
     bytes k4(256, 0);
     for (int sb = 0; sb < 8; sb++) put_f16(k4, 2 * sb, 0x3C00);
     for (int i = 32; i < 256; i++) k4[i] = (uint8_t)(i * 5 + 1);

@@ -28,7 +28,11 @@ def test_header_symbols_exported():
 
 def test_sizes_and_version():
     L = rocmforge_amd.lib()
-    assert L.rfq_version() == 100
+    header = open(os.path.join(os.path.dirname(__file__), "..", "include", "rfq.h")).read()
+    crate = open(os.path.join(os.path.dirname(__file__), "..", "rust", "rocmforge-mi355-sys", "src", "lib.rs")).read()
+    declared = int(re.search(r"#define\s+RFQ_VERSION\s+(\d+)", header).group(1))
+    assert L.rfq_version() == declared == int(re.search(r"RFQ_VERSION: c_int = (\d+);", crate).group(1))
+    assert declared >= 102
     assert [L.rfq_block_bytes(f) for f in (2, 8, 12, 14, 20, 21, 22)] == [20, 36, 256, 256, 17, 25, 25]
     assert [L.rfq_block_elems(f) for f in (2, 8, 12, 14, 20, 21, 22)] == [32, 32, 256, 256, 32, 32, 32]
     assert L.rfq_block_bytes(3) == 0 and L.rfq_block_elems(99) == 0

@@ -5,14 +5,15 @@ orientation its matmuls compute (q4_0.rs:274-311 with src/tensor/matmul.rs:219-2
 What pins what:
   * the reference's own vector for the int8 decoder (quantized/q8_0.rs:113-131) and the recipe of its GPU test
     (quantized/q4_0.rs:343-435: shapes and byte pattern), evaluated independently in float64;
-  * IEEE widening for every normal binary16 pattern (what f16_to_f32_cpu must return there);
+  * f16_to_f32_cpu on all 65 536 patterns against a statement of it in numpy integers of Rust's widths (its mantissa
+    shift runs in u16 and keeps mantissa bits 0..2 only), a closed form, and hand values;
   * whole-array numpy statements of the three layouts written from the Rust, compared bit for bit on random blocks
     (a wrong stride, nibble order, sign extension or operand order fails them);
-  * the canonical decoders wherever the two families must agree (Q6_K with normal scales; sub-block 0 of Q4_K,
-    whose nibbles start at byte 32 under either stride).
-rf_f16_to_f32_mm for exponent fields 0 and 31 is "parity unpinned": the closed form checked here is what the
-reference's arithmetic gives by reading it (its zero/subnormal branch can never be taken); the reference holds
-no vector for it."""
+  * the canonical decoders wherever the two families must agree (normal scales whose mantissa bits 3..9 are clear, the
+    only ones both widenings read alike: Q6_K as a whole; sub-block 0 of Q4_K, whose nibbles start at byte 32 under
+    either stride), and that they part ways on any other scale.
+The reference holds no vector for f16_to_f32_cpu itself; what is checked is its arithmetic as written, branch
+included (the branch for zero and subnormals can never be taken: the exponent it tests is field + 112)."""
 import struct
 
 import numpy as np
@@ -28,30 +29,50 @@ def f32le(v):
 
 
 def mm_f16_numpy(bits):
-    """sign | (field + 112) << 23 | mantissa << 13, as float32."""
-    b = bits.astype(np.uint32)
-    return (((b & 0x8000) << 16) | ((((b >> 10) & 31) + 112) << 23) | ((b & 0x3FF) << 13)).astype(np.uint32).view(np.float32)
+    """f16_to_f32_cpu (quantized/common.rs:44-60) with every intermediate in the integer width Rust gives it:
+    `bits` is u16, so `(bits & 0x03FF) << 13` is a 16-bit shift whose high bits fall off before `as u32`."""
+    bits = np.asarray(bits).astype(np.uint16)
+    sign = np.where((bits & np.uint16(0x8000)) != 0, np.uint32(1 << 31), np.uint32(0)).astype(np.uint32)
+    exp = ((bits & np.uint16(0x7C00)) >> np.uint16(10)).astype(np.int32) - 15 + 127
+    mant16 = (bits & np.uint16(0x03FF)) << np.uint16(13)
+    assert mant16.dtype == np.uint16                                  # the shift stayed in 16 bits
+    mant = mant16.astype(np.uint32)
+    normal = (sign | (exp.astype(np.uint32) << np.uint32(23)) | mant).astype(np.uint32).view(np.float32)
+    zero = sign.view(np.float32)
+    return np.where(exp <= 0, np.where((bits & np.uint16(0x7FFF)) == 0, zero, np.float32(0.0)), normal).astype(np.float32)
 
 
-def test_f16_mm_equals_ieee_for_normal_numbers(oracle):
+def test_f16_mm_all_patterns(oracle):
     L = oracle.lib()
     bits = np.arange(65536, dtype=np.uint32).astype(np.uint16)
     got = np.array([L.rf_f16_to_f32_mm(int(b)) for b in bits], dtype=np.float32)
+    want = mm_f16_numpy(bits)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    # closed form: +-2^(field - 15) * (1 + (bits & 7) / 1024) -- mantissa bits 3..9 never arrive
+    b = bits.astype(np.int64)
+    closed = np.where(b & 0x8000, -1.0, 1.0) * 2.0 ** (((b >> 10) & 31) - 15.0) * (1.0 + (b & 7) / 1024.0)
+    assert np.array_equal(got.astype(np.float64), closed)
+    # it equals IEEE widening exactly where mantissa bits 3..9 are clear and the number is normal (1/128 of them), and by
+    # coincidence on the subnormal +-0x0200 = 2^-15, which this routine reads as 2^-15 * (1 + 0)
+    ieee = bits.view(np.float16).astype(np.float32)
     field = (bits >> 10) & 31
-    normal = (field >= 1) & (field <= 30)
-    want = bits.view(np.float16).astype(np.float32)
-    assert np.array_equal(got[normal].view(np.uint32), want[normal].view(np.uint32))
-    assert normal.sum() == 2 * 30 * 1024
+    same = got.view(np.uint32) == ieee.view(np.uint32)
+    assert np.array_equal(same, ((field >= 1) & (field <= 30) & ((bits & 0x03F8) == 0)) | ((bits & 0x7FFF) == 0x0200))
+    assert same.sum() == 2 * 30 * 8 + 2
 
 
-def test_f16_mm_outside_the_normal_range_unpinned(oracle):
-    # closed form of what the reference's bit arithmetic yields there: 2^(field - 15) * (1 + m / 1024)
+def test_f16_mm_hand_values(oracle):
     L = oracle.lib()
-    for bits in (0x0000, 0x8000, 0x0001, 0x03FF, 0x83FF, 0x7C00, 0xFC00, 0x7E00, 0x7FFF):
-        field, m, sign = (bits >> 10) & 31, bits & 0x3FF, -1.0 if bits & 0x8000 else 1.0
-        want = sign * 2.0 ** (field - 15) * (1.0 + m / 1024.0)
-        assert L.rf_f16_to_f32_mm(bits) == np.float32(want), hex(bits)
+    assert L.rf_f16_to_f32_mm(0x3C00) == np.float32(1.0)               # the powers of two the reference's tests use
+    assert L.rf_f16_to_f32_mm(0x4000) == np.float32(2.0)
+    assert L.rf_f16_to_f32_mm(0x3E00) == np.float32(1.0)               # IEEE 1.5: mantissa bit 9 is shifted out
+    assert L.rf_f16_to_f32_mm(0x2E66) == np.float32(0.0625 * (1.0 + 6.0 / 1024.0))   # IEEE 0.1 -> 0.062866...
+    assert abs(L.rf_f16_to_f32_mm(0x2E66) - 0.0628662109375) == 0.0
+    assert L.rf_f16_to_f32_mm(0xC007) == np.float32(-2.0 * (1.0 + 7.0 / 1024.0))
     assert L.rf_f16_to_f32_mm(0) == np.float32(2.0 ** -15)             # not 0.0: the zero branch is dead code
+    assert L.rf_f16_to_f32_mm(0x8000) == np.float32(-(2.0 ** -15))
+    assert L.rf_f16_to_f32_mm(0x7C00) == np.float32(65536.0)           # not inf
+    assert L.rf_f16_to_f32_mm(0x03FF) == np.float32(2.0 ** -15 * (1.0 + 7.0 / 1024.0))
 
 
 def test_mm_q8_0_reference_vector(oracle):
@@ -102,10 +123,16 @@ def test_mm_q4_k_numpy_statement(oracle):
 
 
 def test_mm_q4_k_agrees_with_the_canonical_decoder_where_it_must(oracle):
-    # sub-block 0 reads bytes 32..47 under either stride; with normal scales both widenings are exact
+    # sub-block 0 reads bytes 32..47 under either stride; both widenings agree on normal scales with mantissa bits 3..9 clear
     rng = np.random.default_rng(13)
     nb = 64
-    blocks = Q.synth_q4_k(nb, rng)
+    full = Q.synth_q4_k(nb, rng)
+    blocks = full.reshape(nb, 256).copy()
+    blocks[:, 0:16] = (blocks[:, 0:16].copy().view("<u2") & np.uint16(0xFC07)).view(np.uint8)
+    blocks = blocks.ravel()
+    # with the generator's own scales (all ten mantissa bits in use) even sub-block 0 differs
+    assert not np.array_equal(oracle.dequantize(MM_Q4_K, full, nb * 256).reshape(nb, 8, 32)[:, 0],
+                              oracle.dequantize(Q.Q4_K, full, nb * 256).reshape(nb, 8, 32)[:, 0])
     a = oracle.dequantize(MM_Q4_K, blocks, nb * 256).reshape(nb, 8, 32)
     b = oracle.dequantize(Q.Q4_K, blocks, nb * 256).reshape(nb, 8, 32)
     assert np.array_equal(a[:, 0].view(np.uint32), b[:, 0].view(np.uint32))
@@ -119,20 +146,35 @@ def test_mm_q4_k_agrees_with_the_canonical_decoder_where_it_must(oracle):
     assert np.array_equal(c.view(np.uint32), b.view(np.uint32))
 
 
-def test_mm_q6_k_is_the_canonical_decoder_for_normal_scales(oracle):
+def test_mm_q6_k_is_the_canonical_decoder_where_the_widenings_agree(oracle):
     rng = np.random.default_rng(14)
     w = (rng.standard_normal((8, 1024)) * 0.02).astype(np.float32)
-    blocks = Q.quantize_q6_k(w, rng)
+    full = Q.quantize_q6_k(w, rng)
+    nb = w.size // 256
+    blocks = full.reshape(nb, 256).copy()
+    blocks[:, 0:32] = (blocks[:, 0:32].copy().view("<u2") & np.uint16(0xFC07)).view(np.uint8)
+    blocks = blocks.ravel()
     a = oracle.dequantize(MM_Q6_K, blocks, w.size)
     b = oracle.dequantize(Q.Q6_K, blocks, w.size)
     assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
-    # a subnormal scale: the canonical decoder widens it exactly, this one reads 2^-15 * (1 + m / 1024)
-    blk = blocks[:256].copy()
-    blk[0:2] = np.array([0x0200], "<u2").view(np.uint8)
+    # a real quantiser's scales use every mantissa bit: there this decoder returns other numbers
+    a, b = oracle.dequantize(MM_Q6_K, full, w.size), oracle.dequantize(Q.Q6_K, full, w.size)
+    assert not np.array_equal(a, b)
+    scale = mm_f16_numpy(full.reshape(nb, 256)[:, 0:32].copy().view("<u2"))          # [nb, 16]
+    codes = np.where(b.reshape(nb, 16, 16) != 0, 1, 0)                                # same zero pattern: the codes are shared
+    assert np.array_equal(np.where(a.reshape(nb, 16, 16) != 0, 1, 0), codes)
+    ieee = full.reshape(nb, 256)[:, 0:32].copy().view("<f2").astype(np.float32)
+    ratio = (scale / ieee)[:, :, None]                                                # this widening never exceeds IEEE's
+    assert np.all(ratio <= 1.0) and np.all(ratio > 0.5)
+    assert np.allclose(a.reshape(nb, 16, 16), b.reshape(nb, 16, 16) * ratio, rtol=1e-6, atol=0)
+    # a subnormal scale: the canonical decoder widens 0x0201 to 513 * 2^-24, this one reads 2^-15 * (1 + 1 / 1024)
+    blk = full[:256].copy()
+    blk[0:2] = np.array([0x0201], "<u2").view(np.uint8)
     a, b = oracle.dequantize(MM_Q6_K, blk, 256), oracle.dequantize(Q.Q6_K, blk, 256)
-    # 0x0200 is the subnormal 2^-15; this decoder reads 2^-15 * (1 + 512 / 1024): every value 1.5 times larger
-    assert np.any(b[:16] != 0) and np.array_equal(a[:16], b[:16] * np.float32(1.5))
-    assert np.array_equal(a[16:], b[16:])
+    nz = b[:16] != 0
+    assert nz.any()
+    q = (b[:16] / np.float32(513 * 2.0 ** -24)).astype(np.float32)                    # the signed codes
+    assert np.array_equal(a[:16], (q * np.float32(2.0 ** -15 * (1 + 1 / 1024))).astype(np.float32))
 
 
 # The loops of the three decoders, element by element, with the Rust's early exits.
