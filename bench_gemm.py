@@ -117,6 +117,42 @@ def kq_gemm(torch, fmt, m=512, n=14336, k=4096, steps=300, warmup=300, arranged=
     return res
 
 
+def mfma_probe(torch, only_variant=None):
+    """What the fp16 matrix pipe delivers alone and beside a fused kernel's operand traffic (rfq_bench_mfma_f16_probe):
+    instruction shape x (VALU, LDS fragment reads, global fragment loads per round) x workgroups x wavefronts per SIMD x
+    operand data, each launched for about 20 ms before the timed launch."""
+    import ctypes as C
+    from rocmforge_amd import _lib
+    L = _lib.lib()
+    torch.zeros(1, device="cuda")
+    rows = []
+    mixes = {0: [(0, 0, 0), (2, 0, 0), (4, 0, 0), (0, 4, 0), (0, 8, 0), (0, 0, 2), (0, 0, 4), (0, 4, 2), (2, 4, 2), (3, 4, 2), (3, 6, 0)],
+             1: [(0, 0, 0), (1, 0, 0), (2, 0, 0), (0, 7, 0), (0, 0, 4), (0, 7, 4), (1, 7, 4), (2, 7, 4)]}
+    if only_variant is not None:
+        mixes = {only_variant: mixes[only_variant]}
+    for variant, name in ((0, "32x32x16_f16"), (1, "16x16x32_f16")):
+        for valu, ldsr, gld in mixes.get(variant, []):
+            for wgs, waves in ((128, 4), (224, 4), (256, 4), (224, 8), (256, 8)):
+                for rnd in (1, 0):
+                    if (not rnd) and (valu or ldsr or gld or wgs != 256):
+                        continue
+                    if wgs == 128 and (valu or ldsr or gld):
+                        continue
+                    us, cpm, ghz, tf = C.c_float(), C.c_float(), C.c_float(), C.c_float()
+                    iters = (4000 if variant == 0 else 2288) // (waves // 4)     # about 0.5 ms per launch
+                    _lib.check(L.rfq_bench_mfma_f16_probe(variant, valu, ldsr, gld, wgs, waves, rnd, iters, 30, None,
+                                                          C.byref(us), C.byref(cpm), C.byref(ghz), C.byref(tf)))
+                    rows.append({"instruction": name, "valu_per_mfma": valu, "lds_reads_per_round": ldsr, "global_loads_per_round": gld,
+                                 "workgroups": wgs, "waves_per_simd": waves // 4, "operands": "random" if rnd else "zero",
+                                 "launch_us": round(us.value, 1),
+                                 "clocks_per_mfma_and_simd": round(us.value * ghz.value * 1e3 / (iters * (8 if variant == 0 else 28) * (waves // 4)), 2),
+                                 "clocks_per_mfma_in_loop": round(cpm.value, 2),
+                                 "shader_ghz": round(ghz.value, 3), "tflops": round(tf.value, 1),
+                                 "frac_of_2500": round(tf.value / 2500.0, 3)})
+                    print(json.dumps(rows[-1]), flush=True)
+    return rows
+
+
 def run(torch):
     from rocmforge_amd import quantize as Q
     res = {}
@@ -137,11 +173,15 @@ if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--only", choices=["mxfp4", "mxfp6", "q4_k", "gguf_q4_k"], help="one configuration (for profiling runs)")
     ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--probe-mfma", action="store_true", help="the fp16 matrix pipe alone and beside a fused kernel's operand traffic")
+    ap.add_argument("--probe-variant", type=int, choices=[0, 1], help="only v_mfma_f32_32x32x16_f16 (0) or v_mfma_f32_16x16x32_f16 (1)")
     ap.add_argument("--data", choices=["packer", "window"], default="packer", help="MXFP4 operands: the reference packer's, or full-entropy")
     a = ap.parse_args()
     import torch
     from rocmforge_amd import quantize as Q
-    if a.only in ("q4_k", "gguf_q4_k"):
+    if a.probe_mfma:
+        mfma_probe(torch, a.probe_variant)
+    elif a.only in ("q4_k", "gguf_q4_k"):
         print(json.dumps(kq_gemm(torch, Q.Q4_K if a.only == "q4_k" else Q.GGUF_Q4_K, steps=a.steps, arranged=True)))
     elif a.only:
         print(json.dumps(mx_gemm(torch, Q.MXFP4 if a.only == "mxfp4" else Q.MXFP6_E2M3, steps=a.steps, data=a.data)))

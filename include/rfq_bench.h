@@ -78,6 +78,20 @@ RFQ_API int rfq_bench_mlp_swiglu(int fmt_gate_up, const void *const *d_gate_copi
                                  void *d_scratch, size_t scratch_bytes, int one_call, int warmup, int steps,
                                  void *stream, float *elapsed_ms);
 
+/* What the fp16 matrix pipe delivers, alone and beside the operand traffic of a fused kernel (the ceiling
+ * rfq_gemm_f16 is held against): `workgroups` x `waves_per_workgroup` (4 or 8; one workgroup per CU) wavefronts each
+ * run iters (even) rounds of independent matrix instructions -- variant 0: 8 x v_mfma_f32_32x32x16_f16 per round, 1:
+ * 28 x v_mfma_f32_16x16x32_f16 -- plus, per round, valu_per_mfma packed fp16 multiplies per matrix instruction,
+ * lds_reads_per_round 16-byte-per-lane fragment reads from LDS and global_loads_per_round 16-byte-per-lane loads from
+ * a 2 MiB window in global memory (cache hits); loaded fragments are the next round's operands.  Only some
+ * combinations are compiled (RFQ_E_UNSUPPORTED otherwise).  The kernel is launched `launches` times back to back; the
+ * last launch is timed, and the shader clocks each wavefront counted around its loop (s_memtime, against the constant
+ * 100 MHz clock) give clocks per instruction and SIMD and the clock the part held. */
+RFQ_API int rfq_bench_mfma_f16_probe(int variant, int valu_per_mfma, int lds_reads_per_round, int global_loads_per_round,
+                                     int workgroups, int waves_per_workgroup, int random_operands, int iters,
+                                     int launches, void *stream, float *last_launch_us, float *clocks_per_mfma,
+                                     float *shader_ghz, float *tflops);
+
 #ifdef __cplusplus
 }
 #endif

@@ -74,6 +74,8 @@ _SIGNATURES = {
     "rfq_bench_get_rows": ([_i, _vp, _sz, _i, _i, _vp, _i, _vp, _i, _i, _i, _vp, C.POINTER(C.c_float)], _i),
     "rfq_bench_gemm_f16_arranged": ([_i, _vp, _sz, _vp, _sz, _vp, _i, _i, _i, _i, _i, _i, _vp, C.POINTER(C.c_float)], _i),
     "rfq_bench_gemm_mx": ([_vp, _sz, _i, _vp, _sz, _i, _vp, _i, _i, _i, _i, _i, _i, _vp, C.POINTER(C.c_float)], _i),
+    "rfq_bench_mfma_f16_probe": ([_i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, C.POINTER(C.c_float), C.POINTER(C.c_float),
+                                  C.POINTER(C.c_float), C.POINTER(C.c_float)], _i),
 }
 
 

@@ -1,6 +1,9 @@
 // Native timing loops for the benchmark driver (see include/rfq_bench.h).
 #include "rfq_bench.h"
 
+#include <type_traits>
+#include <vector>
+
 #include "rfq_common.hpp"
 
 namespace {
@@ -58,6 +61,85 @@ read_floor_kernel(const uint8_t *__restrict__ p, size_t n16, uint32_t never, uin
         for (int d = 0; d < D; d++) acc += (v[d][0] ^ v[d][1]) + (v[d][2] ^ v[d][3]);
     }
     if (acc == never && never != 0) sink[t & 63] = acc;
+}
+
+// What the fp16 matrix pipe delivers, alone and beside the operand traffic of a fused kernel.  Every wavefront runs
+// `iters` rounds of NACC independent matrix instructions (VARIANT 0: v_mfma_f32_32x32x16_f16, 8 per round; 1:
+// v_mfma_f32_16x16x32_f16, 28 per round); per round it also issues VALU * NACC packed fp16 multiplies (standing for a
+// fused kernel's decode work), LDSR 16-byte-per-lane fragment reads from LDS and GLD 16-byte-per-lane loads from a 2 MiB
+// window of global memory that all workgroups share (cache hits).  What a round loads feeds the next round's matrix
+// instructions, as in a software-pipelined GEMM.  Lane 0 of every wavefront records the shader clock (s_memtime) and
+// the constant 100 MHz clock (s_memrealtime) around its loop.  The kernel's LDS request keeps it to one workgroup per CU.
+typedef _Float16 probe_v8h __attribute__((ext_vector_type(8)));
+typedef _Float16 probe_v2h __attribute__((ext_vector_type(2)));
+typedef float probe_v16f __attribute__((ext_vector_type(16)));
+typedef float probe_v4f __attribute__((ext_vector_type(4)));
+constexpr int PROBE_LDS_BYTES = 96 * 1024, PROBE_WINDOW_BYTES = 2 << 20;
+
+template <int VARIANT, int VALU, int LDSR, int GLD>
+__global__ void __launch_bounds__(512)
+mfma_f16_probe_kernel(const probe_v8h *__restrict__ in, const probe_v8h *__restrict__ window, float *__restrict__ out,
+                      unsigned long long *__restrict__ clocks, int iters)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t probe_lds[];
+    constexpr int NACC = VARIANT == 0 ? 8 : 28, NA = GLD > 0 ? GLD : 1, NB = LDSR > 0 ? LDSR : 1;
+    typedef typename std::conditional<VARIANT == 0, probe_v16f, probe_v4f>::type Acc;
+    constexpr int NR = VARIANT == 0 ? 16 : 4;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    probe_v8h *lds = reinterpret_cast<probe_v8h *>(probe_lds);
+    for (int i = threadIdx.x; i < 64 * 1024 / 16; i += blockDim.x) lds[i] = in[i & 1023];
+    __syncthreads();
+    probe_v8h a[2][NA], b[2][NB];
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+#pragma unroll
+        for (int g = 0; g < NA; g++) a[h][g] = in[(threadIdx.x + 64 * g) & 1023];
+#pragma unroll
+        for (int r = 0; r < NB; r++) b[h][r] = in[(512 + threadIdx.x + 64 * r) & 1023];
+    }
+    probe_v2h t[4];
+#pragma unroll
+    for (int q = 0; q < 4; q++) t[q] = probe_v2h{a[0][0][2 * q], b[0][0][2 * q + 1]};
+    const probe_v2h one = {in[1023][0], in[1023][1]};                 // 1.0 from memory: a constant would be folded away
+    Acc acc[NACC];
+#pragma unroll
+    for (int q = 0; q < NACC; q++)
+#pragma unroll
+        for (int r = 0; r < NR; r++) acc[q][r] = 0.0f;
+    auto round = [&](int it, int cur) __attribute__((always_inline)) {
+        const int nxt = cur ^ 1;
+#pragma unroll
+        for (int g = 0; g < GLD; g++)
+            a[nxt][g] = window[((((it * GLD + g) * 8 + wave) * 64) & (PROBE_WINDOW_BYTES / 16 - 1)) + lane];
+#pragma unroll
+        for (int r = 0; r < LDSR; r++) b[nxt][r] = lds[((((it * LDSR + r) * 8 + wave) * 64) & (64 * 1024 / 16 - 1)) + lane];
+#pragma unroll
+        for (int q = 0; q < NACC; q++) {
+            if constexpr (VARIANT == 0) acc[q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[cur][q % NA], b[cur][q % NB], acc[q], 0, 0, 0);
+            else acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[cur][q % NA], b[cur][q % NB], acc[q], 0, 0, 0);
+#pragma unroll
+            for (int v = 0; v < VALU; v++) t[(q + v) & 3] = t[(q + v) & 3] * one;
+        }
+    };
+    const unsigned long long c0 = __builtin_readcyclecounter(), r0 = __builtin_amdgcn_s_memrealtime();
+    for (int it = 0; it < iters; it += 2) {
+        round(it, 0);
+        round(it + 1, 1);
+    }
+    const unsigned long long c1 = __builtin_readcyclecounter(), r1 = __builtin_amdgcn_s_memrealtime();
+    float s = 0.0f;
+#pragma unroll
+    for (int q = 0; q < NACC; q++)
+#pragma unroll
+        for (int r = 0; r < NR; r++) s += acc[q][r];
+#pragma unroll
+    for (int q = 0; q < 4; q++) s += (float)t[q][0] + (float)t[q][1];
+    out[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = s;
+    if (lane == 0) {
+        const size_t w = (size_t)blockIdx.x * (blockDim.x / 64) + wave;
+        clocks[2 * w] = c1 - c0;
+        clocks[2 * w + 1] = r1 - r0;
+    }
 }
 
 } // namespace
@@ -192,6 +274,83 @@ int rfq_bench_mlp_swiglu(int fmt_gate_up, const void *const *d_gate_copies, cons
         if (rc == RFQ_OK) rc = rfq_gemv(fmt_down, d_down_copies[c], down_bytes, h, d_out, m, hidden_size, intermediate_size, stream);
         return rc;
     });
+}
+
+int rfq_bench_mfma_f16_probe(int variant, int valu_per_mfma, int lds_reads_per_round, int global_loads_per_round,
+                             int workgroups, int waves_per_workgroup, int random_operands, int iters, int launches,
+                             void *stream, float *last_launch_us, float *clocks_per_mfma, float *shader_ghz, float *tflops)
+{
+    using namespace rfq;
+    if ((variant != 0 && variant != 1) || workgroups <= 0 || workgroups > 4096 ||
+        (waves_per_workgroup != 4 && waves_per_workgroup != 8) || iters <= 0 || iters % 2 != 0 || launches <= 0 ||
+        !last_launch_us || !clocks_per_mfma || !shader_ghz || !tflops)
+        return fail(RFQ_E_BADARG, "rfq_bench_mfma_f16_probe: bad arguments");
+    hipStream_t s = (hipStream_t)stream;
+    const int threads = 64 * waves_per_workgroup, waves = workgroups * waves_per_workgroup;
+    const int nacc = variant == 0 ? 8 : 28;
+    std::vector<uint16_t> host(PROBE_WINDOW_BYTES / 2);
+    uint32_t lcg = 12345u;
+    for (auto &h : host) {
+        lcg = lcg * 1664525u + 1013904223u;
+        // random fp16 values of magnitude 2^-4 .. 2 with random mantissas and signs, or all zero
+        h = random_operands ? (uint16_t)(((lcg >> 16) & 0x83FFu) | ((11u + ((lcg >> 8) % 5u)) << 10)) : (uint16_t)0;
+    }
+    std::vector<uint16_t> first(host.begin(), host.begin() + 1024 * 8);
+    first[1023 * 8] = first[1023 * 8 + 1] = 0x3C00;
+    void *d_in = nullptr, *d_win = nullptr, *d_out = nullptr, *d_clk = nullptr;
+    RFQ_HIP(hipMalloc(&d_in, first.size() * 2));
+    RFQ_HIP(hipMalloc(&d_win, host.size() * 2));
+    RFQ_HIP(hipMalloc(&d_out, (size_t)workgroups * threads * 4));
+    RFQ_HIP(hipMalloc(&d_clk, (size_t)waves * 16));
+    RFQ_HIP(hipMemcpy(d_in, first.data(), first.size() * 2, hipMemcpyHostToDevice));
+    RFQ_HIP(hipMemcpy(d_win, host.data(), host.size() * 2, hipMemcpyHostToDevice));
+    const void *fn = nullptr;
+#define RFQ_PROBE_CASE(V, VA, L, G) \
+    if (variant == V && valu_per_mfma == VA && lds_reads_per_round == L && global_loads_per_round == G) \
+        fn = reinterpret_cast<const void *>(&mfma_f16_probe_kernel<V, VA, L, G>);
+    RFQ_PROBE_CASE(0, 0, 0, 0) RFQ_PROBE_CASE(0, 2, 0, 0) RFQ_PROBE_CASE(0, 4, 0, 0) RFQ_PROBE_CASE(0, 0, 4, 0)
+    RFQ_PROBE_CASE(0, 0, 8, 0) RFQ_PROBE_CASE(0, 0, 0, 2) RFQ_PROBE_CASE(0, 0, 0, 4) RFQ_PROBE_CASE(0, 0, 4, 2)
+    RFQ_PROBE_CASE(0, 3, 4, 2) RFQ_PROBE_CASE(0, 2, 4, 2) RFQ_PROBE_CASE(0, 3, 6, 0)
+    RFQ_PROBE_CASE(1, 0, 0, 0) RFQ_PROBE_CASE(1, 2, 0, 0) RFQ_PROBE_CASE(1, 1, 0, 0) RFQ_PROBE_CASE(1, 0, 7, 4) RFQ_PROBE_CASE(1, 1, 7, 4)
+    RFQ_PROBE_CASE(1, 2, 7, 4) RFQ_PROBE_CASE(1, 0, 7, 0) RFQ_PROBE_CASE(1, 0, 0, 4)
+#undef RFQ_PROBE_CASE
+    if (!fn) return fail(RFQ_E_UNSUPPORTED, "rfq_bench_mfma_f16_probe: combination not compiled");
+    RFQ_HIP(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, PROBE_LDS_BYTES));
+    hipEvent_t e0, e1;
+    RFQ_HIP(hipEventCreate(&e0));
+    RFQ_HIP(hipEventCreate(&e1));
+    const void *in = d_in, *win = d_win;
+    float *out = static_cast<float *>(d_out);
+    unsigned long long *clk = static_cast<unsigned long long *>(d_clk);
+    void *args[] = {(void *)&in, (void *)&win, (void *)&out, (void *)&clk, (void *)&iters};
+    for (int i = 0; i < launches; i++) {
+        if (i == launches - 1) RFQ_HIP(hipEventRecord(e0, s));
+        RFQ_HIP(hipLaunchKernel(fn, dim3(workgroups), dim3(threads), args, PROBE_LDS_BYTES, s));
+    }
+    RFQ_HIP(hipEventRecord(e1, s));
+    RFQ_HIP(hipEventSynchronize(e1));
+    float ms = 0.0f;
+    RFQ_HIP(hipEventElapsedTime(&ms, e0, e1));
+    std::vector<unsigned long long> ticks((size_t)waves * 2);
+    RFQ_HIP(hipMemcpy(ticks.data(), d_clk, ticks.size() * 8, hipMemcpyDeviceToHost));
+    double core = 0.0, real = 0.0;
+    for (int w = 0; w < waves; w++) {
+        core += (double)ticks[2 * w];
+        real += (double)ticks[2 * w + 1];
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    (void)hipFree(d_in);
+    (void)hipFree(d_win);
+    (void)hipFree(d_out);
+    (void)hipFree(d_clk);
+    const double per_wave = (double)iters * nacc;
+    *last_launch_us = ms * 1000.0f;
+    // clocks per matrix instruction and SIMD: a SIMD's wavefronts share its matrix pipe
+    *clocks_per_mfma = (float)(core / waves / per_wave / (waves_per_workgroup / 4));
+    *shader_ghz = real > 0.0 ? (float)(core / real * 0.1) : 0.0f;               // the constant clock ticks at 100 MHz
+    *tflops = (float)(per_wave * waves * (variant == 0 ? 32768.0 : 16384.0) / (ms * 1e-3) / 1e12);
+    return RFQ_OK;
 }
 
 } // extern "C"
