@@ -87,8 +87,9 @@ def mx_gemm(torch, w_fmt, m=2048, n=28672, k=8192, steps=200, warmup=40, data="p
     return res
 
 
-def kq_gemm(torch, fmt, m=512, n=14336, k=4096, steps=300, warmup=300, arranged=False):
-    """Q4_K / Q6_K prefill GEMM on the fp16 matrix cores, fp16 in and out."""
+def kq_gemm(torch, fmt, m=512, n=14336, k=4096, steps=300, warmup=300, arranged=False, one_plane=False):
+    """Q4_K / Q6_K prefill GEMM on the fp16 matrix cores, fp16 in and out.  one_plane: RFQ_GEMM_ONE_PLANE (every weight
+    as one fp16 operand) beside the default two (hi + lo)."""
     from rocmforge_amd import _lib, quantize as Q
     dev = torch.device("cuda:0")
     w = torch.from_numpy(Q.make_weights(fmt, n, k, seed=20260004)).to(dev)
@@ -103,7 +104,15 @@ def kq_gemm(torch, fmt, m=512, n=14336, k=4096, steps=300, warmup=300, arranged=
     t = ms.value / 1e3 / steps
     flops = 2.0 * m * n * k
     res = {"TFLOP/s": round(flops / t / 1e12, 1), "us": round(t * 1e6, 1), "mfma_frac": round(flops / t / 2.5e15, 4),
-           "peak_TFLOP/s": 2500.0, "warmup_launches": warmup, "timed_launches": steps}
+           "peak_TFLOP/s": 2500.0, "warmup_launches": warmup, "timed_launches": steps,
+           "fp16_operands_per_weight": 1 if fmt == Q.Q4_K else 2}
+    if one_plane and fmt != Q.Q4_K:
+        args1 = args[:5] + (_lib.F16 | _lib.GEMM_ONE_PLANE,) + args[6:]
+        _lib.check(L.rfq_bench_gemm_f16(*args1, warmup, steps, stream, C.byref(ms)))
+        t1 = ms.value / 1e3 / steps
+        res["one_fp16_operand_per_weight"] = {"us": round(t1 * 1e6, 1), "TFLOP/s": round(flops / t1 / 1e12, 1),
+                                              "mfma_frac": round(flops / t1 / 2.5e15, 4),
+                                              "what": "RFQ_GEMM_ONE_PLANE: weights rounded once to fp16 (8e-4 of rms(out) from the reference)"}
     if arranged:
         # the same GEMM on activations arranged once (the second and third projection of one input)
         from rocmforge_amd import ops
@@ -157,9 +166,9 @@ def run(torch):
     from rocmforge_amd import quantize as Q
     res = {}
     res["Q4_K gemm 512x4096x14336 fp16"] = kq_gemm(torch, Q.Q4_K, arranged=True)
-    res["Q6_K gemm 512x4096x14336 fp16"] = kq_gemm(torch, Q.Q6_K)
-    res["GGUF_Q4_K gemm 512x4096x14336 fp16"] = kq_gemm(torch, Q.GGUF_Q4_K)
-    res["GGUF_Q6_K gemm 512x4096x14336 fp16"] = kq_gemm(torch, Q.GGUF_Q6_K)
+    res["Q6_K gemm 512x4096x14336 fp16"] = kq_gemm(torch, Q.Q6_K, one_plane=True)
+    res["GGUF_Q4_K gemm 512x4096x14336 fp16"] = kq_gemm(torch, Q.GGUF_Q4_K, one_plane=True)
+    res["GGUF_Q6_K gemm 512x4096x14336 fp16"] = kq_gemm(torch, Q.GGUF_Q6_K, one_plane=True)
     res["MXFP4 gemm 2048x8192x28672 bf16"] = mx_gemm(torch, Q.MXFP4)
     res["MXFP4 gemm 2048x8192x28672 bf16, full-entropy operands"] = mx_gemm(torch, Q.MXFP4, data="window")
     res["MXFP6-weight gemm 2048x8192x28672 bf16"] = mx_gemm(torch, Q.MXFP6_E2M3)

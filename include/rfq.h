@@ -32,7 +32,7 @@ extern "C" {
 
 /* Raised whenever an exported signature or the meaning of a format changes: a caller compares
  * rfq_version() with the RFQ_VERSION it was built against before its first call. */
-#define RFQ_VERSION 102 /* 0.1.2 */
+#define RFQ_VERSION 103 /* 0.1.3 */
 
 #if defined(_WIN32)
 #define RFQ_API
@@ -97,6 +97,10 @@ typedef enum rfq_status {
 } rfq_status;
 
 typedef enum rfq_dtype { RFQ_F32 = 0, RFQ_F16 = 1, RFQ_BF16 = 2 } rfq_dtype;
+/* Or-ed into the out_dtype of rfq_gemm_f16 / _static / _arranged: contract every decoded weight as ONE fp16
+ * operand (relative 2^-12 per weight) instead of two (see rfq_gemm_f16); about half the time, outside the
+ * 1e-3 tolerance on outputs that are small against the typical size. */
+#define RFQ_GEMM_ONE_PLANE 0x100
 
 /* Operand encodings of a prepared MXFP matrix (see rfq_mx_prepare). */
 typedef enum rfq_mx_kind { RFQ_MX_AUTO = 0, RFQ_MX_FP4 = 4, RFQ_MX_FP8 = 8, RFQ_MX_FP4_UNCHECKED = 0x104 } rfq_mx_kind;
@@ -306,9 +310,14 @@ RFQ_API int rfq_mlp_swiglu(int fmt_gate_up, const void *d_gate_w, const void *d_
 /* ---- prefill GEMM ----------------------------------------------------------- */
 
 /* d_out[m, n] = d_a[m, k] (fp16) . dequant(W)[n, k]^T on the fp16 matrix
- * cores with fp32 accumulation; out_dtype is RFQ_F32 or RFQ_F16.  Formats:
- * Q4_0, Q8_0, Q4_K, Q6_K and the four GGUF file layouts (weights decoded to
- * f32 as the format defines and rounded once to fp16).  k a multiple of 256
+ * cores with fp32 accumulation; out_dtype is RFQ_F32 or RFQ_F16, optionally
+ * or-ed with RFQ_GEMM_ONE_PLANE.  Formats: Q4_0, Q8_0, Q4_K, Q6_K and the four
+ * GGUF file layouts.  Weights are decoded to f32 as the format defines and
+ * contracted as two fp16 operands, hi = fp16(v) and lo = fp16(v - hi) (v to
+ * 2^-22: the result is that of an fp32 contraction, 5e-6 of rms(out) from the
+ * reference's at 512 x 4096 x 14336); the 256-byte Q4_K layout, whose integer
+ * mins are contracted exactly and apart, takes q * scale as one operand.  With
+ * RFQ_GEMM_ONE_PLANE every format takes one (8e-4 of rms(out)).  k a multiple of 256
  * for the K-formats, of 32 otherwise; d_a_f16 16-byte aligned, d_w 4-byte aligned.  Up to 64 MiB of
  * temporary device memory (the activations in matrix-operand order) is kept
  * per stream between calls; larger temporaries are allocated and released in

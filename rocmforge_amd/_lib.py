@@ -10,6 +10,7 @@ _SO = os.path.join(_HERE, "librfq.so")
 
 OK, E_BADARG, E_SIZE, E_UNSUPPORTED, E_HIP, E_NOMEM = 0, -1, -2, -3, -4, -5
 F32, F16, BF16 = 0, 1, 2
+GEMM_ONE_PLANE = 0x100              # or-ed into rfq_gemm_f16's out_dtype: one fp16 operand per weight
 MX_AUTO, MX_FP4, MX_FP8, MX_FP4_UNCHECKED = 0, 4, 8, 0x104
 
 

@@ -415,7 +415,7 @@ int rfq_gemm_f16(int fmt, const void *d_w, size_t w_bytes, const void *d_a_f16, 
 {
     int rc = check_gemv("rfq_gemm_f16", fmt, d_w, w_bytes, true, d_a_f16, d_out, m, n, k);
     if (rc != RFQ_OK) return rc;
-    if (out_dtype != RFQ_F32 && out_dtype != RFQ_F16)
+    if ((out_dtype & ~RFQ_GEMM_ONE_PLANE) != RFQ_F32 && (out_dtype & ~RFQ_GEMM_ONE_PLANE) != RFQ_F16)
         return fail(RFQ_E_BADARG, "rfq_gemm_f16: out_dtype %d is neither F32 nor F16", out_dtype);
     return launch_gemm_f16(fmt, (const uint8_t *)d_w, d_a_f16, d_out, out_dtype, m, n, k, false, nullptr, (hipStream_t)stream);
 }
@@ -425,7 +425,7 @@ int rfq_gemm_f16_static(int fmt, const void *d_w, size_t w_bytes, const void *d_
 {
     int rc = check_gemv("rfq_gemm_f16_static", fmt, d_w, w_bytes, true, d_a_f16, d_out, m, n, k);
     if (rc != RFQ_OK) return rc;
-    if (out_dtype != RFQ_F32 && out_dtype != RFQ_F16)
+    if ((out_dtype & ~RFQ_GEMM_ONE_PLANE) != RFQ_F32 && (out_dtype & ~RFQ_GEMM_ONE_PLANE) != RFQ_F16)
         return fail(RFQ_E_BADARG, "rfq_gemm_f16_static: out_dtype %d is neither F32 nor F16", out_dtype);
     return launch_gemm_f16(fmt, (const uint8_t *)d_w, d_a_f16, d_out, out_dtype, m, n, k, true, nullptr, (hipStream_t)stream);
 }
@@ -448,7 +448,7 @@ int rfq_gemm_f16_arranged(int fmt, const void *d_w, size_t w_bytes, const void *
 {
     int rc = check_gemv("rfq_gemm_f16_arranged", fmt, d_w, w_bytes, true, d_arranged, d_out, m, n, k);
     if (rc != RFQ_OK) return rc;
-    if (out_dtype != RFQ_F32 && out_dtype != RFQ_F16)
+    if ((out_dtype & ~RFQ_GEMM_ONE_PLANE) != RFQ_F32 && (out_dtype & ~RFQ_GEMM_ONE_PLANE) != RFQ_F16)
         return fail(RFQ_E_BADARG, "rfq_gemm_f16_arranged: out_dtype %d is neither F32 nor F16", out_dtype);
     const size_t need = gemm_f16_arranged_bytes(m, k);
     if (need == 0 || arranged_bytes < need)

@@ -127,7 +127,10 @@ arrange_a_kernel(const _Float16 *__restrict__ a, v4u *__restrict__ at, _Float16 
     }
 }
 
-template <int FMT, bool OUT_F16>
+// PLANES = 2: every stage of k is walked twice, first with the weights' fp16 values (hi) and then with what the
+// rounding to fp16 left over (lo = fp16(v - hi)), as two consecutive stages of the same pipeline over the same
+// activations: the contraction then carries the weights to 2^-22 instead of 2^-12.
+template <int FMT, bool OUT_F16, int PLANES>
 __global__ void __launch_bounds__(256)
 gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const _Float16 *__restrict__ s2,
                void *__restrict__ outp, int M, int N, int K)
@@ -144,7 +147,8 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
     const int m0 = tm * BM, n0 = tn * BN;
     const int groups = K / 32;                                    // 32-element groups per row
     const size_t row_bytes = (size_t)(K / Fmt<FMT>::BE) * Fmt<FMT>::BB;
-    const int nstages = (K + BK - 1) / BK;
+    const int kstages = (K + BK - 1) / BK;                        // stages of k
+    const int nstages = kstages * PLANES;                         // stages the pipeline walks
 
     // Weights: thread t decodes group t%2 of row t/2 of each stage into LDS.
     const int wr = tid >> 1, wh = tid & 1;
@@ -170,7 +174,7 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
     for (int i = 0; i < TI; i++) {
         const int mt = m0 / 32 + wave_u * 2 + i;
         a_tile[i] = __builtin_amdgcn_make_buffer_rsrc(
-            const_cast<v4u *>(at + (size_t)(mt < tiles32 ? mt : tiles32 - 1) * nstages * 256), 0, nstages * 4096, 0x00020000);
+            const_cast<v4u *>(at + (size_t)(mt < tiles32 ? mt : tiles32 - 1) * kstages * 256), 0, kstages * 4096, 0x00020000);
     }
 
     // Global loads run three stages ahead of the arithmetic through a ring of
@@ -197,12 +201,12 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
     auto fetch_w = [&](auto slotc, int st) __attribute__((always_inline)) {
         // the last stage of a row with an odd number of groups has no second
         // group: both lanes of the row then read the first (zeroed when decoded)
-        const int sc = st < nstages ? st : nstages - 1;
+        const int sc = (st < nstages ? st : nstages - 1) / PLANES;
         const int whc = Fmt<FMT>::BE == 32 && sc * 2 + 1 >= groups ? 0 : wh;
         raw_of(slotc).load(w_tile, w_off, sc, whc);
     };
     auto fetch_a = [&](auto slotc, int st, int i, int c) __attribute__((always_inline)) {
-        const int sc = st < nstages ? st : nstages - 1;
+        const int sc = (st < nstages ? st : nstages - 1) / PLANES;
         ra_of(slotc)[i][c] = __builtin_amdgcn_raw_buffer_load_b128(a_tile[i], lane16 + c * 1024, sc * 4096, 0);
     };
     auto fetch_a_all = [&](auto slotc, int st) __attribute__((always_inline)) {
@@ -217,9 +221,10 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
         Raw32<FMT> &raw = raw_of(slotc);
         Raw32<FMT> z;
         z.zero();
-        raw.settle(wh, pair, decltype(slotc)::value);             // (group 2*stage + wh has the parity of wh; ring slot = stage % 4)
+        // (group 2*stage + wh has the parity of wh; with one plane the ring slot is the stage's number within its super-block)
+        raw.settle(wh, pair, PLANES == 1 ? decltype(slotc)::value : (st / PLANES) & 3);
 #pragma unroll
-        for (int i = 0; i < Raw32<FMT>::ND; i++) raw.d[i] = st * 2 + wh < groups ? raw.d[i] : z.d[i];
+        for (int i = 0; i < Raw32<FMT>::ND; i++) raw.d[i] = (st / PLANES) * 2 + wh < groups ? raw.d[i] : z.d[i];
     };
 
     // Four LDS buffers of decoded weights (buffer = stage % 4, a compile-time
@@ -375,8 +380,8 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
                     constexpr int LATE[6] = {0, 3, 5, 8, 10, 13}, EARLY[6] = {16, 18, 20, 22, 26, 29};
 #pragma unroll
                     for (int q = 0; q < 6; q++) {
-                        if (p == LATE[q]) raw_late.step(6 + q, hw_late, dec_tmp);
-                        if (p == EARLY[q]) raw_early.step(q, hw_early, dec_tmp);
+                        if (p == LATE[q]) raw_late.template step<(S2 % PLANES) != 0>(6 + q, hw_late, dec_tmp);
+                        if (p == EARLY[q]) raw_early.template step<(S3 % PLANES) != 0>(q, hw_early, dec_tmp);
                     }
                 }
                 if (p == 15) settle(IC<S3>{}, st + 3, S == 0 ? hsA[3] : hsB[S3]);   // stage st+3 is number S3 of its super-block
@@ -419,19 +424,19 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
         asm volatile("v_mov_b32 %0, %1" : "=v"(hmA) : "v"(hmA));
         settle(IC<0>{}, 0, hsA[0]);
 #pragma unroll
-        for (int T = 0; T < 12; T++) raw0.step(T, hw, dec_tmp);
+        for (int T = 0; T < 12; T++) raw0.template step<false>(T, hw, dec_tmp);
 #pragma unroll
         for (int c = 0; c < 4; c++) stash(0, c, hw);
         fetch_w(IC<0>{}, 4);
         settle(IC<1>{}, 1, hsA[1]);
 #pragma unroll
-        for (int T = 0; T < 12; T++) raw1.step(T, hw, dec_tmp);
+        for (int T = 0; T < 12; T++) raw1.template step<(1 % PLANES) != 0>(T, hw, dec_tmp);
 #pragma unroll
         for (int c = 0; c < 4; c++) stash(1, c, hw);
         fetch_w(IC<1>{}, 5);
         settle(IC<2>{}, 2, hsA[2]);
 #pragma unroll
-        for (int T = 0; T < 6; T++) raw2.step(T, hw_even, dec_tmp);
+        for (int T = 0; T < 6; T++) raw2.template step<false>(T, hw_even, dec_tmp);
         lds_barrier();
 #pragma unroll
         for (int j = 0; j < TJ; j++) fw[0][j] = read_frag(0, j, 0);
@@ -532,7 +537,7 @@ size_t arranged_at_bytes(int m, int k) { return (size_t)((m + 31) / 32) * ((k + 
 size_t arranged_s2_bytes(int m, int k) { return k % 256 == 0 ? (size_t)((m + 31) / 32) * (k / 256) * 1024 : 0; }
 
 // `arranged` != nullptr: the caller's buffer from launch_arrange_a (activations and sums); a is not read.
-template <int FMT, bool OUT_F16>
+template <int FMT, bool OUT_F16, int PLANES>
 int launch_cfg(const uint8_t *w, const void *a, void *out, int m, int n, int k, uint8_t *static_tmp, const uint8_t *arranged,
                hipStream_t s)
 {
@@ -541,7 +546,7 @@ int launch_cfg(const uint8_t *w, const void *a, void *out, int m, int n, int k, 
     static std::once_flag once;
     static hipError_t attr_err = hipSuccess;
     std::call_once(once, [] {
-        attr_err = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_kq_kernel<FMT, OUT_F16>),
+        attr_err = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_kq_kernel<FMT, OUT_F16, PLANES>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
     });
     if (attr_err != hipSuccess) return hip_fail(attr_err, "hipFuncSetAttribute(gemm_kq_kernel)");
@@ -549,7 +554,7 @@ int launch_cfg(const uint8_t *w, const void *a, void *out, int m, int n, int k, 
     if (arranged != nullptr) {
         const v4u *at = reinterpret_cast<const v4u *>(arranged);
         const _Float16 *s2 = reinterpret_cast<const _Float16 *>(arranged + arranged_at_bytes(m, k));
-        hipLaunchKernelGGL((gemm_kq_kernel<FMT, OUT_F16>), dim3(tiles), dim3(256), LDS, s, w, at, s2, out, m, n, k);
+        hipLaunchKernelGGL((gemm_kq_kernel<FMT, OUT_F16, PLANES>), dim3(tiles), dim3(256), LDS, s, w, at, s2, out, m, n, k);
         RFQ_LAUNCH_CHECK("gemm_kq_kernel");
         return RFQ_OK;
     }
@@ -570,7 +575,7 @@ int launch_cfg(const uint8_t *w, const void *a, void *out, int m, int n, int k, 
     _Float16 *s2 = reinterpret_cast<_Float16 *>(tmp + at_bytes);
     hipLaunchKernelGGL((arrange_a_kernel<FMT == RFQ_Q4_K>), dim3((unsigned)(tiles32 * ((nst + 3) / 4))), dim3(256), 0, s,
                        reinterpret_cast<const _Float16 *>(a), at, s2, m, k, tiles32, nst);
-    hipLaunchKernelGGL((gemm_kq_kernel<FMT, OUT_F16>), dim3(tiles), dim3(256), LDS, s, w, at, s2, out, m, n, k);
+    hipLaunchKernelGGL((gemm_kq_kernel<FMT, OUT_F16, PLANES>), dim3(tiles), dim3(256), LDS, s, w, at, s2, out, m, n, k);
     hipError_t launch_err = hipGetLastError();
     if (transient) {
         hipError_t free_err = hipFreeAsync(tmp, s);
@@ -584,8 +589,16 @@ template <int FMT>
 int launch_fmt(const uint8_t *w, const void *a, void *out, int out_dtype, int m, int n, int k, uint8_t *static_tmp,
                const uint8_t *arranged, hipStream_t s)
 {
-    return out_dtype == RFQ_F16 ? launch_cfg<FMT, true>(w, a, out, m, n, k, static_tmp, arranged, s)
-                                : launch_cfg<FMT, false>(w, a, out, m, n, k, static_tmp, arranged, s);
+    // The 256-byte Q4_K layout is contracted in one plane (its large part, the integer mins, is exact and q * scale is
+    // small beside it); every other format in two unless the caller asks for one.
+    const bool f16 = (out_dtype & ~RFQ_GEMM_ONE_PLANE) == RFQ_F16;
+    if constexpr (FMT != RFQ_Q4_K) {
+        if ((out_dtype & RFQ_GEMM_ONE_PLANE) == 0)
+            return f16 ? launch_cfg<FMT, true, 2>(w, a, out, m, n, k, static_tmp, arranged, s)
+                       : launch_cfg<FMT, false, 2>(w, a, out, m, n, k, static_tmp, arranged, s);
+    }
+    return f16 ? launch_cfg<FMT, true, 1>(w, a, out, m, n, k, static_tmp, arranged, s)
+               : launch_cfg<FMT, false, 1>(w, a, out, m, n, k, static_tmp, arranged, s);
 }
 
 // The address of this device's copy of `scratch`, resolved on the first call on each device.
@@ -740,7 +753,7 @@ int launch_gemm_f16(int fmt, const uint8_t *d_w, const void *d_a, void *d_out, i
     if (use_static_scratch) {
         if (int rc = static_scratch(&st)) return rc;
     }
-    if (out_dtype != RFQ_F16 && out_dtype != RFQ_F32)
+    if ((out_dtype & ~RFQ_GEMM_ONE_PLANE) != RFQ_F16 && (out_dtype & ~RFQ_GEMM_ONE_PLANE) != RFQ_F32)
         return fail(RFQ_E_BADARG, "rfq_gemm_f16: out_dtype %d (want RFQ_F32 or RFQ_F16)", out_dtype);
     if (d_arranged != nullptr) {
         if ((reinterpret_cast<uintptr_t>(d_arranged) & 15u) != 0 || k % 8 != 0)

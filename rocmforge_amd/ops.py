@@ -190,13 +190,14 @@ def mlp_swiglu(fmt_gate_up: int, gate_w: torch.Tensor, up_w: torch.Tensor, fmt_d
 
 
 def gemm_f16(fmt: int, w: torch.Tensor, a: torch.Tensor, n: int, k: int, out_dtype=torch.float16,
-             out: torch.Tensor | None = None) -> torch.Tensor:
-    """out[m, n] = a[m, k] (fp16) . dequant(W)[n, k]^T on the fp16 matrix cores."""
+             out: torch.Tensor | None = None, one_plane: bool = False) -> torch.Tensor:
+    """out[m, n] = a[m, k] (fp16) . dequant(W)[n, k]^T on the fp16 matrix cores.  one_plane: every weight as a single
+    fp16 operand (relative 2^-12 per weight, about half the time) instead of the pair hi + lo."""
     w = _dev_u8(w)
     if not (a.is_cuda and a.dtype == torch.float16 and a.is_contiguous() and a.dim() == 2 and a.shape[1] == k):
         raise ValueError(f"a must be a contiguous [m, {k}] float16 device tensor")
     m = a.shape[0]
-    code = {torch.float32: _lib.F32, torch.float16: _lib.F16}[out_dtype]
+    code = {torch.float32: _lib.F32, torch.float16: _lib.F16}[out_dtype] | (_lib.GEMM_ONE_PLANE if one_plane else 0)
     out = _out(out, (m, n), out_dtype, a)
     check(lib().rfq_gemm_f16(fmt, _ptr(w), w.numel(), _ptr(a), _ptr(out), code, m, n, k, _stream()))
     return out

@@ -28,6 +28,8 @@ pub const RFQ_MM_Q8_0: c_int = 208;
 pub const RFQ_MM_Q4_K: c_int = 212;
 pub const RFQ_MM_Q6_K: c_int = 214;
 pub const RFQ_TABLE_F32: c_int = 0;
+/// Or-ed into the `out_dtype` of `rfq_gemm_f16*`: one fp16 operand per weight instead of two.
+pub const RFQ_GEMM_ONE_PLANE: c_int = 0x100;
 
 // rfq_status
 pub const RFQ_OK: c_int = 0;
@@ -48,7 +50,7 @@ pub const RFQ_MX_FP4: c_int = 4;
 pub const RFQ_MX_FP8: c_int = 8;
 pub const RFQ_MX_FP4_UNCHECKED: c_int = 0x104;
 
-pub const RFQ_VERSION: c_int = 102;
+pub const RFQ_VERSION: c_int = 103;
 
 #[link(name = "rfq")]
 extern "C" {

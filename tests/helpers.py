@@ -20,16 +20,19 @@ def assert_bit_exact(got, want, what=""):
 # GEMV / GEMM tolerance: "max relative error 1e-3 with fp32 accumulation".  Three figures are computed:
 #   rel_err        max_j |y_j - ref_j| / max(|ref_j|, rms(ref)): plain relative error wherever the reference is
 #                  at least of typical size, relative to the typical size for outputs near zero;
-#   rel_err_plain  max_j |y_j - ref_j| / |ref_j| over the outputs with |ref_j| > rms(ref) / 10.  Reported, not gated:
-#                  the error of an output does not shrink with the output (it is a sum of k rounding errors whose
-#                  size follows rms(ref)), so an output ten times below typical size carries ten times the ratio;
+#   rel_err_plain  max_j |y_j - ref_j| / |ref_j| over the outputs with |ref_j| > rms(ref) / 10: the plain relative
+#                  error of every output that is not small against the typical size (the error of an output does
+#                  not shrink with the output -- it is a sum of k rounding errors whose size follows rms(ref) -- so
+#                  an output ten times below typical size carries ten times the ratio);
 #   rel_err_floor  max_j |y_j - ref_j| / max(|ref_j|, 1e-3 * rms(ref)): the same ratio with a floor a thousand
 #                  times lower.  Reported, not gated: among 10^4 outputs the smallest |ref_j| are about
 #                  1e-4 * rms, and there two fp32 summation orders of the SAME products already differ by several
 #                  1e-3 under this figure (the reference's own sequential fp32 sum is about sqrt(k) * 2^-24 * rms
 #                  away from the exact sum; tests/test_oracle_kat.py::test_tolerance_floor_of_fp32_summation
 #                  measures it), so it cannot tell a correct kernel from a wrong one.
-# A result passes when rel_err <= 1e-3.
+# A result passes when rel_err <= 1e-3 and rel_err_plain <= 1e-3.  (One kernel is exempt from the second figure at
+# short k and says so where it is tested: the fp16 GEMM over the 256-byte Q4_K layout, which contracts q * scale as a
+# single fp16 operand.)
 REL_TOL = 1e-3
 
 
@@ -69,7 +72,12 @@ def error_report(got, ref):
             f"{rel_err_floor(got, ref):.2e} (floor 1e-3 rms, reported only)")
 
 
-def assert_close(got, ref, what="", tol=REL_TOL):
+def assert_close(got, ref, what="", tol=REL_TOL, plain_tol="same"):
     e = rel_err(got, ref)
     assert e <= tol, f"{what}: max relative error {e:.3e} > {tol:.1e}"
+    if plain_tol == "same":
+        plain_tol = tol
+    if plain_tol is not None:
+        p = rel_err_plain(got, ref)
+        assert p <= plain_tol, f"{what}: max plain relative error {p:.3e} > {plain_tol:.1e} (outputs with |ref| > rms / 10)"
     return e

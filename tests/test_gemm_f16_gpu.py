@@ -42,16 +42,19 @@ def gguf_q4_k_fused(w, n, k):
     return (d1 * q - m1).astype(np.float32).reshape(n, k)
 
 
-def rounded_weight_product(oracle, fmt, w, a, n, k):
-    """What the kernel is built to compute: the contraction of the weights rounded once to fp16 (float64 sums)."""
+def exact_weight_product(oracle, fmt, w, a, n, k):
+    """The contraction of the decoded f32 weights with the fp16 activations, float64 sums: what the two-plane kernel
+    is built to compute to 2^-22 per weight (hi = fp16(v), lo = fp16(v - hi))."""
     w32 = gguf_q4_k_fused(w, n, k) if fmt == Q.GGUF_Q4_K else oracle.dequantize(fmt, w, n * k).reshape(n, k)
-    return a.astype(np.float64) @ w32.astype(np.float16).astype(np.float64).T
+    return a.astype(np.float64) @ w32.astype(np.float64).T
 
 
-# The one rounding of each weight to fp16 (the matrix instruction's operand type) is the whole error budget:
-# about 2e-4 of rms(y) per output, random in sign, so the worst of 1e5 outputs lands near 1e-3.  Every case
-# below is inside 1e-3 except this one, whose CPU emulation of exactly that rounding gives the same 1.055e-3.
-ROUNDING_TAIL = {(Q.GGUF_Q6_K, 512, 259, 768): 1.1e-3}
+# The 256-byte Q4_K layout is contracted with q * scale as ONE fp16 operand (relative 2^-12 per weight) beside its exact
+# integer mins; at the size of config 4 its plain relative error is 4.9e-4, at short k it can pass 1e-3 on outputs a
+# tenth of the typical size, so for that format the small shapes are held to the first figure only.  Every other format
+# runs two planes and is held to both.
+def plain_tol_of(fmt, k):
+    return None if fmt == Q.Q4_K and k < 4096 else 1e-3
 
 
 def run(fmt, w, a, n, k, cuda, out_dtype):
@@ -69,12 +72,11 @@ def test_small_shapes_fp32_out(fmt, m, n, k, oracle, cuda):
     w, a = weights(fmt, n, k, 100 + fmt + m), acts(m, k, 200 + n)
     out = run(fmt, w, a, n, k, cuda, torch.float32).cpu().numpy()
     want = oracle.qmatmul_nk(fmt, w, a.astype(np.float32), m, n, k)
-    assert_close(out, want, f"{Q.NAMES[fmt]} {m}x{n}x{k}", tol=ROUNDING_TAIL.get((fmt, m, n, k), 1e-3))
-    # against the fp16-rounded weights only the fp32 summation order is left (the 256-byte Q4_K layout is
-    # not rounded as a whole: its integer mins are contracted apart from q * scale, so it sits closer to the oracle)
+    assert_close(out, want, f"{Q.NAMES[fmt]} {m}x{n}x{k}", plain_tol=plain_tol_of(fmt, k))
+    # against the float64 contraction of the same weights only the fp32 summation order is left
     if fmt != Q.Q4_K:
-        assert_close(out, rounded_weight_product(oracle, fmt, w, a, n, k), f"{Q.NAMES[fmt]} {m}x{n}x{k} (rounded weights)",
-                     tol=2e-5)
+        assert_close(out, exact_weight_product(oracle, fmt, w, a, n, k), f"{Q.NAMES[fmt]} {m}x{n}x{k} (float64 sums)", tol=2e-5,
+                     plain_tol=2e-4)
 
 
 @pytest.mark.parametrize("fmt", [Q.Q4_0, Q.Q8_0, Q.GGUF_Q4_0, Q.GGUF_Q8_0])
@@ -84,6 +86,7 @@ def test_k_not_a_multiple_of_the_stage(fmt, oracle, cuda):
     w, a = weights(fmt, n, k, 7), acts(m, k, 8)
     out = run(fmt, w, a, n, k, cuda, torch.float32).cpu().numpy()
     assert_close(out, oracle.qmatmul_nk(fmt, w, a.astype(np.float32), m, n, k), "k tail")
+    assert_close(out, exact_weight_product(oracle, fmt, w, a, n, k), "k tail (float64 sums)", tol=2e-5, plain_tol=2e-4)
 
 
 @pytest.mark.parametrize("fmt", FORMATS)
@@ -121,6 +124,25 @@ def test_full_size_sampled(fmt, oracle, cuda):
     assert_close(check, a.astype(np.float64) @ wsum, "row checksums", tol=1e-3)
 
 
+@pytest.mark.parametrize("fmt", [Q.Q6_K, Q.GGUF_Q4_K, Q.GGUF_Q6_K, Q.Q8_0])
+def test_one_plane_is_the_fp16_rounded_contraction(fmt, oracle, cuda):
+    """RFQ_GEMM_ONE_PLANE: every weight as one fp16 operand.  Pinned by the float64 contraction of the weights rounded
+    once to fp16; against the oracle its worst output lands at about 1e-3 of the typical output size (1.003e-3 for
+    Q6_K here), which is why it is not the default."""
+    import torch
+    from rocmforge_amd import ops
+    m, n, k = 300, 200, 512
+    w, a = weights(fmt, n, k, 41), acts(m, k, 42)
+    out = ops.gemm_f16(fmt, torch.from_numpy(w).to(cuda), torch.from_numpy(a).to(cuda), n, k, out_dtype=torch.float32,
+                       one_plane=True).cpu().numpy()
+    w32 = gguf_q4_k_fused(w, n, k) if fmt == Q.GGUF_Q4_K else oracle.dequantize(fmt, w, n * k).reshape(n, k)
+    rounded = a.astype(np.float64) @ w32.astype(np.float16).astype(np.float64).T
+    assert_close(out, rounded, "one plane (rounded weights)", tol=2e-5, plain_tol=2e-4)
+    assert_close(out, oracle.qmatmul_nk(fmt, w, a.astype(np.float32), m, n, k), "one plane", tol=1.5e-3, plain_tol=None)
+    two = ops.gemm_f16(fmt, torch.from_numpy(w).to(cuda), torch.from_numpy(a).to(cuda), n, k, out_dtype=torch.float32).cpu().numpy()
+    assert not np.array_equal(out, two)
+
+
 def test_weights_at_a_4_byte_offset_and_kept_temporary(oracle, cuda):
     """The weight loads need 4-byte alignment only; the per-stream temporary is
     reused by a smaller call after a larger one (and grown by a larger one)."""
@@ -134,7 +156,7 @@ def test_weights_at_a_4_byte_offset_and_kept_temporary(oracle, cuda):
         buf[4:] = torch.from_numpy(w).to(cuda)
         out = ops.gemm_f16(fmt, buf[4:], torch.from_numpy(a).to(cuda), n, k, out_dtype=torch.float32)
         torch.cuda.synchronize()
-        assert_close(out.cpu().numpy(), oracle.qmatmul_nk(fmt, w, a.astype(np.float32), m, n, k), f"{m}x{n}x{k}")
+        assert_close(out.cpu().numpy(), oracle.qmatmul_nk(fmt, w, a.astype(np.float32), m, n, k), f"{m}x{n}x{k}", plain_tol=None)
         outs.append(out.cpu().numpy())
     assert np.array_equal(outs[0], outs[2])
     from rocmforge_amd import _lib

@@ -60,7 +60,7 @@ def test_constants_match_the_header():
     header = open(os.path.join(ROOT, "include", "rfq.h")).read()
     header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
     enums = dict(re.findall(r"\b(RFQ_[A-Z0-9_]+)\s*=\s*(-?(?:0x[0-9A-Fa-f]+|\d+))", header))
-    enums.update(dict(re.findall(r"#define\s+(RFQ_(?:VERSION|TABLE_F32))\s+(\d+)", header)))
+    enums.update(dict(re.findall(r"#define\s+(RFQ_(?:VERSION|TABLE_F32|GEMM_ONE_PLANE))\s+(0x[0-9A-Fa-f]+|\d+)", header)))
     _, text = rust_functions()
     consts = dict(re.findall(r"pub const (RFQ_[A-Z0-9_]+): c_int = (-?(?:0x[0-9A-Fa-f]+|\d+));", text))
     assert len(enums) >= 30
