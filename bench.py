@@ -31,11 +31,22 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 N, K = 14336, 4096
 CACHE_BYTES = 256 << 20
-# HBM bytes one launch of the headline kernel moves, from FETCH_SIZE / WRITE_SIZE
-# profiler counters scaled by a copy kernel of known size
-# (profiles/gemv_q4k_14336x4096_hbm_counters.txt): 57,576.4 KiB read + 64.0 KiB written.
-MEASURED_TRAFFIC_BYTES = 59033935
+# HBM bytes one launch of the headline kernel moves, from FETCH_SIZE / WRITE_SIZE profiler counters scaled by a copy
+# kernel of known size: read from the committed summary of those runs, so that the figure cannot outlive its source.
 TRAFFIC_SOURCE = "profiles/gemv_q4k_14336x4096_hbm_counters.txt"
+
+
+def measured_traffic_bytes():
+    """(bytes per launch, kernel the counters belong to) from the line 'traffic per launch = ... = N bytes' and the
+    kernel named in the per-dispatch table of TRAFFIC_SOURCE; (None, None) when the file or the line is missing."""
+    import re
+    try:
+        text = open(os.path.join(ROOT, TRAFFIC_SOURCE)).read()
+    except OSError:
+        return None, None
+    m = re.search(r"traffic per launch\s*=.*?=\s*([\d,]+)\s*bytes", text)
+    kern = re.search(r"^\s*(gemv_\w+<[^>]*>).*FETCH_SIZE", text, re.M)
+    return (int(m.group(1).replace(",", "")) if m else None), (kern.group(1) if kern else None)
 # launch shapes of the read-only kernel that the floor is taken over (workgroups, threads, loads in flight, non-temporal)
 PREHEAT_MS = 30.0
 READ_FLOOR_SHAPES = ((256, 512, 4, 1), (256, 768, 4, 1), (256, 1024, 8, 1), (512, 512, 8, 1), (256, 512, 4, 0))
@@ -416,10 +427,14 @@ def main():
         _, d, *_ = time_gemv(torch, f, n_, k_, m_, c, args.steps, args.warmup, Q, 20260060)
         b = algorithmic_bytes(f, n_, k_, m_, Q)
         from rocmforge_amd import _lib
+        kern = _lib.lib().rfq_bench_last_gemv_kernel().decode()
+        # the floor for these bytes: a kernel that only reads them, launched the same way
+        floor_s, floor_shape = read_floor(torch, Q.packed_bytes(f, n_ * k_), c, min(args.steps, 500), min(args.warmup, 50))
         print(json.dumps({f"{name} gemv {n_}x{k_} m{m_}": {
             "GB/s": round(b / (d / args.steps) / 1e9, 1), "us": round(d / args.steps * 1e6, 2),
             "hbm_frac": round(b / (d / args.steps) / 1e9 / HBM_PEAK_GBS, 4), "algorithmic_bytes": b, "weight_copies": c,
-            "kernel": _lib.lib().rfq_bench_last_gemv_kernel().decode()}}))
+            "kernel": kern, "read_only_kernel_us": round(floor_s * 1e6, 2), "read_only_kernel": floor_shape,
+            "over_read_only_kernel": round(d / args.steps / floor_s - 1.0, 4)}}))
         return
 
     if args.only_gguf:
@@ -457,6 +472,15 @@ def main():
     if not args.no_warm:
         _, dev_w, *_ = time_gemv(torch, fmt, N, K, 1, 1, args.steps, args.warmup, Q, 20260003)
 
+    # the counters of the committed profile belong to one kernel: report them only while the dispatcher still takes it
+    import re
+    traffic, traffic_kernel = measured_traffic_bytes()
+    def _shape(name):                                      # "gemv_idot_kernel<12, 1, 2, 7, false>" / "...<Q4_K,1,2,7>" -> (name, [1, 2, 7])
+        m_ = re.match(r"(\w+)<([^>]*)>", name or "")
+        return (m_.group(1), [t.strip() for t in m_.group(2).split(",")][1:4]) if m_ else None
+    if _shape(traffic_kernel) != _shape(kernel_name):
+        traffic = None
+
     out = {
         "metric": "Q4_K decode GEMV GB/s (% HBM peak); quant prefill GEMM TFLOP/s (% MFMA peak)",
         "value": round(value, 1),
@@ -479,8 +503,8 @@ def main():
                    "launches, so that the part has left its idle clocks; the same K launches straight out of idle are "
                    "roofline.avg_launch_us_from_idle"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
-                     "traffic_source": TRAFFIC_SOURCE,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+                     "traffic_source": TRAFFIC_SOURCE, "traffic_kernel": traffic_kernel,
                      "kernel": kernel_name, "avg_launch_us": round(dev_s / args.steps * 1e6, 3),
                      "avg_launch_us_from_idle": round(idle_s / args.steps * 1e6, 3),
                      "read_only_kernel_us": round(floor_s * 1e6, 3), "read_only_kernel": floor_shape,

@@ -125,6 +125,9 @@ RFQ_API const char *rfq_last_error(void);
  * about to be destroyed (it frees the buffer once the stream's work is done;
  * a buffer that a capture used stays allocated until rfq_release_temporaries),
  * so that a later stream with the same handle value does not inherit it.
+ * Calls that use a stream's kept buffer must come from one host thread at a
+ * time per stream (a second thread that makes the buffer grow would free it
+ * under the first thread's launches); different streams are independent.
  * No counterpart in the reference, whose kernels take no temporaries. */
 RFQ_API int rfq_release_temporaries(void);
 RFQ_API int rfq_release_stream_temporaries(void *stream);

@@ -628,6 +628,8 @@ int static_scratch(uint8_t **out)
 // only when a larger one is needed: a stream-ordered allocation and release
 // around every call costs about 6 us of idle GPU between calls.  Larger
 // requests are allocated and released in stream order, per call.
+// One host thread per stream: the pointer is handed out under the lock but used after it, so a second thread that
+// grows the same stream's buffer meanwhile would free it under the first thread's launches.
 // While the stream is being captured nothing is allocated or freed: the call
 // gets the stream's buffer if it is large enough and an error otherwise.  A
 // buffer handed out under capture is baked into the graph, so when a later
@@ -662,11 +664,12 @@ int workspace(hipStream_t s, size_t bytes, uint8_t **out, bool *transient)
         if (capturing)
             return fail(RFQ_E_UNSUPPORTED, "the call needs %zu bytes of temporary memory and the stream being captured holds %zu: run the call once on this stream before capturing it",
                         bytes, kept.device == device ? kept.bytes : (size_t)0);
-        if (kept.ptr != nullptr) {
-            if (kept.captured || kept.device != device) ws_retired.push_back(kept);   // a graph (or another device's stream) may hold it
-            else RFQ_HIP(hipFree(kept.ptr));                                          // (waits for the work that uses it)
+        const Kept old = kept;
+        kept = Kept{nullptr, 0, device, false};                                       // (whatever fails below, the entry no longer names the old buffer)
+        if (old.ptr != nullptr) {
+            if (old.captured || old.device != device) ws_retired.push_back(old);      // a graph (or another device's stream) may hold it
+            else RFQ_HIP(hipFree(old.ptr));                                           // (waits for the work that uses it)
         }
-        kept = Kept{nullptr, 0, device, false};
         RFQ_HIP(hipMalloc(reinterpret_cast<void **>(&kept.ptr), bytes));
         kept.bytes = bytes;
     }
