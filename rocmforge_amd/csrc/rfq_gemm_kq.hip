@@ -129,7 +129,8 @@ arrange_a_kernel(const _Float16 *__restrict__ a, v4u *__restrict__ at, _Float16 
 
 // PLANES = 2: every stage of k is walked twice, first with the weights' fp16 values (hi) and then with what the
 // rounding to fp16 left over (lo = fp16(v - hi)), as two consecutive stages of the same pipeline over the same
-// activations: the contraction then carries the weights to 2^-22 instead of 2^-12.
+// activations and the same raw weight bytes (loaded once per pair): the contraction then carries the weights to 2^-22
+// instead of 2^-12.
 template <int FMT, bool OUT_F16, int PLANES>
 __global__ void __launch_bounds__(256)
 gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const _Float16 *__restrict__ s2,
@@ -343,10 +344,14 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
     v2h dec_tmp[4];                                               // a chunk between its decode steps
     auto iter = [&](auto sc, int st) __attribute__((always_inline)) {
         constexpr int S = decltype(sc)::value, S1 = (S + 1) & 3, S2 = (S + 2) & 3, S3 = (S + 3) & 3;
-        Raw32<FMT> &raw_late = raw_of(IC<S2>{}), &raw_early = raw_of(IC<S3>{});
+        // With two planes the two stages of a pair (even ring slot = hi, odd = lo) are the same 64 k: the odd slot has
+        // no registers of its own, it decodes and multiplies out of its even neighbour's (SH = the slot that holds
+        // the data), which is refilled once both have used it.
+        constexpr int SH0 = PLANES == 2 ? (S & ~1) : S, SH2 = PLANES == 2 ? (S2 & ~1) : S2, SH3 = PLANES == 2 ? (S3 & ~1) : S3;
+        Raw32<FMT> &raw_late = raw_of(IC<SH2>{}), &raw_early = raw_of(IC<SH3>{});
         v8h (&hw_late)[4] = (S & 1) ? hw_odd : hw_even;
         v8h (&hw_early)[4] = (S & 1) ? hw_even : hw_odd;
-        v4u (&ra)[TI][4] = ra_of(sc);
+        v4u (&ra)[TI][4] = ra_of(IC<SH0>{});
         if constexpr (FMT == RFQ_Q4_K) {
             if (S == 0) {                                          // this trip's sums arrived with stage st's A
 #pragma unroll
@@ -384,10 +389,11 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
                         if (p == EARLY[q]) raw_early.template step<(S3 % PLANES) != 0>(q, hw_early, dec_tmp);
                     }
                 }
-                if (p == 15) settle(IC<S3>{}, st + 3, S == 0 ? hsA[3] : hsB[S3]);   // stage st+3 is number S3 of its super-block
+                if (p == 15 && SH3 == S3) settle(IC<S3>{}, st + 3, S == 0 ? hsA[3] : hsB[S3]);   // stage st+3 is number S3 of its super-block
                 if (p >= 17 && p <= 23 && (p & 1)) stash(S2, (p - 17) / 2, hw_late);
                 if (p == 25) {
-                    fetch_w(IC<S2>{}, st + 6);
+                    if constexpr (PLANES == 1) fetch_w(IC<S2>{}, st + 6);
+                    else if constexpr (S2 & 1) fetch_w(IC<SH2>{}, st + 5);   // both planes of the pair are decoded: its slot takes the next pair
                     if (S == 2) fetch_hdr((st + 6) / 4);
                 }
                 if constexpr (FMT == RFQ_Q4_K) {
@@ -395,7 +401,11 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
                     if (S == 0 && p == 24) stash_mins();
                     if (S == 3 && p >= 28) fm[p - 28] = *reinterpret_cast<const v8h *>(mn_rd + (p - 28) * 32 * MNR);
                 }
-                if (j == 3) fetch_a(sc, st + 4, i, c);
+                if constexpr (PLANES == 1) {
+                    if (j == 3) fetch_a(sc, st + 4, i, c);
+                } else if constexpr (S & 1) {
+                    if (j == 3) fetch_a(IC<SH0>{}, st + 3, i, c);   // the lo stage was the chunk's last reader
+                }
                 __builtin_amdgcn_sched_barrier(0);
             }
         lds_barrier();
@@ -413,12 +423,16 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
         }
         fetch_w(IC<0>{}, 0);
         fetch_a_all(IC<0>{}, 0);
-        fetch_w(IC<1>{}, 1);
-        fetch_a_all(IC<1>{}, 1);
+        if constexpr (PLANES == 1) {
+            fetch_w(IC<1>{}, 1);
+            fetch_a_all(IC<1>{}, 1);
+        }
         fetch_w(IC<2>{}, 2);
         fetch_a_all(IC<2>{}, 2);
-        fetch_w(IC<3>{}, 3);
-        fetch_a_all(IC<3>{}, 3);
+        if constexpr (PLANES == 1) {
+            fetch_w(IC<3>{}, 3);
+            fetch_a_all(IC<3>{}, 3);
+        }
         // (a real move: the loop must not inherit a pending load on hmA, or its
         // first use in the loop body would wait for younger loads every trip)
         asm volatile("v_mov_b32 %0, %1" : "=v"(hmA) : "v"(hmA));
@@ -427,13 +441,19 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
         for (int T = 0; T < 12; T++) raw0.template step<false>(T, hw, dec_tmp);
 #pragma unroll
         for (int c = 0; c < 4; c++) stash(0, c, hw);
-        fetch_w(IC<0>{}, 4);
-        settle(IC<1>{}, 1, hsA[1]);
+        if constexpr (PLANES == 1) {
+            fetch_w(IC<0>{}, 4);
+            settle(IC<1>{}, 1, hsA[1]);
 #pragma unroll
-        for (int T = 0; T < 12; T++) raw1.template step<(1 % PLANES) != 0>(T, hw, dec_tmp);
+            for (int T = 0; T < 12; T++) raw1.template step<false>(T, hw, dec_tmp);
+        } else {
+#pragma unroll
+            for (int T = 0; T < 12; T++) raw0.template step<true>(T, hw, dec_tmp);
+        }
 #pragma unroll
         for (int c = 0; c < 4; c++) stash(1, c, hw);
-        fetch_w(IC<1>{}, 5);
+        if constexpr (PLANES == 1) fetch_w(IC<1>{}, 5);
+        else fetch_w(IC<0>{}, 4);
         settle(IC<2>{}, 2, hsA[2]);
 #pragma unroll
         for (int T = 0; T < 6; T++) raw2.template step<false>(T, hw_even, dec_tmp);
