@@ -341,6 +341,13 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
     // reads the buffer the next iteration overwrites (st+3 = st-1 mod 4).
     v8h fw[2][TJ];
     v8h hw_even[4], hw_odd[4];                                    // decoded weights of the even / odd stage in progress
+    // Two planes: a pair's raw bytes are decoded once, during the hi stage's steps, into both operands; the lo values
+    // wait here until the lo stage's turn to go to LDS (two sets: the next pair's steps start before that).
+    v8h hw_lo0[4], hw_lo1[4];
+    auto lo_of = [&](auto pc) -> v8h (&)[4] {
+        if constexpr (decltype(pc)::value == 0) return hw_lo0;
+        else return hw_lo1;
+    };
     v2h dec_tmp[4];                                               // a chunk between its decode steps
     auto iter = [&](auto sc, int st) __attribute__((always_inline)) {
         constexpr int S = decltype(sc)::value, S1 = (S + 1) & 3, S2 = (S + 2) & 3, S3 = (S + 3) & 3;
@@ -385,12 +392,20 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
                     constexpr int LATE[6] = {0, 3, 5, 8, 10, 13}, EARLY[6] = {16, 18, 20, 22, 26, 29};
 #pragma unroll
                     for (int q = 0; q < 6; q++) {
-                        if (p == LATE[q]) raw_late.template step<(S2 % PLANES) != 0>(6 + q, hw_late, dec_tmp);
-                        if (p == EARLY[q]) raw_early.template step<(S3 % PLANES) != 0>(q, hw_early, dec_tmp);
+                        if constexpr (PLANES == 1) {
+                            if (p == LATE[q]) raw_late.template step<false>(6 + q, hw_late, hw_late, dec_tmp);
+                            if (p == EARLY[q]) raw_early.template step<false>(q, hw_early, hw_early, dec_tmp);
+                        } else {
+                            if ((S2 & 1) == 0 && p == LATE[q]) raw_late.template step<true>(6 + q, hw_late, lo_of(IC<(S2 >> 1) & 1>{}), dec_tmp);
+                            if ((S3 & 1) == 0 && p == EARLY[q]) raw_early.template step<true>(q, hw_early, lo_of(IC<(S3 >> 1) & 1>{}), dec_tmp);
+                        }
                     }
                 }
                 if (p == 15 && SH3 == S3) settle(IC<S3>{}, st + 3, S == 0 ? hsA[3] : hsB[S3]);   // stage st+3 is number S3 of its super-block
-                if (p >= 17 && p <= 23 && (p & 1)) stash(S2, (p - 17) / 2, hw_late);
+                if (p >= 17 && p <= 23 && (p & 1)) {
+                    if constexpr (PLANES == 2 && (S2 & 1) != 0) stash(S2, (p - 17) / 2, lo_of(IC<(S2 >> 1) & 1>{}));
+                    else stash(S2, (p - 17) / 2, hw_late);
+                }
                 if (p == 25) {
                     if constexpr (PLANES == 1) fetch_w(IC<S2>{}, st + 6);
                     else if constexpr (S2 & 1) fetch_w(IC<SH2>{}, st + 5);   // both planes of the pair are decoded: its slot takes the next pair
@@ -438,25 +453,25 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
         asm volatile("v_mov_b32 %0, %1" : "=v"(hmA) : "v"(hmA));
         settle(IC<0>{}, 0, hsA[0]);
 #pragma unroll
-        for (int T = 0; T < 12; T++) raw0.template step<false>(T, hw, dec_tmp);
+        for (int T = 0; T < 12; T++) raw0.template step<PLANES == 2>(T, hw, hw_lo0, dec_tmp);
 #pragma unroll
         for (int c = 0; c < 4; c++) stash(0, c, hw);
         if constexpr (PLANES == 1) {
             fetch_w(IC<0>{}, 4);
             settle(IC<1>{}, 1, hsA[1]);
 #pragma unroll
-            for (int T = 0; T < 12; T++) raw1.template step<false>(T, hw, dec_tmp);
+            for (int T = 0; T < 12; T++) raw1.template step<false>(T, hw, hw, dec_tmp);
+#pragma unroll
+            for (int c = 0; c < 4; c++) stash(1, c, hw);
         } else {
 #pragma unroll
-            for (int T = 0; T < 12; T++) raw0.template step<true>(T, hw, dec_tmp);
+            for (int c = 0; c < 4; c++) stash(1, c, hw_lo0);
         }
-#pragma unroll
-        for (int c = 0; c < 4; c++) stash(1, c, hw);
         if constexpr (PLANES == 1) fetch_w(IC<1>{}, 5);
         else fetch_w(IC<0>{}, 4);
         settle(IC<2>{}, 2, hsA[2]);
 #pragma unroll
-        for (int T = 0; T < 6; T++) raw2.template step<false>(T, hw_even, dec_tmp);
+        for (int T = 0; T < 6; T++) raw2.template step<PLANES == 2>(T, hw_even, hw_lo1, dec_tmp);
         lds_barrier();
 #pragma unroll
         for (int j = 0; j < TJ; j++) fw[0][j] = read_frag(0, j, 0);

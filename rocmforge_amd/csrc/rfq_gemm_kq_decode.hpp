@@ -38,13 +38,12 @@ typedef __amdgpu_buffer_rsrc_t Rsrc;
 // instruction's k slots works as long as both operands use it).
 __device__ __forceinline__ constexpr int chunk_pos(int e) { return ((e & 3) << 1) | (e >> 2); }
 
-// The two fp16 operands a decoded weight v (f32) is contracted as when the kernel runs two planes: hi = fp16(v)
-// (round to nearest even) and lo = fp16(v - hi), so that hi + lo = v to 2^-22 of v; with one plane only hi is used.
-template <bool LO> __device__ __forceinline__ _Float16 fp16_part(float v)
+// The fp16 operands a decoded weight v (f32) is contracted as: hi = fp16(v) (round to nearest even) and, when the
+// kernel runs two planes, lo = fp16(v - hi), so that hi + lo = v to 2^-22 of v.
+template <bool BOTH> __device__ __forceinline__ void fp16_parts(float v, _Float16 &hi, _Float16 &lo)
 {
-    const _Float16 hi = (_Float16)v;
-    if constexpr (!LO) return hi;
-    else return (_Float16)(v - (float)hi);
+    hi = (_Float16)v;
+    if constexpr (BOTH) lo = (_Float16)(v - (float)hi);
 }
 
 // Every format decodes a 32-element group in 12 steps (chunk c = T/3 of 8
@@ -72,11 +71,16 @@ template <> struct Raw32<RFQ_Q4_0> {
         // scale * (q - 8) as a fused multiply-add of q: 8 * scale is exact, so the one rounding is the product's
         return __builtin_fmaf(__uint_as_float(d[0]), (float)q, -8.0f * __uint_as_float(d[0]));
     }
-    template <bool LO> __device__ __forceinline__ void step(int T, v8h (&h)[4], v2h (&)[4]) const
+    template <bool BOTH> __device__ __forceinline__ void step(int T, v8h (&h)[4], v8h (&l)[4], v2h (&)[4]) const
     {
         const int c = T / 3, e0 = 3 * (T % 3), e1 = e0 + 3 < 8 ? e0 + 3 : 8;
 #pragma unroll
-        for (int e = e0; e < e1; e++) h[c][chunk_pos(e)] = fp16_part<LO>(value(8 * c + e));
+        for (int e = e0; e < e1; e++) {
+            _Float16 hi, lo = (_Float16)0.0f;
+            fp16_parts<BOTH>(value(8 * c + e), hi, lo);
+            h[c][chunk_pos(e)] = hi;
+            if constexpr (BOTH) l[c][chunk_pos(e)] = lo;
+        }
     }
 };
 
@@ -106,11 +110,16 @@ template <> struct Raw32<RFQ_Q8_0> {
         // (b - 128) * scale as a fused multiply-add of b: 128 * scale is exact, so the one rounding is the product's
         return __builtin_fmaf(__uint_as_float(d[0]), (float)b, -128.0f * __uint_as_float(d[0]));
     }
-    template <bool LO> __device__ __forceinline__ void step(int T, v8h (&h)[4], v2h (&)[4]) const
+    template <bool BOTH> __device__ __forceinline__ void step(int T, v8h (&h)[4], v8h (&l)[4], v2h (&)[4]) const
     {
         const int c = T / 3, e0 = 3 * (T % 3), e1 = e0 + 3 < 8 ? e0 + 3 : 8;
 #pragma unroll
-        for (int e = e0; e < e1; e++) h[c][chunk_pos(e)] = fp16_part<LO>(value(8 * c + e));
+        for (int e = e0; e < e1; e++) {
+            _Float16 hi, lo = (_Float16)0.0f;
+            fp16_parts<BOTH>(value(8 * c + e), hi, lo);
+            h[c][chunk_pos(e)] = hi;
+            if constexpr (BOTH) l[c][chunk_pos(e)] = lo;
+        }
     }
 };
 
@@ -136,7 +145,7 @@ template <> struct Raw32<RFQ_Q4_K> {
     // 0x5400 | (q << 4) reads 64 + q, so one and-or per pair (k0,k4), (k1,k5),
     // and of the dword shifted by 8, (k2,k6), (k3,k7); then subtract the
     // offset (exact) and multiply by the scale (one rounding).
-    template <bool LO> __device__ __forceinline__ void step(int T, v8h (&h)[4], v2h (&t)[4]) const
+    template <bool BOTH> __device__ __forceinline__ void step(int T, v8h (&h)[4], v8h (&)[4], v2h (&t)[4]) const
     {
         const int c = T / 3, ph = T % 3;
         if (ph == 0) {
@@ -194,11 +203,16 @@ template <> struct Raw32<RFQ_Q6_K> {
         uint64_t two = (uint64_t)d[1 + w] | ((uint64_t)d[1 + (w < 5 ? w + 1 : w)] << 32);
         return (float)sbfe6((uint32_t)(two >> o), 0) * scale;
     }
-    template <bool LO> __device__ __forceinline__ void step(int T, v8h (&h)[4], v2h (&)[4]) const
+    template <bool BOTH> __device__ __forceinline__ void step(int T, v8h (&h)[4], v8h (&l)[4], v2h (&)[4]) const
     {
         const int c = T / 3, e0 = 3 * (T % 3), e1 = e0 + 3 < 8 ? e0 + 3 : 8;
 #pragma unroll
-        for (int e = e0; e < e1; e++) h[c][chunk_pos(e)] = fp16_part<LO>(value(8 * c + e));
+        for (int e = e0; e < e1; e++) {
+            _Float16 hi, lo = (_Float16)0.0f;
+            fp16_parts<BOTH>(value(8 * c + e), hi, lo);
+            h[c][chunk_pos(e)] = hi;
+            if constexpr (BOTH) l[c][chunk_pos(e)] = lo;
+        }
     }
 };
 
@@ -227,11 +241,16 @@ template <> struct Raw32<RFQ_GGUF_Q4_0> {
         const float sc = __uint_as_float(d[0]);
         return __builtin_fmaf(sc, (float)q, -8.0f * sc);
     }
-    template <bool LO> __device__ __forceinline__ void step(int T, v8h (&h)[4], v2h (&)[4]) const
+    template <bool BOTH> __device__ __forceinline__ void step(int T, v8h (&h)[4], v8h (&l)[4], v2h (&)[4]) const
     {
         const int c = T / 3, e0 = 3 * (T % 3), e1 = e0 + 3 < 8 ? e0 + 3 : 8;
 #pragma unroll
-        for (int e = e0; e < e1; e++) h[c][chunk_pos(e)] = fp16_part<LO>(value(8 * c + e));
+        for (int e = e0; e < e1; e++) {
+            _Float16 hi, lo = (_Float16)0.0f;
+            fp16_parts<BOTH>(value(8 * c + e), hi, lo);
+            h[c][chunk_pos(e)] = hi;
+            if constexpr (BOTH) l[c][chunk_pos(e)] = lo;
+        }
     }
 };
 
@@ -259,11 +278,16 @@ template <> struct Raw32<RFQ_GGUF_Q8_0> {
         const int b = (int)(int8_t)((d[1 + (e >> 2)] >> (8 * (e & 3))) & 255u);
         return (float)b * __uint_as_float(d[0]);
     }
-    template <bool LO> __device__ __forceinline__ void step(int T, v8h (&h)[4], v2h (&)[4]) const
+    template <bool BOTH> __device__ __forceinline__ void step(int T, v8h (&h)[4], v8h (&l)[4], v2h (&)[4]) const
     {
         const int c = T / 3, e0 = 3 * (T % 3), e1 = e0 + 3 < 8 ? e0 + 3 : 8;
 #pragma unroll
-        for (int e = e0; e < e1; e++) h[c][chunk_pos(e)] = fp16_part<LO>(value(8 * c + e));
+        for (int e = e0; e < e1; e++) {
+            _Float16 hi, lo = (_Float16)0.0f;
+            fp16_parts<BOTH>(value(8 * c + e), hi, lo);
+            h[c][chunk_pos(e)] = hi;
+            if constexpr (BOTH) l[c][chunk_pos(e)] = lo;
+        }
     }
 };
 
@@ -315,11 +339,16 @@ template <> struct Raw32<RFQ_GGUF_Q4_K> {
         const uint32_t q = (d[4 + (e >> 2)] >> (8 * (e & 3))) & 255u;
         return __builtin_fmaf(__uint_as_float(d[0]), (float)q, __uint_as_float(d[1]));
     }
-    template <bool LO> __device__ __forceinline__ void step(int T, v8h (&h)[4], v2h (&)[4]) const
+    template <bool BOTH> __device__ __forceinline__ void step(int T, v8h (&h)[4], v8h (&l)[4], v2h (&)[4]) const
     {
         const int c = T / 3, e0 = 3 * (T % 3), e1 = e0 + 3 < 8 ? e0 + 3 : 8;
 #pragma unroll
-        for (int e = e0; e < e1; e++) h[c][chunk_pos(e)] = fp16_part<LO>(value(8 * c + e));
+        for (int e = e0; e < e1; e++) {
+            _Float16 hi, lo = (_Float16)0.0f;
+            fp16_parts<BOTH>(value(8 * c + e), hi, lo);
+            h[c][chunk_pos(e)] = hi;
+            if constexpr (BOTH) l[c][chunk_pos(e)] = lo;
+        }
     }
 };
 
@@ -370,11 +399,16 @@ template <> struct Raw32<RFQ_GGUF_Q6_K> {
         const uint32_t q = (d[e >> 2] >> (8 * (e & 3))) & 255u;
         return __builtin_fmaf(__uint_as_float(d[8 + (e >> 4)]), (float)q, __uint_as_float(d[10 + (e >> 4)]));
     }
-    template <bool LO> __device__ __forceinline__ void step(int T, v8h (&h)[4], v2h (&)[4]) const
+    template <bool BOTH> __device__ __forceinline__ void step(int T, v8h (&h)[4], v8h (&l)[4], v2h (&)[4]) const
     {
         const int c = T / 3, e0 = 3 * (T % 3), e1 = e0 + 3 < 8 ? e0 + 3 : 8;
 #pragma unroll
-        for (int e = e0; e < e1; e++) h[c][chunk_pos(e)] = fp16_part<LO>(value(8 * c + e));
+        for (int e = e0; e < e1; e++) {
+            _Float16 hi, lo = (_Float16)0.0f;
+            fp16_parts<BOTH>(value(8 * c + e), hi, lo);
+            h[c][chunk_pos(e)] = hi;
+            if constexpr (BOTH) l[c][chunk_pos(e)] = lo;
+        }
     }
 };
 
