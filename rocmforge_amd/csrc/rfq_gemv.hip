@@ -1254,6 +1254,44 @@ template <> struct IUnit<RFQ_GGUF_Q6_K> : Unit<RFQ_GGUF_Q6_K> {
     }
 };
 
+// The 256-byte Q6_K layout: a unit is 24 stream bytes = 32 two's-complement 6-bit codes, LSB first, and two f16 scales
+// (src/kernels/quant/q6_k.rs:221-261).  Four codes are three bytes: the 24-bit window of a group is spread over the
+// four bytes of a dword by three shifts that each write one byte (sub-dword destination select), one mask clears what
+// the shifts dragged in, and code ^ 32 = value + 32 is an unsigned byte for the byte dot products; the offset goes
+// through the sums of x over the unit's two halves, which have a scale each.
+template <> struct IUnit<RFQ_Q6_K> : Unit<RFQ_Q6_K> {
+    static constexpr bool PAIR = false;
+    static constexpr bool NIBBLE = false;
+    static constexpr uint32_t TOPOFF = 0;
+    static __device__ __forceinline__ uint32_t bytes_of(uint32_t t)    // t: four 6-bit codes in bits 0..23 (anything above)
+    {
+        uint32_t v = t;
+        asm("v_lshrrev_b32_sdwa %0, %2, %1 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(v) : "v"(t), "i"(6));
+        asm("v_lshrrev_b32_sdwa %0, %2, %1 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(v) : "v"(t), "i"(12));
+        asm("v_lshrrev_b32_sdwa %0, %2, %1 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(v) : "v"(t), "i"(18));
+        return (v & 0x3F3F3F3Fu) ^ 0x20202020u;
+    }
+    __device__ __forceinline__ float idot(const XPrep &xp) const
+    {
+        uint32_t alo[2] = {0, 0}, amid[2] = {0, 0};
+        int atop[2] = {0, 0};
+#pragma unroll
+        for (int g = 0; g < 8; g++) {
+            const int b = 3 * (g & 3), d = 3 * (g >> 2);               // window at byte b of dwords d .. d + 2
+            const uint32_t t = b == 0 ? q.v[d] : b == 9 ? q.v[d + 2] >> 8 : __builtin_amdgcn_alignbit(q.v[d + b / 4 + 1], q.v[d + b / 4], 8 * (b & 3));
+            const uint32_t v = bytes_of(t);
+            const uint32_t *L = &xp.l[g * 3];
+            alo[g >> 2] = __builtin_amdgcn_udot4(v, L[0], alo[g >> 2], false);
+            amid[g >> 2] = __builtin_amdgcn_udot4(v, L[1], amid[g >> 2], false);
+            atop[g >> 2] = __builtin_amdgcn_sdot4((int)v, (int)L[2], atop[g >> 2], false);
+        }
+        const float S0 = __builtin_fmaf((float)atop[0], 65536.0f, __builtin_fmaf((float)amid[0], 256.0f, (float)alo[0]));
+        const float S1 = __builtin_fmaf((float)atop[1], 65536.0f, __builtin_fmaf((float)amid[1], 256.0f, (float)alo[1]));
+        const float h0 = __builtin_fmaf(xp.s, S0, -32.0f * xp.xh0), h1 = __builtin_fmaf(xp.s, S1, -32.0f * xp.xh1);
+        return __builtin_fmaf(f16_bits_to_f32((uint16_t)(sc2 & 0xFFFFu)), h0, f16_bits_to_f32((uint16_t)(sc2 >> 16)) * h1);
+    }
+};
+
 // The formats without paired units never call idot_pair.
 template <typename IU>
 __device__ __forceinline__ float idot_pair_of(const IU &u, const XPrep &xe, const XPrep &xo)
@@ -1794,7 +1832,9 @@ template <> struct HasIdot<RFQ_GGUF_Q4_K> { static constexpr bool value = true; 
 template <> struct HasIdot<RFQ_GGUF_Q6_K> { static constexpr bool value = true; };
 template <> struct HasIdot<RFQ_MM_Q4_K> { static constexpr bool value = true; };
 template <> struct HasIdot<RFQ_MM_Q8_0> { static constexpr bool value = true; };
+template <> struct HasIdot<RFQ_Q6_K> { static constexpr bool value = true; };
 template <int FMT> struct HasIdotBatch { static constexpr bool value = HasIdot<FMT>::value; };
+template <> struct HasIdotBatch<RFQ_Q6_K> { static constexpr bool value = false; };   // batches keep one decode launch per vector
 
 template <int FMT, int UPL, int WPR, int R, bool FUSE>
 int launch_idot(const uint8_t *w, const float *x, float *y, int n, int k, int blocks, int groups, const GemvFuse &f,
@@ -1808,10 +1848,12 @@ int launch_idot(const uint8_t *w, const float *x, float *y, int n, int k, int bl
     return RFQ_OK;
 }
 
+// prefer_idot = false: a format that has both kernels takes the float one for this shape.
 template <int FMT, int UPL, int WPR, bool FUSE>
-int run_idot(const uint8_t *w, const float *x, float *y, int n, int k, const GemvFuse &f, hipStream_t s)
+int run_idot(const uint8_t *w, const float *x, float *y, int n, int k, const GemvFuse &f, hipStream_t s, bool prefer_idot = true)
 {
     if constexpr (HasIdot<FMT>::value) {
+        if (!prefer_idot) return run_xreg<FMT, UPL, WPR, FUSE>(w, x, y, n, k, f, s);
         constexpr int TEAMS = IDOT_WAVES / WPR;
         // Aim at eight resident wavefronts per CU, every team walking the same number
         // of rows (a straggler is expensive on a ~10 us kernel).  Rows per team
@@ -1965,6 +2007,19 @@ template <int FMT, bool FUSE>
 int run_rows(const uint8_t *w, const float *x, float *y, int n, int k, const GemvFuse &f, hipStream_t s)
 {
     const int ku = k / 32;
+    // The 256-byte Q6_K layout has both kernels, a few per cent apart either way (measured on 14336, 11008, 4096 and
+    // 32000 rows of 4096, 4096 rows of 8192 and of 14336): the integer-dot one where a team walks a single group of rows
+    // of 65..128 units or rows longer than 256 units, the float one elsewhere and in the fused forms.
+    if constexpr (FMT == RFQ_Q6_K) {
+        const int cus = device_cu_count();
+        if (FUSE || !((ku > 64 && ku <= 128 && n >= cus * 56 && n <= cus * 64) || ku > 256)) {
+            if (ku <= 64) return run_idot<FMT, 1, 1, FUSE>(w, x, y, n, k, f, s, false);
+            if (!FUSE && ku <= 128 && n >= cus * 32) return run_idot<FMT, 1, 2, FUSE>(w, x, y, n, k, f, s, false);
+            if (ku <= 128) return run_idot<FMT, 2, 1, FUSE>(w, x, y, n, k, f, s, false);
+            if (ku <= 256) return run_idot<FMT, 2, 2, FUSE>(w, x, y, n, k, f, s, false);
+            return run_idot<FMT, 2, 4, FUSE>(w, x, y, n, k, f, s, false);
+        }
+    }
     if (ku <= 64) return run_idot<FMT, 1, 1, FUSE>(w, x, y, n, k, f, s);
     // Rows of 65..128 units with at least seven rows per team in that form: one unit per lane, two
     // wavefronts per row, sixteen wavefronts per CU (14336 x 4096: 11.67 -> 11.30 us; 4096 rows would lose 6 %)
