@@ -977,7 +977,11 @@ __device__ __forceinline__ void prep_load8(const float *xp, float (&xv)[8])
     }
 }
 
-template <bool NIBBLE, uint32_t TOPOFF>
+// QSUM: the slot of the first half's sum holds s * sum(X) instead, the sum of the unit's values as rounded to block
+// fixed point.  A format that subtracts an offset times the sum of x from its byte dot products (MXFP4: 16) takes it:
+// the offset then cancels exactly, where the sum of the unrounded x would leave offset * s * (sum of the 32 rounding
+// errors) in every row alike.
+template <bool NIBBLE, uint32_t TOPOFF, bool QSUM = false>
 __device__ __forceinline__ void prep_convert_quarter(const float (&xv)[8], int quarter, uint32_t *lds_unit)
 {
     float m = 0.f, sum = 0.f;
@@ -1007,6 +1011,14 @@ __device__ __forceinline__ void prep_convert_quarter(const float (&xv)[8], int q
 #pragma unroll
     for (int i = 0; i < 8; i++)
         X[i] = __float_as_uint(__builtin_fmaf(xv[i], inv_s, 12582912.0f)) - 0x4B400000u + TOPOFF;
+    if constexpr (QSUM) {
+        int isum = 0;
+#pragma unroll
+        for (int i = 0; i < 8; i++) isum += (int)(X[i] - TOPOFF);
+        isum += __builtin_amdgcn_update_dpp(0, isum, 0xB1, 0xF, 0xF, true);
+        isum += __builtin_amdgcn_update_dpp(0, isum, 0x4E, 0xF, 0xF, true);
+        if (quarter == 0) lds_unit[26] = __float_as_uint((float)isum * sc);
+    }
     uint32_t *o = lds_unit + quarter * 6;
     if (NIBBLE) {
         limbs4(X[0], X[2], X[4], X[6], o);
@@ -1019,7 +1031,9 @@ __device__ __forceinline__ void prep_convert_quarter(const float (&xv)[8], int q
         lds_unit[24] = __float_as_uint(sc);
         lds_unit[25] = __float_as_uint(sum);
     }
-    if ((quarter & 1) == 0) lds_unit[26 + (quarter >> 1)] = __float_as_uint(half_sum);
+    if constexpr (!QSUM) {
+        if ((quarter & 1) == 0) lds_unit[26 + (quarter >> 1)] = __float_as_uint(half_sum);
+    }
 }
 
 // sum_i nibble_i * X_i for 16 weight bytes in low-nibble-first order.
@@ -1042,6 +1056,8 @@ __device__ __forceinline__ float nib_idot(const U4 &q, const XPrep &xp)
 }
 
 template <int FMT> struct IUnit;
+template <int FMT> struct WantsQSum { static constexpr bool value = false; };
+template <> struct WantsQSum<RFQ_MXFP4> { static constexpr bool value = true; };
 
 template <> struct IUnit<RFQ_Q4_K> : Unit<RFQ_Q4_K> {
     static constexpr bool PAIR = false;
@@ -1292,6 +1308,57 @@ template <> struct IUnit<RFQ_Q6_K> : Unit<RFQ_Q6_K> {
     }
 };
 
+// MXFP4 (src/loader/dequant.rs:41-82, mxfp.rs:234-244): the code values doubled are small integers,
+// {0, 2, 2, 4, 4, 8, 8, 16} for codes 0..7 and {-1, -2, -2, -4, -4, -8, -8, -16} for 8..15, so a unit is a byte dot product
+// like the others once codes are bytes: two 8-entry byte tables (v_perm_b32 looks four codes up at once) hold the
+// values + 16 for either sign, the sign bit of each code becomes a byte mask by the same instruction's sign-fill
+// selectors, and the offset of 16 goes through the sum of the unit's fixed-point x (exactly: the scales are all
+// positive, so a residue common to all rows would add up over a column of outputs).  Element 2j is the HIGH nibble of byte j.  The +-8 clamp
+// of the reference bites only for exponents >= 1, where it is a bound 2^(4 - e) on the doubled value (from e = 4 on
+// every value but 0 sits at the bound and the unit's scale is 8): such units rebuild their tables with that bound.
+template <> struct IUnit<RFQ_MXFP4> : Unit<RFQ_MXFP4> {
+    static constexpr bool PAIR = false;
+    static constexpr bool NIBBLE = true;
+    static constexpr uint32_t TOPOFF = 0;
+    static __device__ __forceinline__ uint32_t pack4(uint32_t a, uint32_t b, uint32_t c, uint32_t d) { return a | (b << 8) | (c << 16) | (d << 24); }
+    __device__ __forceinline__ float idot(const XPrep &xp) const
+    {
+        uint32_t plo = 0x14121210u, phi = 0x20181814u;               // 16 + {0, 2, 2, 4 | 4, 8, 8, 16}
+        uint32_t nlo = 0x0C0E0E0Fu, nhi = 0x0008080Cu;               // 16 - {1, 2, 2, 4 | 4, 8, 8, 16}
+        int ee = e;
+        if (__builtin_amdgcn_ballot_w64(e >= 1) != 0) {              // (weights below 1 never have such a unit)
+            const uint32_t b = e <= 0 ? 16u : (e >= 4 ? 1u : (16u >> e));
+            auto lim = [&](uint32_t m) { return m < b ? m : b; };
+            plo = pack4(16u, 16u + lim(2), 16u + lim(2), 16u + lim(4));
+            phi = pack4(16u + lim(4), 16u + lim(8), 16u + lim(8), 16u + lim(16));
+            nlo = pack4(16u - lim(1), 16u - lim(2), 16u - lim(2), 16u - lim(4));
+            nhi = pack4(16u - lim(4), 16u - lim(8), 16u - lim(8), 16u - lim(16));
+            ee = e > 4 ? 4 : e;
+        }
+        uint32_t alo = 0, amid = 0;
+        int atop = 0;
+#pragma unroll
+        for (int d = 0; d < 4; d++) {
+            const uint32_t x = q.v[d];
+            const uint32_t sl = x & 0x07070707u, sh = (x >> 4) & 0x07070707u;
+            const uint32_t ml = __builtin_amdgcn_perm(x << 4, x << 12, 0x0B090A08u);   // 0xFF where the low code's sign bit is set
+            const uint32_t mh = __builtin_amdgcn_perm(x, x << 8, 0x0B090A08u);         // likewise for the high code
+            const uint32_t pl = __builtin_amdgcn_perm(phi, plo, sl), nl = __builtin_amdgcn_perm(nhi, nlo, sl);
+            const uint32_t ph = __builtin_amdgcn_perm(phi, plo, sh), nh = __builtin_amdgcn_perm(nhi, nlo, sh);
+            const uint32_t rl = (ml & nl) | (~ml & pl), rh = (mh & nh) | (~mh & ph);
+            const uint32_t *H = &xp.l[(2 * d) * 3], *L = &xp.l[(2 * d + 1) * 3];      // elements 8d + {0, 2, 4, 6} / {1, 3, 5, 7}
+            alo = __builtin_amdgcn_udot4(rh, H[0], alo, false);
+            amid = __builtin_amdgcn_udot4(rh, H[1], amid, false);
+            atop = __builtin_amdgcn_sdot4((int)rh, (int)H[2], atop, false);
+            alo = __builtin_amdgcn_udot4(rl, L[0], alo, false);
+            amid = __builtin_amdgcn_udot4(rl, L[1], amid, false);
+            atop = __builtin_amdgcn_sdot4((int)rl, (int)L[2], atop, false);
+        }
+        const float S = __builtin_fmaf((float)atop, 65536.0f, __builtin_fmaf((float)amid, 256.0f, (float)alo));
+        return mx_scale(ee) * (0.5f * __builtin_fmaf(xp.s, S, -16.0f * xp.xh0));     // xh0: s * sum(X), see prep_convert_quarter
+    }
+};
+
 // The formats without paired units never call idot_pair.
 template <typename IU>
 __device__ __forceinline__ float idot_pair_of(const IU &u, const XPrep &xe, const XPrep &xo)
@@ -1399,7 +1466,7 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
                 for (int i = 0; i < 8; i++) { ssq = __builtin_fmaf(xv[c][i], xv[c][i], ssq); xv[c][i] *= nv[c][i]; }
             }
         }
-        if (prep[c]) prep_convert_quarter<IU::NIBBLE, IU::TOPOFF>(xv[c], h & 3, xlds + (size_t)(h >> 2) * 28);
+        if (prep[c]) prep_convert_quarter<IU::NIBBLE, IU::TOPOFF, WantsQSum<FMT>::value>(xv[c], h & 3, xlds + (size_t)(h >> 2) * 28);
     }
     __shared__ float ssq_part[WAVES];
     if constexpr (FUSE) {
@@ -1833,8 +1900,10 @@ template <> struct HasIdot<RFQ_GGUF_Q6_K> { static constexpr bool value = true; 
 template <> struct HasIdot<RFQ_MM_Q4_K> { static constexpr bool value = true; };
 template <> struct HasIdot<RFQ_MM_Q8_0> { static constexpr bool value = true; };
 template <> struct HasIdot<RFQ_Q6_K> { static constexpr bool value = true; };
+template <> struct HasIdot<RFQ_MXFP4> { static constexpr bool value = true; };
 template <int FMT> struct HasIdotBatch { static constexpr bool value = HasIdot<FMT>::value; };
 template <> struct HasIdotBatch<RFQ_Q6_K> { static constexpr bool value = false; };   // batches keep one decode launch per vector
+template <> struct HasIdotBatch<RFQ_MXFP4> { static constexpr bool value = false; };
 
 template <int FMT, int UPL, int WPR, int R, bool FUSE>
 int launch_idot(const uint8_t *w, const float *x, float *y, int n, int k, int blocks, int groups, const GemvFuse &f,
@@ -2010,6 +2079,18 @@ int run_rows(const uint8_t *w, const float *x, float *y, int n, int k, const Gem
     // The 256-byte Q6_K layout has both kernels, a few per cent apart either way (measured on 14336, 11008, 4096 and
     // 32000 rows of 4096, 4096 rows of 8192 and of 14336): the integer-dot one where a team walks a single group of rows
     // of 65..128 units or rows longer than 256 units, the float one elsewhere and in the fused forms.
+    // MXFP4 has both kernels too: the integer-dot one for few rows (up to 16 per CU: 4096 x 4096 5.5 -> 4.9 us) and for
+    // rows longer than 256 units (4096 x 14336 13.4 -> 11.7 us); elsewhere the two are level or the float one (code
+    // values from a table in LDS) is ahead (32000 x 4096 20.1 against 21.7 us), and the fused forms keep it.
+    if constexpr (FMT == RFQ_MXFP4) {
+        if (FUSE || !(ku > 256 || n <= device_cu_count() * 16)) {
+            if (ku <= 64) return run_idot<FMT, 1, 1, FUSE>(w, x, y, n, k, f, s, false);
+            if (!FUSE && ku <= 128 && n >= device_cu_count() * 32) return run_idot<FMT, 1, 2, FUSE>(w, x, y, n, k, f, s, false);
+            if (ku <= 128) return run_idot<FMT, 2, 1, FUSE>(w, x, y, n, k, f, s, false);
+            if (ku <= 256) return run_idot<FMT, 2, 2, FUSE>(w, x, y, n, k, f, s, false);
+            return run_idot<FMT, 2, 4, FUSE>(w, x, y, n, k, f, s, false);
+        }
+    }
     if constexpr (FMT == RFQ_Q6_K) {
         const int cus = device_cu_count();
         if (FUSE || !((ku > 64 && ku <= 128 && n >= cus * 56 && n <= cus * 64) || ku > 256)) {
