@@ -137,9 +137,11 @@ template <int FMT> struct Unit;
 // ---- pieces that do not start on a multiple of 4 ------------------------------------------
 // A 16-byte load from an address that is not a multiple of 4 runs at a fraction of the aligned rate on this part
 // (17-byte blocks streamed as stored, a byte and 16 bytes per lane: 9.2 us for 31 MB; through aligned windows of whole
-// dwords: 6.8 us).  For the units whose kernels are bound by their instructions the byte permutes that move a window
-// into place cost more than the loads gain (measured: MXFP4 / MXFP6 / GGUF_Q4_0 / GGUF_Q8_0 GEMV 1..5 % slower with
-// windows); the 210-byte GGUF_Q6_K block, two 32-byte pieces per unit at 2-byte alignment, gains 3 %.
+// dwords: 6.8 us).  The units of the layouts whose blocks start at odd or 2-byte offsets (MXFP4 17 bytes, MXFP6 25,
+// GGUF_Q4_0 18, GGUF_Q8_0 34, GGUF_Q6_K 210) are therefore fetched as the aligned dwords that hold them and moved
+// into place with byte permutes, the lane's byte offset in the selector: 14336 x 4096 MXFP6 14.2 -> 13.4 us, GGUF_Q8_0
+// 15.0 -> 13.1 us; 128256 x 4096 MXFP6 108 -> 93 us, GGUF_Q4_0 75 -> 57 us, GGUF_Q8_0 138 -> 101 us (GGUF_Q4_0 14336 x
+// 4096 alone measured 3 % slower, 9.5 -> 9.7 us).
 template <int NW> __device__ __forceinline__ void load_dwords_a4(const uint8_t *a, uint32_t (&d)[NW])
 {
     typedef uint32_t v4a4 __attribute__((ext_vector_type(4), aligned(4)));
@@ -171,8 +173,27 @@ __device__ __forceinline__ U8 load32_a2(const uint8_t *c)
     return r;
 }
 
+// A piece of 4 * NQ bytes that starts `skip` bytes into a block at any byte address p (an exponent byte in front of
+// the codes): the NQ + 1 dwords from the multiple of 4 at or before p, the piece moved into place with byte permutes.
+// Returns the byte offset of p in the first dword.  With skip >= 1 every dword read holds at least one byte of the
+// block (the last one starts at or before the piece's last byte), so a window never touches a dword that lies wholly
+// outside the tensor.
+template <int NQ> __device__ __forceinline__ uint32_t load_window(const uint8_t *p, uint32_t skip, uint32_t &first, uint32_t (&q)[NQ])
+{
+    const uint32_t o = (uint32_t)(reinterpret_cast<uintptr_t>(p) & 3u);
+    uint32_t d[NQ + 1];
+    load_dwords_a4<NQ + 1>(p - o, d);
+    const uint32_t sel = 0x03020100u + 0x01010101u * (o + skip);        // skip + o <= 4: bytes of a dword pair
+#pragma unroll
+    for (int i = 0; i < NQ; i++) q[i] = __builtin_amdgcn_perm(d[i + 1], d[i], sel);
+    first = d[0];
+    return o;
+}
+
 template <int FMT> struct NeedsAlignedTensor { static constexpr bool value = false; };
 template <> struct NeedsAlignedTensor<RFQ_GGUF_Q6_K> { static constexpr bool value = true; };
+template <> struct NeedsAlignedTensor<RFQ_GGUF_Q4_0> { static constexpr bool value = true; };   // (blocks at even offsets
+template <> struct NeedsAlignedTensor<RFQ_GGUF_Q8_0> { static constexpr bool value = true; };   // of the window's first dword)
 
 template <> struct Unit<RFQ_Q4_0> {
     static constexpr bool NEEDS_XSUM = true;
@@ -308,11 +329,12 @@ template <int FMT> __device__ __forceinline__ void unit_tables_init()
 template <> struct Unit<RFQ_MXFP4> {
     static constexpr bool NEEDS_XSUM = false;
     int e; U4 q;
+    // (a 17-byte unit starts at any byte address: through an aligned window, see load_window)
     __device__ __forceinline__ void load(const uint8_t *row, int u)
     {
-        const uint8_t *p = row + (size_t)u * 17;
-        e = (int)(int8_t)p[0];
-        q = ld<U4>(p + 1);
+        uint32_t first;
+        const uint32_t o = load_window<4>(row + (size_t)u * 17, 1u, first, q.v);
+        e = __builtin_amdgcn_sbfe((int)first, 8u * o, 8u);
     }
     template <bool CLAMP> __device__ __forceinline__ float dot_as(const float (&x)[32]) const
     {
@@ -346,9 +368,9 @@ template <> struct Unit<RFQ_MXFP6_E2M3> {
     int e; U6 q;
     __device__ __forceinline__ void load(const uint8_t *row, int u)
     {
-        const uint8_t *p = row + (size_t)u * 25;
-        e = (int)(int8_t)p[0];
-        q = ld<U6>(p + 1);
+        uint32_t first;
+        const uint32_t o = load_window<6>(row + (size_t)u * 25, 1u, first, q.v);
+        e = __builtin_amdgcn_sbfe((int)first, 8u * o, 8u);
     }
     template <bool CLAMP> __device__ __forceinline__ float dot_as(const float (&x)[32]) const
     {
@@ -397,6 +419,12 @@ template <> struct Unit<RFQ_GGUF_Q4_0> {
     uint16_t d; U4 q;
     __device__ __forceinline__ void load(const uint8_t *row, int u)
     {
+        uint32_t first;
+        const uint32_t o = load_window<4>(row + (size_t)u * 18, 2u, first, q.v);   // o = 0 or 2 (see NeedsAlignedTensor)
+        d = (uint16_t)(first >> (8u * o));
+    }
+    __device__ __forceinline__ void load_bytes(const uint8_t *row, int u)
+    {
         const uint8_t *p = row + (size_t)u * 18;
         d = ld<uint16_t>(p);
         q = ld<U4>(p + 2);
@@ -422,6 +450,12 @@ template <> struct Unit<RFQ_GGUF_Q8_0> {
     static constexpr bool NEEDS_XSUM = true;
     uint16_t d; U8 q;
     __device__ __forceinline__ void load(const uint8_t *row, int u)
+    {
+        uint32_t first;
+        const uint32_t o = load_window<8>(row + (size_t)u * 34, 2u, first, q.v);   // o = 0 or 2 (see NeedsAlignedTensor)
+        d = (uint16_t)(first >> (8u * o));
+    }
+    __device__ __forceinline__ void load_bytes(const uint8_t *row, int u)
     {
         const uint8_t *p = row + (size_t)u * 34;
         d = ld<uint16_t>(p);
@@ -1316,46 +1350,103 @@ template <> struct IUnit<RFQ_Q6_K> : Unit<RFQ_Q6_K> {
 // positive, so a residue common to all rows would add up over a column of outputs).  Element 2j is the HIGH nibble of byte j.  The +-8 clamp
 // of the reference bites only for exponents >= 1, where it is a bound 2^(4 - e) on the doubled value (from e = 4 on
 // every value but 0 sits at the bound and the unit's scale is 8): such units rebuild their tables with that bound.
+// MXFP4.  The codes 0..7 decode to {0, 1, 1, 2, 2, 4, 4, 8} and 8..15 to -{1/2, 1, 1, 2, 2, 4, 4, 8}
+// (MxfpBlock::decode_e2m1, src/loader/mxfp.rs:234-244: 0 for code 0, otherwise sign * (1 + mant) * 2^(exp - 1)), so
+// 16 + 2 * value is a byte.  A weight byte holds two
+// codes (elements 2i in the high, 2i+1 in the low nibble) and is translated to its two value bytes by ONE 16-bit
+// load from a 256-entry table in LDS; two look-ups, joined by a shift-or, make the four bytes that v_dot4 multiplies
+// with four consecutive elements of x (the loads that write only one half of a register are of no use here: with
+// ECC on the register file they clear the other half).  The table is replicated per lane (entry stride 256 bytes =
+// 64 lanes x 4) so that no two lanes of a look-up meet in a bank, and the address is entry * 256 + lane * 4: one
+// v_perm_b32 per look-up.  16 address + 16 LDS + 8 join + 24 dot instructions per 32 weights, where spreading the
+// codes with v_perm_b32 tables in registers took 56 + 24.
+// The reference clamps value * scale to +-8 (mxfp.rs:196-203), which changes a value only when the exponent is >= 1;
+// a wavefront that holds such a unit (one ballot) takes the slower path that builds clamped tables in registers.
+constexpr size_t MX4_LUT_BYTES = 256 * 256;
+
+// 16 + 2 * decode_e2m1(code)
+__device__ __forceinline__ uint32_t mx4_value_byte(uint32_t code)
+{
+    const uint32_t t = code == 0u ? 0u : 1u << (((code & 7u) + 1u) >> 1);
+    return (code & 8u) ? 16u - t : 16u + t;
+}
+
+// Fills the block's table: entry b, replicated over the 64 lane slots, holds the value bytes of b's high nibble (low
+// byte) and low nibble (next byte).
+template <int THREADS> __device__ __forceinline__ void mx4_fill_lut(uint32_t *lut, int tid)
+{
+    static_assert(THREADS == 512, "eight 16-byte pieces (four lane slots of one entry) per thread");
+    // piece tid + 512 j belongs to entry b = (tid >> 4) + 32 j: its low nibble is the thread's own, its high nibble
+    // 2 j + (tid >> 8), one of two neighbouring bytes of the value bytes of the sixteen codes
+    constexpr uint64_t POS = 0x2018181414121210ull, NEG = 0x0008080C0C0E0E0Full;
+    const uint32_t second = mx4_value_byte(((uint32_t)tid >> 4) & 15u) << 8;
+    const uint32_t odd = ((uint32_t)tid >> 8) * 8u;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        const uint32_t two = (uint32_t)(((j < 4 ? POS : NEG) >> (16 * (j & 3))) & 0xFFFFu);
+        const uint32_t v = second | __builtin_amdgcn_ubfe(two, odd, 8u);
+        reinterpret_cast<uint4 *>(lut)[tid + THREADS * j] = make_uint4(v, v, v, v);
+    }
+}
+
 template <> struct IUnit<RFQ_MXFP4> : Unit<RFQ_MXFP4> {
     static constexpr bool PAIR = false;
-    static constexpr bool NIBBLE = true;
+    static constexpr bool NIBBLE = false;                                // x limbs in plain element order
     static constexpr uint32_t TOPOFF = 0;
     static __device__ __forceinline__ uint32_t pack4(uint32_t a, uint32_t b, uint32_t c, uint32_t d) { return a | (b << 8) | (c << 16) | (d << 24); }
-    __device__ __forceinline__ float idot(const XPrep &xp) const
+    static __device__ __forceinline__ void dot3(uint32_t r, const uint32_t *L, uint32_t &alo, uint32_t &amid, int &atop)
     {
-        uint32_t plo = 0x14121210u, phi = 0x20181814u;               // 16 + {0, 2, 2, 4 | 4, 8, 8, 16}
-        uint32_t nlo = 0x0C0E0E0Fu, nhi = 0x0008080Cu;               // 16 - {1, 2, 2, 4 | 4, 8, 8, 16}
-        int ee = e;
-        if (__builtin_amdgcn_ballot_w64(e >= 1) != 0) {              // (weights below 1 never have such a unit)
-            const uint32_t b = e <= 0 ? 16u : (e >= 4 ? 1u : (16u >> e));
-            auto lim = [&](uint32_t m) { return m < b ? m : b; };
-            plo = pack4(16u, 16u + lim(2), 16u + lim(2), 16u + lim(4));
-            phi = pack4(16u + lim(4), 16u + lim(8), 16u + lim(8), 16u + lim(16));
-            nlo = pack4(16u - lim(1), 16u - lim(2), 16u - lim(2), 16u - lim(4));
-            nhi = pack4(16u - lim(4), 16u - lim(8), 16u - lim(8), 16u - lim(16));
-            ee = e > 4 ? 4 : e;
-        }
+        alo = __builtin_amdgcn_udot4(r, L[0], alo, false);
+        amid = __builtin_amdgcn_udot4(r, L[1], amid, false);
+        atop = __builtin_amdgcn_sdot4((int)r, (int)L[2], atop, false);
+    }
+    // The two value bytes of the weight byte whose table slot is at LDS address a.
+    static __device__ __forceinline__ uint32_t lut_at(uint32_t a)
+    {
+        return *reinterpret_cast<const uint16_t __attribute__((address_space(3))) *>((uintptr_t)a);
+    }
+    // slot: the LDS address of this lane's slot of entry 0 of the block's table (mx4_fill_lut), the table at a
+    // multiple of 64 KiB: entry b's slot is then `slot` with b as its second byte.
+    __device__ __forceinline__ float idot_lut(const XPrep &xp, uint32_t slot) const
+    {
         uint32_t alo = 0, amid = 0;
         int atop = 0;
+        int ee = e;
+        if (__builtin_amdgcn_ballot_w64(e >= 1) == 0) {
 #pragma unroll
-        for (int d = 0; d < 4; d++) {
-            const uint32_t x = q.v[d];
-            const uint32_t sl = x & 0x07070707u, sh = (x >> 4) & 0x07070707u;
-            const uint32_t ml = __builtin_amdgcn_perm(x << 4, x << 12, 0x0B090A08u);   // 0xFF where the low code's sign bit is set
-            const uint32_t mh = __builtin_amdgcn_perm(x, x << 8, 0x0B090A08u);         // likewise for the high code
-            const uint32_t pl = __builtin_amdgcn_perm(phi, plo, sl), nl = __builtin_amdgcn_perm(nhi, nlo, sl);
-            const uint32_t ph = __builtin_amdgcn_perm(phi, plo, sh), nh = __builtin_amdgcn_perm(nhi, nlo, sh);
-            const uint32_t rl = (ml & nl) | (~ml & pl), rh = (mh & nh) | (~mh & ph);
-            const uint32_t *H = &xp.l[(2 * d) * 3], *L = &xp.l[(2 * d + 1) * 3];      // elements 8d + {0, 2, 4, 6} / {1, 3, 5, 7}
-            alo = __builtin_amdgcn_udot4(rh, H[0], alo, false);
-            amid = __builtin_amdgcn_udot4(rh, H[1], amid, false);
-            atop = __builtin_amdgcn_sdot4((int)rh, (int)H[2], atop, false);
-            alo = __builtin_amdgcn_udot4(rl, L[0], alo, false);
-            amid = __builtin_amdgcn_udot4(rl, L[1], amid, false);
-            atop = __builtin_amdgcn_sdot4((int)rl, (int)L[2], atop, false);
+            for (int d = 0; d < 4; d++) {
+                const uint32_t x = q.v[d];
+                const uint32_t t0 = lut_at(__builtin_amdgcn_perm(x, slot, 0x03020400u)), t1 = lut_at(__builtin_amdgcn_perm(x, slot, 0x03020500u));
+                const uint32_t t2 = lut_at(__builtin_amdgcn_perm(x, slot, 0x03020600u)), t3 = lut_at(__builtin_amdgcn_perm(x, slot, 0x03020700u));
+                dot3(t0 | (t1 << 16), &xp.l[(2 * d) * 3], alo, amid, atop);
+                dot3(t2 | (t3 << 16), &xp.l[(2 * d + 1) * 3], alo, amid, atop);
+            }
+        } else {                                                         // (weights below 1 never have such a unit)
+            // magnitudes capped at 8 / 2^e in units of 1/2: tables 16 + {0, 2, 2, 4 | 4, 8, 8, 16}, 16 - {1, 2, 2, 4 | 4, 8, 8, 16}
+            const uint32_t b = e <= 0 ? 16u : (e >= 4 ? 1u : (16u >> e));
+            auto lim = [&](uint32_t m) { return m < b ? m : b; };
+            const uint32_t plo = pack4(16u, 16u + lim(2), 16u + lim(2), 16u + lim(4));
+            const uint32_t phi = pack4(16u + lim(4), 16u + lim(8), 16u + lim(8), 16u + lim(16));
+            const uint32_t nlo = pack4(16u - lim(1), 16u - lim(2), 16u - lim(2), 16u - lim(4));
+            const uint32_t nhi = pack4(16u - lim(4), 16u - lim(8), 16u - lim(8), 16u - lim(16));
+            ee = e > 4 ? 4 : e;
+#pragma unroll
+            for (int d = 0; d < 4; d++) {
+                const uint32_t x = q.v[d];
+                const uint32_t sl = x & 0x07070707u, sh = (x >> 4) & 0x07070707u;
+                const uint32_t ml = __builtin_amdgcn_perm(x << 4, x << 12, 0x0B090A08u);   // 0xFF where the low code's sign bit is set
+                const uint32_t mh = __builtin_amdgcn_perm(x, x << 8, 0x0B090A08u);         // likewise for the high code
+                const uint32_t pl = __builtin_amdgcn_perm(phi, plo, sl), nl = __builtin_amdgcn_perm(nhi, nlo, sl);
+                const uint32_t ph = __builtin_amdgcn_perm(phi, plo, sh), nh = __builtin_amdgcn_perm(nhi, nlo, sh);
+                const uint32_t rl = (ml & nl) | (~ml & pl), rh = (mh & nh) | (~mh & ph);   // odd / even elements of 8d .. 8d+7
+                dot3(__builtin_amdgcn_perm(rl, rh, 0x05010400u), &xp.l[(2 * d) * 3], alo, amid, atop);
+                dot3(__builtin_amdgcn_perm(rl, rh, 0x07030602u), &xp.l[(2 * d + 1) * 3], alo, amid, atop);
+            }
         }
         const float S = __builtin_fmaf((float)atop, 65536.0f, __builtin_fmaf((float)amid, 256.0f, (float)alo));
-        return mx_scale(ee) * (0.5f * __builtin_fmaf(xp.s, S, -16.0f * xp.xh0));     // xh0: s * sum(X), see prep_convert_quarter
+        // xh0: s * sum(X), see prep_convert_quarter; the scale of exponent -128 is 0 (mx_scale)
+        const float v = __builtin_fmaf(0.5f * xp.s, S, -8.0f * xp.xh0);
+        return __builtin_ldexpf(v, ee == -128 ? -300 : ee);
     }
 };
 
@@ -1392,8 +1483,10 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
     // measured 3..7 there at 14336 x 4096: 11.58, 11.41, 11.30, 11.72, 11.95 us)
     constexpr int DW = (UPL == 1 && WPR == 2) ? 5 : 3;
     constexpr int D = R < DW ? R : DW;
-    extern __shared__ __attribute__((aligned(16))) uint32_t xlds[]; // [units][28]
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    extern __shared__ __attribute__((aligned(16))) uint32_t idot_lds[]; // (MXFP4: the code table,) [units][28]
+    constexpr size_t LUT_DWORDS = FMT == RFQ_MXFP4 ? MX4_LUT_BYTES / 4 : 0;
+    uint32_t *const xlds = idot_lds + LUT_DWORDS;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int team = wave / WPR, wit = wave % WPR;
     const int tl = wit * 64 + lane;
     const int ku = k >> 5;
@@ -1455,6 +1548,8 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
 #pragma unroll
     for (int d = 0; d < D; d++) load_row(d, d);
 
+    if constexpr (FMT == RFQ_MXFP4) mx4_fill_lut<THREADS>(idot_lds, threadIdx.x);
+
     // Cooperative conversion of x: 4*ku quarter-units (eight values each) over the block's threads.
     float ssq = 0.f;
 #pragma unroll
@@ -1468,7 +1563,19 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
         }
         if (prep[c]) prep_convert_quarter<IU::NIBBLE, IU::TOPOFF, WantsQSum<FMT>::value>(xv[c], h & 3, xlds + (size_t)(h >> 2) * 28);
     }
-    __shared__ float ssq_part[WAVES];
+    // With the table the block keeps no static LDS (the table then starts at LDS address 0 and a look-up address
+    // needs no base added): the partial sums follow the prepared x in the dynamic part.
+    float *ssq_part;
+    float (*part)[R][WAVES];
+    if constexpr (LUT_DWORDS != 0) {
+        part = reinterpret_cast<float (*)[R][WAVES]>(xlds + (size_t)ku * 28);
+        ssq_part = reinterpret_cast<float *>(part + 2);
+    } else {
+        __shared__ float ssq_part_static[WAVES];
+        __shared__ float part_static[2][R][WAVES];
+        ssq_part = ssq_part_static;
+        part = part_static;
+    }
     if constexpr (FUSE) {
         if (norm) {
             ssq = wave_sum(ssq);
@@ -1507,7 +1614,9 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
     // load in flight behind it.  Only the group size that long walks choose is compiled this way (the same ring
     // measured on the other forms and on the float kernel gained 0..2 % or lost).
     constexpr bool RING = R == 5 && D == 5;
-    __shared__ float part[2][R][WAVES];
+    // (a kernel with the table has no static LDS, which launch_idot checks: the table starts at LDS address 0)
+    const uint32_t lut_slot = (uint32_t)(uintptr_t)idot_lds + 4u * (uint32_t)lane;
+    (void)lut_slot;
     for (int g = 0; g < groups; g++) {
         const int base = g * R;
         if (!RING && g > 0) {
@@ -1524,7 +1633,9 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
             } else {
 #pragma unroll
                 for (int j = 0; j < UPL; j++) {
-                    float t = buf[i % D][j].idot(xp[j]);
+                    float t;
+                    if constexpr (FMT == RFQ_MXFP4) t = buf[i % D][j].idot_lut(xp[j], lut_slot);
+                    else t = buf[i % D][j].idot(xp[j]);
                     acc += live[j] ? t : 0.f;
                 }
             }
@@ -1910,6 +2021,22 @@ int launch_idot(const uint8_t *w, const float *x, float *y, int n, int k, int bl
                 hipStream_t s)
 {
     size_t lds = (size_t)(k / 32) * 28 * sizeof(uint32_t);
+    if constexpr (FMT == RFQ_MXFP4) {
+        lds += MX4_LUT_BYTES + (2 * R + 1) * IDOT_WAVES * sizeof(float);   // the table; partial sums (no static LDS)
+        static std::once_flag once;
+        static hipError_t attr_err = hipSuccess;
+        static bool table_at_zero = false;
+        std::call_once(once, [] {
+            const void *kernel = reinterpret_cast<const void *>(&gemv_idot_kernel<FMT, UPL, WPR, R, FUSE>);
+            hipFuncAttributes fa;
+            attr_err = hipFuncGetAttributes(&fa, kernel);
+            if (attr_err != hipSuccess) return;
+            table_at_zero = fa.sharedSizeBytes == 0;                     // no static LDS in front of the table
+            attr_err = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 4096);
+        });
+        if (attr_err != hipSuccess) return hip_fail(attr_err, "hipFuncSetAttribute(gemv_idot_kernel)");
+        if (!table_at_zero) return run_xreg<FMT, UPL, WPR, FUSE>(w, x, y, n, k, f, s);   // (not expected: the float kernel)
+    }
     note_kernel(FUSE ? "gemv_idot_kernel<%s,%d,%d,%d,fused>" : "gemv_idot_kernel<%s,%d,%d,%d>", FMT, UPL, WPR, R);
     hipLaunchKernelGGL((gemv_idot_kernel<FMT, UPL, WPR, R, FUSE>), dim3(blocks), dim3(64 * IDOT_WAVES), lds, s, w, x, y, n, k, groups,
                        f);
@@ -2079,11 +2206,13 @@ int run_rows(const uint8_t *w, const float *x, float *y, int n, int k, const Gem
     // The 256-byte Q6_K layout has both kernels, a few per cent apart either way (measured on 14336, 11008, 4096 and
     // 32000 rows of 4096, 4096 rows of 8192 and of 14336): the integer-dot one where a team walks a single group of rows
     // of 65..128 units or rows longer than 256 units, the float one elsewhere and in the fused forms.
-    // MXFP4 has both kernels too: the integer-dot one for few rows (up to 16 per CU: 4096 x 4096 5.5 -> 4.9 us) and for
-    // rows longer than 256 units (4096 x 14336 13.4 -> 11.7 us); elsewhere the two are level or the float one (code
-    // values from a table in LDS) is ahead (32000 x 4096 20.1 against 21.7 us), and the fused forms keep it.
+    // MXFP4 has both kernels too: the integer-dot one for few rows (up to 16 per CU: 4096 x 4096 6.1 -> 5.5 us), for
+    // rows longer than 128 units (4096 x 8192 8.7 -> 8.0 us, 4096 x 14336 12.4 -> 12.0 us) and around 56 rows per CU
+    // (14336 x 4096 10.4 -> 10.2 us); elsewhere the float one (code values from a table of floats in LDS) is ahead
+    // (11008 x 4096 9.8 against 10.2 us, 32000 x 4096 17.2 against 18.8 us), and the fused forms keep it.
     if constexpr (FMT == RFQ_MXFP4) {
-        if (FUSE || !(ku > 256 || n <= device_cu_count() * 16)) {
+        const int cus = device_cu_count();
+        if (FUSE || !(ku > 128 || n <= cus * 16 || (n >= cus * 52 && n <= cus * 64))) {
             if (ku <= 64) return run_idot<FMT, 1, 1, FUSE>(w, x, y, n, k, f, s, false);
             if (!FUSE && ku <= 128 && n >= device_cu_count() * 32) return run_idot<FMT, 1, 2, FUSE>(w, x, y, n, k, f, s, false);
             if (ku <= 128) return run_idot<FMT, 2, 1, FUSE>(w, x, y, n, k, f, s, false);
@@ -2230,9 +2359,10 @@ int launch_gemv_fused(int fmt, const uint8_t *d_w, const uint8_t *d_w2, const fl
     if (k % fmt_block_elems(fmt) != 0) return RFQ_E_UNSUPPORTED;
     const GemvFuse f{d_w2, d_norm_w, eps, d_w2 != nullptr ? 1 : 0};
     const int rows = d_w2 != nullptr ? 2 * n : n;
-    // (GGUF_Q6_K pieces are fetched through aligned windows: both matrices must start on a multiple of 4, else the
-    // caller composes the separate steps, which take the byte-exact kernel)
-    if (canonical_format(fmt) == RFQ_GGUF_Q6_K &&
+    // (the 2-byte aligned GGUF blocks are fetched through aligned windows: both matrices must start on a multiple of
+    // 4, else the caller composes the separate steps, which take the byte-exact kernel)
+    const int cf = canonical_format(fmt);
+    if ((cf == RFQ_GGUF_Q6_K || cf == RFQ_GGUF_Q4_0 || cf == RFQ_GGUF_Q8_0) &&
         ((reinterpret_cast<uintptr_t>(d_w) | (d_w2 ? reinterpret_cast<uintptr_t>(d_w2) : 0)) & 3u) != 0)
         return RFQ_E_UNSUPPORTED;
     switch (canonical_format(fmt)) {

@@ -212,8 +212,8 @@ def test_long_matrices_one_unit_per_lane(fmt, n, k, oracle, cuda):
     assert_close(got, oracle.qmatmul_nk(fmt, w, x, 1, n, k), f"{Q.NAMES[fmt]} {n}x{k}")
 
 
-# The 17-, 25-, 18-, 34- and 210-byte layouts are read in place at whatever alignment their blocks have (the 210-byte
-# one through aligned windows of whole dwords when the tensor starts on a multiple of 4, byte-exactly otherwise):
+# The 17-, 25-, 18-, 34- and 210-byte layouts are read in place at whatever alignment their blocks have, through
+# aligned windows of whole dwords (the GGUF ones when the tensor starts on a multiple of 4, byte-exactly otherwise):
 # weights at odd device addresses, and tensors whose byte count is not a multiple of 4, must agree with the oracle.
 @pytest.mark.parametrize("fmt", [Q.MXFP4, Q.MXFP6_E2M3, Q.GGUF_Q4_0, Q.GGUF_Q8_0, Q.GGUF_Q6_K])
 def test_gemv_windowed_layouts_at_any_address(fmt, oracle, cuda):
