@@ -93,6 +93,53 @@ class GemvRun:
         return wall, ms.value / 1e3
 
 
+TIMELINE_POINTS = ["wavefront started", "x and first rows requested, x arrived", "x converted (before the barrier)", "past the barrier",
+                   "prepared x of its units in registers"] + \
+                  [t for i in range(7) for t in (f"row {i} in registers", f"row {i} reduced")] + ["results stored"]
+
+
+def gemv_timeline(torch, fmt, n, k, copies, warmup, Q, seed):
+    """One launch of the decode GEMV with every wavefront stamping the constant 100 MHz clock at fixed points
+    (rfq_bench_gemv_timeline), after `warmup` ordinary launches over the rotating weight copies.  Returns the kernel
+    name and the stamps in microseconds after the first wavefront's start, shape [wavefronts, points], or None when
+    the kernel this shape takes has no such build."""
+    import ctypes as C
+
+    import numpy as np
+    from rocmforge_amd import _lib
+    g = GemvRun(torch, fmt, n, k, 1, copies, Q, seed)
+    cap = 1 << 16
+    trace = torch.zeros((cap, 20), dtype=torch.int64, device="cuda:0")
+    waves, stamps = C.c_int(0), C.c_int(0)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    _lib.check(_lib.lib().rfq_bench_gemv_timeline(fmt, g.ptrs, copies, g.w.size, C.c_void_p(g.dx.data_ptr()), C.c_void_p(g.y.data_ptr()),
+                                                  n, k, warmup, stream, C.c_void_p(trace.data_ptr()), cap, C.byref(waves), C.byref(stamps)))
+    torch.cuda.synchronize()
+    kern = _lib.lib().rfq_bench_last_gemv_kernel().decode()
+    if waves.value == 0:
+        return kern, None
+    assert stamps.value == 20
+    t = trace[:waves.value].cpu().numpy().astype(np.float64)
+    return kern, (t - t[:, 0].min()) / 100.0                # 100 MHz ticks -> microseconds
+
+
+def print_timeline(name, n, k, kern, us, warmup):
+    import numpy as np
+    print(f"# {name} decode GEMV {n} x {k}: one launch of {kern} after {warmup} ordinary launches; {us.shape[0]} wavefronts;")
+    print("# microseconds after the first wavefront's start (constant 100 MHz clock, 10 ns a tick): the point was reached by")
+    print(f"# {'point':42s} {'first':>7s} {'10 %':>7s} {'median':>7s} {'90 %':>7s} {'last':>7s}")
+    for i, label in enumerate(TIMELINE_POINTS):
+        c = us[:, i]
+        print(f"  {label:42s} {c.min():7.2f} {np.percentile(c, 10):7.2f} {np.median(c):7.2f} {np.percentile(c, 90):7.2f} {c.max():7.2f}")
+    d = lambda a, b: np.median(us[:, a] - us[:, b])
+    print("# median over wavefronts of the time between points:")
+    print(f"  start -> requests issued and x arrived {d(1, 0):.2f}; conversion {d(2, 1):.2f}; wait at the barrier {d(3, 2):.2f}; prepared x {d(4, 3):.2f};")
+    print("  row i: wait for its bytes / dot products and reduction: " +
+          "  ".join(f"{d(5 + 2 * i, 4 + 2 * i):.2f} / {d(6 + 2 * i, 5 + 2 * i):.2f}" for i in range(7)))
+    print(f"  store {d(19, 18):.2f}; a wavefront's life {np.median(us[:, 19] - us[:, 0]):.2f}; first start to last store {us[:, 19].max():.2f}")
+
+
 def time_gemv(torch, fmt, n, k, m, copies, steps, warmup, Q, seed):
     """Returns (wall seconds, device seconds, w, x, y) for `steps` rfq_gemv calls."""
     g = GemvRun(torch, fmt, n, k, m, copies, Q, seed)
@@ -390,6 +437,8 @@ def main():
     ap.add_argument("--only-gguf", action="store_true", help="only the GGUF-layout Q4_K GEMV line (profiling runs)")
     ap.add_argument("--only-dequant", action="store_true", help="only the dequantisation lines (profiling runs)")
     ap.add_argument("--only-gemv", metavar="FMT:NxK:M", help="only one decode GEMV, e.g. MXFP4:14336x4096:1 (profiling runs)")
+    ap.add_argument("--timeline", metavar="FMT:NxK", help="where one decode GEMV launch spends its time, from clock readings "
+                    "inside the kernel, e.g. Q4_K:14336x4096 (text, not JSON)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build is single-GPU (one MI355X per box); run with --gpus 1. "
@@ -416,6 +465,18 @@ def main():
             res[name] = {"GB/s": round(b / t / 1e9, 1), "us": round(t * 1e6, 2), "hbm_frac": round(b / t / 1e9 / HBM_PEAK_GBS, 4),
                          "algorithmic_bytes": b}
         print(json.dumps(res))
+        return
+
+    if args.timeline:
+        name, shape = args.timeline.split(":")
+        f = {v: k_ for k_, v in Q.NAMES.items()}[name]
+        n_, k_ = (int(t) for t in shape.split("x"))
+        c = min(-(-int(2.5 * CACHE_BYTES) // Q.packed_bytes(f, n_ * k_)), 64)
+        kern, us = gemv_timeline(torch, f, n_, k_, c, args.warmup, Q, 20260061)
+        if us is None:
+            print(f"{kern}: no build of this kernel stamps its timeline")
+        else:
+            print_timeline(name, n_, k_, kern, us, args.warmup)
         return
 
     if args.only_gemv:

@@ -25,6 +25,21 @@ RFQ_API int rfq_bench_gemv(int fmt, const void *const *d_w_copies, int copies, s
                            float *d_y, int m, int n, int k, int warmup, int steps, void *stream,
                            float *elapsed_ms);
 
+/* Where the time of one decode GEMV launch (m = 1) goes, seen from inside the kernel: after `warmup` ordinary calls
+ * over the rotating weight copies, one launch of a build of the same kernel in which every wavefront reads the
+ * constant 100 MHz clock (s_memrealtime, 10 ns a tick) at fixed points and stores the readings; the call returns
+ * after the launch has finished.  d_trace (device memory, capacity_waves * 20 readings of 8 bytes) receives
+ * [wavefront][reading]: 0 wavefront started, 1 its part of x in registers (the reading stands behind the requests for
+ * x and for the first rows of weights, which issue in order and block while the CU's memory pipeline is full: with
+ * the loads of x removed it comes no earlier), 2 x converted (before the barrier),
+ * 3 past the barrier, 4 the prepared x of its units in registers, 5 + 2 i row i of its first group of rows in
+ * registers, 6 + 2 i row i reduced (i < 7), 19 the group's results stored.  *waves = wavefronts written, 0 when the
+ * kernel this format and shape take has no such build (Q4_K and MXFP4 with 65..128 units per row and seven rows
+ * per group, GGUF_Q4_K with seven rows per group: the 14336 x 4096 projections). */
+RFQ_API int rfq_bench_gemv_timeline(int fmt, const void *const *d_w_copies, int copies, size_t w_bytes, const float *d_x,
+                                    float *d_y, int n, int k, int warmup, void *stream, unsigned long long *d_trace,
+                                    size_t capacity_waves, int *waves, int *stamps_per_wave);
+
 /* Step i reads input copy i % copies and writes the n_elems floats at
  * d_out + (i % out_copies) * n_elems: with enough of both, neither the packed
  * input nor the previous output of the same lines sits in the last-level cache. */

@@ -65,6 +65,7 @@ _SIGNATURES = {
     "rfq_gemm_mx": ([_vp, _sz, _i, _vp, _sz, _i, _vp, _i, _i, _i, _i, _vp], _i),
     # include/rfq_bench.h
     "rfq_bench_gemv": ([_i, _vp, _i, _sz, _vp, _vp, _i, _i, _i, _i, _i, _vp, C.POINTER(C.c_float)], _i),
+    "rfq_bench_gemv_timeline": ([_i, _vp, _i, _sz, _vp, _vp, _i, _i, _i, _vp, _vp, _sz, C.POINTER(C.c_int), C.POINTER(C.c_int)], _i),
     "rfq_bench_dequant": ([_i, _vp, _i, _sz, _vp, _sz, _i, _i, _i, _vp, C.POINTER(C.c_float)], _i),
     "rfq_bench_gemm_f16": ([_i, _vp, _sz, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, C.POINTER(C.c_float)], _i),
     "rfq_bench_mlp_swiglu": ([_i, _vp, _vp, _sz, _i, _vp, _sz, _i, _vp, _vp, C.c_float, _vp, _i, _i, _i, _vp, _sz, _i, _i,

@@ -180,6 +180,25 @@ int rfq_bench_gemv(int fmt, const void *const *d_w_copies, int copies, size_t w_
     });
 }
 
+int rfq_bench_gemv_timeline(int fmt, const void *const *d_w_copies, int copies, size_t w_bytes, const float *d_x,
+                            float *d_y, int n, int k, int warmup, void *stream, unsigned long long *d_trace,
+                            size_t capacity_waves, int *waves, int *stamps_per_wave)
+{
+    if (!d_w_copies || copies <= 0 || !d_trace || !waves || !stamps_per_wave)
+        return rfq::fail(RFQ_E_BADARG, "rfq_bench_gemv_timeline: null argument");
+    *stamps_per_wave = rfq::GEMV_TRACE_STAMPS;
+    if (warmup < 1) warmup = 1;                          // (an ordinary call first: it checks the arguments)
+    for (int i = 0; i < warmup; i++) {
+        const int rc = rfq_gemv(fmt, d_w_copies[i % copies], w_bytes, d_x, d_y, 1, n, k, stream);
+        if (rc != RFQ_OK) return rc;
+    }
+    const int rc = rfq::launch_gemv_traced(fmt, (const uint8_t *)d_w_copies[warmup % copies], d_x, d_y, n, k, d_trace, capacity_waves,
+                                           waves, (hipStream_t)stream);
+    if (rc != RFQ_OK) return rc;
+    const hipError_t e = hipStreamSynchronize((hipStream_t)stream);
+    return e == hipSuccess ? RFQ_OK : rfq::hip_fail(e, "rfq_bench_gemv_timeline: hipStreamSynchronize");
+}
+
 int rfq_bench_dequant(int fmt, const void *const *d_in_copies, int copies, size_t packed_bytes, float *d_out,
                       size_t n_elems, int out_copies, int warmup, int steps, void *stream, float *elapsed_ms)
 {

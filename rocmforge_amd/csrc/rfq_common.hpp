@@ -96,6 +96,9 @@ int launch_rms_norm(int src_fmt, const void *d_x, const float *d_weight, float *
                     hipStream_t s);
 int launch_swiglu(const float *d_gate, const float *d_up, float *d_out, size_t total, hipStream_t s);
 int launch_gemv(int fmt, const uint8_t *d_w, const float *d_x, float *d_y, int m, int n, int k, hipStream_t s);
+constexpr int GEMV_TRACE_STAMPS = 20;                    // readings per wavefront, see WaveTrace in rfq_gemv.hip
+int launch_gemv_traced(int fmt, const uint8_t *d_w, const float *d_x, float *d_y, int n, int k, unsigned long long *d_trace,
+                       size_t capacity_waves, int *waves, hipStream_t s);
 // y[n] = sum_l x[l] * Wd[l * n + j] over the flat stream of n * k elements (one row of x).
 int launch_gemv_kn(int fmt, const uint8_t *d_w, const float *d_x, float *d_y, int n, int k, hipStream_t s);
 int launch_gemv_fused(int fmt, const uint8_t *d_w, const uint8_t *d_w2, const float *d_x, const float *d_norm_w,

@@ -155,40 +155,47 @@ template <int NW> __device__ __forceinline__ void load_dwords_a4(const uint8_t *
     for (; i < NW; i++) d[i] = *reinterpret_cast<const uint32_t *>(a + 4 * i);
 }
 
-// 32 bytes at a 2-byte aligned address inside a larger block: the window of 9 dwords from the multiple of 4 at or
-// before it, moved into place with byte permutes.  The 4 bytes read behind the piece belong to the same block; the
-// up to 2 bytes read before it stay inside the tensor as long as the tensor starts on a multiple of 4, which the
-// launcher checks (a tensor at another address takes the byte-exact load_bytes in the generic kernel).
-__device__ __forceinline__ U8 load32_a2(const uint8_t *c)
-{
-    // (stepping back from c rather than building a pointer from the masked integer: the loads stay global loads
-    // instead of flat ones, which also count against the LDS counter)
-    const uint8_t *a = c - (reinterpret_cast<uintptr_t>(c) & 3u);
-    const uint32_t sel = 0x03020100u + 0x01010101u * (uint32_t)(reinterpret_cast<uintptr_t>(c) & 3u);
-    uint32_t d[9];
-    load_dwords_a4<9>(a, d);
-    U8 r;
+// A piece of 4 * NQ bytes that starts SKIP bytes (a header: an exponent byte, an f16 scale) behind p, at any byte
+// address: the NQ + 1 dwords from the multiple of 4 at or before p are fetched, and the piece is moved into place with
+// byte permutes only where it is used -- permutes issued with the loads would make a wavefront wait for every row it
+// has in flight before it can touch the first.  With SKIP >= 1 every dword read holds a byte of the block; with
+// SKIP = 0 the last one can lie behind the piece (inside the block for the pieces this is used on).  The bytes read
+// before p stay inside the tensor when the tensor starts on a multiple of 4.
+template <int NQ> struct Window {
+    uint32_t d[NQ + 1], o;                               // o: the byte offset of p in d[0]
+    __device__ __forceinline__ void load(const uint8_t *p)
+    {
+        // (stepping back from p rather than building a pointer from the masked integer: the loads stay global loads
+        // instead of flat ones, which also count against the LDS counter)
+        o = (uint32_t)(reinterpret_cast<uintptr_t>(p) & 3u);
+        load_dwords_a4<NQ + 1>(p - o, d);
+    }
+    // The same content from byte-exact loads (a tensor at an address the windows cannot take).
+    template <uint32_t SKIP> __device__ __forceinline__ void load_bytes(const uint8_t *p)
+    {
+        static_assert(SKIP <= 2, "no header, a byte or two bytes");
+        struct Piece { uint32_t v[NQ]; };
+        const Piece q = ld<Piece>(p + SKIP);
+        if constexpr (SKIP == 0) {
+            o = 0;
 #pragma unroll
-    for (int i = 0; i < 8; i++) r.v[i] = __builtin_amdgcn_perm(d[i + 1], d[i], sel);
-    return r;
-}
-
-// A piece of 4 * NQ bytes that starts `skip` bytes into a block at any byte address p (an exponent byte in front of
-// the codes): the NQ + 1 dwords from the multiple of 4 at or before p, the piece moved into place with byte permutes.
-// Returns the byte offset of p in the first dword.  With skip >= 1 every dword read holds at least one byte of the
-// block (the last one starts at or before the piece's last byte), so a window never touches a dword that lies wholly
-// outside the tensor.
-template <int NQ> __device__ __forceinline__ uint32_t load_window(const uint8_t *p, uint32_t skip, uint32_t &first, uint32_t (&q)[NQ])
-{
-    const uint32_t o = (uint32_t)(reinterpret_cast<uintptr_t>(p) & 3u);
-    uint32_t d[NQ + 1];
-    load_dwords_a4<NQ + 1>(p - o, d);
-    const uint32_t sel = 0x03020100u + 0x01010101u * (o + skip);        // skip + o <= 4: bytes of a dword pair
+            for (int i = 0; i < NQ; i++) d[i] = q.v[i];
+            d[NQ] = 0;
+        } else {
+            o = 4u - SKIP;
+            d[0] = (SKIP == 1 ? (uint32_t)p[0] : (uint32_t)ld<uint16_t>(p)) << (8u * o);
 #pragma unroll
-    for (int i = 0; i < NQ; i++) q[i] = __builtin_amdgcn_perm(d[i + 1], d[i], sel);
-    first = d[0];
-    return o;
-}
+            for (int i = 0; i < NQ; i++) d[i + 1] = q.v[i];
+        }
+    }
+    template <uint32_t SKIP> __device__ __forceinline__ void piece(uint32_t (&q)[NQ]) const
+    {
+        const uint32_t sel = 0x03020100u + 0x01010101u * (o + SKIP);    // o + SKIP <= 4: bytes of a dword pair
+#pragma unroll
+        for (int i = 0; i < NQ; i++) q[i] = __builtin_amdgcn_perm(d[i + 1], d[i], sel);
+    }
+    __device__ __forceinline__ uint32_t head() const { return d[0] >> (8u * o); }   // the block's first bytes (4 - o of them)
+};
 
 template <int FMT> struct NeedsAlignedTensor { static constexpr bool value = false; };
 template <> struct NeedsAlignedTensor<RFQ_GGUF_Q6_K> { static constexpr bool value = true; };
@@ -326,16 +333,11 @@ template <int FMT> __device__ __forceinline__ void unit_tables_init()
     }
 }
 
-template <> struct Unit<RFQ_MXFP4> {
-    static constexpr bool NEEDS_XSUM = false;
+// Opened<FMT>: the fields of a unit that was fetched as windows (Unit<FMT>::open), with the unit's arithmetic.
+template <int FMT> struct Opened;
+
+template <> struct Opened<RFQ_MXFP4> {
     int e; U4 q;
-    // (a 17-byte unit starts at any byte address: through an aligned window, see load_window)
-    __device__ __forceinline__ void load(const uint8_t *row, int u)
-    {
-        uint32_t first;
-        const uint32_t o = load_window<4>(row + (size_t)u * 17, 1u, first, q.v);
-        e = __builtin_amdgcn_sbfe((int)first, 8u * o, 8u);
-    }
     template <bool CLAMP> __device__ __forceinline__ float dot_as(const float (&x)[32]) const
     {
         // bound on |code value|: 8 / 2^e when e >= 1 (exact, 2^(3-e)), else 8.
@@ -362,16 +364,22 @@ template <> struct Unit<RFQ_MXFP4> {
         return __builtin_amdgcn_ballot_w64(e >= 1) != 0 ? dot_as<true>(x) : dot_as<false>(x);
     }
 };
-
-template <> struct Unit<RFQ_MXFP6_E2M3> {
+template <> struct Unit<RFQ_MXFP4> {
     static constexpr bool NEEDS_XSUM = false;
-    int e; U6 q;
-    __device__ __forceinline__ void load(const uint8_t *row, int u)
+    Window<4> w;
+    __device__ __forceinline__ void load(const uint8_t *row, int u) { w.load(row + (size_t)u * 17); }
+    __device__ __forceinline__ Opened<RFQ_MXFP4> open() const
     {
-        uint32_t first;
-        const uint32_t o = load_window<6>(row + (size_t)u * 25, 1u, first, q.v);
-        e = __builtin_amdgcn_sbfe((int)first, 8u * o, 8u);
+        Opened<RFQ_MXFP4> r;
+        r.e = __builtin_amdgcn_sbfe((int)w.d[0], 8u * w.o, 8u);
+        w.piece<1>(r.q.v);
+        return r;
     }
+    __device__ __forceinline__ float dot(const float (&x)[32], float xsum) const { return open().dot(x, xsum); }
+};
+
+template <> struct Opened<RFQ_MXFP6_E2M3> {
+    int e; U6 q;
     template <bool CLAMP> __device__ __forceinline__ float dot_as(const float (&x)[32]) const
     {
         // 7.5 * 2^-e for e >= 1: 7.5 = 0x40F00000 (biased exponent 129).
@@ -410,25 +418,25 @@ template <> struct Unit<RFQ_MXFP6_E2M3> {
         return __builtin_amdgcn_ballot_w64(e >= 1) != 0 ? dot_as<true>(x) : dot_as<false>(x);
     }
 };
+template <> struct Unit<RFQ_MXFP6_E2M3> {
+    static constexpr bool NEEDS_XSUM = false;
+    Window<6> w;
+    __device__ __forceinline__ void load(const uint8_t *row, int u) { w.load(row + (size_t)u * 25); }
+    __device__ __forceinline__ Opened<RFQ_MXFP6_E2M3> open() const
+    {
+        Opened<RFQ_MXFP6_E2M3> r;
+        r.e = __builtin_amdgcn_sbfe((int)w.d[0], 8u * w.o, 8u);
+        w.piece<1>(r.q.v);
+        return r;
+    }
+    __device__ __forceinline__ float dot(const float (&x)[32], float xsum) const { return open().dot(x, xsum); }
+};
 
 // ---- GGUF file layouts (ggml block_q4_0 / q8_0 / q4_K / q6_K) -----------------
 // Blocks are 2-byte aligned only; loads are byte-exact copies.
 
-template <> struct Unit<RFQ_GGUF_Q4_0> {
-    static constexpr bool NEEDS_XSUM = true;
+template <> struct Opened<RFQ_GGUF_Q4_0> {
     uint16_t d; U4 q;
-    __device__ __forceinline__ void load(const uint8_t *row, int u)
-    {
-        uint32_t first;
-        const uint32_t o = load_window<4>(row + (size_t)u * 18, 2u, first, q.v);   // o = 0 or 2 (see NeedsAlignedTensor)
-        d = (uint16_t)(first >> (8u * o));
-    }
-    __device__ __forceinline__ void load_bytes(const uint8_t *row, int u)
-    {
-        const uint8_t *p = row + (size_t)u * 18;
-        d = ld<uint16_t>(p);
-        q = ld<U4>(p + 2);
-    }
     // element j = low nibble of byte j, element 16 + j = high nibble
     __device__ __forceinline__ float dot(const float (&x)[32], float xsum) const
     {
@@ -445,22 +453,24 @@ template <> struct Unit<RFQ_GGUF_Q4_0> {
         return f16_bits_to_f32(d) * __builtin_fmaf(-8.0f, xsum, s0 + s1);
     }
 };
-
-template <> struct Unit<RFQ_GGUF_Q8_0> {
+// (blocks at even addresses, see NeedsAlignedTensor: o = 0 or 2 and the f16 scale lies inside the first dword)
+template <> struct Unit<RFQ_GGUF_Q4_0> {
     static constexpr bool NEEDS_XSUM = true;
+    Window<4> w;
+    __device__ __forceinline__ void load(const uint8_t *row, int u) { w.load(row + (size_t)u * 18); }
+    __device__ __forceinline__ void load_bytes(const uint8_t *row, int u) { w.load_bytes<2>(row + (size_t)u * 18); }
+    __device__ __forceinline__ Opened<RFQ_GGUF_Q4_0> open() const
+    {
+        Opened<RFQ_GGUF_Q4_0> r;
+        r.d = (uint16_t)w.head();
+        w.piece<2>(r.q.v);
+        return r;
+    }
+    __device__ __forceinline__ float dot(const float (&x)[32], float xsum) const { return open().dot(x, xsum); }
+};
+
+template <> struct Opened<RFQ_GGUF_Q8_0> {
     uint16_t d; U8 q;
-    __device__ __forceinline__ void load(const uint8_t *row, int u)
-    {
-        uint32_t first;
-        const uint32_t o = load_window<8>(row + (size_t)u * 34, 2u, first, q.v);   // o = 0 or 2 (see NeedsAlignedTensor)
-        d = (uint16_t)(first >> (8u * o));
-    }
-    __device__ __forceinline__ void load_bytes(const uint8_t *row, int u)
-    {
-        const uint8_t *p = row + (size_t)u * 34;
-        d = ld<uint16_t>(p);
-        q = ld<U8>(p + 2);
-    }
     // int8 q = (q ^ 0x80) - 128 with the left term read as an unsigned byte
     __device__ __forceinline__ float dot(const float (&x)[32], float xsum) const
     {
@@ -475,6 +485,20 @@ template <> struct Unit<RFQ_GGUF_Q8_0> {
         }
         return f16_bits_to_f32(d) * __builtin_fmaf(-128.0f, xsum, s0 + s1);
     }
+};
+template <> struct Unit<RFQ_GGUF_Q8_0> {
+    static constexpr bool NEEDS_XSUM = true;
+    Window<8> w;
+    __device__ __forceinline__ void load(const uint8_t *row, int u) { w.load(row + (size_t)u * 34); }
+    __device__ __forceinline__ void load_bytes(const uint8_t *row, int u) { w.load_bytes<2>(row + (size_t)u * 34); }
+    __device__ __forceinline__ Opened<RFQ_GGUF_Q8_0> open() const
+    {
+        Opened<RFQ_GGUF_Q8_0> r;
+        r.d = (uint16_t)w.head();
+        w.piece<2>(r.q.v);
+        return r;
+    }
+    __device__ __forceinline__ float dot(const float (&x)[32], float xsum) const { return open().dot(x, xsum); }
 };
 
 // Unit u of a 144-byte super-block: chunk c = u >> 1 of 64 elements, half h = u & 1
@@ -512,29 +536,8 @@ template <> struct Unit<RFQ_GGUF_Q4_K> {
 // Unit u of a 210-byte super-block: half n = (u >> 2) & 1 of 128 elements, quarter t = u & 3:
 // low nibbles from ql[64 n + 32 (t & 1) + l] (>> 4 for t >= 2), bits 4-5 from qh[32 n + l] >> 2 t,
 // scales sc[8 n + 2 t + l / 16]; value = d * sc * (q - 32).
-template <> struct Unit<RFQ_GGUF_Q6_K> {
-    static constexpr bool NEEDS_XSUM = true;
+template <> struct Opened<RFQ_GGUF_Q6_K> {
     U8 ql, qh; uint16_t sc2, d; int t;
-    __device__ __forceinline__ void load(const uint8_t *row, int u)
-    {
-        const uint8_t *blk = row + (size_t)(u >> 3) * 210;
-        const int half = (u >> 2) & 1;
-        t = u & 3;
-        ql = load32_a2(blk + 64 * half + 32 * (t & 1));
-        qh = load32_a2(blk + 128 + 32 * half);
-        sc2 = ld<uint16_t>(blk + 192 + 8 * half + 2 * t);
-        d = ld<uint16_t>(blk + 208);
-    }
-    __device__ __forceinline__ void load_bytes(const uint8_t *row, int u)
-    {
-        const uint8_t *blk = row + (size_t)(u >> 3) * 210;
-        const int half = (u >> 2) & 1;
-        t = u & 3;
-        ql = ld<U8>(blk + 64 * half + 32 * (t & 1));
-        qh = ld<U8>(blk + 128 + 32 * half);
-        sc2 = ld<uint16_t>(blk + 192 + 8 * half + 2 * t);
-        d = ld<uint16_t>(blk + 208);
-    }
     __device__ __forceinline__ float dot(const float (&x)[32], float xsum) const
     {
         const int shl = 4 * (t >> 1), shh = 2 * t;
@@ -555,6 +558,36 @@ template <> struct Unit<RFQ_GGUF_Q6_K> {
         const float c0 = (float)(int8_t)(sc2 & 255u), c1 = (float)(int8_t)(sc2 >> 8);
         return f16_bits_to_f32(d) * __builtin_fmaf(c0, g0, c1 * g1);
     }
+};
+template <> struct Unit<RFQ_GGUF_Q6_K> {
+    static constexpr bool NEEDS_XSUM = true;
+    Window<8> wl, wh; uint16_t sc2, d; int t;
+    template <bool BYTES> __device__ __forceinline__ void load_as(const uint8_t *row, int u)
+    {
+        const uint8_t *blk = row + (size_t)(u >> 3) * 210;
+        const int half = (u >> 2) & 1;
+        t = u & 3;
+        if constexpr (BYTES) {
+            wl.load_bytes<0>(blk + 64 * half + 32 * (t & 1));
+            wh.load_bytes<0>(blk + 128 + 32 * half);
+        } else {
+            wl.load(blk + 64 * half + 32 * (t & 1));
+            wh.load(blk + 128 + 32 * half);
+        }
+        sc2 = ld<uint16_t>(blk + 192 + 8 * half + 2 * t);
+        d = ld<uint16_t>(blk + 208);
+    }
+    __device__ __forceinline__ void load(const uint8_t *row, int u) { load_as<false>(row, u); }
+    __device__ __forceinline__ void load_bytes(const uint8_t *row, int u) { load_as<true>(row, u); }
+    __device__ __forceinline__ Opened<RFQ_GGUF_Q6_K> open() const
+    {
+        Opened<RFQ_GGUF_Q6_K> r;
+        wl.piece<0>(r.ql.v);
+        wh.piece<0>(r.qh.v);
+        r.sc2 = sc2; r.d = d; r.t = t;
+        return r;
+    }
+    __device__ __forceinline__ float dot(const float (&x)[32], float xsum) const { return open().dot(x, xsum); }
 };
 
 // ---- the matmul module's own decoders (src/kernels/matmul/quantized/) -------------
@@ -1178,6 +1211,9 @@ template <> struct IUnit<RFQ_GGUF_Q4_0> : Unit<RFQ_GGUF_Q4_0> {
     // low nibbles of dword w are elements 4w .. 4w+3 (group w), high nibbles elements 16+4w .. (group 4+w)
     __device__ __forceinline__ float idot(const XPrep &xp) const
     {
+        const Opened<RFQ_GGUF_Q4_0> b = open();
+        const U4 &q = b.q;
+        const uint16_t d = b.d;
         uint32_t alo = 0, amid = 0;
         int atop = 0;
 #pragma unroll
@@ -1202,6 +1238,9 @@ template <> struct IUnit<RFQ_GGUF_Q8_0> : Unit<RFQ_GGUF_Q8_0> {
     static constexpr uint32_t TOPOFF = 0x400000u; // offset-binary weight bytes reach 255: keep every limb unsigned
     __device__ __forceinline__ float idot(const XPrep &xp) const
     {
+        const Opened<RFQ_GGUF_Q8_0> b = open();
+        const U8 &q = b.q;
+        const uint16_t d = b.d;
         uint32_t alo = 0, amid = 0, atop = 0, bsum = 0;
 #pragma unroll
         for (int g = 0; g < 8; g++) {
@@ -1284,6 +1323,9 @@ template <> struct IUnit<RFQ_GGUF_Q6_K> : Unit<RFQ_GGUF_Q6_K> {
     {
         // bits 4-5 of a code: the bit pair at 2t of its qh byte, brought to bits 4-5 by one rotation (what it drags in
         // from the neighbouring bytes is masked away)
+        U8 ql, qh;
+        wl.piece<0>(ql.v);
+        wh.piece<0>(qh.v);
         const int shl = 4 * (t >> 1), rot = (2 * t + 28) & 31;
         uint32_t alo[2] = {0, 0}, amid[2] = {0, 0};
         int atop[2] = {0, 0};
@@ -1409,6 +1451,9 @@ template <> struct IUnit<RFQ_MXFP4> : Unit<RFQ_MXFP4> {
     // multiple of 64 KiB: entry b's slot is then `slot` with b as its second byte.
     __device__ __forceinline__ float idot_lut(const XPrep &xp, uint32_t slot) const
     {
+        const Opened<RFQ_MXFP4> b = open();
+        const U4 &q = b.q;
+        const int e = b.e;
         uint32_t alo = 0, amid = 0;
         int atop = 0;
         int ee = e;
@@ -1472,7 +1517,62 @@ __device__ __forceinline__ float idot_pair_of(const IU &u, const XPrep &xe, cons
 // each thread converts a quarter unit.
 constexpr int IDOT_WAVES = 8;
 
-template <int FMT, int UPL, int WPR, int R, bool FUSE>
+// ---- a timeline from inside the kernel (rfq_bench_gemv_timeline) ------------------------------------------------
+// gemv_idot_kernel<..., TRACE = true> has every wavefront read the constant 100 MHz clock (s_memrealtime) at the
+// points below and write the readings, lane 0, to g_gemv_trace[wavefront][TRACE_STAMPS] when it ends.  A reading is
+// ordered behind the data it marks the arrival of by an empty asm that consumes the register.  Only a few
+// configurations are compiled with the flag (TraceCompiled); a launch takes the flagged kernel when the calling
+// thread has asked for it (trace_request).
+//   0 entry   1 x in registers (behind the requests for x and the first rows, which block while the CU's memory
+//   pipeline is full)   2 x converted (before the barrier)   3 after the barrier   4 prepared x in registers
+//   5 + 2 i  row i of the first group in registers   6 + 2 i  row i reduced   (i < 7)
+//   19 group stored (end)
+constexpr int TRACE_STAMPS = 20;
+__device__ unsigned long long *g_gemv_trace;
+struct TraceRequest { unsigned long long *d_buf; size_t capacity_waves; int waves_written; };
+thread_local TraceRequest trace_request = {nullptr, 0, 0};
+
+// (a register that the unit's loads fill, for the formats whose kernels are compiled with the trace)
+__device__ __forceinline__ uint32_t first_word_of(const Unit<RFQ_Q4_K> &u) { return u.q.v[3]; }
+__device__ __forceinline__ uint32_t first_word_of(const Unit<RFQ_GGUF_Q4_K> &u) { return u.q.v[7]; }
+__device__ __forceinline__ uint32_t first_word_of(const Unit<RFQ_MXFP4> &u) { return u.w.d[4]; }
+template <int FMT> __device__ __forceinline__ uint32_t first_word_of(const Unit<FMT> &) { return 0; }
+
+template <bool ON> struct WaveTrace {
+    __device__ __forceinline__ void stamp(int) {}
+    __device__ __forceinline__ void stamp_after(int, uint32_t) {}
+    __device__ __forceinline__ void flush(int, int, int) {}
+};
+template <> struct WaveTrace<true> {
+    unsigned long long t[TRACE_STAMPS];
+    __device__ __forceinline__ void stamp(int i)
+    {
+        unsigned long long now;
+        asm volatile("s_memrealtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(now) :: "memory");
+        t[i] = now;
+    }
+    __device__ __forceinline__ void stamp_after(int i, uint32_t arrived)
+    {
+        asm volatile("" :: "v"(arrived) : "memory");
+        stamp(i);
+    }
+    __device__ __forceinline__ void flush(int block_wave, int lane, int waves_total)
+    {
+        (void)waves_total;
+        if (lane == 0) {
+            unsigned long long *o = g_gemv_trace + (size_t)block_wave * TRACE_STAMPS;
+#pragma unroll
+            for (int i = 0; i < TRACE_STAMPS; i++) o[i] = t[i];
+        }
+    }
+};
+template <int FMT, int UPL, int WPR, int R, bool FUSE> struct TraceCompiled {
+    static constexpr bool value = !FUSE && R == 7 && ((FMT == RFQ_Q4_K && UPL == 1 && WPR == 2) ||
+                                                      (FMT == RFQ_MXFP4 && UPL == 1 && WPR == 2) ||
+                                                      (FMT == RFQ_GGUF_Q4_K && UPL == 2 && WPR == 1));
+};
+
+template <int FMT, int UPL, int WPR, int R, bool FUSE, bool TRACE = false>
 __global__ void __launch_bounds__(64 * IDOT_WAVES)
 gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, float *__restrict__ y, int n, int k,
                  int groups, GemvFuse f)
@@ -1486,6 +1586,8 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
     extern __shared__ __attribute__((aligned(16))) uint32_t idot_lds[]; // (MXFP4: the code table,) [units][28]
     constexpr size_t LUT_DWORDS = FMT == RFQ_MXFP4 ? MX4_LUT_BYTES / 4 : 0;
     uint32_t *const xlds = idot_lds + LUT_DWORDS;
+    WaveTrace<TRACE> trace;
+    trace.stamp(0);
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int team = wave / WPR, wit = wave % WPR;
     const int tl = wit * 64 + lane;
@@ -1520,12 +1622,13 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
     // behind the first rows' weights would hold the barrier below, and with it every wavefront's first dot, until
     // those rows had arrived (Q4_K 4096 x 14336: 12.2 -> 11.5 us, 8192 x 8192: 14.0 -> 12.8 us).
     constexpr int NX = (4 * 64 * WPR * UPL + THREADS - 1) / THREADS;
+    const int xthread = threadIdx.x;
     float xv[NX][8], nv[FUSE ? NX : 1][8];
     bool prep[NX];
     const bool norm = FUSE && f.norm_w != nullptr;
 #pragma unroll
     for (int i = 0; i < NX; i++) {
-        const int h = threadIdx.x + i * THREADS;
+        const int h = xthread + i * THREADS;
         prep[i] = h < 4 * ku;
         if (prep[i]) prep_load8(x + (size_t)h * 8, xv[i]);
         if constexpr (FUSE) {
@@ -1550,11 +1653,13 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
 
     if constexpr (FMT == RFQ_MXFP4) mx4_fill_lut<THREADS>(idot_lds, threadIdx.x);
 
+    if constexpr (TRACE) trace.stamp_after(1, __float_as_uint(xv[0][0]));
+
     // Cooperative conversion of x: 4*ku quarter-units (eight values each) over the block's threads.
     float ssq = 0.f;
 #pragma unroll
     for (int c = 0; c < NX; c++) {
-        const int h = threadIdx.x + c * THREADS;
+        const int h = xthread + c * THREADS;
         if constexpr (FUSE) {
             if (norm && prep[c]) {
 #pragma unroll
@@ -1582,7 +1687,9 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
             if (lane == 0) ssq_part[wave] = ssq;
         }
     }
+    trace.stamp(2);
     __syncthreads();
+    trace.stamp(3);
     float rinv = 1.0f;
     if constexpr (FUSE) {
         if (norm) {
@@ -1607,6 +1714,8 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
         xp[j].xh1 = __uint_as_float(src[27]);
     }
 
+    if constexpr (TRACE) trace.stamp_after(4, xp[0].l[0] ^ xp[UPL - 1].l[23]);
+
     // With R = D a row's slot is the same in every group, and the ring of rows in flight runs on across the groups:
     // the slot a row leaves takes the same row of the next group (past the last group: the team's last row again,
     // a cache hit whose result is never used).  Otherwise a group starts by requesting its first D rows with nothing
@@ -1627,6 +1736,9 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
 #pragma unroll
         for (int i = 0; i < R; i++) {
             float acc = 0.f;
+            if constexpr (TRACE) {
+                if (g == 0) trace.stamp_after(5 + 2 * i, first_word_of(buf[i % D][0]));
+            }
             if constexpr (IU::PAIR && UPL == 2) {
                 const float t = idot_pair_of(buf[i % D][0], xp[0], xp[1]);
                 acc = live[0] ? t : 0.f;
@@ -1642,10 +1754,17 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
             if (i + D < R) load_row(i % D, base + i + D);
             else if (RING) load_row(i % D, base + i + D);
             res[i] = wave_sum(acc);
+            if constexpr (TRACE) {
+                if (g == 0) trace.stamp_after(6 + 2 * i, __float_as_uint(res[i]));
+            }
         }
         // (`groups` is uniform over the block: every wavefront stores the same number of groups)
         store_group<R, WPR, FUSE, WAVES, true>(res, part[g & 1], y, row0 + base, row_end, lane, wave, f, rinv);
+        if constexpr (TRACE) {
+            if (g == 0) trace.stamp(19);
+        }
     }
+    trace.flush(blockIdx.x * WAVES + wave, lane, gridDim.x * WAVES);
 }
 
 // ---- 2 <= m <= 8: the same integer-dot scheme with M activation vectors ----------
@@ -2038,6 +2157,23 @@ int launch_idot(const uint8_t *w, const float *x, float *y, int n, int k, int bl
         if (!table_at_zero) return run_xreg<FMT, UPL, WPR, FUSE>(w, x, y, n, k, f, s);   // (not expected: the float kernel)
     }
     note_kernel(FUSE ? "gemv_idot_kernel<%s,%d,%d,%d,fused>" : "gemv_idot_kernel<%s,%d,%d,%d>", FMT, UPL, WPR, R);
+    if constexpr (TraceCompiled<FMT, UPL, WPR, R, FUSE>::value) {
+        if (trace_request.d_buf != nullptr && (size_t)blocks * IDOT_WAVES <= trace_request.capacity_waves) {
+            if constexpr (FMT == RFQ_MXFP4) {
+                const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_idot_kernel<FMT, UPL, WPR, R, FUSE, true>),
+                                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 4096);
+                if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(gemv_idot_kernel, traced)");
+            }
+            const hipError_t e = hipMemcpyToSymbol(HIP_SYMBOL(g_gemv_trace), &trace_request.d_buf, sizeof(trace_request.d_buf), 0,
+                                                   hipMemcpyHostToDevice);    // (blocking: a tool of the benchmark driver)
+            if (e != hipSuccess) return hip_fail(e, "hipMemcpyToSymbol(g_gemv_trace)");
+            hipLaunchKernelGGL((gemv_idot_kernel<FMT, UPL, WPR, R, FUSE, true>), dim3(blocks), dim3(64 * IDOT_WAVES), lds, s, w, x, y, n,
+                               k, groups, f);
+            RFQ_LAUNCH_CHECK("gemv_idot_kernel (traced)");
+            trace_request.waves_written = blocks * IDOT_WAVES;
+            return RFQ_OK;
+        }
+    }
     hipLaunchKernelGGL((gemv_idot_kernel<FMT, UPL, WPR, R, FUSE>), dim3(blocks), dim3(64 * IDOT_WAVES), lds, s, w, x, y, n, k, groups,
                        f);
     RFQ_LAUNCH_CHECK("gemv_idot_kernel");
@@ -2206,13 +2342,13 @@ int run_rows(const uint8_t *w, const float *x, float *y, int n, int k, const Gem
     // The 256-byte Q6_K layout has both kernels, a few per cent apart either way (measured on 14336, 11008, 4096 and
     // 32000 rows of 4096, 4096 rows of 8192 and of 14336): the integer-dot one where a team walks a single group of rows
     // of 65..128 units or rows longer than 256 units, the float one elsewhere and in the fused forms.
-    // MXFP4 has both kernels too: the integer-dot one for few rows (up to 16 per CU: 4096 x 4096 6.1 -> 5.5 us), for
-    // rows longer than 128 units (4096 x 8192 8.7 -> 8.0 us, 4096 x 14336 12.4 -> 12.0 us) and around 56 rows per CU
-    // (14336 x 4096 10.4 -> 10.2 us); elsewhere the float one (code values from a table of floats in LDS) is ahead
-    // (11008 x 4096 9.8 against 10.2 us, 32000 x 4096 17.2 against 18.8 us), and the fused forms keep it.
+    // MXFP4 has both kernels too: the integer-dot one for rows longer than 256 units (4096 x 14336 11.6 -> 11.1 us)
+    // and, with up to 128 units, for few rows (up to 16 per CU: 4096 x 4096 5.0 -> 4.6 us) and around 56 rows per CU
+    // (14336 x 4096 9.8 -> 9.4 us); elsewhere the float one (code values from a table of floats in LDS) is level or
+    // ahead (8192 x 8192 10.5 against 11.1 us, 32000 x 4096 16.8 against 18.8 us), and the fused forms keep it.
     if constexpr (FMT == RFQ_MXFP4) {
         const int cus = device_cu_count();
-        if (FUSE || !(ku > 128 || n <= cus * 16 || (n >= cus * 52 && n <= cus * 64))) {
+        if (FUSE || !(ku > 256 || (ku <= 128 && (n <= cus * 16 || (n >= cus * 52 && n <= cus * 64))))) {
             if (ku <= 64) return run_idot<FMT, 1, 1, FUSE>(w, x, y, n, k, f, s, false);
             if (!FUSE && ku <= 128 && n >= device_cu_count() * 32) return run_idot<FMT, 1, 2, FUSE>(w, x, y, n, k, f, s, false);
             if (ku <= 128) return run_idot<FMT, 2, 1, FUSE>(w, x, y, n, k, f, s, false);
@@ -2378,6 +2514,18 @@ int launch_gemv_fused(int fmt, const uint8_t *d_w, const uint8_t *d_w2, const fl
     case RFQ_GGUF_Q6_K: return run_rows<RFQ_GGUF_Q6_K, true>(d_w, d_x, d_y, rows, k, f, s);
     default: return fail(RFQ_E_BADARG, "fused gemv: unknown format %d", fmt);
     }
+}
+
+// One m = 1 launch with the in-kernel timeline (see WaveTrace): the same dispatch as launch_gemv; *waves = 0 when the
+// kernel it takes for this format and shape is not compiled with the trace.
+int launch_gemv_traced(int fmt, const uint8_t *d_w, const float *d_x, float *d_y, int n, int k, unsigned long long *d_trace,
+                       size_t capacity_waves, int *waves, hipStream_t s)
+{
+    trace_request = TraceRequest{d_trace, capacity_waves, 0};
+    const int rc = launch_gemv(fmt, d_w, d_x, d_y, 1, n, k, s);
+    *waves = trace_request.waves_written;
+    trace_request = TraceRequest{nullptr, 0, 0};
+    return rc;
 }
 
 } // namespace rfq
