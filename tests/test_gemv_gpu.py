@@ -235,3 +235,45 @@ def test_gemv_windowed_layouts_at_any_address(fmt, oracle, cuda):
                                   C.c_void_p(y.data_ptr()), m, n, k, None))
             torch.cuda.synchronize()
             assert_close(y.cpu().numpy(), want, f"{Q.NAMES[fmt]} m={m} n={n} k={k} offset {off}")
+
+
+@pytest.mark.parametrize("fmt", [Q.Q4_K, Q.MXFP4, Q.GGUF_Q4_K])
+def test_timeline_build_computes_the_same_and_stamps_in_order(fmt, oracle, cuda):
+    """rfq_bench_gemv_timeline launches the build of the decode kernel that stamps a clock at 20 points per wavefront:
+    its output must be the ordinary kernel's, every wavefront's stamps must not go backwards, and a shape whose
+    kernel has no such build reports zero wavefronts."""
+    import torch
+    from rocmforge_amd import _lib
+    L = _lib.lib()
+    n, k = 14336, 4096
+    w = Q.make_weights(fmt, n, k, seed=8800 + fmt)
+    x = x_for(1, k, 8801)
+    want = gpu_gemv(fmt, w, x, n, k, cuda)
+    dw = torch.from_numpy(w).to(cuda)
+    dx = torch.from_numpy(x).to(cuda)
+    y = torch.zeros((1, n), dtype=torch.float32, device=cuda)
+    cap = 8192
+    trace = torch.zeros((cap, 20), dtype=torch.int64, device=cuda)
+    ptrs = (C.c_void_p * 1)(dw.data_ptr())
+    waves, stamps = C.c_int(-1), C.c_int(-1)
+    _lib.check(L.rfq_bench_gemv_timeline(fmt, ptrs, 1, w.size, C.c_void_p(dx.data_ptr()), C.c_void_p(y.data_ptr()), n, k, 2, None,
+                                         C.c_void_p(trace.data_ptr()), cap, C.byref(waves), C.byref(stamps)))
+    torch.cuda.synchronize()
+    assert stamps.value == 20 and waves.value in (2048, 4096), (stamps.value, waves.value)
+    np.testing.assert_array_equal(y.cpu().numpy().reshape(-1), np.asarray(want).reshape(-1))
+    t = trace[:waves.value].cpu().numpy()
+    assert (t[:, 0] > 0).all() and (np.diff(t, axis=1) >= 0).all()
+    assert (t[:, 19] - t[:, 0]).max() < 100 * 1000                  # (100 MHz ticks: under a millisecond)
+    # a shape whose kernel has no such build: ordinary launch, nothing written
+    n2, k2 = 256, 1024
+    w2 = Q.make_weights(fmt, n2, k2, seed=8802)
+    dw2 = torch.from_numpy(w2).to(cuda)
+    x2 = x_for(1, k2, 8803)
+    dx2 = torch.from_numpy(x2).to(cuda)
+    y2 = torch.zeros((1, n2), dtype=torch.float32, device=cuda)
+    ptrs2 = (C.c_void_p * 1)(dw2.data_ptr())
+    _lib.check(L.rfq_bench_gemv_timeline(fmt, ptrs2, 1, w2.size, C.c_void_p(dx2.data_ptr()), C.c_void_p(y2.data_ptr()), n2, k2, 1, None,
+                                         C.c_void_p(trace.data_ptr()), cap, C.byref(waves), C.byref(stamps)))
+    torch.cuda.synchronize()
+    assert waves.value == 0
+    assert_close(y2.cpu().numpy(), oracle.qmatmul_nk(fmt, w2, x2, 1, n2, k2), f"{Q.NAMES[fmt]} untraced shape")
