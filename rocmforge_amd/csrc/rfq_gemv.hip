@@ -2208,7 +2208,10 @@ int run_idot(const uint8_t *w, const float *x, float *y, int n, int k, const Gem
             if (r == 5 && !(FIVE && groups > 1)) continue;
             int blocks = (n + TEAMS * r * groups - 1) / (TEAMS * r * groups);
             long waves_of_blocks = (blocks + slots - 1) / slots;
-            long cost = waves_of_blocks * r * groups * (r == 5 && groups > 1 ? 19 : 20);
+            // (a group that starts with nothing in flight costs a team of several wavefronts per row about as much as
+            // a row and a half: 5120 x 5120 in three groups of 2 rows 8.15 us, in one of 7 7.48 us; 13824 x 5120 in four
+            // of 4 17.2 us, in two of 8 15.2 us)
+            long cost = waves_of_blocks * (r * groups * (r == 5 && groups > 1 ? 19 : 20) + (UPL == 2 && WPR >= 2 ? 30 * (groups - 1) : 0));
             if (best_cost < 0 || cost < best_cost || (cost == best_cost && r > best_r)) {
                 best_cost = cost; best_r = r; best_groups = groups; best_blocks = blocks;
             }
@@ -2350,7 +2353,7 @@ int run_rows(const uint8_t *w, const float *x, float *y, int n, int k, const Gem
         const int cus = device_cu_count();
         if (FUSE || !(ku > 256 || (ku <= 128 && (n <= cus * 16 || (n >= cus * 52 && n <= cus * 64))))) {
             if (ku <= 64) return run_idot<FMT, 1, 1, FUSE>(w, x, y, n, k, f, s, false);
-            if (!FUSE && ku <= 128 && n >= device_cu_count() * 32) return run_idot<FMT, 1, 2, FUSE>(w, x, y, n, k, f, s, false);
+            if (!FUSE && ku <= 128 && (n > cus * 16 || n <= cus * 8)) return run_idot<FMT, 1, 2, FUSE>(w, x, y, n, k, f, s, false);
             if (ku <= 128) return run_idot<FMT, 2, 1, FUSE>(w, x, y, n, k, f, s, false);
             if (ku <= 256) return run_idot<FMT, 2, 2, FUSE>(w, x, y, n, k, f, s, false);
             return run_idot<FMT, 2, 4, FUSE>(w, x, y, n, k, f, s, false);
@@ -2360,26 +2363,42 @@ int run_rows(const uint8_t *w, const float *x, float *y, int n, int k, const Gem
         const int cus = device_cu_count();
         if (FUSE || !((ku > 64 && ku <= 128 && n >= cus * 56 && n <= cus * 64) || ku > 256)) {
             if (ku <= 64) return run_idot<FMT, 1, 1, FUSE>(w, x, y, n, k, f, s, false);
-            if (!FUSE && ku <= 128 && n >= cus * 32) return run_idot<FMT, 1, 2, FUSE>(w, x, y, n, k, f, s, false);
+            if (!FUSE && ku <= 128 && (n > cus * 16 || n <= cus * 8)) return run_idot<FMT, 1, 2, FUSE>(w, x, y, n, k, f, s, false);
             if (ku <= 128) return run_idot<FMT, 2, 1, FUSE>(w, x, y, n, k, f, s, false);
             if (ku <= 256) return run_idot<FMT, 2, 2, FUSE>(w, x, y, n, k, f, s, false);
             return run_idot<FMT, 2, 4, FUSE>(w, x, y, n, k, f, s, false);
         }
     }
     if (ku <= 64) return run_idot<FMT, 1, 1, FUSE>(w, x, y, n, k, f, s);
-    // Rows of 65..128 units with at least seven rows per team in that form: one unit per lane, two
-    // wavefronts per row, sixteen wavefronts per CU (14336 x 4096: 11.67 -> 11.30 us; 4096 rows would lose 6 %)
-    // The float formats likewise (their kernels are bound by instructions and gain most from sixteen wavefronts
-    // per CU: Q6_K 14336 x 4096 16.5 -> 13.8 us).
-    // (from 32 rows per CU on: Q6_K 11008 x 4096 14.6 -> 11.8 us, 8192 x 4096 the same either way)
-    if constexpr (!HasIdot<FMT>::value && !FUSE) {
-        if (ku > 64 && ku <= 128 && n >= device_cu_count() * 32) return run_xreg<FMT, 1, 2, FUSE>(w, x, y, n, k, f, s);
-    }
+    // Rows of 65..128 units: one unit per lane and two wavefronts per row (sixteen wavefronts per CU) against two units
+    // per lane and one wavefront per row (eight).  Measured per format on 1024, 4096, 6144, 11008, 14336, 32000 and
+    // 128256 rows of 4096 with every group size either form offers:
+    //  * up to eight rows per CU the first form puts twice as many CUs to work (1024 rows: Q4_K 3.87 -> 3.10 us, Q8_0
+    //    3.42 -> 2.92, Q6_K 3.29 -> 2.83, MXFP4 4.24 -> 3.31, MXFP6 4.27 -> 3.57, GGUF_Q8_0 3.74 -> 2.94, GGUF_Q6_K 4.73 -> 3.39);
+    //  * the float formats, bound by their instructions, take it from 16 rows per CU on (6144 rows: Q6_K 7.70 -> 6.53 us,
+    //    MXFP4 6.84 -> 5.99, MXFP6 8.86 -> 7.26; 14336 rows: Q6_K 16.5 -> 13.8);
+    //  * the integer-dot formats from 56 rows per CU on (Q4_K 14336 x 4096: 11.67 -> 11.30 us; at 11008 rows the second
+    //    form is ahead, Q4_K 10.4 against 9.0 us), GGUF_Q4_0 and GGUF_Q8_0 between 16 and 32 rows per CU as well (6144
+    //    rows: GGUF_Q4_0 5.69 -> 5.26 us, GGUF_Q8_0 7.24 -> 7.05);
+    //  * GGUF_Q6_K up to 16 rows per CU only (4096 rows 6.16 -> 5.55 us; 14336 rows 13.4 against 14.9), and GGUF_Q4_K
+    //    never: its two units per lane share their bytes.
     // (the plain GEMV only: the fused gate/up form measured slower this way, 22.5 -> 25 us)
-    // (all integer-dot formats but the two GGUF K-layouts: GGUF_Q4_K needs two units per lane for its shared
-    // bytes, GGUF_Q6_K measured slower this way, 17.1 -> 17.7 us; Q8_0 13.7 -> 12.9 us, the 4-bit ones 1 %)
-    if constexpr (HasIdot<FMT>::value && FMT != RFQ_GGUF_Q4_K && FMT != RFQ_GGUF_Q6_K && !FUSE) {
-        if (ku > 64 && ku <= 128 && n >= device_cu_count() * 56) return run_idot<FMT, 1, 2, FUSE>(w, x, y, n, k, f, s);
+    if constexpr (!FUSE && FMT != RFQ_GGUF_Q4_K) {
+        if (ku > 64 && ku <= 128) {
+            const int cus = device_cu_count();
+            bool two_wavefronts_per_row = n <= cus * 8;
+            if constexpr (!HasIdot<FMT>::value) two_wavefronts_per_row |= n > cus * 16;
+            else if constexpr (FMT == RFQ_GGUF_Q6_K) two_wavefronts_per_row |= n <= cus * 16;
+            else {
+                two_wavefronts_per_row |= n >= cus * 56;
+                if constexpr (FMT == RFQ_GGUF_Q4_0 || FMT == RFQ_GGUF_Q8_0)
+                    two_wavefronts_per_row |= n > cus * 16 && n < cus * 32;
+            }
+            if (two_wavefronts_per_row) {
+                if constexpr (HasIdot<FMT>::value) return run_idot<FMT, 1, 2, FUSE>(w, x, y, n, k, f, s);
+                else return run_xreg<FMT, 1, 2, FUSE>(w, x, y, n, k, f, s);
+            }
+        }
     }
     if (ku <= 128) return run_idot<FMT, 2, 1, FUSE>(w, x, y, n, k, f, s);
     if (ku <= 256) return run_idot<FMT, 2, 2, FUSE>(w, x, y, n, k, f, s);
