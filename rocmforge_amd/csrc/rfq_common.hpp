@@ -96,6 +96,21 @@ int launch_rms_norm(int src_fmt, const void *d_x, const float *d_weight, float *
                     hipStream_t s);
 int launch_swiglu(const float *d_gate, const float *d_up, float *d_out, size_t total, hipStream_t s);
 int launch_gemv(int fmt, const uint8_t *d_w, const float *d_x, float *d_y, int m, int n, int k, hipStream_t s);
+// rfq_gemv.hip is compiled in four parts (the kernels of some formats each; part 0 also holds launch_gemv and
+// launch_gemv_fused, which hand a call to its format's part).  `fuse` points at the part-internal GemvFuse.
+struct GemvLastKernel { const char *name; int fmt, a, b, c; };
+extern thread_local GemvLastKernel g_gemv_last_kernel;   // which kernel this thread's last GEMV launch took
+struct GemvTraceRequest { unsigned long long *d_buf; size_t capacity_waves; int waves_written; };
+extern thread_local GemvTraceRequest g_gemv_trace_request;   // set around a launch that is to stamp its timeline
+#define RFQ_GEMV_PART_DECL(N)                                                                                                 \
+    int launch_gemv_part##N(int canonical, const uint8_t *d_w, const float *d_x, float *d_y, int m, int n, int k, hipStream_t s); \
+    int launch_gemv_fused_part##N(int canonical, const uint8_t *d_w, const float *d_x, float *d_y, int rows, int k,          \
+                                  const void *fuse, hipStream_t s);
+RFQ_GEMV_PART_DECL(0)
+RFQ_GEMV_PART_DECL(1)
+RFQ_GEMV_PART_DECL(2)
+RFQ_GEMV_PART_DECL(3)
+#undef RFQ_GEMV_PART_DECL
 constexpr int GEMV_TRACE_STAMPS = 20;                    // readings per wavefront, see WaveTrace in rfq_gemv.hip
 int launch_gemv_traced(int fmt, const uint8_t *d_w, const float *d_x, float *d_y, int n, int k, unsigned long long *d_trace,
                        size_t capacity_waves, int *waves, hipStream_t s);

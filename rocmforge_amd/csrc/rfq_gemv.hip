@@ -24,14 +24,41 @@
 
 #include "rfq_common.hpp"
 
+// This file is compiled RFQ_GEMV_PARTS times, -DRFQ_GEMV_PART=0 .. RFQ_GEMV_PARTS-1: every part holds the kernels of
+// some of the formats (gemv_part_of) behind launch_gemv_part<N> / launch_gemv_fused_part<N>, and part 0 holds the entry
+// points that hand a call to its format's part, so the formats compile side by side.  -DRFQ_GEMV_ONLY=<format> builds
+// part 0 with that format alone (a quick build while working on one format's kernel).
+#ifndef RFQ_GEMV_PART
+#error "compile with -DRFQ_GEMV_PART=0 .. 3 (see the Makefile)"
+#endif
+
 namespace rfq {
+
+constexpr int gemv_part_of(int canonical)
+{
+#ifdef RFQ_GEMV_ONLY
+    return canonical == RFQ_GEMV_ONLY ? 0 : -1;
+#else
+    switch (canonical) {
+    case RFQ_Q4_K: case RFQ_Q4_0: case RFQ_MM_Q4_K: return 0;
+    case RFQ_Q8_0: case RFQ_GGUF_Q8_0: case RFQ_MM_Q8_0: return 1;
+    case RFQ_Q6_K: case RFQ_MM_Q6_K: case RFQ_MXFP4: case RFQ_MXFP6_E2M3: return 2;
+    case RFQ_GGUF_Q4_0: case RFQ_GGUF_Q4_K: case RFQ_GGUF_Q6_K: return 3;
+    default: return -1;
+    }
+#endif
+}
+
+#if RFQ_GEMV_PART == 0
+thread_local GemvLastKernel g_gemv_last_kernel = {"", 0, 0, 0, 0};
+thread_local GemvTraceRequest g_gemv_trace_request = {nullptr, 0, 0};
+#endif
+
 namespace {
 
 // Which kernel the last GEMV launch of this thread took (name and template arguments), for the benchmark
 // driver's report: plain stores on the launch path, formatted only when asked for.
-struct LastKernel { const char *name; int fmt, a, b, c; };
-thread_local LastKernel g_last_kernel = {"", 0, 0, 0, 0};
-inline void note_kernel(const char *name, int fmt, int a, int b, int c) { g_last_kernel = LastKernel{name, fmt, a, b, c}; }
+inline void note_kernel(const char *name, int fmt, int a, int b, int c) { g_gemv_last_kernel = GemvLastKernel{name, fmt, a, b, c}; }
 
 // ---- wavefront reduction -----------------------------------------------------
 
@@ -1522,15 +1549,13 @@ constexpr int IDOT_WAVES = 8;
 // points below and write the readings, lane 0, to g_gemv_trace[wavefront][TRACE_STAMPS] when it ends.  A reading is
 // ordered behind the data it marks the arrival of by an empty asm that consumes the register.  Only a few
 // configurations are compiled with the flag (TraceCompiled); a launch takes the flagged kernel when the calling
-// thread has asked for it (trace_request).
+// thread has asked for it (g_gemv_trace_request).
 //   0 entry   1 x in registers (behind the requests for x and the first rows, which block while the CU's memory
 //   pipeline is full)   2 x converted (before the barrier)   3 after the barrier   4 prepared x in registers
 //   5 + 2 i  row i of the first group in registers   6 + 2 i  row i reduced   (i < 7)
 //   19 group stored (end)
 constexpr int TRACE_STAMPS = 20;
 __device__ unsigned long long *g_gemv_trace;
-struct TraceRequest { unsigned long long *d_buf; size_t capacity_waves; int waves_written; };
-thread_local TraceRequest trace_request = {nullptr, 0, 0};
 
 // (a register that the unit's loads fill, for the formats whose kernels are compiled with the trace)
 __device__ __forceinline__ uint32_t first_word_of(const Unit<RFQ_Q4_K> &u) { return u.q.v[3]; }
@@ -1588,7 +1613,7 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
     uint32_t *const xlds = idot_lds + LUT_DWORDS;
     WaveTrace<TRACE> trace;
     trace.stamp(0);
-    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;   // (made uniform with readfirstlane the headline kernel measured 2 % slower)
     const int team = wave / WPR, wit = wave % WPR;
     const int tl = wit * 64 + lane;
     const int ku = k >> 5;
@@ -2158,19 +2183,19 @@ int launch_idot(const uint8_t *w, const float *x, float *y, int n, int k, int bl
     }
     note_kernel(FUSE ? "gemv_idot_kernel<%s,%d,%d,%d,fused>" : "gemv_idot_kernel<%s,%d,%d,%d>", FMT, UPL, WPR, R);
     if constexpr (TraceCompiled<FMT, UPL, WPR, R, FUSE>::value) {
-        if (trace_request.d_buf != nullptr && (size_t)blocks * IDOT_WAVES <= trace_request.capacity_waves) {
+        if (g_gemv_trace_request.d_buf != nullptr && (size_t)blocks * IDOT_WAVES <= g_gemv_trace_request.capacity_waves) {
             if constexpr (FMT == RFQ_MXFP4) {
                 const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_idot_kernel<FMT, UPL, WPR, R, FUSE, true>),
                                                          hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 4096);
                 if (e != hipSuccess) return hip_fail(e, "hipFuncSetAttribute(gemv_idot_kernel, traced)");
             }
-            const hipError_t e = hipMemcpyToSymbol(HIP_SYMBOL(g_gemv_trace), &trace_request.d_buf, sizeof(trace_request.d_buf), 0,
+            const hipError_t e = hipMemcpyToSymbol(HIP_SYMBOL(g_gemv_trace), &g_gemv_trace_request.d_buf, sizeof(g_gemv_trace_request.d_buf), 0,
                                                    hipMemcpyHostToDevice);    // (blocking: a tool of the benchmark driver)
             if (e != hipSuccess) return hip_fail(e, "hipMemcpyToSymbol(g_gemv_trace)");
             hipLaunchKernelGGL((gemv_idot_kernel<FMT, UPL, WPR, R, FUSE, true>), dim3(blocks), dim3(64 * IDOT_WAVES), lds, s, w, x, y, n,
                                k, groups, f);
             RFQ_LAUNCH_CHECK("gemv_idot_kernel (traced)");
-            trace_request.waves_written = blocks * IDOT_WAVES;
+            g_gemv_trace_request.waves_written = blocks * IDOT_WAVES;
             return RFQ_OK;
         }
     }
@@ -2481,26 +2506,85 @@ int run_mm(const uint8_t *w, const float *x, float *y, int m, int n, int k, hipS
 
 } // namespace
 
+#define RFQ_GEMV_CAT2(a, b) a##b
+#define RFQ_GEMV_CAT(a, b) RFQ_GEMV_CAT2(a, b)
+
+// The formats of this part (the others' kernels are not instantiated here).
+int RFQ_GEMV_CAT(launch_gemv_part, RFQ_GEMV_PART)(int canonical, const uint8_t *d_w, const float *d_x, float *d_y, int m, int n,
+                                                  int k, hipStream_t s)
+{
+    constexpr int PART = RFQ_GEMV_PART;
+    return [&](auto part) -> int {
+        constexpr int P = decltype(part)::value;
+#define RFQ_GEMV_CASE(F, RUN)                                                             \
+    case F:                                                                              \
+        if constexpr (gemv_part_of(F) == P) return RUN<F>(d_w, d_x, d_y, m, n, k, s);   \
+        break;
+        switch (canonical) {
+            RFQ_GEMV_CASE(RFQ_Q4_0, run)
+            RFQ_GEMV_CASE(RFQ_Q8_0, run)
+            RFQ_GEMV_CASE(RFQ_Q4_K, run)
+            RFQ_GEMV_CASE(RFQ_Q6_K, run)
+            RFQ_GEMV_CASE(RFQ_MXFP4, run)
+            RFQ_GEMV_CASE(RFQ_MXFP6_E2M3, run)
+            RFQ_GEMV_CASE(RFQ_GGUF_Q4_0, run)
+            RFQ_GEMV_CASE(RFQ_GGUF_Q8_0, run)
+            RFQ_GEMV_CASE(RFQ_GGUF_Q4_K, run)
+            RFQ_GEMV_CASE(RFQ_GGUF_Q6_K, run)
+            RFQ_GEMV_CASE(RFQ_MM_Q8_0, run_mm)
+            RFQ_GEMV_CASE(RFQ_MM_Q4_K, run_mm)
+            RFQ_GEMV_CASE(RFQ_MM_Q6_K, run_mm)
+        default: break;
+        }
+#undef RFQ_GEMV_CASE
+        return fail(RFQ_E_UNSUPPORTED, "rfq_gemv: format %d is not in this part of the build", canonical);
+    }(std::integral_constant<int, PART>{});
+}
+
+int RFQ_GEMV_CAT(launch_gemv_fused_part, RFQ_GEMV_PART)(int canonical, const uint8_t *d_w, const float *d_x, float *d_y, int rows,
+                                                        int k, const void *fuse, hipStream_t s)
+{
+    constexpr int PART = RFQ_GEMV_PART;
+    const GemvFuse &f = *static_cast<const GemvFuse *>(fuse);
+    return [&](auto part) -> int {
+        constexpr int P = decltype(part)::value;
+#define RFQ_GEMV_CASE(F)                                                                             \
+    case F:                                                                                          \
+        if constexpr (gemv_part_of(F) == P) return run_rows<F, true>(d_w, d_x, d_y, rows, k, f, s); \
+        break;
+        switch (canonical) {
+            RFQ_GEMV_CASE(RFQ_Q4_0)
+            RFQ_GEMV_CASE(RFQ_Q8_0)
+            RFQ_GEMV_CASE(RFQ_Q4_K)
+            RFQ_GEMV_CASE(RFQ_Q6_K)
+            RFQ_GEMV_CASE(RFQ_MXFP4)
+            RFQ_GEMV_CASE(RFQ_MXFP6_E2M3)
+            RFQ_GEMV_CASE(RFQ_GGUF_Q4_0)
+            RFQ_GEMV_CASE(RFQ_GGUF_Q8_0)
+            RFQ_GEMV_CASE(RFQ_GGUF_Q4_K)
+            RFQ_GEMV_CASE(RFQ_GGUF_Q6_K)
+        default: break;
+        }
+#undef RFQ_GEMV_CASE
+        return fail(RFQ_E_UNSUPPORTED, "fused gemv: format %d is not in this part of the build", canonical);
+    }(std::integral_constant<int, PART>{});
+}
+
+#if RFQ_GEMV_PART == 0
+
 int launch_gemv(int fmt, const uint8_t *d_w, const float *d_x, float *d_y, int m, int n, int k, hipStream_t s)
 {
-    switch (canonical_format(fmt)) {
-    case RFQ_Q4_0: return run<RFQ_Q4_0>(d_w, d_x, d_y, m, n, k, s);
-    case RFQ_Q8_0: return run<RFQ_Q8_0>(d_w, d_x, d_y, m, n, k, s);
-    case RFQ_Q4_K: return run<RFQ_Q4_K>(d_w, d_x, d_y, m, n, k, s);
-    case RFQ_Q6_K: return run<RFQ_Q6_K>(d_w, d_x, d_y, m, n, k, s);
-    case RFQ_MXFP4: return run<RFQ_MXFP4>(d_w, d_x, d_y, m, n, k, s);
-    case RFQ_MXFP6_E2M3: return run<RFQ_MXFP6_E2M3>(d_w, d_x, d_y, m, n, k, s);
-    case RFQ_GGUF_Q4_0: return run<RFQ_GGUF_Q4_0>(d_w, d_x, d_y, m, n, k, s);
-    case RFQ_GGUF_Q8_0: return run<RFQ_GGUF_Q8_0>(d_w, d_x, d_y, m, n, k, s);
-    case RFQ_GGUF_Q4_K: return run<RFQ_GGUF_Q4_K>(d_w, d_x, d_y, m, n, k, s);
-    case RFQ_GGUF_Q6_K: return run<RFQ_GGUF_Q6_K>(d_w, d_x, d_y, m, n, k, s);
-    case RFQ_MM_Q8_0: return run_mm<RFQ_MM_Q8_0>(d_w, d_x, d_y, m, n, k, s);
-    case RFQ_MM_Q4_K: return run_mm<RFQ_MM_Q4_K>(d_w, d_x, d_y, m, n, k, s);
-    case RFQ_MM_Q6_K: return run_mm<RFQ_MM_Q6_K>(d_w, d_x, d_y, m, n, k, s);
+    const int cf = canonical_format(fmt);
+    switch (gemv_part_of(cf)) {
+    case 0: return launch_gemv_part0(cf, d_w, d_x, d_y, m, n, k, s);
+#ifndef RFQ_GEMV_ONLY
+    case 1: return launch_gemv_part1(cf, d_w, d_x, d_y, m, n, k, s);
+    case 2: return launch_gemv_part2(cf, d_w, d_x, d_y, m, n, k, s);
+    case 3: return launch_gemv_part3(cf, d_w, d_x, d_y, m, n, k, s);
+#endif
     default: return fail(RFQ_E_BADARG, "rfq_gemv: unknown format %d", fmt);
     }
 }
-
 
 // One launch for RMSNorm -> GEMV (norm_w != nullptr) and / or two GEMVs sharing
 // x -> SwiGLU (w2 != nullptr: y[j] = swiglu(w row j . x, w2 row j . x), n counts
@@ -2520,17 +2604,14 @@ int launch_gemv_fused(int fmt, const uint8_t *d_w, const uint8_t *d_w2, const fl
     if ((cf == RFQ_GGUF_Q6_K || cf == RFQ_GGUF_Q4_0 || cf == RFQ_GGUF_Q8_0) &&
         ((reinterpret_cast<uintptr_t>(d_w) | (d_w2 ? reinterpret_cast<uintptr_t>(d_w2) : 0)) & 3u) != 0)
         return RFQ_E_UNSUPPORTED;
-    switch (canonical_format(fmt)) {
-    case RFQ_Q4_0: return run_rows<RFQ_Q4_0, true>(d_w, d_x, d_y, rows, k, f, s);
-    case RFQ_Q8_0: return run_rows<RFQ_Q8_0, true>(d_w, d_x, d_y, rows, k, f, s);
-    case RFQ_Q4_K: return run_rows<RFQ_Q4_K, true>(d_w, d_x, d_y, rows, k, f, s);
-    case RFQ_Q6_K: return run_rows<RFQ_Q6_K, true>(d_w, d_x, d_y, rows, k, f, s);
-    case RFQ_MXFP4: return run_rows<RFQ_MXFP4, true>(d_w, d_x, d_y, rows, k, f, s);
-    case RFQ_MXFP6_E2M3: return run_rows<RFQ_MXFP6_E2M3, true>(d_w, d_x, d_y, rows, k, f, s);
-    case RFQ_GGUF_Q4_0: return run_rows<RFQ_GGUF_Q4_0, true>(d_w, d_x, d_y, rows, k, f, s);
-    case RFQ_GGUF_Q8_0: return run_rows<RFQ_GGUF_Q8_0, true>(d_w, d_x, d_y, rows, k, f, s);
-    case RFQ_GGUF_Q4_K: return run_rows<RFQ_GGUF_Q4_K, true>(d_w, d_x, d_y, rows, k, f, s);
-    case RFQ_GGUF_Q6_K: return run_rows<RFQ_GGUF_Q6_K, true>(d_w, d_x, d_y, rows, k, f, s);
+    if (cf == RFQ_MM_Q8_0 || cf == RFQ_MM_Q4_K || cf == RFQ_MM_Q6_K) return fail(RFQ_E_BADARG, "fused gemv: unknown format %d", fmt);
+    switch (gemv_part_of(cf)) {
+    case 0: return launch_gemv_fused_part0(cf, d_w, d_x, d_y, rows, k, &f, s);
+#ifndef RFQ_GEMV_ONLY
+    case 1: return launch_gemv_fused_part1(cf, d_w, d_x, d_y, rows, k, &f, s);
+    case 2: return launch_gemv_fused_part2(cf, d_w, d_x, d_y, rows, k, &f, s);
+    case 3: return launch_gemv_fused_part3(cf, d_w, d_x, d_y, rows, k, &f, s);
+#endif
     default: return fail(RFQ_E_BADARG, "fused gemv: unknown format %d", fmt);
     }
 }
@@ -2540,19 +2621,22 @@ int launch_gemv_fused(int fmt, const uint8_t *d_w, const uint8_t *d_w2, const fl
 int launch_gemv_traced(int fmt, const uint8_t *d_w, const float *d_x, float *d_y, int n, int k, unsigned long long *d_trace,
                        size_t capacity_waves, int *waves, hipStream_t s)
 {
-    trace_request = TraceRequest{d_trace, capacity_waves, 0};
+    g_gemv_trace_request = GemvTraceRequest{d_trace, capacity_waves, 0};
     const int rc = launch_gemv(fmt, d_w, d_x, d_y, 1, n, k, s);
-    *waves = trace_request.waves_written;
-    trace_request = TraceRequest{nullptr, 0, 0};
+    *waves = g_gemv_trace_request.waves_written;
+    g_gemv_trace_request = GemvTraceRequest{nullptr, 0, 0};
     return rc;
 }
 
+#endif // part 0
+
 } // namespace rfq
 
+#if RFQ_GEMV_PART == 0
 extern "C" RFQ_API const char *rfq_bench_last_gemv_kernel(void)
 {
     static thread_local char text[128];
-    const rfq::LastKernel &k = rfq::g_last_kernel;
+    const rfq::GemvLastKernel &k = rfq::g_gemv_last_kernel;
     const char *f = "?";
     switch (k.fmt) {
     case RFQ_Q4_0: f = "Q4_0"; break;
@@ -2573,3 +2657,4 @@ extern "C" RFQ_API const char *rfq_bench_last_gemv_kernel(void)
     snprintf(text, sizeof text, k.name, f, k.a, k.b, k.c);
     return text;
 }
+#endif // part 0
