@@ -778,6 +778,41 @@ __device__ __forceinline__ void store_group(const float (&res)[R], float (*part)
     }
 }
 
+// The plain GEMV of the integer-dot kernel reduces the R rows of a group together: every lane keeps its partial sum of
+// each row until the group is done, rows16_sum_of leaves lane l with the sum of row l % 8 over its 16-lane row (25
+// instructions where R wavefront sums took 11 each), and the four lane rows of each of the team's wavefronts meet in
+// LDS: part[row][4 * wavefront + lane row].  The caller alternates between two `part` arrays from group to group, so a
+// group's partial sums cannot be overwritten before they are read and one barrier per group is enough (none for a team
+// of one wavefront, whose LDS operations complete in order).
+constexpr int JOINT_ROWS = 8;
+template <int FMT> struct JointRows { static constexpr bool value = false; };
+template <> struct JointRows<RFQ_Q4_0> { static constexpr bool value = true; };
+template <> struct JointRows<RFQ_Q6_K> { static constexpr bool value = true; };
+template <> struct JointRows<RFQ_GGUF_Q4_0> { static constexpr bool value = true; };
+template <> struct JointRows<RFQ_GGUF_Q8_0> { static constexpr bool value = true; };
+template <> struct JointRows<RFQ_GGUF_Q6_K> { static constexpr bool value = true; };
+template <int R, int WPR, int WAVES>
+__device__ __forceinline__ void store_group_joint(const float (&acc)[R], float (*part)[WAVES * 4], float *__restrict__ y,
+                                                  int row_first, int row_end, int lane, int wave)
+{
+    static_assert(R <= JOINT_ROWS, "at most eight rows per group");
+    constexpr int M = R <= 2 ? 2 : (R <= 4 ? 4 : 8);
+    float a[M];
+#pragma unroll
+    for (int i = 0; i < M; i++) a[i] = i < R ? acc[i] : 0.f;
+    const float f = rows16_sum_of<M>(a, lane);
+    const int team = wave / WPR, wit = wave % WPR;
+    if ((lane & 15) < R) part[lane & 15][wave * 4 + (lane >> 4)] = f;   // (lanes 8..15 of a row repeat 0..7: same value, same slot)
+    if (WPR > 1) __syncthreads();
+    if (wit == 0 && lane < R) {
+        float t = 0.f;
+#pragma unroll
+        for (int q = 0; q < 4 * WPR; q++) t += part[lane][team * WPR * 4 + q];
+        const int r = row_first + lane;
+        if (r < row_end) y[r] = t;
+    }
+}
+
 // ---- m == 1, x resident in registers ----------------------------------------
 //
 // Block = 4 wavefronts = 4 / WPR teams.  Lane `tl` of a team (0 .. 64*WPR-1)
@@ -1695,17 +1730,28 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
     }
     // With the table the block keeps no static LDS (the table then starts at LDS address 0 and a look-up address
     // needs no base added): the partial sums follow the prepared x in the dynamic part.
-    float *ssq_part;
-    float (*part)[R][WAVES];
+    // (the fused forms keep one reduction per row, and so do the formats and forms where the joint one measured level
+    // or slower, 14336 x 4096: Q4_K 10.47 -> 10.53 us, GGUF_Q4_K 7.7 -> 9.2, MXFP4 9.4 -> 10.6, Q8_0 level; taken by
+    // GGUF_Q4_0 8.44 -> 7.86, GGUF_Q6_K 14.2 -> 13.1, Q6_K 12.1 -> 11.7, Q4_0 8.19 -> 7.88, GGUF_Q8_0 12.3 -> 12.0)
+    constexpr bool JOINT = !FUSE && JointRows<FMT>::value && WPR <= 2;
+    float *ssq_part = nullptr;
+    float (*part)[R][WAVES] = nullptr;
+    float (*partj)[JOINT_ROWS][WAVES * 4] = nullptr;
     if constexpr (LUT_DWORDS != 0) {
+        // (two workgroups with the table fit a CU's 160 KiB only with the small arrays: such a format reduces row by row)
+        static_assert(!JOINT, "the dynamic part of LDS is sized for one reduction per row");
         part = reinterpret_cast<float (*)[R][WAVES]>(xlds + (size_t)ku * 28);
         ssq_part = reinterpret_cast<float *>(part + 2);
+    } else if constexpr (JOINT) {
+        __shared__ float partj_static[2][JOINT_ROWS][WAVES * 4];
+        partj = partj_static;
     } else {
         __shared__ float ssq_part_static[WAVES];
         __shared__ float part_static[2][R][WAVES];
         ssq_part = ssq_part_static;
         part = part_static;
     }
+    (void)part; (void)partj; (void)ssq_part;
     if constexpr (FUSE) {
         if (norm) {
             ssq = wave_sum(ssq);
@@ -1778,13 +1824,15 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
             }
             if (i + D < R) load_row(i % D, base + i + D);
             else if (RING) load_row(i % D, base + i + D);
-            res[i] = wave_sum(acc);
+            if constexpr (JOINT) res[i] = acc;
+            else res[i] = wave_sum(acc);
             if constexpr (TRACE) {
                 if (g == 0) trace.stamp_after(6 + 2 * i, __float_as_uint(res[i]));
             }
         }
         // (`groups` is uniform over the block: every wavefront stores the same number of groups)
-        store_group<R, WPR, FUSE, WAVES, true>(res, part[g & 1], y, row0 + base, row_end, lane, wave, f, rinv);
+        if constexpr (JOINT) store_group_joint<R, WPR, WAVES>(res, partj[g & 1], y, row0 + base, row_end, lane, wave);
+        else store_group<R, WPR, FUSE, WAVES, true>(res, part[g & 1], y, row0 + base, row_end, lane, wave, f, rinv);
         if constexpr (TRACE) {
             if (g == 0) trace.stamp(19);
         }
