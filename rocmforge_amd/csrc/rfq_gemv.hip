@@ -2281,6 +2281,14 @@ int run_idot(const uint8_t *w, const float *x, float *y, int n, int k, const Gem
         static const int RS[5] = {2, 4, 5, 7, 8};
         int best_r = 8, best_groups = 1, best_blocks = 0;
         long best_cost = -1;
+        // (one row per team where two would leave CUs without a workgroup -- a key/value projection of a long hidden
+        // state: 1024 x 8192 4.38 -> 3.58 us, 1024 x 5120 3.50 -> 3.03, 512 x 8192 4.10 -> 3.11; teams of several
+        // wavefronts, plain GEMV)
+        constexpr bool ONE = UPL == 2 && WPR >= 2 && !FUSE;
+        if (ONE && want == 1 && n <= slots * TEAMS) {
+            const int blocks = (n + TEAMS - 1) / TEAMS;
+            return launch_idot<FMT, UPL, WPR, ONE ? 1 : 2, FUSE>(w, x, y, n, k, blocks, 1, f, s);
+        }
         for (int idx = 0; idx < 5; idx++) {
             int r = RS[idx];
             if (FUSE && f.glu && (r & 1)) continue;
