@@ -137,6 +137,10 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
                void *__restrict__ outp, int M, int N, int K)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    // INT: integer operands sc * q; acc runs in units of the current super-block's d (f32), rescaled between super-blocks
+    constexpr bool INT = FMT == KQ_GGUF_Q4_K_INT;
+    constexpr bool SUMS = FMT == RFQ_Q4_K || INT;                 // the min term goes through the activations' group sums
+    static_assert(!INT || PLANES == 1, "the integer operands are exact: one plane");
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int fr = lane & 31, fh = lane >> 5;                     // fragment row, k half
     const int tiles_m = (M + BM - 1) / BM;
@@ -225,7 +229,8 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
         // (group 2*stage + wh has the parity of wh; with one plane the ring slot is the stage's number within its super-block)
         raw.settle(wh, pair, PLANES == 1 ? decltype(slotc)::value : (st / PLANES) & 3);
 #pragma unroll
-        for (int i = 0; i < Raw32<FMT>::ND; i++) raw.d[i] = (st / PLANES) * 2 + wh < groups ? raw.d[i] : z.d[i];
+        // (the integer-operand decoder: sc = 0 makes every weight zero; its mask and offset dwords stay what every stage has)
+        for (int i = 0; i < (INT ? 2 : Raw32<FMT>::ND); i++) raw.d[i] = (st / PLANES) * 2 + wh < groups ? raw.d[i] : z.d[i];
     };
 
     // Four LDS buffers of decoded weights (buffer = stage % 4, a compile-time
@@ -265,11 +270,12 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
     uint32_t hm_ring = 0, hmA = 0, hmB = 0;
     v4u sa_cur[TI], sa_ring[TI];
     __amdgpu_buffer_rsrc_t s_tile[TI];
-    v8h fm[TJ];
+    v8h fm[TJ], fm_lo[TJ];
+    float d_unit = 1.0f;                                          // INT: the unit acc is in, for the row this thread decodes
     constexpr int MNR = 48;                                       // bytes per row of the min area (32 used)
     uint8_t *mn_wr = lds + 4 * W_BYTES + wr * MNR + wh * 16;
     const uint8_t *mn_rd = lds + 4 * W_BYTES + fr * MNR + fh * 16;
-    if constexpr (FMT == RFQ_Q4_K) {
+    if constexpr (SUMS) {
 #pragma unroll
         for (int i = 0; i < TI; i++) {
             const int mt = m0 / 32 + wave_u * 2 + i;
@@ -286,7 +292,7 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
         }
     };
     auto fetch_sums = [&](int trip) __attribute__((always_inline)) {
-        if constexpr (FMT == RFQ_Q4_K) {
+        if constexpr (SUMS) {
             const int t = trip < K / 256 ? trip : K / 256 - 1;
 #pragma unroll
             for (int i = 0; i < TI; i++) sa_ring[i] = __builtin_amdgcn_raw_buffer_load_b128(s_tile[i], lane16, t * 1024, 0);
@@ -309,16 +315,64 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
         }
         *reinterpret_cast<v8h *>(mn_wr) = h;
     };
-    auto compute_min = [&]() __attribute__((always_inline)) {
-        if constexpr (FMT == RFQ_Q4_K) {
+    constexpr int INT_AREA = 2 * BN * MNR + 2 * BN * 4;           // min fragments (hi, lo), ratio and unit of one super-block
+    uint8_t *const int_base = lds + 4 * W_BYTES + BN * MNR;
+    auto compute_min = [&](int parity) __attribute__((always_inline)) {
+        if constexpr (INT) {
+            const uint8_t *area = int_base + parity * INT_AREA + fr * MNR + fh * 16;
+#pragma unroll
+            for (int j = 0; j < TJ; j++) {
+                fm[j] = *reinterpret_cast<const v8h *>(area + j * 32 * MNR);
+                fm_lo[j] = *reinterpret_cast<const v8h *>(area + BN * MNR + j * 32 * MNR);
+            }
+        }
+        if constexpr (SUMS) {
 #pragma unroll
             for (int i = 0; i < TI; i++) {
                 v8h fa;
                 __builtin_memcpy(&fa, &sa_cur[i], 16);
 #pragma unroll
-                for (int j = 0; j < TJ; j++)
+                for (int j = 0; j < TJ; j++) {
                     acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fm[j], fa, acc[j][i], 0, 0, 0);
+                    if constexpr (INT) acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fm_lo[j], fa, acc[j][i], 0, 0, 0);
+                }
             }
+        }
+    };
+    // INT: acc is kept in units of the running super-block's d: sum over the super-blocks so far of (d_b / d) * sum
+    // (sc * q) * a - the matrix cores add the integer products, and between two super-blocks acc is multiplied by
+    // d_prev / d_next per weight row (f32; sixteen such roundings at k = 4096).  The min term -(dmin * m) * S is
+    // divided by d to join it.  A super-block's header goes to LDS when its first stage is settled (three stages
+    // before it is multiplied), into one of two areas by the super-block's parity: the two min fragments, the
+    // ratio that takes acc into its unit, and the unit itself (the epilogue multiplies by the last one).  A
+    // super-block with d = 0 has zero weights (settle() clears its sc) and keeps the previous unit.
+    auto stash_header = [&](const Raw32<FMT> &raw, int parity) __attribute__((always_inline)) {
+        if constexpr (INT) {
+            float ratio;
+            v8h m_hi, m_lo;
+            raw.header(wh, d_unit, ratio, m_hi, m_lo);
+            uint8_t *area = int_base + parity * INT_AREA;
+            *reinterpret_cast<v8h *>(area + wr * MNR + wh * 16) = m_hi;
+            *reinterpret_cast<v8h *>(area + BN * MNR + wr * MNR + wh * 16) = m_lo;
+            *reinterpret_cast<float *>(area + 2 * BN * MNR + wh * BN * 4 + wr * 4) = wh ? d_unit : ratio;
+        }
+    };
+    // acc *= f[n] (register r of a tile: n = 8*(r/4) + 4*fh + r%4: four factors side by side); which = 0: the ratio
+    // into the unit of the super-block of that parity, 1: that unit itself
+    auto rescale = [&](int parity, int which) __attribute__((always_inline)) {
+        if constexpr (INT) {
+            typedef float v4f __attribute__((ext_vector_type(4)));
+            const uint8_t *src = int_base + parity * INT_AREA + 2 * BN * MNR + which * BN * 4 + fh * 16;
+#pragma unroll
+            for (int j = 0; j < TJ; j++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const v4f f4 = *reinterpret_cast<const v4f *>(src + (j * 32 + 8 * g) * 4);
+#pragma unroll
+                    for (int i = 0; i < TI; i++)
+#pragma unroll
+                        for (int e = 0; e < 4; e++) acc[j][i][4 * g + e] *= f4[e];
+                }
         }
     };
 
@@ -359,12 +413,14 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
         v8h (&hw_late)[4] = (S & 1) ? hw_odd : hw_even;
         v8h (&hw_early)[4] = (S & 1) ? hw_even : hw_odd;
         v4u (&ra)[TI][4] = ra_of(IC<SH0>{});
-        if constexpr (FMT == RFQ_Q4_K) {
+        if constexpr (SUMS) {
             if (S == 0) {                                          // this trip's sums arrived with stage st's A
 #pragma unroll
                 for (int i = 0; i < TI; i++) sa_cur[i] = sa_ring[i];
                 fetch_sums(st / 4 + 1);
             }
+        }
+        if constexpr (FMT == RFQ_Q4_K) {
             if (S == 1) {                                          // stage st+3 opens the next super-block
                 // (real moves: merged with hs_ring's registers, the copy would
                 // turn into one at the end of the loop body that waits for the
@@ -400,6 +456,10 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
                             if ((S3 & 1) == 0 && p == EARLY[q]) raw_early.template step<true>(q, hw_early, lo_of(IC<(S3 >> 1) & 1>{}), dec_tmp);
                         }
                     }
+                }
+                if constexpr (INT) {
+                    // stage st+3 opens the next super-block: its header goes to the other area before settle() reuses the dwords
+                    if (S == 1 && p == 14) stash_header(raw_of(IC<S3>{}), ((st + 3) >> 2) & 1);
                 }
                 if (p == 15 && SH3 == S3) settle(IC<S3>{}, st + 3, S == 0 ? hsA[3] : hsB[S3]);   // stage st+3 is number S3 of its super-block
                 if (p >= 17 && p <= 23 && (p & 1)) {
@@ -451,6 +511,7 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
         // (a real move: the loop must not inherit a pending load on hmA, or its
         // first use in the loop body would wait for younger loads every trip)
         asm volatile("v_mov_b32 %0, %1" : "=v"(hmA) : "v"(hmA));
+        stash_header(raw0, 0);
         settle(IC<0>{}, 0, hsA[0]);
 #pragma unroll
         for (int T = 0; T < 12; T++) raw0.template step<PLANES == 2>(T, hw, hw_lo0, dec_tmp);
@@ -483,7 +544,8 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
         iter(IC<1>{}, st + 1);
         iter(IC<2>{}, st + 2);
         iter(IC<3>{}, st + 3);
-        compute_min();
+        compute_min((st >> 2) & 1);
+        rescale(((st >> 2) + 1) & 1, 0);                          // into the next super-block's unit
         if constexpr (FMT == RFQ_Q4_K) {
             hsA = hsB;
             hmA = hmB;
@@ -497,6 +559,7 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
     // 32 rows of a wavefront at a time in an area of its own, so that each
     // output row goes out as full 16-byte pieces of consecutive n instead of 8-
     // or 16-byte pieces one row apart.
+    rescale(((K / 256) - 1) & 1, 1);                               // INT: from the last super-block's unit to values
     typedef typename std::conditional<OUT_F16, _Float16, float>::type OutT;
     constexpr int ROWB = BN * (int)sizeof(OutT) + 16;             // bytes per staged row (row stride = 4 banks mod 32)
     static_assert(4 * 32 * ROWB <= 4 * W_BYTES, "staging area");
@@ -576,7 +639,8 @@ template <int FMT, bool OUT_F16, int PLANES>
 int launch_cfg(const uint8_t *w, const void *a, void *out, int m, int n, int k, uint8_t *static_tmp, const uint8_t *arranged,
                hipStream_t s)
 {
-    constexpr int LDS = 4 * W_BYTES + BN * 48;                  // four weight stages + the Q4_K min fragment
+    // four weight stages + the Q4_K min fragment (+ the integer-operand kernel's two header areas)
+    constexpr int LDS = 4 * W_BYTES + BN * 48 + (FMT == KQ_GGUF_Q4_K_INT ? 2 * (2 * BN * 48 + 2 * BN * 4) : 0);
     static_assert(LDS <= 160 * 1024, "LDS budget");
     static std::once_flag once;
     static hipError_t attr_err = hipSuccess;
@@ -596,7 +660,8 @@ int launch_cfg(const uint8_t *w, const void *a, void *out, int m, int n, int k, 
     // the temporary: the arranged activations, then the Q4_K group sums
     const int tiles32 = (m + 31) / 32, nst = (k + BK - 1) / BK;
     const size_t at_bytes = (size_t)tiles32 * nst * 4096;
-    const size_t s2_bytes = FMT == RFQ_Q4_K ? (size_t)tiles32 * (k / 256) * 1024 : 0;
+    constexpr bool SUMS = FMT == RFQ_Q4_K || FMT == KQ_GGUF_Q4_K_INT;
+    const size_t s2_bytes = SUMS ? (size_t)tiles32 * (k / 256) * 1024 : 0;
     uint8_t *tmp = static_tmp;
     bool transient = false;
     if (static_tmp != nullptr) {
@@ -608,7 +673,7 @@ int launch_cfg(const uint8_t *w, const void *a, void *out, int m, int n, int k, 
     }
     v4u *at = reinterpret_cast<v4u *>(tmp);
     _Float16 *s2 = reinterpret_cast<_Float16 *>(tmp + at_bytes);
-    hipLaunchKernelGGL((arrange_a_kernel<FMT == RFQ_Q4_K>), dim3((unsigned)(tiles32 * ((nst + 3) / 4))), dim3(256), 0, s,
+    hipLaunchKernelGGL((arrange_a_kernel<SUMS>), dim3((unsigned)(tiles32 * ((nst + 3) / 4))), dim3(256), 0, s,
                        reinterpret_cast<const _Float16 *>(a), at, s2, m, k, tiles32, nst);
     hipLaunchKernelGGL((gemm_kq_kernel<FMT, OUT_F16, PLANES>), dim3(tiles), dim3(256), LDS, s, w, at, s2, out, m, n, k);
     hipError_t launch_err = hipGetLastError();
@@ -627,7 +692,14 @@ int launch_fmt(const uint8_t *w, const void *a, void *out, int out_dtype, int m,
     // The 256-byte Q4_K layout is contracted in one plane (its large part, the integer mins, is exact and q * scale is
     // small beside it); every other format in two unless the caller asks for one.
     const bool f16 = (out_dtype & ~RFQ_GEMM_ONE_PLANE) == RFQ_F16;
-    if constexpr (FMT != RFQ_Q4_K) {
+    if constexpr (FMT == RFQ_GGUF_Q4_K) {
+        // exact in one pass: integer operands, d and dmin applied in f32
+        if ((out_dtype & RFQ_GEMM_ONE_PLANE) == 0) {
+            if (k % 256 != 0) return fail(RFQ_E_SIZE, "rfq_gemm_f16: k=%d is not whole Q4_K super-blocks", k);
+            return f16 ? launch_cfg<KQ_GGUF_Q4_K_INT, true, 1>(w, a, out, m, n, k, static_tmp, arranged, s)
+                       : launch_cfg<KQ_GGUF_Q4_K_INT, false, 1>(w, a, out, m, n, k, static_tmp, arranged, s);
+        }
+    } else if constexpr (FMT != RFQ_Q4_K) {
         if ((out_dtype & RFQ_GEMM_ONE_PLANE) == 0)
             return f16 ? launch_cfg<FMT, true, 2>(w, a, out, m, n, k, static_tmp, arranged, s)
                        : launch_cfg<FMT, false, 2>(w, a, out, m, n, k, static_tmp, arranged, s);

@@ -6,6 +6,10 @@
 #include "rfq_common.hpp"
 
 namespace rfq {
+// RFQ_GGUF_Q4_K bytes decoded to the integer operand sc * q (Raw32<KQ_GGUF_Q4_K_INT> below): a name inside this
+// library, not a format of the C ABI.
+constexpr int KQ_GGUF_Q4_K_INT = 0x1000 + RFQ_GGUF_Q4_K;
+template <> struct Fmt<KQ_GGUF_Q4_K_INT> { static constexpr int BE = 256, BB = 144; };
 namespace kq {
 
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
@@ -348,6 +352,102 @@ template <> struct Raw32<RFQ_GGUF_Q4_K> {
             fp16_parts<BOTH>(value(8 * c + e), hi, lo);
             h[c][chunk_pos(e)] = hi;
             if constexpr (BOTH) l[c][chunk_pos(e)] = lo;
+        }
+    }
+};
+
+// block_q4_K contracted exactly in one pass: the operand is the integer sc * q (at most 63 * 15 = 945, exact in
+// fp16), summed over a super-block by the matrix cores; d multiplies that sum in f32 and -(dmin * m) goes through
+// the sub-block sums of the activations (the kernel does both).
+template <> struct Raw32<KQ_GGUF_Q4_K_INT> {
+    static constexpr int ND = 12;
+    uint32_t d[ND];
+    __device__ __forceinline__ void load(Rsrc w, uint32_t row_off, int st, int)
+    {
+        const int blk = (st >> 2) * 144;
+        v4u h = __builtin_amdgcn_raw_buffer_load_b128(w, row_off, blk, 0);
+        v4u q0 = __builtin_amdgcn_raw_buffer_load_b128(w, row_off + 16, blk + 32 * (st & 3), 0);
+        v4u q1 = __builtin_amdgcn_raw_buffer_load_b128(w, row_off + 32, blk + 32 * (st & 3), 0);
+        d[0] = h[0]; d[1] = h[1]; d[2] = h[2]; d[3] = h[3];
+        d[4] = q0[0]; d[5] = q0[1]; d[6] = q0[2]; d[7] = q0[3];
+        d[8] = q1[0]; d[9] = q1[1]; d[10] = q1[2]; d[11] = q1[3];
+    }
+    __device__ __forceinline__ void zero()
+    {
+#pragma unroll
+        for (int i = 0; i < ND; i++) d[i] = 0;
+    }
+    // Before settle().  `unit` comes in as the d the accumulators are in and leaves as this super-block's d (the old
+    // one when d = 0: such a super-block has zero weights, settle() clears its sc); ratio = old / new.  For the
+    // thread's four sub-blocks 4*wh .. 4*wh+3, v = -(dmin * m) / unit (dmin * m is exact in f32: 11 x 6 bits) as the
+    // fp16 pairs (hi, hi) and (lo, 0) with hi + lo = v: contracted with the activations' group sums (S_hi, S_lo)
+    // they give hi * S_hi + hi * S_lo + lo * S_hi.
+    __device__ __forceinline__ void header(int wh, float &unit, float &ratio, v8h &m_hi, v8h &m_lo) const
+    {
+        const float dv = f16_bits_to_f32((uint16_t)(d[0] & 0xFFFFu));
+        const float dmin = f16_bits_to_f32((uint16_t)(d[0] >> 16));
+        const float next = dv != 0.0f ? dv : unit;
+        const float inv = 1.0f / next;
+        ratio = unit * inv;
+        unit = next;
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            // (both halves unpacked with compile-time sub-block numbers, the thread's half chosen after)
+            const uint32_t m0 = gguf_scale_min_k4(q, d[1], d[2], d[3]) >> 8, m1 = gguf_scale_min_k4(4 + q, d[1], d[2], d[3]) >> 8;
+            const float v = -(dmin * (float)(wh ? m1 : m0)) * inv;
+            const _Float16 hi = (_Float16)v, lo = (_Float16)(v - (float)hi);
+            m_hi[2 * q] = hi;
+            m_hi[2 * q + 1] = hi;
+            m_lo[2 * q] = lo;
+            m_lo[2 * q + 1] = (_Float16)0.0f;
+        }
+    }
+    // d[0] = (sc, sc) as fp16, d[1] = -(offset * sc) twice, d[2] = the nibble mask of this half, d[3] = the fp16 bits the
+    // nibbles are or-ed into: low nibbles read 1024 + q (0x6400 | q), high nibbles 64 + q (0x5400 | q << 4).
+    // c = the stage's number within its super-block (a compile-time constant at the call), wh = the thread's nibble half.
+    __device__ __forceinline__ void settle(int wh, uint32_t, int c)
+    {
+        const uint32_t s0 = gguf_scale_min_k4(2 * c, d[1], d[2], d[3]) & 255u, s1 = gguf_scale_min_k4(2 * c + 1, d[1], d[2], d[3]) & 255u;
+        const float sc = (d[0] & 0x7FFFu) != 0 ? (float)(wh ? s1 : s0) : 0.0f;   // d = 0: zero weights
+        const _Float16 h = (_Float16)sc, o = (_Float16)(-(wh ? 64.0f : 1024.0f) * sc);   // both exact (sc < 64)
+        uint16_t hb, ob;
+        __builtin_memcpy(&hb, &h, 2);
+        __builtin_memcpy(&ob, &o, 2);
+        d[0] = hb * 0x10001u;
+        d[1] = ob * 0x10001u;
+        d[2] = wh ? 0x00F000F0u : 0x000F000Fu;
+        d[3] = wh ? 0x54005400u : 0x64006400u;
+    }
+    // Chunk c = elements 8c .. 8c+7 of the sub-block = bytes 8c .. 8c+7 of the stage's 32: dwords x0 (k0..k3) and x1
+    // (k4..k7).  Their low halves side by side are the bytes (k0 k1 k4 k5): one and-or gives the pair (k0, k4), the same
+    // on the dword shifted by 8 (k1, k5); the high halves (k2, k6) and (k3, k7) - the order the activations are in.
+    // (offset + q) * sc - offset * sc as one fp16 fused multiply-add: sc * q, exact.
+    template <bool BOTH> __device__ __forceinline__ void step(int T, v8h (&h)[4], v8h (&)[4], v2h (&t)[4]) const
+    {
+        const int c = T / 3, ph = T % 3;
+        if (ph == 0) {
+            const uint32_t u0 = __builtin_amdgcn_perm(d[5 + 2 * c], d[4 + 2 * c], 0x05040100u);
+            const uint32_t u1 = __builtin_amdgcn_perm(d[5 + 2 * c], d[4 + 2 * c], 0x07060302u);
+            const uint32_t b0 = (u0 & d[2]) | d[3], b1 = ((u0 >> 8) & d[2]) | d[3];
+            __builtin_memcpy(&t[0], &b0, 4);
+            __builtin_memcpy(&t[1], &b1, 4);
+            __builtin_memcpy(&t[2], &u1, 4);
+        } else if (ph == 1) {
+            uint32_t u1;
+            __builtin_memcpy(&u1, &t[2], 4);
+            const uint32_t b2 = (u1 & d[2]) | d[3], b3 = ((u1 >> 8) & d[2]) | d[3];
+            __builtin_memcpy(&t[2], &b2, 4);
+            __builtin_memcpy(&t[3], &b3, 4);
+        } else {
+            v2h s2, o2;
+            __builtin_memcpy(&s2, &d[0], 4);
+            __builtin_memcpy(&o2, &d[1], 4);
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const v2h v = __builtin_elementwise_fma(t[q], s2, o2);
+                h[c][2 * q] = v[0];
+                h[c][2 * q + 1] = v[1];
+            }
         }
     }
 };
