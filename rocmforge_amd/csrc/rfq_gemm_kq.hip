@@ -50,9 +50,21 @@
 // holds its own copy of this array until the process ends.  Host code never uses the array's name as an address:
 // static_scratch() resolves the copy of the current device once and hands out that pointer.
 constexpr size_t RFQ_STATIC_SCRATCH_BYTES = (size_t)16 << 20;
+// This file is compiled in two parts (RFQ_KQ_PART): part 1 holds only the integer-operand kernel of GGUF_Q4_K, whose
+// accumulators are multiplied by vector instructions between super-blocks and therefore want to live in ordinary
+// vector registers (-amdgpu-mfma-vgpr-form: 83.6 -> 77.1 us at 512 x 4096 x 14336); the other kernels measured
+// slower that way (Q4_K 65.6 -> 68.0 us) and are part 0, with the entry points and everything that owns memory.
+#ifndef RFQ_KQ_PART
+#define RFQ_KQ_PART 0
+#endif
+#if RFQ_KQ_PART == 0
 static __device__ __align__(256) uint8_t scratch[RFQ_STATIC_SCRATCH_BYTES];
+#endif
 
 namespace rfq {
+// (defined in part 1 of this file)
+int launch_gguf_q4_k_int(const uint8_t *w, const void *a, void *out, bool out_f16, int m, int n, int k, uint8_t *static_tmp,
+                         const uint8_t *arranged, hipStream_t s);
 namespace {
 
 using namespace kq;
@@ -376,6 +388,45 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
         }
     };
 
+    // INT, the end of a super-block: its min term (two k-steps per tile: the hi and the lo fragment against the group
+    // sums), then acc into the next super-block's unit.  The multiplications of one pair of tiles run beside the
+    // matrix instructions of the next pair.
+    auto trip_end = [&](int parity) __attribute__((always_inline)) {
+        if constexpr (INT) {
+            typedef float v4f __attribute__((ext_vector_type(4)));
+            const uint8_t *area = int_base + parity * INT_AREA + fr * MNR + fh * 16;
+            const uint8_t *src = int_base + (parity ^ 1) * INT_AREA + 2 * BN * MNR + fh * 16;
+            v8h fa[TI];
+#pragma unroll
+            for (int i = 0; i < TI; i++) __builtin_memcpy(&fa[i], &sa_cur[i], 16);
+            v4f f4[2][4];
+#pragma unroll
+            for (int j = 0; j < TJ; j++) {
+                fm[j] = *reinterpret_cast<const v8h *>(area + j * 32 * MNR);
+                fm_lo[j] = *reinterpret_cast<const v8h *>(area + BN * MNR + j * 32 * MNR);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j <= TJ; j++) {
+                if (j < TJ) {
+#pragma unroll
+                    for (int g = 0; g < 4; g++) f4[j & 1][g] = *reinterpret_cast<const v4f *>(src + (j * 32 + 8 * g) * 4);
+#pragma unroll
+                    for (int i = 0; i < TI; i++) acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fm[j], fa[i], acc[j][i], 0, 0, 0);
+#pragma unroll
+                    for (int i = 0; i < TI; i++) acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fm_lo[j], fa[i], acc[j][i], 0, 0, 0);
+                }
+                if (j > 0) {
+#pragma unroll
+                    for (int i = 0; i < TI; i++)
+#pragma unroll
+                        for (int r = 0; r < 16; r++) acc[j - 1][i][r] *= f4[(j - 1) & 1][r >> 2][r & 3];
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    };
+
     // One wavefront per SIMD: nothing hides a stall, so the body of a stage is
     // laid out by hand as 32 slots of one matrix instruction plus a share of
     // the stage's other work, and pinned in that order.  Iteration st (S =
@@ -544,8 +595,8 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
         iter(IC<1>{}, st + 1);
         iter(IC<2>{}, st + 2);
         iter(IC<3>{}, st + 3);
-        compute_min((st >> 2) & 1);
-        rescale(((st >> 2) + 1) & 1, 0);                          // into the next super-block's unit
+        if constexpr (INT) trip_end((st >> 2) & 1);
+        else compute_min((st >> 2) & 1);
         if constexpr (FMT == RFQ_Q4_K) {
             hsA = hsB;
             hmA = hmB;
@@ -685,6 +736,7 @@ int launch_cfg(const uint8_t *w, const void *a, void *out, int m, int n, int k, 
     return RFQ_OK;
 }
 
+#if RFQ_KQ_PART == 0
 template <int FMT>
 int launch_fmt(const uint8_t *w, const void *a, void *out, int out_dtype, int m, int n, int k, uint8_t *static_tmp,
                const uint8_t *arranged, hipStream_t s)
@@ -696,8 +748,7 @@ int launch_fmt(const uint8_t *w, const void *a, void *out, int out_dtype, int m,
         // exact in one pass: integer operands, d and dmin applied in f32
         if ((out_dtype & RFQ_GEMM_ONE_PLANE) == 0) {
             if (k % 256 != 0) return fail(RFQ_E_SIZE, "rfq_gemm_f16: k=%d is not whole Q4_K super-blocks", k);
-            return f16 ? launch_cfg<KQ_GGUF_Q4_K_INT, true, 1>(w, a, out, m, n, k, static_tmp, arranged, s)
-                       : launch_cfg<KQ_GGUF_Q4_K_INT, false, 1>(w, a, out, m, n, k, static_tmp, arranged, s);
+            return launch_gguf_q4_k_int(w, a, out, f16, m, n, k, static_tmp, arranged, s);
         }
     } else if constexpr (FMT != RFQ_Q4_K) {
         if ((out_dtype & RFQ_GEMM_ONE_PLANE) == 0)
@@ -727,7 +778,18 @@ int static_scratch(uint8_t **out)
     return RFQ_OK;
 }
 
+#endif // RFQ_KQ_PART == 0
+
 } // namespace
+
+#if RFQ_KQ_PART == 1
+int launch_gguf_q4_k_int(const uint8_t *w, const void *a, void *out, bool out_f16, int m, int n, int k, uint8_t *static_tmp,
+                         const uint8_t *arranged, hipStream_t s)
+{
+    return out_f16 ? launch_cfg<KQ_GGUF_Q4_K_INT, true, 1>(w, a, out, m, n, k, static_tmp, arranged, s)
+                   : launch_cfg<KQ_GGUF_Q4_K_INT, false, 1>(w, a, out, m, n, k, static_tmp, arranged, s);
+}
+#else
 
 // Temporary device memory for one call.  Up to WS_KEEP bytes it is a buffer
 // the library keeps per stream (calls on one stream run in order, so the next
@@ -884,5 +946,7 @@ int launch_gemm_f16(int fmt, const uint8_t *d_w, const void *d_a, void *d_out, i
     default: return fail(RFQ_E_UNSUPPORTED, "rfq_gemm_f16: no fp16 matrix-core kernel for format %d", fmt);
     }
 }
+
+#endif // RFQ_KQ_PART
 
 } // namespace rfq
