@@ -105,7 +105,9 @@ def kq_gemm(torch, fmt, m=512, n=14336, k=4096, steps=300, warmup=300, arranged=
     flops = 2.0 * m * n * k
     res = {"TFLOP/s": round(flops / t / 1e12, 1), "us": round(t * 1e6, 1), "mfma_frac": round(flops / t / 2.5e15, 4),
            "peak_TFLOP/s": 2500.0, "warmup_launches": warmup, "timed_launches": steps,
-           "fp16_operands_per_weight": 1 if fmt == Q.Q4_K else 2}
+           "fp16_operands_per_weight": 1 if fmt in (Q.Q4_K, Q.GGUF_Q4_K) else 2}
+    if fmt == Q.GGUF_Q4_K:
+        res["what"] = "exact in one pass: integer operands sc*q, d and dmin applied in f32 per super-block"
     if one_plane and fmt != Q.Q4_K:
         args1 = args[:5] + (_lib.F16 | _lib.GEMM_ONE_PLANE,) + args[6:]
         _lib.check(L.rfq_bench_gemm_f16(*args1, warmup, steps, stream, C.byref(ms)))

@@ -319,8 +319,10 @@ RFQ_API int rfq_mlp_swiglu(int fmt_gate_up, const void *d_gate_w, const void *d_
  * contracted as two fp16 operands, hi = fp16(v) and lo = fp16(v - hi) (v to
  * 2^-22: the result is that of an fp32 contraction, 5e-6 of rms(out) from the
  * reference's at 512 x 4096 x 14336); the 256-byte Q4_K layout, whose integer
- * mins are contracted exactly and apart, takes q * scale as one operand.  With
- * RFQ_GEMM_ONE_PLANE every format takes one (8e-4 of rms(out)).  k a multiple of 256
+ * mins are contracted exactly and apart, takes q * scale as one operand, and
+ * RFQ_GGUF_Q4_K is contracted exactly in one pass (integer operands sc * q,
+ * the super-block's d and dmin applied in f32).  With
+ * RFQ_GEMM_ONE_PLANE every format takes one rounded operand (8e-4 of rms(out)).  k a multiple of 256
  * for the K-formats, of 32 otherwise; d_a_f16 16-byte aligned, d_w 4-byte aligned.  Up to 64 MiB of
  * temporary device memory (the activations in matrix-operand order) is kept
  * per stream between calls; larger temporaries are allocated and released in

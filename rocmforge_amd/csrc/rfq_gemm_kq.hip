@@ -283,6 +283,8 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
     v4u sa_cur[TI], sa_ring[TI];
     __amdgpu_buffer_rsrc_t s_tile[TI];
     v8h fm[TJ], fm_lo[TJ];
+    typedef float v4f __attribute__((ext_vector_type(4)));
+    v4f f4[2][4];                                                 // INT: the ratios of the tile rescaled next
     float d_unit = 1.0f;                                          // INT: the unit acc is in, for the row this thread decodes
     constexpr int MNR = 48;                                       // bytes per row of the min area (32 used)
     uint8_t *mn_wr = lds + 4 * W_BYTES + wr * MNR + wh * 16;
@@ -330,15 +332,7 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
     constexpr int INT_AREA = 2 * BN * MNR + 2 * BN * 4;           // min fragments (hi, lo), ratio and unit of one super-block
     uint8_t *const int_base = lds + 4 * W_BYTES + BN * MNR;
     auto compute_min = [&](int parity) __attribute__((always_inline)) {
-        if constexpr (INT) {
-            const uint8_t *area = int_base + parity * INT_AREA + fr * MNR + fh * 16;
-#pragma unroll
-            for (int j = 0; j < TJ; j++) {
-                fm[j] = *reinterpret_cast<const v8h *>(area + j * 32 * MNR);
-                fm_lo[j] = *reinterpret_cast<const v8h *>(area + BN * MNR + j * 32 * MNR);
-            }
-        }
-        if constexpr (SUMS) {
+        if constexpr (SUMS && !INT) {
 #pragma unroll
             for (int i = 0; i < TI; i++) {
                 v8h fa;
@@ -346,7 +340,6 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
 #pragma unroll
                 for (int j = 0; j < TJ; j++) {
                     acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fm[j], fa, acc[j][i], 0, 0, 0);
-                    if constexpr (INT) acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fm_lo[j], fa, acc[j][i], 0, 0, 0);
                 }
             }
         }
@@ -385,45 +378,6 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
 #pragma unroll
                         for (int e = 0; e < 4; e++) acc[j][i][4 * g + e] *= f4[e];
                 }
-        }
-    };
-
-    // INT, the end of a super-block: its min term (two k-steps per tile: the hi and the lo fragment against the group
-    // sums), then acc into the next super-block's unit.  The multiplications of one pair of tiles run beside the
-    // matrix instructions of the next pair.
-    auto trip_end = [&](int parity) __attribute__((always_inline)) {
-        if constexpr (INT) {
-            typedef float v4f __attribute__((ext_vector_type(4)));
-            const uint8_t *area = int_base + parity * INT_AREA + fr * MNR + fh * 16;
-            const uint8_t *src = int_base + (parity ^ 1) * INT_AREA + 2 * BN * MNR + fh * 16;
-            v8h fa[TI];
-#pragma unroll
-            for (int i = 0; i < TI; i++) __builtin_memcpy(&fa[i], &sa_cur[i], 16);
-            v4f f4[2][4];
-#pragma unroll
-            for (int j = 0; j < TJ; j++) {
-                fm[j] = *reinterpret_cast<const v8h *>(area + j * 32 * MNR);
-                fm_lo[j] = *reinterpret_cast<const v8h *>(area + BN * MNR + j * 32 * MNR);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int j = 0; j <= TJ; j++) {
-                if (j < TJ) {
-#pragma unroll
-                    for (int g = 0; g < 4; g++) f4[j & 1][g] = *reinterpret_cast<const v4f *>(src + (j * 32 + 8 * g) * 4);
-#pragma unroll
-                    for (int i = 0; i < TI; i++) acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fm[j], fa[i], acc[j][i], 0, 0, 0);
-#pragma unroll
-                    for (int i = 0; i < TI; i++) acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fm_lo[j], fa[i], acc[j][i], 0, 0, 0);
-                }
-                if (j > 0) {
-#pragma unroll
-                    for (int i = 0; i < TI; i++)
-#pragma unroll
-                        for (int r = 0; r < 16; r++) acc[j - 1][i][r] *= f4[(j - 1) & 1][r >> 2][r & 3];
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
         }
     };
 
@@ -509,6 +463,31 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
                     }
                 }
                 if constexpr (INT) {
+                    // The super-block's min term rides on its first stage: behind the first k-step's matrix
+                    // instruction of a tile the hi fragment against the group sums, behind the second the lo fragment.
+                    if (S == 0 && c < 2) {
+                        v8h fs;
+                        __builtin_memcpy(&fs, &sa_cur[i], 16);
+                        acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(c == 0 ? fm[j] : fm_lo[j], fs, acc[j][i], 0, 0, 0);
+                    }
+                    // A tile goes into the next super-block's unit in the slot after its last matrix instruction
+                    // of this one (the last tile at the start of the next stage); the ratios of a tile's 16
+                    // weight rows are read one slot before.
+                    const uint8_t *next_area = int_base + (((st >> 2) + 1) & 1) * INT_AREA;
+                    if ((S == 3 && p >= 25) || (S == 0 && p == 0)) {
+                        const int tile = S == 3 ? p - 25 : 7;
+#pragma unroll
+                        for (int r = 0; r < 16; r++) acc[tile & 3][tile >> 2][r] *= f4[tile & 1][r >> 2][r & 3];
+                    }
+                    if (S == 3 && p >= 24) {
+#pragma unroll
+                        for (int g = 0; g < 4; g++)
+                            f4[t & 1][g] = *reinterpret_cast<const v4f *>(next_area + 2 * BN * MNR + fh * 16 + (j * 32 + 8 * g) * 4);
+                    }
+                    // the fragments of the next super-block's min term
+                    if (S == 3 && p >= 28) fm[p - 28] = *reinterpret_cast<const v8h *>(next_area + fr * MNR + fh * 16 + (p - 28) * 32 * MNR);
+                    if (S == 0 && p < 4)
+                        fm_lo[p] = *reinterpret_cast<const v8h *>(int_base + ((st >> 2) & 1) * INT_AREA + BN * MNR + fr * MNR + fh * 16 + p * 32 * MNR);
                     // stage st+3 opens the next super-block: its header goes to the other area before settle() reuses the dwords
                     if (S == 1 && p == 14) stash_header(raw_of(IC<S3>{}), ((st + 3) >> 2) & 1);
                 }
@@ -587,6 +566,12 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
         lds_barrier();
 #pragma unroll
         for (int j = 0; j < TJ; j++) fw[0][j] = read_frag(0, j, 0);
+        if constexpr (INT) {
+#pragma unroll
+            for (int j = 0; j < TJ; j++) fm[j] = *reinterpret_cast<const v8h *>(int_base + fr * MNR + fh * 16 + j * 32 * MNR);
+#pragma unroll
+            for (int r = 0; r < 16; r++) f4[1][r >> 2][r & 3] = 1.0f;   // (the first stage multiplies the empty last tile by these)
+        }
     }
     // Whole trips through the ring only (no branch between the four bodies);
     // stages past the end multiply zero weights.
@@ -595,8 +580,7 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
         iter(IC<1>{}, st + 1);
         iter(IC<2>{}, st + 2);
         iter(IC<3>{}, st + 3);
-        if constexpr (INT) trip_end((st >> 2) & 1);
-        else compute_min((st >> 2) & 1);
+        compute_min((st >> 2) & 1);
         if constexpr (FMT == RFQ_Q4_K) {
             hsA = hsB;
             hmA = hmB;

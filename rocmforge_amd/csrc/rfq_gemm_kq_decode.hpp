@@ -377,18 +377,27 @@ template <> struct Raw32<KQ_GGUF_Q4_K_INT> {
 #pragma unroll
         for (int i = 0; i < ND; i++) d[i] = 0;
     }
-    // Before settle().  `unit` comes in as the d the accumulators are in and leaves as this super-block's d (the old
-    // one when d = 0: such a super-block has zero weights, settle() clears its sc); ratio = old / new.  For the
-    // thread's four sub-blocks 4*wh .. 4*wh+3, v = -(dmin * m) / unit (dmin * m is exact in f32: 11 x 6 bits) as the
-    // fp16 pairs (hi, hi) and (lo, 0) with hi + lo = v: contracted with the activations' group sums (S_hi, S_lo)
-    // they give hi * S_hi + hi * S_lo + lo * S_hi.
+    // The unit a super-block's sums are kept in is d * 2^j: j > 0 only where -(dmin * m) / d would leave the fp16 range
+    // (data far from zero against its spread: |dmin| * 64 >= 2^15 * |d|); the operand is then sc * q * 2^-j, still exact
+    // (945 * 2^-24 is an fp16 number).  j from the f32 exponent fields: |dmin * 63 / d| < 2^(e_dmin - e_d + 7).
+    static __device__ __forceinline__ int unit_shift(float dv, float dmin)
+    {
+        const int j = (int)((__float_as_uint(dmin) >> 23) & 255u) - (int)((__float_as_uint(dv) >> 23) & 255u) - 8;
+        return j < 0 ? 0 : (j > 24 ? 24 : j);
+    }
+    // Before settle().  `unit` comes in as the unit the accumulators are in and leaves as this super-block's;
+    // ratio = old / new.  A super-block with d = 0 has no q term (settle() clears its sc) and takes |dmin| as its
+    // unit, or the old one when dmin is 0 too.  For the thread's four sub-blocks 4*wh .. 4*wh+3,
+    // v = -(dmin * m) / unit (dmin * m is exact in f32: 11 x 6 bits) as the fp16 pairs (hi, hi) and (lo, 0) with
+    // hi + lo = v: contracted with the activations' group sums (S_hi, S_lo) they give hi * S_hi + hi * S_lo + lo * S_hi.
     __device__ __forceinline__ void header(int wh, float &unit, float &ratio, v8h &m_hi, v8h &m_lo) const
     {
         const float dv = f16_bits_to_f32((uint16_t)(d[0] & 0xFFFFu));
         const float dmin = f16_bits_to_f32((uint16_t)(d[0] >> 16));
-        const float next = dv != 0.0f ? dv : unit;
+        const float scaled = dv * __uint_as_float((uint32_t)(127 + unit_shift(dv, dmin)) << 23);
+        const float next = dv != 0.0f ? scaled : (dmin != 0.0f ? __builtin_fabsf(dmin) : unit);
         const float inv = 1.0f / next;
-        ratio = unit * inv;
+        ratio = next == unit ? 1.0f : unit * inv;
         unit = next;
 #pragma unroll
         for (int q = 0; q < 4; q++) {
@@ -402,14 +411,16 @@ template <> struct Raw32<KQ_GGUF_Q4_K_INT> {
             m_lo[2 * q + 1] = (_Float16)0.0f;
         }
     }
-    // d[0] = (sc, sc) as fp16, d[1] = -(offset * sc) twice, d[2] = the nibble mask of this half, d[3] = the fp16 bits the
-    // nibbles are or-ed into: low nibbles read 1024 + q (0x6400 | q), high nibbles 64 + q (0x5400 | q << 4).
+    // d[0] = (s, s) as fp16 with s = sc * 2^-j, d[1] = -(offset * s) twice, d[2] = the nibble mask of this half, d[3] =
+    // the fp16 bits the nibbles are or-ed into: low nibbles read 1024 + q (0x6400 | q), high nibbles 64 + q (0x5400 | q << 4).
     // c = the stage's number within its super-block (a compile-time constant at the call), wh = the thread's nibble half.
     __device__ __forceinline__ void settle(int wh, uint32_t, int c)
     {
         const uint32_t s0 = gguf_scale_min_k4(2 * c, d[1], d[2], d[3]) & 255u, s1 = gguf_scale_min_k4(2 * c + 1, d[1], d[2], d[3]) & 255u;
-        const float sc = (d[0] & 0x7FFFu) != 0 ? (float)(wh ? s1 : s0) : 0.0f;   // d = 0: zero weights
-        const _Float16 h = (_Float16)sc, o = (_Float16)(-(wh ? 64.0f : 1024.0f) * sc);   // both exact (sc < 64)
+        const float dv = f16_bits_to_f32((uint16_t)(d[0] & 0xFFFFu)), dmin = f16_bits_to_f32((uint16_t)(d[0] >> 16));
+        const float down = __uint_as_float((uint32_t)(127 - unit_shift(dv, dmin)) << 23);
+        const float sc = dv != 0.0f ? (float)(wh ? s1 : s0) * down : 0.0f;   // d = 0: no q term
+        const _Float16 h = (_Float16)sc, o = (_Float16)(-(wh ? 64.0f : 1024.0f) * sc);   // both exact (sc < 64, j <= 24)
         uint16_t hb, ob;
         __builtin_memcpy(&hb, &h, 2);
         __builtin_memcpy(&ob, &o, 2);

@@ -143,6 +143,45 @@ def test_one_plane_is_the_fp16_rounded_contraction(fmt, oracle, cuda):
     assert not np.array_equal(out, two)
 
 
+def test_gguf_q4_k_super_block_scales_of_any_size(oracle, cuda):
+    """GGUF_Q4_K is contracted with integer operands and its accumulators run in units of the current super-block's d:
+    super-blocks whose d is +0, -0, negative, or 2^+-8 times the neighbour's (also in a row's first and last block,
+    and a whole row of zeros) must come out as the oracle's."""
+    import torch
+    m, n, k = 70, 140, 2048                                               # 8 super-blocks per row
+    w = weights(Q.GGUF_Q4_K, n, k, 51).copy()
+    blocks = w.reshape(n, k // 256, 144)
+    d = blocks[:, :, 0:2].copy().view("<f2")[..., 0]                      # [n, 8]
+    rng = np.random.Generator(np.random.PCG64(52))
+    d[0, :] = 0.0                                                         # a row without any scale (its mins remain)
+    d[1, 0] = 0.0                                                         # zero first, later not
+    d[2, 7] = 0.0
+    d[3, 3] = -0.0
+    d[4, :] = -d[4, :]
+    d[5, 1::2] *= np.float16(256.0)
+    d[6, 1::2] /= np.float16(256.0)
+    pick = rng.integers(0, 8, size=n)
+    for r in range(7, n, 3): d[r, pick[r]] = 0.0
+    for r in range(8, n, 5): d[r, pick[r]] *= np.float16(-64.0)
+    blocks[:, :, 0:2] = d.astype("<f2")[..., None].view(np.uint8)
+    dmin = blocks[:, :, 2:4].copy().view("<f2")[..., 0]
+    dmin[9::4, 2] = 0.0
+    dmin[10::7, :] = -dmin[10::7, :]
+    blocks[:, :, 2:4] = dmin.astype("<f2")[..., None].view(np.uint8)
+    a = acts(m, k, 53)
+    out = run(Q.GGUF_Q4_K, w, a, n, k, cuda, torch.float32).cpu().numpy()
+    assert np.isfinite(out).all()
+    want = oracle.qmatmul_nk(Q.GGUF_Q4_K, w, a.astype(np.float32), m, n, k)
+    exact = exact_weight_product(oracle, Q.GGUF_Q4_K, w, a, n, k)
+    for col in range(n):                                                  # (each weight row against its own output size)
+        assert_close(out[:, col], want[:, col], f"GGUF_Q4_K special super-block scales, weight row {col}")
+        assert_close(out[:, col], exact[:, col], f"same (float64 sums), weight row {col}", tol=2e-5, plain_tol=2e-4)
+    A = torch.from_numpy(a).to(cuda)
+    from rocmforge_amd import ops
+    wd = torch.from_numpy(w).to(cuda)
+    assert torch.equal(ops.gemm_f16_arranged(Q.GGUF_Q4_K, wd, ops.ArrangedA(A), n, out_dtype=torch.float32).cpu(), torch.from_numpy(out))
+
+
 def test_weights_at_a_4_byte_offset_and_kept_temporary(oracle, cuda):
     """The weight loads need 4-byte alignment only; the per-stream temporary is
     reused by a smaller call after a larger one (and grown by a larger one)."""
