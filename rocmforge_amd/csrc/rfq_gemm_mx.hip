@@ -742,12 +742,14 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
 
     // Epilogue of one tile.  Accumulator register r of tile (i, j) is row
     // 8*(r/4) + 4*(lane/32) + r%4, column lane%32 of the tile: a lane owns
-    // single elements scattered over rows.  RB rows of a 32-row band at a time
-    // go through this wavefront's LDS staging area (behind the ring) and leave
-    // as whole rows: 16-byte stores for blocks inside the matrix with aligned
-    // rows, a bounds-checked element loop otherwise.  LDS operations of one
-    // wavefront execute in order, so no barrier is needed around its private
-    // staging area.
+    // single elements scattered over rows.  A tile inside the matrix leaves straight
+    // from the registers (32 lanes = one aligned 64- or 128-byte piece of a row per
+    // store; staged through LDS into 16-byte row stores the same tile took 2 % longer
+    // per launch: the round trip is a chain of waits).  A tile that crosses the
+    // matrix edge goes, RB rows of a 32-row band at a time, through this wavefront's
+    // LDS staging area (behind the ring) into a bounds-checked element loop.  LDS
+    // operations of one wavefront execute in order, so no barrier is needed around
+    // its private staging area.
     constexpr int ES = OUT_BF16 ? 2 : 4;
     constexpr int RB = C::template staging_rows<OUT_BF16>();
     constexpr int ROW_STRIDE = C::template staging_row_stride<OUT_BF16>(); // +4 dwords: the two half-waves (rows R, R+4) miss each other's banks
@@ -765,15 +767,39 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
         lds_w8_ptr stage3 = (lds_w8_ptr)lds + C::RING_BYTES + wave * RB * ROW_STRIDE;
         // this lane's accumulator elements: rows 4*(lane/32) + {0..3, 8..11, 16..19, 24..27}, column lane%32 of a tile
         lds_w8_ptr wr = stage3 + 4 * (lane >> 5) * ROW_STRIDE + (lane & 31) * ES;
-        // whole rows leave in 16-byte stores: a pass moves `rpi` rows, lane l
-        // the chunk l % cpr of row l / cpr (rpi: the largest power of two with
-        // rpi * cpr <= 64)
-        constexpr int cpr = TJ * 32 * ES / 16;           // 16-byte chunks per row
-        constexpr int rpi = cpr <= 2 ? 32 : cpr <= 4 ? 16 : cpr <= 8 ? 8 : cpr <= 16 ? 4 : cpr <= 32 ? 2 : 1;
-        static_assert(cpr <= 64 && rpi <= RB, "row store mapping");
-        const int row_l = lane / cpr, col16 = lane - row_l * cpr;
-        lds_w8_ptr rd = stage3 + row_l * ROW_STRIDE + col16 * 16;
-        const size_t pass_bytes = (size_t)rpi * N * ES;
+        if (interior) {
+            // Straight from the accumulators: a register's lanes 0..31 are 32 consecutive columns of one row (64 bytes
+            // of bf16, 128 of f32) and lanes 32..63 the row four below, so a store instruction writes two whole
+            // aligned segments; the row is a scalar base, the lane a 32-bit offset, the tile column an immediate.
+            uint8_t *tile_out = reinterpret_cast<uint8_t *>(outp) + ((size_t)m_base * N + n_base) * ES;
+            const uint32_t voff = (uint32_t)(((lane >> 5) * 4 * (size_t)N + (lane & 31)) * ES);
+            const size_t row_bytes = (size_t)N * ES;
+            // (the bases are rebuilt from scalar integers: naming the global address space keeps these global stores)
+            typedef __attribute__((address_space(1))) uint16_t *GlobalU16;
+            typedef __attribute__((address_space(1))) float *GlobalF32;
+#pragma unroll
+            for (int i = 0; i < TI; i++)
+#pragma unroll
+                for (int r = 0; r < 16; r += 2) {
+                    uint8_t *row0 = const_cast<uint8_t *>(uniform_ptr(tile_out + (size_t)(32 * i + 8 * (r >> 2) + (r & 3)) * row_bytes));
+                    uint8_t *row1 = const_cast<uint8_t *>(uniform_ptr(row0 + row_bytes));
+#pragma unroll
+                    for (int j = 0; j < TJ; j++) {
+                        if (OUT_BF16) {
+                            f32x2_t v = {acc[i][j][r], acc[i][j][r + 1]};
+                            bf16x2_t b = __builtin_convertvector(v, bf16x2_t);
+                            uint32_t u;
+                            __builtin_memcpy(&u, &b, 4);
+                            __builtin_nontemporal_store((uint16_t)u, reinterpret_cast<GlobalU16>(reinterpret_cast<uintptr_t>(row0 + voff + 32 * j * ES)));
+                            __builtin_nontemporal_store((uint16_t)(u >> 16), reinterpret_cast<GlobalU16>(reinterpret_cast<uintptr_t>(row1 + voff + 32 * j * ES)));
+                        } else {
+                            __builtin_nontemporal_store(acc[i][j][r], reinterpret_cast<GlobalF32>(reinterpret_cast<uintptr_t>(row0 + voff + 32 * j * ES)));
+                            __builtin_nontemporal_store(acc[i][j][r + 1], reinterpret_cast<GlobalF32>(reinterpret_cast<uintptr_t>(row1 + voff + 32 * j * ES)));
+                        }
+                    }
+                }
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < TI; i++)
 #pragma unroll
@@ -798,16 +824,7 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
                         }
                     }
                 const int m0 = m_base + 32 * i + h * RB;
-                if (interior) {
-                    uint8_t *o = reinterpret_cast<uint8_t *>(outp) + ((size_t)(m0 + row_l) * N + n_base) * ES + col16 * 16;
-                    if (lane < rpi * cpr) {
-#pragma unroll
-                        for (int it = 0; it < RB / rpi; it++) {
-                            v4i v = *reinterpret_cast<const __attribute__((address_space(3))) v4i *>(rd + it * rpi * ROW_STRIDE);
-                            __builtin_nontemporal_store(v, reinterpret_cast<v4i *>(o + it * pass_bytes)); // written once, never read here
-                        }
-                    }
-                } else {
+                {
                     const uint8_t *stagebuf = lds + C::RING_BYTES + (size_t)wave * RB * ROW_STRIDE;
                     const int ncols = TJ * 32;
 #pragma nounroll
