@@ -220,7 +220,8 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
         // group: both lanes of the row then read the first (zeroed when decoded)
         const int sc = (st < nstages ? st : nstages - 1) / PLANES;
         const int whc = Fmt<FMT>::BE == 32 && sc * 2 + 1 >= groups ? 0 : wh;
-        raw_of(slotc).load(w_tile, w_off, sc, whc);
+        if constexpr (INT) raw_of(slotc).template load_slot<decltype(slotc)::value>(w_tile, w_off, sc);   // (one plane: slot = stage % 4)
+        else raw_of(slotc).load(w_tile, w_off, sc, whc);
     };
     auto fetch_a = [&](auto slotc, int st, int i, int c) __attribute__((always_inline)) {
         const int sc = (st < nstages ? st : nstages - 1) / PLANES;
@@ -232,6 +233,7 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
 #pragma unroll
             for (int c = 0; c < 4; c++) fetch_a(slotc, st, i, c);
     };
+    uint32_t int_s2[2] = {0, 0}, int_o2[2] = {0, 0};              // INT: the scales of the super-block being settled, as fp16 operands
     // groups past the end of the row become zero weights (here, not at the
     // load: a select right behind the load would wait for it)
     auto settle = [&](auto slotc, int st, uint32_t pair) __attribute__((always_inline)) {
@@ -239,7 +241,9 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
         Raw32<FMT> z;
         z.zero();
         // (group 2*stage + wh has the parity of wh; with one plane the ring slot is the stage's number within its super-block)
-        raw.settle(wh, pair, PLANES == 1 ? decltype(slotc)::value : (st / PLANES) & 3);
+        // (INT: the super-block's scales come from its header hand-over, which precedes the settling of its four stages)
+        if constexpr (INT) raw.settle_packed(wh, int_s2, int_o2, decltype(slotc)::value);
+        else raw.settle(wh, pair, PLANES == 1 ? decltype(slotc)::value : (st / PLANES) & 3);
 #pragma unroll
         // (the integer-operand decoder: sc = 0 makes every weight zero; its mask and offset dwords stay what every stage has)
         for (int i = 0; i < (INT ? 2 : Raw32<FMT>::ND); i++) raw.d[i] = (st / PLANES) * 2 + wh < groups ? raw.d[i] : z.d[i];
@@ -355,7 +359,7 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
         if constexpr (INT) {
             float ratio;
             v8h m_hi, m_lo;
-            raw.header(wh, d_unit, ratio, m_hi, m_lo);
+            raw.header(wh, d_unit, ratio, int_s2, int_o2, m_hi, m_lo);
             uint8_t *area = int_base + parity * INT_AREA;
             *reinterpret_cast<v8h *>(area + wr * MNR + wh * 16) = m_hi;
             *reinterpret_cast<v8h *>(area + BN * MNR + wr * MNR + wh * 16) = m_lo;

@@ -362,13 +362,16 @@ template <> struct Raw32<RFQ_GGUF_Q4_K> {
 template <> struct Raw32<KQ_GGUF_Q4_K_INT> {
     static constexpr int ND = 12;
     uint32_t d[ND];
-    __device__ __forceinline__ void load(Rsrc w, uint32_t row_off, int st, int)
+    // Stage number C within its super-block (the ring slot): only a super-block's first stage fetches the header.
+    template <int C> __device__ __forceinline__ void load_slot(Rsrc w, uint32_t row_off, int st)
     {
         const int blk = (st >> 2) * 144;
-        v4u h = __builtin_amdgcn_raw_buffer_load_b128(w, row_off, blk, 0);
+        if constexpr (C == 0) {
+            v4u h = __builtin_amdgcn_raw_buffer_load_b128(w, row_off, blk, 0);
+            d[0] = h[0]; d[1] = h[1]; d[2] = h[2]; d[3] = h[3];
+        }
         v4u q0 = __builtin_amdgcn_raw_buffer_load_b128(w, row_off + 16, blk + 32 * (st & 3), 0);
         v4u q1 = __builtin_amdgcn_raw_buffer_load_b128(w, row_off + 32, blk + 32 * (st & 3), 0);
-        d[0] = h[0]; d[1] = h[1]; d[2] = h[2]; d[3] = h[3];
         d[4] = q0[0]; d[5] = q0[1]; d[6] = q0[2]; d[7] = q0[3];
         d[8] = q1[0]; d[9] = q1[1]; d[10] = q1[2]; d[11] = q1[3];
     }
@@ -390,11 +393,29 @@ template <> struct Raw32<KQ_GGUF_Q4_K_INT> {
     // unit, or the old one when dmin is 0 too.  For the thread's four sub-blocks 4*wh .. 4*wh+3,
     // v = -(dmin * m) / unit (dmin * m is exact in f32: 11 x 6 bits) as the fp16 pairs (hi, hi) and (lo, 0) with
     // hi + lo = v: contracted with the activations' group sums (S_hi, S_lo) they give hi * S_hi + hi * S_lo + lo * S_hi.
-    __device__ __forceinline__ void header(int wh, float &unit, float &ratio, v8h &m_hi, v8h &m_lo) const
+    // s2 / o2: for the thread's sub-block 2c + wh of each stage c = 0..3 of the super-block, s = sc * 2^-j (0 where d
+    // is 0: no q term) and -(offset * s) as fp16, two per dword: what settle_packed() spreads into a stage's registers.
+    __device__ __forceinline__ void header(int wh, float &unit, float &ratio, uint32_t (&s2)[2], uint32_t (&o2)[2], v8h &m_hi, v8h &m_lo) const
     {
         const float dv = f16_bits_to_f32((uint16_t)(d[0] & 0xFFFFu));
         const float dmin = f16_bits_to_f32((uint16_t)(d[0] >> 16));
-        const float scaled = dv * __uint_as_float((uint32_t)(127 + unit_shift(dv, dmin)) << 23);
+        const int j = unit_shift(dv, dmin);
+        const float scaled = dv * __uint_as_float((uint32_t)(127 + j) << 23);
+        const float down = dv != 0.0f ? __uint_as_float((uint32_t)(127 - j) << 23) : 0.0f;
+#pragma unroll
+        for (int p = 0; p < 2; p++) {
+            v2h sv, ov;
+#pragma unroll
+            for (int e = 0; e < 2; e++) {
+                const int c = 2 * p + e;
+                const uint32_t s0 = gguf_scale_min_k4(2 * c, d[1], d[2], d[3]) & 255u, s1 = gguf_scale_min_k4(2 * c + 1, d[1], d[2], d[3]) & 255u;
+                const float sc = (float)(wh ? s1 : s0) * down;
+                sv[e] = (_Float16)sc;                                             // exact (sc < 64, j <= 24)
+                ov[e] = (_Float16)(-(wh ? 64.0f : 1024.0f) * sc);                 // exact
+            }
+            __builtin_memcpy(&s2[p], &sv, 4);
+            __builtin_memcpy(&o2[p], &ov, 4);
+        }
         const float next = dv != 0.0f ? scaled : (dmin != 0.0f ? __builtin_fabsf(dmin) : unit);
         const float inv = 1.0f / next;
         ratio = next == unit ? 1.0f : unit * inv;
@@ -411,24 +432,19 @@ template <> struct Raw32<KQ_GGUF_Q4_K_INT> {
             m_lo[2 * q + 1] = (_Float16)0.0f;
         }
     }
-    // d[0] = (s, s) as fp16 with s = sc * 2^-j, d[1] = -(offset * s) twice, d[2] = the nibble mask of this half, d[3] =
-    // the fp16 bits the nibbles are or-ed into: low nibbles read 1024 + q (0x6400 | q), high nibbles 64 + q (0x5400 | q << 4).
-    // c = the stage's number within its super-block (a compile-time constant at the call), wh = the thread's nibble half.
-    __device__ __forceinline__ void settle(int wh, uint32_t, int c)
+    // d[0] = (s, s) as fp16, d[1] = -(offset * s) twice (both from header(), by the stage's number c within its
+    // super-block, a compile-time constant at the call), d[2] = the nibble mask of the thread's half wh, d[3] = the fp16
+    // bits the nibbles are or-ed into: low nibbles read 1024 + q (0x6400 | q), high nibbles 64 + q (0x5400 | q << 4).
+    __device__ __forceinline__ void settle_packed(int wh, const uint32_t (&s2)[2], const uint32_t (&o2)[2], int c)
     {
-        const uint32_t s0 = gguf_scale_min_k4(2 * c, d[1], d[2], d[3]) & 255u, s1 = gguf_scale_min_k4(2 * c + 1, d[1], d[2], d[3]) & 255u;
-        const float dv = f16_bits_to_f32((uint16_t)(d[0] & 0xFFFFu)), dmin = f16_bits_to_f32((uint16_t)(d[0] >> 16));
-        const float down = __uint_as_float((uint32_t)(127 - unit_shift(dv, dmin)) << 23);
-        const float sc = dv != 0.0f ? (float)(wh ? s1 : s0) * down : 0.0f;   // d = 0: no q term
-        const _Float16 h = (_Float16)sc, o = (_Float16)(-(wh ? 64.0f : 1024.0f) * sc);   // both exact (sc < 64, j <= 24)
-        uint16_t hb, ob;
-        __builtin_memcpy(&hb, &h, 2);
-        __builtin_memcpy(&ob, &o, 2);
-        d[0] = hb * 0x10001u;
-        d[1] = ob * 0x10001u;
+        const uint32_t sel = (c & 1) ? 0x03020302u : 0x01000100u;
+        d[0] = __builtin_amdgcn_perm(s2[c >> 1], s2[c >> 1], sel);
+        d[1] = __builtin_amdgcn_perm(o2[c >> 1], o2[c >> 1], sel);
         d[2] = wh ? 0x00F000F0u : 0x000F000Fu;
         d[3] = wh ? 0x54005400u : 0x64006400u;
     }
+    __device__ __forceinline__ void settle(int, uint32_t, int) {}
+    __device__ __forceinline__ void load(Rsrc, uint32_t, int, int) {}
     // Chunk c = elements 8c .. 8c+7 of the sub-block = bytes 8c .. 8c+7 of the stage's 32: dwords x0 (k0..k3) and x1
     // (k4..k7).  Their low halves side by side are the bytes (k0 k1 k4 k5): one and-or gives the pair (k0, k4), the same
     // on the dword shifted by 8 (k1, k5); the high halves (k2, k6) and (k3, k7) - the order the activations are in.
