@@ -355,15 +355,20 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
     // before it is multiplied), into one of two areas by the super-block's parity: the two min fragments, the
     // ratio that takes acc into its unit, and the unit itself (the epilogue multiplies by the last one).  A
     // super-block with d = 0 has zero weights (settle() clears its sc) and keeps the previous unit.
+    struct NoHeader {};
+    typename std::conditional<INT, typename Raw32<KQ_GGUF_Q4_K_INT>::Header, NoHeader>::type hdr;
+    auto write_header = [&](int parity) __attribute__((always_inline)) {
+        if constexpr (INT) {
+            uint8_t *area = int_base + parity * INT_AREA;
+            *reinterpret_cast<v8h *>(area + wr * MNR + wh * 16) = hdr.m_hi;
+            *reinterpret_cast<v8h *>(area + BN * MNR + wr * MNR + wh * 16) = hdr.m_lo;
+            *reinterpret_cast<float *>(area + 2 * BN * MNR + wh * BN * 4 + wr * 4) = wh ? d_unit : hdr.ratio;
+        }
+    };
     auto stash_header = [&](const Raw32<FMT> &raw, int parity) __attribute__((always_inline)) {
         if constexpr (INT) {
-            float ratio;
-            v8h m_hi, m_lo;
-            raw.header(wh, d_unit, ratio, int_s2, int_o2, m_hi, m_lo);
-            uint8_t *area = int_base + parity * INT_AREA;
-            *reinterpret_cast<v8h *>(area + wr * MNR + wh * 16) = m_hi;
-            *reinterpret_cast<v8h *>(area + BN * MNR + wr * MNR + wh * 16) = m_lo;
-            *reinterpret_cast<float *>(area + 2 * BN * MNR + wh * BN * 4 + wr * 4) = wh ? d_unit : ratio;
+            raw.header(wh, d_unit, int_s2, int_o2, hdr);
+            write_header(parity);
         }
     };
     // acc *= f[n] (register r of a tile: n = 8*(r/4) + 4*fh + r%4: four factors side by side); which = 0: the ratio
@@ -493,7 +498,19 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
                     if (S == 0 && p < 4)
                         fm_lo[p] = *reinterpret_cast<const v8h *>(int_base + ((st >> 2) & 1) * INT_AREA + BN * MNR + fr * MNR + fh * 16 + p * 32 * MNR);
                     // stage st+3 opens the next super-block: its header goes to the other area before settle() reuses the dwords
-                    if (S == 1 && p == 14) stash_header(raw_of(IC<S3>{}), ((st + 3) >> 2) & 1);
+                    // (in eight pieces between the stage's other work; no stage is being settled meanwhile)
+                    if (S == 1) {
+                        constexpr int AT[8] = {1, 2, 4, 6, 7, 9, 11, 14};
+                        const Raw32<FMT> &next_hdr = raw_of(IC<S3>{});
+                        if (p == AT[0]) next_hdr.template header_phase<0>(wh, d_unit, int_s2, int_o2, hdr);
+                        if (p == AT[1]) next_hdr.template header_phase<1>(wh, d_unit, int_s2, int_o2, hdr);
+                        if (p == AT[2]) next_hdr.template header_phase<2>(wh, d_unit, int_s2, int_o2, hdr);
+                        if (p == AT[3]) next_hdr.template header_phase<3>(wh, d_unit, int_s2, int_o2, hdr);
+                        if (p == AT[4]) next_hdr.template header_phase<4>(wh, d_unit, int_s2, int_o2, hdr);
+                        if (p == AT[5]) next_hdr.template header_phase<5>(wh, d_unit, int_s2, int_o2, hdr);
+                        if (p == AT[6]) next_hdr.template header_phase<6>(wh, d_unit, int_s2, int_o2, hdr);
+                        if (p == AT[7]) write_header(((st + 3) >> 2) & 1);
+                    }
                 }
                 if (p == 15 && SH3 == S3) settle(IC<S3>{}, st + 3, S == 0 ? hsA[3] : hsB[S3]);   // stage st+3 is number S3 of its super-block
                 if (p >= 17 && p <= 23 && (p & 1)) {

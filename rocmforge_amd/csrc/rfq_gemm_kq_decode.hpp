@@ -395,42 +395,59 @@ template <> struct Raw32<KQ_GGUF_Q4_K_INT> {
     // hi + lo = v: contracted with the activations' group sums (S_hi, S_lo) they give hi * S_hi + hi * S_lo + lo * S_hi.
     // s2 / o2: for the thread's sub-block 2c + wh of each stage c = 0..3 of the super-block, s = sc * 2^-j (0 where d
     // is 0: no q term) and -(offset * s) as fp16, two per dword: what settle_packed() spreads into a stage's registers.
-    __device__ __forceinline__ void header(int wh, float &unit, float &ratio, uint32_t (&s2)[2], uint32_t (&o2)[2], v8h &m_hi, v8h &m_lo) const
+    // The work is cut into eight phases so that the kernel can lay them between matrix instructions: 0 = units and
+    // ratio, 1-2 = the scales, 3-6 = the mins, (7 = the kernel's LDS writes).  header() runs them all.
+    struct Header {
+        float ratio, dmin, inv, down;
+        v8h m_hi, m_lo;
+    };
+    template <int PH>
+    __device__ __forceinline__ void header_phase(int wh, float &unit, uint32_t (&s2)[2], uint32_t (&o2)[2], Header &h) const
     {
-        const float dv = f16_bits_to_f32((uint16_t)(d[0] & 0xFFFFu));
-        const float dmin = f16_bits_to_f32((uint16_t)(d[0] >> 16));
-        const int j = unit_shift(dv, dmin);
-        const float scaled = dv * __uint_as_float((uint32_t)(127 + j) << 23);
-        const float down = dv != 0.0f ? __uint_as_float((uint32_t)(127 - j) << 23) : 0.0f;
-#pragma unroll
-        for (int p = 0; p < 2; p++) {
+        if constexpr (PH == 0) {
+            const float dv = f16_bits_to_f32((uint16_t)(d[0] & 0xFFFFu));
+            h.dmin = f16_bits_to_f32((uint16_t)(d[0] >> 16));
+            const int j = unit_shift(dv, h.dmin);
+            const float scaled = dv * __uint_as_float((uint32_t)(127 + j) << 23);
+            h.down = dv != 0.0f ? __uint_as_float((uint32_t)(127 - j) << 23) : 0.0f;
+            const float next = dv != 0.0f ? scaled : (h.dmin != 0.0f ? __builtin_fabsf(h.dmin) : unit);
+            h.inv = 1.0f / next;
+            h.ratio = next == unit ? 1.0f : unit * h.inv;
+            unit = next;
+        } else if constexpr (PH <= 2) {
+            constexpr int p = PH - 1;
             v2h sv, ov;
 #pragma unroll
             for (int e = 0; e < 2; e++) {
                 const int c = 2 * p + e;
                 const uint32_t s0 = gguf_scale_min_k4(2 * c, d[1], d[2], d[3]) & 255u, s1 = gguf_scale_min_k4(2 * c + 1, d[1], d[2], d[3]) & 255u;
-                const float sc = (float)(wh ? s1 : s0) * down;
+                const float sc = (float)(wh ? s1 : s0) * h.down;
                 sv[e] = (_Float16)sc;                                             // exact (sc < 64, j <= 24)
                 ov[e] = (_Float16)(-(wh ? 64.0f : 1024.0f) * sc);                 // exact
             }
             __builtin_memcpy(&s2[p], &sv, 4);
             __builtin_memcpy(&o2[p], &ov, 4);
-        }
-        const float next = dv != 0.0f ? scaled : (dmin != 0.0f ? __builtin_fabsf(dmin) : unit);
-        const float inv = 1.0f / next;
-        ratio = next == unit ? 1.0f : unit * inv;
-        unit = next;
-#pragma unroll
-        for (int q = 0; q < 4; q++) {
+        } else if constexpr (PH <= 6) {
+            constexpr int q = PH - 3;
             // (both halves unpacked with compile-time sub-block numbers, the thread's half chosen after)
             const uint32_t m0 = gguf_scale_min_k4(q, d[1], d[2], d[3]) >> 8, m1 = gguf_scale_min_k4(4 + q, d[1], d[2], d[3]) >> 8;
-            const float v = -(dmin * (float)(wh ? m1 : m0)) * inv;
+            const float v = -(h.dmin * (float)(wh ? m1 : m0)) * h.inv;
             const _Float16 hi = (_Float16)v, lo = (_Float16)(v - (float)hi);
-            m_hi[2 * q] = hi;
-            m_hi[2 * q + 1] = hi;
-            m_lo[2 * q] = lo;
-            m_lo[2 * q + 1] = (_Float16)0.0f;
+            h.m_hi[2 * q] = hi;
+            h.m_hi[2 * q + 1] = hi;
+            h.m_lo[2 * q] = lo;
+            h.m_lo[2 * q + 1] = (_Float16)0.0f;
         }
+    }
+    __device__ __forceinline__ void header(int wh, float &unit, uint32_t (&s2)[2], uint32_t (&o2)[2], Header &h) const
+    {
+        header_phase<0>(wh, unit, s2, o2, h);
+        header_phase<1>(wh, unit, s2, o2, h);
+        header_phase<2>(wh, unit, s2, o2, h);
+        header_phase<3>(wh, unit, s2, o2, h);
+        header_phase<4>(wh, unit, s2, o2, h);
+        header_phase<5>(wh, unit, s2, o2, h);
+        header_phase<6>(wh, unit, s2, o2, h);
     }
     // d[0] = (s, s) as fp16, d[1] = -(offset * s) twice (both from header(), by the stage's number c within its
     // super-block, a compile-time constant at the call), d[2] = the nibble mask of the thread's half wh, d[3] = the fp16
