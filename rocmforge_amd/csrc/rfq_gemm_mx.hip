@@ -744,8 +744,10 @@ gemm_mx_kernel(const uint8_t *__restrict__ ap, const uint8_t *__restrict__ bp, v
     // 8*(r/4) + 4*(lane/32) + r%4, column lane%32 of the tile: a lane owns
     // single elements scattered over rows.  A tile inside the matrix leaves straight
     // from the registers (32 lanes = one aligned 64- or 128-byte piece of a row per
-    // store; staged through LDS into 16-byte row stores the same tile took 2 % longer
-    // per launch: the round trip is a chain of waits).  A tile that crosses the
+    // store).  Staged through LDS into 16-byte row stores the launch measured the
+    // same once the part's clock had settled (171.6 against 171.2 us at 2048 x 8192
+    // x 28672) and 1-2 % longer over its first 240 launches: the stores are not what
+    // the epilogue waits for, and this form needs no LDS.  A tile that crosses the
     // matrix edge goes, RB rows of a 32-row band at a time, through this wavefront's
     // LDS staging area (behind the ring) into a bounds-checked element loop.  LDS
     // operations of one wavefront execute in order, so no barrier is needed around
