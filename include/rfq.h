@@ -32,7 +32,7 @@ extern "C" {
 
 /* Raised whenever an exported signature or the meaning of a format changes: a caller compares
  * rfq_version() with the RFQ_VERSION it was built against before its first call. */
-#define RFQ_VERSION 103 /* 0.1.3 */
+#define RFQ_VERSION 104 /* 0.1.4 */
 
 #if defined(_WIN32)
 #define RFQ_API
@@ -327,7 +327,13 @@ RFQ_API int rfq_mlp_swiglu(int fmt_gate_up, const void *d_gate_w, const void *d_
  * temporary device memory (the activations in matrix-operand order) is kept
  * per stream between calls; larger temporaries are allocated and released in
  * stream order.  (A stream's first call, or a larger shape than before,
- * allocates: run the call once on the stream before capturing it into a graph.)  The reference has no fused prefill GEMM (its matmul_q* hard-wire
+ * allocates: run the call once on the stream before capturing it into a graph.)
+ * A shape with few output tiles and a long k (an attention or down projection
+ * of 512 tokens: 64 tiles of 256 x 128 for 256 CUs) is split along k into
+ * rfq_gemm_f16_k_parts(m, n, k) parts of whole super-blocks, whose f32 tiles
+ * (parts * m * n * 4 more bytes of temporary) a second kernel adds in a fixed
+ * order: the results are deterministic and differ from a single pass only in
+ * the order of the fp32 sums.  The reference has no fused prefill GEMM (its matmul_q* hard-wire
  * m = 1, src/kernels/matmul/quantized/q4_0.rs:169; larger m goes through
  * dequantise + hipBLAS SGEMM, src/tensor/matmul.rs:134-214); this is the same
  * contraction. */
@@ -357,12 +363,16 @@ RFQ_API int rfq_gemm_f16_static(int fmt, const void *d_w, size_t w_bytes, const 
  * RFQ_Q4_K kernel wants, into a caller's buffer of
  * rfq_gemm_f16_arranged_bytes(m, k) bytes (16-byte aligned; 0 = bad shape);
  * rfq_gemm_f16_arranged multiplies any of the formats of rfq_gemm_f16 with it.
- * Results are bit-identical to rfq_gemm_f16 on the same A.  Neither call
+ * Results are bit-identical to rfq_gemm_f16 on the same A where that call takes
+ * one pass over k (rfq_gemm_f16_k_parts(m, n, k) == 1; this entry point never
+ * splits: it has no temporary for the parts).  Neither call
  * allocates or keeps anything, so both may be recorded under stream capture.
  * The reference has no fused prefill GEMM (see rfq_gemm_f16); its
  * counterpart is the shared input of the three SGEMMs of
  * HipBackend::mlp_swiglu (src/backend/hip_backend/backend.rs:1153-1278). */
 RFQ_API size_t rfq_gemm_f16_arranged_bytes(int m, int k);
+/* How many parts along k rfq_gemm_f16 takes for this shape (1 = a single pass). */
+RFQ_API int rfq_gemm_f16_k_parts(int m, int n, int k);
 RFQ_API int rfq_gemm_f16_arrange(const void *d_a_f16, int m, int k, void *d_arranged, size_t arranged_bytes,
                                  void *stream);
 RFQ_API int rfq_gemm_f16_arranged(int fmt, const void *d_w, size_t w_bytes, const void *d_arranged,

@@ -60,6 +60,7 @@ _SIGNATURES = {
     "rfq_mx_prepare": ([_i, _i, _vp, _sz, _i, _i, _vp, _sz, C.POINTER(C.c_int), _vp], _i),
     "rfq_release_stream_temporaries": ([_vp], _i),
     "rfq_gemm_f16_arranged_bytes": ([_i, _i], _sz),
+    "rfq_gemm_f16_k_parts": ([_i, _i, _i], _i),
     "rfq_gemm_f16_arrange": ([_vp, _i, _i, _vp, _sz, _vp], _i),
     "rfq_gemm_f16_arranged": ([_i, _vp, _sz, _vp, _sz, _vp, _i, _i, _i, _i, _vp], _i),
     "rfq_gemm_mx": ([_vp, _sz, _i, _vp, _sz, _i, _vp, _i, _i, _i, _i, _vp], _i),

@@ -431,6 +431,7 @@ int rfq_gemm_f16_static(int fmt, const void *d_w, size_t w_bytes, const void *d_
 }
 
 size_t rfq_gemm_f16_arranged_bytes(int m, int k) { return gemm_f16_arranged_bytes(m, k); }
+int rfq_gemm_f16_k_parts(int m, int n, int k) { return m > 0 && n > 0 && k > 0 ? gemm_f16_k_parts(m, n, k) : 1; }
 
 int rfq_gemm_f16_arrange(const void *d_a_f16, int m, int k, void *d_arranged, size_t arranged_bytes, void *stream)
 {

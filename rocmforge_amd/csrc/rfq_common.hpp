@@ -120,6 +120,7 @@ int launch_gemv_fused(int fmt, const uint8_t *d_w, const uint8_t *d_w2, const fl
                       float eps, float *d_y, int n, int k, hipStream_t s);
 // use_static_scratch: the temporaries live in the library's static device array instead of workspace().
 size_t gemm_f16_arranged_bytes(int m, int k);
+int gemm_f16_k_parts(int m, int n, int k);
 int launch_arrange_a(const void *d_a, int m, int k, uint8_t *d_arranged, hipStream_t s);
 // d_arranged != nullptr: activations already in operand order (launch_arrange_a); d_a is not read.
 int launch_gemm_f16(int fmt, const uint8_t *d_w, const void *d_a, void *d_out, int out_dtype, int m, int n,

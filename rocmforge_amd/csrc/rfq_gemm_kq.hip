@@ -131,7 +131,8 @@ arrange_a_kernel(const _Float16 *__restrict__ a, v4u *__restrict__ at, _Float16 
 #pragma unroll
             for (int e = 0; e < 8; e++) sum += (float)h[e];
         }
-        const _Float16 hi = (_Float16)sum, lo = (_Float16)(sum - (float)hi);
+        _Float16 hi, lo;
+        fp16_pair(sum, hi, lo);
         const int g = k0 / 32, sb = g & 7;
         const size_t t = ((((size_t)mt * (K / 256) + (g >> 3)) * 2 + (sb >> 2)) * 32 + fr) * 4 + (sb & 3);
         s2[2 * t] = hi;
@@ -146,8 +147,12 @@ arrange_a_kernel(const _Float16 *__restrict__ a, v4u *__restrict__ at, _Float16 
 template <int FMT, bool OUT_F16, int PLANES>
 __global__ void __launch_bounds__(256)
 gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const _Float16 *__restrict__ s2,
-               void *__restrict__ outp, int M, int N, int K)
+               void *__restrict__ outp, int M, int N, int Kfull, int kparts)
 {
+    // kparts > 1 (few output tiles, long k): the launch holds kparts workgroups per tile, each contracts a whole number
+    // of super-blocks [k0, k0 + K) of the rows and writes its f32 partial tile to outp[part][M][N]; reduce_parts_kernel
+    // adds the parts in order.
+    const int K = Kfull / kparts;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     // INT: integer operands sc * q; acc runs in units of the current super-block's d (f32), rescaled between super-blocks
     constexpr bool INT = FMT == KQ_GGUF_Q4_K_INT;
@@ -159,19 +164,23 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
     // Workgroups are dealt round-robin to the 8 XCDs (blockIdx.x % 8), each with an L2 of its own: hand every XCD a
     // contiguous run of tiles, so that the m tiles of one W tile meet in one L2 and W comes from HBM once.
     const int nwg = gridDim.x;
-    const int tile = nwg % 8 == 0 ? (int)(blockIdx.x % 8) * (nwg / 8) + (int)(blockIdx.x / 8) : (int)blockIdx.x;
+    const int slot = nwg % 8 == 0 ? (int)(blockIdx.x % 8) * (nwg / 8) + (int)(blockIdx.x / 8) : (int)blockIdx.x;
+    const int tiles_all = nwg / kparts, part = slot / tiles_all, tile = slot % tiles_all;
+    const int k0 = part * K;
     const int tm = tile % tiles_m, tn = tile / tiles_m;             // the m tiles of one W tile are neighbours
     const int m0 = tm * BM, n0 = tn * BN;
     const int groups = K / 32;                                    // 32-element groups per row
-    const size_t row_bytes = (size_t)(K / Fmt<FMT>::BE) * Fmt<FMT>::BB;
+    const size_t row_bytes = (size_t)(Kfull / Fmt<FMT>::BE) * Fmt<FMT>::BB;
+    const size_t k0_bytes = (size_t)(k0 / Fmt<FMT>::BE) * Fmt<FMT>::BB;     // (kparts > 1: k0 is whole super-blocks)
+    const int kstages_full = (Kfull + BK - 1) / BK;
     const int kstages = (K + BK - 1) / BK;                        // stages of k
     const int nstages = kstages * PLANES;                         // stages the pipeline walks
 
     // Weights: thread t decodes group t%2 of row t/2 of each stage into LDS.
     const int wr = tid >> 1, wh = tid & 1;
     // (a buffer descriptor from the tile's first row to the end of W, plus a 32-bit lane offset)
-    const size_t w_left = (size_t)(N - n0) * row_bytes;
-    const Rsrc w_tile = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(w) + (size_t)n0 * row_bytes, 0,
+    const size_t w_left = (size_t)(N - n0) * row_bytes - k0_bytes;
+    const Rsrc w_tile = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(w) + (size_t)n0 * row_bytes + k0_bytes, 0,
                                                           w_left < 0xFFFFFFFFu ? (int)(uint32_t)w_left : -1, 0x00020000);
     const uint32_t w_off = (uint32_t)((n0 + wr < N ? wr : N - 1 - n0) * (int)row_bytes);
     // Activations never pass through LDS: they arrive arranged in the order
@@ -191,7 +200,7 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
     for (int i = 0; i < TI; i++) {
         const int mt = m0 / 32 + wave_u * 2 + i;
         a_tile[i] = __builtin_amdgcn_make_buffer_rsrc(
-            const_cast<v4u *>(at + (size_t)(mt < tiles32 ? mt : tiles32 - 1) * kstages * 256), 0, kstages * 4096, 0x00020000);
+            const_cast<v4u *>(at + ((size_t)(mt < tiles32 ? mt : tiles32 - 1) * kstages_full + k0 / BK) * 256), 0, kstages * 4096, 0x00020000);
     }
 
     // Global loads run three stages ahead of the arithmetic through a ring of
@@ -298,7 +307,7 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
         for (int i = 0; i < TI; i++) {
             const int mt = m0 / 32 + wave_u * 2 + i;
             s_tile[i] = __builtin_amdgcn_make_buffer_rsrc(
-                const_cast<uint8_t *>(reinterpret_cast<const uint8_t *>(s2)) + (size_t)(mt < tiles32 ? mt : tiles32 - 1) * (K / 256) * 1024,
+                const_cast<uint8_t *>(reinterpret_cast<const uint8_t *>(s2)) + ((size_t)(mt < tiles32 ? mt : tiles32 - 1) * (Kfull / 256) + k0 / 256) * 1024,
                 0, (K / 256) * 1024, 0x00020000);
         }
     }
@@ -617,6 +626,7 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
     // or 16-byte pieces one row apart.
     rescale(((K / 256) - 1) & 1, 1);                               // INT: from the last super-block's unit to values
     typedef typename std::conditional<OUT_F16, _Float16, float>::type OutT;
+    outp = reinterpret_cast<uint8_t *>(outp) + (size_t)part * M * N * sizeof(OutT);
     constexpr int ROWB = BN * (int)sizeof(OutT) + 16;             // bytes per staged row (row stride = 4 banks mod 32)
     static_assert(4 * 32 * ROWB <= 4 * W_BYTES, "staging area");
     if (m0 + BM <= M && n0 + BN <= N && (N * sizeof(OutT)) % 16 == 0 && (reinterpret_cast<uintptr_t>(outp) & 15u) == 0) {
@@ -685,6 +695,40 @@ gemm_kq_kernel(const uint8_t *__restrict__ w, const v4u *__restrict__ at, const 
         }
 }
 
+// out[i] = parts[0][i] + parts[1][i] + ... (in that order), i < count; four elements per thread where the count allows.
+template <bool OUT_F16>
+__global__ void __launch_bounds__(256)
+reduce_parts_kernel(const float *__restrict__ parts, void *__restrict__ out, size_t count, int kparts)
+{
+    const size_t i4 = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i4 >= count) return;
+    float v[4] = {0.f, 0.f, 0.f, 0.f};
+    const int live = count - i4 >= 4 ? 4 : (int)(count - i4);
+    for (int p = 0; p < kparts; p++) {
+        const float *src = parts + (size_t)p * count + i4;
+        if (live == 4 && (count & 3) == 0) {
+            const float4 f = *reinterpret_cast<const float4 *>(src);
+            v[0] += f.x; v[1] += f.y; v[2] += f.z; v[3] += f.w;
+        } else {
+            for (int e = 0; e < live; e++) v[e] += src[e];
+        }
+    }
+    for (int e = 0; e < live; e++) {
+        if (OUT_F16) reinterpret_cast<_Float16 *>(out)[i4 + e] = (_Float16)v[e];
+        else reinterpret_cast<float *>(out)[i4 + e] = v[e];
+    }
+}
+
+// Parts of k for a launch with few output tiles: as many as fill the part (256 CUs), whole super-blocks each.
+int k_parts_for(int m, int n, int k)
+{
+    const int tiles = ((m + BM - 1) / BM) * ((n + BN - 1) / BN);
+    if (tiles > 128 || k % 256 != 0) return 1;
+    for (int p = 256 / tiles < 8 ? 256 / tiles : 8; p >= 2; p--)
+        if (k % (p * 256) == 0 && k / p >= 1024) return p;
+    return 1;
+}
+
 // Bytes of the arranged activations of an [m, k] matrix, and of the group sums that follow them when k is whole
 // super-blocks (the Q4_K kernel reads them; the others ignore them).
 size_t arranged_at_bytes(int m, int k) { return (size_t)((m + 31) / 32) * ((k + BK - 1) / BK) * 4096; }
@@ -698,18 +742,23 @@ int launch_cfg(const uint8_t *w, const void *a, void *out, int m, int n, int k, 
     // four weight stages + the Q4_K min fragment (+ the integer-operand kernel's two header areas)
     constexpr int LDS = 4 * W_BYTES + BN * 48 + (FMT == KQ_GGUF_Q4_K_INT ? 2 * (2 * BN * 48 + 2 * BN * 4) : 0);
     static_assert(LDS <= 160 * 1024, "LDS budget");
+    // (both output types: a launch split along k writes f32 parts whatever the caller's type)
     static std::once_flag once;
     static hipError_t attr_err = hipSuccess;
     std::call_once(once, [] {
         attr_err = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_kq_kernel<FMT, OUT_F16, PLANES>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+        if (attr_err == hipSuccess && OUT_F16)
+            attr_err = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_kq_kernel<FMT, false, PLANES>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
     });
     if (attr_err != hipSuccess) return hip_fail(attr_err, "hipFuncSetAttribute(gemm_kq_kernel)");
     const int tiles = ((m + BM - 1) / BM) * ((n + BN - 1) / BN);
     if (arranged != nullptr) {
+        // (the caller's buffer holds the arranged activations only: nowhere to put parts, no split along k)
         const v4u *at = reinterpret_cast<const v4u *>(arranged);
         const _Float16 *s2 = reinterpret_cast<const _Float16 *>(arranged + arranged_at_bytes(m, k));
-        hipLaunchKernelGGL((gemm_kq_kernel<FMT, OUT_F16, PLANES>), dim3(tiles), dim3(256), LDS, s, w, at, s2, out, m, n, k);
+        hipLaunchKernelGGL((gemm_kq_kernel<FMT, OUT_F16, PLANES>), dim3(tiles), dim3(256), LDS, s, w, at, s2, out, m, n, k, 1);
         RFQ_LAUNCH_CHECK("gemm_kq_kernel");
         return RFQ_OK;
     }
@@ -718,20 +767,36 @@ int launch_cfg(const uint8_t *w, const void *a, void *out, int m, int n, int k, 
     const size_t at_bytes = (size_t)tiles32 * nst * 4096;
     constexpr bool SUMS = FMT == RFQ_Q4_K || FMT == KQ_GGUF_Q4_K_INT;
     const size_t s2_bytes = SUMS ? (size_t)tiles32 * (k / 256) * 1024 : 0;
+    // Few output tiles and a long k (an attention or down projection of 512 tokens: 64 tiles for 256 CUs): the launch is
+    // split along k, the parts' f32 tiles follow the arranged activations in the temporary, reduce_parts_kernel adds them.
+    int kparts = k_parts_for(m, n, k);
+    const size_t head_bytes = (at_bytes + s2_bytes + 255) & ~(size_t)255;
+    size_t parts_bytes = kparts > 1 ? (size_t)kparts * m * n * sizeof(float) : 0;
     uint8_t *tmp = static_tmp;
     bool transient = false;
     if (static_tmp != nullptr) {
         if (at_bytes + s2_bytes > RFQ_STATIC_SCRATCH_BYTES)
             return fail(RFQ_E_SIZE, "rfq_gemm_f16_static: m=%d k=%d needs %zu bytes of temporary memory, the static buffer holds %zu",
                         m, k, at_bytes + s2_bytes, RFQ_STATIC_SCRATCH_BYTES);
-    } else if (int rc = workspace(s, at_bytes + s2_bytes, &tmp, &transient)) {
+        if (head_bytes + parts_bytes > RFQ_STATIC_SCRATCH_BYTES) {                   // no room for parts: one pass over k
+            kparts = 1;
+            parts_bytes = 0;
+        }
+    } else if (int rc = workspace(s, head_bytes + parts_bytes, &tmp, &transient)) {
         return rc;
     }
     v4u *at = reinterpret_cast<v4u *>(tmp);
     _Float16 *s2 = reinterpret_cast<_Float16 *>(tmp + at_bytes);
     hipLaunchKernelGGL((arrange_a_kernel<SUMS>), dim3((unsigned)(tiles32 * ((nst + 3) / 4))), dim3(256), 0, s,
                        reinterpret_cast<const _Float16 *>(a), at, s2, m, k, tiles32, nst);
-    hipLaunchKernelGGL((gemm_kq_kernel<FMT, OUT_F16, PLANES>), dim3(tiles), dim3(256), LDS, s, w, at, s2, out, m, n, k);
+    if (kparts > 1) {
+        float *parts = reinterpret_cast<float *>(tmp + head_bytes);
+        const size_t count = (size_t)m * n;
+        hipLaunchKernelGGL((gemm_kq_kernel<FMT, false, PLANES>), dim3(tiles * kparts), dim3(256), LDS, s, w, at, s2, parts, m, n, k, kparts);
+        hipLaunchKernelGGL((reduce_parts_kernel<OUT_F16>), dim3((unsigned)((count + 1023) / 1024)), dim3(256), 0, s, parts, out, count, kparts);
+    } else {
+        hipLaunchKernelGGL((gemm_kq_kernel<FMT, OUT_F16, PLANES>), dim3(tiles), dim3(256), LDS, s, w, at, s2, out, m, n, k, 1);
+    }
     hipError_t launch_err = hipGetLastError();
     if (transient) {
         hipError_t free_err = hipFreeAsync(tmp, s);
@@ -898,6 +963,8 @@ int release_workspaces()
     if (first != hipSuccess) return hip_fail(first, "rfq_release_temporaries");
     return RFQ_OK;
 }
+
+int gemm_f16_k_parts(int m, int n, int k) { return k_parts_for(m, n, k); }
 
 size_t gemm_f16_arranged_bytes(int m, int k)
 {

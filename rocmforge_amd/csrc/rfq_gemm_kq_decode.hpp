@@ -44,10 +44,22 @@ __device__ __forceinline__ constexpr int chunk_pos(int e) { return ((e & 3) << 1
 
 // The fp16 operands a decoded weight v (f32) is contracted as: hi = fp16(v) (round to nearest even) and, when the
 // kernel runs two planes, lo = fp16(v - hi), so that hi + lo = v to 2^-22 of v.
+// v goes through an opaque statement first when both are wanted: the compiler otherwise folds the multiplication that
+// produced v into ONE of the two conversions it emits (v_fma_mixlo_f16 rounds the exact product, v_cvt_f16_f32 the
+// f32-rounded one), and where the f32 value is a tie of the fp16 grid the stored hi and the hi that lo was formed
+// against then differ by an fp16 ulp.
+__device__ __forceinline__ void fp16_pair(float v, _Float16 &hi, _Float16 &lo)
+{
+    asm("" : "+v"(v));
+    hi = (_Float16)v;
+    float back = (float)hi;
+    asm("" : "+v"(back));
+    lo = (_Float16)(v - back);
+}
 template <bool BOTH> __device__ __forceinline__ void fp16_parts(float v, _Float16 &hi, _Float16 &lo)
 {
-    hi = (_Float16)v;
-    if constexpr (BOTH) lo = (_Float16)(v - (float)hi);
+    if constexpr (BOTH) fp16_pair(v, hi, lo);
+    else hi = (_Float16)v;
 }
 
 // Every format decodes a 32-element group in 12 steps (chunk c = T/3 of 8
@@ -432,7 +444,8 @@ template <> struct Raw32<KQ_GGUF_Q4_K_INT> {
             // (both halves unpacked with compile-time sub-block numbers, the thread's half chosen after)
             const uint32_t m0 = gguf_scale_min_k4(q, d[1], d[2], d[3]) >> 8, m1 = gguf_scale_min_k4(4 + q, d[1], d[2], d[3]) >> 8;
             const float v = -(h.dmin * (float)(wh ? m1 : m0)) * h.inv;
-            const _Float16 hi = (_Float16)v, lo = (_Float16)(v - (float)hi);
+            _Float16 hi, lo;
+            fp16_pair(v, hi, lo);
             h.m_hi[2 * q] = hi;
             h.m_hi[2 * q + 1] = hi;
             h.m_lo[2 * q] = lo;

@@ -50,7 +50,7 @@ pub const RFQ_MX_FP4: c_int = 4;
 pub const RFQ_MX_FP8: c_int = 8;
 pub const RFQ_MX_FP4_UNCHECKED: c_int = 0x104;
 
-pub const RFQ_VERSION: c_int = 103;
+pub const RFQ_VERSION: c_int = 104;
 
 #[link(name = "rfq")]
 extern "C" {
@@ -120,6 +120,7 @@ extern "C" {
                                d_out: *mut c_void, out_dtype: c_int, m: c_int, n: c_int, k: c_int,
                                stream: *mut c_void) -> c_int;
     pub fn rfq_gemm_f16_arranged_bytes(m: c_int, k: c_int) -> usize;
+    pub fn rfq_gemm_f16_k_parts(m: c_int, n: c_int, k: c_int) -> c_int;
     pub fn rfq_gemm_f16_arrange(d_a_f16: *const c_void, m: c_int, k: c_int, d_arranged: *mut c_void,
                                 arranged_bytes: usize, stream: *mut c_void) -> c_int;
     pub fn rfq_gemm_f16_arranged(fmt: c_int, d_w: *const c_void, w_bytes: usize, d_arranged: *const c_void,

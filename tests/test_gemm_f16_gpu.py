@@ -117,6 +117,18 @@ def test_full_size_sampled(fmt, oracle, cuda):
     print(f"{Q.NAMES[fmt]} 512x14336x4096, {cols.size} sampled columns, fp32 out: {error_report(got, want)}")
     got16 = f16[:, torch.from_numpy(cols).to(cuda)].float().cpu().numpy()
     assert_close(got16, want, "sampled fp16", tol=1e-3 + 2.0 ** -11)      # one fp16 rounding on top
+    # every output against the float64 contraction of the decoded weights (a handful of weight rows gone wrong would
+    # pass between the sampled columns and under the checksum): the exact forms to fp32 level, the 256-byte Q4_K
+    # layout's single rounded operand to its 2^-12 per weight
+    w64 = (gguf_q4_k_fused(w, n, k) if fmt == Q.GGUF_Q4_K else oracle.dequantize(fmt, w, n * k).reshape(n, k)).astype(np.float64)
+    full = a.astype(np.float64) @ w64.T
+    got_all = f32.cpu().numpy()
+    rms = float(np.sqrt(np.mean(full * full)))
+    per_row = np.max(np.abs(got_all - full), axis=0) / rms                  # worst output of each weight row
+    print(f"{Q.NAMES[fmt]} all {m * n} outputs against float64: worst weight row {per_row.max():.2e} of rms(out), "
+          f"median {np.median(per_row):.2e}")
+    assert per_row.max() <= (1e-3 if fmt == Q.Q4_K else 2e-5), (Q.NAMES[fmt], int(np.argmax(per_row)), float(per_row.max()))
+    del w64, full, got_all
     wsum = oracle.dequantize(fmt, w, n * k).reshape(n, k).astype(np.float64).sum(axis=0)
     check = f32.double().sum(dim=1).cpu().numpy()
     # each output carries the fp16 rounding of its weights (about 1e-4 rms, random sign): the sums of
@@ -179,7 +191,48 @@ def test_gguf_q4_k_super_block_scales_of_any_size(oracle, cuda):
     A = torch.from_numpy(a).to(cuda)
     from rocmforge_amd import ops
     wd = torch.from_numpy(w).to(cuda)
-    assert torch.equal(ops.gemm_f16_arranged(Q.GGUF_Q4_K, wd, ops.ArrangedA(A), n, out_dtype=torch.float32).cpu(), torch.from_numpy(out))
+    # (this shape is split along k in two parts by rfq_gemm_f16; the arranged entry point takes it in one pass)
+    one_pass = ops.gemm_f16_arranged(Q.GGUF_Q4_K, wd, ops.ArrangedA(A), n, out_dtype=torch.float32).cpu().numpy()
+    for col in range(n):
+        assert_close(one_pass[:, col], want[:, col], f"one pass over k, weight row {col}")
+        assert_close(one_pass[:, col], exact[:, col], f"one pass over k (float64 sums), weight row {col}", tol=2e-5, plain_tol=2e-4)
+
+
+@pytest.mark.parametrize("fmt", FORMATS)
+@pytest.mark.parametrize("m,n,k,parts", [(300, 200, 2048, 2), (64, 130, 4096, 4), (33, 70, 8192, 8)])
+def test_split_along_k(fmt, m, n, k, parts, oracle, cuda):
+    """Few output tiles and a long k: the launch is split along k into whole super-blocks, the parts' f32 tiles are
+    added in a fixed order: against the oracle, deterministic, and the fp16 output is the rounded fp32 output."""
+    import torch
+    from rocmforge_amd import _lib
+    assert _lib.lib().rfq_gemm_f16_k_parts(m, n, k) == parts
+    w, a = weights(fmt, n, k, 61 + fmt), acts(m, k, 62 + n)
+    out = run(fmt, w, a, n, k, cuda, torch.float32)
+    again = run(fmt, w, a, n, k, cuda, torch.float32)
+    assert torch.equal(out, again)
+    assert torch.equal(run(fmt, w, a, n, k, cuda, torch.float16), out.to(torch.float16))
+    want = oracle.qmatmul_nk(fmt, w, a.astype(np.float32), m, n, k)
+    # (the 256-byte Q4_K layout here holds one-sided sub-blocks, mins of 0: its single fp16 operand q * scale then carries
+    # the whole value and the plain figure is 4-7e-3 at any k, in one pass over k as in parts; held to the first figure)
+    assert_close(out.cpu().numpy(), want, f"{Q.NAMES[fmt]} {m}x{n}x{k} in {parts} parts", plain_tol=None if fmt == Q.Q4_K else 1e-3)
+    if fmt != Q.Q4_K:
+        assert_close(out.cpu().numpy(), exact_weight_product(oracle, fmt, w, a, n, k), "same (float64 sums)", tol=2e-5, plain_tol=2e-4)
+    else:
+        w = weights(fmt, n, k, 62 + fmt)                                  # the synthetic blocks with integer mins: both figures
+        out = run(fmt, w, a, n, k, cuda, torch.float32).cpu().numpy()
+        assert_close(out, oracle.qmatmul_nk(fmt, w, a.astype(np.float32), m, n, k), f"Q4_K synthetic blocks {m}x{n}x{k} in {parts} parts")
+
+
+def test_k_parts_rule():
+    from rocmforge_amd import _lib
+    L = _lib.lib()
+    assert L.rfq_gemm_f16_k_parts(512, 14336, 4096) == 1        # 224 tiles: the part is full
+    assert L.rfq_gemm_f16_k_parts(512, 4096, 14336) == 4        # 64 tiles, 56 super-blocks: 4 x 14
+    assert L.rfq_gemm_f16_k_parts(512, 4096, 4096) == 4
+    assert L.rfq_gemm_f16_k_parts(512, 1024, 4096) == 4         # 16 tiles: k / parts stays >= 1024
+    assert L.rfq_gemm_f16_k_parts(300, 384, 1024) == 1
+    assert L.rfq_gemm_f16_k_parts(64, 128, 4128) == 1           # k not whole super-blocks
+    assert L.rfq_gemm_f16_k_parts(0, 128, 4096) == 1
 
 
 def test_weights_at_a_4_byte_offset_and_kept_temporary(oracle, cuda):
@@ -272,13 +325,21 @@ def test_arranged_activations_give_the_same_bits(fmt, m, n, k, cuda):
     w = torch.from_numpy(weights(fmt, n, k, 31)).to(cuda)
     a = torch.from_numpy(acts(m, k, 32)).to(cuda)
     A = ops.ArrangedA(a)
+    from rocmforge_amd import _lib
+    split = _lib.lib().rfq_gemm_f16_k_parts(m, n, k) > 1      # rfq_gemm_f16 then adds k in parts: another order of the fp32 sums
+    assert split == ((m, n, k) == (512, 256, 4096))
     for dt in (torch.float32, torch.float16):
         want = ops.gemm_f16(fmt, w, a, n, k, out_dtype=dt)
         got = ops.gemm_f16_arranged(fmt, w, A, n, out_dtype=dt)
         torch.cuda.synchronize()
-        assert torch.equal(got, want), f"{Q.NAMES[fmt]} {m}x{n}x{k} {dt}"
+        if split:
+            assert_close(got.float().cpu().numpy(), want.float().cpu().numpy(), f"{Q.NAMES[fmt]} {m}x{n}x{k} {dt}",
+                         tol=2e-5 if dt == torch.float32 else 2.0 ** -10, plain_tol=None)
+        else:
+            assert torch.equal(got, want), f"{Q.NAMES[fmt]} {m}x{n}x{k} {dt}"
     w2 = torch.from_numpy(weights(fmt, n, k, 33)).to(cuda)                  # a second projection of the same input
-    assert torch.equal(ops.gemm_f16_arranged(fmt, w2, A, n), ops.gemm_f16(fmt, w2, a, n, k))
+    if not split:
+        assert torch.equal(ops.gemm_f16_arranged(fmt, w2, A, n), ops.gemm_f16(fmt, w2, a, n, k))
 
 
 def test_arranged_activations_in_a_graph_and_bad_sizes(cuda):
