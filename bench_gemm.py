@@ -171,6 +171,12 @@ def run(torch):
     res["Q6_K gemm 512x4096x14336 fp16"] = kq_gemm(torch, Q.Q6_K, one_plane=True)
     res["GGUF_Q4_K gemm 512x4096x14336 fp16"] = kq_gemm(torch, Q.GGUF_Q4_K, one_plane=True)
     res["GGUF_Q6_K gemm 512x4096x14336 fp16"] = kq_gemm(torch, Q.GGUF_Q6_K, one_plane=True)
+    # the down projection of the same layer: 64 output tiles, split along k in four parts (rfq_gemm_f16_k_parts)
+    for fmt in (Q.Q4_K, Q.GGUF_Q4_K):
+        r = kq_gemm(torch, fmt, n=4096, k=14336, steps=100, warmup=100, arranged=True)
+        r["k_parts"] = 4
+        r["activations_arranged_once"]["what"] += " (a single pass over k: that entry point has no temporary for parts)"
+        res[f"{Q.NAMES[fmt]} gemm 512x14336x4096 fp16 (down projection)"] = r
     res["MXFP4 gemm 2048x8192x28672 bf16"] = mx_gemm(torch, Q.MXFP4)
     res["MXFP4 gemm 2048x8192x28672 bf16, full-entropy operands"] = mx_gemm(torch, Q.MXFP4, data="window")
     res["MXFP6-weight gemm 2048x8192x28672 bf16"] = mx_gemm(torch, Q.MXFP6_E2M3)
