@@ -343,8 +343,11 @@ RFQ_API int rfq_gemm_f16(int fmt, const void *d_w, size_t w_bytes, const void *d
 /* rfq_gemm_f16 for callers that cannot allocate device memory: code under
  * stream capture, tight serving loops, harnesses that forbid hipMalloc.  No
  * counterpart in the reference.  Same arguments, same kernels and bit-identical
- * results, but the temporaries (the activations in matrix-operand order, the
- * Q4_K group sums) live in a 16 MiB array that is part of the library's device
+ * results (a shape that rfq_gemm_f16 splits along k is split here too when the
+ * parts' f32 tiles fit the array beside the rest, and taken in one pass over k
+ * otherwise: then the order of the fp32 sums differs), but the temporaries (the
+ * activations in matrix-operand order, the Q4_K group sums, the parts) live in a
+ * 16 MiB array that is part of the library's device
  * image, one copy per GPU, held until the process ends; the call allocates
  * and frees nothing.  Shapes whose temporaries exceed the array fail with
  * RFQ_E_SIZE: ceil(m / 32) * ceil(k / 64) * 4096 bytes, plus ceil(m / 32) * k * 4
