@@ -588,12 +588,14 @@ template <> struct Opened<RFQ_GGUF_Q6_K> {
 };
 template <> struct Unit<RFQ_GGUF_Q6_K> {
     static constexpr bool NEEDS_XSUM = true;
-    Window<8> wl, wh; uint16_t sc2, d; int t;
+    Window<8> wl, wh; uint16_t sc2, sc2b, d; int t;
     template <bool BYTES> __device__ __forceinline__ void load_as(const uint8_t *row, int u)
     {
         const uint8_t *blk = row + (size_t)(u >> 3) * 210;
         const int half = (u >> 2) & 1;
         t = u & 3;
+        // (the scales of quarter t | 2, which shares this unit's bytes: what the paired form multiplies as well)
+        sc2b = ld<uint16_t>(blk + 192 + 8 * half + 2 * (t | 2));
         if constexpr (BYTES) {
             wl.load_bytes<0>(blk + 64 * half + 32 * (t & 1));
             wh.load_bytes<0>(blk + 128 + 32 * half);
@@ -1331,6 +1333,8 @@ template <> struct IUnit<RFQ_GGUF_Q4_K> : Unit<RFQ_GGUF_Q4_K> {
     static constexpr bool NIBBLE = false;
     static constexpr uint32_t TOPOFF = 0;
     static constexpr bool PAIR = true;            // units 2p and 2p+1 read the same bytes: give both to one lane
+    static __device__ __forceinline__ int pair_first(int p) { return 2 * p; }
+    static __device__ __forceinline__ int pair_second(int p) { return 2 * p + 1; }
     // byte l of the chunk holds element l of this unit in its low (even unit) or high (odd unit) nibble
     __device__ __forceinline__ float idot(const XPrep &xp) const
     {
@@ -1385,9 +1389,46 @@ template <> struct IUnit<RFQ_GGUF_Q4_K> : Unit<RFQ_GGUF_Q4_K> {
 // four weights), which is what the byte dot products take; the two int8 scales of the unit
 // get a sum each, and the offset of 32 goes through the sums of x over the two halves.
 template <> struct IUnit<RFQ_GGUF_Q6_K> : Unit<RFQ_GGUF_Q6_K> {
-    static constexpr bool PAIR = false;
+    // Quarters t and t + 2 of a half read the same 32 ql bytes (low and high nibbles) and the same 32 qh bytes: one lane
+    // takes both from one fetch (units 4h + t and 4h + t + 2, t < 2), which halves the loads and the window moves per weight.
+    static constexpr bool PAIR = true;
+    static __device__ __forceinline__ int pair_first(int p) { return ((p >> 1) << 2) | (p & 1); }
+    static __device__ __forceinline__ int pair_second(int p) { return pair_first(p) + 2; }
     static constexpr bool NIBBLE = false;
     static constexpr uint32_t TOPOFF = 0;
+    __device__ __forceinline__ float idot_pair(const XPrep &xa, const XPrep &xb) const    // this unit (t < 2) and the one two on
+    {
+        U8 ql, qh;
+        wl.piece<0>(ql.v);
+        wh.piece<0>(qh.v);
+        const int shr = 2 * t;
+        uint32_t alo[2] = {0, 0}, amid[2] = {0, 0}, blo[2] = {0, 0}, bmid[2] = {0, 0};
+        int atop[2] = {0, 0}, btop[2] = {0, 0};
+#pragma unroll
+        for (int w = 0; w < 8; w++) {
+            // bits 4-5 of a code: the bit pair at 2t (this unit) or 2t + 4 (the other) of its qh byte; what a shift drags in
+            // from the neighbouring byte is masked away
+            const uint32_t r = qh.v[w] >> shr;
+            const uint32_t va = ((r << 4) & 0x30303030u) | (ql.v[w] & 0x0F0F0F0Fu);
+            const uint32_t vb = (r & 0x30303030u) | ((ql.v[w] >> 4) & 0x0F0F0F0Fu);
+            const uint32_t *A = &xa.l[w * 3], *B = &xb.l[w * 3];
+            alo[w >> 2] = __builtin_amdgcn_udot4(va, A[0], alo[w >> 2], false);
+            amid[w >> 2] = __builtin_amdgcn_udot4(va, A[1], amid[w >> 2], false);
+            atop[w >> 2] = __builtin_amdgcn_sdot4((int)va, (int)A[2], atop[w >> 2], false);
+            blo[w >> 2] = __builtin_amdgcn_udot4(vb, B[0], blo[w >> 2], false);
+            bmid[w >> 2] = __builtin_amdgcn_udot4(vb, B[1], bmid[w >> 2], false);
+            btop[w >> 2] = __builtin_amdgcn_sdot4((int)vb, (int)B[2], btop[w >> 2], false);
+        }
+        const float SA0 = __builtin_fmaf((float)atop[0], 65536.0f, __builtin_fmaf((float)amid[0], 256.0f, (float)alo[0]));
+        const float SA1 = __builtin_fmaf((float)atop[1], 65536.0f, __builtin_fmaf((float)amid[1], 256.0f, (float)alo[1]));
+        const float SB0 = __builtin_fmaf((float)btop[0], 65536.0f, __builtin_fmaf((float)bmid[0], 256.0f, (float)blo[0]));
+        const float SB1 = __builtin_fmaf((float)btop[1], 65536.0f, __builtin_fmaf((float)bmid[1], 256.0f, (float)blo[1]));
+        const float a0 = (float)(int)(int8_t)(sc2 & 255u), a1 = (float)(int)(int8_t)(sc2 >> 8);
+        const float b0 = (float)(int)(int8_t)(sc2b & 255u), b1 = (float)(int)(int8_t)(sc2b >> 8);
+        const float ha0 = __builtin_fmaf(xa.s, SA0, -32.0f * xa.xh0), ha1 = __builtin_fmaf(xa.s, SA1, -32.0f * xa.xh1);
+        const float hb0 = __builtin_fmaf(xb.s, SB0, -32.0f * xb.xh0), hb1 = __builtin_fmaf(xb.s, SB1, -32.0f * xb.xh1);
+        return f16_bits_to_f32(d) * (__builtin_fmaf(a0, ha0, a1 * ha1) + __builtin_fmaf(b0, hb0, b1 * hb1));
+    }
     __device__ __forceinline__ float idot(const XPrep &xp) const
     {
         // bits 4-5 of a code: the bit pair at 2t of its qh byte, brought to bits 4-5 by one rotation (what it drags in
@@ -1648,7 +1689,8 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
     constexpr int WAVES = IDOT_WAVES, TEAMS = WAVES / WPR, TL = 64 * WPR, THREADS = 64 * WAVES;
     // rows in flight per lane: three, or five in the form with one unit per lane (its registers allow it;
     // measured 3..7 there at 14336 x 4096: 11.58, 11.41, 11.30, 11.72, 11.95 us)
-    constexpr int DW = (UPL == 1 && WPR == 2) ? 5 : 3;
+    // (GGUF_Q6_K in its paired form, one fetch per two units: four -- 14336 x 4096 with 3, 4, 5 in flight: 13.8, 13.2, 13.8 us)
+    constexpr int DW = (UPL == 1 && WPR == 2) ? 5 : (FMT == RFQ_GGUF_Q6_K && UPL == 2) ? 4 : 3;
     constexpr int D = R < DW ? R : DW;
     extern __shared__ __attribute__((aligned(16))) uint32_t idot_lds[]; // (MXFP4: the code table,) [units][28]
     constexpr size_t LUT_DWORDS = FMT == RFQ_MXFP4 ? MX4_LUT_BYTES / 4 : 0;
@@ -1664,12 +1706,13 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
     bool live[UPL];
     int unit[UPL];
     if constexpr (IU::PAIR && UPL == 2) {
-        // lane p owns units 2p and 2p+1 (the unit count of such a format is even: both live or both past the end)
+        // lane p owns the two units of pair p (the unit count of such a format is a multiple of eight: both live or
+        // both past the end)
         const bool in = 2 * tl < ku;
         const int p = in ? tl : (ku >> 1) - 1;
         live[0] = live[1] = in;
-        unit[0] = 2 * p;
-        unit[1] = 2 * p + 1;
+        unit[0] = IU::pair_first(p);
+        unit[1] = IU::pair_second(p);
     } else {
 #pragma unroll
         for (int j = 0; j < UPL; j++) {
