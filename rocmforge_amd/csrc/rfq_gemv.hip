@@ -217,7 +217,9 @@ template <int NQ> struct Window {
     }
     template <uint32_t SKIP> __device__ __forceinline__ void piece(uint32_t (&q)[NQ]) const
     {
-        const uint32_t sel = 0x03020100u + 0x01010101u * (o + SKIP);    // o + SKIP <= 4: bytes of a dword pair
+        // o + SKIP <= 4: bytes of a dword pair.  (o in all four bytes by a byte permute: a 32-bit multiply runs at a
+        // quarter of the rate)
+        const uint32_t sel = (0x03020100u + 0x01010101u * SKIP) + __builtin_amdgcn_perm(0u, o, 0u);
 #pragma unroll
         for (int i = 0; i < NQ; i++) q[i] = __builtin_amdgcn_perm(d[i + 1], d[i], sel);
     }
@@ -1567,7 +1569,8 @@ template <> struct IUnit<RFQ_MXFP4> : Unit<RFQ_MXFP4> {
         uint32_t alo = 0, amid = 0;
         int atop = 0;
         int ee = e;
-        if (__builtin_amdgcn_ballot_w64(e >= 1) == 0) {
+        // (e + 127 as unsigned: 0 .. 127 for the plain exponents -127 .. 0, beyond for e >= 1 and for -128)
+        if (__builtin_amdgcn_ballot_w64((uint32_t)(e + 127) > 127u) == 0) {
 #pragma unroll
             for (int d = 0; d < 4; d++) {
                 const uint32_t x = q.v[d];
@@ -1578,13 +1581,15 @@ template <> struct IUnit<RFQ_MXFP4> : Unit<RFQ_MXFP4> {
             }
         } else {                                                         // (weights below 1 never have such a unit)
             // magnitudes capped at 8 / 2^e in units of 1/2: tables 16 + {0, 2, 2, 4 | 4, 8, 8, 16}, 16 - {1, 2, 2, 4 | 4, 8, 8, 16}
-            const uint32_t b = e <= 0 ? 16u : (e >= 4 ? 1u : (16u >> e));
+            int es = e;
+            asm volatile("" : "+v"(es));                                 // (keeps this path's set-up out of the common one)
+            const uint32_t b = es <= 0 ? 16u : (es >= 4 ? 1u : (16u >> es));
             auto lim = [&](uint32_t m) { return m < b ? m : b; };
             const uint32_t plo = pack4(16u, 16u + lim(2), 16u + lim(2), 16u + lim(4));
             const uint32_t phi = pack4(16u + lim(4), 16u + lim(8), 16u + lim(8), 16u + lim(16));
             const uint32_t nlo = pack4(16u - lim(1), 16u - lim(2), 16u - lim(2), 16u - lim(4));
             const uint32_t nhi = pack4(16u - lim(4), 16u - lim(8), 16u - lim(8), 16u - lim(16));
-            ee = e > 4 ? 4 : e;
+            ee = es > 4 ? 4 : (es == -128 ? -300 : es);
 #pragma unroll
             for (int d = 0; d < 4; d++) {
                 const uint32_t x = q.v[d];
@@ -1601,7 +1606,7 @@ template <> struct IUnit<RFQ_MXFP4> : Unit<RFQ_MXFP4> {
         const float S = __builtin_fmaf((float)atop, 65536.0f, __builtin_fmaf((float)amid, 256.0f, (float)alo));
         // xh0: s * sum(X), see prep_convert_quarter; the scale of exponent -128 is 0 (mx_scale)
         const float v = __builtin_fmaf(0.5f * xp.s, S, -8.0f * xp.xh0);
-        return __builtin_ldexpf(v, ee == -128 ? -300 : ee);
+        return __builtin_ldexpf(v, ee);                                  // (-300 for the exponent -128: scale 0)
     }
 };
 
