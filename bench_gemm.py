@@ -193,13 +193,15 @@ if __name__ == "__main__":
     ap.add_argument("--probe-mfma", action="store_true", help="the fp16 matrix pipe alone and beside a fused kernel's operand traffic")
     ap.add_argument("--probe-variant", type=int, choices=[0, 1], help="only v_mfma_f32_32x32x16_f16 (0) or v_mfma_f32_16x16x32_f16 (1)")
     ap.add_argument("--data", choices=["packer", "window"], default="packer", help="MXFP4 operands: the reference packer's, or full-entropy")
+    ap.add_argument("--down", action="store_true", help="with --only q4_k / gguf_q4_k: the down projection 512 x 14336 -> 4096 (split along k)")
     a = ap.parse_args()
     import torch
     from rocmforge_amd import quantize as Q
     if a.probe_mfma:
         mfma_probe(torch, a.probe_variant)
     elif a.only in ("q4_k", "gguf_q4_k"):
-        print(json.dumps(kq_gemm(torch, Q.Q4_K if a.only == "q4_k" else Q.GGUF_Q4_K, steps=a.steps, arranged=True)))
+        shape = dict(n=4096, k=14336) if a.down else {}
+        print(json.dumps(kq_gemm(torch, Q.Q4_K if a.only == "q4_k" else Q.GGUF_Q4_K, steps=a.steps, arranged=not a.down, **shape)))
     elif a.only:
         print(json.dumps(mx_gemm(torch, Q.MXFP4 if a.only == "mxfp4" else Q.MXFP6_E2M3, steps=a.steps, data=a.data)))
     else:
