@@ -837,7 +837,9 @@ gemv_xreg_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
     constexpr int TEAMS = 4 / WPR, TL = 64 * WPR;
     // rows in flight per lane: three, or five in the form with one unit per lane and two wavefronts per row
     // (Q6_K 14336 x 4096 in that form: 14.6 us with three, 13.8 us with five)
-    constexpr int DW = (UPL == 1 && WPR == 2) ? 5 : 3;
+    // (MXFP4 in that form, whose look-ups go through LDS: three -- 32000 x 4096 16.3 -> 15.2 us, level at 8192 rows;
+    // MXFP6 with three: 32000 x 4096 23.1 -> 24.7)
+    constexpr int DW = (UPL == 1 && WPR == 2) ? (FMT == RFQ_MXFP4 ? 3 : 5) : 3;
     constexpr int D = R < DW ? R : DW;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int team = wave / WPR, wit = wave % WPR;
@@ -1632,6 +1634,12 @@ __device__ __forceinline__ float idot_pair_of(const IU &u, const XPrep &xe, cons
 // each thread converts a quarter unit.
 constexpr int IDOT_WAVES = 8;
 
+// Rows in flight per lane in the form with one unit per lane and two wavefronts per row.
+constexpr int idot_rows_in_flight_12(int fmt)
+{
+    return fmt == RFQ_MXFP4 ? 2 : (fmt == RFQ_Q6_K || fmt == RFQ_MM_Q6_K) ? 3 : 5;
+}
+
 // ---- a timeline from inside the kernel (rfq_bench_gemv_timeline) ------------------------------------------------
 // gemv_idot_kernel<..., TRACE = true> has every wavefront read the constant 100 MHz clock (s_memrealtime) at the
 // points below and write the readings, lane 0, to g_gemv_trace[wavefront][TRACE_STAMPS] when it ends.  A reading is
@@ -1695,7 +1703,12 @@ gemv_idot_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
     // rows in flight per lane: three, or five in the form with one unit per lane (its registers allow it;
     // measured 3..7 there at 14336 x 4096: 11.58, 11.41, 11.30, 11.72, 11.95 us)
     // (GGUF_Q6_K in its paired form, one fetch per two units: four -- 14336 x 4096 with 3, 4, 5 in flight: 13.8, 13.2, 13.8 us)
-    constexpr int DW = (UPL == 1 && WPR == 2) ? 5 : (FMT == RFQ_GGUF_Q6_K && UPL == 2) ? 4 : 3;
+    // (MXFP4 and Q6_K, bound by their instructions, want fewer in that form, 14336 x 4096 with 5 / 3 / 2 in flight:
+    // MXFP4 8.93 / 8.51 / 8.29 us (9.87 with one; 11008 rows 8.27 -> 7.70), Q6_K 11.62 / 11.52 / 11.87; Q4_K, bound by
+    // its bytes, 10.43 with 5, 10.67 with 4, 10.86 with 3; GGUF_Q4_0 and GGUF_Q8_0 gain 1-2 % there with three but
+    // lose the ring of five rows on long walks: 50000 x 4096 22.2 -> 25.1 and 39.2 -> 40.4 us)
+    constexpr int DW12 = idot_rows_in_flight_12(FMT);
+    constexpr int DW = (UPL == 1 && WPR == 2) ? DW12 : (FMT == RFQ_GGUF_Q6_K && UPL == 2) ? 4 : 3;
     constexpr int D = R < DW ? R : DW;
     extern __shared__ __attribute__((aligned(16))) uint32_t idot_lds[]; // (MXFP4: the code table,) [units][28]
     constexpr size_t LUT_DWORDS = FMT == RFQ_MXFP4 ? MX4_LUT_BYTES / 4 : 0;
@@ -2325,7 +2338,7 @@ int run_idot(const uint8_t *w, const float *x, float *y, int n, int k, const Gem
         const int slots = device_cu_count() * 8 / IDOT_WAVES * (UPL == 1 && WPR == 2 ? 2 : 1);
         int want = (n + slots * TEAMS - 1) / (slots * TEAMS);
         if (want < 1) want = 1;
-        constexpr bool FIVE = UPL == 1 && WPR == 2 && !FUSE;
+        constexpr bool FIVE = UPL == 1 && WPR == 2 && !FUSE && idot_rows_in_flight_12(FMT) == 5;   // (groups of five ring on only with five in flight)
         static const int RS[5] = {2, 4, 5, 7, 8};
         int best_r = 8, best_groups = 1, best_blocks = 0;
         long best_cost = -1;
