@@ -93,7 +93,7 @@ def mx_gemm(torch, w_fmt, m=2048, n=28672, k=8192, steps=200, warmup=200, data="
     return res
 
 
-def kq_gemm(torch, fmt, m=512, n=14336, k=4096, steps=300, warmup=300, arranged=False, one_plane=False):
+def kq_gemm(torch, fmt, m=512, n=14336, k=4096, steps=300, warmup=600, arranged=False, one_plane=False):
     """Q4_K / Q6_K prefill GEMM on the fp16 matrix cores, fp16 in and out.  one_plane: RFQ_GEMM_ONE_PLANE (every weight
     as one fp16 operand) beside the default two (hi + lo)."""
     from rocmforge_amd import _lib, quantize as Q
