@@ -179,7 +179,7 @@ def run(torch):
     res["GGUF_Q6_K gemm 512x4096x14336 fp16"] = kq_gemm(torch, Q.GGUF_Q6_K, one_plane=True)
     # the down projection of the same layer: 64 output tiles, split along k in four parts (rfq_gemm_f16_k_parts)
     for fmt in (Q.Q4_K, Q.GGUF_Q4_K):
-        r = kq_gemm(torch, fmt, n=4096, k=14336, steps=100, warmup=100, arranged=True)
+        r = kq_gemm(torch, fmt, n=4096, k=14336, steps=200, warmup=400, arranged=True)
         r["k_parts"] = 4
         r["activations_arranged_once"]["what"] += " (a single pass over k: that entry point has no temporary for parts)"
         res[f"{Q.NAMES[fmt]} gemm 512x14336x4096 fp16 (down projection)"] = r
