@@ -192,6 +192,10 @@ def time_dequant(torch, fmt, n, k, steps, warmup, Q, seed):
     L = _lib.lib()
     _lib.check(L.rfq_bench_dequant(fmt, ptrs, copies, w.size, C.c_void_p(out.data_ptr()), n * k, out_copies, 0, warmup, stream,
                                    C.byref(ms)))
+    # PREHEAT_MS of untimed calls, as for the GEMV lines (out of idle the first milliseconds run on ramping clocks)
+    preheat = max(1, int(PREHEAT_MS / max(ms.value / warmup, 2e-3)))
+    _lib.check(L.rfq_bench_dequant(fmt, ptrs, copies, w.size, C.c_void_p(out.data_ptr()), n * k, out_copies, 0, preheat, stream,
+                                   C.byref(ms)))
     _lib.check(L.rfq_bench_dequant(fmt, ptrs, copies, w.size, C.c_void_p(out.data_ptr()), n * k, out_copies, 0, steps, stream,
                                    C.byref(ms)))
     return ms.value / 1e3 / steps, w.size + 4 * n * k
