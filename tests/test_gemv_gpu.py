@@ -102,20 +102,21 @@ def test_gemv_mx_random_codes_and_clamp(fmt, oracle, cuda):
     assert_close(gpu_gemv(fmt, w, x, n, k, cuda), oracle.qmatmul_nk(fmt, w, x, 1, n, k)[0], Q.NAMES[fmt])
 
 
+@pytest.mark.parametrize("fmt", [Q.MXFP4, Q.MXFP6_E2M3])
 @pytest.mark.parametrize("n,k", [(96, 4096), (2100, 4096), (14336, 4096), (300, 12288)])
-def test_gemv_mxfp4_extreme_exponents(n, k, oracle, cuda):
+def test_gemv_mx_extreme_exponents(fmt, n, k, oracle, cuda):
     """Exponent bytes -128 (the reference's scale is 0 there) and 127 (every non-zero code clamps to +-8) among ordinary
-    and clamping ones, at shapes that take the integer-dot kernel (96, 14336 and 300 rows) and the float one (2100)."""
-    rng = np.random.default_rng(7700 + n)
-    w = Q.random_blocks(Q.MXFP4, n * k // 32, rng, exp_range=(-9, 3)).copy()
-    blocks = w.reshape(-1, 17)
+    and clamping ones, at shapes where MXFP4 takes the integer-dot kernel (96, 14336 and 300 rows) and the float one (2100)."""
+    rng = np.random.default_rng(7700 + n + fmt)
+    w = Q.random_blocks(fmt, n * k // 32, rng, exp_range=(-9, 3)).copy()
+    blocks = w.reshape(-1, Q.BLOCK_BYTES[fmt])
     blocks[rng.random(blocks.shape[0]) < 0.02, 0] = 0x80
     blocks[rng.random(blocks.shape[0]) < 0.02, 0] = 0x7F
     x = x_for(1, k, 7701)
     x[64:96] = 0.0
-    got = gpu_gemv(Q.MXFP4, w, x, n, k, cuda)
+    got = gpu_gemv(fmt, w, x, n, k, cuda)
     assert np.isfinite(got).all()
-    assert_close(got, oracle.qmatmul_nk(Q.MXFP4, w, x, 1, n, k)[0], f"MXFP4 n={n} k={k} with exponents -128 and 127")
+    assert_close(got, oracle.qmatmul_nk(fmt, w, x, 1, n, k)[0], f"{Q.NAMES[fmt]} n={n} k={k} with exponents -128 and 127")
 
 
 # The benchmark configurations: Q4_0 4864x896; Q8_0 4096x4096 at m = 1 and 8; Q4_K and Q6_K 14336x4096.
