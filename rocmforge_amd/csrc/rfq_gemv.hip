@@ -841,7 +841,9 @@ gemv_xreg_kernel(const uint8_t *__restrict__ w, const float *__restrict__ x, flo
     // MXFP6 with three: 32000 x 4096 23.1 -> 24.7)
     // (MXFP6 with two units per lane: two -- 4096 x 8192 9.36 -> 8.69 us, 8192 x 8192 13.5 -> 12.8, 4096 x 5120 8.05 -> 7.57,
     // 4096 x 14336 14.6 -> 14.0, 28672 x 8192 38.0 -> 37.8; MXFP4 28672 x 8192 with two 28.0 -> 29.0, Q6_K mixed)
-    constexpr int DW = (UPL == 1 && WPR == 2) ? (FMT == RFQ_MXFP4 ? 3 : 5) : (FMT == RFQ_MXFP6_E2M3 ? 2 : 3);
+    // (groups of up to four rows, any format: two -- Q6_K 4096 x 8192 8.40 -> 7.76 us, 4096 x 5120 6.85 -> 6.34,
+    // 4096 x 6144 7.31 -> 6.83, MXFP4 4096 x 5120 6.60 -> 6.44; with longer groups Q6_K and MXFP4 measured mixed)
+    constexpr int DW = (UPL == 1 && WPR == 2) ? (FMT == RFQ_MXFP4 ? 3 : 5) : ((FMT == RFQ_MXFP6_E2M3 || R <= 4) ? 2 : 3);
     constexpr int D = R < DW ? R : DW;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int team = wave / WPR, wit = wave % WPR;
