@@ -1925,7 +1925,9 @@ gemv_idot_batch_kernel(const uint8_t *__restrict__ w, const float *__restrict__ 
 {
     using IU = IUnit<FMT>;
     constexpr int TEAMS = 4 / WPR, TL = 64 * WPR;
-    constexpr int D = R < 3 ? R : 3;
+    // (two rows in flight: with three, Q8_0 4096 x 4096 m = 2 6.83 -> 6.50 us, m = 4 9.15 -> 8.92, Q4_K 14336 x 4096 m = 4
+    // 17.7 -> 17.3; with four 7.58, 10.16 and 18.7)
+    constexpr int D = R < 2 ? R : 2;
     static_assert(R * M <= 64, "one lane per (row, vector) in the cross-wavefront sum");
     extern __shared__ __attribute__((aligned(16))) uint32_t xlds[]; // [M][units][28]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
