@@ -713,6 +713,17 @@ reduce_parts_kernel(const float *__restrict__ parts, void *__restrict__ out, siz
             for (int e = 0; e < live; e++) v[e] += src[e];
         }
     }
+    if (live == 4 && (count & 3) == 0) {                               // one store per thread
+        if (OUT_F16) {
+            // (no alignment promise beyond the element's: global memory takes such stores at any address)
+            typedef _Float16 h4 __attribute__((ext_vector_type(4), aligned(2)));
+            *reinterpret_cast<h4 *>(reinterpret_cast<_Float16 *>(out) + i4) = h4{(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
+        } else {
+            typedef float f4 __attribute__((ext_vector_type(4), aligned(4)));
+            *reinterpret_cast<f4 *>(reinterpret_cast<float *>(out) + i4) = f4{v[0], v[1], v[2], v[3]};
+        }
+        return;
+    }
     for (int e = 0; e < live; e++) {
         if (OUT_F16) reinterpret_cast<_Float16 *>(out)[i4 + e] = (_Float16)v[e];
         else reinterpret_cast<float *>(out)[i4 + e] = v[e];
