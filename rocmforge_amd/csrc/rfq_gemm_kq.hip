@@ -135,8 +135,8 @@ arrange_a_kernel(const _Float16 *__restrict__ a, v4u *__restrict__ at, _Float16 
         fp16_pair(sum, hi, lo);
         const int g = k0 / 32, sb = g & 7;
         const size_t t = ((((size_t)mt * (K / 256) + (g >> 3)) * 2 + (sb >> 2)) * 32 + fr) * 4 + (sb & 3);
-        s2[2 * t] = hi;
-        s2[2 * t + 1] = lo;
+        typedef _Float16 h2 __attribute__((ext_vector_type(2), aligned(2)));
+        *reinterpret_cast<h2 *>(s2 + 2 * t) = h2{hi, lo};              // (one store for the pair)
     }
 }
 
